@@ -1,0 +1,107 @@
+// Expression IR for element-wise kernels.
+//
+// The text form is what custos' `ToCLSource` impls print for a `Combiner`
+// tree (reference: src/two_way_ops/ops.rs, ops/unary.rs, ops/cmps.rs,
+// resolve.rs:131-141, to_cl_source.rs:7-11) and what
+// `operations_to_fused_src` prints for a fused chain (src/devices/fusing.rs:4-19).
+// It is parsed into a small DAG, hashed structurally, and emitted as typed
+// HIP C in SSA form with one statement (= one rounding) per node.
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace custos_hip {
+
+enum class Op : uint8_t {
+    Var,
+    Const,
+    // binary
+    Add,
+    Sub,
+    Mul,
+    Div,
+    Pow,
+    Min,
+    Max,
+    GEq,
+    LEq,
+    Eq,
+    // unary
+    Sin,
+    Cos,
+    Tan,
+    Tanh,
+    Exp,
+    Ln,
+    Abs,
+    Neg,
+    Sqrt,
+};
+
+bool op_is_binary(Op op);
+bool op_is_unary(Op op);
+
+struct Node {
+    Op op = Op::Const;
+    int a = -1;       // operand node index
+    int b = -1;       // second operand node index (binary ops)
+    int var = 0;      // Op::Var: operand index
+    std::string lit;  // Op::Const: literal text as given
+};
+
+// Nodes are stored in evaluation order; operands always precede their user.
+struct Expr {
+    std::vector<Node> nodes;
+    int root = -1;
+    int n_vars = 0;
+};
+
+// Element types; numeric values equal `custos_hip_dtype`.
+enum class DType : int32_t {
+    F32 = 0,
+    F64 = 1,
+    I32 = 2,
+    I64 = 3,
+    F16 = 4,
+    BF16 = 5,
+    U8 = 6,
+    I8 = 7,
+    I16 = 8,
+    U16 = 9,
+    U32 = 10,
+    U64 = 11,
+};
+
+bool dtype_valid(int32_t v);
+size_t dtype_size(DType t);
+bool dtype_is_float(DType t);
+bool dtype_is_signed(DType t);
+const char* dtype_storage_c(DType t);  // C type of an element in memory
+const char* dtype_compute_c(DType t);  // C type the nodes are evaluated in
+
+struct ParseError {
+    int code = 0;  // a custos_hip_status value, 0 = ok
+    std::string message;
+};
+
+// Parses either one expression or a statement list "m = e;\n m = e;\n" in which
+// `m` must be markers[0] and every statement reads the previous one's value.
+bool parse_expr(const std::string& src, const std::vector<std::string>& markers, Expr* out,
+                ParseError* err);
+
+// Re-prints a tree in the reference's ToCLSource format (literals as given).
+std::string to_cl_source(const Expr& e, const std::vector<std::string>& markers);
+
+// Structural 64-bit hash: node kinds, operand wiring and the literal *values*
+// after conversion to the element type ("2", "2.0" and "2.00" hash alike).
+bool hash_expr(const Expr& e, DType dtype, uint64_t* hash, ParseError* err);
+
+// Emits the body of `custos_expr`: SSA statements over v0..v{n-1} of the
+// compute type and a final `return`.
+bool emit_expr_body(const Expr& e, DType dtype, std::string* out, ParseError* err);
+
+uint64_t fnv1a64(const void* data, size_t n, uint64_t seed = 0xcbf29ce484222325ull);
+
+}  // namespace custos_hip

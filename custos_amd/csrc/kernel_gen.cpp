@@ -1,0 +1,224 @@
+#include "kernel_gen.hpp"
+
+#include <algorithm>
+
+#include "../../include/custos_hip.h"
+
+namespace custos_hip {
+
+Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int nontemporal) {
+    Tuning t;
+    if (block_threads > 0) {
+        block_threads = std::max(64, std::min(1024, block_threads));
+        t.block_threads = (block_threads / 64) * 64;
+    }
+    if (unroll > 0) t.unroll = std::min(16, unroll);
+    t.blocks_per_cu = blocks_per_cu > 0 ? std::min(64, blocks_per_cu) : 0;
+    t.nontemporal = nontemporal < 0 ? 0 : (nontemporal & 3);
+    return t;
+}
+
+std::vector<std::string> hiprtc_options(const std::string& arch) {
+    return {
+        "--offload-arch=" + arch,
+        "-O3",
+        "-std=c++17",
+        // a*b+c must stay two roundings: the CPU device never fuses
+        "-ffp-contract=off",
+        // IEEE division and square root (bit-exact with the CPU device)
+        "-fhip-fp32-correctly-rounded-divide-sqrt",
+        // keep f32 arithmetic on the scalar-per-lane instructions
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    };
+}
+
+namespace {
+
+// Conversions between the storage and the compute type, and the math wrappers
+// the emitted expression calls.
+std::string prelude(DType dtype, int vec) {
+    std::string s;
+    s += "typedef unsigned long long u64;\n";
+    s += std::string("typedef ") + dtype_storage_c(dtype) + " S;\n";
+    s += std::string("typedef ") + dtype_compute_c(dtype) + " C;\n";
+    s += "typedef S vec_t __attribute__((ext_vector_type(" + std::to_string(vec) + ")));\n";
+    if (dtype == DType::BF16) {
+        s += R"(static __device__ __forceinline__ C custos_load(S s) {
+    return __builtin_bit_cast(float, (unsigned int)s << 16);
+}
+static __device__ __forceinline__ S custos_store(C c) {
+    unsigned int x = __builtin_bit_cast(unsigned int, c);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (S)((x >> 16) | 0x0040u);
+    x += 0x7fffu + ((x >> 16) & 1u);
+    return (S)(x >> 16);
+}
+)";
+    } else {
+        s += "static __device__ __forceinline__ C custos_load(S s) { return (C)s; }\n";
+        s += "static __device__ __forceinline__ S custos_store(C c) { return (S)c; }\n";
+    }
+    if (dtype == DType::F64) {
+        s += R"(static __device__ __forceinline__ double custos_sin(double a) { return sin(a); }
+static __device__ __forceinline__ double custos_cos(double a) { return cos(a); }
+static __device__ __forceinline__ double custos_tan(double a) { return tan(a); }
+static __device__ __forceinline__ double custos_tanh(double a) { return tanh(a); }
+static __device__ __forceinline__ double custos_exp(double a) { return exp(a); }
+static __device__ __forceinline__ double custos_log(double a) { return log(a); }
+static __device__ __forceinline__ double custos_sqrt(double a) { return sqrt(a); }
+)";
+    } else if (dtype_is_float(dtype)) {
+        s += R"(static __device__ __forceinline__ float custos_sin(float a) { return sinf(a); }
+static __device__ __forceinline__ float custos_cos(float a) { return cosf(a); }
+static __device__ __forceinline__ float custos_tan(float a) { return tanf(a); }
+static __device__ __forceinline__ float custos_tanh(float a) { return tanhf(a); }
+static __device__ __forceinline__ float custos_exp(float a) { return expf(a); }
+static __device__ __forceinline__ float custos_log(float a) { return logf(a); }
+static __device__ __forceinline__ float custos_sqrt(float a) { return sqrtf(a); }
+)";
+    }
+    return s;
+}
+
+std::string expr_fn(const KernelSpec& k, const std::string& body) {
+    std::string s = "static __device__ __forceinline__ C custos_expr(";
+    for (int i = 0; i < k.expr.n_vars; i++) {
+        if (i) s += ", ";
+        s += "const C v" + std::to_string(i);
+    }
+    s += ") {\n" + body + "}\n";
+    return s;
+}
+
+// lhs_grad + (out_grad * d): product rounded, then the sum rounded
+// (src/devices/cpu_stack_ops.rs:27-29); integers wrap.
+std::string grad_fn(DType dtype) {
+    if (dtype_is_float(dtype))
+        return "static __device__ __forceinline__ C custos_grad(const C g, const C o, const C d) {\n"
+               "    const C prod = o * d;\n    const C sum = g + prod;\n    return sum;\n}\n";
+    const char* U = dtype_size(dtype) == 8 ? "unsigned long long" : "unsigned int";
+    return std::string("static __device__ __forceinline__ C custos_grad(const C g, const C o, const C d) {\n") +
+           "    const C prod = (C)((" + U + ")o * (" + U + ")d);\n" +
+           "    return (C)((" + U + ")g + (" + U + ")prod);\n}\n";
+}
+
+}  // namespace
+
+bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
+                       const std::vector<std::string>& markers, const Tuning& tuning,
+                       KernelSpec* out, ParseError* err) {
+    KernelSpec k;
+    k.kind = kind;
+    k.dtype = dtype;
+    k.tuning = tuning;
+    if (!parse_expr(src, markers, &k.expr, err)) return false;
+    if (kind == Kind::UnaryGrad && k.expr.n_vars != 1) {
+        err->code = CUSTOS_HIP_ERR_ARITY_MISMATCH;
+        err->message = "a unary gradient expression takes exactly one marker";
+        return false;
+    }
+    uint64_t h;
+    if (!hash_expr(k.expr, dtype, &h, err)) return false;
+    int32_t tail[6] = {static_cast<int32_t>(kind), tuning.block_threads, tuning.unroll,
+                       tuning.blocks_per_cu, tuning.nontemporal, 2 /* template version */};
+    k.hash = fnv1a64(tail, sizeof tail, h);
+    k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
+
+    std::string body;
+    if (!emit_expr_body(k.expr, dtype, &body, err)) return false;
+
+    const int n_in = k.expr.n_vars;
+    const bool nt_load = tuning.nontemporal & 1, nt_store = tuning.nontemporal & 2;
+
+    std::string s;
+    s += "// generated by custos-hip: " + to_cl_source(k.expr, markers) + "\n";
+    s += "#define CUSTOS_BLOCK " + std::to_string(tuning.block_threads) + "\n";
+    s += "#define CUSTOS_UNROLL " + std::to_string(tuning.unroll) + "\n";
+    s += "#define CUSTOS_VEC " + std::to_string(k.vec_elems) + "\n";
+    s += nt_load ? "#define CUSTOS_LD(p) __builtin_nontemporal_load(p)\n" : "#define CUSTOS_LD(p) (*(p))\n";
+    s += nt_store ? "#define CUSTOS_ST(p, v) __builtin_nontemporal_store(v, p)\n"
+                  : "#define CUSTOS_ST(p, v) (*(p) = (v))\n";
+    s += prelude(dtype, k.vec_elems);
+    s += expr_fn(k, body);
+
+    // Per-element function on storage values: `custos_elem(in0.., [g])`.
+    // Pointers that are read and written (`out`, `lhs_grad`) carry no
+    // __restrict__: the output may be exactly one of the inputs.
+    std::string params, vec_ptrs, elem_params, elem_call_s, elem_call_v, loads;
+    if (kind == Kind::Apply) {
+        s += "static __device__ __forceinline__ S custos_elem(";
+        for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "const S s" + std::to_string(i);
+        s += ") {\n    return custos_store(custos_expr(";
+        for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "custos_load(s" + std::to_string(i) + ")";
+        s += "));\n}\n";
+        for (int i = 0; i < n_in; i++) {
+            std::string id = std::to_string(i);
+            params += "const S* in" + id + ", ";
+            vec_ptrs += "    const vec_t* vin" + id + " = (const vec_t*)(in" + id + " + head);\n";
+        }
+        params += "S* out";
+        vec_ptrs += "    vec_t* vout = (vec_t*)(out + head);\n";
+    } else {
+        s += grad_fn(dtype);
+        s += "static __device__ __forceinline__ S custos_elem(const S s0, const S s1, const S s2) {\n"
+             "    return custos_store(custos_grad(custos_load(s1), custos_load(s2), custos_expr(custos_load(s0))));\n}\n";
+        // operand order inside the kernel: 0 = lhs, 1 = lhs_grad (also the output), 2 = out_grad
+        params = "const S* in0, S* out, const S* in2";
+        vec_ptrs = "    const vec_t* vin0 = (const vec_t*)(in0 + head);\n"
+                   "    const vec_t* vin2 = (const vec_t*)(in2 + head);\n"
+                   "    vec_t* vout = (vec_t*)(out + head);\n"
+                   "    const vec_t* vin1 = vout;\n"
+                   "    const S* in1 = out;\n";
+    }
+    const int n_ops = kind == Kind::Apply ? n_in : 3;
+    auto list = [&](const std::string& pre, const std::string& post) {
+        std::string r;
+        for (int i = 0; i < n_ops; i++) r += std::string(i ? ", " : "") + pre + std::to_string(i) + post;
+        return r;
+    };
+
+    s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
+    s += std::string(kKernelName) + "(" + params + ", const u64 n, const u64 head, const u64 n_vec) {\n";
+    s += vec_ptrs;
+    s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
+    s += "    const u64 n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;\n";
+    s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {\n";
+    s += "        const u64 base = tile * tile_vecs + threadIdx.x;\n";
+    s += "        if (base + (u64)(CUSTOS_UNROLL - 1) * CUSTOS_BLOCK < n_vec) {\n";
+    for (int i = 0; i < n_ops; i++) s += "            vec_t a" + std::to_string(i) + "[CUSTOS_UNROLL];\n";
+    s += "#pragma unroll\n            for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+    for (int i = 0; i < n_ops; i++) {
+        std::string id = std::to_string(i);
+        s += "                a" + id + "[u] = CUSTOS_LD(vin" + id + " + base + (u64)u * CUSTOS_BLOCK);\n";
+    }
+    s += "            }\n";
+    s += "#pragma unroll\n            for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+    s += "                vec_t r;\n#pragma unroll\n                for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
+         list("a", "[u][k]") + ");\n";
+    s += "                CUSTOS_ST(vout + base + (u64)u * CUSTOS_BLOCK, r);\n            }\n";
+    s += "        } else {\n";
+    s += "#pragma unroll\n            for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+    s += "                const u64 idx = base + (u64)u * CUSTOS_BLOCK;\n";
+    s += "                if (idx < n_vec) {\n";
+    for (int i = 0; i < n_ops; i++) {
+        std::string id = std::to_string(i);
+        s += "                    const vec_t b" + id + " = CUSTOS_LD(vin" + id + " + idx);\n";
+    }
+    s += "                    vec_t r;\n#pragma unroll\n                    for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
+         list("b", "[k]") + ");\n";
+    s += "                    CUSTOS_ST(vout + idx, r);\n                }\n            }\n";
+    s += "        }\n    }\n";
+    // Elements outside the 16-byte aligned body: `head` leading ones and the
+    // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
+    s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
+    s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BLOCK;\n";
+    s += "    if (gid < head) out[gid] = custos_elem(" + list("in", "[gid]") + ");\n";
+    s += "    for (u64 i = head + n_vec * CUSTOS_VEC + gid; i < n; i += n_threads) out[i] = custos_elem(" +
+         list("in", "[i]") + ");\n";
+    s += "}\n";
+
+    k.source = std::move(s);
+    *out = std::move(k);
+    return true;
+}
+
+}  // namespace custos_hip

@@ -1,0 +1,672 @@
+// C ABI of the MI355X element-wise backend: device handle, memory, run-time
+// compiled expression kernels, launches, graph capture/replay.
+// Interface and reference citations: include/custos_hip.h.
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/custos_hip.h"
+#include "expr.hpp"
+#include "kernel_gen.hpp"
+
+using namespace custos_hip;
+
+struct custos_hip_kernel {
+    KernelSpec spec;
+    hipModule_t module = nullptr;
+    hipFunction_t fn = nullptr;
+};
+
+struct custos_hip_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    size_t kernel_nodes = 0;
+};
+
+struct custos_hip_device {
+    int idx = 0;
+    hipStream_t stream = nullptr;    // compute stream: every launch, in call order
+    hipStream_t transfer = nullptr;  // copies that must not be recorded while capturing
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    hipDeviceProp_t props{};
+    std::string arch;
+    Tuning tuning;
+    bool capturing = false;
+    uint64_t compiles = 0, hits = 0;
+    std::string last_error;
+    std::unordered_map<uint64_t, std::vector<std::unique_ptr<custos_hip_kernel>>> cache;
+    std::vector<custos_hip_graph*> graphs;
+};
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int32_t set_error(custos_hip_device* dev, int32_t code, const std::string& msg) {
+    (dev ? dev->last_error : g_last_error) = msg;
+    return code;
+}
+
+int32_t hip_fail(custos_hip_device* dev, hipError_t e, const char* what) {
+    // clear the sticky "last error" of the runtime so it is not reported twice
+    (void)hipGetLastError();
+    return set_error(dev, static_cast<int32_t>(e),
+                     std::string(what) + ": " + hipGetErrorName(e) + " (" + hipGetErrorString(e) + ")");
+}
+
+#define HIP_TRY(dev, call)                                   \
+    do {                                                     \
+        hipError_t e__ = (call);                             \
+        if (e__ != hipSuccess) return hip_fail(dev, e__, #call); \
+    } while (0)
+
+#define REQUIRE_DEV(dev)                                                                    \
+    do {                                                                                    \
+        if (!(dev)) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "device handle is null"); \
+        HIP_TRY(dev, hipSetDevice((dev)->idx));                                             \
+    } while (0)
+
+// ---- zero fill: 16-byte stores over the aligned body, bytes at the edges ----
+
+__global__ void __launch_bounds__(256) custos_fill_zero(unsigned char* p, unsigned long long bytes,
+                                                        unsigned long long head,
+                                                        unsigned long long n_vec) {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    u4* v = reinterpret_cast<u4*>(p + head);
+    const unsigned long long gid = (unsigned long long)blockIdx.x * 256 + threadIdx.x;
+    const unsigned long long n_threads = (unsigned long long)gridDim.x * 256;
+    const u4 z = {0u, 0u, 0u, 0u};
+    for (unsigned long long i = gid; i < n_vec; i += n_threads) v[i] = z;
+    if (gid < head) p[gid] = 0;
+    for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads) p[i] = 0;
+}
+
+int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream) {
+    unsigned long long head = (16 - (dptr & 15)) & 15;
+    if (head > bytes) head = bytes;
+    unsigned long long n_vec = (bytes - head) / 16;
+    unsigned long long want = (n_vec + 255) / 256;
+    // 8 vectors per thread at most: enough workgroups to fill the chip, not one per 4 KiB
+    unsigned long long cap = static_cast<unsigned long long>(dev->props.multiProcessorCount) * 64;
+    unsigned int grid = static_cast<unsigned int>(std::max(1ull, std::min(want, std::max(cap, (want + 7) / 8))));
+    grid = std::min(grid, 1u << 22);
+    hipLaunchKernelGGL(custos_fill_zero, dim3(grid), dim3(256), 0, stream,
+                       reinterpret_cast<unsigned char*>(dptr), static_cast<unsigned long long>(bytes),
+                       head, n_vec);
+    HIP_TRY(dev, hipGetLastError());
+    return CUSTOS_HIP_OK;
+}
+
+// ---- hiprtc ----
+
+int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec,
+                               const std::string& arch, std::vector<char>* code) {
+    hiprtcProgram prog = nullptr;
+    hiprtcResult r = hiprtcCreateProgram(&prog, spec.source.c_str(), "custos_kernel.hip", 0, nullptr, nullptr);
+    if (r != HIPRTC_SUCCESS)
+        return set_error(dev, CUSTOS_HIP_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
+    std::vector<std::string> opts = hiprtc_options(arch);
+    std::vector<const char*> copts;
+    for (const std::string& o : opts) copts.push_back(o.c_str());
+    r = hiprtcCompileProgram(prog, static_cast<int>(copts.size()), copts.data());
+    if (r != HIPRTC_SUCCESS) {
+        size_t log_size = 0;
+        hiprtcGetProgramLogSize(prog, &log_size);
+        std::string log(log_size, '\0');
+        if (log_size) hiprtcGetProgramLog(prog, &log[0]);
+        hiprtcDestroyProgram(&prog);
+        return set_error(dev, CUSTOS_HIP_ERR_COMPILE,
+                         std::string("hiprtcCompileProgram: ") + hiprtcGetErrorString(r) + "\n" + log +
+                             "\n--- source ---\n" + spec.source);
+    }
+    size_t size = 0;
+    hiprtcGetCodeSize(prog, &size);
+    code->resize(size);
+    hiprtcGetCode(prog, code->data());
+    hiprtcDestroyProgram(&prog);
+    return CUSTOS_HIP_OK;
+}
+
+bool markers_from_c(const char* const* markers, int32_t n, std::vector<std::string>* out) {
+    if (!markers || n < 1 || n > 4) return false;
+    for (int i = 0; i < n; i++) {
+        if (!markers[i] || !markers[i][0]) return false;
+        out->push_back(markers[i]);
+    }
+    return true;
+}
+
+int32_t spec_from_c(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
+                    const char* const* markers, int32_t n_markers, const Tuning& tuning,
+                    KernelSpec* spec) {
+    if (!src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");
+    if (kind != CUSTOS_HIP_KIND_APPLY && kind != CUSTOS_HIP_KIND_UNARY_GRAD)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown kernel kind");
+    if (!dtype_valid(dtype)) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown element type");
+    std::vector<std::string> m;
+    if (!markers_from_c(markers, n_markers, &m))
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 4 non-empty markers are required");
+    ParseError err;
+    if (!build_kernel_spec(static_cast<Kind>(kind), static_cast<DType>(dtype), src, m, tuning, spec, &err))
+        return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+    return CUSTOS_HIP_OK;
+}
+
+Tuning tuning_from_c(const custos_hip_tuning* t) {
+    if (!t) return normalize_tuning(0, 0, 0, 0);
+    return normalize_tuning(t->block_threads, t->unroll, t->blocks_per_cu, t->nontemporal);
+}
+
+int32_t copy_out_string(const std::string& s, char* buf, size_t cap, size_t* needed) {
+    if (needed) *needed = s.size() + 1;
+    if (buf && cap) {
+        size_t n = std::min(cap - 1, s.size());
+        std::memcpy(buf, s.data(), n);
+        buf[n] = '\0';
+    }
+    return CUSTOS_HIP_OK;
+}
+
+struct Range {
+    uint64_t ptr;
+    bool written;
+};
+
+// Checks operand addresses and computes how the element range splits into a
+// scalar head, 16-byte vectors and a scalar tail.
+int32_t plan_launch(custos_hip_device* dev, const custos_hip_kernel* k, const std::vector<Range>& ops,
+                    size_t n, unsigned long long* head, unsigned long long* n_vec, unsigned int* grid) {
+    const size_t es = dtype_size(k->spec.dtype);
+    if (n > (1ull << 40)) return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "more than 2^40 elements");
+    const uint64_t bytes = static_cast<uint64_t>(n) * es;
+    for (const Range& r : ops) {
+        if (r.ptr == 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null device pointer");
+        if (r.ptr % es) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "device pointer is not aligned to the element size");
+    }
+    for (const Range& w : ops) {
+        if (!w.written) continue;
+        for (const Range& r : ops) {
+            if (&r == &w || r.ptr == w.ptr) continue;
+            if (r.ptr < w.ptr + bytes && w.ptr < r.ptr + bytes)
+                return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP,
+                                 "the output range partially overlaps an input range");
+        }
+    }
+    bool same_phase = true;
+    for (const Range& r : ops) same_phase = same_phase && (r.ptr & 15) == (ops[0].ptr & 15);
+    unsigned long long h = 0, nv = 0;
+    if (same_phase) {
+        h = ((16 - (ops[0].ptr & 15)) & 15) / es;
+        if (h > n) h = n;
+        nv = (n - h) / k->spec.vec_elems;
+    }
+    const Tuning& t = k->spec.tuning;
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+    unsigned long long tiles = (nv + tile_vecs - 1) / tile_vecs;
+    unsigned long long scalar = n - nv * k->spec.vec_elems;
+    const unsigned long long cus = static_cast<unsigned long long>(dev->props.multiProcessorCount);
+    unsigned long long scalar_blocks = std::min((scalar + t.block_threads - 1) / t.block_threads, cus * 32);
+    if (t.blocks_per_cu > 0) tiles = std::min(tiles, cus * t.blocks_per_cu);
+    unsigned long long g = std::max(1ull, std::max(tiles, scalar_blocks));
+    g = std::min(g, 1ull << 22);
+    *head = h;
+    *n_vec = nv;
+    *grid = static_cast<unsigned int>(g);
+    return CUSTOS_HIP_OK;
+}
+
+int32_t launch(custos_hip_device* dev, custos_hip_kernel* k, std::vector<void*>& args, unsigned int grid) {
+    HIP_TRY(dev, hipModuleLaunchKernel(k->fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
+                                       1, 1, 0, dev->stream, args.data(), nullptr));
+    return CUSTOS_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t custos_hip_device_count(int32_t* count) {
+    if (!count) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "count is null");
+    int c = 0;
+    hipError_t e = hipGetDeviceCount(&c);
+    if (e != hipSuccess) {
+        *count = 0;
+        return hip_fail(nullptr, e, "hipGetDeviceCount");
+    }
+    *count = c;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_chosen_device_idx(void) {
+    const char* v = std::getenv("CUSTOS_HIP_DEVICE_IDX");
+    if (!v || !*v) return 0;
+    char* end = nullptr;
+    long idx = std::strtol(v, &end, 10);
+    if (*end != '\0' || idx < 0) return 0;
+    return static_cast<int32_t>(idx);
+}
+
+int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
+    if (!out) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "out handle is null");
+    *out = nullptr;
+    int count = 0;
+    HIP_TRY(nullptr, hipGetDeviceCount(&count));
+    if (idx < 0 || idx >= count)
+        return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_DEVICE_INDEX,
+                         "device index " + std::to_string(idx) + " out of range: " + std::to_string(count) + " device(s)");
+    std::unique_ptr<custos_hip_device> dev(new custos_hip_device);
+    dev->idx = idx;
+    HIP_TRY(nullptr, hipSetDevice(idx));
+    HIP_TRY(nullptr, hipGetDeviceProperties(&dev->props, idx));
+    dev->arch = dev->props.gcnArchName;
+    dev->tuning = normalize_tuning(0, 0, 0, 0);
+    HIP_TRY(nullptr, hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking));
+    HIP_TRY(nullptr, hipStreamCreateWithFlags(&dev->transfer, hipStreamNonBlocking));
+    HIP_TRY(nullptr, hipEventCreate(&dev->t0));
+    HIP_TRY(nullptr, hipEventCreate(&dev->t1));
+    *out = dev.release();
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_device_destroy(custos_hip_device* dev) {
+    if (!dev) return CUSTOS_HIP_OK;
+    (void)hipSetDevice(dev->idx);
+    if (dev->capturing) {
+        hipGraph_t g = nullptr;
+        (void)hipStreamEndCapture(dev->stream, &g);
+        if (g) (void)hipGraphDestroy(g);
+    }
+    (void)hipStreamSynchronize(dev->stream);
+    (void)hipStreamSynchronize(dev->transfer);
+    for (custos_hip_graph* g : dev->graphs) {
+        if (g->exec) (void)hipGraphExecDestroy(g->exec);
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        delete g;
+    }
+    for (auto& bucket : dev->cache)
+        for (auto& k : bucket.second)
+            if (k->module) (void)hipModuleUnload(k->module);
+    (void)hipEventDestroy(dev->t0);
+    (void)hipEventDestroy(dev->t1);
+    (void)hipStreamDestroy(dev->stream);
+    (void)hipStreamDestroy(dev->transfer);
+    delete dev;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_get_device_info(custos_hip_device* dev, custos_hip_device_info* info) {
+    REQUIRE_DEV(dev);
+    if (!info) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "info is null");
+    std::memset(info, 0, sizeof *info);
+    std::snprintf(info->name, sizeof info->name, "%s", dev->props.name);
+    std::snprintf(info->arch, sizeof info->arch, "%s", dev->props.gcnArchName);
+    info->compute_units = dev->props.multiProcessorCount;
+    info->wavefront_size = dev->props.warpSize;
+    info->clock_khz = dev->props.clockRate;
+    info->memory_clock_khz = dev->props.memoryClockRate;
+    info->memory_bus_bits = dev->props.memoryBusWidth;
+    info->l2_bytes = dev->props.l2CacheSize;
+    info->total_memory = dev->props.totalGlobalMem;
+    return CUSTOS_HIP_OK;
+}
+
+const char* custos_hip_last_error(custos_hip_device* dev) {
+    return dev ? dev->last_error.c_str() : g_last_error.c_str();
+}
+
+int32_t custos_hip_sync(custos_hip_device* dev) {
+    REQUIRE_DEV(dev);
+    if (dev->capturing)
+        return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot wait for a stream that is recording");
+    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_tuning(custos_hip_device* dev, const custos_hip_tuning* tuning) {
+    REQUIRE_DEV(dev);
+    dev->tuning = tuning_from_c(tuning);
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_get_tuning(custos_hip_device* dev, custos_hip_tuning* tuning) {
+    REQUIRE_DEV(dev);
+    if (!tuning) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "tuning is null");
+    tuning->block_threads = dev->tuning.block_threads;
+    tuning->unroll = dev->tuning.unroll;
+    tuning->blocks_per_cu = dev->tuning.blocks_per_cu;
+    tuning->nontemporal = dev->tuning.nontemporal;
+    return CUSTOS_HIP_OK;
+}
+
+// ---- memory ----
+
+int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, uint64_t* dptr) {
+    REQUIRE_DEV(dev);
+    if (!dptr) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "dptr is null");
+    *dptr = 0;
+    if (bytes == 0) return set_error(dev, CUSTOS_HIP_ERR_ZERO_LENGTH_BUFFER, "zero length buffers are not supported");
+    void* p = nullptr;
+    HIP_TRY(dev, hipMalloc(&p, bytes));
+    uint64_t addr = reinterpret_cast<uint64_t>(p);
+    if (flags != CUSTOS_HIP_ALLOC_UNINIT) {
+        // While recording, the fill must run now and not become part of the graph.
+        hipStream_t s = dev->capturing ? dev->transfer : dev->stream;
+        int32_t rc = launch_fill_zero(dev, addr, bytes, s);
+        if (rc == CUSTOS_HIP_OK && dev->capturing) {
+            hipError_t e = hipStreamSynchronize(dev->transfer);
+            if (e != hipSuccess) rc = hip_fail(dev, e, "hipStreamSynchronize(transfer)");
+        }
+        if (rc != CUSTOS_HIP_OK) {
+            (void)hipFree(p);
+            return rc;
+        }
+    }
+    *dptr = addr;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_free(custos_hip_device* dev, uint64_t dptr) {
+    REQUIRE_DEV(dev);
+    if (dptr == 0) return CUSTOS_HIP_OK;
+    // work that still uses the range must finish first
+    if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    HIP_TRY(dev, hipFree(reinterpret_cast<void*>(dptr)));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_write(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    if (dev->capturing) {
+        HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), src, bytes, hipMemcpyHostToDevice, dev->transfer));
+        HIP_TRY(dev, hipStreamSynchronize(dev->transfer));
+        return CUSTOS_HIP_OK;
+    }
+    HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), src, bytes, hipMemcpyHostToDevice, dev->stream));
+    // the caller may reuse `src` right away
+    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_read(custos_hip_device* dev, void* dst, uint64_t src, size_t bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    HIP_TRY(dev, hipMemcpyAsync(dst, reinterpret_cast<const void*>(src), bytes, hipMemcpyDeviceToHost, dev->transfer));
+    HIP_TRY(dev, hipStreamSynchronize(dev->transfer));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src), bytes,
+                                hipMemcpyDeviceToDevice, dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_clear(custos_hip_device* dev, uint64_t dptr, size_t bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dptr) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    return launch_fill_zero(dev, dptr, bytes, dev->stream);
+}
+
+// ---- expression kernels ----
+
+int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
+                                const char* const* markers, int32_t n_markers,
+                                custos_hip_kernel** kernel) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "kernel out pointer is null");
+    *kernel = nullptr;
+    std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
+    int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, dev->tuning, &k->spec);
+    if (rc != CUSTOS_HIP_OK) return rc;
+
+    auto& bucket = dev->cache[k->spec.hash];
+    for (auto& cached : bucket) {
+        // the generated text starts with the caller's spelling of the expression
+        // as a comment; compare what is compiled, i.e. everything after it
+        const std::string& a = cached->spec.source;
+        const std::string& b = k->spec.source;
+        if (a.compare(a.find('\n'), std::string::npos, b, b.find('\n'), std::string::npos) == 0) {
+            dev->hits++;
+            *kernel = cached.get();
+            return CUSTOS_HIP_OK;
+        }
+    }
+    std::vector<char> code;
+    rc = compile_to_code_object(dev, k->spec, dev->arch, &code);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    HIP_TRY(dev, hipModuleLoadData(&k->module, code.data()));
+    hipError_t e = hipModuleGetFunction(&k->fn, k->module, kKernelName);
+    if (e != hipSuccess) {
+        (void)hipModuleUnload(k->module);
+        return hip_fail(dev, e, "hipModuleGetFunction");
+    }
+    dev->compiles++;
+    *kernel = k.get();
+    bucket.push_back(std::move(k));
+    return CUSTOS_HIP_OK;
+}
+
+const char* custos_hip_kernel_source(const custos_hip_kernel* kernel) {
+    return kernel ? kernel->spec.source.c_str() : "";
+}
+
+uint64_t custos_hip_kernel_hash(const custos_hip_kernel* kernel) { return kernel ? kernel->spec.hash : 0; }
+
+int32_t custos_hip_kernel_arity(const custos_hip_kernel* kernel) {
+    return kernel ? kernel->spec.expr.n_vars : 0;
+}
+
+int32_t custos_hip_cache_stats(custos_hip_device* dev, uint64_t* compiles, uint64_t* hits) {
+    REQUIRE_DEV(dev);
+    if (compiles) *compiles = dev->compiles;
+    if (hits) *hits = dev->hits;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_expr_emit(int32_t kind, int32_t dtype, const char* src, const char* const* markers,
+                             int32_t n_markers, const custos_hip_tuning* tuning, char* buf, size_t cap,
+                             size_t* needed, uint64_t* hash) {
+    KernelSpec spec;
+    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), &spec);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    if (hash) *hash = spec.hash;
+    return copy_out_string(spec.source, buf, cap, needed);
+}
+
+int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const char* src,
+                                          const char* const* markers, int32_t n_markers,
+                                          const custos_hip_tuning* tuning, size_t* code_size) {
+    KernelSpec spec;
+    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), &spec);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    std::vector<char> code;
+    rc = compile_to_code_object(nullptr, spec, "gfx950", &code);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    if (code_size) *code_size = code.size();
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_expr_canonical(const char* src, const char* const* markers, int32_t n_markers,
+                                  char* buf, size_t cap, size_t* needed) {
+    if (!src) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");
+    std::vector<std::string> m;
+    if (!markers_from_c(markers, n_markers, &m))
+        return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 4 non-empty markers are required");
+    Expr e;
+    ParseError err;
+    if (!parse_expr(src, m, &e, &err)) return set_error(nullptr, err.code, err.message);
+    return copy_out_string(to_cl_source(e, m), buf, cap, needed);
+}
+
+// ---- launches ----
+
+int32_t custos_hip_apply_fn_n(custos_hip_device* dev, custos_hip_kernel* kernel, const uint64_t* ins,
+                              int32_t n_ins, uint64_t out, size_t n) {
+    REQUIRE_DEV(dev);
+    if (!kernel || !ins) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel or operand list");
+    if (kernel->spec.kind != Kind::Apply)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled as an apply kernel");
+    if (n_ins != kernel->spec.expr.n_vars)
+        return set_error(dev, CUSTOS_HIP_ERR_ARITY_MISMATCH,
+                         "kernel takes " + std::to_string(kernel->spec.expr.n_vars) + " operand(s), got " + std::to_string(n_ins));
+    if (n == 0) return CUSTOS_HIP_OK;
+    std::vector<Range> ops;
+    for (int i = 0; i < n_ins; i++) ops.push_back({ins[i], false});
+    ops.push_back({out, true});
+    unsigned long long head, n_vec, count = n;
+    unsigned int grid;
+    int32_t rc = plan_launch(dev, kernel, ops, n, &head, &n_vec, &grid);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    uint64_t ptrs[5];
+    std::vector<void*> args;
+    for (int i = 0; i < n_ins; i++) {
+        ptrs[i] = ins[i];
+        args.push_back(&ptrs[i]);
+    }
+    ptrs[4] = out;
+    args.push_back(&ptrs[4]);
+    args.push_back(&count);
+    args.push_back(&head);
+    args.push_back(&n_vec);
+    return launch(dev, kernel, args, grid);
+}
+
+int32_t custos_hip_apply_fn(custos_hip_device* dev, custos_hip_kernel* kernel, uint64_t x, uint64_t out, size_t n) {
+    return custos_hip_apply_fn_n(dev, kernel, &x, 1, out, n);
+}
+
+int32_t custos_hip_apply_fn2(custos_hip_device* dev, custos_hip_kernel* kernel, uint64_t lhs, uint64_t rhs,
+                             uint64_t out, size_t n) {
+    uint64_t ins[2] = {lhs, rhs};
+    return custos_hip_apply_fn_n(dev, kernel, ins, 2, out, n);
+}
+
+int32_t custos_hip_add_unary_grad(custos_hip_device* dev, custos_hip_kernel* kernel, uint64_t lhs,
+                                  uint64_t lhs_grad, uint64_t out_grad, size_t n) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel");
+    if (kernel->spec.kind != Kind::UnaryGrad)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled as a unary-gradient kernel");
+    if (n == 0) return CUSTOS_HIP_OK;
+    std::vector<Range> ops = {{lhs, false}, {lhs_grad, true}, {out_grad, false}};
+    unsigned long long head, n_vec, count = n;
+    unsigned int grid;
+    int32_t rc = plan_launch(dev, kernel, ops, n, &head, &n_vec, &grid);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    std::vector<void*> args = {&lhs, &lhs_grad, &out_grad, &count, &head, &n_vec};
+    return launch(dev, kernel, args, grid);
+}
+
+// ---- capture / replay ----
+
+int32_t custos_hip_capture_begin(custos_hip_device* dev) {
+    REQUIRE_DEV(dev);
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the stream is already recording");
+    // relaxed: allocation, reads and writes stay legal while recording; they are
+    // issued on the transfer stream and are not part of the graph
+    HIP_TRY(dev, hipStreamBeginCapture(dev->stream, hipStreamCaptureModeRelaxed));
+    dev->capturing = true;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_capture_end(custos_hip_device* dev, custos_hip_graph** graph) {
+    REQUIRE_DEV(dev);
+    if (!graph) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph out pointer is null");
+    *graph = nullptr;
+    if (!dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the stream is not recording");
+    dev->capturing = false;
+    std::unique_ptr<custos_hip_graph> g(new custos_hip_graph);
+    HIP_TRY(dev, hipStreamEndCapture(dev->stream, &g->graph));
+    if (!g->graph) HIP_TRY(dev, hipGraphCreate(&g->graph, 0));  // nothing was recorded
+    size_t n_nodes = 0;
+    HIP_TRY(dev, hipGraphGetNodes(g->graph, nullptr, &n_nodes));
+    if (n_nodes) {
+        std::vector<hipGraphNode_t> nodes(n_nodes);
+        HIP_TRY(dev, hipGraphGetNodes(g->graph, nodes.data(), &n_nodes));
+        for (hipGraphNode_t node : nodes) {
+            hipGraphNodeType type;
+            if (hipGraphNodeGetType(node, &type) == hipSuccess && type == hipGraphNodeTypeKernel) g->kernel_nodes++;
+        }
+    }
+    hipError_t e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g->graph);
+        return hip_fail(dev, e, "hipGraphInstantiate");
+    }
+    dev->graphs.push_back(g.get());
+    *graph = g.release();
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_is_capturing(custos_hip_device* dev, int32_t* capturing) {
+    REQUIRE_DEV(dev);
+    if (!capturing) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "capturing is null");
+    *capturing = dev->capturing ? 1 : 0;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_launch(custos_hip_device* dev, custos_hip_graph* graph) {
+    REQUIRE_DEV(dev);
+    if (!graph) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph is null");
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot replay while recording");
+    HIP_TRY(dev, hipGraphLaunch(graph->exec, dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_node_count(custos_hip_graph* graph, size_t* kernel_nodes) {
+    if (!graph || !kernel_nodes) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    *kernel_nodes = graph->kernel_nodes;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_destroy(custos_hip_device* dev, custos_hip_graph* graph) {
+    REQUIRE_DEV(dev);
+    if (!graph) return CUSTOS_HIP_OK;
+    auto it = std::find(dev->graphs.begin(), dev->graphs.end(), graph);
+    if (it == dev->graphs.end()) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph does not belong to this device");
+    dev->graphs.erase(it);
+    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    delete graph;
+    return CUSTOS_HIP_OK;
+}
+
+// ---- timing ----
+
+int32_t custos_hip_timer_begin(custos_hip_device* dev) {
+    REQUIRE_DEV(dev);
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot time a recording stream");
+    HIP_TRY(dev, hipEventRecord(dev->t0, dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_timer_end(custos_hip_device* dev, double* ms) {
+    REQUIRE_DEV(dev);
+    if (!ms) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "ms is null");
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot time a recording stream");
+    HIP_TRY(dev, hipEventRecord(dev->t1, dev->stream));
+    HIP_TRY(dev, hipEventSynchronize(dev->t1));
+    float f = 0.f;
+    HIP_TRY(dev, hipEventElapsedTime(&f, dev->t0, dev->t1));
+    *ms = f;
+    return CUSTOS_HIP_OK;
+}
+
+}  // extern "C"

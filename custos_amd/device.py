@@ -1,0 +1,251 @@
+"""`HIP` device over the C ABI with the call contract of custos' device traits.
+
+Mirrors, for the element-wise path, what `CUDA<Base>` offers in the reference:
+`buffer` / `read` / `write` / `clear` (src/devices/cuda/ops.rs:17-117),
+`apply_fn` (src/unary.rs:7-28, src/devices/cuda/ops.rs:119-141),
+`add_unary_grad` (src/unary.rs:31-58, src/devices/cuda/ops.rs:179-199), the
+fused unary op (src/devices/cuda/fusing.rs:3-51) and graph capture / replay
+(src/devices/cuda/lazy.rs:10-72).  All arithmetic happens in the HIP kernels.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+from .expr import Expr, Resolve, _wrap, fused_source
+
+
+def _np_dtype(dtype: str):
+    return np.dtype(capi.DTYPES[dtype][1])
+
+
+class Buffer:
+    """A device allocation of `len` elements (`Buffer<T, HIP>` with `CUDAPtr`-like
+    base: address, length, ownership flag -- src/devices/cuda/cuda_ptr.rs:7-15)."""
+
+    def __init__(self, device: "HIP", ptr: int, length: int, dtype: str, owned: bool = True):
+        self.device = device
+        self.ptr = ptr
+        self.len = length
+        self.dtype = dtype
+        self.owned = owned
+
+    def __len__(self):
+        return self.len
+
+    @property
+    def id(self) -> int:
+        return self.ptr
+
+    @property
+    def nbytes(self) -> int:
+        return self.len * _np_dtype(self.dtype).itemsize
+
+    def read(self) -> np.ndarray:
+        return self.device.read(self)
+
+    def write(self, data) -> None:
+        self.device.write(self, data)
+
+    def clear(self) -> None:
+        self.device.clear(self)
+
+    def slice(self, start: int, stop: int) -> "Buffer":
+        """Non-owning view of elements [start, stop)."""
+        if not (0 <= start <= stop <= self.len):
+            raise IndexError("slice out of range")
+        item = _np_dtype(self.dtype).itemsize
+        return Buffer(self.device, self.ptr + start * item, stop - start, self.dtype, owned=False)
+
+    def free(self) -> None:
+        if self.owned and self.ptr and self.device is not None and self.device.handle:
+            self.device._check(self.device.lib.custos_hip_free(self.device.handle, self.ptr))
+        self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Graph:
+    """An instantiated, replayable capture (`LazyCudaGraph`, src/devices/cuda/lazy.rs:10-29)."""
+
+    def __init__(self, device: "HIP", handle):
+        self.device = device
+        self.handle = handle
+
+    def launch(self) -> None:
+        self.device._check(self.device.lib.custos_hip_graph_launch(self.device.handle, self.handle))
+
+    @property
+    def kernel_nodes(self) -> int:
+        n = C.c_size_t(0)
+        self.device._check(self.device.lib.custos_hip_graph_node_count(self.handle, C.byref(n)))
+        return n.value
+
+    def destroy(self) -> None:
+        if self.handle and self.device.handle:
+            self.device._check(self.device.lib.custos_hip_graph_destroy(self.device.handle, self.handle))
+        self.handle = None
+
+
+class HIP:
+    """`HIP::<Base>::new(idx)`: eager execution, plain allocation."""
+
+    def __init__(self, idx: int | None = None):
+        self.lib = capi.load_library()
+        self.handle = None
+        if idx is None:
+            idx = self.lib.custos_hip_chosen_device_idx()
+        h = C.c_void_p()
+        capi.check(self.lib.custos_hip_device_create(idx, C.byref(h)))
+        self.handle = h
+
+    # -- plumbing --
+    def _check(self, rc: int) -> None:
+        capi.check(rc, self.handle)
+
+    def close(self) -> None:
+        if self.handle:
+            self.lib.custos_hip_device_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def info(self) -> capi.DeviceInfo:
+        info = capi.DeviceInfo()
+        self._check(self.lib.custos_hip_get_device_info(self.handle, C.byref(info)))
+        return info
+
+    def sync(self) -> None:
+        self._check(self.lib.custos_hip_sync(self.handle))
+
+    def set_tuning(self, block_threads=0, unroll=0, blocks_per_cu=0, nontemporal=0) -> None:
+        t = capi.Tuning(block_threads, unroll, blocks_per_cu, nontemporal)
+        self._check(self.lib.custos_hip_set_tuning(self.handle, C.byref(t)))
+
+    def cache_stats(self):
+        a, b = C.c_uint64(0), C.c_uint64(0)
+        self._check(self.lib.custos_hip_cache_stats(self.handle, C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    # -- Alloc / Read / WriteBuf / ClearBuf --
+    def alloc(self, length: int, dtype: str = "f32", zeroed: bool = True) -> Buffer:
+        ptr = C.c_uint64(0)
+        nbytes = length * _np_dtype(dtype).itemsize
+        flags = capi.ALLOC_ZEROED if zeroed else capi.ALLOC_UNINIT
+        self._check(self.lib.custos_hip_alloc(self.handle, nbytes, flags, C.byref(ptr)))
+        return Buffer(self, ptr.value, length, dtype)
+
+    def buffer(self, data, dtype: str = "f32") -> Buffer:
+        """`device.buffer([...])` / `Buffer::from((&device, slice))`."""
+        arr = np.ascontiguousarray(data, dtype=_np_dtype(dtype))
+        buf = self.alloc(arr.size, dtype, zeroed=False)
+        self.write(buf, arr)
+        return buf
+
+    def write(self, buf: Buffer, data) -> None:
+        arr = np.ascontiguousarray(data, dtype=_np_dtype(buf.dtype))
+        if arr.size != buf.len:
+            raise ValueError(f"write of {arr.size} elements into a buffer of {buf.len}")
+        self._check(self.lib.custos_hip_write(self.handle, buf.ptr, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
+
+    def read(self, buf: Buffer) -> np.ndarray:
+        out = np.empty(buf.len, dtype=_np_dtype(buf.dtype))
+        self._check(self.lib.custos_hip_read(self.handle, out.ctypes.data_as(C.c_void_p), buf.ptr, out.nbytes))
+        return out
+
+    def clear(self, buf: Buffer) -> None:
+        self._check(self.lib.custos_hip_clear(self.handle, buf.ptr, buf.nbytes))
+
+    def copy(self, dst: Buffer, src: Buffer) -> None:
+        if dst.nbytes != src.nbytes:
+            raise ValueError("size mismatch")
+        self._check(self.lib.custos_hip_copy(self.handle, dst.ptr, src.ptr, src.nbytes))
+
+    # -- kernels --
+    def compile(self, kind: int, dtype: str, src: str, markers=("x",)):
+        arr, n = capi.c_markers(list(markers))
+        k = C.c_void_p()
+        self._check(self.lib.custos_hip_expr_compile(self.handle, kind, capi.DTYPES[dtype][0], src.encode(), arr, n, C.byref(k)))
+        return k
+
+    def kernel_source(self, kernel) -> str:
+        return self.lib.custos_hip_kernel_source(kernel).decode()
+
+    def apply_fn(self, buf: Buffer, f, out: Buffer | None = None) -> Buffer:
+        """`device.apply_fn(&buf, |x| ...)`: out[i] = f(buf[i]) in a new buffer."""
+        src = _wrap(f(Resolve("x"))).to_cl_source(buf.dtype)
+        kernel = self.compile(capi.KIND_APPLY, buf.dtype, src, ("x",))
+        if out is None:
+            out = self.alloc(buf.len, buf.dtype, zeroed=False)
+        self._check(self.lib.custos_hip_apply_fn(self.handle, kernel, buf.ptr, out.ptr, buf.len))
+        return out
+
+    def apply_fn2(self, lhs: Buffer, rhs: Buffer, f, out: Buffer | None = None) -> Buffer:
+        """Two-operand expression: out[i] = f(lhs[i], rhs[i])."""
+        if lhs.len != rhs.len or lhs.dtype != rhs.dtype:
+            raise ValueError("operands differ in length or element type")
+        src = _wrap(f(Resolve("x", 0), Resolve("y", 1))).to_cl_source(lhs.dtype)
+        kernel = self.compile(capi.KIND_APPLY, lhs.dtype, src, ("x", "y"))
+        if out is None:
+            out = self.alloc(lhs.len, lhs.dtype, zeroed=False)
+        self._check(self.lib.custos_hip_apply_fn2(self.handle, kernel, lhs.ptr, rhs.ptr, out.ptr, lhs.len))
+        return out
+
+    def apply_fn_n(self, ins, f, out: Buffer | None = None) -> Buffer:
+        """k-operand expression (k <= 4) over markers a, b, c, d."""
+        names = ("a", "b", "c", "d")[: len(ins)]
+        src = _wrap(f(*[Resolve(n, i) for i, n in enumerate(names)])).to_cl_source(ins[0].dtype)
+        kernel = self.compile(capi.KIND_APPLY, ins[0].dtype, src, names)
+        if out is None:
+            out = self.alloc(ins[0].len, ins[0].dtype, zeroed=False)
+        ptrs = (C.c_uint64 * len(ins))(*[b.ptr for b in ins])
+        self._check(self.lib.custos_hip_apply_fn_n(self.handle, kernel, ptrs, len(ins), out.ptr, ins[0].len))
+        return out
+
+    def fused_apply_fn(self, buf: Buffer, ops, out: Buffer | None = None) -> Buffer:
+        """The op `unary_fuse_op` returns: all `ops` applied in sequence in one kernel."""
+        src = fused_source(ops, buf.dtype)
+        kernel = self.compile(capi.KIND_APPLY, buf.dtype, src, ("x",))
+        if out is None:
+            out = self.alloc(buf.len, buf.dtype, zeroed=False)
+        self._check(self.lib.custos_hip_apply_fn(self.handle, kernel, buf.ptr, out.ptr, buf.len))
+        return out
+
+    def add_unary_grad(self, lhs: Buffer, lhs_grad: Buffer, out_grad: Buffer, lhs_grad_fn) -> None:
+        """`device.add_unary_grad(&lhs, &mut lhs_grad, &out_grad, |x| ...)`."""
+        src = _wrap(lhs_grad_fn(Resolve("x"))).to_cl_source(lhs.dtype)
+        kernel = self.compile(capi.KIND_UNARY_GRAD, lhs.dtype, src, ("x",))
+        self._check(self.lib.custos_hip_add_unary_grad(self.handle, kernel, lhs.ptr, lhs_grad.ptr, out_grad.ptr, lhs.len))
+
+    # -- capture / replay --
+    def capture_begin(self) -> None:
+        self._check(self.lib.custos_hip_capture_begin(self.handle))
+
+    def capture_end(self) -> Graph:
+        g = C.c_void_p()
+        self._check(self.lib.custos_hip_capture_end(self.handle, C.byref(g)))
+        return Graph(self, g)
+
+    def is_capturing(self) -> bool:
+        v = C.c_int32(0)
+        self._check(self.lib.custos_hip_is_capturing(self.handle, C.byref(v)))
+        return bool(v.value)
+
+    # -- timing --
+    def timer_begin(self) -> None:
+        self._check(self.lib.custos_hip_timer_begin(self.handle))
+
+    def timer_end(self) -> float:
+        ms = C.c_double(0)
+        self._check(self.lib.custos_hip_timer_end(self.handle, C.byref(ms)))
+        return ms.value

@@ -1,0 +1,233 @@
+/*
+ * custos_hip.h -- C ABI of the MI355X (gfx950) element-wise backend for custos.
+ *
+ * This is the boundary a custos `HIP<Mods>` device binds through FFI.  It
+ * covers what the reference's CUDA device reaches through its own driver
+ * wrappers (src/devices/cuda/api/ffi.rs:165-264, api/nvrtc/ffi.rs:36-54) for
+ * the element-wise path: device memory, expression kernels compiled at run
+ * time, the three launches (apply / two-operand apply / unary gradient) and
+ * graph capture + replay for `Lazy`.
+ *
+ * Conventions
+ *   - every function returns a status: 0 on success, a HIP error number
+ *     (hipError_t, 1..9999) or a library code (>= 10000, see below).
+ *     `custos_hip_last_error` returns a message for the last failure.
+ *   - handles are opaque; a device handle and everything created from it is
+ *     used by one thread at a time (the reference's devices are `!Sync`:
+ *     RefCell state in src/devices/cuda/cuda_device.rs:14-29).
+ *   - device pointers are `uint64_t` addresses, so a buffer id can be the
+ *     address as in src/devices/cuda/cuda_ptr.rs:44-49.  Sub-ranges of an
+ *     allocation (address + offset) are accepted wherever a pointer is.
+ *   - all work is issued on the device handle's compute stream, in call order.
+ */
+#ifndef CUSTOS_HIP_H
+#define CUSTOS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct custos_hip_device custos_hip_device;
+typedef struct custos_hip_kernel custos_hip_kernel;
+typedef struct custos_hip_graph custos_hip_graph;
+
+/* Library status codes (HIP's own error numbers stay below 10000). */
+enum custos_hip_status {
+    CUSTOS_HIP_OK = 0,
+    CUSTOS_HIP_ERR_INVALID_ARGUMENT = 10001,
+    /* zero-byte allocation: src/devices/cuda/api/cuda.rs:69-71,
+     * DeviceError::ZeroLengthBuffer (src/error.rs) */
+    CUSTOS_HIP_ERR_ZERO_LENGTH_BUFFER = 10002,
+    /* device index out of range: src/devices/cuda/api/cuda.rs:36-39 */
+    CUSTOS_HIP_ERR_INVALID_DEVICE_INDEX = 10003,
+    CUSTOS_HIP_ERR_EXPR_SYNTAX = 10010,      /* expression text does not follow the grammar */
+    CUSTOS_HIP_ERR_EXPR_UNKNOWN_MARKER = 10011,
+    CUSTOS_HIP_ERR_EXPR_UNSUPPORTED = 10012, /* node not defined for the element type */
+    CUSTOS_HIP_ERR_COMPILE = 10020,          /* hiprtc rejected the generated kernel */
+    CUSTOS_HIP_ERR_KIND_MISMATCH = 10030,    /* kernel launched through the wrong entry point */
+    CUSTOS_HIP_ERR_ARITY_MISMATCH = 10031,
+    CUSTOS_HIP_ERR_CAPTURE_STATE = 10040,    /* begin while capturing / end while not / op illegal in capture */
+    CUSTOS_HIP_ERR_BAD_OVERLAP = 10050,      /* output partially overlaps an input */
+    CUSTOS_HIP_ERR_TOO_LARGE = 10060
+};
+
+/* Element types: the reference's CDatatype list (src/devices/cdatatype.rs:7-62).
+ * F16 / BF16 are storage types: values are widened to f32, the whole expression
+ * is computed in f32 and rounded once (nearest even) at the store. */
+enum custos_hip_dtype {
+    CUSTOS_HIP_F32 = 0,
+    CUSTOS_HIP_F64 = 1,
+    CUSTOS_HIP_I32 = 2,
+    CUSTOS_HIP_I64 = 3,
+    CUSTOS_HIP_F16 = 4,
+    CUSTOS_HIP_BF16 = 5,
+    CUSTOS_HIP_U8 = 6,
+    CUSTOS_HIP_I8 = 7,
+    CUSTOS_HIP_I16 = 8,
+    CUSTOS_HIP_U16 = 9,
+    CUSTOS_HIP_U32 = 10,
+    CUSTOS_HIP_U64 = 11
+};
+
+/* Kernel kinds. */
+enum custos_hip_kind {
+    /* out[i] = f(in0[i], .., in{k-1}[i]), k = number of markers (1..4).
+     * One marker: `applyFn` (src/devices/cuda/ops.rs:144-177) and, when the
+     * source is a statement list "x = ..;\n x = ..;\n", the fused unary chain
+     * (src/devices/cuda/fusing.rs:21-48, src/devices/fusing.rs:4-19).
+     * Two markers: the two-operand expressions of src/two_way_ops/mod.rs:96-104. */
+    CUSTOS_HIP_KIND_APPLY = 0,
+    /* lhs_grad[i] += out_grad[i] * f(lhs[i]): `addUnaryGrad`
+     * (src/devices/cuda/ops.rs:201-234). One marker. */
+    CUSTOS_HIP_KIND_UNARY_GRAD = 1
+};
+
+/* Allocation flags. */
+enum custos_hip_alloc_flags {
+    CUSTOS_HIP_ALLOC_ZEROED = 0,  /* like CPU alloc (src/devices/cpu/cpu_ptr.rs:74-85) */
+    CUSTOS_HIP_ALLOC_UNINIT = 1   /* like CUDAPtr::new (src/devices/cuda/cuda_ptr.rs:21-30) */
+};
+
+typedef struct custos_hip_device_info {
+    char name[128];
+    char arch[64];           /* e.g. "gfx950:sramecc+:xnack-" */
+    int32_t compute_units;
+    int32_t wavefront_size;
+    int32_t clock_khz;
+    int32_t memory_clock_khz;
+    int32_t memory_bus_bits;
+    int32_t l2_bytes;
+    uint64_t total_memory;
+} custos_hip_device_info;
+
+/* Launch shape knobs of the generated kernels.  Zero fields keep the default.
+ * They are part of the kernel cache key. */
+typedef struct custos_hip_tuning {
+    int32_t block_threads;   /* threads per workgroup (multiple of 64), default 256 */
+    int32_t unroll;          /* 16-byte vectors per thread per tile, default 4 */
+    int32_t blocks_per_cu;   /* > 0: persistent grid of CUs*blocks_per_cu workgroups that
+                                stride over the tiles; <= 0 (default): one tile per workgroup */
+    int32_t nontemporal;     /* bit 0: non-temporal loads, bit 1: non-temporal stores; -1 = off */
+} custos_hip_tuning;
+
+/* ---- device (src/devices/cuda/cuda.rs:53-67, cuda_device.rs:31-128) ---- */
+
+int32_t custos_hip_device_count(int32_t *count);
+/* Creates the handle: selects device `idx`, creates the compute stream.
+ * The reference reads the index from CUSTOS_CU_DEVICE_IDX
+ * (src/devices/cuda/mod.rs:35-42); callers here may read CUSTOS_HIP_DEVICE_IDX
+ * with custos_hip_chosen_device_idx. */
+int32_t custos_hip_device_create(int32_t idx, custos_hip_device **dev);
+int32_t custos_hip_device_destroy(custos_hip_device *dev);
+int32_t custos_hip_chosen_device_idx(void);
+int32_t custos_hip_get_device_info(custos_hip_device *dev, custos_hip_device_info *info);
+/* Message of the last failed call on `dev`; with dev == NULL, of the last
+ * failed call of this thread that had no device (create, emit). */
+const char *custos_hip_last_error(custos_hip_device *dev);
+/* Blocks until the compute stream is idle (Stream::sync, src/devices/cuda/api/cuda.rs). */
+int32_t custos_hip_sync(custos_hip_device *dev);
+int32_t custos_hip_set_tuning(custos_hip_device *dev, const custos_hip_tuning *tuning);
+int32_t custos_hip_get_tuning(custos_hip_device *dev, custos_hip_tuning *tuning);
+
+/* ---- memory (src/devices/cuda/cuda.rs:114-138, cuda_ptr.rs:21-77, ops.rs:17-117) ---- */
+
+/* Alloc::alloc.  bytes == 0 fails with ZERO_LENGTH_BUFFER. */
+int32_t custos_hip_alloc(custos_hip_device *dev, size_t bytes, int32_t flags, uint64_t *dptr);
+/* Drop of an owning CUDAPtr (src/devices/cuda/cuda_ptr.rs:64-77). 0 is ignored. */
+int32_t custos_hip_free(custos_hip_device *dev, uint64_t dptr);
+/* WriteBuf::write: host -> device, ordered on the compute stream; the host
+ * range may be reused as soon as the call returns. */
+int32_t custos_hip_write(custos_hip_device *dev, uint64_t dst, const void *src, size_t bytes);
+/* Read::read: waits for the compute stream unless it is capturing, then copies
+ * device -> host and waits for the copy (src/devices/cuda/ops.rs:32-48). */
+int32_t custos_hip_read(custos_hip_device *dev, void *dst, uint64_t src, size_t bytes);
+/* WriteBuf::write_buf / CopySlice / CloneBuf: device -> device. */
+int32_t custos_hip_copy(custos_hip_device *dev, uint64_t dst, uint64_t src, size_t bytes);
+/* ClearBuf::clear / ZeroGrad::zero_grad (`cu_clear`, src/devices/cuda/mod.rs:59-74).
+ * Implemented as a fill kernel, so it may be captured into a graph. */
+int32_t custos_hip_clear(custos_hip_device *dev, uint64_t dptr, size_t bytes);
+
+/* ---- expression kernels (src/devices/cuda/kernel_cache.rs:10-73, source.rs:21-66) ---- */
+
+/*
+ * Compiles (or fetches from the cache) the kernel for one expression.
+ *
+ * `src` is the text custos' `ToCLSource` produces (src/two_way_ops/ops.rs,
+ * ops/unary.rs, ops/cmps.rs), e.g. "((x * 2.0) + 1.0)", "pow((x * 3.0), (y + 1.0))",
+ * "-(tan(x))", or a fused body "x = sin(x);\nx = (x * 2.0);\n"
+ * (src/devices/fusing.rs:4-19).  `markers[k]` is the name the caller gave to
+ * operand k (`Resolve::marker`, src/two_way_ops/resolve.rs:25-30); an index
+ * suffix as in "x[idx]" is part of the name.
+ * Numeric literals take the element type (a "2.0" in an f32 expression is the
+ * f32 2.0), nothing is contracted into fma and no fast-math is applied, so
+ * + - * / compare min max abs neg are bit-identical to the CPU device.
+ * Kernels are cached per device by (expression structure, dtype, kind,
+ * tuning): the same expression is compiled once.
+ * The kernel handle stays valid until the device is destroyed.
+ */
+int32_t custos_hip_expr_compile(custos_hip_device *dev, int32_t kind, int32_t dtype,
+                                const char *src, const char *const *markers, int32_t n_markers,
+                                custos_hip_kernel **kernel);
+/* Generated HIP source of a kernel, its 64-bit cache key and its arity. */
+const char *custos_hip_kernel_source(const custos_hip_kernel *kernel);
+uint64_t custos_hip_kernel_hash(const custos_hip_kernel *kernel);
+int32_t custos_hip_kernel_arity(const custos_hip_kernel *kernel);
+/* Number of hiprtc compilations / cache hits since the device was created. */
+int32_t custos_hip_cache_stats(custos_hip_device *dev, uint64_t *compiles, uint64_t *hits);
+
+/* Host-only helpers (no GPU needed): parse + emit the HIP source of a kernel
+ * into `buf` (`*needed` = bytes including the terminator), and run the hiprtc
+ * compilation for gfx950 without loading the result (`*code_size` = bytes). */
+int32_t custos_hip_expr_emit(int32_t kind, int32_t dtype, const char *src,
+                             const char *const *markers, int32_t n_markers,
+                             const custos_hip_tuning *tuning, char *buf, size_t cap,
+                             size_t *needed, uint64_t *hash);
+int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const char *src,
+                                          const char *const *markers, int32_t n_markers,
+                                          const custos_hip_tuning *tuning, size_t *code_size);
+/* Canonical re-print of an expression in the reference's ToCLSource format. */
+int32_t custos_hip_expr_canonical(const char *src, const char *const *markers, int32_t n_markers,
+                                  char *buf, size_t cap, size_t *needed);
+
+/* ---- launches ---- */
+
+/* ApplyFunction::apply_fn body: out[i] = f(x[i]), i < n  (src/devices/cuda/ops.rs:126-177).
+ * `out == x` (exact alias) is allowed; partial overlap is rejected. */
+int32_t custos_hip_apply_fn(custos_hip_device *dev, custos_hip_kernel *kernel, uint64_t x,
+                            uint64_t out, size_t n);
+/* Two-operand expression: out[i] = f(lhs[i], rhs[i]). */
+int32_t custos_hip_apply_fn2(custos_hip_device *dev, custos_hip_kernel *kernel, uint64_t lhs,
+                             uint64_t rhs, uint64_t out, size_t n);
+/* k-operand expression (k = kernel arity, 1..4). */
+int32_t custos_hip_apply_fn_n(custos_hip_device *dev, custos_hip_kernel *kernel,
+                              const uint64_t *ins, int32_t n_ins, uint64_t out, size_t n);
+/* UnaryGrad::add_unary_grad body: lhs_grad[i] += out_grad[i] * f(lhs[i])
+ * (src/devices/cuda/ops.rs:186-234), evaluated as g + (o * d), two roundings. */
+int32_t custos_hip_add_unary_grad(custos_hip_device *dev, custos_hip_kernel *kernel, uint64_t lhs,
+                                  uint64_t lhs_grad, uint64_t out_grad, size_t n);
+
+/* ---- lazy run: capture once, replay (src/devices/cuda/lazy.rs:10-72) ---- */
+
+/* LazySetup::lazy_setup: from here on launches/clears/copies are recorded, not run. */
+int32_t custos_hip_capture_begin(custos_hip_device *dev);
+/* Ends recording and instantiates an executable graph (LazyCudaGraph::new). */
+int32_t custos_hip_capture_end(custos_hip_device *dev, custos_hip_graph **graph);
+int32_t custos_hip_is_capturing(custos_hip_device *dev, int32_t *capturing);
+/* LazyCudaGraph::launch on the compute stream (no wait; call custos_hip_sync). */
+int32_t custos_hip_graph_launch(custos_hip_device *dev, custos_hip_graph *graph);
+int32_t custos_hip_graph_node_count(custos_hip_graph *graph, size_t *kernel_nodes);
+int32_t custos_hip_graph_destroy(custos_hip_device *dev, custos_hip_graph *graph);
+
+/* ---- timing on the compute stream (bench support) ---- */
+
+int32_t custos_hip_timer_begin(custos_hip_device *dev);
+/* Records the end event, waits for it, returns milliseconds since timer_begin. */
+int32_t custos_hip_timer_end(custos_hip_device *dev, double *ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
