@@ -14,7 +14,7 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
     }
     if (unroll > 0) t.unroll = std::min(16, unroll);
     t.blocks_per_cu = blocks_per_cu > 0 ? std::min(64, blocks_per_cu) : 0;
-    t.nontemporal = nontemporal < 0 ? 0 : (nontemporal & 3);
+    if (nontemporal != 0) t.nontemporal = nontemporal < 0 ? 0 : (nontemporal & 3);
     return t;
 }
 

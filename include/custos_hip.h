@@ -106,11 +106,12 @@ typedef struct custos_hip_device_info {
 /* Launch shape knobs of the generated kernels.  Zero fields keep the default.
  * They are part of the kernel cache key. */
 typedef struct custos_hip_tuning {
-    int32_t block_threads;   /* threads per workgroup (multiple of 64), default 256 */
-    int32_t unroll;          /* 16-byte vectors per thread per tile, default 4 */
+    int32_t block_threads;   /* threads per workgroup (multiple of 64), default 512 */
+    int32_t unroll;          /* 16-byte vectors per thread per tile, default 2 */
     int32_t blocks_per_cu;   /* > 0: persistent grid of CUs*blocks_per_cu workgroups that
                                 stride over the tiles; <= 0 (default): one tile per workgroup */
-    int32_t nontemporal;     /* bit 0: non-temporal loads, bit 1: non-temporal stores; -1 = off */
+    int32_t nontemporal;     /* bit 0: non-temporal loads, bit 1: non-temporal stores;
+                                0 = default (3: both), -1 = off */
 } custos_hip_tuning;
 
 /* ---- device (src/devices/cuda/cuda.rs:53-67, cuda_device.rs:31-128) ---- */

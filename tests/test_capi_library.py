@@ -1,0 +1,95 @@
+"""The C-ABI library loads, exports every symbol the header declares, and its
+run-time compilation pipeline produces gfx950 code objects.  No GPU needed."""
+import os
+import re
+import subprocess
+
+import pytest
+
+import custos_amd
+from custos_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "custos_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(custos_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = custos_amd.load_library()
+    names = declared_functions()
+    assert len(names) >= 30
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in include/custos_hip.h but not exported"
+
+
+def test_binding_covers_the_header():
+    assert sorted(capi.PROTOTYPES) == declared_functions()
+
+
+def test_exported_symbols_are_only_the_c_abi():
+    out = subprocess.run(["nm", "-D", "--defined-only", custos_amd.lib_path()], capture_output=True, text=True, check=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if " T " in line}
+    assert set(declared_functions()) <= exported
+
+
+def test_header_is_plain_c():
+    src = '#include "custos_hip.h"\nint main(void){ custos_hip_tuning t = {0}; (void)t; return CUSTOS_HIP_OK; }\n'
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-fsyntax-only", "-I", os.path.dirname(HEADER), "-x", "c", "-"],
+                       input=src, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
+def test_no_device_means_error_not_fallback():
+    """Without a GPU, creating a device fails with a HIP error or an index error: nothing computes on the CPU."""
+    import ctypes as C
+    lib = custos_amd.load_library()
+    count = C.c_int32(-1)
+    rc = lib.custos_hip_device_count(C.byref(count))
+    if rc == 0 and count.value > 0:
+        pytest.skip("a GPU is present")
+    h = C.c_void_p()
+    rc = lib.custos_hip_device_create(0, C.byref(h))
+    assert rc != 0 and not h.value
+    assert capi.last_error(None)
+    with pytest.raises(capi.CustosHipError):
+        custos_amd.HIP(0)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "f16", "bf16", "i32", "i64", "u8", "i8", "i16", "u16", "u32", "u64"])
+def test_offline_compile_every_dtype(dtype):
+    text = "((x * 2) + 1)" if dtype[0] in "iu" else "sqrt(abs(((x * 2.0) + 1.0)))"
+    assert capi.expr_build_code_object(capi.KIND_APPLY, dtype, text, ["x"]) > 1000
+    assert capi.expr_build_code_object(capi.KIND_UNARY_GRAD, dtype, text, ["x"]) > 1000
+
+
+def test_offline_compile_all_nodes_and_arities():
+    text = "pow(min(max((sin(a) + cos(b)), (tan(c) - tanh(d))), exp(a)), (log(abs(b)) / (-(c) * (a >= b))))"
+    assert capi.expr_build_code_object(capi.KIND_APPLY, "f32", text, ["a", "b", "c", "d"]) > 1000
+    assert capi.expr_build_code_object(capi.KIND_APPLY, "f64", "((a <= b) == c)", ["a", "b", "c"]) > 1000
+    fused = "x = sin(x);\nx = (x * 2.0);\nx = (x + 1.0);\nx = max(x, 0.0);\nx = (x - 0.5);\n"
+    assert capi.expr_build_code_object(capi.KIND_APPLY, "f32", fused, ["x"]) > 1000
+
+
+def test_chosen_device_idx_env(monkeypatch):
+    lib = custos_amd.load_library()
+    monkeypatch.delenv("CUSTOS_HIP_DEVICE_IDX", raising=False)
+    assert lib.custos_hip_chosen_device_idx() == 0
+    monkeypatch.setenv("CUSTOS_HIP_DEVICE_IDX", "3")
+    assert lib.custos_hip_chosen_device_idx() == 3
+    monkeypatch.setenv("CUSTOS_HIP_DEVICE_IDX", "junk")
+    assert lib.custos_hip_chosen_device_idx() == 0
+
+
+def test_product_never_imports_the_oracle():
+    """The shipped package and library must not reference the CPU oracle."""
+    pkg = os.path.join(ROOT, "custos_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f), errors="replace").read()
+                assert "cpu_oracle" not in text and "custos_cpu_oracle" not in text, os.path.join(dirpath, f)

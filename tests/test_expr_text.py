@@ -1,0 +1,160 @@
+"""Expression text: the Python `Combiner` mirror must print the strings the
+reference asserts for `to_cl_source`, and the library's parser must accept
+them, re-print them unchanged and emit typed HIP C for them.  CPU only."""
+import re
+
+import pytest
+
+from custos_amd import Const, Resolve, capi, to_marker, to_val
+from custos_amd.expr import format_float, fused_source
+
+
+def test_reference_strings():
+    x = Resolve("x")
+    assert x.exp().to_cl_source() == "exp(x)"                                              # mod.rs:73
+    assert Resolve("val").tan().neg().to_cl_source() == "-(tan(val))"                      # mod.rs:90
+    xx, yy = to_marker("x", "y")
+    assert xx.mul(3.).pow(yy.add(1.)).to_cl_source() == "pow((x * 3.0), (y + 1.0))"        # mod.rs:103
+    vx, other = to_marker("var_x", "other")
+    assert vx.eq(other).to_cl_source("i32") == "(var_x == other)"                          # mod.rs:116
+    assert vx.geq(0).mul(vx).to_cl_source("i32") == "((var_x >= 0) * var_x)"               # mod.rs:130
+    assert vx.add(3).to_cl_source("i32") == "(var_x + 3)"                                  # mod.rs:144
+    assert vx.geq(4).to_cl_source("i32") == "(var_x >= 4)"                                 # mod.rs:158
+    assert xx.add(yy).to_cl_source() == "(x + y)"                                          # mod.rs:176
+    assert xx.add(yy).mul(3.6).sub(yy).to_cl_source() == "(((x + y) * 3.6) - y)"           # mod.rs:192
+    assert x.add(2.).mul(x).add(x.mul(8.)).mul(5.).to_cl_source() == "((((x + 2.0) * x) + (x * 8.0)) * 5.0)"  # mod.rs:201
+    assert x.mul(x).add(2.).to_cl_source() == "((x * x) + 2.0)"                            # resolve.rs:22
+    assert x.add(x).mul(2.).to_cl_source() == "((x + x) * 2.0)"                            # resolve.rs:117
+    assert to_marker("x").to_cl_source() == "x"                                            # resolve.rs:40
+    assert x.sin().to_cl_source() == "sin(x)" and x.cos().to_cl_source() == "cos(x)"       # op_hint.rs:63,71
+    assert x.ln().to_cl_source() == "log(x)"                                               # op_hint.rs:79
+    assert x.identity().to_cl_source() == "x"                                              # ops/unary.rs:19-24
+    assert x.max(3.).min(5.).to_cl_source() == "min(max(x, 3.0), 5.0)"
+    assert x.add("1.0").to_cl_source() == "(x + 1.0)"                                      # cuda/ops.rs:254
+    assert to_val(2.0).to_cl_source("f64") == "2.0"
+
+
+def test_fused_source():
+    # src/devices/fusing.rs:104-120
+    ops = [lambda x: x.sin(), lambda x: x.neg(), lambda x: x.cos()]
+    assert fused_source(ops) == "x = sin(x);\nx = -(x);\nx = cos(x);\n"
+
+
+def test_float_formatting():
+    assert format_float(2.0) == "2.0" and format_float(3.6) == "3.6" and format_float(-0.5) == "-0.5"
+    assert format_float(float("inf")) == "inf" and format_float(float("-inf")) == "-inf"
+    assert format_float(float("nan")) == "NaN"
+    assert format_float(0.1, "f64") == "0.1"
+    assert float(format_float(1e-7)) == pytest.approx(1e-7)
+
+
+REFERENCE_TEXTS = [
+    ("exp(x)", ["x"]),
+    ("-(tan(val))", ["val"]),
+    ("pow((x * 3.0), (y + 1.0))", ["x", "y"]),
+    ("(var_x == other)", ["var_x", "other"]),
+    ("((var_x >= 0) * var_x)", ["var_x"]),
+    ("(var_x + 3)", ["var_x"]),
+    ("(x + y)", ["x", "y"]),
+    ("(((x + y) * 3.6) - y)", ["x", "y"]),
+    ("((((x + 2.0) * x) + (x * 8.0)) * 5.0)", ["x"]),
+    ("min(max(x, 3.0), 5.0)", ["x"]),
+    ("(x[idx] + 1.0)", ["x[idx]"]),                   # marker used by cuda/ops.rs:165
+    ("(lhs[idx] * -2.5e-3)", ["lhs[idx]"]),
+    ("sqrt(abs(x))", ["x"]),
+    ("((x <= inf) * -inf)", ["x"]),
+    ("2.0", ["x"]),
+    ("x", ["x"]),
+]
+
+
+@pytest.mark.parametrize("text,markers", REFERENCE_TEXTS)
+def test_parser_round_trip(text, markers):
+    assert capi.expr_canonical(text, markers) == text
+
+
+def test_fused_statement_list_nests():
+    got = capi.expr_canonical("x = sin(x);\nx = -(x);\nx = cos(x);\n", ["x"])
+    assert got == "cos(-(sin(x)))"
+
+
+@pytest.mark.parametrize("bad,code", [
+    ("(x +)", capi.ERR_EXPR_SYNTAX),
+    ("sin(x", capi.ERR_EXPR_SYNTAX),
+    ("foo(x)", capi.ERR_EXPR_SYNTAX),
+    ("(x + y)", capi.ERR_EXPR_UNKNOWN_MARKER),
+    ("", capi.ERR_EXPR_SYNTAX),
+    ("x x", capi.ERR_EXPR_SYNTAX),
+    ("y = sin(x);", capi.ERR_EXPR_UNKNOWN_MARKER),
+])
+def test_parser_errors(bad, code):
+    with pytest.raises(capi.CustosHipError) as e:
+        capi.expr_canonical(bad, ["x"])
+    assert e.value.code == code
+    assert e.value.message  # a message is always set
+
+
+def test_emit_types_literals_and_no_contraction():
+    src, _ = capi.expr_emit(capi.KIND_APPLY, "f32", "((x * 2.0) + 1.0)", ["x"])
+    assert "0x1p+1f" in src and "0x1p+0f" in src          # f32-typed literals, never a double 2.0
+    assert not re.search(r"[^x0-9a-f.p+]2\.0[^f]", src.split("\n", 1)[1])
+    assert "fma" not in src.lower()
+    assert "const float t2 = (float)(t0 * t1);" in src     # one statement per node
+    src64, _ = capi.expr_emit(capi.KIND_APPLY, "f64", "((x * 2.0) + 1.0)", ["x"])
+    assert "typedef double S;" in src64 and "0x1p+1;" in src64
+    srci, _ = capi.expr_emit(capi.KIND_APPLY, "i32", "((x >= 0) * x)", ["x"])
+    assert "typedef int S;" in srci and "(unsigned int)" in srci
+    srch, _ = capi.expr_emit(capi.KIND_APPLY, "f16", "(exp((x * 0.5)) * x)", ["x"])
+    assert "typedef _Float16 S;" in srch and "typedef float C;" in srch
+    assert "ext_vector_type(8)" in srch                     # 16-byte vectors of halves
+
+
+def test_min_max_emitted_as_selects():
+    src, _ = capi.expr_emit(capi.KIND_APPLY, "f32", "min(max(x, 0.0), 6.0)", ["x"])
+    assert "fmax" not in src and "fmin" not in src
+    assert "(t0 > t1) ? t0 : t1" in src
+
+
+def test_hash_ignores_literal_spelling_but_not_value_or_type():
+    h = lambda text, dt="f32", kind=capi.KIND_APPLY: capi.expr_emit(kind, dt, text, ["x"])[1]
+    assert h("(x * 2.0)") == h("(x * 2)") == h("(x * 2.00)") == h("(x*2.0)")
+    assert h("(x * 2.0)") != h("(x * 2.5)")
+    assert h("(x * 2.0)") != h("(x * 2.0)", "f64")
+    assert h("(x * 2.0)") != h("(x * 2.0)", "f32", capi.KIND_UNARY_GRAD)
+    assert h("(x * 2.0)") != h("(2.0 * x)")
+    # f32 rounding of the literal decides, not the text
+    assert h("(x * 0.1)") == h("(x * 0.100000001)")
+    assert h("(x * 0.1)", "f64") != h("(x * 0.100000001)", "f64")
+
+
+def test_tuning_is_part_of_the_key_and_source():
+    t = capi.Tuning(256, 4, 0, -1)
+    src, h1 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], t)
+    assert "#define CUSTOS_BLOCK 256" in src and "#define CUSTOS_UNROLL 4" in src
+    assert "__builtin_nontemporal" not in src
+    src2, h2 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"])
+    assert "#define CUSTOS_BLOCK 512" in src2 and "__builtin_nontemporal_load" in src2
+    assert h1 != h2
+
+
+def test_integer_rejects_transcendentals_and_fractions():
+    for bad in ("sin(x)", "pow(x, 2)", "(x + 1.5)"):
+        with pytest.raises(capi.CustosHipError) as e:
+            capi.expr_emit(capi.KIND_APPLY, "i32", bad, ["x"])
+        assert e.value.code == capi.ERR_EXPR_UNSUPPORTED
+    capi.expr_emit(capi.KIND_APPLY, "i32", "(x + 1.0)", ["x"])  # integral value is fine
+
+
+def test_unary_grad_takes_one_marker():
+    with pytest.raises(capi.CustosHipError) as e:
+        capi.expr_emit(capi.KIND_UNARY_GRAD, "f32", "(x + y)", ["x", "y"])
+    assert e.value.code == capi.ERR_ARITY_MISMATCH
+    src, _ = capi.expr_emit(capi.KIND_UNARY_GRAD, "f32", "cos(x)", ["x"])
+    assert "const C prod = o * d;" in src and "const C sum = g + prod;" in src
+
+
+def test_marker_arguments_validated():
+    for markers in ([], ["x", "x"], ["a", "b", "c", "d", "e"]):
+        with pytest.raises(capi.CustosHipError) as e:
+            capi.expr_emit(capi.KIND_APPLY, "f32", "x", markers)
+        assert e.value.code == capi.ERR_INVALID_ARGUMENT
