@@ -1,0 +1,317 @@
+"""GPU parity for node semantics, element types, addressing and error paths."""
+import numpy as np
+import pytest
+
+from custos_amd import Const, capi, synth
+from tests.helpers import assert_bits_equal, ulp_distance_f32
+
+pytestmark = pytest.mark.gpu
+
+SPECIALS = np.array([0.0, -0.0, 1.0, -1.0, 0.5, 3.0, -3.0, np.inf, -np.inf, np.nan, 1e-40, -1e-40, 1.17549435e-38,
+                     3.4028235e38, -3.4028235e38, 1e-45, 2.5, -2.5, 65504.0, 1e20], dtype=np.float32)
+
+
+def pairs():
+    a = np.repeat(SPECIALS, SPECIALS.size)
+    b = np.tile(SPECIALS, SPECIALS.size)
+    return a, b
+
+
+BINARY_EXACT = {
+    "add": lambda p, q: p.add(q), "sub": lambda p, q: p.sub(q), "mul": lambda p, q: p.mul(q),
+    "div": lambda p, q: p.div(q), "min": lambda p, q: p.min(q), "max": lambda p, q: p.max(q),
+    "geq": lambda p, q: p.geq(q), "leq": lambda p, q: p.leq(q), "eq": lambda p, q: p.eq(q),
+}
+
+
+@pytest.mark.parametrize("name", sorted(BINARY_EXACT))
+def test_binary_nodes_on_special_values(hip, oracle, name):
+    """+ - * / min max and the comparisons are bit-exact, including signed zeros,
+    NaN, infinities and denormals (nothing is flushed, min/max are selects)."""
+    a, b = pairs()
+    f = BINARY_EXACT[name]
+    got = hip.apply_fn2(hip.buffer(a), hip.buffer(b), f).read()
+    assert_bits_equal(got, oracle.apply_fn(f, a, b), name)
+
+
+@pytest.mark.parametrize("name,f", [("neg", lambda v: v.neg()), ("abs", lambda v: v.abs()), ("identity", lambda v: v.identity()),
+                                    ("sqrt", lambda v: v.sqrt()), ("relu_geq", lambda v: v.geq(0.).mul(v)),
+                                    ("relu_max", lambda v: v.max(0.)), ("clip", lambda v: v.max(3.).min(5.))])
+def test_unary_exact_nodes(hip, oracle, name, f):
+    x = np.concatenate([SPECIALS, synth.uniform_f32(11, 5000, -10, 10), synth.uniform_f32(12, 5000, 0, 1e-38)])
+    got = hip.apply_fn(hip.buffer(x), f).read()
+    assert_bits_equal(got, oracle.apply_fn(f, x), name)
+
+
+def test_division_and_sqrt_are_correctly_rounded(hip, oracle):
+    n = 1 << 18
+    a = synth.uniform_f32(21, n, -100, 100)
+    b = synth.uniform_f32(22, n, -7, 7)
+    assert_bits_equal(hip.apply_fn2(hip.buffer(a), hip.buffer(b), lambda p, q: p.div(q)).read(),
+                      oracle.apply_fn(lambda p, q: p.div(q), a, b))
+    c = np.abs(a) * np.float32(1e-3)
+    assert_bits_equal(hip.apply_fn(hip.buffer(c), lambda v: v.sqrt()).read(), oracle.apply_fn(lambda v: v.sqrt(), c))
+
+
+def test_mul_add_is_not_contracted(hip, oracle):
+    n = 1 << 16
+    a = synth.uniform_f32(31, n, 1, 2)
+    b = synth.uniform_f32(32, n, 1, 2)
+    f = lambda p, q: p.mul(q).sub(2.25)
+    want = oracle.apply_fn(f, a, b)
+    fused = (a.astype(np.float64) * b.astype(np.float64) - 2.25).astype(np.float32)
+    assert (want != fused).any()  # the inputs do distinguish fma from mul+add
+    assert_bits_equal(hip.apply_fn2(hip.buffer(a), hip.buffer(b), f).read(), want)
+
+
+TRANSCENDENTAL = {
+    "exp": (lambda v: v.exp(), -87.0, 88.0), "sin": (lambda v: v.sin(), -100.0, 100.0),
+    "cos": (lambda v: v.cos(), -100.0, 100.0), "tan": (lambda v: v.tan(), -1.5, 1.5),
+    "tanh": (lambda v: v.tanh(), -10.0, 10.0), "ln": (lambda v: v.ln(), 1e-30, 1e30),
+}
+
+
+@pytest.mark.parametrize("name", sorted(TRANSCENDENTAL))
+def test_transcendental_ulp(hip, oracle, name):
+    """f32 transcendentals: within 4 ulp of the CPU path (libm)."""
+    f, lo, hi = TRANSCENDENTAL[name]
+    n = 1 << 19
+    x = synth.uniform_f32(41, n, lo, hi)
+    if name == "ln":
+        x = np.exp(synth.uniform_f32(41, n, np.log(lo), np.log(hi))).astype(np.float32)
+    got = hip.apply_fn(hip.buffer(x), f).read()
+    want = oracle.apply_fn(f, x)
+    d = ulp_distance_f32(got, want)
+    assert d.max() <= 4, (name, int(d.max()), x[np.argmax(d)])
+
+
+def test_pow_ulp(hip, oracle):
+    n = 1 << 18
+    a = synth.uniform_f32(51, n, 0.01, 20)
+    b = synth.uniform_f32(52, n, -5, 5)
+    f = lambda p, q: p.pow(q)
+    d = ulp_distance_f32(hip.apply_fn2(hip.buffer(a), hip.buffer(b), f).read(), oracle.apply_fn(f, a, b))
+    assert d.max() <= 4
+    # src/two_way_ops/mod.rs:96-100: an exact case
+    got = hip.apply_fn2(hip.buffer([3.0]), hip.buffer([2.0]), lambda x, y: x.mul(3.).pow(y.add(1.))).read()
+    assert got[0] == 729.0
+
+
+def test_sin_large_arguments(hip, oracle):
+    x = np.concatenate([synth.uniform_f32(61, 1 << 16, -1e6, 1e6), synth.uniform_f32(62, 1 << 16, -1e30, 1e30)])
+    got = hip.apply_fn(hip.buffer(x), lambda v: v.sin()).read()
+    assert ulp_distance_f32(got, oracle.apply_fn(lambda v: v.sin(), x)).max() <= 4
+
+
+def test_reference_int_vectors(hip):
+    # src/two_way_ops/mod.rs:236-245, src/devices/cuda/ops.rs:259-272,279-294 (eager here)
+    out = hip.apply_fn(hip.buffer([3, 3, 4, 5, 3, 2], "i32"), lambda x: x.add(3))
+    assert out.read().tolist() == [6, 6, 7, 8, 6, 5]
+    lhs = hip.buffer([1, 2, 3, 4, 5, 6], "i32")
+    g = hip.buffer([1, 2, 3, 4, 5, 6], "i32")
+    o = hip.buffer([1, 1, 1, 1, 1, 1], "i32")
+    hip.add_unary_grad(lhs, g, o, lambda x: x.mul(2).add(1))
+    assert g.read().tolist() == [4, 7, 10, 13, 16, 19]
+    out = hip.apply_fn(hip.buffer([1., 2., 3., 4., 5., 6.]), lambda x: x.add("1.0"))  # cuda/ops.rs:250-257
+    assert out.read().tolist() == [2., 3., 4., 5., 6., 7.]
+    out = hip.apply_fn(hip.buffer([1., 3., 4., 6., 3., 2.]), lambda x: x.max(3.).min(5.))  # mod.rs:206-217
+    assert out.read().tolist() == [3., 3., 4., 5., 3., 3.]
+
+
+def test_unary_grad_doc_example(hip):
+    # src/unary.rs:40-47
+    from custos_amd import to_val
+    a = hip.buffer([1., 2., 3., 3., 2., 1.], "f64")
+    og = hip.buffer([1.] * 6, "f64")
+    g = hip.buffer([0.] * 6, "f64")
+    hip.add_unary_grad(a, g, og, lambda x: to_val(2.0))
+    assert g.read().tolist() == [2.] * 6
+
+
+INT_TYPES = ["i8", "u8", "i16", "u16", "i32", "u32", "i64", "u64"]
+
+
+@pytest.mark.parametrize("dtype", INT_TYPES)
+def test_integer_types_wrap_like_the_cpu(hip, oracle, dtype):
+    npdt = np.dtype(capi.DTYPES[dtype][1])
+    info = np.iinfo(npdt)
+    rng = np.random.default_rng(7)
+    x = rng.integers(info.min, info.max, size=10007, dtype=npdt, endpoint=True)
+    y = rng.integers(info.min, info.max, size=10007, dtype=npdt, endpoint=True)
+    f = lambda p, q: p.mul(q).add(p).sub(3).max(q).geq(p).add(p.min(q)).mul(5)
+    got = hip.apply_fn2(hip.buffer(x, dtype), hip.buffer(y, dtype), f).read()
+    assert_bits_equal(got, oracle.apply_fn(f, x, y, dtype=dtype), dtype)
+    g = rng.integers(info.min, info.max, size=10007, dtype=npdt, endpoint=True)
+    gb = hip.buffer(g, dtype)
+    hip.add_unary_grad(hip.buffer(x, dtype), gb, hip.buffer(y, dtype), lambda v: v.mul(2).add(1))
+    assert_bits_equal(gb.read(), oracle.add_unary_grad(lambda v: v.mul(2).add(1), x, g, y, dtype=dtype), dtype + " grad")
+
+
+def test_integer_division(hip, oracle):
+    x = np.array([7, -7, 100, -100, 0, 5], dtype=np.int32)
+    y = np.array([2, 2, -3, -3, 5, 5], dtype=np.int32)
+    f = lambda p, q: p.div(q)
+    assert_bits_equal(hip.apply_fn2(hip.buffer(x, "i32"), hip.buffer(y, "i32"), f).read(), oracle.apply_fn(f, x, y, dtype="i32"))
+
+
+def test_f64(hip, oracle):
+    n = 50001
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-3, 3, n)
+    exact = lambda v: v.mul(1.7).add(0.3).max(0.25).sub(v).div(3.0).abs().neg()
+    assert_bits_equal(hip.apply_fn(hip.buffer(x, "f64"), exact).read(), oracle.apply_fn(exact, x, dtype="f64"))
+    got = hip.apply_fn(hip.buffer(x, "f64"), lambda v: v.mul(2.).add(4.).sin().mul(v).add(1.)).read()
+    want = oracle.apply_fn(lambda v: v.mul(2.).add(4.).sin().mul(v).add(1.), x, dtype="f64")
+    assert np.max(np.abs(got - want)) <= 8 * np.finfo(np.float64).eps
+    # src/two_way_ops/mod.rs:262-283
+    ref = hip.apply_fn(hip.buffer([3., 3., 4., 5., 3., 2.], "f64"), lambda v: v.mul(2.).add(4.).sin().mul(v).add(1.)).read()
+    assert np.allclose(ref, [-0.6320633326681093, -0.6320633326681093, -1.1462916720017398, 5.953036778474352,
+                             -0.6320633326681093, 2.978716493246764], rtol=0, atol=1e-14)
+
+
+def test_bf16(hip, oracle):
+    n = 40003
+    x32 = synth.uniform_f32(71, n, -4, 4)
+    xb = (x32.view(np.uint32) >> 16).astype(np.uint16)
+    f = lambda v: v.mul(1.5).add(v.mul(v)).sub(0.125)
+    got = hip.apply_fn(hip.buffer(xb, "bf16"), f).read()
+    assert_bits_equal(got, oracle.apply_fn(f, xb, dtype="bf16"))
+
+
+def test_f16_specials_and_rounding(hip, oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    f = lambda v: v.mul(1.0009765625).add(0.00006103515625)   # forces re-rounding of every half
+    got = hip.apply_fn(hip.buffer(bits.view(np.float16), "f16"), f).read().view(np.uint16)
+    want = oracle.apply_fn(f, bits, dtype="f16")
+    nan = np.isnan(want.view(np.float16))
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.isnan(got.view(np.float16)[nan]).all()
+
+
+@pytest.mark.parametrize("off_in,off_out", [(0, 0), (1, 1), (3, 3), (1, 2), (0, 3), (2, 0)])
+@pytest.mark.parametrize("n", [1, 2, 7, 1000, 8191, 70000])
+def test_unaligned_views(hip, oracle, off_in, off_out, n):
+    """Sub-ranges that are not 16-byte aligned: equal phase takes the vector path with a
+    scalar head and tail, different phases take the scalar path; neighbours stay untouched."""
+    total = n + 8
+    x = synth.uniform_f32(81, total, -2, 2)
+    xb = hip.buffer(x)
+    outb = hip.buffer(np.full(total, 7.0, dtype=np.float32))
+    f = lambda v: v.mul(3.0).sub(1.0)
+    hip.apply_fn(xb.slice(off_in, off_in + n), f, out=outb.slice(off_out, off_out + n))
+    got = outb.read()
+    want = np.full(total, 7.0, dtype=np.float32)
+    want[off_out:off_out + n] = oracle.apply_fn(f, x[off_in:off_in + n])
+    assert_bits_equal(got, want)
+
+
+def test_f16_unaligned_views(hip, oracle):
+    total = 5000
+    xb = synth.uniform_f16_bits(5, total, -2, 2)
+    buf = hip.buffer(xb.view(np.float16), "f16")
+    out = hip.buffer(np.zeros(total, dtype=np.float16), "f16")
+    f = lambda v: v.mul(2.0).add(0.5)
+    for off, n in [(1, 4000), (3, 17), (8, 4992), (5, 1)]:
+        out.clear()
+        hip.apply_fn(buf.slice(off, off + n), f, out=out.slice(off, off + n))
+        got = out.read().view(np.uint16)
+        want = np.zeros(total, dtype=np.uint16)
+        want[off:off + n] = oracle.apply_fn(f, xb[off:off + n], dtype="f16")
+        assert_bits_equal(got, want)
+
+
+def test_in_place_and_overlap(hip, oracle):
+    n = 100000
+    x = synth.uniform_f32(91, n, -2, 2)
+    xb = hip.buffer(x)
+    f = lambda v: v.mul(v).add(1.0)
+    hip.apply_fn(xb, f, out=xb)  # exact alias is allowed
+    assert_bits_equal(xb.read(), oracle.apply_fn(f, x))
+    with pytest.raises(capi.CustosHipError) as e:
+        hip.apply_fn(xb.slice(0, 1000), f, out=xb.slice(4, 1004))
+    assert e.value.code == capi.ERR_BAD_OVERLAP
+
+
+def test_four_operands(hip, oracle):
+    n = 30011
+    arrs = [synth.uniform_f32(100 + i, n, -2, 2) for i in range(4)]
+    f = lambda a, b, c, d: a.mul(b).add(c).max(d).sub(a.min(d))
+    got = hip.apply_fn_n([hip.buffer(v) for v in arrs], f).read()
+    assert_bits_equal(got, oracle.apply_fn(f, *arrs))
+
+
+def test_tuning_variants_agree(hip, oracle):
+    n = 300007
+    x = synth.uniform_f32(111, n, -2, 2)
+    f = lambda v: v.mul(1.25).add(0.5).max(0.0)
+    want = oracle.apply_fn(f, x)
+    xb = hip.buffer(x)
+    try:
+        for block, unroll, bpc, nt in [(64, 1, 0, -1), (256, 4, 0, 1), (1024, 8, 0, 2), (256, 3, 2, 3), (512, 2, 1, 0)]:
+            hip.set_tuning(block, unroll, bpc, nt)
+            assert_bits_equal(hip.apply_fn(xb, f).read(), want, f"{block}x{unroll} bpc={bpc} nt={nt}")
+    finally:
+        hip.set_tuning()
+
+
+def test_kernel_cache(hip):
+    c0, h0 = hip.cache_stats()
+    k1 = hip.compile(capi.KIND_APPLY, "f32", "((x * 41.0) + 0.125)", ("x",))
+    k2 = hip.compile(capi.KIND_APPLY, "f32", "((x*41) + 0.1250)", ("x",))
+    k3 = hip.compile(capi.KIND_APPLY, "f32", "((y * 41.0) + 0.125)", ("y",))
+    c1, h1 = hip.cache_stats()
+    assert k1.value == k2.value == k3.value
+    assert c1 - c0 == 1 and h1 - h0 == 2
+    k4 = hip.compile(capi.KIND_UNARY_GRAD, "f32", "((x * 41.0) + 0.125)", ("x",))
+    assert k4.value != k1.value
+    assert "custos_kernel" in hip.kernel_source(k1)
+
+
+def test_error_paths(hip):
+    with pytest.raises(capi.CustosHipError) as e:
+        hip.alloc(0)
+    assert e.value.code == capi.ERR_ZERO_LENGTH_BUFFER          # src/devices/cuda/api/cuda.rs:69-71
+    import custos_amd
+    with pytest.raises(capi.CustosHipError) as e:
+        custos_amd.HIP(1000)
+    assert e.value.code == capi.ERR_INVALID_DEVICE_INDEX        # src/devices/cuda/api/cuda.rs:36-39
+    k_apply = hip.compile(capi.KIND_APPLY, "f32", "(x + 1.0)", ("x",))
+    k_grad = hip.compile(capi.KIND_UNARY_GRAD, "f32", "(x + 1.0)", ("x",))
+    b = hip.alloc(16)
+    rc = hip.lib.custos_hip_add_unary_grad(hip.handle, k_apply, b.ptr, b.ptr, b.ptr, 16)
+    assert rc == capi.ERR_KIND_MISMATCH
+    rc = hip.lib.custos_hip_apply_fn(hip.handle, k_grad, b.ptr, b.ptr, 16)
+    assert rc == capi.ERR_KIND_MISMATCH
+    k2 = hip.compile(capi.KIND_APPLY, "f32", "(x + y)", ("x", "y"))
+    rc = hip.lib.custos_hip_apply_fn(hip.handle, k2, b.ptr, b.ptr, 16)
+    assert rc == capi.ERR_ARITY_MISMATCH
+    rc = hip.lib.custos_hip_apply_fn(hip.handle, k_apply, 0, b.ptr, 16)
+    assert rc == capi.ERR_INVALID_ARGUMENT
+    rc = hip.lib.custos_hip_apply_fn(hip.handle, k_apply, b.ptr + 2, b.ptr, 4)
+    assert rc == capi.ERR_INVALID_ARGUMENT                       # not aligned to the element size
+    assert hip.lib.custos_hip_apply_fn(hip.handle, k_apply, b.ptr, b.ptr, 0) == 0   # empty input is a no-op
+    with pytest.raises(capi.CustosHipError):
+        hip.compile(capi.KIND_APPLY, "f32", "(x +", ("x",))
+    # the device is still usable after errors
+    assert hip.apply_fn(hip.buffer([1.0, 2.0]), lambda v: v.add(1.0)).read().tolist() == [2.0, 3.0]
+
+
+def test_alloc_is_zeroed_and_clear_write_copy(hip):
+    for n in (1, 5, 1000, 100003):
+        assert not hip.alloc(n).read().any()
+        assert not hip.alloc(n, "u8").read().any()
+    x = synth.uniform_f32(5, 1001, 1, 2)
+    b = hip.buffer(x)
+    c = hip.alloc(1001)
+    hip.copy(c, b)
+    assert_bits_equal(c.read(), x)
+    v = b.slice(3, 990)
+    v.clear()
+    want = x.copy()
+    want[3:990] = 0
+    assert_bits_equal(b.read(), want)                            # neighbours of a cleared view stay
+    b.write(np.arange(1001, dtype=np.float32))
+    assert b.read()[1000] == 1000.0
+    u = hip.buffer([1, 2, 3, 4, 5, 6], "u32")                    # src/devices/cuda/ops.rs:242-247
+    u.clear()
+    assert u.read().tolist() == [0] * 6
