@@ -27,6 +27,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 
+# HBM bytes per launch of the fused chain at N = 2^28 with the default launch shape, from two
+# `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE) scaled by the identity-copy kernel of
+# known size; commands and raw counter values: profiles/fused_chain_f32_n2p28_hbm_traffic.md
+MEASURED_TRAFFIC_C2_N2P28 = 2147505869
+
 C2_OPS = [
     lambda v: v.sin(),
     lambda v: v.mul(2.0),
@@ -88,6 +93,7 @@ def bench_c2(dev, args):
     from custos_amd.expr import fused_source
 
     n = 1 << args.log2n
+    tuned = bool(args.block or args.unroll or args.blocks_per_cu or args.nontemporal)
     x = gen_chunked(lambda m, off: synth.uniform_f32(0, m, -np.pi, np.pi, off), n)
     xb = dev.buffer(x)
     out = dev.alloc(n, "f32")
@@ -116,6 +122,16 @@ def bench_c2(dev, args):
 
     ums, _ = time_steps(dev, unfused_step, max(1, args.steps // 4), max(1, args.warmup // 2))
     unfused_ms = ums / max(1, args.steps // 4)
+
+    # plain copy (identity expression) over the same buffers: the achievable 1R+1W rate on
+    # this box, and the known-size dispatch the profiler counters are scaled by
+    copy_kernel = dev.compile(capi.KIND_APPLY, "f32", "x", ("x",))
+
+    def copy_step():
+        capi.check(lib.custos_hip_apply_fn(h, copy_kernel, xb.ptr, tmp_a.ptr, n), h)
+
+    cms, _ = time_steps(dev, copy_step, max(1, args.steps // 2), max(1, args.warmup // 2))
+    copy_ms = cms / max(1, args.steps // 2)
 
     # parity of the very buffer that was timed, on the CPU sample
     fused_step()
@@ -146,6 +162,12 @@ def bench_c2(dev, args):
             "moved_GBps_on_40B_basis": round(5 * algo_bytes / (unfused_ms * 1e-3) / 1e9, 2),
             "speedup_fused": round(unfused_ms / per_launch_ms, 3),
         },
+        "copy_kernel": {
+            "name": dev.kernel_name(copy_kernel),
+            "ms_per_launch": round(copy_ms, 5),
+            "GBps": round(algo_bytes / (copy_ms * 1e-3) / 1e9, 2),
+            "bytes_per_launch": algo_bytes,
+        },
         "max_abs_diff_vs_cpu_oracle": diff,
         "roofline": {
             "bound": "hbm",
@@ -153,8 +175,8 @@ def bench_c2(dev, args):
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
-            "kernel": "custos_kernel (fused apply, f32)",
+            "traffic": MEASURED_TRAFFIC_C2_N2P28 if (args.log2n == 28 and not tuned) else None,
+            "kernel": dev.kernel_name(kernel),
             "algorithmic_bytes_per_launch": algo_bytes,
             "avg_launch_ms": round(per_launch_ms, 5),
         },

@@ -99,6 +99,7 @@ PROTOTYPES = {
     "custos_hip_clear": (C.c_int32, [_P, C.c_uint64, C.c_size_t]),
     "custos_hip_expr_compile": (C.c_int32, [_P, C.c_int32, C.c_int32, C.c_char_p, _STRS, C.c_int32, _PP]),
     "custos_hip_kernel_source": (C.c_char_p, [_P]),
+    "custos_hip_kernel_name": (C.c_char_p, [_P]),
     "custos_hip_kernel_hash": (C.c_uint64, [_P]),
     "custos_hip_kernel_arity": (C.c_int32, [_P]),
     "custos_hip_cache_stats": (C.c_int32, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),

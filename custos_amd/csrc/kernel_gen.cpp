@@ -1,6 +1,7 @@
 #include "kernel_gen.hpp"
 
 #include <algorithm>
+#include <cstdio>
 
 #include "../../include/custos_hip.h"
 
@@ -122,6 +123,14 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
                        tuning.blocks_per_cu, tuning.nontemporal, 2 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
+    {
+        static const char* const dtype_names[] = {"f32", "f64", "i32", "i64", "f16", "bf16",
+                                                  "u8",  "i8",  "i16", "u16", "u32", "u64"};
+        char hex[17];
+        std::snprintf(hex, sizeof hex, "%016llx", static_cast<unsigned long long>(k.hash));
+        k.name = std::string(kind == Kind::Apply ? "custos_apply_" : "custos_unary_grad_") +
+                 dtype_names[static_cast<int>(dtype)] + "_" + hex;
+    }
 
     std::string body;
     if (!emit_expr_body(k.expr, dtype, &body, err)) return false;
@@ -143,7 +152,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     // Per-element function on storage values: `custos_elem(in0.., [g])`.
     // Pointers that are read and written (`out`, `lhs_grad`) carry no
     // __restrict__: the output may be exactly one of the inputs.
-    std::string params, vec_ptrs, elem_params, elem_call_s, elem_call_v, loads;
+    std::string params, vec_ptrs;
     if (kind == Kind::Apply) {
         s += "static __device__ __forceinline__ S custos_elem(";
         for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "const S s" + std::to_string(i);
@@ -177,7 +186,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     };
 
     s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-    s += std::string(kKernelName) + "(" + params + ", const u64 n, const u64 head, const u64 n_vec) {\n";
+    s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec) {\n";
     s += vec_ptrs;
     s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
     s += "    const u64 n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;\n";

@@ -36,11 +36,11 @@ struct KernelSpec {
     Expr expr;
     Tuning tuning;
     uint64_t hash = 0;   // cache key: expression, dtype, kind, tuning
+    std::string name;    // entry point: custos_<kind>_<dtype>_<hash>, unique per kernel so
+                         // that profiler output tells the kernels apart
     std::string source;  // complete translation unit
     int vec_elems = 4;   // elements per 16-byte vector
 };
-
-constexpr const char* kKernelName = "custos_kernel";
 
 // Parses, hashes and emits. On failure returns false and fills `err`.
 bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,

@@ -451,7 +451,7 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
     rc = compile_to_code_object(dev, k->spec, dev->arch, &code);
     if (rc != CUSTOS_HIP_OK) return rc;
     HIP_TRY(dev, hipModuleLoadData(&k->module, code.data()));
-    hipError_t e = hipModuleGetFunction(&k->fn, k->module, kKernelName);
+    hipError_t e = hipModuleGetFunction(&k->fn, k->module, k->spec.name.c_str());
     if (e != hipSuccess) {
         (void)hipModuleUnload(k->module);
         return hip_fail(dev, e, "hipModuleGetFunction");
@@ -464,6 +464,10 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
 
 const char* custos_hip_kernel_source(const custos_hip_kernel* kernel) {
     return kernel ? kernel->spec.source.c_str() : "";
+}
+
+const char* custos_hip_kernel_name(const custos_hip_kernel* kernel) {
+    return kernel ? kernel->spec.name.c_str() : "";
 }
 
 uint64_t custos_hip_kernel_hash(const custos_hip_kernel* kernel) { return kernel ? kernel->spec.hash : 0; }

@@ -181,6 +181,9 @@ class HIP:
     def kernel_source(self, kernel) -> str:
         return self.lib.custos_hip_kernel_source(kernel).decode()
 
+    def kernel_name(self, kernel) -> str:
+        return self.lib.custos_hip_kernel_name(kernel).decode()
+
     def apply_fn(self, buf: Buffer, f, out: Buffer | None = None) -> Buffer:
         """`device.apply_fn(&buf, |x| ...)`: out[i] = f(buf[i]) in a new buffer."""
         src = _wrap(f(Resolve("x"))).to_cl_source(buf.dtype)

@@ -172,8 +172,10 @@ int32_t custos_hip_clear(custos_hip_device *dev, uint64_t dptr, size_t bytes);
 int32_t custos_hip_expr_compile(custos_hip_device *dev, int32_t kind, int32_t dtype,
                                 const char *src, const char *const *markers, int32_t n_markers,
                                 custos_hip_kernel **kernel);
-/* Generated HIP source of a kernel, its 64-bit cache key and its arity. */
+/* Generated HIP source of a kernel, the name of its entry point (what a
+ * profiler lists: custos_<kind>_<dtype>_<key>), its 64-bit cache key and arity. */
 const char *custos_hip_kernel_source(const custos_hip_kernel *kernel);
+const char *custos_hip_kernel_name(const custos_hip_kernel *kernel);
 uint64_t custos_hip_kernel_hash(const custos_hip_kernel *kernel);
 int32_t custos_hip_kernel_arity(const custos_hip_kernel *kernel);
 /* Number of hiprtc compilations / cache hits since the device was created. */

@@ -264,7 +264,8 @@ def test_kernel_cache(hip):
     assert c1 - c0 == 1 and h1 - h0 == 2
     k4 = hip.compile(capi.KIND_UNARY_GRAD, "f32", "((x * 41.0) + 0.125)", ("x",))
     assert k4.value != k1.value
-    assert "custos_kernel" in hip.kernel_source(k1)
+    assert hip.kernel_name(k1).startswith("custos_apply_f32_") and hip.kernel_name(k1) in hip.kernel_source(k1)
+    assert hip.kernel_name(k4).startswith("custos_unary_grad_f32_")
 
 
 def test_error_paths(hip):
