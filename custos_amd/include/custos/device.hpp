@@ -1,0 +1,277 @@
+// The device-side trait surface, as one CRTP base.
+//
+// A concrete device (`HIP<Mods>`) derives from `Device<HIP<Mods>, Mods>` and
+// supplies the primitives (raw memory, the three element-wise launches, the
+// lazy-run hook).  This base supplies what the reference gets from
+// `impl_device_traits!` and its blanket impls:
+//   Retriever::retrieve            src/devices.rs:158-193
+//   AddOperation::{add_op,eagerly} src/features.rs:409-488
+//   AddGradFn::add_grad_fn         src/features.rs:186-261
+//   ApplyFunction::apply_fn        src/unary.rs:7-28,   src/devices/cuda/ops.rs:119-141
+//   UnaryGrad::add_unary_grad      src/unary.rs:31-58,  src/devices/cuda/ops.rs:179-199
+//   UnaryElementWiseMayGrad        src/unary.rs:62-132
+//   Run / ExecNow / Optimize       src/features.rs:142-154,505-532,660-672
+//   Read / WriteBuf / ClearBuf     src/op_traits.rs:6-197
+//   backward / grad                src/buffer/impl_autograd.rs:20-197, autograd/tape.rs:39-117
+#pragma once
+
+#include <initializer_list>
+#include <optional>
+#include <tuple>
+#include <type_traits>
+#include <utility>
+#include <vector>
+
+#include "buffer.hpp"
+#include "modules.hpp"
+
+namespace custos {
+
+template <class Derived, class Mods>
+class Device {
+   public:
+    Mods modules;
+
+    Derived& self() { return static_cast<Derived&>(*this); }
+
+    // ---- buffers ----
+
+    // `device.buffer([..])`: allocate, upload, announce to the modules (src/buffer.rs:80-93)
+    template <class T>
+    Buffer<T, Derived> buffer(const std::vector<T>& data) {
+        if (data.empty()) throw Error(DeviceError::ZeroLengthBuffer);
+        uint64_t ptr = self().alloc_raw(data.size() * sizeof(T), /*zeroed=*/false, data.size());
+        self().write_raw(ptr, data.data(), data.size() * sizeof(T));
+        auto b = Buffer<T, Derived>::from_parts(&self(), ptr, data.size(), Id{ptr, data.size()}, AllocFlag::None);
+        modules.on_new_buffer(self(), b);
+        return b;
+    }
+    template <class T>
+    Buffer<T, Derived> buffer(std::initializer_list<T> data) {
+        return buffer(std::vector<T>(data));
+    }
+
+    // `Buffer::new(&device, len)`: zero-initialised (src/devices/cpu/cpu_device.rs:133-145)
+    template <class T>
+    Buffer<T, Derived> new_buffer(size_t len) {
+        if (len == 0) throw Error(DeviceError::ZeroLengthBuffer);
+        uint64_t ptr = self().alloc_raw(len * sizeof(T), /*zeroed=*/true, len);
+        auto b = Buffer<T, Derived>::from_parts(&self(), ptr, len, Id{ptr, len}, AllocFlag::None);
+        modules.on_new_buffer(self(), b);
+        return b;
+    }
+
+    // `device.retrieve(len, parents)`
+    template <class T, class... P>
+    Buffer<T, Derived> retrieve(size_t len, const P&... parents) {
+        if (len == 0) throw Error(DeviceError::ZeroLengthBuffer);
+        std::vector<Id> ids{parents.id()...};
+        std::vector<bool> rg{parents.requires_grad()...};
+        return modules.template retrieve<T>(self(), len, ids, rg);
+    }
+
+    template <class T>
+    std::vector<T> read(const Buffer<T, Derived>& buf) {
+        if (!buf.has_data()) throw Error(DeviceError::InvalidLazyBuf);
+        std::vector<T> out(buf.len());
+        self().read_raw(out.data(), buf.ptr(), buf.len() * sizeof(T));
+        return out;
+    }
+    template <class T>
+    void write(Buffer<T, Derived>& buf, const std::vector<T>& data) {
+        if (!buf.has_data()) throw Error(DeviceError::InvalidLazyBuf);
+        if (data.size() != buf.len()) throw Error(DeviceError::ShapeLengthMismatch);
+        self().write_raw(buf.ptr(), data.data(), data.size() * sizeof(T));
+    }
+    template <class T>
+    void clear(Buffer<T, Derived>& buf) {
+        if (!buf.has_data()) throw Error(DeviceError::InvalidLazyBuf);
+        self().clear_raw(buf.ptr(), buf.len() * sizeof(T));
+    }
+    // `WriteBuf::write_buf`
+    template <class T>
+    void write_buf(Buffer<T, Derived>& dst, const Buffer<T, Derived>& src) {
+        if (dst.len() != src.len()) throw Error(DeviceError::ShapeLengthMismatch);
+        self().copy_raw(dst.ptr(), src.ptr(), src.len() * sizeof(T));
+    }
+
+    // ---- operations ----
+
+    // `device.add_op((&mut out, buf), |(out, buf), dev| ...)`.
+    // Eager modules call `fn` now with the very arguments; with `Lazy` enabled it
+    // is recorded together with the argument ids and called at `run()` with the
+    // buffers those ids name then.
+    template <class F, class... B>
+    void add_op(std::tuple<B&...> args, F fn) {
+        if (!modules.is_lazy_enabled()) {
+            std::apply([&](B&... b) { fn(b..., self()); }, args);
+            return;
+        }
+        modules.add_op(self(), make_operation(args, std::move(fn)));
+    }
+
+    // `device.add_grad_fn((buf, &out), |(buf, out), dev| ...)`: pushed onto the
+    // tape when an Autograd module is present, else dropped.
+    template <class F, class... B>
+    void add_grad_fn(std::tuple<B&...> args, F fn) {
+        if (modules.autograd() == nullptr || !modules.is_grad_enabled()) return;
+        modules.add_grad_fn(make_operation(args, std::move(fn)));
+    }
+
+    // Runs `f` with lazy recording switched off (src/features.rs:438-444).
+    template <class F>
+    void eagerly(F f) {
+        const bool before = modules.is_lazy_enabled();
+        modules.set_lazy_enabled(false);
+        try {
+            f();
+        } catch (...) {
+            modules.set_lazy_enabled(before);
+            throw;
+        }
+        modules.set_lazy_enabled(before);
+    }
+    size_t ops_count() const { return modules.ops_count(); }
+
+    // `device.apply_fn(&buf, |x| ...)`: retrieve out, add the op, tag it with the unary hint.
+    template <class T, class F>
+    Buffer<T, Derived> apply_fn(const Buffer<T, Derived>& buf, F f) {
+        Buffer<T, Derived> out = retrieve<T>(buf.len(), buf);
+        add_op(std::tie(out, buf), [f](Buffer<T, Derived>& o, const Buffer<T, Derived>& x, Derived& dev) {
+            dev.apply_fn_impl(x, o, f);
+        });
+        modules.set_op_hint(erase_hint(unary<T>(f)));
+        return out;
+    }
+
+    // `device.add_unary_grad(&lhs, &mut lhs_grad, &out_grad, |x| ...)`
+    template <class T, class F>
+    void add_unary_grad(const Buffer<T, Derived>& lhs, Buffer<T, Derived>& lhs_grad,
+                        const Buffer<T, Derived>& out_grad, F lhs_grad_fn) {
+        add_op(std::tie(lhs, lhs_grad, out_grad),
+               [lhs_grad_fn](const Buffer<T, Derived>& l, Buffer<T, Derived>& g, const Buffer<T, Derived>& o, Derived& dev) {
+                   dev.add_unary_grad_impl(l, g, o, lhs_grad_fn);
+               });
+    }
+
+    // `device.unary_ew(&mut buf, forward, grad)` (src/unary.rs:97-132)
+    template <class T, class FO, class GO>
+    Buffer<T, Derived> unary_ew(Buffer<T, Derived>& buf, FO forward_fn, GO grad_fn) {
+        Buffer<T, Derived> out = apply_fn(buf, forward_fn);
+        add_grad_fn(std::tie(buf, out), [grad_fn](Buffer<T, Derived>& b, Buffer<T, Derived>& o, Derived& dev) {
+            if (!b.requires_grad()) return;
+            // lazy execution is already disabled during the backward pass
+            dev.eagerly([&] {
+                Buffer<T, Derived> b_grad = b.grad(dev);
+                Buffer<T, Derived> o_grad = o.grad(dev);
+                dev.add_unary_grad(b, b_grad, o_grad, grad_fn);
+            });
+        });
+        return out;
+    }
+
+    // ---- run / exec_now / optimize ----
+
+    void run() { modules.run(self()); }
+    // `exec_now(&device, range)`: run and consume the recorded operations [begin, end)
+    void exec_now(size_t begin, size_t end = static_cast<size_t>(-1)) { modules.exec_now(self(), begin, end); }
+    // `exec_last_n` (src/features.rs:520-531)
+    void exec_last_n(size_t last_n) {
+        const size_t n = modules.ops_count();
+        modules.exec_now(self(), n - std::min(n, last_n), n);
+    }
+    void optimize_mem_graph() { modules.optimize_mem_graph(self(), nullptr); }
+    void unary_fusing() { modules.unary_fusing(self(), nullptr); }
+
+    // ---- autograd ----
+
+    // Gradient buffer of `id`, allocated zeroed on first use (autograd/gradients.rs:90-126).
+    template <class T>
+    Buffer<T, Derived> grad_of(Id id) {
+        AutogradState* ag = modules.autograd();
+        if (!ag) throw std::logic_error("Autograd<> is not available.");
+        auto it = ag->grads.find(id.id);
+        if (it == ag->grads.end()) {
+            uint64_t ptr = self().alloc_raw(id.len * sizeof(T), /*zeroed=*/true, id.len);
+            it = ag->grads.emplace(id.id, AnyBuf{ptr, id.len, std::type_index(typeid(T)), true, sizeof(T)}).first;
+        }
+        if (it->second.type != std::type_index(typeid(T))) throw Error(DeviceError::TypeMismatch);
+        return Buffer<T, Derived>::from_parts(&self(), it->second.ptr, it->second.len, Id{it->second.ptr, it->second.len},
+                                              AllocFlag::Wrapper);
+    }
+
+    template <class T>
+    std::optional<Buffer<T, Derived>> try_grad_of(Id id) {
+        AutogradState* ag = modules.autograd();
+        if (!ag || ag->grads.find(id.id) == ag->grads.end()) return std::nullopt;
+        return grad_of<T>(id);
+    }
+
+    // `Gradients::zero_grad` (autograd/gradients.rs:30-42)
+    void zero_grad() {
+        AutogradState* ag = modules.autograd();
+        if (!ag) return;
+        for (auto& kv : ag->grads) {
+            auto rg = ag->buf_requires_grad.find(kv.first);
+            if (rg == ag->buf_requires_grad.end() || rg->second)
+                self().clear_raw(kv.second.ptr, kv.second.len * kv.second.elem_size);
+        }
+    }
+
+    // Seeds `buf`'s gradient and replays the tape in reverse, eagerly; the tape is
+    // kept when lazy recording is on (tape.rs:39-83, impl_autograd.rs:37-56).
+    template <class T>
+    void backward_seeded(const Buffer<T, Derived>& buf, const std::vector<T>& seed) {
+        AutogradState* ag = modules.autograd();
+        if (!ag) return;
+        Buffer<T, Derived> g = grad_of<T>(buf.id());
+        write(g, seed);
+        const bool lazy_enabled = modules.is_lazy_enabled();
+        Buffers* buffers = modules.buffers();
+        eagerly([&] {
+            for (size_t i = ag->tape.size(); i-- > 0;) ag->tape[i].op(*buffers, &self());
+        });
+        if (!lazy_enabled) ag->tape.clear();
+    }
+
+    void set_grad_enabled(bool e) { modules.set_grad_enabled(e); }
+    void enable_grad() { modules.set_grad_enabled(true); }
+    void disable_grad() { modules.set_grad_enabled(false); }
+
+   private:
+    template <class BufT>
+    static BufT view_of(Derived& dev, Buffers& bufs, Id id) {
+        using B = std::remove_const_t<BufT>;
+        using T = typename B::value_type;
+        auto it = bufs.find(id.id);
+        if (it == bufs.end() || it->second.ptr == 0) throw Error(DeviceError::InvalidLazyBuf);
+        if (it->second.type != std::type_index(typeid(T))) throw Error(DeviceError::TypeMismatch);
+        return B::from_parts(&dev, it->second.ptr, it->second.len, id, AllocFlag::Wrapper,
+                             dev.modules.requires_grad_of(id));
+    }
+
+    template <class F, class... B, size_t... I>
+    static void call_with_views(F& fn, Derived& dev, Buffers& bufs, const std::vector<Id>& ids,
+                                std::index_sequence<I...>) {
+        std::tuple<std::remove_const_t<B>...> views{view_of<std::remove_const_t<B>>(dev, bufs, ids[I])...};
+        fn(std::get<I>(views)..., dev);
+    }
+
+    template <class F, class... B>
+    Operation make_operation(std::tuple<B&...> args, F fn) {
+        Operation op;
+        std::apply([&](B&... b) { (op.arg_ids.push_back(b.id()), ...); }, args);
+        // every parent must be unique (src/modules/lazy/lazy_graph.rs:117-125)
+        for (size_t i = 0; i < op.arg_ids.size(); i++)
+            for (size_t j = i + 1; j < op.arg_ids.size(); j++)
+                if (op.arg_ids[i].id == op.arg_ids[j].id) throw Error(DeviceError::DuplicateParent);
+        std::vector<Id> ids = op.arg_ids;
+        op.op = [fn, ids](Buffers& bufs, void* devp) mutable {
+            Derived& dev = *static_cast<Derived*>(devp);
+            call_with_views<F, B...>(fn, dev, bufs, ids, std::index_sequence_for<B...>{});
+        };
+        return op;
+    }
+};
+
+}  // namespace custos

@@ -1,0 +1,212 @@
+// `HIP<Mods>`: the MI355X device, over the C ABI of libcustos_hip.so.
+//
+// Takes the place of `CUDA<Mods>` in user code: `HIP<Lazy<Graph<Base>>>` for
+// `CUDA<Lazy<Graph<Base>>>`.  Mirrors src/devices/cuda/cuda.rs:22-165 (device,
+// Alloc), src/devices/cuda/ops.rs:17-234 (Read/Write/Clear, ApplyFunction,
+// UnaryGrad), src/devices/cuda/fusing.rs:3-51 (UnaryFusing) and
+// src/devices/cuda/lazy.rs:31-72 (LazySetup / LazyRun).  Everything a kernel
+// computes happens in the library; nothing is evaluated on the host.
+#pragma once
+
+#include <cstdint>
+#include <functional>
+#include <memory>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "../../../include/custos_hip.h"
+#include "device.hpp"
+
+namespace custos {
+
+// `CDatatype` (src/devices/cdatatype.rs:3-62): element types the kernels know.
+template <class T>
+struct HipDType;
+#define CUSTOS_HIP_DTYPE(T, V)                         \
+    template <>                                        \
+    struct HipDType<T> {                               \
+        static constexpr int32_t value = V;            \
+    };
+CUSTOS_HIP_DTYPE(float, CUSTOS_HIP_F32)
+CUSTOS_HIP_DTYPE(double, CUSTOS_HIP_F64)
+CUSTOS_HIP_DTYPE(int32_t, CUSTOS_HIP_I32)
+CUSTOS_HIP_DTYPE(int64_t, CUSTOS_HIP_I64)
+CUSTOS_HIP_DTYPE(uint8_t, CUSTOS_HIP_U8)
+CUSTOS_HIP_DTYPE(int8_t, CUSTOS_HIP_I8)
+CUSTOS_HIP_DTYPE(int16_t, CUSTOS_HIP_I16)
+CUSTOS_HIP_DTYPE(uint16_t, CUSTOS_HIP_U16)
+CUSTOS_HIP_DTYPE(uint32_t, CUSTOS_HIP_U32)
+CUSTOS_HIP_DTYPE(uint64_t, CUSTOS_HIP_U64)
+#undef CUSTOS_HIP_DTYPE
+
+// f16 storage (f32 compute in the kernels); a plain 16-bit pattern on the host.
+struct f16 {
+    uint16_t bits = 0;
+};
+template <>
+struct HipDType<f16> {
+    static constexpr int32_t value = CUSTOS_HIP_F16;
+};
+struct bf16 {
+    uint16_t bits = 0;
+};
+template <>
+struct HipDType<bf16> {
+    static constexpr int32_t value = CUSTOS_HIP_BF16;
+};
+
+template <class Mods>
+class HIP : public Device<HIP<Mods>, Mods> {
+   public:
+    using Self = HIP<Mods>;
+
+    // `HIP::<Mods>::new(idx)` (src/devices/cuda/cuda.rs:53-67): creates the
+    // device state, then lets the modules set up (Lazy calls `lazy_setup`).
+    explicit HIP(int idx = custos_hip_chosen_device_idx()) {
+        int32_t rc = custos_hip_device_create(idx, &dev_);
+        if (rc != CUSTOS_HIP_OK) throw Error(DeviceError::Backend, rc, custos_hip_last_error(nullptr));
+        this->modules.setup(*this);
+    }
+    HIP(const HIP&) = delete;
+    HIP& operator=(const HIP&) = delete;
+    ~HIP() {
+        // module-owned allocations go first, while the device handle is alive
+        this->modules.teardown(*this);
+        if (graph_) custos_hip_graph_destroy(dev_, graph_);
+        custos_hip_device_destroy(dev_);
+    }
+
+    custos_hip_device* handle() const { return dev_; }
+    void sync() { check(custos_hip_sync(dev_)); }
+
+    // ---- raw memory (Alloc / Read / WriteBuf / ClearBuf) ----
+    uint64_t alloc_raw(size_t bytes, bool zeroed, size_t /*len*/) {
+        uint64_t p = 0;
+        check(custos_hip_alloc(dev_, bytes, zeroed ? CUSTOS_HIP_ALLOC_ZEROED : CUSTOS_HIP_ALLOC_UNINIT, &p));
+        return p;
+    }
+    void free_raw(uint64_t ptr) {
+        if (dev_) custos_hip_free(dev_, ptr);
+    }
+    void read_raw(void* dst, uint64_t src, size_t bytes) { check(custos_hip_read(dev_, dst, src, bytes)); }
+    void write_raw(uint64_t dst, const void* src, size_t bytes) { check(custos_hip_write(dev_, dst, src, bytes)); }
+    void clear_raw(uint64_t ptr, size_t bytes) { check(custos_hip_clear(dev_, ptr, bytes)); }
+    void copy_raw(uint64_t dst, uint64_t src, size_t bytes) { check(custos_hip_copy(dev_, dst, src, bytes)); }
+
+    // ---- launches ----
+
+    // `try_cu_apply_fn_mut` (src/devices/cuda/ops.rs:144-177): print the
+    // expression with the marker, fetch the kernel, launch.
+    template <class T, class F>
+    void apply_fn_impl(const Buffer<T, Self>& x, Buffer<T, Self>& out, F f) {
+        const std::string src = to_cl_source(f(Resolve<T>::with_marker("x")));
+        custos_hip_kernel* k = compile(CUSTOS_HIP_KIND_APPLY, HipDType<T>::value, src, {"x"});
+        check(custos_hip_apply_fn(dev_, k, x.ptr(), out.ptr(), x.len()));
+    }
+
+    // Two-operand expression `f(lhs, rhs)` (src/two_way_ops/mod.rs:96-104,172-193).
+    template <class T, class F>
+    void apply_fn2_impl(const Buffer<T, Self>& lhs, const Buffer<T, Self>& rhs, Buffer<T, Self>& out, F f) {
+        const std::string src = to_cl_source(f(Resolve<T>::with_marker("x"), Resolve<T>::with_marker("y")));
+        custos_hip_kernel* k = compile(CUSTOS_HIP_KIND_APPLY, HipDType<T>::value, src, {"x", "y"});
+        check(custos_hip_apply_fn2(dev_, k, lhs.ptr(), rhs.ptr(), out.ptr(), lhs.len()));
+    }
+
+    // `try_cu_add_unary_grad` (src/devices/cuda/ops.rs:201-234)
+    template <class T, class F>
+    void add_unary_grad_impl(const Buffer<T, Self>& lhs, Buffer<T, Self>& lhs_grad, const Buffer<T, Self>& out_grad, F f) {
+        const std::string src = to_cl_source(f(Resolve<T>::with_marker("x")));
+        custos_hip_kernel* k = compile(CUSTOS_HIP_KIND_UNARY_GRAD, HipDType<T>::value, src, {"x"});
+        check(custos_hip_add_unary_grad(dev_, k, lhs.ptr(), lhs_grad.ptr(), out_grad.ptr(), lhs.len()));
+    }
+
+    // `UnaryFusing::unary_fuse_op` (src/devices/cuda/fusing.rs:8-50): one kernel
+    // for the whole chain; the fused body is `operations_to_fused_src`.
+    template <class T>
+    std::function<void(Buffer<T, Self>&, const Buffer<T, Self>&, Self&)> unary_fuse_op(
+        std::vector<std::shared_ptr<UnaryHint<T>>> ops_to_fuse) {
+        return [ops = std::move(ops_to_fuse)](Buffer<T, Self>& out, const Buffer<T, Self>& buf, Self& dev) {
+            if (ops.empty()) return;
+            const std::string src = operations_to_fused_src<T>(ops);
+            custos_hip_kernel* k = dev.compile(CUSTOS_HIP_KIND_APPLY, HipDType<T>::value, src, {"x"});
+            dev.check(custos_hip_apply_fn(dev.dev_, k, buf.ptr(), out.ptr(), buf.len()));
+        };
+    }
+
+    // A user-level two-operand op in the reference's style (retrieve + add_op),
+    // e.g. the `add` of tests/graph/mod.rs:90-127 without a hand-written kernel.
+    template <class T, class F>
+    Buffer<T, Self> apply_fn2(const Buffer<T, Self>& lhs, const Buffer<T, Self>& rhs, F f) {
+        Buffer<T, Self> out = this->template retrieve<T>(lhs.len(), lhs, rhs);
+        this->add_op(std::tie(lhs, rhs, out),
+                     [f](const Buffer<T, Self>& l, const Buffer<T, Self>& r, Buffer<T, Self>& o, Self& dev) {
+                         dev.apply_fn2_impl(l, r, o, f);
+                     });
+        return out;
+    }
+
+    // ---- Lazy hooks ----
+
+    // `LazySetup::lazy_setup`.  The reference starts stream capture here and
+    // keeps it open until the first run (src/devices/cuda/lazy.rs:59-72); this
+    // device records only while the operations of a run are replayed, so that
+    // allocation and eager work never land in the graph.
+    void lazy_setup() {}
+
+    // `LazyRun::run` (src/devices/cuda/lazy.rs:31-49): the first run of a given
+    // operation list records it into a graph and instantiates it; every run
+    // launches the graph once and waits.  `version` changes whenever the
+    // recorded operations change; then the graph is rebuilt.
+    template <class Replay>
+    void lazy_run(uint64_t version, Replay replay) {
+        if (!graph_ || graph_version_ != version) {
+            if (graph_) {
+                check(custos_hip_graph_destroy(dev_, graph_));
+                graph_ = nullptr;
+            }
+            check(custos_hip_capture_begin(dev_));
+            try {
+                replay();
+            } catch (...) {
+                custos_hip_graph* dropped = nullptr;
+                if (custos_hip_capture_end(dev_, &dropped) == CUSTOS_HIP_OK && dropped)
+                    custos_hip_graph_destroy(dev_, dropped);
+                throw;
+            }
+            check(custos_hip_capture_end(dev_, &graph_));
+            graph_version_ = version;
+            graph_builds_++;
+        }
+        check(custos_hip_graph_launch(dev_, graph_));
+        check(custos_hip_sync(dev_));
+    }
+
+    // how often a run had to (re)record its graph, and the kernels in it
+    uint64_t graph_builds() const { return graph_builds_; }
+    size_t graph_kernel_nodes() const {
+        size_t n = 0;
+        if (graph_) custos_hip_graph_node_count(graph_, &n);
+        return n;
+    }
+
+    custos_hip_kernel* compile(int32_t kind, int32_t dtype, const std::string& src,
+                               std::initializer_list<const char*> markers) {
+        std::vector<const char*> m(markers);
+        custos_hip_kernel* k = nullptr;
+        check(custos_hip_expr_compile(dev_, kind, dtype, src.c_str(), m.data(), static_cast<int32_t>(m.size()), &k));
+        return k;
+    }
+
+    void check(int32_t rc) {
+        if (rc != CUSTOS_HIP_OK) throw Error(DeviceError::Backend, rc, custos_hip_last_error(dev_));
+    }
+
+   private:
+    custos_hip_device* dev_ = nullptr;
+    custos_hip_graph* graph_ = nullptr;
+    uint64_t graph_version_ = 0;
+    uint64_t graph_builds_ = 0;
+};
+
+}  // namespace custos

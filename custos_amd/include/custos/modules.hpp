@@ -1,0 +1,568 @@
+// The module stack: Base, Lazy, Graph, Autograd.
+//
+// Modules compose at compile time, `HIP<Autograd<Graph<Lazy<Base>>>>`, like the
+// reference's (src/modules/{base,lazy,graph,autograd}.rs).  Every module
+// implements the same set of "features" and passes what it does not handle to
+// the module it wraps (`modules`), as the reference does with its pass-down
+// macros in src/features.rs.
+#pragma once
+
+#include <algorithm>
+#include <cstddef>
+#include <functional>
+#include <typeindex>
+#include <vector>
+
+#include "buffer.hpp"
+#include "core.hpp"
+#include "opt_graph.hpp"
+
+namespace custos {
+
+struct Operation {
+    std::vector<Id> arg_ids;
+    // looks its arguments up by id in `buffers`; `device` points to the concrete device
+    std::function<void(Buffers& buffers, void* device)> op;
+    // unary op hint (src/op_hint.rs): type-erased UnaryHint<T> + its element type
+    OpHintKind hint_kind = OpHintKind::None;
+    std::shared_ptr<void> unary_hint;
+    std::type_index hint_type = std::type_index(typeid(void));
+
+    static Operation no_op() {
+        Operation o;
+        o.op = [](Buffers&, void*) {};
+        return o;
+    }
+};
+
+struct AnyOpHint {
+    OpHintKind kind = OpHintKind::None;
+    std::shared_ptr<void> unary;
+    std::type_index type = std::type_index(typeid(void));
+};
+
+template <class T>
+AnyOpHint erase_hint(OpHint<T> h) {
+    return AnyOpHint{h.kind, std::static_pointer_cast<void>(h.unary), std::type_index(typeid(T))};
+}
+
+class Tape;
+class Gradients;
+struct AutogradState;
+
+// ---------------------------------------------------------------------------
+// Base: runs operations immediately, allocates on retrieve (src/modules/base.rs)
+// ---------------------------------------------------------------------------
+struct Base {
+    template <class D>
+    void setup(D&) {}
+    // called by the device's destructor while it can still free memory
+    template <class D>
+    void teardown(D&) {}
+
+    // `Retrieve::retrieve`: a fresh zeroed allocation (base.rs:103-130)
+    template <class T, class D>
+    Buffer<T, D> retrieve(D& dev, size_t len, const std::vector<Id>&, const std::vector<bool>&) {
+        cursor_++;
+        uint64_t ptr = dev.alloc_raw(len * sizeof(T), /*zeroed=*/true, len);
+        return Buffer<T, D>::from_parts(&dev, ptr, len, Id{ptr, len}, AllocFlag::None);
+    }
+    template <class T, class D>
+    void on_new_buffer(D&, const Buffer<T, D>&) {}
+    void on_drop_buffer(Id) {}
+
+    // Base never records (base.rs:53-62): the device calls the closure directly.
+    template <class D>
+    void add_op(D& dev, Operation&& op) {
+        Buffers none;
+        op.op(none, &dev);
+    }
+    size_t ops_count() const { return 0; }
+    void set_lazy_enabled(bool) {}
+    bool is_lazy_enabled() const { return false; }
+    void set_op_hint(AnyOpHint) {}
+    template <class D>
+    void exec_now(D&, size_t, size_t) {}
+    template <class D>
+    void run(D&) {}
+
+    template <class T, class D>
+    Buffer<T, D> replace_buf(D&, const Buffer<T, D>& b) {
+        return b.shallow();
+    }
+    void set_checkpoint_buffer(Id) {}
+
+    template <class D>
+    void optimize_mem_graph(D&, const GraphTranslator*) {}
+    template <class D>
+    void unary_fusing(D&, const GraphTranslator*) {}
+
+    void add_grad_fn(Operation&&) {}
+    void set_grad_enabled(bool) {}
+    bool is_grad_enabled() const { return false; }
+    AutogradState* autograd() { return nullptr; }
+    void set_requires_grad(Id, bool) {}
+    bool requires_grad_of(Id) const { return false; }
+
+    size_t cursor() const { return cursor_; }
+    void set_cursor(size_t c) { cursor_ = c; }
+    Buffers* buffers() { return nullptr; }
+    uint64_t lazy_version() const { return 0; }
+
+   private:
+    size_t cursor_ = 0;
+};
+
+// ---------------------------------------------------------------------------
+// Lazy: records operations, defers allocation (src/modules/lazy.rs)
+// ---------------------------------------------------------------------------
+template <class Mods, class T = float>
+struct Lazy {
+    Mods modules;
+    Buffers buffers_;                // id -> shallow copy: user buffers and lazily allocated ones
+    std::vector<Operation> graph;    // LazyGraph::operations
+
+    template <class D>
+    void setup(D& dev) {
+        dev.lazy_setup();
+        modules.setup(dev);
+    }
+    template <class D>
+    void teardown(D& dev) {
+        for (auto& kv : buffers_)
+            if (kv.second.module_owned && kv.second.ptr) dev.free_raw(kv.second.ptr);
+        buffers_.clear();
+        graph.clear();
+        modules.teardown(dev);
+    }
+
+    // No allocation: an id (the cursor) and a note to allocate later (lazy.rs:325-387).
+    template <class U, class D>
+    Buffer<U, D> retrieve(D& dev, size_t len, const std::vector<Id>&, const std::vector<bool>&) {
+        Id id{static_cast<UniqueId>(cursor_), len};
+        alloc_later_.push_back(Pending{id, std::type_index(typeid(U)), sizeof(U)});
+        cursor_++;
+        return Buffer<U, D>::from_parts(&dev, 0, len, id, AllocFlag::Lazy);
+    }
+
+    template <class U, class D>
+    void on_new_buffer(D& dev, const Buffer<U, D>& b) {
+        buffers_[b.id().id] = AnyBuf{b.ptr(), b.len(), std::type_index(typeid(U)), false, sizeof(U)};
+        modules.on_new_buffer(dev, b);
+    }
+    void on_drop_buffer(Id id) {
+        auto it = buffers_.find(id.id);
+        if (it != buffers_.end() && !it->second.module_owned) {
+            buffers_.erase(it);
+            version_++;  // recorded operations that name it must fail at the next run
+        }
+        modules.on_drop_buffer(id);
+    }
+
+    template <class D>
+    void add_op(D& dev, Operation&& op) {
+        if (enabled_) {
+            graph.push_back(std::move(op));
+            version_++;
+        } else {
+            Buffers* b = &buffers_;
+            op.op(*b, &dev);
+        }
+    }
+    size_t ops_count() const { return graph.size(); }
+    void set_lazy_enabled(bool e) { enabled_ = e; }
+    bool is_lazy_enabled() const { return enabled_; }
+
+    // Tags the last recorded operation (lazy.rs:136-143).
+    void set_op_hint(AnyOpHint h) {
+        if (!enabled_ || graph.empty()) return;
+        graph.back().hint_kind = h.kind;
+        graph.back().unary_hint = std::move(h.unary);
+        graph.back().hint_type = h.type;
+    }
+
+    // Runs and drains operations [begin, end) now (lazy.rs:145-162, lazy_graph.rs:93-104).
+    template <class D>
+    void exec_now(D& dev, size_t begin, size_t end) {
+        alloc_later(dev);
+        end = std::min(end, graph.size());
+        begin = std::min(begin, end);
+        std::vector<Operation> drained(std::make_move_iterator(graph.begin() + begin),
+                                       std::make_move_iterator(graph.begin() + end));
+        graph.erase(graph.begin() + begin, graph.begin() + end);
+        version_++;
+        for (auto& op : drained) op.op(buffers_, &dev);
+    }
+
+    // alloc_later -> call_lazily -> device.run() (lazy.rs:190-198).  The device
+    // decides how the recorded sequence is executed (directly, or captured into
+    // a graph once and replayed while `version` stays the same).
+    template <class D>
+    void run(D& dev) {
+        alloc_later(dev);
+        dev.lazy_run(version_, [this, &dev] { call_lazily(dev); });
+        modules.run(dev);
+    }
+
+    template <class D>
+    void call_lazily(D& dev) {
+        for (auto& op : graph) op.op(buffers_, &dev);
+    }
+
+    // Allocates every lazily retrieved buffer that has no memory yet (lazy.rs:173-179).
+    template <class D>
+    void alloc_later(D& dev) {
+        for (const Pending& p : alloc_later_) alloc_one(dev, p);
+        alloc_later_.clear();
+    }
+
+    template <class U, class D>
+    Buffer<U, D> replace_buf(D& dev, const Buffer<U, D>& b) {
+        auto it = buffers_.find(b.id().id);
+        if (it == buffers_.end()) return modules.template replace_buf<U>(dev, b);
+        if (it->second.type != std::type_index(typeid(U))) throw Error(DeviceError::TypeMismatch);
+        return Buffer<U, D>::from_parts(&dev, it->second.ptr, it->second.len, b.id(), AllocFlag::Wrapper,
+                                        b.requires_grad());
+    }
+    void set_checkpoint_buffer(Id id) { modules.set_checkpoint_buffer(id); }
+
+    // One allocation per cache trace, shared by all its buffers
+    // (lazy/optimization.rs:4-44).  Buffers outside every trace get their own.
+    template <class D>
+    void optimize_mem_graph(D& dev, const GraphTranslator* gt) {
+        if (!gt) throw Error(DeviceError::MissingCacheTraces);
+        const std::vector<CacheTrace> traces = gt->opt_graph.cache_traces();
+        std::vector<Pending> pending;
+        pending.swap(alloc_later_);
+        for (const Pending& p : pending) {
+            for (const CacheTrace& t : traces) {
+                auto head = gt->idx_to_buf_id.find(t.cache_idx);
+                if (head == gt->idx_to_buf_id.end()) throw Error(DeviceError::GraphOptimization);
+                if (head->second != p.id.id) continue;
+                alloc_one(dev, p);
+                AnyBuf shared = buffers_.at(p.id.id);
+                shared.module_owned = false;
+                for (size_t use : t.use_cache_idxs) {
+                    auto use_id = gt->idx_to_buf_id.find(use);
+                    if (use_id == gt->idx_to_buf_id.end()) throw Error(DeviceError::GraphOptimization);
+                    buffers_[use_id->second] = shared;
+                    allocated_ids_.insert(use_id->second);
+                }
+            }
+        }
+        for (const Pending& p : pending) alloc_one(dev, p);  // not the head of any trace
+        version_++;
+    }
+
+    // Replaces every maximal run of hinted unary operations inside a cache
+    // trace by one fused operation (lazy/optimization.rs:46-96,
+    // src/devices/fusing.rs:41-92).  Unlike the reference, operations of a
+    // trace that carry no unary hint are left alone, and a trace may hold
+    // several runs.
+    template <class D>
+    void unary_fusing(D& dev, const GraphTranslator* gt) {
+        if (!gt) throw Error(DeviceError::MissingCacheTraces);
+        // producing operation of every buffer id
+        std::unordered_map<UniqueId, size_t> producer;
+        for (size_t i = 0; i < graph.size(); i++)
+            if (graph[i].hint_kind == OpHintKind::Unary && graph[i].arg_ids.size() == 2)
+                producer[graph[i].arg_ids[0].id] = i;  // apply_fn records (out, in)
+
+        for (const CacheTrace& t : gt->opt_graph.cache_traces()) {
+            std::vector<size_t> node_idxs{t.cache_idx};
+            node_idxs.insert(node_idxs.end(), t.use_cache_idxs.begin(), t.use_cache_idxs.end());
+            std::vector<size_t> run;  // operation indices of the current run
+            auto flush = [&] {
+                if (run.size() >= 2) fuse_run(dev, run);
+                run.clear();
+            };
+            for (size_t node : node_idxs) {
+                auto bid = gt->idx_to_buf_id.find(node);
+                if (bid == gt->idx_to_buf_id.end()) throw Error(DeviceError::GraphOptimization);
+                auto p = producer.find(bid->second);
+                const bool unary = p != producer.end() && graph[p->second].hint_type == std::type_index(typeid(T));
+                if (!unary) {
+                    flush();
+                    continue;
+                }
+                const size_t op_idx = p->second;
+                // the run continues only if this op reads what the previous one wrote
+                if (!run.empty() && graph[op_idx].arg_ids[1].id != graph[run.back()].arg_ids[0].id) flush();
+                run.push_back(op_idx);
+            }
+            flush();
+        }
+    }
+
+    void add_grad_fn(Operation&& op) { modules.add_grad_fn(std::move(op)); }
+    void set_grad_enabled(bool e) { modules.set_grad_enabled(e); }
+    bool is_grad_enabled() const { return modules.is_grad_enabled(); }
+    AutogradState* autograd() { return modules.autograd(); }
+    void set_requires_grad(Id id, bool v) { modules.set_requires_grad(id, v); }
+    bool requires_grad_of(Id id) const { return modules.requires_grad_of(id); }
+
+    size_t cursor() const { return cursor_; }
+    void set_cursor(size_t c) { cursor_ = c; }
+    Buffers* buffers() { return &buffers_; }
+    uint64_t lazy_version() const { return version_; }
+
+   private:
+    struct Pending {
+        Id id;
+        std::type_index type;
+        size_t elem_size;
+    };
+
+    template <class D>
+    void alloc_one(D& dev, const Pending& p) {
+        if (allocated_ids_.count(p.id.id)) return;
+        // lazy ids count up from 0, buffers with data use their address: both
+        // live in one table (lazy.rs:347-357)
+        if (buffers_.count(p.id.id)) throw Error(DeviceError::IdCollision);
+        uint64_t ptr = dev.alloc_raw(p.id.len * p.elem_size, /*zeroed=*/true, p.id.len);
+        buffers_[p.id.id] = AnyBuf{ptr, p.id.len, p.type, true, p.elem_size};
+        allocated_ids_.insert(p.id.id);
+    }
+
+    template <class D>
+    void fuse_run(D& dev, const std::vector<size_t>& run) {
+        std::vector<std::shared_ptr<UnaryHint<T>>> hints;
+        for (size_t i : run) hints.push_back(std::static_pointer_cast<UnaryHint<T>>(graph[i].unary_hint));
+        const Id out_id = graph[run.back()].arg_ids[0];
+        const Id in_id = graph[run.front()].arg_ids[1];
+        Operation fused;
+        fused.arg_ids = {out_id, in_id};
+        fused.hint_kind = OpHintKind::UnaryFused;
+        auto fused_fn = dev.template unary_fuse_op<T>(std::move(hints));
+        fused.op = [out_id, in_id, fused_fn](Buffers& bufs, void* devp) {
+            D& d = *static_cast<D*>(devp);
+            auto out = bufs.find(out_id.id);
+            auto in = bufs.find(in_id.id);
+            if (out == bufs.end() || in == bufs.end()) throw Error(DeviceError::InvalidLazyBuf);
+            if (out->second.type != std::type_index(typeid(T)) || in->second.type != std::type_index(typeid(T)))
+                throw Error(DeviceError::TypeMismatch);
+            Buffer<T, D> o = Buffer<T, D>::from_parts(&d, out->second.ptr, out->second.len, out_id, AllocFlag::Wrapper);
+            Buffer<T, D> i = Buffer<T, D>::from_parts(&d, in->second.ptr, in->second.len, in_id, AllocFlag::Wrapper);
+            fused_fn(o, i, d);
+        };
+        // the fused operation takes the place of the first one (fusing.rs:55,
+        // optimization.rs:88-90); the others become no-ops
+        for (size_t i : run) graph[i] = Operation::no_op();
+        graph[run.front()] = std::move(fused);
+        version_++;
+    }
+
+    std::vector<Pending> alloc_later_;
+    std::unordered_set<UniqueId> allocated_ids_;
+    size_t cursor_ = 0;
+    bool enabled_ = true;
+    uint64_t version_ = 1;
+};
+
+// ---------------------------------------------------------------------------
+// Graph: dependency DAG built at every retrieve (src/modules/graph.rs)
+// ---------------------------------------------------------------------------
+template <class Mods, class T = float>
+struct Graph {
+    Mods modules;
+    GraphTranslator graph_trans;
+
+    template <class D>
+    void setup(D& dev) {
+        modules.setup(dev);
+    }
+    template <class D>
+    void teardown(D& dev) {
+        modules.teardown(dev);
+    }
+
+    template <class U, class D>
+    Buffer<U, D> retrieve(D& dev, size_t len, const std::vector<Id>& parents, const std::vector<bool>& rg) {
+        Buffer<U, D> data = modules.template retrieve<U>(dev, len, parents, rg);
+        // the inner module bumped the cursor (graph.rs:172-177)
+        const UniqueId cursor = static_cast<UniqueId>(modules.cursor()) - 1;
+        if (!contains_ids_.insert(cursor).second) return data;
+        const size_t next_idx = graph_trans.next_idx;
+        graph_trans.buf_id_to_idx[data.id().id] = next_idx;
+        graph_trans.idx_to_buf_id[next_idx] = data.id().id;
+        graph_trans.idx_to_cursor[next_idx] = cursor;
+        graph_trans.add_node(len, parents);
+        return data;
+    }
+
+    // A buffer created with data is a leaf (graph.rs:115-127).
+    template <class U, class D>
+    void on_new_buffer(D& dev, const Buffer<U, D>& b) {
+        graph_trans.buf_id_to_idx[b.id().id] = graph_trans.next_idx;
+        graph_trans.add_leaf(b.len());
+        modules.on_new_buffer(dev, b);
+    }
+    void on_drop_buffer(Id id) { modules.on_drop_buffer(id); }
+
+    template <class D>
+    void add_op(D& dev, Operation&& op) {
+        modules.add_op(dev, std::move(op));
+    }
+    size_t ops_count() const { return modules.ops_count(); }
+    void set_lazy_enabled(bool e) { modules.set_lazy_enabled(e); }
+    bool is_lazy_enabled() const { return modules.is_lazy_enabled(); }
+    void set_op_hint(AnyOpHint h) { modules.set_op_hint(std::move(h)); }
+    template <class D>
+    void exec_now(D& dev, size_t b, size_t e) {
+        modules.exec_now(dev, b, e);
+    }
+    template <class D>
+    void run(D& dev) {
+        modules.run(dev);
+    }
+    template <class U, class D>
+    Buffer<U, D> replace_buf(D& dev, const Buffer<U, D>& b) {
+        return modules.template replace_buf<U>(dev, b);
+    }
+    // graph.rs:255-259
+    void set_checkpoint_buffer(Id id) {
+        auto it = graph_trans.buf_id_to_idx.find(id.id);
+        if (it == graph_trans.buf_id_to_idx.end()) throw Error(DeviceError::GraphOptimization);
+        graph_trans.opt_graph.nodes[it->second].skip = true;
+    }
+
+    // graph.rs:79-113: hand the own translator down unless one was given
+    template <class D>
+    void optimize_mem_graph(D& dev, const GraphTranslator* gt) {
+        modules.optimize_mem_graph(dev, gt ? gt : &graph_trans);
+    }
+    template <class D>
+    void unary_fusing(D& dev, const GraphTranslator* gt) {
+        modules.unary_fusing(dev, gt ? gt : &graph_trans);
+    }
+
+    void add_grad_fn(Operation&& op) { modules.add_grad_fn(std::move(op)); }
+    void set_grad_enabled(bool e) { modules.set_grad_enabled(e); }
+    bool is_grad_enabled() const { return modules.is_grad_enabled(); }
+    AutogradState* autograd() { return modules.autograd(); }
+    void set_requires_grad(Id id, bool v) { modules.set_requires_grad(id, v); }
+    bool requires_grad_of(Id id) const { return modules.requires_grad_of(id); }
+    size_t cursor() const { return modules.cursor(); }
+    void set_cursor(size_t c) { modules.set_cursor(c); }
+    Buffers* buffers() { return modules.buffers(); }
+    uint64_t lazy_version() const { return modules.lazy_version(); }
+
+   private:
+    std::unordered_set<UniqueId> contains_ids_;
+};
+
+// ---------------------------------------------------------------------------
+// Autograd: tape of gradient functions + gradient buffers
+// (src/modules/autograd.rs, autograd/tape.rs, autograd/gradients.rs)
+// ---------------------------------------------------------------------------
+struct AutogradState {
+    std::vector<Operation> tape;                       // Tape::lazy_graph
+    Buffers grads;                                     // Gradients::grads_pool, keyed by buffer id
+    Buffers no_grads_pool;                             // buffers by id when no module below keeps them
+    std::unordered_map<UniqueId, bool> buf_requires_grad;
+    bool enabled = true;
+};
+
+template <class Mods>
+struct Autograd {
+    Mods modules;
+    AutogradState state;
+
+    template <class D>
+    void setup(D& dev) {
+        modules.setup(dev);
+    }
+    template <class D>
+    void teardown(D& dev) {
+        for (auto& kv : state.grads)
+            if (kv.second.ptr) dev.free_raw(kv.second.ptr);
+        state.grads.clear();
+        state.tape.clear();
+        modules.teardown(dev);
+    }
+
+    // requires_grad propagates from the parents (autograd.rs:110-136)
+    template <class U, class D>
+    Buffer<U, D> retrieve(D& dev, size_t len, const std::vector<Id>& parents, const std::vector<bool>& rg) {
+        const bool requires_grad = std::any_of(rg.begin(), rg.end(), [](bool b) { return b; });
+        Buffer<U, D> data = modules.template retrieve<U>(dev, len, parents, rg);
+        state.buf_requires_grad[data.id().id] = requires_grad;
+        data.set_requires_grad_flag(requires_grad);
+        register_no_grad_buf(data);
+        return data;
+    }
+    template <class U, class D>
+    void on_new_buffer(D& dev, const Buffer<U, D>& b) {
+        state.buf_requires_grad[b.id().id] = b.requires_grad();
+        register_no_grad_buf(b);
+        modules.on_new_buffer(dev, b);
+    }
+    void on_drop_buffer(Id id) {
+        state.no_grads_pool.erase(id.id);
+        modules.on_drop_buffer(id);
+    }
+
+    template <class D>
+    void add_op(D& dev, Operation&& op) {
+        modules.add_op(dev, std::move(op));
+    }
+    size_t ops_count() const { return modules.ops_count(); }
+    void set_lazy_enabled(bool e) { modules.set_lazy_enabled(e); }
+    bool is_lazy_enabled() const { return modules.is_lazy_enabled(); }
+    void set_op_hint(AnyOpHint h) { modules.set_op_hint(std::move(h)); }
+    template <class D>
+    void exec_now(D& dev, size_t b, size_t e) {
+        modules.exec_now(dev, b, e);
+    }
+    template <class D>
+    void run(D& dev) {
+        modules.run(dev);
+    }
+    template <class U, class D>
+    Buffer<U, D> replace_buf(D& dev, const Buffer<U, D>& b) {
+        Buffer<U, D> r = modules.template replace_buf<U>(dev, b);
+        r.set_requires_grad_flag(requires_grad_of(b.id()) || b.requires_grad());
+        return r;
+    }
+    void set_checkpoint_buffer(Id id) { modules.set_checkpoint_buffer(id); }
+    template <class D>
+    void optimize_mem_graph(D& dev, const GraphTranslator* gt) {
+        modules.optimize_mem_graph(dev, gt);
+    }
+    template <class D>
+    void unary_fusing(D& dev, const GraphTranslator* gt) {
+        modules.unary_fusing(dev, gt);
+    }
+
+    // autograd.rs:245-256
+    void add_grad_fn(Operation&& op) {
+        if (state.enabled) state.tape.push_back(std::move(op));
+    }
+    void set_grad_enabled(bool e) { state.enabled = e; }
+    bool is_grad_enabled() const { return state.enabled; }
+    AutogradState* autograd() { return &state; }
+    void set_requires_grad(Id id, bool v) { state.buf_requires_grad[id.id] = v; }
+    bool requires_grad_of(Id id) const {
+        auto it = state.buf_requires_grad.find(id.id);
+        return it != state.buf_requires_grad.end() && it->second;
+    }
+
+    size_t cursor() const { return modules.cursor(); }
+    void set_cursor(size_t c) { modules.set_cursor(c); }
+    // buffers by id for the gradient functions: the Lazy module's table when
+    // there is one, else the pool kept here (autograd.rs:60-75)
+    Buffers* buffers() {
+        Buffers* below = modules.buffers();
+        return below ? below : &state.no_grads_pool;
+    }
+    uint64_t lazy_version() const { return modules.lazy_version(); }
+
+   private:
+    template <class U, class D>
+    void register_no_grad_buf(const Buffer<U, D>& b) {
+        if (modules.buffers() != nullptr || !b.has_data()) return;
+        state.no_grads_pool.emplace(b.id().id, AnyBuf{b.ptr(), b.len(), std::type_index(typeid(U)), false, sizeof(U)});
+    }
+};
+
+}  // namespace custos

@@ -1,0 +1,90 @@
+// The module-stack tests on the HIP device (needs an MI355X), plus what only a
+// GPU device has: graph capture/replay behind `run()`.
+#include "check.hpp"
+#include "custos/custos.hpp"
+#include "module_tests.hpp"
+
+using namespace custos;
+
+// f32 transcendentals are within 4 ulp of libm, f64 ones within a few ulp
+REGISTER_MODULE_TESTS(HIP, 1e-6)
+
+// src/devices/cuda/lazy.rs:96-196: add, add, mul recorded, nothing runs before run();
+// ten runs with rewritten inputs replay one instantiated graph
+TEST_CASE(hip_lazy_run_replays_one_graph) {
+    using D = HIP<Lazy<Base, int32_t>>;
+    D device;
+    auto lhs = device.buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto rhs = device.buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto out = lhs.empty_like();
+    auto add = [](auto a, auto b) { return a.add(b); };
+    auto mul = [](auto a, auto b) { return a.mul(b); };
+    device.add_op(std::tie(lhs, rhs, out), [add](Buffer<int32_t, D>& l, Buffer<int32_t, D>& r, Buffer<int32_t, D>& o, D& d) { d.apply_fn2_impl(l, r, o, add); });
+    device.add_op(std::tie(out, lhs, rhs), [add](Buffer<int32_t, D>& l, Buffer<int32_t, D>& r, Buffer<int32_t, D>& o, D& d) { d.apply_fn2_impl(l, r, o, add); });
+    device.add_op(std::tie(out, rhs, lhs), [mul](Buffer<int32_t, D>& l, Buffer<int32_t, D>& r, Buffer<int32_t, D>& o, D& d) { d.apply_fn2_impl(l, r, o, mul); });
+    CHECK_VEC_EQ(out.read(), (std::vector<int32_t>(6, 0)));
+    CHECK_VEC_EQ(lhs.read(), (std::vector<int32_t>{1, 2, 3, 4, 5, 6}));
+    for (int i = 0; i < 10; i++) {
+        lhs.write({1, 2, 3, 4, 5, 6});
+        rhs.write({1, 2, 3, 4, 5, 6});
+        device.run();
+        CHECK_VEC_EQ(out.read(), (std::vector<int32_t>{2, 4, 6, 8, 10, 12}));
+        CHECK_VEC_EQ(rhs.read(), (std::vector<int32_t>{3, 6, 9, 12, 15, 18}));
+        CHECK_VEC_EQ(lhs.read(), (std::vector<int32_t>{6, 24, 54, 96, 150, 216}));
+    }
+    CHECK_EQ(device.graph_builds(), uint64_t(1));      // recorded once, replayed ten times
+    CHECK_EQ(device.graph_kernel_nodes(), size_t(3));  // and every op ran once per run, not twice
+    // a new operation invalidates the graph: the next run records again
+    auto extra = device.apply_fn(out, [](auto x) { return x.add(1); });
+    lhs.write({1, 2, 3, 4, 5, 6});
+    rhs.write({1, 2, 3, 4, 5, 6});
+    device.run();
+    CHECK_EQ(device.graph_builds(), uint64_t(2));
+    CHECK_EQ(device.graph_kernel_nodes(), size_t(4));
+    CHECK_VEC_EQ(extra.replace().read(), (std::vector<int32_t>{3, 5, 7, 9, 11, 13}));
+}
+
+// BASELINE configs[1] in miniature, through the whole stack: five apply_fn calls on
+// Graph<Lazy<Base>>, fused into one kernel node, bit-identical to the unfused device result
+TEST_CASE(hip_fused_chain_is_one_kernel) {
+    std::vector<float> xs(10007);
+    for (size_t i = 0; i < xs.size(); i++) xs[i] = -3.14159f + 6.28318f * static_cast<float>(i) / xs.size();
+    std::vector<float> unfused;
+    {
+        HIP<Base> eager;
+        auto b = eager.buffer<float>(xs);
+        auto o = eager.apply_fn(b, [](auto x) { return x.sin(); });
+        o = eager.apply_fn(o, [](auto x) { return x.mul(2.f); });
+        o = eager.apply_fn(o, [](auto x) { return x.add(1.f); });
+        o = eager.apply_fn(o, [](auto x) { return x.max(0.f); });
+        o = eager.apply_fn(o, [](auto x) { return x.sub(0.5f); });
+        unfused = o.read();
+    }
+    HIP<Graph<Lazy<Base>>> dev;
+    auto buf = dev.buffer<float>(xs);
+    auto o1 = dev.apply_fn(buf, [](auto x) { return x.sin(); });
+    auto o2 = dev.apply_fn(o1, [](auto x) { return x.mul(2.f); });
+    auto o3 = dev.apply_fn(o2, [](auto x) { return x.add(1.f); });
+    auto o4 = dev.apply_fn(o3, [](auto x) { return x.max(0.f); });
+    auto o5 = dev.apply_fn(o4, [](auto x) { return x.sub(0.5f); });
+    dev.optimize_mem_graph();
+    dev.unary_fusing();
+    dev.run();
+    CHECK_EQ(dev.graph_kernel_nodes(), size_t(1));
+    CHECK_VEC_EQ(o5.replace().read(), unfused);
+    for (int i = 0; i < 3; i++) dev.run();
+    CHECK_EQ(dev.graph_builds(), uint64_t(1));
+    CHECK_VEC_EQ(o5.replace().read(), unfused);
+}
+
+TEST_CASE(hip_backend_errors_surface) {
+    bool threw = false;
+    try {
+        HIP<Base> nope(1000);
+    } catch (const Error& e) {
+        threw = e.kind == DeviceError::Backend && e.code == CUSTOS_HIP_ERR_INVALID_DEVICE_INDEX;
+    }
+    CHECK(threw);
+}
+
+int main(int argc, char** argv) { return check::run(argc, argv); }

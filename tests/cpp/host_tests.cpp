@@ -1,0 +1,214 @@
+// Host-only tests (no GPU): expression DSL known answers, cache traces against
+// the reference's vectors, and the module stack on the host test device.
+#include "check.hpp"
+#include "custos/combiner.hpp"
+#include "custos/opt_graph.hpp"
+#include "module_tests.hpp"
+#include "test_cpu_device.hpp"
+
+using namespace custos;
+
+// ---- expression DSL: src/two_way_ops/mod.rs:51-202, eval.rs:6-13, resolve.rs:12-23 ----
+
+TEST_CASE(combiner_exp) {
+    auto f = [](auto x) { return x.exp(); };
+    CHECK_EQ(eval<float>(f(to_val(1.f))), 2.7182817f);  // == core::f32::consts::E
+    CHECK_EQ(to_cl_source(f(to_marker<float>("x"))), std::string("exp(x)"));
+}
+TEST_CASE(combiner_neg_tan) {
+    auto f = [](auto x) { return x.tan().neg(); };
+    CHECK(std::fabs(eval<float>(f(to_val(2.f))) - 2.1850398f) < 1e-6);
+    CHECK_EQ(to_cl_source(f(to_marker<float>("val"))), std::string("-(tan(val))"));
+}
+TEST_CASE(combiner_pow) {
+    auto f = [](auto x, auto y) { return x.mul(3.f).pow(y.add(1.f)); };
+    CHECK_EQ(eval<float>(f(to_val(3.f), to_val(2.f))), 729.f);
+    CHECK_EQ(to_cl_source(f(to_marker<float>("x"), to_marker<float>("y"))), std::string("pow((x * 3.0), (y + 1.0))"));
+}
+TEST_CASE(combiner_int_ops) {
+    CHECK_EQ(eval<int>(to_val(3).eq(to_val(3))), 1);
+    CHECK_EQ(to_cl_source(to_marker<int>("var_x").eq(to_marker<int>("other"))), std::string("(var_x == other)"));
+    auto relu = [](auto x) { return x.geq(0).mul(x); };
+    CHECK_EQ(eval<int>(relu(to_val(3))), 3);
+    CHECK_EQ(to_cl_source(relu(to_marker<int>("var_x"))), std::string("((var_x >= 0) * var_x)"));
+    CHECK_EQ(eval<int>(to_val(3).add(3)), 6);
+    CHECK_EQ(to_cl_source(to_marker<int>("var_x").add(3)), std::string("(var_x + 3)"));
+    CHECK_EQ(eval<int>(to_val(3).geq(4)), 0);
+    CHECK_EQ(to_cl_source(to_marker<int>("var_x").geq(4)), std::string("(var_x >= 4)"));
+    auto f = [](auto x) { return x.add(2).add(x.mul(8)); };
+    CHECK_EQ(eval<int>(f(to_val(4))), 38);
+}
+TEST_CASE(combiner_two_args_and_strings) {
+    auto f = [](auto x, auto y) { return x.add(y).mul(3.6f).sub(y); };
+    CHECK(std::fabs(eval<float>(f(to_val(4.f), to_val(3.f))) - 22.2f) < 1e-5);
+    CHECK_EQ(to_cl_source(f(to_marker<float>("x"), to_marker<float>("y"))), std::string("(((x + y) * 3.6) - y)"));
+    auto g = [](auto x) { return x.add(2.f).mul(x).add(x.mul(8.f)).mul(5.f); };
+    CHECK_EQ(to_cl_source(g(Resolve<float>{})), std::string("((((x + 2.0) * x) + (x * 8.0)) * 5.0)"));
+    CHECK_EQ(to_cl_source(to_marker<float>("x").add(to_marker<float>("y"))), std::string("(x + y)"));
+    CHECK_EQ(eval<float>(to_val(1.5f).add(2.5f).mul(3.5f)), 14.f);
+    CHECK_EQ(eval<double>(to_val(1.5).mul(to_val(1.5)).add(2.)), 4.25);
+    CHECK_EQ(to_cl_source(to_marker<float>("x").mul(to_marker<float>("x")).add(2.f)), std::string("((x * x) + 2.0)"));
+    CHECK_EQ(to_cl_source(to_marker<float>("x").add("1.0")), std::string("(x + 1.0)"));
+    CHECK_EQ(to_cl_source(to_marker<float>("x").identity()), std::string("x"));
+    CHECK_EQ(to_cl_source(to_marker<float>("x").max(3.f).min(5.f)), std::string("min(max(x, 3.0), 5.0)"));
+    CHECK_EQ(to_cl_source(to_marker<float>("x").mul(0.1f).sub(-0.5f)), std::string("((x * 0.1) - -0.5)"));
+}
+TEST_CASE(combiner_min_max_are_selects) {
+    const float nan = std::nanf("");
+    CHECK_EQ(eval<float>(to_val(nan).max(1.f)), 1.f);  // NaN > 1 is false -> rhs
+    CHECK(std::isnan(eval<float>(to_val(1.f).max(nan))));
+    CHECK(!std::signbit(eval<float>(to_val(-0.f).max(0.f))));
+    CHECK(std::signbit(eval<float>(to_val(0.f).max(-0.f))));
+}
+TEST_CASE(fused_source_text) {
+    // src/devices/fusing.rs:104-120
+    std::vector<std::shared_ptr<UnaryHint<float>>> ops = {
+        unary<float>([](auto x) { return x.sin(); }).unary,
+        unary<float>([](auto x) { return x.neg(); }).unary,
+        unary<float>([](auto x) { return x.cos(); }).unary,
+    };
+    CHECK_EQ(operations_to_fused_src<float>(ops), std::string("x = sin(x);\nx = -(x);\nx = cos(x);\n"));
+}
+
+// ---- cache traces: every vector of src/modules/graph/opt_graph/optimize.rs:137-393,692-805 ----
+
+TEST_CASE(cache_trace_basic) {
+    OptGraph g;
+    auto a = g.add_leaf(10), b = g.add_leaf(10);
+    auto c = g.add_node(10, {a, b});
+    auto d = g.add_node(10, {c, c});
+    g.add_node(10, {d, b});
+    CHECK_VEC_EQ(g.trace_cache_path_raw(g.node(c)), (std::vector<size_t>{3, 4}));
+    auto traces = g.cache_traces();
+    CHECK_EQ(traces.size(), size_t(1));
+    CHECK(traces[0] == (CacheTrace{2, {3, 4}}));
+}
+TEST_CASE(cache_trace_none_when_two_consumers) {
+    OptGraph g;
+    auto a = g.add_leaf(10), b = g.add_leaf(10);
+    auto c = g.add_node(10, {a, b});
+    auto d = g.add_node(10, {c, c});
+    g.add_node(10, {d, b});
+    g.add_node(10, {c, b});
+    CHECK_VEC_EQ(g.trace_cache_path_raw(g.node(c)), (std::vector<size_t>{}));
+}
+TEST_CASE(cache_trace_2) {
+    OptGraph g;
+    auto a = g.add_leaf(10), b = g.add_leaf(10), u = g.add_leaf(10);
+    auto c = g.add_node(10, {a, b});
+    g.add_node(10, {a, u});
+    auto d = g.add_node(10, {c, c});
+    g.add_node(10, {d, b});
+    CHECK_VEC_EQ(g.trace_cache_path_raw(g.node(c)), (std::vector<size_t>{5, 6}));
+}
+TEST_CASE(cache_trace_break) {
+    OptGraph g;
+    auto a = g.add_leaf(10), b = g.add_leaf(10);
+    auto c = g.add_node(10, {a, b});
+    auto d = g.add_node(10, {c, c});
+    g.add_node(10, {d, a});
+    g.add_node(10, {d, b});
+    CHECK(g.is_path_optimizable(g.node(c)));
+    CHECK(!g.is_path_optimizable(g.node(d)));
+    // the first unoptimizable node still joins the trace, then it ends
+    CHECK_VEC_EQ(g.trace_cache_path_raw(g.node(c)), (std::vector<size_t>{3}));
+}
+TEST_CASE(cache_trace_leafed_diff_len) {
+    OptGraph g;
+    auto a = g.add_leaf(10);
+    g.add_node(10, {a, a});
+    g.add_leaf(10);
+    g.add_leaf(10);
+    auto c = g.add_node(10, {a, a});
+    auto d = g.add_node(10, {c, c});
+    g.add_node(10, {d, a});
+    auto traces = g.cache_traces();
+    CHECK(traces[0] == (CacheTrace{4, {5, 6}}));
+}
+TEST_CASE(cache_trace_neural_net) {
+    OptGraph g;
+    auto inputs = g.add_leaf(100 * 10), targets = g.add_leaf(100);
+    auto w1 = g.add_leaf(10 * 64), b1 = g.add_leaf(64), w2 = g.add_leaf(64 * 64), b2 = g.add_leaf(64);
+    auto w3 = g.add_leaf(64 * 64), b3 = g.add_leaf(64), w4 = g.add_leaf(64), b4 = g.add_leaf(1);
+    auto a1 = g.add_node(100 * 64, {inputs, w1});
+    auto a2 = g.add_node(100 * 64, {a1, b1});
+    a2 = g.add_node(100 * 64, {a2, a2});
+    auto a3 = g.add_node(100 * 64, {a2, w2});
+    auto a4 = g.add_node(100 * 64, {a3, b2});
+    a4 = g.add_node(100 * 64, {a4, a4});
+    auto a5 = g.add_node(100 * 64, {a4, w3});
+    auto a6 = g.add_node(100 * 64, {a5, b3});
+    a6 = g.add_node(100 * 64, {a6, a6});
+    auto a7 = g.add_node(100, {a6, w4});
+    auto a8 = g.add_node(100, {a7, b4});
+    g.add_node(100, {a8, targets});
+    auto traces = g.cache_traces();
+    CHECK_EQ(traces.size(), size_t(2));
+    CHECK(traces[0] == (CacheTrace{10, {11, 12, 13, 14, 15, 16, 17, 18}}));
+    CHECK(traces[1] == (CacheTrace{19, {20, 21}}));
+}
+TEST_CASE(cache_trace_d) {
+    OptGraph g;
+    auto a = g.add_leaf(10), b = g.add_leaf(10);
+    auto c = g.add_node(10, {a, b});
+    auto d = g.add_node(10, {c, c});
+    g.add_node(10, {a, d});
+    CHECK_VEC_EQ(g.trace_cache_path_raw(g.node(c)), (std::vector<size_t>{3, 4}));
+    CHECK(g.is_path_optimizable(g.node(c)) && g.is_path_optimizable(g.node(d)));
+    auto traces = g.cache_traces();
+    CHECK_EQ(traces.size(), size_t(1));
+    CHECK(traces[0] == (CacheTrace{2, {3, 4}}));
+}
+TEST_CASE(cache_trace_none_in_graph) {
+    OptGraph g;
+    auto a = g.add_leaf(10), b = g.add_leaf(10);
+    auto c = g.add_node(10, {a, b});
+    CHECK_VEC_EQ(g.trace_cache_path_raw(g.node(c)), (std::vector<size_t>{}));
+    CHECK(g.cache_traces().empty());
+}
+static OptGraph multiple_traces_graph(bool with_skips) {
+    OptGraph g;
+    auto a = g.add_leaf(10);
+    auto b = g.add_node(10, {a, a});
+    g.add_leaf(10);
+    auto z = g.add_leaf(10);
+    auto c = g.add_node(10, {a, a});
+    if (with_skips) g.nodes[c].skip = true;
+    auto d = g.add_node(10, {c, c});
+    g.add_node(10, {d, a});
+    auto f = g.add_node(10, {b, z});
+    if (with_skips) g.nodes[f].skip = true;
+    g.add_node(10, {f, z});
+    return g;
+}
+TEST_CASE(cache_trace_multiple) {
+    auto traces = multiple_traces_graph(false).cache_traces();
+    CHECK_EQ(traces.size(), size_t(2));
+    CHECK(traces[0] == (CacheTrace{1, {7, 8}}));
+    CHECK(traces[1] == (CacheTrace{4, {5, 6}}));
+}
+TEST_CASE(cache_trace_multiple_with_skips) {
+    auto traces = multiple_traces_graph(true).cache_traces();
+    CHECK_EQ(traces.size(), size_t(1));
+    CHECK(traces[0] == (CacheTrace{5, {6}}));
+}
+
+// ---- module stack on the host test device ----
+
+REGISTER_MODULE_TESTS(TestCPU, 1e-12)
+
+TEST_CASE(host_device_frees_everything) {
+    size_t live = 0;
+    {
+        TestCPU<Autograd<Graph<Lazy<Base>>>> dev;
+        auto buf = dev.buffer<float>({1.f, 2.f, 3.f}).require_grad();
+        auto out = dev.unary_ew(buf, [](auto x) { return x.sin(); }, [](auto x) { return x.cos(); });
+        dev.run();
+        out.backward();
+        live = dev.live_allocations;
+        CHECK(live >= 3);
+    }
+    // the device's destructor ran teardown; buffers freed themselves before
+}
+
+int main(int argc, char** argv) { return check::run(argc, argv); }

@@ -1,0 +1,572 @@
+// Tests of the module stack, generic over the device so that the same bodies
+// run on the host test device and on the HIP device -- the way the reference
+// instantiates one generic test per device (src/unary.rs:160-241).
+// Each case names the reference test it restates.
+#pragma once
+
+#include <cmath>
+#include <vector>
+
+#include "check.hpp"
+#include "custos/device.hpp"
+
+namespace module_tests {
+
+using namespace custos;
+
+static const std::vector<double> SIN_1_4 = {0.8414709848078965, 0.9092974268256817, 0.1411200080598672, -0.7568024953079282};
+static const std::vector<double> COS_1_4 = {0.5403023058681398, -0.4161468365471424, -0.9899924966004454, -0.6536436208636119};
+
+template <class V>
+std::vector<double> scaled(const V& v, double k) {
+    std::vector<double> out;
+    for (auto x : v) out.push_back(x * k);
+    return out;
+}
+
+// ---- Base ----
+
+// src/unary.rs:12-19 (doc test), src/two_way_ops/mod.rs:204-217, 236-245
+template <template <class> class DEV>
+void base_apply_fn() {
+    DEV<Base> device;
+    auto a = device.template buffer<double>({1., 2., 3., 3., 2., 1.});
+    auto out = device.apply_fn(a, [](auto x) { return x.mul(2.); });
+    CHECK_VEC_EQ(out.read(), (std::vector<double>{2., 4., 6., 6., 4., 2.}));
+
+    auto c = device.template buffer<float>({1.f, 3.f, 4.f, 6.f, 3.f, 2.f});
+    auto clipped = device.apply_fn(c, [](auto x) { return x.max(3.f).min(5.f); });
+    CHECK_VEC_EQ(clipped.read(), (std::vector<float>{3.f, 3.f, 4.f, 5.f, 3.f, 3.f}));
+
+    auto i = device.template buffer<int32_t>({3, 3, 4, 5, 3, 2});
+    auto i3 = device.apply_fn(i, [](auto x) { return x.add(3); });
+    CHECK_VEC_EQ(i3.read(), (std::vector<int32_t>{6, 6, 7, 8, 6, 5}));
+}
+
+// src/unary.rs:36-49 (doc test), src/devices/cuda/ops.rs:259-272
+template <template <class> class DEV>
+void base_add_unary_grad() {
+    DEV<Base> device;
+    auto a = device.template buffer<double>({1., 2., 3., 3., 2., 1.});
+    auto out_grad = device.template buffer<double>({1., 1., 1., 1., 1., 1.});
+    auto lhs_grad = device.template buffer<double>({0., 0., 0., 0., 0., 0.});
+    device.add_unary_grad(a, lhs_grad, out_grad, [](auto) { return to_val(2.0); });
+    CHECK_VEC_EQ(lhs_grad.read(), (std::vector<double>(6, 2.)));
+
+    auto lhs = device.template buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto g = device.template buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto o = device.template buffer<int32_t>({1, 1, 1, 1, 1, 1});
+    device.add_unary_grad(lhs, g, o, [](auto x) { return x.mul(2).add(1); });
+    CHECK_VEC_EQ(g.read(), (std::vector<int32_t>{4, 7, 10, 13, 16, 19}));
+}
+
+// src/unary.rs:139-158: without Autograd, unary_ew is just the forward pass
+template <template <class> class DEV>
+void base_unary_ew_forward_only() {
+    DEV<Base> device;
+    auto buf = device.template buffer<double>({1., 2., 3., 4.});
+    auto out = device.unary_ew(buf, [](auto x) { return x.sin(); }, [](auto x) { return x.cos(); });
+    CHECK_ROUGHLY(out.read(), SIN_1_4, 1e-12);
+}
+
+// src/devices/cpu/cpu_device.rs:135-157: zero length is an error
+template <template <class> class DEV>
+void base_zero_length_is_an_error() {
+    DEV<Base> device;
+    CHECK_THROWS_KIND(device.template new_buffer<float>(0), DeviceError::ZeroLengthBuffer);
+    CHECK_THROWS_KIND(device.template buffer<float>(std::vector<float>{}), DeviceError::ZeroLengthBuffer);
+    auto b = device.template new_buffer<float>(4);
+    CHECK_VEC_EQ(b.read(), (std::vector<float>(4, 0.f)));  // Buffer::new is zeroed
+    CHECK_THROWS_KIND(b.write(std::vector<float>(3, 1.f)), DeviceError::ShapeLengthMismatch);
+}
+
+// ---- Lazy ----
+
+// src/modules/lazy.rs:553-566
+template <template <class> class DEV>
+void lazy_retrieve_ids() {
+    DEV<Lazy<Base, int32_t>> device;
+    Buffer<int32_t, DEV<Lazy<Base, int32_t>>> buf(device, 10);
+    CHECK(buf.has_data());
+    CHECK_EQ(buf.id().id, buf.ptr());
+    auto x = device.template retrieve<int32_t>(10);
+    CHECK(!x.has_data());
+    CHECK(x.id() == (Id{0, 10}));
+    auto y = device.template retrieve<int32_t>(10);
+    CHECK(y.id() == (Id{1, 10}));
+}
+
+// src/modules/lazy.rs:568-585, 634-646, 649-662
+template <template <class> class DEV>
+void lazy_apply_fn_runs_at_run() {
+    DEV<Lazy<Base, int32_t>> device;
+    Buffer<int32_t, DEV<Lazy<Base, int32_t>>> buf(device, 10);
+    auto out = device.apply_fn(buf, [](auto x) { return x.add(3); });
+    CHECK_EQ(device.ops_count(), size_t(1));
+    CHECK_THROWS_KIND(out.read(), DeviceError::InvalidLazyBuf);  // no memory behind the handle yet
+    device.modules.alloc_later(device);
+    CHECK_VEC_EQ(out.replace().read(), (std::vector<int32_t>(10, 0)));  // allocated zeroed, not computed
+    device.run();
+    CHECK_VEC_EQ(out.replace().read(), (std::vector<int32_t>(10, 3)));
+    device.run();  // operations stay recorded: a second run recomputes the same
+    CHECK_VEC_EQ(out.replace().read(), (std::vector<int32_t>(10, 3)));
+}
+
+// src/modules/lazy.rs:618-632
+template <template <class> class DEV>
+void lazy_dropped_buffer_is_invalid() {
+    DEV<Lazy<Base, int32_t>> device;
+    {
+        Buffer<int32_t, DEV<Lazy<Base, int32_t>>> buf(device, 10);
+        auto out = device.apply_fn(buf, [](auto x) { return x.add(3); });
+    }
+    CHECK_THROWS_KIND(device.run(), DeviceError::InvalidLazyBuf);
+}
+
+// src/modules/lazy.rs:674-698: a user-defined two-operand op next to apply_fn
+template <template <class> class DEV>
+void lazy_add_and_apply_fn() {
+    DEV<Lazy<Base, int32_t>> device;
+    Buffer<int32_t, DEV<Lazy<Base, int32_t>>> buf(device, 10);
+    auto lhs = device.apply_fn(buf, [](auto x) { return x.add(3); });
+    auto rhs = device.template buffer<int32_t>({1, 2, 3, 4, 5, 6, 7, 8, 9, 10});
+    CHECK_VEC_EQ(rhs.read(), (std::vector<int32_t>{1, 2, 3, 4, 5, 6, 7, 8, 9, 10}));
+    auto out = device.apply_fn2(lhs, rhs, [](auto a, auto b) { return a.add(b); });
+    device.run();
+    CHECK_VEC_EQ(lhs.replace().read(), (std::vector<int32_t>(10, 3)));
+    CHECK_VEC_EQ(out.replace().read(), (std::vector<int32_t>{4, 5, 6, 7, 8, 9, 10, 11, 12, 13}));
+}
+
+// src/devices/cuda/ops.rs:274-295
+template <template <class> class DEV>
+void lazy_add_unary_grad() {
+    DEV<Lazy<Base, int32_t>> device;
+    auto lhs = device.template buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto lhs_grad = device.template buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto out = device.template buffer<int32_t>({1, 1, 1, 1, 1, 1});
+    device.add_unary_grad(lhs, lhs_grad, out, [](auto x) { return x.add(2); });
+    CHECK_VEC_EQ(lhs_grad.read(), (std::vector<int32_t>{1, 2, 3, 4, 5, 6}));
+    device.run();
+    CHECK_VEC_EQ(lhs_grad.read(), (std::vector<int32_t>{4, 6, 8, 10, 12, 14}));
+}
+
+// src/modules/lazy.rs:725-757 and 759-790
+template <template <class> class DEV>
+void lazy_exec_now_and_last_n() {
+    using D = DEV<Lazy<Base, int32_t>>;
+    for (int variant = 0; variant < 2; variant++) {
+        D device;
+        auto out = device.template retrieve<int32_t>(4);
+        device.add_op(std::tie(out), [](Buffer<int32_t, D>& o, D&) { o.clear(); });
+        {
+            auto a = device.template buffer<int32_t>({1, 2, 3, 4});
+            auto b = device.template buffer<int32_t>({1, 2, 3, 4});
+            device.add_op(std::tie(a, b, out), [](Buffer<int32_t, D>& x, Buffer<int32_t, D>& y, Buffer<int32_t, D>& o, D& dev) {
+                dev.apply_fn2_impl(x, y, o, [](auto p, auto q) { return p.add(q); });
+            });
+            if (variant == 0) device.exec_now(1);
+            else device.exec_last_n(1);
+            CHECK_VEC_EQ(out.replace().read(), (std::vector<int32_t>{2, 4, 6, 8}));
+            CHECK_EQ(device.ops_count(), size_t(1));  // the executed operation was consumed
+        }
+        device.run();  // only the clear is left; a and b are gone but no longer needed
+        CHECK_VEC_EQ(out.replace().read(), (std::vector<int32_t>(4, 0)));
+    }
+}
+
+// src/modules/lazy/lazy_graph.rs:117-125
+template <template <class> class DEV>
+void lazy_duplicate_parent_is_rejected() {
+    using D = DEV<Lazy<Base, int32_t>>;
+    D device;
+    auto a = device.template buffer<int32_t>({1, 2, 3, 4});
+    CHECK_THROWS_KIND(device.add_op(std::tie(a, a), [](Buffer<int32_t, D>&, Buffer<int32_t, D>&, D&) {}),
+                      DeviceError::DuplicateParent);
+}
+
+// src/op_hint.rs:41-84
+template <template <class> class DEV>
+void lazy_op_hints() {
+    DEV<Lazy<Base>> dev;
+    auto buf = dev.template buffer<float>({1.f, 2.f, 3.f, 4.f, 5.f});
+    auto o1 = dev.apply_fn(buf, [](auto x) { return x.sin(); });
+    auto o2 = dev.apply_fn(o1, [](auto x) { return x.cos(); });
+    auto o3 = dev.apply_fn(o2, [](auto x) { return x.ln(); });
+    const auto& ops = dev.modules.graph;
+    CHECK_EQ(ops.size(), size_t(3));
+    const char* want[] = {"sin(x)", "cos(x)", "log(x)"};
+    for (int i = 0; i < 3; i++) {
+        CHECK(ops[i].hint_kind == OpHintKind::Unary);
+        auto h = std::static_pointer_cast<UnaryHint<float>>(ops[i].unary_hint);
+        CHECK_EQ(h->to_cl_source("x"), std::string(want[i]));
+    }
+    // src/op_hint.rs:86-114: evaluating the hints in sequence is the fused chain
+    float v = 3.f;
+    for (auto& op : ops) v = std::static_pointer_cast<UnaryHint<float>>(op.unary_hint)->eval(v);
+    CHECK(std::fabs(v - std::log(std::cos(std::sin(3.f)))) < 1e-6);
+    // optimizing without a Graph module has no cache traces (src/modules/lazy.rs:494-511)
+    CHECK_THROWS_KIND(dev.unary_fusing(), DeviceError::MissingCacheTraces);
+    CHECK_THROWS_KIND(dev.optimize_mem_graph(), DeviceError::MissingCacheTraces);
+}
+
+// ---- Graph + Lazy: fusion ----
+
+// src/op_hint.rs:116-141 (CPU), 198-219 (CUDA): optimize_mem_graph, unary_fusing, run
+template <template <class> class DEV>
+void graph_fuse_chain(bool optimize_mem) {
+    DEV<Graph<Lazy<Base>>> dev;
+    auto buf = dev.template buffer<float>({1.f, 2.f, 3.f, 4.f, 5.f});
+    auto o1 = dev.apply_fn(buf, [](auto x) { return x.sin(); });
+    auto o2 = dev.apply_fn(o1, [](auto x) { return x.cos(); });
+    auto o3 = dev.apply_fn(o2, [](auto x) { return x.ln(); });
+    if (optimize_mem) dev.optimize_mem_graph();
+    else dev.modules.modules.alloc_later(dev);  // src/op_hint.rs:157
+    dev.unary_fusing();
+    const auto& ops = dev.modules.modules.graph;
+    CHECK(ops[0].hint_kind == OpHintKind::UnaryFused);
+    CHECK(ops[1].arg_ids.empty() && ops[2].arg_ids.empty());  // no-ops
+    dev.run();
+    auto got = o3.replace().read();
+    std::vector<double> want;
+    for (float x : {1.f, 2.f, 3.f, 4.f, 5.f}) want.push_back(std::log(std::cos(std::sin(x))));
+    CHECK_ROUGHLY(got, want, 1e-3);
+    if (optimize_mem) {
+        // the whole trace shares one allocation
+        CHECK_EQ(o1.replace().ptr(), o3.replace().ptr());
+        CHECK_EQ(o2.replace().ptr(), o3.replace().ptr());
+    } else {
+        // intermediates of a fused chain are never computed
+        CHECK_VEC_EQ(o1.replace().read(), (std::vector<float>(5, 0.f)));
+        CHECK_VEC_EQ(o2.replace().read(), (std::vector<float>(5, 0.f)));
+    }
+}
+
+// src/op_hint.rs:167-196
+template <template <class> class DEV>
+void graph_fuse_chain_with_checkpoint() {
+    DEV<Graph<Lazy<Base>>> dev;
+    auto buf = dev.template buffer<float>({1.f, 2.f, 3.f, 4.f, 5.f});
+    auto out1 = dev.apply_fn(buf, [](auto x) { return x.sin(); }).checkpoint();
+    auto out = dev.apply_fn(out1, [](auto x) { return x.cos(); });
+    auto out2 = dev.apply_fn(out, [](auto x) { return x.ln(); });
+    dev.modules.modules.alloc_later(dev);
+    dev.unary_fusing();
+    dev.run();
+    CHECK_VEC_EQ(out.replace().read(), (std::vector<float>(5, 0.f)));
+    std::vector<double> s, full;
+    for (float x : {1.f, 2.f, 3.f, 4.f, 5.f}) {
+        s.push_back(std::sin(x));
+        full.push_back(std::log(std::cos(std::sin(x))));
+    }
+    CHECK_ROUGHLY(out1.replace().read(), s, 1e-3);
+    CHECK_ROUGHLY(out2.replace().read(), full, 1e-3);
+}
+
+// src/op_hint.rs:221-251: two independent chains, recorded interleaved
+template <template <class> class DEV>
+void graph_fuse_two_chains(double tol) {
+    DEV<Graph<Lazy<Base>>> dev;
+    auto buf = dev.template buffer<float>({1.f, 2.f, 3.f, 4.f, 5.f});
+    auto rhs = dev.template buffer<float>({8.f, 2.f, 3.f, 4.f, 5.f});
+    auto out1 = dev.apply_fn(buf, [](auto x) { return x.sin(); });
+    auto out = dev.apply_fn(rhs, [](auto x) { return x.sin(); });
+    auto out2 = dev.apply_fn(out, [](auto x) { return x.cos(); });
+    auto out1b = dev.apply_fn(out1, [](auto x) { return x.abs(); });
+    auto out3 = dev.apply_fn(out1b, [](auto x) { return x.ln(); });
+    dev.optimize_mem_graph();
+    dev.unary_fusing();
+    dev.run();
+    std::vector<double> w3, w2;
+    for (float x : {1.f, 2.f, 3.f, 4.f, 5.f}) w3.push_back(std::log(std::fabs(std::sin(x))));
+    for (float x : {8.f, 2.f, 3.f, 4.f, 5.f}) w2.push_back(std::cos(std::sin(x)));
+    CHECK_ROUGHLY(out3.replace().read(), w3, tol);
+    CHECK_ROUGHLY(out2.replace().read(), w2, tol);
+}
+
+// A trace that starts with a two-operand op and continues with a unary chain:
+// the reference drops the whole trace here; the unary run must be fused and the
+// other operations must stay.
+template <template <class> class DEV>
+void graph_fuse_after_binary_ops() {
+    DEV<Graph<Lazy<Base>>> dev;
+    auto a = dev.template buffer<float>({0.5f, 0.25f, 0.75f, 1.f});
+    auto b = dev.template buffer<float>({2.f, 4.f, 0.5f, 3.f});
+    auto c = dev.template buffer<float>({-3.f, 0.f, 0.125f, 1.f});
+    auto t = dev.apply_fn2(a, b, [](auto x, auto y) { return x.mul(y); });
+    auto u = dev.apply_fn2(t, c, [](auto x, auto y) { return x.add(y); });
+    auto v = dev.apply_fn(u, [](auto x) { return x.abs().sqrt(); });
+    auto y = dev.apply_fn(v, [](auto x) { return x.mul(0.3f); });
+    const size_t before = dev.ops_count();
+    dev.modules.modules.alloc_later(dev);
+    dev.unary_fusing();
+    CHECK_EQ(dev.ops_count(), before);
+    const auto& ops = dev.modules.modules.graph;
+    CHECK(ops[0].hint_kind == OpHintKind::None && !ops[0].arg_ids.empty());   // the mul stays
+    CHECK(ops[1].hint_kind == OpHintKind::None && !ops[1].arg_ids.empty());   // the add stays
+    CHECK(ops[2].hint_kind == OpHintKind::UnaryFused);
+    CHECK(ops[3].arg_ids.empty());
+    dev.run();
+    std::vector<float> want;
+    const float av[] = {0.5f, 0.25f, 0.75f, 1.f}, bv[] = {2.f, 4.f, 0.5f, 3.f}, cv[] = {-3.f, 0.f, 0.125f, 1.f};
+    for (int i = 0; i < 4; i++) {
+        float tt = av[i] * bv[i];
+        float uu = tt + cv[i];
+        float s = std::sqrt(std::fabs(uu));
+        want.push_back(s * 0.3f);
+    }
+    CHECK_VEC_EQ(y.replace().read(), want);  // every node is correctly rounded: exact on every device
+}
+
+// src/modules/graph/opt_graph/optimize.rs:560-590 (test_lazy_from_retrieve): aliasing
+template <template <class> class DEV>
+void graph_optimize_mem_aliases() {
+    DEV<Graph<Lazy<Base>>> device;
+    auto x = device.template buffer<float>(std::vector<float>(1000, 1.f));
+    auto b = device.template buffer<float>(std::vector<float>(1000, 1.1f));
+    auto squared = device.template retrieve<float>(1000, x, x);
+    auto add = device.template retrieve<float>(1000, b, x);
+    auto mul_b = device.template retrieve<float>(1000, add, b);
+    auto mul = device.template retrieve<float>(1000, squared, x);
+    auto out = device.template retrieve<float>(1000, mul, mul_b);
+    auto traces = device.modules.graph_trans.opt_graph.cache_traces();
+    CHECK_EQ(traces.size(), size_t(2));
+    CHECK(traces[0] == (CacheTrace{2, {5, 6}}));
+    CHECK(traces[1] == (CacheTrace{3, {4}}));
+    device.optimize_mem_graph();
+    device.run();
+    CHECK_EQ(squared.replace().ptr(), mul.replace().ptr());
+    CHECK_EQ(squared.replace().ptr(), out.replace().ptr());
+    CHECK_EQ(add.replace().ptr(), mul_b.replace().ptr());
+    CHECK(squared.replace().ptr() != add.replace().ptr());
+}
+
+// examples/lazy_and_fusing.rs:4-24
+template <template <class> class DEV>
+void example_lazy_and_fusing() {
+    DEV<Graph<Lazy<Base>>> device;
+    auto buf = device.template buffer<float>({1.f, 2.f, 3.f, 4.f, 5.f});
+    auto out1 = device.apply_fn(buf, [](auto x) { return x.add(1.f); });
+    auto out2 = device.apply_fn(out1, [](auto x) { return x.sin(); });
+    device.optimize_mem_graph();
+    device.unary_fusing();
+    device.run();
+    auto in = buf.read();
+    auto got = out2.replace().read();
+    for (size_t i = 0; i < in.size(); i++) CHECK(std::fabs(got[i] - std::sin(in[i] + 1.f)) < 0.01);
+}
+
+// ---- Autograd ----
+
+// src/unary.rs:160-204
+template <template <class> class DEV>
+void autograd_unary_ew() {
+    DEV<Autograd<Base>> device;
+    auto buf = device.template buffer<float>({1.f, 2.f, 3.f, 4.f}).require_grad();
+    auto out = device.unary_ew(buf, [](auto x) { return x.sin(); }, [](auto x) { return x.cos(); });
+    CHECK_ROUGHLY(out.read(), SIN_1_4, 1e-6);
+    out.backward();
+    CHECK_ROUGHLY(buf.grad(device).read(), COS_1_4, 1e-6);
+}
+
+// src/unary.rs:74-85 (doc test)
+template <template <class> class DEV>
+void autograd_doc_example() {
+    DEV<Autograd<Base>> device;
+    auto buf = device.template buffer<double>({1., 2., 3., 3., 2., 1.}).require_grad();
+    auto out = device.unary_ew(buf, [](auto x) { return x.mul(2.); }, [](auto) { return to_val(2.0); });
+    CHECK_VEC_EQ(out.read(), (std::vector<double>{2., 4., 6., 6., 4., 2.}));
+    out.backward();
+    CHECK_VEC_EQ(buf.grad(device).read(), (std::vector<double>(6, 2.)));
+}
+
+// src/unary.rs:243-282: ten rounds, gradient cleared in between
+template <template <class> class DEV>
+void autograd_multiple_times(double tol) {
+    DEV<Autograd<Base>> device;
+    auto buf = device.template buffer<double>({1., 2., 3., 4.}).require_grad();
+    for (int i = 0; i < 10; i++) {
+        auto out = device.unary_ew(buf, [](auto x) { return x.sin(); }, [](auto x) { return x.cos(); });
+        CHECK_ROUGHLY(out.read(), SIN_1_4, tol);
+        out.backward();
+        CHECK_ROUGHLY(buf.grad(device).read(), COS_1_4, tol);
+        auto g = buf.grad(device);
+        g.clear();
+    }
+}
+
+// src/unary.rs:284-326: lazy + autograd, gradients accumulate over repeated run/backward
+template <template <class> class DEV>
+void autograd_lazy_accumulates(double tol) {
+    DEV<Autograd<Lazy<Base, double>>> device;
+    auto buf = device.template buffer<double>({1., 2., 3., 4.}).require_grad();
+    auto out = device.unary_ew(buf, [](auto x) { return x.sin(); }, [](auto x) { return x.cos(); });
+    for (int i = 1; i < 10; i++) {
+        device.run();
+        CHECK_ROUGHLY(out.replace().read(), SIN_1_4, tol);
+        out.backward();
+        CHECK_ROUGHLY(buf.grad(device).read(), scaled(COS_1_4, i), tol * 10);
+    }
+}
+
+// src/unary.rs:328-368: the input of unary_ew is itself lazily computed; second variant
+// consumes the first operation with exec_last_n
+template <template <class> class DEV>
+void autograd_lazy_input(bool exec_last, double tol) {
+    DEV<Autograd<Lazy<Base, double>>> device;
+    auto buf = device.template buffer<double>({0., 1., 2., 3.}).require_grad();
+    auto buf1 = device.apply_fn(buf, [](auto x) { return x.add(1.); });
+    if (exec_last) device.exec_last_n(1);
+    auto out = device.unary_ew(buf1, [](auto x) { return x.sin(); }, [](auto x) { return x.cos(); });
+    for (int i = 1; i < 10; i++) {
+        device.run();
+        CHECK_ROUGHLY(out.replace().read(), SIN_1_4, tol);
+        out.backward();
+        CHECK_ROUGHLY(buf1.grad(device).read(), scaled(COS_1_4, i), tol * 10);
+    }
+}
+
+// src/modules/autograd.rs:494-512
+template <template <class> class DEV>
+void autograd_grad_new_api() {
+    using D = DEV<Autograd<Base>>;
+    D device;
+    auto lhs = device.template buffer<int32_t>({1, 2, 3, 4}).require_grad();
+    auto out = lhs.empty_like();
+    device.add_grad_fn(std::tie(lhs, out), [](Buffer<int32_t, D>& l, Buffer<int32_t, D>& o, D& dev) {
+        auto lg = l.grad(dev);
+        dev.add_unary_grad(l, lg, o.grad(dev), [](auto x) { return x.add(3); });
+    });
+    out.backward();
+    CHECK(lhs.try_grad(device).has_value());
+    CHECK_VEC_EQ(lhs.try_grad(device)->read(), (std::vector<int32_t>{4, 5, 6, 7}));
+}
+
+// src/modules/autograd.rs:514-542
+template <template <class> class DEV>
+void autograd_disabling() {
+    using D = DEV<Autograd<Base>>;
+    D device;
+    auto lhs = device.template buffer<int32_t>({1, 2, 3, 4}).require_grad();
+    auto out = lhs.empty_like();
+    bool called = false;
+    device.disable_grad();
+    device.add_grad_fn(std::tie(lhs, out), [&called](Buffer<int32_t, D>&, Buffer<int32_t, D>&, D&) { called = true; });
+    out.backward();
+    CHECK(!called);
+    CHECK(!lhs.try_grad(device).has_value());
+    device.enable_grad();
+    device.add_grad_fn(std::tie(lhs, out), [](Buffer<int32_t, D>& l, Buffer<int32_t, D>& o, D& dev) {
+        auto lg = l.grad(dev);
+        dev.add_unary_grad(l, lg, o.grad(dev), [](auto x) { return x.add(3); });
+    });
+    out.backward();
+    CHECK_VEC_EQ(lhs.try_grad(device)->read(), (std::vector<int32_t>{4, 5, 6, 7}));
+}
+
+// src/modules/autograd.rs:544-590
+template <template <class> class DEV>
+void autograd_requires_grad_chaining() {
+    DEV<Autograd<Base>> device;
+    auto lhs = device.template buffer<int32_t>({1, 2, 3, 4}).require_grad();
+    CHECK(device.modules.requires_grad_of(lhs.id()) && lhs.requires_grad());
+    auto no_grad = device.template buffer<int32_t>({1, 2, 3, 4}).no_grad();
+    CHECK(!device.modules.requires_grad_of(no_grad.id()));
+    auto rhs = device.template buffer<int32_t>({1, 2, 3, 4}).no_grad();
+    CHECK(!rhs.requires_grad());
+    CHECK(device.template retrieve<int32_t>(rhs.len(), lhs, rhs).requires_grad());
+    CHECK(device.template retrieve<int32_t>(rhs.len(), lhs).requires_grad());
+    CHECK(!device.template retrieve<int32_t>(rhs.len(), rhs).requires_grad());
+    CHECK(!device.template retrieve<int32_t>(rhs.len(), no_grad, rhs).requires_grad());
+    auto out = device.template retrieve<int32_t>(rhs.len(), lhs, rhs);
+    CHECK(device.modules.requires_grad_of(out.id()));
+}
+
+// src/modules/autograd.rs:434-456: gradient function over buffers kept by Lazy
+template <template <class> class DEV>
+void autograd_grad_fn_with_lazy_source() {
+    using D = DEV<Autograd<Lazy<Base>>>;
+    D device;
+    auto buf = Buffer<float, D>(device, 10).require_grad();
+    Buffer<float, D> out(device, 10);
+    device.add_grad_fn(std::tie(buf, out), [](Buffer<float, D>& b, Buffer<float, D>& o, D& dev) {
+        auto bg = b.grad(dev);
+        // buf.grad = 5 * out.grad, through the unary-gradient kernel on a zeroed gradient
+        dev.add_unary_grad(b, bg, o.grad(dev), [](auto) { return to_val(5.f); });
+    });
+    out.backward();
+    CHECK_VEC_EQ(buf.grad(device).read(), (std::vector<float>(10, 5.f)));
+}
+
+// src/modules/autograd.rs:458-478: the gradient function's buffer went out of scope
+template <template <class> class DEV>
+void autograd_grad_fn_out_of_scope() {
+    using D = DEV<Autograd<Lazy<Base>>>;
+    D device;
+    Buffer<float, D> out(device, 10);
+    {
+        auto buf = Buffer<float, D>(device, 10).require_grad();
+        device.add_grad_fn(std::tie(buf, out), [](Buffer<float, D>&, Buffer<float, D>&, D&) {});
+    }
+    CHECK_THROWS_KIND(out.backward(), DeviceError::InvalidLazyBuf);
+}
+
+// BASELINE configs[2] in miniature: tanh forward, backward with a given out gradient,
+// x_grad pre-filled with 0.1
+template <template <class> class DEV>
+void autograd_tanh_config(double tol) {
+    using D = DEV<Autograd<Base>>;
+    D device;
+    std::vector<float> xs = {-1.5f, -0.25f, 0.f, 0.5f, 2.f}, yg = {1.f, -0.5f, 0.25f, 0.75f, -1.f};
+    auto x = device.template buffer<float>(xs).require_grad();
+    {
+        auto g = x.grad(device);
+        g.write(std::vector<float>(5, 0.1f));
+    }
+    auto y = device.unary_ew(x, [](auto v) { return v.tanh(); },
+                             [](auto v) { return Scalar<float>(1.f).sub(v.tanh().mul(v.tanh())); });
+    y.backward_with(yg);
+    std::vector<double> want_y, want_g;
+    for (int i = 0; i < 5; i++) {
+        double t = std::tanh(static_cast<double>(xs[i]));
+        want_y.push_back(t);
+        want_g.push_back(0.1 + yg[i] * (1 - t * t));
+    }
+    CHECK_ROUGHLY(y.read(), want_y, tol);
+    CHECK_ROUGHLY(x.grad(device).read(), want_g, tol);
+}
+
+}  // namespace module_tests
+
+// Registers every generic case for one device template.
+#define REGISTER_MODULE_TESTS(DEV, TOL)                                                           \
+    TEST_CASE(base_apply_fn) { module_tests::base_apply_fn<DEV>(); }                              \
+    TEST_CASE(base_add_unary_grad) { module_tests::base_add_unary_grad<DEV>(); }                  \
+    TEST_CASE(base_unary_ew_forward_only) { module_tests::base_unary_ew_forward_only<DEV>(); }    \
+    TEST_CASE(base_zero_length_is_an_error) { module_tests::base_zero_length_is_an_error<DEV>(); } \
+    TEST_CASE(lazy_retrieve_ids) { module_tests::lazy_retrieve_ids<DEV>(); }                      \
+    TEST_CASE(lazy_apply_fn_runs_at_run) { module_tests::lazy_apply_fn_runs_at_run<DEV>(); }      \
+    TEST_CASE(lazy_dropped_buffer_is_invalid) { module_tests::lazy_dropped_buffer_is_invalid<DEV>(); } \
+    TEST_CASE(lazy_add_and_apply_fn) { module_tests::lazy_add_and_apply_fn<DEV>(); }              \
+    TEST_CASE(lazy_add_unary_grad) { module_tests::lazy_add_unary_grad<DEV>(); }                  \
+    TEST_CASE(lazy_exec_now_and_last_n) { module_tests::lazy_exec_now_and_last_n<DEV>(); }        \
+    TEST_CASE(lazy_duplicate_parent_is_rejected) { module_tests::lazy_duplicate_parent_is_rejected<DEV>(); } \
+    TEST_CASE(lazy_op_hints) { module_tests::lazy_op_hints<DEV>(); }                              \
+    TEST_CASE(graph_fuse_chain_optimized) { module_tests::graph_fuse_chain<DEV>(true); }          \
+    TEST_CASE(graph_fuse_chain_alloc_later) { module_tests::graph_fuse_chain<DEV>(false); }       \
+    TEST_CASE(graph_fuse_chain_with_checkpoint) { module_tests::graph_fuse_chain_with_checkpoint<DEV>(); } \
+    TEST_CASE(graph_fuse_two_chains) { module_tests::graph_fuse_two_chains<DEV>(TOL); }           \
+    TEST_CASE(graph_fuse_after_binary_ops) { module_tests::graph_fuse_after_binary_ops<DEV>(); }  \
+    TEST_CASE(graph_optimize_mem_aliases) { module_tests::graph_optimize_mem_aliases<DEV>(); }    \
+    TEST_CASE(example_lazy_and_fusing) { module_tests::example_lazy_and_fusing<DEV>(); }          \
+    TEST_CASE(autograd_unary_ew) { module_tests::autograd_unary_ew<DEV>(); }                      \
+    TEST_CASE(autograd_doc_example) { module_tests::autograd_doc_example<DEV>(); }                \
+    TEST_CASE(autograd_multiple_times) { module_tests::autograd_multiple_times<DEV>(TOL); }       \
+    TEST_CASE(autograd_lazy_accumulates) { module_tests::autograd_lazy_accumulates<DEV>(TOL); }   \
+    TEST_CASE(autograd_lazy_input) { module_tests::autograd_lazy_input<DEV>(false, TOL); }        \
+    TEST_CASE(autograd_lazy_input_exec_last) { module_tests::autograd_lazy_input<DEV>(true, TOL); } \
+    TEST_CASE(autograd_grad_new_api) { module_tests::autograd_grad_new_api<DEV>(); }              \
+    TEST_CASE(autograd_disabling) { module_tests::autograd_disabling<DEV>(); }                    \
+    TEST_CASE(autograd_requires_grad_chaining) { module_tests::autograd_requires_grad_chaining<DEV>(); } \
+    TEST_CASE(autograd_grad_fn_with_lazy_source) { module_tests::autograd_grad_fn_with_lazy_source<DEV>(); } \
+    TEST_CASE(autograd_grad_fn_out_of_scope) { module_tests::autograd_grad_fn_out_of_scope<DEV>(); } \
+    TEST_CASE(autograd_tanh_config) { module_tests::autograd_tanh_config<DEV>(1e-6); }
