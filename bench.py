@@ -10,7 +10,11 @@ Prints ONE JSON line: metric/value (GB/s on the algorithmic 8 B per element),
 the roofline of the fused kernel (HIP-event timed on the compute stream) and a
 CPU baseline (the oracle's compiled loop, one thread, on a stated sample).
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5] [--log2n L]
+The same line carries `other_configs`: the other four BASELINE configurations
+(c1 exp, c3 tanh forward+backward, c4 f16 chain, c5 graph replay), each with
+elements/s, GB/s and the CPU port timed beside it (skip with --no-others).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--log2n L] [--no-others]
 """
 from __future__ import annotations
 
@@ -184,12 +188,134 @@ def bench_c2(dev, args):
     }
 
 
+def _cpu_time(fn, *a):
+    t0 = time.perf_counter()
+    r = fn(*a)
+    return time.perf_counter() - t0, r
+
+
+def _entry(name, n, bytes_per_elt, ms, cpu_s, cpu_n, note=""):
+    gbs = bytes_per_elt * n / (ms * 1e-3) / 1e9
+    return {
+        "workload": name,
+        "elements": n,
+        "algorithmic_bytes_per_element": bytes_per_elt,
+        "ms": round(ms, 5),
+        "GBps": round(gbs, 2),
+        "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "elements_per_s": round(n / (ms * 1e-3), 1),
+        "cpu_port_1thread": {
+            "elements_per_s": round(cpu_n / cpu_s, 1),
+            "GBps": round(bytes_per_elt * cpu_n / cpu_s / 1e9, 4),
+            "sample_elements": cpu_n,
+        },
+        **({"note": note} if note else {}),
+    }
+
+
+def bench_others(dev, args):
+    """The other BASELINE configurations (c1, c3, c4, c5), each with its CPU port beside it."""
+    import custos_amd
+    from custos_amd import Const, capi, synth
+    from custos_amd.expr import fused_source
+    from oracle import cpu_oracle
+
+    lib, h = dev.lib, dev.handle
+    steps, warm = max(5, args.steps // 2), max(2, args.warmup // 2)
+    out = {}
+
+    # c1: apply_fn(exp), f32 N = 2^20 (latency-bound: 8 MiB of traffic)
+    n = 1 << 20
+    x = synth.uniform_f32(0, n, -4, 4)
+    xb, ob = dev.buffer(x), dev.alloc(n)
+    k = dev.compile(capi.KIND_APPLY, "f32", "exp(x)", ("x",))
+    ms, _ = time_steps(dev, lambda: capi.check(lib.custos_hip_apply_fn(h, k, xb.ptr, ob.ptr, n), h), steps * 4, warm)
+    cpu_s, want = _cpu_time(cpu_oracle.c1_exp, x)
+    got = ob.read()
+    assert np.max(np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))) <= 4
+    out["c1"] = _entry("c1: apply_fn(exp), f32 N=2^20, U[-4,4) seed 0", n, 8, ms / (steps * 4), cpu_s, n)
+
+    # c3: unary_ew tanh forward + backward, f32 N = 2^26
+    n = 1 << 26
+    x = gen_chunked(lambda m, off: synth.normal_f32(0, m, off), n)
+    yg = gen_chunked(lambda m, off: synth.uniform_f32(1, m, -1, 1, off), n)
+    xb, ygb, yb = dev.buffer(x), dev.buffer(yg), dev.alloc(n)
+    gb = dev.buffer(np.full(n, 0.1, dtype=np.float32))
+    kf = dev.compile(capi.KIND_APPLY, "f32", "tanh(x)", ("x",))
+    grad_src = Const(1.0).sub(custos_amd.Resolve("x").tanh().mul(custos_amd.Resolve("x").tanh())).to_cl_source("f32")
+    kb = dev.compile(capi.KIND_UNARY_GRAD, "f32", grad_src, ("x",))
+
+    def c3_step():
+        capi.check(lib.custos_hip_apply_fn(h, kf, xb.ptr, yb.ptr, n), h)
+        capi.check(lib.custos_hip_add_unary_grad(h, kb, xb.ptr, gb.ptr, ygb.ptr, n), h)
+
+    ms, _ = time_steps(dev, c3_step, steps, warm)
+    ms_f, _ = time_steps(dev, lambda: capi.check(lib.custos_hip_apply_fn(h, kf, xb.ptr, yb.ptr, n), h), steps, warm)
+    ms_b, _ = time_steps(dev, lambda: capi.check(lib.custos_hip_add_unary_grad(h, kb, xb.ptr, gb.ptr, ygb.ptr, n), h), steps, warm)
+    cn = min(n, 1 << 24)
+    g0 = np.full(cn, 0.1, dtype=np.float32)
+    cpu_s, _ = _cpu_time(lambda: (cpu_oracle.c3_tanh_fwd(x[:cn]), cpu_oracle.c3_tanh_bwd(x[:cn], g0, yg[:cn])))
+    e = _entry("c3: unary_ew tanh fwd + bwd (x_grad += y_grad*(1-tanh(x)^2)), f32 N=2^26", n, 24, ms / steps, cpu_s, cn)
+    e["forward"] = {"ms": round(ms_f / steps, 5), "GBps": round(8 * n / (ms_f / steps * 1e-3) / 1e9, 2)}
+    e["backward"] = {"ms": round(ms_b / steps, 5), "GBps": round(16 * n / (ms_b / steps * 1e-3) / 1e9, 2)}
+    out["c3"] = e
+    del xb, ygb, yb, gb
+
+    # c4: f16 storage / f32 compute chain exp(x*0.5)*x + x^2, N = 2^28
+    n = 1 << args.log2n
+    xh = gen_chunked(lambda m, off: synth.uniform_f16_bits(0, m, -2, 2, off), n)
+    xb, ob = dev.buffer(xh.view(np.float16), "f16"), dev.alloc(n, "f16")
+    c4 = lambda v: v.mul(0.5).exp().mul(v).add(v.mul(v))
+    k = dev.compile(capi.KIND_APPLY, "f16", c4(custos_amd.Resolve("x")).to_cl_source("f16"), ("x",))
+    ms, _ = time_steps(dev, lambda: capi.check(lib.custos_hip_apply_fn(h, k, xb.ptr, ob.ptr, n), h), steps, warm)
+    cn = min(n, 1 << 24)
+    cpu_s, want = _cpu_time(cpu_oracle.c4_chain_f16, np.ascontiguousarray(xh[:cn]))
+    got = ob.slice(0, cn).read().view(np.uint16)
+    d = np.abs(got.view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
+    assert d.max() <= 1, "c4 differs from the CPU port by more than 1 f16 ulp"
+    out["c4"] = _entry(f"c4: f16 chain exp(x*0.5)*x + x^2, f32 compute, N=2^{args.log2n}", n, 4, ms / steps, cpu_s, cn)
+    del xb, ob
+
+    # c5: 1024 buffers x 4096 f32: t=a*b; u=t+c; y=sqrt(abs(u))*0.3, one graph, 100 replays
+    nbuf, m = 1024, 4096
+    mk = lambda seed: dev.buffer(gen_chunked(lambda q, off: synth.uniform_f32(seed, q, 0, 1, off), nbuf * m))
+    A, B, Cc = mk(1), mk(2), mk(3)
+    T, U, Y = dev.alloc(nbuf * m), dev.alloc(nbuf * m), dev.alloc(nbuf * m)
+    kmul = dev.compile(capi.KIND_APPLY, "f32", "(x * y)", ("x", "y"))
+    kadd = dev.compile(capi.KIND_APPLY, "f32", "(x + y)", ("x", "y"))
+    kun = dev.compile(capi.KIND_APPLY, "f32", fused_source([lambda v: v.abs().sqrt(), lambda v: v.mul(0.3)]), ("x",))
+    dev.capture_begin()
+    for i in range(nbuf):
+        o = i * m * 4
+        capi.check(lib.custos_hip_apply_fn2(h, kmul, A.ptr + o, B.ptr + o, T.ptr + o, m), h)
+        capi.check(lib.custos_hip_apply_fn2(h, kadd, T.ptr + o, Cc.ptr + o, U.ptr + o, m), h)
+        capi.check(lib.custos_hip_apply_fn(h, kun, U.ptr + o, Y.ptr + o, m), h)
+    t0 = time.perf_counter()
+    graph = dev.capture_end()
+    build_s = time.perf_counter() - t0
+    replays = 100
+    ms, wall = time_steps(dev, graph.launch, replays, 3)
+    a, b, c = A.read(), B.read(), Cc.read()
+    cpu_s, (_, _, want) = _cpu_time(cpu_oracle.c5_graph, a, b, c)
+    assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), "c5 replay differs from the CPU port"
+    e = _entry("c5: 1024 x f32[4096], t=a*b; u=t+c; y=sqrt(abs(u))*0.3, one hipGraph, 100 replays", nbuf * m, 16,
+               ms / replays, cpu_s, nbuf * m, note="GB/s on the minimal 16 B/element; the recorded 3-kernel form moves 32 B/element")
+    e["us_per_replay"] = round(ms / replays * 1e3, 2)
+    e["wall_us_per_replay"] = round(wall / replays * 1e3, 2)
+    e["graph_kernel_nodes"] = graph.kernel_nodes
+    e["recorded_launches"] = 3 * nbuf
+    e["graph_build_ms"] = round(build_s * 1e3, 2)
+    out["c5"] = e
+    graph.destroy()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2")
+    ap.add_argument("--workload", default="c2", choices=["c2"])
     ap.add_argument("--log2n", type=int, default=28)
     ap.add_argument("--cpu-log2n", dest="cpu_log2n", type=int, default=28,
                     help="log2 of the element count of the CPU baseline sample")
@@ -197,6 +323,8 @@ def main():
     ap.add_argument("--unroll", type=int, default=0)
     ap.add_argument("--blocks-per-cu", dest="blocks_per_cu", type=int, default=0)
     ap.add_argument("--nontemporal", type=int, default=0)
+    ap.add_argument("--no-others", dest="others", action="store_false",
+                    help="skip the other BASELINE configurations (c1, c3, c4, c5)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU; the element-wise path needs no second one "
@@ -209,6 +337,8 @@ def main():
         dev.set_tuning(args.block, args.unroll, args.blocks_per_cu, args.nontemporal)
     info = dev.info()
     res = {"c2": bench_c2}[args.workload](dev, args)
+    if args.others:
+        res["other_configs"] = bench_others(dev, args)
     res.update({
         "n_gpus": 1,
         "steps": args.steps,

@@ -118,6 +118,8 @@ PROTOTYPES = {
     "custos_hip_is_capturing": (C.c_int32, [_P, C.POINTER(C.c_int32)]),
     "custos_hip_graph_launch": (C.c_int32, [_P, _P]),
     "custos_hip_graph_node_count": (C.c_int32, [_P, C.POINTER(C.c_size_t)]),
+    "custos_hip_graph_stats": (C.c_int32, [_P, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "custos_hip_set_graph_batching": (C.c_int32, [_P, C.c_int32]),
     "custos_hip_graph_destroy": (C.c_int32, [_P, _P]),
     "custos_hip_timer_begin": (C.c_int32, [_P]),
     "custos_hip_timer_end": (C.c_int32, [_P, C.POINTER(C.c_double)]),

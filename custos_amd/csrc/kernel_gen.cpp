@@ -68,11 +68,24 @@ static __device__ __forceinline__ double custos_log(double a) { return log(a); }
 static __device__ __forceinline__ double custos_sqrt(double a) { return sqrt(a); }
 )";
     } else if (dtype_is_float(dtype)) {
+        // 16-bit storage types: the result is rounded to 11 (f16) or 8 (bf16)
+        // significant bits at the store, so exp may take the hardware exp2
+        // directly: relative error <= |a| * 2^-24 (argument rounding) + 1 ulp,
+        // below 5e-6 over the whole finite range, against a half-ulp of 2.4e-4
+        // for f16.  The correctly-rounded-to-f32 path costs about 3x the ALU work
+        // and makes the f16 chain ALU-bound instead of HBM-bound.  sin / cos /
+        // tanh / log keep the full-precision routines: their results pass through
+        // zero, where only a relative bound in f32 keeps the 16-bit result within
+        // one ulp.
+        if (dtype == DType::F16 || dtype == DType::BF16)
+            s += "static __device__ __forceinline__ float custos_exp(float a) {\n"
+                 "    return __builtin_amdgcn_exp2f(a * 0x1.715476p+0f);\n}\n";
+        else
+            s += "static __device__ __forceinline__ float custos_exp(float a) { return expf(a); }\n";
         s += R"(static __device__ __forceinline__ float custos_sin(float a) { return sinf(a); }
 static __device__ __forceinline__ float custos_cos(float a) { return cosf(a); }
 static __device__ __forceinline__ float custos_tan(float a) { return tanf(a); }
 static __device__ __forceinline__ float custos_tanh(float a) { return tanhf(a); }
-static __device__ __forceinline__ float custos_exp(float a) { return expf(a); }
 static __device__ __forceinline__ float custos_log(float a) { return logf(a); }
 static __device__ __forceinline__ float custos_sqrt(float a) { return sqrtf(a); }
 )";
@@ -120,7 +133,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     uint64_t h;
     if (!hash_expr(k.expr, dtype, &h, err)) return false;
     int32_t tail[6] = {static_cast<int32_t>(kind), tuning.block_threads, tuning.unroll,
-                       tuning.blocks_per_cu, tuning.nontemporal, 2 /* template version */};
+                       tuning.blocks_per_cu, tuning.nontemporal, 4 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -185,37 +198,49 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
         return r;
     };
 
+    // One tile: every lane loads all its vectors, then computes and stores.
+    // `base` is the lane's first vector; a partial last tile takes the masked path.
+    std::string tile_params, tile_args;
+    for (int i = 0; i < n_ops; i++) {
+        if (kind == Kind::UnaryGrad && i == 1) continue;  // vin1 is vout
+        tile_params += "const vec_t* vin" + std::to_string(i) + ", ";
+        tile_args += "vin" + std::to_string(i) + ", ";
+    }
+    s += "static __device__ __forceinline__ void custos_tile(" + tile_params + "vec_t* vout, const u64 base, const u64 n_vec) {\n";
+    if (kind == Kind::UnaryGrad) s += "    const vec_t* vin1 = vout;\n";
+    s += "    if (base + (u64)(CUSTOS_UNROLL - 1) * CUSTOS_BLOCK < n_vec) {\n";
+    for (int i = 0; i < n_ops; i++) s += "        vec_t a" + std::to_string(i) + "[CUSTOS_UNROLL];\n";
+    s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+    for (int i = 0; i < n_ops; i++) {
+        std::string id = std::to_string(i);
+        s += "            a" + id + "[u] = CUSTOS_LD(vin" + id + " + base + (u64)u * CUSTOS_BLOCK);\n";
+    }
+    s += "        }\n";
+    s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+    s += "            vec_t r;\n#pragma unroll\n            for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
+         list("a", "[u][k]") + ");\n";
+    s += "            CUSTOS_ST(vout + base + (u64)u * CUSTOS_BLOCK, r);\n        }\n";
+    s += "    } else {\n";
+    s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+    s += "            const u64 idx = base + (u64)u * CUSTOS_BLOCK;\n";
+    s += "            if (idx < n_vec) {\n";
+    for (int i = 0; i < n_ops; i++) {
+        std::string id = std::to_string(i);
+        s += "                const vec_t b" + id + " = CUSTOS_LD(vin" + id + " + idx);\n";
+    }
+    s += "                vec_t r;\n#pragma unroll\n                for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
+         list("b", "[k]") + ");\n";
+    s += "                CUSTOS_ST(vout + idx, r);\n            }\n        }\n";
+    s += "    }\n}\n";
+
+    // Entry point for one launch over one set of operands.
     s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
     s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec) {\n";
     s += vec_ptrs;
     s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
     s += "    const u64 n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;\n";
-    s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {\n";
-    s += "        const u64 base = tile * tile_vecs + threadIdx.x;\n";
-    s += "        if (base + (u64)(CUSTOS_UNROLL - 1) * CUSTOS_BLOCK < n_vec) {\n";
-    for (int i = 0; i < n_ops; i++) s += "            vec_t a" + std::to_string(i) + "[CUSTOS_UNROLL];\n";
-    s += "#pragma unroll\n            for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
-    for (int i = 0; i < n_ops; i++) {
-        std::string id = std::to_string(i);
-        s += "                a" + id + "[u] = CUSTOS_LD(vin" + id + " + base + (u64)u * CUSTOS_BLOCK);\n";
-    }
-    s += "            }\n";
-    s += "#pragma unroll\n            for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
-    s += "                vec_t r;\n#pragma unroll\n                for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
-         list("a", "[u][k]") + ");\n";
-    s += "                CUSTOS_ST(vout + base + (u64)u * CUSTOS_BLOCK, r);\n            }\n";
-    s += "        } else {\n";
-    s += "#pragma unroll\n            for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
-    s += "                const u64 idx = base + (u64)u * CUSTOS_BLOCK;\n";
-    s += "                if (idx < n_vec) {\n";
-    for (int i = 0; i < n_ops; i++) {
-        std::string id = std::to_string(i);
-        s += "                    const vec_t b" + id + " = CUSTOS_LD(vin" + id + " + idx);\n";
-    }
-    s += "                    vec_t r;\n#pragma unroll\n                    for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
-         list("b", "[k]") + ");\n";
-    s += "                    CUSTOS_ST(vout + idx, r);\n                }\n            }\n";
-    s += "        }\n    }\n";
+    s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x)\n";
+    s += "        custos_tile(" + tile_args + "vout, tile * tile_vecs + threadIdx.x, n_vec);\n";
     // Elements outside the 16-byte aligned body: `head` leading ones and the
     // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
     s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
@@ -224,6 +249,32 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     s += "    for (u64 i = head + n_vec * CUSTOS_VEC + gid; i < n; i += n_threads) out[i] = custos_elem(" +
          list("in", "[i]") + ");\n";
     s += "}\n";
+
+    // Entry point for many independent launches of equal length in one grid
+    // (graph replay of many small buffers).  `table` holds, per segment, the
+    // operand addresses in the order of the single-launch parameters; every
+    // address is 16-byte aligned.  Workgroup b works on tile b % tiles_per_seg
+    // of segment b / tiles_per_seg; the last tile of a segment also does the tail.
+    const int n_ptrs = kind == Kind::Apply ? n_in + 1 : 3;
+    s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
+    s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg) {\n";
+    s += "    const u64 seg = blockIdx.x / tiles_per_seg;\n";
+    s += "    const u64 tile = blockIdx.x - seg * tiles_per_seg;\n";
+    s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs) + ";\n";
+    s += "    const u64 head = 0;\n";
+    if (kind == Kind::Apply) {
+        for (int i = 0; i < n_in; i++)
+            s += "    const S* in" + std::to_string(i) + " = (const S*)ptrs[" + std::to_string(i) + "];\n";
+        s += "    S* out = (S*)ptrs[" + std::to_string(n_in) + "];\n";
+    } else {
+        s += "    const S* in0 = (const S*)ptrs[0];\n    S* out = (S*)ptrs[1];\n    const S* in2 = (const S*)ptrs[2];\n";
+    }
+    s += vec_ptrs;
+    s += "    custos_tile(" + tile_args + "vout, tile * (u64)CUSTOS_BLOCK * CUSTOS_UNROLL + threadIdx.x, n_vec);\n";
+    s += "    if (tile == tiles_per_seg - 1)\n";
+    s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
+         list("in", "[i]") + ");\n";
+    s += "    (void)head;\n}\n";
 
     k.source = std::move(s);
     *out = std::move(k);

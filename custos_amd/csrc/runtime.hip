@@ -23,12 +23,31 @@ struct custos_hip_kernel {
     KernelSpec spec;
     hipModule_t module = nullptr;
     hipFunction_t fn = nullptr;
+    hipFunction_t fn_batched = nullptr;
 };
 
 struct custos_hip_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
-    size_t kernel_nodes = 0;
+    void* table = nullptr;    // operand address tables of the batched nodes (device memory)
+    size_t kernel_nodes = 0;  // kernel nodes in the instantiated graph
+    size_t recorded = 0;      // launches, clears and copies that were recorded
+    size_t levels = 0;        // dependency levels
+};
+
+// One recorded piece of work (while the device is recording, nothing is launched).
+struct Access {
+    uint64_t begin, end;
+    bool write;
+};
+struct RecNode {
+    enum Type { Kernel, Fill, Copy } type = Kernel;
+    custos_hip_kernel* k = nullptr;
+    std::vector<uint64_t> ptrs;  // kernel: operand addresses in parameter order; fill: {ptr}; copy: {dst, src}
+    unsigned long long n = 0, head = 0, n_vec = 0, bytes = 0;
+    unsigned int grid = 1;
+    std::vector<Access> acc;
+    int level = 0;
 };
 
 struct custos_hip_device {
@@ -39,7 +58,9 @@ struct custos_hip_device {
     hipDeviceProp_t props{};
     std::string arch;
     Tuning tuning;
-    bool capturing = false;
+    bool capturing = false;          // recording: launches, clears and copies go to `recorded`
+    bool batching = true;            // merge equal independent launches of a level into one grid
+    std::vector<RecNode> recorded;
     uint64_t compiles = 0, hits = 0;
     std::string last_error;
     std::unordered_map<uint64_t, std::vector<std::unique_ptr<custos_hip_kernel>>> cache;
@@ -89,15 +110,30 @@ __global__ void __launch_bounds__(256) custos_fill_zero(unsigned char* p, unsign
     for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads) p[i] = 0;
 }
 
+unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec) {
+    unsigned long long want = (n_vec + 255) / 256;
+    // 8 vectors per thread at most: enough workgroups to fill the chip, not one per 4 KiB
+    unsigned long long cap = static_cast<unsigned long long>(dev->props.multiProcessorCount) * 64;
+    unsigned long long g = std::max(1ull, std::min(want, std::max(cap, (want + 7) / 8)));
+    return static_cast<unsigned int>(std::min(g, 1ull << 22));
+}
+
 int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream) {
     unsigned long long head = (16 - (dptr & 15)) & 15;
     if (head > bytes) head = bytes;
     unsigned long long n_vec = (bytes - head) / 16;
-    unsigned long long want = (n_vec + 255) / 256;
-    // 8 vectors per thread at most: enough workgroups to fill the chip, not one per 4 KiB
-    unsigned long long cap = static_cast<unsigned long long>(dev->props.multiProcessorCount) * 64;
-    unsigned int grid = static_cast<unsigned int>(std::max(1ull, std::min(want, std::max(cap, (want + 7) / 8))));
-    grid = std::min(grid, 1u << 22);
+    if (dev->capturing && stream == dev->stream) {
+        RecNode node;
+        node.type = RecNode::Fill;
+        node.ptrs = {dptr};
+        node.bytes = bytes;
+        node.head = head;
+        node.n_vec = n_vec;
+        node.acc = {{dptr, dptr + bytes, true}};
+        dev->recorded.push_back(std::move(node));
+        return CUSTOS_HIP_OK;
+    }
+    unsigned int grid = fill_grid(dev, n_vec);
     hipLaunchKernelGGL(custos_fill_zero, dim3(grid), dim3(256), 0, stream,
                        reinterpret_cast<unsigned char*>(dptr), static_cast<unsigned long long>(bytes),
                        head, n_vec);
@@ -223,10 +259,224 @@ int32_t plan_launch(custos_hip_device* dev, const custos_hip_kernel* k, const st
     return CUSTOS_HIP_OK;
 }
 
-int32_t launch(custos_hip_device* dev, custos_hip_kernel* k, std::vector<void*>& args, unsigned int grid) {
+// Launches the kernel over one set of operands, or records the launch while
+// the device is recording.  `ops` are the operand addresses in the order of the
+// kernel's pointer parameters.
+int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n) {
+    unsigned long long head, n_vec, count = n;
+    unsigned int grid;
+    int32_t rc = plan_launch(dev, k, ops, n, &head, &n_vec, &grid);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    if (dev->capturing) {
+        RecNode node;
+        node.type = RecNode::Kernel;
+        node.k = k;
+        node.n = n;
+        node.head = head;
+        node.n_vec = n_vec;
+        node.grid = grid;
+        const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
+        for (const Range& r : ops) {
+            node.ptrs.push_back(r.ptr);
+            // (the gradient operand of a unary-gradient kernel is read and written;
+            // a write access already orders it against every other access)
+            node.acc.push_back({r.ptr, r.ptr + bytes, r.written});
+        }
+        dev->recorded.push_back(std::move(node));
+        return CUSTOS_HIP_OK;
+    }
+    uint64_t ptrs[8];
+    std::vector<void*> args;
+    for (size_t i = 0; i < ops.size(); i++) {
+        ptrs[i] = ops[i].ptr;
+        args.push_back(&ptrs[i]);
+    }
+    args.push_back(&count);
+    args.push_back(&head);
+    args.push_back(&n_vec);
     HIP_TRY(dev, hipModuleLaunchKernel(k->fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
                                        1, 1, 0, dev->stream, args.data(), nullptr));
     return CUSTOS_HIP_OK;
+}
+
+// ---- building a graph from the recorded work ----
+//
+// The recorded list is not replayed launch by launch.  Every node gets a
+// dependency level: one more than the highest level among earlier nodes whose
+// memory it conflicts with (read-after-write, write-after-read or
+// write-after-write on overlapping address ranges).  Nodes of one level are
+// independent of each other, so they run side by side in the graph, and kernel
+// launches of one level that use the same kernel over the same length are
+// merged into ONE grid that walks a table of operand addresses.  1024 small
+// buffers with three operations each become three kernel nodes instead of
+// 3072.
+
+constexpr uint64_t kChunkShift = 21;  // conflict search buckets of 2 MiB
+
+void assign_levels(std::vector<RecNode>& nodes) {
+    struct Seen {
+        uint64_t begin, end;
+        bool write;
+        int level;
+    };
+    std::vector<Seen> seen;
+    std::unordered_map<uint64_t, std::vector<uint32_t>> buckets;
+    for (RecNode& node : nodes) {
+        int level = 0;
+        for (const Access& a : node.acc) {
+            if (a.end <= a.begin) continue;
+            for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) {
+                auto it = buckets.find(c);
+                if (it == buckets.end()) continue;
+                for (uint32_t si : it->second) {
+                    const Seen& s = seen[si];
+                    if (s.level < level) continue;        // cannot raise the level any more
+                    if (!a.write && !s.write) continue;   // two reads never conflict
+                    if (a.begin < s.end && s.begin < a.end) level = s.level + 1;
+                }
+            }
+        }
+        node.level = level;
+        for (const Access& a : node.acc) {
+            if (a.end <= a.begin) continue;
+            const uint32_t idx = static_cast<uint32_t>(seen.size());
+            seen.push_back({a.begin, a.end, a.write, level});
+            for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) buckets[c].push_back(idx);
+        }
+    }
+}
+
+bool batchable(const RecNode& n) {
+    if (n.type != RecNode::Kernel || n.head != 0 || !n.k->fn_batched) return false;
+    for (uint64_t p : n.ptrs)
+        if (p & 15) return false;
+    return true;
+}
+
+int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
+    std::vector<RecNode>& nodes = dev->recorded;
+    assign_levels(nodes);
+    int max_level = -1;
+    for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
+    g->recorded = nodes.size();
+    g->levels = static_cast<size_t>(max_level + 1);
+
+    // plan: per level, either single nodes or batches of node indices
+    struct Planned {
+        std::vector<size_t> members;  // indices into `nodes`; more than one = batched launch
+        size_t table_offset = 0;      // in u64 entries
+    };
+    std::vector<std::vector<Planned>> plan(static_cast<size_t>(max_level + 1));
+    std::vector<uint64_t> host_table;
+    for (int level = 0; level <= max_level; level++) {
+        std::vector<Planned>& out = plan[level];
+        // batches keyed by (kernel, n), in first-seen order
+        std::vector<std::pair<std::pair<custos_hip_kernel*, unsigned long long>, size_t>> keys;
+        for (size_t i = 0; i < nodes.size(); i++) {
+            if (nodes[i].level != level) continue;
+            if (dev->batching && batchable(nodes[i])) {
+                const auto key = std::make_pair(nodes[i].k, nodes[i].n);
+                size_t slot = out.size();
+                for (const auto& kv : keys)
+                    if (kv.first == key) slot = kv.second;
+                if (slot == out.size()) {
+                    keys.push_back({key, slot});
+                    out.emplace_back();
+                }
+                out[slot].members.push_back(i);
+            } else {
+                out.emplace_back();
+                out.back().members.push_back(i);
+            }
+        }
+        for (Planned& p : out) {
+            if (p.members.size() < 2) continue;
+            p.table_offset = host_table.size();
+            for (size_t i : p.members)
+                for (uint64_t ptr : nodes[i].ptrs) host_table.push_back(ptr);
+        }
+    }
+    if (!host_table.empty()) {
+        HIP_TRY(dev, hipMalloc(&g->table, host_table.size() * sizeof(uint64_t)));
+        HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
+    }
+
+    HIP_TRY(dev, hipGraphCreate(&g->graph, 0));
+    std::vector<hipGraphNode_t> prev;  // what the nodes of the current level wait for
+    for (int level = 0; level <= max_level; level++) {
+        std::vector<hipGraphNode_t> deps = prev;
+        if (deps.size() > 1) {  // one join node instead of |prev| x |level| edges
+            hipGraphNode_t join;
+            HIP_TRY(dev, hipGraphAddEmptyNode(&join, g->graph, deps.data(), deps.size()));
+            deps = {join};
+        }
+        std::vector<hipGraphNode_t> made;
+        for (const Planned& p : plan[level]) {
+            const RecNode& first = nodes[p.members[0]];
+            hipGraphNode_t node;
+            if (first.type == RecNode::Copy) {
+                HIP_TRY(dev, hipGraphAddMemcpyNode1D(&node, g->graph, deps.data(), deps.size(),
+                                                     reinterpret_cast<void*>(first.ptrs[0]),
+                                                     reinterpret_cast<const void*>(first.ptrs[1]), first.bytes,
+                                                     hipMemcpyDeviceToDevice));
+                made.push_back(node);
+                continue;
+            }
+            hipKernelNodeParams kp{};
+            kp.sharedMemBytes = 0;
+            kp.extra = nullptr;
+            std::vector<void*> args;
+            uint64_t ptrs[8];
+            unsigned long long a0, a1, a2, a3;
+            if (first.type == RecNode::Fill) {
+                ptrs[0] = first.ptrs[0];
+                a0 = first.bytes, a1 = first.head, a2 = first.n_vec;
+                args = {&ptrs[0], &a0, &a1, &a2};
+                kp.func = reinterpret_cast<void*>(custos_fill_zero);
+                kp.gridDim = dim3(fill_grid(dev, first.n_vec));
+                kp.blockDim = dim3(256);
+            } else if (p.members.size() == 1) {
+                for (size_t i = 0; i < first.ptrs.size(); i++) {
+                    ptrs[i] = first.ptrs[i];
+                    args.push_back(&ptrs[i]);
+                }
+                a0 = first.n, a1 = first.head, a2 = first.n_vec;
+                args.push_back(&a0);
+                args.push_back(&a1);
+                args.push_back(&a2);
+                kp.func = reinterpret_cast<void*>(first.k->fn);
+                kp.gridDim = dim3(first.grid);
+                kp.blockDim = dim3(static_cast<unsigned int>(first.k->spec.tuning.block_threads));
+            } else {
+                const Tuning& t = first.k->spec.tuning;
+                const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+                a3 = std::max(1ull, (first.n_vec + tile_vecs - 1) / tile_vecs);  // tiles per segment
+                const unsigned long long blocks = a3 * p.members.size();
+                if (blocks > (1ull << 31) - 1)
+                    return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a batched launch would need more than 2^31 workgroups");
+                ptrs[0] = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
+                a0 = first.n, a1 = first.n_vec;
+                args = {&ptrs[0], &a0, &a1, &a3};
+                kp.func = reinterpret_cast<void*>(first.k->fn_batched);
+                kp.gridDim = dim3(static_cast<unsigned int>(blocks));
+                kp.blockDim = dim3(static_cast<unsigned int>(t.block_threads));
+            }
+            kp.kernelParams = args.data();
+            HIP_TRY(dev, hipGraphAddKernelNode(&node, g->graph, deps.data(), deps.size(), &kp));
+            g->kernel_nodes++;
+            made.push_back(node);
+        }
+        prev = std::move(made);
+    }
+    HIP_TRY(dev, hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
+    return CUSTOS_HIP_OK;
+}
+
+void destroy_graph(custos_hip_graph* g) {
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    if (g->table) (void)hipFree(g->table);
+    delete g;
 }
 
 }  // namespace
@@ -279,18 +529,9 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
 int32_t custos_hip_device_destroy(custos_hip_device* dev) {
     if (!dev) return CUSTOS_HIP_OK;
     (void)hipSetDevice(dev->idx);
-    if (dev->capturing) {
-        hipGraph_t g = nullptr;
-        (void)hipStreamEndCapture(dev->stream, &g);
-        if (g) (void)hipGraphDestroy(g);
-    }
     (void)hipStreamSynchronize(dev->stream);
     (void)hipStreamSynchronize(dev->transfer);
-    for (custos_hip_graph* g : dev->graphs) {
-        if (g->exec) (void)hipGraphExecDestroy(g->exec);
-        if (g->graph) (void)hipGraphDestroy(g->graph);
-        delete g;
-    }
+    for (custos_hip_graph* g : dev->graphs) destroy_graph(g);
     for (auto& bucket : dev->cache)
         for (auto& k : bucket.second)
             if (k->module) (void)hipModuleUnload(k->module);
@@ -411,6 +652,15 @@ int32_t custos_hip_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size
     REQUIRE_DEV(dev);
     if (bytes == 0) return CUSTOS_HIP_OK;
     if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    if (dev->capturing) {
+        RecNode node;
+        node.type = RecNode::Copy;
+        node.ptrs = {dst, src};
+        node.bytes = bytes;
+        node.acc = {{dst, dst + bytes, true}, {src, src + bytes, false}};
+        dev->recorded.push_back(std::move(node));
+        return CUSTOS_HIP_OK;
+    }
     HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src), bytes,
                                 hipMemcpyDeviceToDevice, dev->stream));
     return CUSTOS_HIP_OK;
@@ -455,6 +705,11 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
     if (e != hipSuccess) {
         (void)hipModuleUnload(k->module);
         return hip_fail(dev, e, "hipModuleGetFunction");
+    }
+    // the second entry point of the module: many equal launches in one grid
+    if (hipModuleGetFunction(&k->fn_batched, k->module, (k->spec.name + "_batched").c_str()) != hipSuccess) {
+        (void)hipGetLastError();
+        k->fn_batched = nullptr;
     }
     dev->compiles++;
     *kernel = k.get();
@@ -533,22 +788,7 @@ int32_t custos_hip_apply_fn_n(custos_hip_device* dev, custos_hip_kernel* kernel,
     std::vector<Range> ops;
     for (int i = 0; i < n_ins; i++) ops.push_back({ins[i], false});
     ops.push_back({out, true});
-    unsigned long long head, n_vec, count = n;
-    unsigned int grid;
-    int32_t rc = plan_launch(dev, kernel, ops, n, &head, &n_vec, &grid);
-    if (rc != CUSTOS_HIP_OK) return rc;
-    uint64_t ptrs[5];
-    std::vector<void*> args;
-    for (int i = 0; i < n_ins; i++) {
-        ptrs[i] = ins[i];
-        args.push_back(&ptrs[i]);
-    }
-    ptrs[4] = out;
-    args.push_back(&ptrs[4]);
-    args.push_back(&count);
-    args.push_back(&head);
-    args.push_back(&n_vec);
-    return launch(dev, kernel, args, grid);
+    return launch_or_record(dev, kernel, ops, n);
 }
 
 int32_t custos_hip_apply_fn(custos_hip_device* dev, custos_hip_kernel* kernel, uint64_t x, uint64_t out, size_t n) {
@@ -569,22 +809,19 @@ int32_t custos_hip_add_unary_grad(custos_hip_device* dev, custos_hip_kernel* ker
         return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled as a unary-gradient kernel");
     if (n == 0) return CUSTOS_HIP_OK;
     std::vector<Range> ops = {{lhs, false}, {lhs_grad, true}, {out_grad, false}};
-    unsigned long long head, n_vec, count = n;
-    unsigned int grid;
-    int32_t rc = plan_launch(dev, kernel, ops, n, &head, &n_vec, &grid);
-    if (rc != CUSTOS_HIP_OK) return rc;
-    std::vector<void*> args = {&lhs, &lhs_grad, &out_grad, &count, &head, &n_vec};
-    return launch(dev, kernel, args, grid);
+    return launch_or_record(dev, kernel, ops, n);
 }
 
 // ---- capture / replay ----
 
 int32_t custos_hip_capture_begin(custos_hip_device* dev) {
     REQUIRE_DEV(dev);
-    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the stream is already recording");
-    // relaxed: allocation, reads and writes stay legal while recording; they are
-    // issued on the transfer stream and are not part of the graph
-    HIP_TRY(dev, hipStreamBeginCapture(dev->stream, hipStreamCaptureModeRelaxed));
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the device is already recording");
+    // Earlier eager work must be complete before anything recorded can run, and
+    // the recorded list starts empty.  Allocation, reads and writes stay legal
+    // while recording: they execute at once and are not part of the graph.
+    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    dev->recorded.clear();
     dev->capturing = true;
     return CUSTOS_HIP_OK;
 }
@@ -593,28 +830,23 @@ int32_t custos_hip_capture_end(custos_hip_device* dev, custos_hip_graph** graph)
     REQUIRE_DEV(dev);
     if (!graph) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph out pointer is null");
     *graph = nullptr;
-    if (!dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the stream is not recording");
+    if (!dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the device is not recording");
     dev->capturing = false;
-    std::unique_ptr<custos_hip_graph> g(new custos_hip_graph);
-    HIP_TRY(dev, hipStreamEndCapture(dev->stream, &g->graph));
-    if (!g->graph) HIP_TRY(dev, hipGraphCreate(&g->graph, 0));  // nothing was recorded
-    size_t n_nodes = 0;
-    HIP_TRY(dev, hipGraphGetNodes(g->graph, nullptr, &n_nodes));
-    if (n_nodes) {
-        std::vector<hipGraphNode_t> nodes(n_nodes);
-        HIP_TRY(dev, hipGraphGetNodes(g->graph, nodes.data(), &n_nodes));
-        for (hipGraphNode_t node : nodes) {
-            hipGraphNodeType type;
-            if (hipGraphNodeGetType(node, &type) == hipSuccess && type == hipGraphNodeTypeKernel) g->kernel_nodes++;
-        }
+    custos_hip_graph* g = new custos_hip_graph;
+    int32_t rc = build_graph(dev, g);
+    dev->recorded.clear();
+    if (rc != CUSTOS_HIP_OK) {
+        destroy_graph(g);
+        return rc;
     }
-    hipError_t e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
-    if (e != hipSuccess) {
-        (void)hipGraphDestroy(g->graph);
-        return hip_fail(dev, e, "hipGraphInstantiate");
-    }
-    dev->graphs.push_back(g.get());
-    *graph = g.release();
+    dev->graphs.push_back(g);
+    *graph = g;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_graph_batching(custos_hip_device* dev, int32_t enabled) {
+    REQUIRE_DEV(dev);
+    dev->batching = enabled != 0;
     return CUSTOS_HIP_OK;
 }
 
@@ -639,6 +871,14 @@ int32_t custos_hip_graph_node_count(custos_hip_graph* graph, size_t* kernel_node
     return CUSTOS_HIP_OK;
 }
 
+int32_t custos_hip_graph_stats(custos_hip_graph* graph, size_t* recorded, size_t* kernel_nodes, size_t* levels) {
+    if (!graph) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph is null");
+    if (recorded) *recorded = graph->recorded;
+    if (kernel_nodes) *kernel_nodes = graph->kernel_nodes;
+    if (levels) *levels = graph->levels;
+    return CUSTOS_HIP_OK;
+}
+
 int32_t custos_hip_graph_destroy(custos_hip_device* dev, custos_hip_graph* graph) {
     REQUIRE_DEV(dev);
     if (!graph) return CUSTOS_HIP_OK;
@@ -646,9 +886,7 @@ int32_t custos_hip_graph_destroy(custos_hip_device* dev, custos_hip_graph* graph
     if (it == dev->graphs.end()) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph does not belong to this device");
     dev->graphs.erase(it);
     HIP_TRY(dev, hipStreamSynchronize(dev->stream));
-    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
-    if (graph->graph) (void)hipGraphDestroy(graph->graph);
-    delete graph;
+    destroy_graph(graph);
     return CUSTOS_HIP_OK;
 }
 

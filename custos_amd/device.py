@@ -87,6 +87,12 @@ class Graph:
         self.device._check(self.device.lib.custos_hip_graph_node_count(self.handle, C.byref(n)))
         return n.value
 
+    def stats(self):
+        """(recorded pieces of work, kernel nodes in the graph, dependency levels)"""
+        a, b, c = C.c_size_t(0), C.c_size_t(0), C.c_size_t(0)
+        self.device._check(self.device.lib.custos_hip_graph_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
     def destroy(self) -> None:
         if self.handle and self.device.handle:
             self.device._check(self.device.lib.custos_hip_graph_destroy(self.device.handle, self.handle))
@@ -238,6 +244,9 @@ class HIP:
         g = C.c_void_p()
         self._check(self.lib.custos_hip_capture_end(self.handle, C.byref(g)))
         return Graph(self, g)
+
+    def set_graph_batching(self, enabled: bool) -> None:
+        self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 
     def is_capturing(self) -> bool:
         v = C.c_int32(0)

@@ -214,14 +214,25 @@ int32_t custos_hip_add_unary_grad(custos_hip_device *dev, custos_hip_kernel *ker
 
 /* ---- lazy run: capture once, replay (src/devices/cuda/lazy.rs:10-72) ---- */
 
-/* LazySetup::lazy_setup: from here on launches/clears/copies are recorded, not run. */
+/* LazySetup::lazy_setup: from here on launches/clears/copies are recorded, not run.
+ * Allocation, reads and writes stay legal while recording and execute at once. */
 int32_t custos_hip_capture_begin(custos_hip_device *dev);
-/* Ends recording and instantiates an executable graph (LazyCudaGraph::new). */
+/* Ends recording and instantiates an executable graph (LazyCudaGraph::new).
+ * The graph is built from the recorded work, not replayed launch by launch:
+ * work that does not touch the same memory runs side by side, and independent
+ * launches of the same kernel over the same length are merged into one grid
+ * (1024 buffers x 3 operations replay as 3 kernel nodes). */
 int32_t custos_hip_capture_end(custos_hip_device *dev, custos_hip_graph **graph);
+/* Switches the merging of equal independent launches off (0) or on (default):
+ * with it off every recorded launch becomes its own kernel node. */
+int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
 int32_t custos_hip_is_capturing(custos_hip_device *dev, int32_t *capturing);
 /* LazyCudaGraph::launch on the compute stream (no wait; call custos_hip_sync). */
 int32_t custos_hip_graph_launch(custos_hip_device *dev, custos_hip_graph *graph);
 int32_t custos_hip_graph_node_count(custos_hip_graph *graph, size_t *kernel_nodes);
+/* Recorded pieces of work, kernel nodes in the instantiated graph, dependency levels. */
+int32_t custos_hip_graph_stats(custos_hip_graph *graph, size_t *recorded, size_t *kernel_nodes,
+                               size_t *levels);
 int32_t custos_hip_graph_destroy(custos_hip_device *dev, custos_hip_graph *graph);
 
 /* ---- timing on the compute stream (bench support) ---- */

@@ -104,26 +104,38 @@ def test_c5_graph_replay(hip, oracle):
     y = [hip.alloc(n) for _ in range(nbuf)]
     unary = [lambda v: v.abs().sqrt(), lambda v: v.mul(0.3)]
 
-    hip.capture_begin()
-    for i in range(nbuf):
-        hip.apply_fn2(ab[i], bb[i], lambda p, q: p.mul(q), out=t[i])
-        hip.apply_fn2(t[i], cb[i], lambda p, q: p.add(q), out=u[i])
-        hip.fused_apply_fn(u[i], unary, out=y[i])
-    graph = hip.capture_end()
-    assert graph.kernel_nodes == 3 * nbuf
-    # nothing ran while recording: outputs are still the zeros of alloc
-    assert not y[0].read().any()
-    for replay in range(3):
-        graph.launch()
-        hip.sync()
-        for i in (0, 1, nbuf // 2, nbuf - 1):
-            tt, uu, yy = oracle.c5_graph(a[i], b[i], c[i])
-            assert_bits_equal(t[i].read(), tt)
-            assert_bits_equal(u[i].read(), uu)
-            assert_bits_equal(y[i].read(), yy, f"replay {replay} buffer {i}")
-        y[0].clear()
-        hip.sync()
-    graph.destroy()
+    def record():
+        hip.capture_begin()
+        for i in range(nbuf):
+            hip.apply_fn2(ab[i], bb[i], lambda p, q: p.mul(q), out=t[i])
+            hip.apply_fn2(t[i], cb[i], lambda p, q: p.add(q), out=u[i])
+            hip.fused_apply_fn(u[i], unary, out=y[i])
+        return hip.capture_end()
+
+    for batching in (True, False):
+        hip.set_graph_batching(batching)
+        try:
+            graph = record()
+        finally:
+            hip.set_graph_batching(True)
+        recorded, kernel_nodes, levels = graph.stats()
+        assert (recorded, levels) == (3 * nbuf, 3)
+        # the 64 independent chains run side by side; with batching every level is ONE launch
+        assert kernel_nodes == (3 if batching else 3 * nbuf)
+        # nothing ran while recording: outputs are still the zeros of alloc / of the last clear
+        assert not y[0].read().any()
+        for replay in range(3):
+            graph.launch()
+            hip.sync()
+            for i in (0, 1, nbuf // 2, nbuf - 1):
+                tt, uu, yy = oracle.c5_graph(a[i], b[i], c[i])
+                assert_bits_equal(t[i].read(), tt)
+                assert_bits_equal(u[i].read(), uu)
+                assert_bits_equal(y[i].read(), yy, f"batching={batching} replay {replay} buffer {i}")
+            for i in range(nbuf):
+                y[i].clear()
+            hip.sync()
+        graph.destroy()
 
 
 @pytest.mark.parametrize("log2n", [28])

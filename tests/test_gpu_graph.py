@@ -115,3 +115,111 @@ def test_capture_state_errors(hip):
     assert g.kernel_nodes == 0
     g.launch()                               # an empty graph replays fine
     hip.sync()
+
+
+def test_batched_launch_with_tails_and_mixed_lengths(hip, oracle):
+    """Independent launches of one kernel: equal lengths merge into one grid (including a
+    scalar tail per buffer), other lengths and unaligned views stay separate nodes."""
+    f = lambda v: v.mul(1.5).add(0.25)
+    lens = [1003] * 40 + [7] * 5 + [4096] * 3 + [1]
+    xs = [synth.uniform_f32(100 + i, n, -2, 2) for i, n in enumerate(lens)]
+    bufs = [hip.buffer(x) for x in xs]
+    outs = [hip.alloc(n) for n in lens]
+    big = hip.buffer(synth.uniform_f32(7, 1003 + 3, -2, 2))
+    big_out = hip.alloc(1003 + 3)
+    hip.capture_begin()
+    for b, o in zip(bufs, outs):
+        hip.apply_fn(b, f, out=o)
+    hip.apply_fn(big.slice(3, 1006), f, out=big_out.slice(3, 1006))   # same length, not 16-byte aligned
+    g = hip.capture_end()
+    recorded, kernel_nodes, levels = g.stats()
+    assert recorded == len(lens) + 1 and levels == 1
+    assert kernel_nodes == 3 + 1 + 1      # batches for 1003, 7, 4096; the single n=1; the unaligned view
+    for _ in range(2):
+        g.launch()
+        hip.sync()
+        for x, o in zip(xs, outs):
+            assert_bits_equal(o.read(), oracle.apply_fn(f, x))
+        assert_bits_equal(big_out.read()[3:], oracle.apply_fn(f, big.read()[3:]))
+        assert not big_out.read()[:3].any()
+
+
+def test_recorded_dependencies_random(hip, oracle):
+    """Random programs over a small pool of buffers, with in-place updates, views and clears:
+    replaying the built graph (levels, side-by-side nodes, merged launches) must equal running
+    the same calls eagerly, bit for bit."""
+    rng = np.random.default_rng(1234)
+    n = 2048
+    fns1 = [lambda v: v.mul(1.25).add(0.5), lambda v: v.neg().max(-3.0), lambda v: v.abs().sqrt(), lambda v: v.mul(v).min(9.0)]
+    fns2 = [lambda p, q: p.add(q), lambda p, q: p.mul(q).sub(0.125), lambda p, q: p.max(q)]
+    for trial in range(6):
+        nbuf = 6
+        init = [synth.uniform_f32(trial * 10 + i, n, -2, 2) for i in range(nbuf)]
+        program = []
+        for _ in range(40):
+            kind = rng.integers(0, 5)
+            lo = int(rng.integers(0, 3)) * 512          # views: [lo, lo + 1024) keeps 16-byte phases equal
+            if kind == 0:
+                program.append(("u", int(rng.integers(len(fns1))), int(rng.integers(nbuf)), int(rng.integers(nbuf)), lo))
+            elif kind in (1, 2):
+                a, b, o = (int(v) for v in rng.integers(nbuf, size=3))
+                program.append(("b", int(rng.integers(len(fns2))), a, b, o, lo))
+            elif kind == 3:
+                program.append(("g", int(rng.integers(len(fns1))), *(int(v) for v in rng.choice(nbuf, size=3, replace=False)), lo))
+            else:
+                program.append(("c", int(rng.integers(nbuf)), lo))
+
+        def run(bufs):
+            for op in program:
+                if op[0] == "u":
+                    _, fi, src, dst, lo = op
+                    if src == dst:
+                        hip.apply_fn(bufs[src].slice(lo, lo + 1024), fns1[fi], out=bufs[dst].slice(lo, lo + 1024))
+                    else:
+                        hip.apply_fn(bufs[src].slice(lo, lo + 1024), fns1[fi], out=bufs[dst].slice(lo, lo + 1024))
+                elif op[0] == "b":
+                    _, fi, a, b, o, lo = op
+                    if a == b or (o in (a, b) and False):
+                        continue
+                    hip.apply_fn2(bufs[a].slice(lo, lo + 1024), bufs[b].slice(lo, lo + 1024), fns2[fi],
+                                  out=bufs[o].slice(lo, lo + 1024))
+                elif op[0] == "g":
+                    _, fi, x, g, o, lo = op
+                    hip.add_unary_grad(bufs[x].slice(lo, lo + 1024), bufs[g].slice(lo, lo + 1024),
+                                       bufs[o].slice(lo, lo + 1024), fns1[fi])
+                else:
+                    _, b, lo = op
+                    bufs[b].slice(lo, lo + 1024).clear()
+
+        eager = [hip.buffer(x) for x in init]
+        run(eager)
+        hip.sync()
+        want = [b.read() for b in eager]
+        lazy = [hip.buffer(x) for x in init]
+        hip.capture_begin()
+        run(lazy)
+        g = hip.capture_end()
+        for b, x in zip(lazy, init):
+            assert_bits_equal(b.read(), x, "nothing may run while recording")
+        g.launch()
+        hip.sync()
+        for i, b in enumerate(lazy):
+            assert_bits_equal(b.read(), want[i], f"trial {trial} buffer {i} (levels {g.stats()})")
+        g.destroy()
+
+
+def test_recorded_copy_nodes(hip):
+    x = synth.uniform_f32(3, 5000, -1, 1)
+    a, b, c = hip.buffer(x), hip.alloc(5000), hip.alloc(5000)
+    hip.capture_begin()
+    hip.copy(b, a)
+    hip.apply_fn(b, lambda v: v.mul(2.0), out=c)
+    hip.copy(a, c)
+    g = hip.capture_end()
+    assert g.stats() == (3, 1, 3)
+    g.launch()
+    hip.sync()
+    assert_bits_equal(a.read(), (x * np.float32(2.0)).astype(np.float32))
+    g.launch()
+    hip.sync()
+    assert_bits_equal(a.read(), (x * np.float32(4.0)).astype(np.float32))
