@@ -19,6 +19,7 @@ elements/s, GB/s and the CPU port timed beside it (skip with --no-others).
 from __future__ import annotations
 
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -305,8 +306,29 @@ def bench_others(dev, args):
     e["graph_kernel_nodes"] = graph.kernel_nodes
     e["recorded_launches"] = 3 * nbuf
     e["graph_build_ms"] = round(build_s * 1e3, 2)
-    out["c5"] = e
     graph.destroy()
+
+    # the same work after element-wise fusing (what `Lazy::elementwise_fusing` of the host stack
+    # records): one three-operand kernel per buffer, 16 B/element, merged into one kernel node
+    kf = dev.compile(capi.KIND_APPLY, "f32", "(sqrt(abs(((a * b) + c))) * 0.3)", ("a", "b", "c"))
+    Y.clear()
+    dev.capture_begin()
+    for i in range(nbuf):
+        o = i * m * 4
+        ptrs = (C.c_uint64 * 3)(A.ptr + o, B.ptr + o, Cc.ptr + o)
+        capi.check(lib.custos_hip_apply_fn_n(h, kf, ptrs, 3, Y.ptr + o, m), h)
+    fgraph = dev.capture_end()
+    fms, fwall = time_steps(dev, fgraph.launch, replays, 3)
+    assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), "c5 fused replay differs from the CPU port"
+    e["fused"] = {
+        "us_per_replay": round(fms / replays * 1e3, 2),
+        "wall_us_per_replay": round(fwall / replays * 1e3, 2),
+        "GBps": round(16 * nbuf * m / (fms / replays * 1e-3) / 1e9, 2),
+        "graph_kernel_nodes": fgraph.kernel_nodes,
+        "expression": "(sqrt(abs(((a * b) + c))) * 0.3)",
+    }
+    out["c5"] = e
+    fgraph.destroy()
     return out
 
 

@@ -112,6 +112,75 @@ OpHint<T> unary(F f) {
     return OpHint<T>{OpHintKind::Unary, std::move(h)};
 }
 
+// ---- expression hints of any arity ----
+//
+// The reference tags only unary operations (`OpHint::Unary`), so only unary
+// chains can be fused.  Every element-wise operation recorded through
+// `apply_fn` / `apply_fn2` additionally carries an `ExprHint`: the expression
+// over k operands, re-printable with any operand texts and evaluable on the
+// host.  `Lazy::elementwise_fusing` composes them across operations.
+template <class T>
+struct ExprHint {
+    int arity = 1;
+    // the expression's text with `operands[i]` in place of the i-th marker
+    std::function<std::string(const std::vector<std::string>& operands)> to_cl_source;
+    // the expression's value for the operand values `vals[0..arity)`
+    std::function<T(const T* vals)> eval;
+};
+
+template <class T, class F>
+std::shared_ptr<ExprHint<T>> expr_hint1(F f) {
+    auto h = std::make_shared<ExprHint<T>>();
+    h->arity = 1;
+    h->to_cl_source = [f](const std::vector<std::string>& m) {
+        return custos::to_cl_source(f(Resolve<T>::with_marker(m[0].c_str())));
+    };
+    h->eval = [f](const T* v) { return custos::eval<T>(f(Resolve<T>::with_val(v[0]))); };
+    return h;
+}
+
+template <class T, class F>
+std::shared_ptr<ExprHint<T>> expr_hint2(F f) {
+    auto h = std::make_shared<ExprHint<T>>();
+    h->arity = 2;
+    h->to_cl_source = [f](const std::vector<std::string>& m) {
+        return custos::to_cl_source(f(Resolve<T>::with_marker(m[0].c_str()), Resolve<T>::with_marker(m[1].c_str())));
+    };
+    h->eval = [f](const T* v) { return custos::eval<T>(f(Resolve<T>::with_val(v[0]), Resolve<T>::with_val(v[1]))); };
+    return h;
+}
+
+// Several hinted operations composed into one expression over `leaves.size()`
+// distinct operand buffers.  Item inputs >= 0 name a leaf, inputs < 0 name
+// another item (~input).
+template <class T>
+struct FusedExpr {
+    struct Item {
+        std::shared_ptr<ExprHint<T>> hint;
+        std::vector<int> inputs;
+    };
+    std::vector<Item> items;
+    int root = 0;
+    std::vector<Id> leaves;
+
+    std::string to_cl_source(const std::vector<std::string>& leaf_markers) const { return print(root, leaf_markers); }
+    T eval(const T* leaf_vals) const { return eval_item(root, leaf_vals); }
+    size_t op_count() const { return items.size(); }
+
+   private:
+    std::string print(int item, const std::vector<std::string>& leaf_markers) const {
+        std::vector<std::string> operands;
+        for (int in : items[item].inputs) operands.push_back(in >= 0 ? leaf_markers[in] : print(~in, leaf_markers));
+        return items[item].hint->to_cl_source(operands);
+    }
+    T eval_item(int item, const T* leaf_vals) const {
+        T vals[8];
+        const auto& ins = items[item].inputs;
+        for (size_t i = 0; i < ins.size(); i++) vals[i] = ins[i] >= 0 ? leaf_vals[ins[i]] : eval_item(~ins[i], leaf_vals);
+        return items[item].hint->eval(vals);
+    }
+};
+
 // `operations_to_fused_src` (src/devices/fusing.rs:4-19)
 template <class T>
 std::string operations_to_fused_src(const std::vector<std::shared_ptr<UnaryHint<T>>>& ops) {

@@ -141,6 +141,21 @@ class Device {
             dev.apply_fn_impl(x, o, f);
         });
         modules.set_op_hint(erase_hint(unary<T>(f)));
+        modules.set_expr_hint(AnyExprHint{expr_hint1<T>(f), std::type_index(typeid(T)), {1}, 0});
+        return out;
+    }
+
+    // A two-operand element-wise operation in the reference's style for user ops
+    // (retrieve + add_op, like the `add` of tests/graph/mod.rs:90-127), with the
+    // expression written in the `Combiner` vocabulary: out[i] = f(lhs[i], rhs[i]).
+    template <class T, class F>
+    Buffer<T, Derived> apply_fn2(const Buffer<T, Derived>& lhs, const Buffer<T, Derived>& rhs, F f) {
+        Buffer<T, Derived> out = retrieve<T>(lhs.len(), lhs, rhs);
+        add_op(std::tie(lhs, rhs, out),
+               [f](const Buffer<T, Derived>& l, const Buffer<T, Derived>& r, Buffer<T, Derived>& o, Derived& dev) {
+                   dev.apply_fn2_impl(l, r, o, f);
+               });
+        modules.set_expr_hint(AnyExprHint{expr_hint2<T>(f), std::type_index(typeid(T)), {0, 1}, 2});
         return out;
     }
 
@@ -182,6 +197,8 @@ class Device {
     }
     void optimize_mem_graph() { modules.optimize_mem_graph(self(), nullptr); }
     void unary_fusing() { modules.unary_fusing(self(), nullptr); }
+    // Fuses element-wise operations of any arity (unary chains included); needs `Graph`.
+    void elementwise_fusing() { modules.elementwise_fusing(self(), nullptr, {}); }
 
     // ---- autograd ----
 

@@ -134,16 +134,25 @@ class HIP : public Device<HIP<Mods>, Mods> {
         };
     }
 
-    // A user-level two-operand op in the reference's style (retrieve + add_op),
-    // e.g. the `add` of tests/graph/mod.rs:90-127 without a hand-written kernel.
-    template <class T, class F>
-    Buffer<T, Self> apply_fn2(const Buffer<T, Self>& lhs, const Buffer<T, Self>& rhs, F f) {
-        Buffer<T, Self> out = this->template retrieve<T>(lhs.len(), lhs, rhs);
-        this->add_op(std::tie(lhs, rhs, out),
-                     [f](const Buffer<T, Self>& l, const Buffer<T, Self>& r, Buffer<T, Self>& o, Self& dev) {
-                         dev.apply_fn2_impl(l, r, o, f);
-                     });
-        return out;
+    // The operation `Lazy::elementwise_fusing` puts in place of several hinted
+    // operations: one kernel over up to four operand buffers.
+    template <class T>
+    std::function<void(Buffer<T, Self>&, const std::vector<Buffer<T, Self>>&, Self&)> elementwise_fuse_op(
+        std::shared_ptr<FusedExpr<T>> expr) {
+        return [expr](Buffer<T, Self>& out, const std::vector<Buffer<T, Self>>& ins, Self& dev) {
+            static const char* const names[] = {"a", "b", "c", "d"};
+            std::vector<std::string> markers;
+            std::vector<const char*> cmarkers;
+            for (size_t i = 0; i < ins.size(); i++) markers.push_back(names[i]);
+            for (size_t i = 0; i < ins.size(); i++) cmarkers.push_back(names[i]);
+            const std::string src = expr->to_cl_source(markers);
+            custos_hip_kernel* k = nullptr;
+            dev.check(custos_hip_expr_compile(dev.dev_, CUSTOS_HIP_KIND_APPLY, HipDType<T>::value, src.c_str(),
+                                              cmarkers.data(), static_cast<int32_t>(cmarkers.size()), &k));
+            uint64_t ptrs[4];
+            for (size_t i = 0; i < ins.size(); i++) ptrs[i] = ins[i].ptr();
+            dev.check(custos_hip_apply_fn_n(dev.dev_, k, ptrs, static_cast<int32_t>(ins.size()), out.ptr(), out.len()));
+        };
     }
 
     // ---- Lazy hooks ----

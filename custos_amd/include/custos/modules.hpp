@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <cstddef>
 #include <functional>
+#include <memory>
 #include <typeindex>
 #include <vector>
 
@@ -27,6 +28,14 @@ struct Operation {
     OpHintKind hint_kind = OpHintKind::None;
     std::shared_ptr<void> unary_hint;
     std::type_index hint_type = std::type_index(typeid(void));
+    // expression hint of any arity (type-erased ExprHint<T>): which arguments the
+    // expression reads, in operand order, and which one it writes
+    std::shared_ptr<void> expr_hint;
+    std::type_index expr_type = std::type_index(typeid(void));
+    std::vector<int> in_args;
+    int out_arg = -1;
+    // text of the expression a fused operation computes, over markers a, b, c, d
+    std::string fused_source;
 
     static Operation no_op() {
         Operation o;
@@ -39,6 +48,13 @@ struct AnyOpHint {
     OpHintKind kind = OpHintKind::None;
     std::shared_ptr<void> unary;
     std::type_index type = std::type_index(typeid(void));
+};
+
+struct AnyExprHint {
+    std::shared_ptr<void> hint;
+    std::type_index type = std::type_index(typeid(void));
+    std::vector<int> in_args;
+    int out_arg = -1;
 };
 
 template <class T>
@@ -81,6 +97,9 @@ struct Base {
     void set_lazy_enabled(bool) {}
     bool is_lazy_enabled() const { return false; }
     void set_op_hint(AnyOpHint) {}
+    void set_expr_hint(AnyExprHint) {}
+    template <class D>
+    void elementwise_fusing(D&, const GraphTranslator*, const std::vector<UniqueId>&) {}
     template <class D>
     void exec_now(D&, size_t, size_t) {}
     template <class D>
@@ -179,6 +198,14 @@ struct Lazy {
         graph.back().hint_kind = h.kind;
         graph.back().unary_hint = std::move(h.unary);
         graph.back().hint_type = h.type;
+    }
+
+    void set_expr_hint(AnyExprHint h) {
+        if (!enabled_ || graph.empty()) return;
+        graph.back().expr_hint = std::move(h.hint);
+        graph.back().expr_type = h.type;
+        graph.back().in_args = std::move(h.in_args);
+        graph.back().out_arg = h.out_arg;
     }
 
     // Runs and drains operations [begin, end) now (lazy.rs:145-162, lazy_graph.rs:93-104).
@@ -294,6 +321,172 @@ struct Lazy {
         }
     }
 
+    // Fuses element-wise operations of any arity across operations: an operation
+    // whose only reader is another hinted operation is inlined into that reader,
+    // repeatedly, so `t = a*b; u = t+c; y = sqrt(abs(u))*0.3` becomes one
+    // three-operand kernel that moves 16 bytes per element instead of 32.
+    // (The reference fuses unary chains only; unary chains are the one-operand
+    // case of this.)  An operation is inlined only if its output
+    //   - was retrieved lazily (not a buffer the user filled),
+    //   - is read by exactly one recorded operation and is not in `keep` (the
+    //     Autograd module lists what its gradient functions read),
+    //   - is not a checkpoint, has the reader's length,
+    //   - and none of its own operands is written between it and the reader;
+    // the fused operation takes the reader's place and may have at most four
+    // distinct operand buffers.  Intermediates are never computed (they keep the
+    // zeros of their allocation), as with unary fusing.
+    template <class D>
+    void elementwise_fusing(D& dev, const GraphTranslator* gt, const std::vector<UniqueId>& keep) {
+        if (!gt) throw Error(DeviceError::MissingCacheTraces);
+        const std::type_index tt(typeid(T));
+        const size_t n_ops = graph.size();
+        auto hinted = [&](size_t i) { return graph[i].expr_hint && graph[i].expr_type == tt && graph[i].out_arg >= 0; };
+
+        // readers of every buffer id; producers of lazily retrieved outputs
+        std::unordered_map<UniqueId, int> readers;
+        std::unordered_map<UniqueId, size_t> producer;
+        for (size_t i = 0; i < n_ops; i++) {
+            if (hinted(i)) {
+                for (int a : graph[i].in_args) readers[graph[i].arg_ids[a].id]++;
+                const Id out = graph[i].arg_ids[graph[i].out_arg];
+                if (producer.count(out.id)) readers[out.id] += 2;  // written twice: leave it alone
+                producer[out.id] = i;
+            } else {
+                for (const Id& id : graph[i].arg_ids) readers[id.id] += 2;  // unknown use: never inline
+            }
+        }
+        for (UniqueId id : keep) readers[id] += 2;  // e.g. what gradient functions will read
+
+        auto skipped = [&](UniqueId id) {
+            auto it = gt->buf_id_to_idx.find(id);
+            return it != gt->buf_id_to_idx.end() && gt->opt_graph.nodes[it->second].skip;
+        };
+        auto written_between = [&](const std::vector<Id>& leaves, size_t from, size_t to) {
+            for (size_t j = from + 1; j < to; j++) {
+                if (graph[j].arg_ids.empty()) continue;
+                for (size_t a = 0; a < graph[j].arg_ids.size(); a++) {
+                    if (hinted(j) && static_cast<int>(a) != graph[j].out_arg) continue;  // only reads it
+                    for (const Id& leaf : leaves)
+                        if (graph[j].arg_ids[a].id == leaf.id) return true;
+                }
+            }
+            return false;
+        };
+
+        std::vector<std::unique_ptr<FusedExpr<T>>> exprs(n_ops);
+        std::vector<bool> absorbed(n_ops, false);
+        for (size_t i = 0; i < n_ops; i++) {
+            if (!hinted(i)) continue;
+            auto e = std::make_unique<FusedExpr<T>>();
+            typename FusedExpr<T>::Item item;
+            item.hint = std::static_pointer_cast<ExprHint<T>>(graph[i].expr_hint);
+            auto leaf_index = [&](FusedExpr<T>& fe, Id id) {
+                for (size_t k = 0; k < fe.leaves.size(); k++)
+                    if (fe.leaves[k].id == id.id) return static_cast<int>(k);
+                fe.leaves.push_back(id);
+                return static_cast<int>(fe.leaves.size()) - 1;
+            };
+            for (int a : graph[i].in_args) item.inputs.push_back(leaf_index(*e, graph[i].arg_ids[a]));
+            e->items.push_back(std::move(item));
+            e->root = 0;
+            const Id out = graph[i].arg_ids[graph[i].out_arg];
+
+            // inline producers of leaves until nothing changes
+            bool changed = true;
+            while (changed) {
+                changed = false;
+                for (size_t k = 0; k < e->leaves.size() && !changed; k++) {
+                    const Id leaf = e->leaves[k];
+                    auto p = producer.find(leaf.id);
+                    if (p == producer.end() || p->second >= i || absorbed[p->second] || !exprs[p->second]) continue;
+                    if (!allocated_lazily(leaf.id) || readers[leaf.id] != 1 || skipped(leaf.id) || leaf.len != out.len) continue;
+                    const FusedExpr<T>& pe = *exprs[p->second];
+                    if (written_between(pe.leaves, p->second, i)) continue;
+                    // distinct operand buffers after the merge
+                    // (the producer's operands take the place of the inlined one)
+                    std::vector<Id> merged;
+                    auto push_unique = [&merged](const Id& id) {
+                        for (const Id& m : merged)
+                            if (m.id == id.id) return;
+                        merged.push_back(id);
+                    };
+                    for (size_t q = 0; q < e->leaves.size(); q++) {
+                        if (q != k) push_unique(e->leaves[q]);
+                        else
+                            for (const Id& pl : pe.leaves) push_unique(pl);
+                    }
+                    if (merged.size() > 4) continue;
+                    // rebuild: items of the producer first, then ours, leaves re-indexed
+                    auto fused = std::make_unique<FusedExpr<T>>();
+                    auto remap_leaf = [&](Id id) {
+                        for (size_t q = 0; q < merged.size(); q++)
+                            if (merged[q].id == id.id) return static_cast<int>(q);
+                        return -1;
+                    };
+                    fused->leaves = merged;
+                    const int p_off = 0, own_off = static_cast<int>(pe.items.size());
+                    for (const auto& it : pe.items) {
+                        typename FusedExpr<T>::Item ni{it.hint, {}};
+                        for (int in : it.inputs) ni.inputs.push_back(in >= 0 ? remap_leaf(pe.leaves[in]) : ~(~in + p_off));
+                        fused->items.push_back(std::move(ni));
+                    }
+                    for (const auto& it : e->items) {
+                        typename FusedExpr<T>::Item ni{it.hint, {}};
+                        for (int in : it.inputs) {
+                            if (in < 0) ni.inputs.push_back(~(~in + own_off));
+                            else if (static_cast<size_t>(in) == k) ni.inputs.push_back(~(pe.root + p_off));
+                            else ni.inputs.push_back(remap_leaf(e->leaves[in]));
+                        }
+                        fused->items.push_back(std::move(ni));
+                    }
+                    fused->root = e->root + own_off;
+                    absorbed[p->second] = true;
+                    e = std::move(fused);
+                    changed = true;
+                }
+            }
+            exprs[i] = std::move(e);
+        }
+
+        for (size_t i = 0; i < n_ops; i++) {
+            if (absorbed[i]) {
+                graph[i] = Operation::no_op();
+                continue;
+            }
+            if (!exprs[i] || exprs[i]->items.size() < 2) continue;
+            std::shared_ptr<FusedExpr<T>> fe(std::move(exprs[i]));
+            const Id out_id = graph[i].arg_ids[graph[i].out_arg];
+            Operation fused;
+            fused.arg_ids.push_back(out_id);
+            for (const Id& l : fe->leaves) fused.arg_ids.push_back(l);
+            fused.hint_kind = OpHintKind::UnaryFused;
+            fused.fused_source = fe->to_cl_source({"a", "b", "c", "d"});
+            auto fn = dev.template elementwise_fuse_op<T>(fe);
+            fused.op = [fe, out_id, fn](Buffers& bufs, void* devp) {
+                D& d = *static_cast<D*>(devp);
+                auto view = [&](Id id) {
+                    auto it = bufs.find(id.id);
+                    if (it == bufs.end() || it->second.ptr == 0) throw Error(DeviceError::InvalidLazyBuf);
+                    if (it->second.type != std::type_index(typeid(T))) throw Error(DeviceError::TypeMismatch);
+                    return Buffer<T, D>::from_parts(&d, it->second.ptr, it->second.len, id, AllocFlag::Wrapper);
+                };
+                Buffer<T, D> out = view(out_id);
+                std::vector<Buffer<T, D>> ins;
+                for (const Id& l : fe->leaves) ins.push_back(view(l));
+                fn(out, ins, d);
+            };
+            graph[i] = std::move(fused);
+        }
+        version_++;
+    }
+
+    bool allocated_lazily(UniqueId id) const {
+        if (allocated_ids_.count(id)) return true;
+        for (const Pending& p : alloc_later_)
+            if (p.id.id == id) return true;
+        return false;
+    }
+
     void add_grad_fn(Operation&& op) { modules.add_grad_fn(std::move(op)); }
     void set_grad_enabled(bool e) { modules.set_grad_enabled(e); }
     bool is_grad_enabled() const { return modules.is_grad_enabled(); }
@@ -407,6 +600,7 @@ struct Graph {
     void set_lazy_enabled(bool e) { modules.set_lazy_enabled(e); }
     bool is_lazy_enabled() const { return modules.is_lazy_enabled(); }
     void set_op_hint(AnyOpHint h) { modules.set_op_hint(std::move(h)); }
+    void set_expr_hint(AnyExprHint h) { modules.set_expr_hint(std::move(h)); }
     template <class D>
     void exec_now(D& dev, size_t b, size_t e) {
         modules.exec_now(dev, b, e);
@@ -434,6 +628,10 @@ struct Graph {
     template <class D>
     void unary_fusing(D& dev, const GraphTranslator* gt) {
         modules.unary_fusing(dev, gt ? gt : &graph_trans);
+    }
+    template <class D>
+    void elementwise_fusing(D& dev, const GraphTranslator* gt, const std::vector<UniqueId>& keep) {
+        modules.elementwise_fusing(dev, gt ? gt : &graph_trans, keep);
     }
 
     void add_grad_fn(Operation&& op) { modules.add_grad_fn(std::move(op)); }
@@ -510,6 +708,7 @@ struct Autograd {
     void set_lazy_enabled(bool e) { modules.set_lazy_enabled(e); }
     bool is_lazy_enabled() const { return modules.is_lazy_enabled(); }
     void set_op_hint(AnyOpHint h) { modules.set_op_hint(std::move(h)); }
+    void set_expr_hint(AnyExprHint h) { modules.set_expr_hint(std::move(h)); }
     template <class D>
     void exec_now(D& dev, size_t b, size_t e) {
         modules.exec_now(dev, b, e);
@@ -532,6 +731,14 @@ struct Autograd {
     template <class D>
     void unary_fusing(D& dev, const GraphTranslator* gt) {
         modules.unary_fusing(dev, gt);
+    }
+    // buffers the gradient functions on the tape will read must stay computed
+    template <class D>
+    void elementwise_fusing(D& dev, const GraphTranslator* gt, const std::vector<UniqueId>& keep) {
+        std::vector<UniqueId> all = keep;
+        for (const Operation& g : state.tape)
+            for (const Id& id : g.arg_ids) all.push_back(id.id);
+        modules.elementwise_fusing(dev, gt, all);
     }
 
     // autograd.rs:245-256

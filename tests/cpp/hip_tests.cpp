@@ -77,6 +77,58 @@ TEST_CASE(hip_fused_chain_is_one_kernel) {
     CHECK_VEC_EQ(o5.replace().read(), unfused);
 }
 
+// BASELINE configs[4] through the whole stack, scaled to 64 buffers: per buffer two
+// two-operand ops and a unary chain are recorded (256 operations); element-wise fusing
+// turns each buffer's four operations into one three-operand kernel, and the graph
+// builder merges the 64 independent launches into ONE kernel node.
+TEST_CASE(hip_config5_fuses_and_batches_to_one_node) {
+    using D = HIP<Graph<Lazy<Base>>>;
+    const size_t nbuf = 64, n = 4096;
+    auto fill = [](size_t seed, size_t n) {
+        std::vector<float> v(n);
+        uint64_t s = 0x9E3779B97F4A7C15ull * (seed + 1);
+        for (auto& x : v) {
+            s ^= s << 13; s ^= s >> 7; s ^= s << 17;
+            x = float(s >> 40) * (1.0f / 16777216.0f);
+        }
+        return v;
+    };
+    D dev;
+    std::vector<Buffer<float, D>> a, b, c, y;
+    std::vector<Buffer<float, D>> keep;
+    for (size_t i = 0; i < nbuf; i++) {
+        a.push_back(dev.buffer<float>(fill(3 * i, n)));
+        b.push_back(dev.buffer<float>(fill(3 * i + 1, n)));
+        c.push_back(dev.buffer<float>(fill(3 * i + 2, n)));
+    }
+    for (size_t i = 0; i < nbuf; i++) {
+        auto t = dev.apply_fn2(a[i], b[i], [](auto p, auto q) { return p.mul(q); });
+        auto u = dev.apply_fn2(t, c[i], [](auto p, auto q) { return p.add(q); });
+        auto v = dev.apply_fn(u, [](auto x) { return x.abs().sqrt(); });
+        y.push_back(dev.apply_fn(v, [](auto x) { return x.mul(0.3f); }));
+        keep.push_back(std::move(t));
+        keep.push_back(std::move(u));
+        keep.push_back(std::move(v));
+    }
+    CHECK_EQ(dev.ops_count(), 4 * nbuf);
+    dev.optimize_mem_graph();
+    dev.elementwise_fusing();
+    for (int r = 0; r < 3; r++) dev.run();
+    CHECK_EQ(dev.graph_builds(), uint64_t(1));
+    CHECK_EQ(dev.graph_kernel_nodes(), size_t(1));
+    for (size_t i : {size_t(0), size_t(17), nbuf - 1}) {
+        auto av = a[i].read(), bv = b[i].read(), cv = c[i].read();
+        std::vector<float> want(n);
+        for (size_t k = 0; k < n; k++) {
+            float t = av[k] * bv[k];
+            float u = t + cv[k];
+            float s = std::sqrt(std::fabs(u));
+            want[k] = s * 0.3f;
+        }
+        CHECK_VEC_EQ(y[i].replace().read(), want);
+    }
+}
+
 TEST_CASE(hip_backend_errors_surface) {
     bool threw = false;
     try {

@@ -535,6 +535,177 @@ void autograd_tanh_config(double tol) {
     CHECK_ROUGHLY(x.grad(device).read(), want_g, tol);
 }
 
+// ---- element-wise fusion of any arity (beyond the reference's unary-only fusing) ----
+
+// BASELINE configs[4] per buffer: t = a*b; u = t+c; y = sqrt(abs(u))*0.3 -> one three-operand kernel
+template <template <class> class DEV>
+void elementwise_fuse_binary_then_unary() {
+    DEV<Graph<Lazy<Base>>> dev;
+    const std::vector<float> av = {0.5f, 0.25f, 0.75f, 1.f, 0.1f}, bv = {2.f, 4.f, 0.5f, 3.f, 0.7f}, cv = {-3.f, 0.f, 0.125f, 1.f, 0.3f};
+    auto a = dev.template buffer<float>(av);
+    auto b = dev.template buffer<float>(bv);
+    auto c = dev.template buffer<float>(cv);
+    auto t = dev.apply_fn2(a, b, [](auto x, auto y) { return x.mul(y); });
+    auto u = dev.apply_fn2(t, c, [](auto x, auto y) { return x.add(y); });
+    auto v = dev.apply_fn(u, [](auto x) { return x.abs().sqrt(); });
+    auto y = dev.apply_fn(v, [](auto x) { return x.mul(0.3f); });
+    dev.optimize_mem_graph();
+    dev.elementwise_fusing();
+    const auto& ops = dev.modules.modules.graph;
+    CHECK_EQ(ops.size(), size_t(4));
+    CHECK(ops[0].arg_ids.empty() && ops[1].arg_ids.empty() && ops[2].arg_ids.empty());  // inlined
+    CHECK(ops[3].hint_kind == OpHintKind::UnaryFused);
+    CHECK_EQ(ops[3].fused_source, std::string("(sqrt(abs(((a * b) + c))) * 0.3)"));
+    CHECK_EQ(ops[3].arg_ids.size(), size_t(4));  // out + three operand buffers
+    dev.run();
+    std::vector<float> want;
+    for (size_t i = 0; i < av.size(); i++) {
+        float tt = av[i] * bv[i];
+        float uu = tt + cv[i];
+        float s = std::sqrt(std::fabs(uu));
+        want.push_back(s * 0.3f);
+    }
+    CHECK_VEC_EQ(y.replace().read(), want);  // one rounding per node: identical to the unfused result
+    dev.run();
+    CHECK_VEC_EQ(y.replace().read(), want);
+}
+
+// what must NOT be inlined: two readers, checkpoints, user-filled outputs, more than four
+// operand buffers, operands overwritten in between, buffers a gradient function needs
+template <template <class> class DEV>
+void elementwise_fuse_respects_limits() {
+    using D = DEV<Graph<Lazy<Base>>>;
+    auto count_live = [](const D& dev) {
+        size_t n = 0;
+        for (const auto& op : dev.modules.modules.graph) n += !op.arg_ids.empty();
+        return n;
+    };
+    {   // two readers of t: t stays, and both readers stay
+        D dev;
+        auto a = dev.template buffer<float>({1.f, 2.f, 3.f});
+        auto t = dev.apply_fn(a, [](auto x) { return x.mul(2.f); });
+        auto u = dev.apply_fn(t, [](auto x) { return x.add(1.f); });
+        auto w = dev.apply_fn(t, [](auto x) { return x.sub(1.f); });
+        dev.elementwise_fusing();
+        CHECK_EQ(count_live(dev), size_t(3));
+        dev.run();
+        CHECK_VEC_EQ(u.replace().read(), (std::vector<float>{3.f, 5.f, 7.f}));
+        CHECK_VEC_EQ(w.replace().read(), (std::vector<float>{1.f, 3.f, 5.f}));
+        CHECK_VEC_EQ(t.replace().read(), (std::vector<float>{2.f, 4.f, 6.f}));
+    }
+    {   // a checkpoint is kept (src/buffer.rs:131-137)
+        D dev;
+        auto a = dev.template buffer<float>({1.f, 2.f, 3.f});
+        auto t = dev.apply_fn(a, [](auto x) { return x.mul(2.f); }).checkpoint();
+        auto u = dev.apply_fn(t, [](auto x) { return x.add(1.f); });
+        auto w = dev.apply_fn(u, [](auto x) { return x.neg(); });
+        dev.elementwise_fusing();
+        CHECK_EQ(count_live(dev), size_t(2));  // t alone, u+w fused
+        dev.run();
+        CHECK_VEC_EQ(t.replace().read(), (std::vector<float>{2.f, 4.f, 6.f}));
+        CHECK_VEC_EQ(w.replace().read(), (std::vector<float>{-3.f, -5.f, -7.f}));
+    }
+    {   // five distinct operand buffers do not fit one kernel: the chain is cut
+        D dev;
+        std::vector<Buffer<float, D>> in;
+        for (int i = 0; i < 6; i++) in.push_back(dev.template buffer<float>({float(i + 1), 1.f, 2.f}));
+        auto add = [](auto x, auto y) { return x.add(y); };
+        auto s1 = dev.apply_fn2(in[0], in[1], add);
+        auto s2 = dev.apply_fn2(s1, in[2], add);
+        auto s3 = dev.apply_fn2(s2, in[3], add);
+        auto s4 = dev.apply_fn2(s3, in[4], add);
+        auto s5 = dev.apply_fn2(s4, in[5], add);
+        dev.elementwise_fusing();
+        for (const auto& op : dev.modules.modules.graph) CHECK(op.arg_ids.size() <= 5);  // out + at most 4 operands
+        CHECK(count_live(dev) < 5 && count_live(dev) >= 2);
+        dev.run();
+        CHECK_VEC_EQ(s5.replace().read(), (std::vector<float>{21.f, 6.f, 12.f}));
+    }
+    {   // an operand is overwritten between producer and reader: no inlining across the write
+        D dev;
+        auto a = dev.template buffer<float>({1.f, 2.f, 3.f});
+        auto g = dev.template buffer<float>({10.f, 10.f, 10.f});
+        auto o = dev.template buffer<float>({1.f, 1.f, 1.f});
+        auto t = dev.apply_fn(g, [](auto x) { return x.mul(2.f); });                  // reads g = 10
+        dev.add_unary_grad(a, g, o, [](auto x) { return x.identity(); });           // g += a  (unhinted: writes g)
+        auto u = dev.apply_fn(t, [](auto x) { return x.add(1.f); });
+        dev.elementwise_fusing();
+        dev.run();
+        CHECK_VEC_EQ(u.replace().read(), (std::vector<float>{21.f, 21.f, 21.f}));   // from g before the update
+        CHECK_VEC_EQ(g.read(), (std::vector<float>{11.f, 12.f, 13.f}));
+    }
+}
+
+// a buffer a gradient function needs is computed even though it has a single reader
+template <template <class> class DEV>
+void elementwise_fuse_keeps_tape_buffers(double tol) {
+    DEV<Autograd<Graph<Lazy<Base, double>, double>>> dev;
+    auto buf = dev.template buffer<double>({0., 1., 2., 3.}).require_grad();
+    auto buf1 = dev.apply_fn(buf, [](auto x) { return x.add(1.); });
+    auto out = dev.unary_ew(buf1, [](auto x) { return x.sin(); }, [](auto x) { return x.cos(); });
+    dev.elementwise_fusing();
+    dev.run();
+    CHECK_ROUGHLY(out.replace().read(), SIN_1_4, tol);
+    CHECK_VEC_EQ(buf1.replace().read(), (std::vector<double>{1., 2., 3., 4.}));  // not inlined away
+    out.backward();
+    CHECK_ROUGHLY(buf1.grad(dev).read(), COS_1_4, tol);
+}
+
+// random element-wise programs: fused and unfused runs agree bit for bit
+template <template <class> class DEV>
+void elementwise_fuse_random_programs() {
+    using D = DEV<Graph<Lazy<Base>>>;
+    uint64_t rng = 0x9E3779B97F4A7C15ull;
+    auto next = [&rng](uint64_t m) {
+        rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
+        return rng % m;
+    };
+    for (int trial = 0; trial < 12; trial++) {
+        std::vector<std::vector<int>> prog;  // {kind, fn, in0, in1}
+        const int n_leaf = 3, n_ops = 10;
+        for (int i = 0; i < n_ops; i++) {
+            int avail = n_leaf + i;
+            prog.push_back({int(next(2)), int(next(3)), int(next(avail)), int(next(avail))});
+        }
+        std::vector<std::vector<float>> results[2];
+        for (int fused = 0; fused < 2; fused++) {
+            D dev;
+            std::vector<Buffer<float, D>> vals;
+            for (int l = 0; l < n_leaf; l++) {
+                std::vector<float> v(37);
+                for (size_t k = 0; k < v.size(); k++) v[k] = 0.1f * float((l + 1) * (k % 11)) - 1.5f;
+                vals.push_back(dev.template buffer<float>(v));
+            }
+            for (const auto& op : prog) {
+                if (op[0] == 0) {
+                    if (op[1] == 0) vals.push_back(dev.apply_fn(vals[op[2]], [](auto x) { return x.mul(1.5f).add(0.25f); }));
+                    else if (op[1] == 1) vals.push_back(dev.apply_fn(vals[op[2]], [](auto x) { return x.abs().sqrt(); }));
+                    else vals.push_back(dev.apply_fn(vals[op[2]], [](auto x) { return x.neg().max(-2.f); }));
+                } else {
+                    int l = op[2], r = op[3];
+                    if (l == r) r = (r + 1) % (int)vals.size();  // operands of one operation are distinct buffers
+                    if (op[1] == 0) vals.push_back(dev.apply_fn2(vals[l], vals[r], [](auto x, auto y) { return x.add(y); }));
+                    else if (op[1] == 1) vals.push_back(dev.apply_fn2(vals[l], vals[r], [](auto x, auto y) { return x.mul(y).sub(0.5f); }));
+                    else vals.push_back(dev.apply_fn2(vals[l], vals[r], [](auto x, auto y) { return x.min(y); }));
+                }
+            }
+            if (fused) dev.elementwise_fusing();
+            else dev.modules.modules.alloc_later(dev);
+            dev.run();
+            // only buffers nobody else reads are guaranteed to be computed after fusing: compare the sinks
+            std::vector<int> reads(vals.size(), 0);
+            for (size_t i = 0; i < prog.size(); i++) {
+                reads[prog[i][2]]++;
+                if (prog[i][0] == 1) reads[prog[i][3] == prog[i][2] ? (prog[i][3] + 1) % int(n_leaf + i) : prog[i][3]]++;
+            }
+            for (size_t i = n_leaf; i < vals.size(); i++)
+                if (reads[i] != 1) results[fused].push_back(vals[i].replace().read());
+        }
+        CHECK_EQ(results[0].size(), results[1].size());
+        for (size_t i = 0; i < results[0].size() && i < results[1].size(); i++) CHECK_VEC_EQ(results[1][i], results[0][i]);
+    }
+}
+
 }  // namespace module_tests
 
 // Registers every generic case for one device template.
@@ -569,4 +740,8 @@ void autograd_tanh_config(double tol) {
     TEST_CASE(autograd_requires_grad_chaining) { module_tests::autograd_requires_grad_chaining<DEV>(); } \
     TEST_CASE(autograd_grad_fn_with_lazy_source) { module_tests::autograd_grad_fn_with_lazy_source<DEV>(); } \
     TEST_CASE(autograd_grad_fn_out_of_scope) { module_tests::autograd_grad_fn_out_of_scope<DEV>(); } \
-    TEST_CASE(autograd_tanh_config) { module_tests::autograd_tanh_config<DEV>(1e-6); }
+    TEST_CASE(autograd_tanh_config) { module_tests::autograd_tanh_config<DEV>(1e-6); }                \
+    TEST_CASE(elementwise_fuse_binary_then_unary) { module_tests::elementwise_fuse_binary_then_unary<DEV>(); } \
+    TEST_CASE(elementwise_fuse_respects_limits) { module_tests::elementwise_fuse_respects_limits<DEV>(); } \
+    TEST_CASE(elementwise_fuse_keeps_tape_buffers) { module_tests::elementwise_fuse_keeps_tape_buffers<DEV>(TOL); } \
+    TEST_CASE(elementwise_fuse_random_programs) { module_tests::elementwise_fuse_random_programs<DEV>(); }

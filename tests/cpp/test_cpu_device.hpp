@@ -81,14 +81,17 @@ class TestCPU : public Device<TestCPU<Mods>, Mods> {
             }
         };
     }
-    template <class T, class F>
-    Buffer<T, Self> apply_fn2(const Buffer<T, Self>& lhs, const Buffer<T, Self>& rhs, F f) {
-        Buffer<T, Self> out = this->template retrieve<T>(lhs.len(), lhs, rhs);
-        this->add_op(std::tie(lhs, rhs, out),
-                     [f](const Buffer<T, Self>& l, const Buffer<T, Self>& r, Buffer<T, Self>& o, Self& dev) {
-                         dev.apply_fn2_impl(l, r, o, f);
-                     });
-        return out;
+    template <class T>
+    std::function<void(Buffer<T, Self>&, const std::vector<Buffer<T, Self>>&, Self&)> elementwise_fuse_op(
+        std::shared_ptr<FusedExpr<T>> expr) {
+        return [expr](Buffer<T, Self>& out, const std::vector<Buffer<T, Self>>& ins, Self&) {
+            T* os = reinterpret_cast<T*>(out.ptr());
+            for (size_t i = 0; i < out.len(); i++) {
+                T vals[4];
+                for (size_t k = 0; k < ins.size(); k++) vals[k] = reinterpret_cast<const T*>(ins[k].ptr())[i];
+                os[i] = expr->eval(vals);
+            }
+        };
     }
 
     void lazy_setup() {}
