@@ -18,10 +18,13 @@ namespace custos_hip {
 enum class Kind : int32_t { Apply = 0, UnaryGrad = 1 };
 
 struct Tuning {
-    // Defaults from a sweep of the fused f32 chain at 2^28 elements on MI355X:
-    // 512 x 2 with streaming (non-temporal) loads and stores was the fastest
-    // of {256,512,1024} x {1,2,4,8} x {plain, nt}; persistent grids were slower.
-    int block_threads = 512;
+    // Defaults from interleaved, repeated timing of the fused f32 chain at 2^28
+    // elements on MI355X: workgroups of 64 or 128 threads with 2 vectors per
+    // thread sustain 3-5 % more than 256..1024-thread workgroups or other unroll
+    // factors (many small workgroups keep the memory channels evenly loaded);
+    // streaming (non-temporal) loads and stores add another 1-2 %; persistent
+    // grids were 5-20 % slower.
+    int block_threads = 128;
     int unroll = 2;
     int blocks_per_cu = 0;  // <= 0: one tile per workgroup
     int nontemporal = 3;    // bit 0 loads, bit 1 stores

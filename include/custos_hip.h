@@ -106,7 +106,7 @@ typedef struct custos_hip_device_info {
 /* Launch shape knobs of the generated kernels.  Zero fields keep the default.
  * They are part of the kernel cache key. */
 typedef struct custos_hip_tuning {
-    int32_t block_threads;   /* threads per workgroup (multiple of 64), default 512 */
+    int32_t block_threads;   /* threads per workgroup (multiple of 64), default 128 */
     int32_t unroll;          /* 16-byte vectors per thread per tile, default 2 */
     int32_t blocks_per_cu;   /* > 0: persistent grid of CUs*blocks_per_cu workgroups that
                                 stride over the tiles; <= 0 (default): one tile per workgroup */

@@ -133,7 +133,7 @@ def test_tuning_is_part_of_the_key_and_source():
     assert "#define CUSTOS_BLOCK 256" in src and "#define CUSTOS_UNROLL 4" in src
     assert "__builtin_nontemporal" not in src
     src2, h2 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"])
-    assert "#define CUSTOS_BLOCK 512" in src2 and "__builtin_nontemporal_load" in src2
+    assert "#define CUSTOS_BLOCK 128" in src2 and "__builtin_nontemporal_load" in src2
     assert h1 != h2
 
 
