@@ -103,6 +103,11 @@ PROTOTYPES = {
     "custos_hip_kernel_hash": (C.c_uint64, [_P]),
     "custos_hip_kernel_arity": (C.c_int32, [_P]),
     "custos_hip_cache_stats": (C.c_int32, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "custos_hip_cache_disk_hits": (C.c_int32, [_P, C.POINTER(C.c_uint64)]),
+    "custos_hip_source_compile": (C.c_int32, [_P, C.c_char_p, C.c_char_p, _PP]),
+    "custos_hip_source_launch": (C.c_int32, [_P, _P, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_uint32,
+                                             C.POINTER(C.c_void_p), C.POINTER(C.c_size_t), C.c_int32]),
+    "custos_hip_source_launch1d": (C.c_int32, [_P, _P, C.c_size_t, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t), C.c_int32]),
     "custos_hip_expr_emit": (C.c_int32, [C.c_int32, C.c_int32, C.c_char_p, _STRS, C.c_int32, C.POINTER(Tuning),
                                          C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint64)]),
     "custos_hip_expr_build_code_object": (C.c_int32, [C.c_int32, C.c_int32, C.c_char_p, _STRS, C.c_int32,

@@ -15,7 +15,7 @@
 
 namespace custos_hip {
 
-enum class Kind : int32_t { Apply = 0, UnaryGrad = 1 };
+enum class Kind : int32_t { Apply = 0, UnaryGrad = 1, Source = 2 /* caller-written kernel source */ };
 
 struct Tuning {
     // Defaults from interleaved, repeated timing of the fused f32 chain at 2^28

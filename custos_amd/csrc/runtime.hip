@@ -4,8 +4,12 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <sys/stat.h>
+#include <unistd.h>
+
 #include <algorithm>
 #include <cstdio>
+#include <fstream>
 #include <cstdlib>
 #include <cstring>
 #include <memory>
@@ -41,13 +45,17 @@ struct Access {
     bool write;
 };
 struct RecNode {
-    enum Type { Kernel, Fill, Copy } type = Kernel;
+    enum Type { Kernel, Fill, Copy, Source } type = Kernel;
     custos_hip_kernel* k = nullptr;
     std::vector<uint64_t> ptrs;  // kernel: operand addresses in parameter order; fill: {ptr}; copy: {dst, src}
     unsigned long long n = 0, head = 0, n_vec = 0, bytes = 0;
     unsigned int grid = 1;
     std::vector<Access> acc;
     int level = 0;
+    // Source: launch shape and a copy of the argument values.  What such a kernel
+    // reads and writes is unknown, so it orders itself against everything.
+    unsigned int grid3[3] = {1, 1, 1}, block3[3] = {1, 1, 1}, shared_mem = 0;
+    std::vector<std::vector<unsigned char>> arg_values;
 };
 
 struct custos_hip_device {
@@ -61,7 +69,7 @@ struct custos_hip_device {
     bool capturing = false;          // recording: launches, clears and copies go to `recorded`
     bool batching = true;            // merge equal independent launches of a level into one grid
     std::vector<RecNode> recorded;
-    uint64_t compiles = 0, hits = 0;
+    uint64_t compiles = 0, hits = 0, disk_hits = 0;
     std::string last_error;
     std::unordered_map<uint64_t, std::vector<std::unique_ptr<custos_hip_kernel>>> cache;
     std::vector<custos_hip_graph*> graphs;
@@ -169,6 +177,75 @@ int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec,
     hiprtcGetCode(prog, code->data());
     hiprtcDestroyProgram(&prog);
     return CUSTOS_HIP_OK;
+}
+
+// ---- code objects on disk ----
+//
+// With CUSTOS_HIP_KERNEL_CACHE_DIR set, every compiled code object is stored as
+// <dir>/<key>-<arch>-<hiprtc version>.co together with the source it was built
+// from; a later process loads it instead of compiling when the stored source is
+// identical (the 64-bit key alone is not trusted).
+
+std::string cache_file(const KernelSpec& spec, const std::string& arch) {
+    const char* dir = std::getenv("CUSTOS_HIP_KERNEL_CACHE_DIR");
+    if (!dir || !*dir) return "";
+    int major = 0, minor = 0;
+    (void)hiprtcVersion(&major, &minor);
+    std::string a = arch;
+    for (char& c : a)
+        if (c == ':' || c == '/' || c == '+') c = '_';
+    char key[17];
+    std::snprintf(key, sizeof key, "%016llx", static_cast<unsigned long long>(spec.hash));
+    return std::string(dir) + "/" + key + "-" + a + "-" + std::to_string(major) + "." + std::to_string(minor) + ".co";
+}
+
+// the text hiprtc compiles: generated kernels start with a comment line that
+// spells the expression as the caller wrote it; it is not part of the identity
+std::string source_identity(const KernelSpec& spec) {
+    if (spec.kind == Kind::Source) return spec.name + "\n" + spec.source;
+    return spec.source.substr(spec.source.find('\n') + 1);
+}
+
+bool load_cached_code(const KernelSpec& spec, const std::string& arch, std::vector<char>* code) {
+    const std::string path = cache_file(spec, arch);
+    if (path.empty()) return false;
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return false;
+    char magic[8] = {0};
+    uint64_t src_len = 0, code_len = 0;
+    f.read(magic, 8);
+    f.read(reinterpret_cast<char*>(&src_len), 8);
+    if (!f || std::memcmp(magic, "CUSTOSC1", 8) != 0 || src_len > (1u << 26)) return false;
+    std::string src(src_len, '\0');
+    f.read(&src[0], static_cast<std::streamsize>(src_len));
+    f.read(reinterpret_cast<char*>(&code_len), 8);
+    if (!f || src != source_identity(spec) || code_len == 0 || code_len > (1u << 28)) return false;
+    code->resize(code_len);
+    f.read(code->data(), static_cast<std::streamsize>(code_len));
+    return static_cast<bool>(f);
+}
+
+void store_cached_code(const KernelSpec& spec, const std::string& arch, const std::vector<char>& code) {
+    const std::string path = cache_file(spec, arch);
+    if (path.empty()) return;
+    (void)mkdir(std::getenv("CUSTOS_HIP_KERNEL_CACHE_DIR"), 0777);
+    const std::string tmp = path + ".tmp" + std::to_string(static_cast<long>(getpid()));
+    {
+        std::ofstream f(tmp, std::ios::binary | std::ios::trunc);
+        if (!f) return;
+        const std::string src = source_identity(spec);
+        const uint64_t src_len = src.size(), code_len = code.size();
+        f.write("CUSTOSC1", 8);
+        f.write(reinterpret_cast<const char*>(&src_len), 8);
+        f.write(src.data(), static_cast<std::streamsize>(src_len));
+        f.write(reinterpret_cast<const char*>(&code_len), 8);
+        f.write(code.data(), static_cast<std::streamsize>(code_len));
+        if (!f) {
+            std::remove(tmp.c_str());
+            return;
+        }
+    }
+    if (std::rename(tmp.c_str(), path.c_str()) != 0) std::remove(tmp.c_str());
 }
 
 bool markers_from_c(const char* const* markers, int32_t n, std::vector<std::string>* out) {
@@ -321,8 +398,15 @@ void assign_levels(std::vector<RecNode>& nodes) {
     };
     std::vector<Seen> seen;
     std::unordered_map<uint64_t, std::vector<uint32_t>> buckets;
+    int highest = -1;  // highest level so far
+    int fence = -1;    // level of the last node with unknown memory use
     for (RecNode& node : nodes) {
-        int level = 0;
+        int level = fence + 1;
+        if (node.type == RecNode::Source) {
+            // unknown reads and writes: after everything before, before everything after
+            node.level = fence = highest = highest + 1;
+            continue;
+        }
         for (const Access& a : node.acc) {
             if (a.end <= a.begin) continue;
             for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) {
@@ -337,6 +421,7 @@ void assign_levels(std::vector<RecNode>& nodes) {
             }
         }
         node.level = level;
+        highest = std::max(highest, level);
         for (const Access& a : node.acc) {
             if (a.end <= a.begin) continue;
             const uint32_t idx = static_cast<uint32_t>(seen.size());
@@ -428,7 +513,13 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
             std::vector<void*> args;
             uint64_t ptrs[8];
             unsigned long long a0, a1, a2, a3;
-            if (first.type == RecNode::Fill) {
+            if (first.type == RecNode::Source) {
+                for (const auto& v : first.arg_values) args.push_back(const_cast<unsigned char*>(v.data()));
+                kp.func = reinterpret_cast<void*>(first.k->fn);
+                kp.gridDim = dim3(first.grid3[0], first.grid3[1], first.grid3[2]);
+                kp.blockDim = dim3(first.block3[0], first.block3[1], first.block3[2]);
+                kp.sharedMemBytes = first.shared_mem;
+            } else if (first.type == RecNode::Fill) {
                 ptrs[0] = first.ptrs[0];
                 a0 = first.bytes, a1 = first.head, a2 = first.n_vec;
                 args = {&ptrs[0], &a0, &a1, &a2};
@@ -469,6 +560,33 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
         prev = std::move(made);
     }
     HIP_TRY(dev, hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
+    return CUSTOS_HIP_OK;
+}
+
+// Code object from the disk cache or from hiprtc, loaded as a module; entry point looked up.
+int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k) {
+    std::vector<char> code;
+    bool from_disk = load_cached_code(k->spec, dev->arch, &code);
+    if (from_disk && hipModuleLoadData(&k->module, code.data()) != hipSuccess) {
+        (void)hipGetLastError();  // a stale or damaged file: compile instead
+        k->module = nullptr;
+        from_disk = false;
+    }
+    if (!from_disk) {
+        int32_t rc = compile_to_code_object(dev, k->spec, dev->arch, &code);
+        if (rc != CUSTOS_HIP_OK) return rc;
+        HIP_TRY(dev, hipModuleLoadData(&k->module, code.data()));
+        store_cached_code(k->spec, dev->arch, code);
+        dev->compiles++;
+    } else {
+        dev->disk_hits++;
+    }
+    hipError_t e = hipModuleGetFunction(&k->fn, k->module, k->spec.name.c_str());
+    if (e != hipSuccess) {
+        (void)hipModuleUnload(k->module);
+        k->module = nullptr;
+        return hip_fail(dev, e, "hipModuleGetFunction");
+    }
     return CUSTOS_HIP_OK;
 }
 
@@ -697,24 +815,93 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
             return CUSTOS_HIP_OK;
         }
     }
-    std::vector<char> code;
-    rc = compile_to_code_object(dev, k->spec, dev->arch, &code);
+    rc = build_module(dev, k.get());
     if (rc != CUSTOS_HIP_OK) return rc;
-    HIP_TRY(dev, hipModuleLoadData(&k->module, code.data()));
-    hipError_t e = hipModuleGetFunction(&k->fn, k->module, k->spec.name.c_str());
-    if (e != hipSuccess) {
-        (void)hipModuleUnload(k->module);
-        return hip_fail(dev, e, "hipModuleGetFunction");
-    }
     // the second entry point of the module: many equal launches in one grid
     if (hipModuleGetFunction(&k->fn_batched, k->module, (k->spec.name + "_batched").c_str()) != hipSuccess) {
         (void)hipGetLastError();
         k->fn_batched = nullptr;
     }
-    dev->compiles++;
     *kernel = k.get();
     bucket.push_back(std::move(k));
     return CUSTOS_HIP_OK;
+}
+
+// ---- caller-written kernels (src/devices/cuda/kernel_cache.rs:39-61, kernel_launch.rs:81-163) ----
+
+int32_t custos_hip_source_compile(custos_hip_device* dev, const char* src, const char* fn_name,
+                                  custos_hip_kernel** kernel) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "kernel out pointer is null");
+    *kernel = nullptr;
+    if (!src || !fn_name || !*fn_name) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "source or function name is null");
+    std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
+    k->spec.kind = Kind::Source;
+    k->spec.name = fn_name;
+    k->spec.source = src;
+    k->spec.hash = fnv1a64(fn_name, std::strlen(fn_name), fnv1a64(src, std::strlen(src), fnv1a64("custos-source-v1", 16)));
+    auto& bucket = dev->cache[k->spec.hash];
+    for (auto& cached : bucket) {
+        if (cached->spec.kind == Kind::Source && cached->spec.name == k->spec.name && cached->spec.source == k->spec.source) {
+            dev->hits++;
+            *kernel = cached.get();
+            return CUSTOS_HIP_OK;
+        }
+    }
+    int32_t rc = build_module(dev, k.get());
+    if (rc != CUSTOS_HIP_OK) return rc;
+    *kernel = k.get();
+    bucket.push_back(std::move(k));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_source_launch(custos_hip_device* dev, custos_hip_kernel* kernel, const uint32_t* grid,
+                                 const uint32_t* block, uint32_t shared_mem_bytes, void* const* params,
+                                 const size_t* param_sizes, int32_t n_params) {
+    REQUIRE_DEV(dev);
+    if (!kernel || !grid || !block || n_params < 0 || (n_params > 0 && (!params || !param_sizes)))
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    if (kernel->spec.kind != Kind::Source)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled from caller-written source");
+    for (int i = 0; i < 3; i++)
+        if (grid[i] == 0 || block[i] == 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "grid and block dimensions must be positive");
+    if (static_cast<uint64_t>(block[0]) * block[1] * block[2] > 1024)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "more than 1024 threads per workgroup");
+    if (dev->capturing) {
+        RecNode node;
+        node.type = RecNode::Source;
+        node.k = kernel;
+        for (int i = 0; i < 3; i++) node.grid3[i] = grid[i], node.block3[i] = block[i];
+        node.shared_mem = shared_mem_bytes;
+        for (int i = 0; i < n_params; i++) {
+            const unsigned char* p = static_cast<const unsigned char*>(params[i]);
+            node.arg_values.emplace_back(p, p + param_sizes[i]);
+        }
+        dev->recorded.push_back(std::move(node));
+        return CUSTOS_HIP_OK;
+    }
+    std::vector<void*> args(params, params + n_params);
+    HIP_TRY(dev, hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                       shared_mem_bytes, dev->stream, args.data(), nullptr));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_source_launch1d(custos_hip_device* dev, custos_hip_kernel* kernel, size_t len,
+                                   void* const* params, const size_t* param_sizes, int32_t n_params) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel");
+    if (kernel->spec.kind != Kind::Source)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled from caller-written source");
+    if (len == 0) return CUSTOS_HIP_OK;
+    // block size from the occupancy calculator, grid = ceil(len / block) (kernel_launch.rs:141-151)
+    int min_grid = 0, block_size = 0;
+    HIP_TRY(dev, hipModuleOccupancyMaxPotentialBlockSize(&min_grid, &block_size, kernel->fn, 0, 0));
+    if (block_size <= 0) block_size = 256;
+    const uint64_t blocks = (len + static_cast<size_t>(block_size) - 1) / static_cast<size_t>(block_size);
+    if (blocks > 0x7fffffffull) return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "more workgroups than a one-dimensional grid holds");
+    const uint32_t grid[3] = {static_cast<uint32_t>(blocks), 1, 1};
+    const uint32_t block[3] = {static_cast<uint32_t>(block_size), 1, 1};
+    return custos_hip_source_launch(dev, kernel, grid, block, 0, params, param_sizes, n_params);
 }
 
 const char* custos_hip_kernel_source(const custos_hip_kernel* kernel) {
@@ -735,6 +922,12 @@ int32_t custos_hip_cache_stats(custos_hip_device* dev, uint64_t* compiles, uint6
     REQUIRE_DEV(dev);
     if (compiles) *compiles = dev->compiles;
     if (hits) *hits = dev->hits;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_cache_disk_hits(custos_hip_device* dev, uint64_t* disk_hits) {
+    REQUIRE_DEV(dev);
+    if (disk_hits) *disk_hits = dev->disk_hits;
     return CUSTOS_HIP_OK;
 }
 

@@ -236,6 +236,46 @@ class HIP:
         kernel = self.compile(capi.KIND_UNARY_GRAD, lhs.dtype, src, ("x",))
         self._check(self.lib.custos_hip_add_unary_grad(self.handle, kernel, lhs.ptr, lhs_grad.ptr, out_grad.ptr, lhs.len))
 
+    # -- caller-written kernels (`launch_kernel` / `launch_kernel1d`, src/devices/cuda/cuda_device.rs:85-112) --
+    def _source_args(self, args):
+        """Buffers pass their device address, ctypes values pass as they are, ints become c_int32,
+        floats c_float (`AsCudaCvoidPtr`, src/devices/cuda/kernel_launch.rs:29-77)."""
+        vals = []
+        for a in args:
+            if isinstance(a, Buffer):
+                vals.append(C.c_uint64(a.ptr))
+            elif isinstance(a, C._SimpleCData):
+                vals.append(a)
+            elif isinstance(a, (bool, int, np.integer)):
+                vals.append(C.c_int32(int(a)))
+            else:
+                vals.append(C.c_float(float(a)))
+        ptrs = (C.c_void_p * len(vals))(*[C.cast(C.pointer(v), C.c_void_p) for v in vals])
+        sizes = (C.c_size_t * len(vals))(*[C.sizeof(v) for v in vals])
+        return vals, ptrs, sizes
+
+    def compile_source(self, src: str, fn_name: str):
+        k = C.c_void_p()
+        self._check(self.lib.custos_hip_source_compile(self.handle, src.encode(), fn_name.encode(), C.byref(k)))
+        return k
+
+    def launch_kernel(self, src: str, fn_name: str, grid, block, shared_mem_bytes: int, args) -> None:
+        k = self.compile_source(src, fn_name)
+        vals, ptrs, sizes = self._source_args(args)
+        g = (C.c_uint32 * 3)(*grid)
+        b = (C.c_uint32 * 3)(*block)
+        self._check(self.lib.custos_hip_source_launch(self.handle, k, g, b, shared_mem_bytes, ptrs, sizes, len(vals)))
+
+    def launch_kernel1d(self, length: int, src: str, fn_name: str, args) -> None:
+        k = self.compile_source(src, fn_name)
+        vals, ptrs, sizes = self._source_args(args)
+        self._check(self.lib.custos_hip_source_launch1d(self.handle, k, length, ptrs, sizes, len(vals)))
+
+    def disk_cache_hits(self) -> int:
+        v = C.c_uint64(0)
+        self._check(self.lib.custos_hip_cache_disk_hits(self.handle, C.byref(v)))
+        return v.value
+
     # -- capture / replay --
     def capture_begin(self) -> None:
         self._check(self.lib.custos_hip_capture_begin(self.handle))

@@ -9,6 +9,7 @@
 #pragma once
 
 #include <cstdint>
+#include <cstring>
 #include <functional>
 #include <memory>
 #include <string>
@@ -155,6 +156,29 @@ class HIP : public Device<HIP<Mods>, Mods> {
         };
     }
 
+    // ---- caller-written kernels ----
+
+    // `device.launch_kernel(src, fn_name, grid, block, shared_mem, args)` and
+    // `device.launch_kernel1d(len, src, fn_name, args)` (src/devices/cuda/cuda_device.rs:85-112).
+    // Buffers pass their device address, numbers pass by value (`AsCudaCvoidPtr`,
+    // src/devices/cuda/kernel_launch.rs:29-77).
+    template <class... Args>
+    void launch_kernel(const std::string& src, const char* fn_name, const uint32_t (&grid)[3], const uint32_t (&block)[3],
+                       uint32_t shared_mem_bytes, const Args&... args) {
+        custos_hip_kernel* k = nullptr;
+        check(custos_hip_source_compile(dev_, src.c_str(), fn_name, &k));
+        KernelArgs<sizeof...(Args)> packed(args...);
+        check(custos_hip_source_launch(dev_, k, grid, block, shared_mem_bytes, packed.ptrs, packed.sizes,
+                                       static_cast<int32_t>(sizeof...(Args))));
+    }
+    template <class... Args>
+    void launch_kernel1d(size_t len, const std::string& src, const char* fn_name, const Args&... args) {
+        custos_hip_kernel* k = nullptr;
+        check(custos_hip_source_compile(dev_, src.c_str(), fn_name, &k));
+        KernelArgs<sizeof...(Args)> packed(args...);
+        check(custos_hip_source_launch1d(dev_, k, len, packed.ptrs, packed.sizes, static_cast<int32_t>(sizeof...(Args))));
+    }
+
     // ---- Lazy hooks ----
 
     // `LazySetup::lazy_setup`.  The reference starts stream capture here and
@@ -212,6 +236,32 @@ class HIP : public Device<HIP<Mods>, Mods> {
     }
 
    private:
+    // argument values laid out for the launch call: 8 bytes of storage each
+    template <size_t N>
+    struct KernelArgs {
+        uint64_t storage[N ? N : 1] = {};
+        void* ptrs[N ? N : 1] = {};
+        size_t sizes[N ? N : 1] = {};
+        template <class... A>
+        explicit KernelArgs(const A&... a) {
+            size_t i = 0;
+            (put(i++, a), ...);
+        }
+        template <class T>
+        void put(size_t i, const Buffer<T, Self>& b) {
+            storage[i] = b.ptr();
+            ptrs[i] = &storage[i];
+            sizes[i] = sizeof(uint64_t);
+        }
+        template <class V, class = std::enable_if_t<std::is_arithmetic_v<V>>>
+        void put(size_t i, const V& v) {
+            static_assert(sizeof(V) <= sizeof(uint64_t), "kernel argument too large");
+            std::memcpy(&storage[i], &v, sizeof(V));
+            ptrs[i] = &storage[i];
+            sizes[i] = sizeof(V);
+        }
+    };
+
     custos_hip_device* dev_ = nullptr;
     custos_hip_graph* graph_ = nullptr;
     uint64_t graph_version_ = 0;

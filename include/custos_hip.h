@@ -181,6 +181,33 @@ int32_t custos_hip_kernel_arity(const custos_hip_kernel *kernel);
 /* Number of hiprtc compilations / cache hits since the device was created. */
 int32_t custos_hip_cache_stats(custos_hip_device *dev, uint64_t *compiles, uint64_t *hits);
 
+/* Disk cache: with the environment variable CUSTOS_HIP_KERNEL_CACHE_DIR set, code
+ * objects are stored there (keyed by cache key, device architecture and hiprtc
+ * version, verified against the stored source) and loaded by later processes
+ * instead of compiling.  `*disk_hits` counts kernels loaded that way. */
+int32_t custos_hip_cache_disk_hits(custos_hip_device *dev, uint64_t *disk_hits);
+
+/* Caller-written kernels: `KernelCache::kernel` + `launch_kernel` / `launch_kernel1d`
+ * (src/devices/cuda/kernel_cache.rs:39-61, kernel_launch.rs:81-163,
+ * cuda_device.rs:85-112).  `src` is HIP source containing `extern "C" __global__
+ * void <fn_name>(...)`; it is compiled once per (source, name) and cached.
+ * `params[i]` points to the value of argument i (a device address is passed as a
+ * pointer to the uint64_t holding it, like `AsCudaCvoidPtr`), `param_sizes[i]` is
+ * its size in bytes.  While recording, the argument values are copied and the
+ * launch becomes a graph node ordered after all earlier and before all later
+ * work (its memory use is unknown). */
+int32_t custos_hip_source_compile(custos_hip_device *dev, const char *src, const char *fn_name,
+                                  custos_hip_kernel **kernel);
+int32_t custos_hip_source_launch(custos_hip_device *dev, custos_hip_kernel *kernel,
+                                 const uint32_t *grid, const uint32_t *block,
+                                 uint32_t shared_mem_bytes, void *const *params,
+                                 const size_t *param_sizes, int32_t n_params);
+/* One-dimensional launch over `len` work items: workgroup size from the occupancy
+ * calculator, grid = ceil(len / workgroup size). */
+int32_t custos_hip_source_launch1d(custos_hip_device *dev, custos_hip_kernel *kernel, size_t len,
+                                   void *const *params, const size_t *param_sizes,
+                                   int32_t n_params);
+
 /* Host-only helpers (no GPU needed): parse + emit the HIP source of a kernel
  * into `buf` (`*needed` = bytes including the terminator), and run the hiprtc
  * compilation for gfx950 without loading the result (`*code_size` = bytes). */

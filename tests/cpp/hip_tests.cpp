@@ -129,6 +129,62 @@ TEST_CASE(hip_config5_fuses_and_batches_to_one_node) {
     }
 }
 
+static std::string ew_src(const char* fn_name, char op) {
+    // src/devices/cuda/lazy.rs:81-93
+    return std::string("extern \"C\" __global__ void ") + fn_name +
+           "(int* lhs, int* rhs, int* out, int len) {\n"
+           "    int idx = blockIdx.x * blockDim.x + threadIdx.x;\n"
+           "    if (idx >= len) return;\n"
+           "    out[idx] = lhs[idx] " + op + " rhs[idx];\n}\n";
+}
+
+// src/devices/cuda/lazy.rs:198-240 (test_cuda_eager_without_lazy): caller-written kernels, launched directly
+TEST_CASE(hip_launch_kernel1d_eager) {
+    HIP<Base> device;
+    auto lhs = device.buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto rhs = device.buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto out = lhs.empty_like();
+    const int len = 6;
+    device.launch_kernel1d(6, ew_src("add", '+'), "add", lhs, rhs, out, len);
+    device.launch_kernel1d(6, ew_src("add", '+'), "add", out, lhs, rhs, len);
+    device.launch_kernel1d(6, ew_src("mul", '*'), "mul", out, rhs, lhs, len);
+    CHECK_VEC_EQ(out.read(), (std::vector<int32_t>{2, 4, 6, 8, 10, 12}));
+    CHECK_VEC_EQ(rhs.read(), (std::vector<int32_t>{3, 6, 9, 12, 15, 18}));
+    CHECK_VEC_EQ(lhs.read(), (std::vector<int32_t>{6, 24, 54, 96, 150, 216}));
+    // explicit launch shape (cuda_device.rs:99-112)
+    const uint32_t grid[3] = {1, 1, 1}, block[3] = {64, 1, 1};
+    device.launch_kernel(ew_src("add", '+'), "add", grid, block, 0, lhs, rhs, out, len);
+    CHECK_VEC_EQ(out.read(), (std::vector<int32_t>{9, 30, 63, 108, 165, 234}));
+}
+
+// src/devices/cuda/lazy.rs:96-196: the same kernels recorded as operations of Lazy and replayed
+TEST_CASE(hip_launch_kernel1d_lazy) {
+    using D = HIP<Lazy<Base, int32_t>>;
+    D device;
+    auto lhs = device.buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto rhs = device.buffer<int32_t>({1, 2, 3, 4, 5, 6});
+    auto out = lhs.empty_like();
+    auto op = [](const char* name, char c) {
+        return [name, c](Buffer<int32_t, D>& l, Buffer<int32_t, D>& r, Buffer<int32_t, D>& o, D& d) {
+            d.launch_kernel1d(l.len(), ew_src(name, c), name, l, r, o, static_cast<int>(l.len()));
+        };
+    };
+    device.add_op(std::tie(lhs, rhs, out), op("add", '+'));
+    device.add_op(std::tie(out, lhs, rhs), op("add", '+'));
+    device.add_op(std::tie(out, rhs, lhs), op("mul", '*'));
+    CHECK_VEC_EQ(out.read(), (std::vector<int32_t>(6, 0)));
+    for (int i = 0; i < 10; i++) {
+        lhs.write({1, 2, 3, 4, 5, 6});
+        rhs.write({1, 2, 3, 4, 5, 6});
+        device.run();
+    }
+    CHECK_EQ(device.graph_builds(), uint64_t(1));
+    CHECK_EQ(device.graph_kernel_nodes(), size_t(3));
+    CHECK_VEC_EQ(out.read(), (std::vector<int32_t>{2, 4, 6, 8, 10, 12}));
+    CHECK_VEC_EQ(rhs.read(), (std::vector<int32_t>{3, 6, 9, 12, 15, 18}));
+    CHECK_VEC_EQ(lhs.read(), (std::vector<int32_t>{6, 24, 54, 96, 150, 216}));
+}
+
 TEST_CASE(hip_backend_errors_surface) {
     bool threw = false;
     try {

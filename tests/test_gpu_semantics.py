@@ -316,3 +316,111 @@ def test_alloc_is_zeroed_and_clear_write_copy(hip):
     u = hip.buffer([1, 2, 3, 4, 5, 6], "u32")                    # src/devices/cuda/ops.rs:242-247
     u.clear()
     assert u.read().tolist() == [0] * 6
+
+
+RELU_SRC = """extern "C" __global__ void relu(float* lhs, float* out, int numElements) {
+    int idx = blockDim.x * blockIdx.x + threadIdx.x;
+    if (idx < numElements) out[idx] = max(lhs[idx], 0.0f);
+}
+"""
+ADD_SRC = """extern "C" __global__ void add(float* lhs, float* rhs, float* out, int numElements) {
+    int idx = blockDim.x * blockIdx.x + threadIdx.x;
+    if (idx < numElements) out[idx] = lhs[idx] + rhs[idx];
+}
+"""
+
+
+def test_caller_written_kernels(hip):
+    """`launch_kernel1d` with user source: the add / relu ops of tests/graph/mod.rs:90-127."""
+    n = 100003
+    a = synth.uniform_f32(1, n, -2, 2)
+    b = synth.uniform_f32(2, n, -2, 2)
+    ab, bb, cb, db = hip.buffer(a), hip.buffer(b), hip.alloc(n), hip.alloc(n)
+    c0, h0 = hip.cache_stats()
+    hip.launch_kernel1d(n, ADD_SRC, "add", [ab, bb, cb, n])
+    hip.launch_kernel1d(n, RELU_SRC, "relu", [cb, db, n])
+    hip.launch_kernel1d(n, ADD_SRC, "add", [db, ab, cb, n])       # cached: same source and name
+    c1, h1 = hip.cache_stats()
+    assert (c1 - c0, h1 - h0) == (2, 1)
+    want = np.maximum(a + b, np.float32(0)) + a
+    assert_bits_equal(cb.read(), want.astype(np.float32))
+    hip.launch_kernel(ADD_SRC, "add", (4, 1, 1), (256, 1, 1), 0, [ab, bb, db, 1000])
+    got = db.read()
+    assert_bits_equal(got[:1000], (a + b)[:1000])
+    assert_bits_equal(got[1000:], np.maximum(a + b, np.float32(0))[1000:])
+    # errors: bad source, wrong entry point for the kernel kind
+    with pytest.raises(capi.CustosHipError) as e:
+        hip.compile_source("this is not HIP", "nope")
+    assert e.value.code == capi.ERR_COMPILE
+    k = hip.compile_source(ADD_SRC, "add")
+    assert hip.lib.custos_hip_apply_fn(hip.handle, k, ab.ptr, cb.ptr, 10) == capi.ERR_KIND_MISMATCH
+
+
+def test_caller_written_kernels_in_a_graph_are_fences(hip, oracle):
+    """A recorded user kernel has unknown memory use: everything before it runs first,
+    everything after it runs later, while the expression kernels around it still merge."""
+    n = 4096
+    xs = [synth.uniform_f32(10 + i, n, -2, 2) for i in range(8)]
+    bufs = [hip.buffer(x) for x in xs]
+    mids = [hip.alloc(n) for _ in xs]
+    outs = [hip.alloc(n) for _ in xs]
+    f = lambda v: v.mul(2.0)
+    hip.capture_begin()
+    for b, m in zip(bufs, mids):
+        hip.apply_fn(b, f, out=m)
+    hip.launch_kernel1d(n, RELU_SRC, "relu", [mids[0], outs[0], n])      # fence
+    for m, o in zip(mids[1:], outs[1:]):
+        hip.apply_fn(m, f, out=o)
+    g = hip.capture_end()
+    assert g.stats() == (8 + 1 + 7, 3, 3)
+    g.launch()
+    hip.sync()
+    assert_bits_equal(outs[0].read(), np.maximum(xs[0] * np.float32(2), np.float32(0)))
+    for x, o in zip(xs[1:], outs[1:]):
+        assert_bits_equal(o.read(), (x * np.float32(4)).astype(np.float32))
+
+
+def test_disk_cache_of_code_objects(tmp_path, monkeypatch):
+    """CUSTOS_HIP_KERNEL_CACHE_DIR: a second device loads the code object instead of compiling."""
+    import custos_amd
+    monkeypatch.setenv("CUSTOS_HIP_KERNEL_CACHE_DIR", str(tmp_path / "kcache"))
+    x = synth.uniform_f32(5, 1000, -1, 1)
+    f = lambda v: v.mul(0.37).add(11.5)
+    first = custos_amd.HIP(0)
+    want = first.apply_fn(first.buffer(x), f).read()
+    assert first.cache_stats()[0] == 1 and first.disk_cache_hits() == 0
+    files = list((tmp_path / "kcache").iterdir())
+    assert len(files) == 1 and files[0].suffix == ".co" and "gfx950" in files[0].name
+    first.close()
+    second = custos_amd.HIP(0)
+    got = second.apply_fn(second.buffer(x), f).read()
+    assert second.cache_stats()[0] == 0 and second.disk_cache_hits() == 1
+    assert_bits_equal(got, want)
+    # a damaged file is ignored and replaced
+    files[0].write_bytes(b"garbage")
+    third = custos_amd.HIP(0)
+    assert_bits_equal(third.apply_fn(third.buffer(x), f).read(), want)
+    assert third.cache_stats()[0] == 1 and third.disk_cache_hits() == 0
+    second.close()
+    third.close()
+
+
+def test_more_than_2p32_bytes_and_elements(hip):
+    """64-bit indexing: a u8 buffer of 2^32 + 77 elements (more than 4 GiB in, 4 GiB out)."""
+    n = (1 << 32) + 77
+    src = hip.alloc(n, "u8", zeroed=False)
+    pattern = (np.arange(1 << 20, dtype=np.uint32) * 7 + 3).astype(np.uint8)
+    hip.write(src.slice(0, 1 << 20), pattern)
+    filled = 1 << 20
+    while filled < n:                                   # replicate on the device by doubling copies
+        step = min(filled, n - filled)
+        hip.copy(src.slice(filled, filled + step), src.slice(0, step))
+        filled += step
+    out = hip.apply_fn(src, lambda v: v.mul(3).add(1))
+    want = (pattern.astype(np.uint32) * 3 + 1).astype(np.uint8)
+    for start in (0, (1 << 31) - (1 << 19), (1 << 32) - (1 << 20), n - (1 << 20)):
+        off = start % (1 << 20)
+        got = out.slice(start, start + (1 << 20)).read()
+        assert_bits_equal(got, np.roll(want, -off), f"window at {start}")
+    tail = out.slice(n - 77, n).read()
+    assert_bits_equal(tail, np.roll(want, -((n - 77) % (1 << 20)))[:77])
