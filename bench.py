@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per launch of the fused chain at N = 2^28 with the default launch shape, from two
 # `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE) scaled by the identity-copy kernel of
 # known size; commands and raw counter values: profiles/fused_chain_f32_n2p28_hbm_traffic.md
-MEASURED_TRAFFIC_C2_N2P28 = 2147505869
+MEASURED_TRAFFIC_C2_N2P28 = 2147591552
 
 C2_OPS = [
     lambda v: v.sin(),
@@ -235,6 +235,7 @@ def bench_others(dev, args):
     got = ob.read()
     assert np.max(np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))) <= 4
     out["c1"] = _entry("c1: apply_fn(exp), f32 N=2^20, U[-4,4) seed 0", n, 8, ms / (steps * 4), cpu_s, n)
+    out["c1"]["kernel"] = dev.kernel_name(k)
 
     # c3: unary_ew tanh forward + backward, f32 N = 2^26
     n = 1 << 26
@@ -257,8 +258,10 @@ def bench_others(dev, args):
     g0 = np.full(cn, 0.1, dtype=np.float32)
     cpu_s, _ = _cpu_time(lambda: (cpu_oracle.c3_tanh_fwd(x[:cn]), cpu_oracle.c3_tanh_bwd(x[:cn], g0, yg[:cn])))
     e = _entry("c3: unary_ew tanh fwd + bwd (x_grad += y_grad*(1-tanh(x)^2)), f32 N=2^26", n, 24, ms / steps, cpu_s, cn)
-    e["forward"] = {"ms": round(ms_f / steps, 5), "GBps": round(8 * n / (ms_f / steps * 1e-3) / 1e9, 2)}
-    e["backward"] = {"ms": round(ms_b / steps, 5), "GBps": round(16 * n / (ms_b / steps * 1e-3) / 1e9, 2)}
+    e["forward"] = {"ms": round(ms_f / steps, 5), "GBps": round(8 * n / (ms_f / steps * 1e-3) / 1e9, 2),
+                    "kernel": dev.kernel_name(kf)}
+    e["backward"] = {"ms": round(ms_b / steps, 5), "GBps": round(16 * n / (ms_b / steps * 1e-3) / 1e9, 2),
+                     "kernel": dev.kernel_name(kb)}
     out["c3"] = e
     del xb, ygb, yb, gb
 
@@ -275,6 +278,7 @@ def bench_others(dev, args):
     d = np.abs(got.view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
     assert d.max() <= 1, "c4 differs from the CPU port by more than 1 f16 ulp"
     out["c4"] = _entry(f"c4: f16 chain exp(x*0.5)*x + x^2, f32 compute, N=2^{args.log2n}", n, 4, ms / steps, cpu_s, cn)
+    out["c4"]["kernel"] = dev.kernel_name(k)
     del xb, ob
 
     # c5: 1024 buffers x 4096 f32: t=a*b; u=t+c; y=sqrt(abs(u))*0.3, one graph, 100 replays
@@ -306,6 +310,7 @@ def bench_others(dev, args):
     e["graph_kernel_nodes"] = graph.kernel_nodes
     e["recorded_launches"] = 3 * nbuf
     e["graph_build_ms"] = round(build_s * 1e3, 2)
+    e["kernels"] = [dev.kernel_name(q) + "_batched" for q in (kmul, kadd, kun)]
     graph.destroy()
 
     # the same work after element-wise fusing (what `Lazy::elementwise_fusing` of the host stack
@@ -326,6 +331,7 @@ def bench_others(dev, args):
         "GBps": round(16 * nbuf * m / (fms / replays * 1e-3) / 1e9, 2),
         "graph_kernel_nodes": fgraph.kernel_nodes,
         "expression": "(sqrt(abs(((a * b) + c))) * 0.3)",
+        "kernel": dev.kernel_name(kf) + "_batched",
     }
     out["c5"] = e
     fgraph.destroy()
