@@ -85,6 +85,29 @@ def test_transcendental_ulp(hip, oracle, name):
     assert d.max() <= 4, (name, int(d.max()), x[np.argmax(d)])
 
 
+WIDE = {
+    "exp": lambda v: v.exp(), "sin": lambda v: v.sin(), "cos": lambda v: v.cos(), "tan": lambda v: v.tan(),
+    "tanh": lambda v: v.tanh(), "ln": lambda v: v.ln(), "sqrt": lambda v: v.sqrt(),
+}
+
+
+@pytest.mark.parametrize("name", sorted(WIDE))
+def test_transcendentals_over_all_float_bit_patterns(hip, oracle, name):
+    """2^22 random f32 bit patterns (every exponent, both signs, denormals, inf, NaN):
+    within 4 ulp of the CPU path everywhere, NaN where it is NaN, same infinities.
+    Overflow, underflow into denormals and huge arguments of sin/cos/tan are all in here."""
+    n = 1 << 22
+    bits = (synth.splitmix64(77, n) >> np.uint64(32)).astype(np.uint32)
+    x = bits.view(np.float32)
+    got = hip.apply_fn(hip.buffer(x), WIDE[name]).read()
+    want = oracle.apply_fn(WIDE[name], x)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan), name
+    d = ulp_distance_f32(got[~nan], want[~nan])
+    worst = int(np.argmax(d))
+    assert d.max() <= (0 if name == "sqrt" else 4), (name, int(d.max()), x[~nan][worst], got[~nan][worst], want[~nan][worst])
+
+
 def test_pow_ulp(hip, oracle):
     n = 1 << 18
     a = synth.uniform_f32(51, n, 0.01, 20)
