@@ -341,8 +341,8 @@ def bench_others(dev, args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c2", choices=["c2"])
     ap.add_argument("--log2n", type=int, default=28)
     ap.add_argument("--cpu-log2n", dest="cpu_log2n", type=int, default=28,
