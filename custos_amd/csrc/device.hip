@@ -1,0 +1,292 @@
+// Device handle, memory, zero fill and timing of the C ABI (include/custos_hip.h).
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "runtime.hpp"
+
+namespace custos_hip {
+
+thread_local std::string g_last_error;
+
+int32_t set_error(custos_hip_device* dev, int32_t code, const std::string& msg) {
+    (dev ? dev->last_error : g_last_error) = msg;
+    return code;
+}
+
+int32_t hip_fail(custos_hip_device* dev, hipError_t e, const char* what) {
+    // clear the sticky "last error" of the runtime so it is not reported twice
+    (void)hipGetLastError();
+    return set_error(dev, static_cast<int32_t>(e),
+                     std::string(what) + ": " + hipGetErrorName(e) + " (" + hipGetErrorString(e) + ")");
+}
+
+const std::string& thread_last_error() { return g_last_error; }
+
+// ---- zero fill: 16-byte stores over the aligned body, bytes at the edges ----
+
+__global__ void __launch_bounds__(256) custos_fill_zero(unsigned char* p, unsigned long long bytes,
+                                                        unsigned long long head,
+                                                        unsigned long long n_vec) {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    u4* v = reinterpret_cast<u4*>(p + head);
+    const unsigned long long gid = (unsigned long long)blockIdx.x * 256 + threadIdx.x;
+    const unsigned long long n_threads = (unsigned long long)gridDim.x * 256;
+    const u4 z = {0u, 0u, 0u, 0u};
+    for (unsigned long long i = gid; i < n_vec; i += n_threads) v[i] = z;
+    if (gid < head) p[gid] = 0;
+    for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads) p[i] = 0;
+}
+
+unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec) {
+    unsigned long long want = (n_vec + 255) / 256;
+    // 8 vectors per thread at most: enough workgroups to fill the chip, not one per 4 KiB
+    unsigned long long cap = static_cast<unsigned long long>(dev->props.multiProcessorCount) * 64;
+    unsigned long long g = std::max(1ull, std::min(want, std::max(cap, (want + 7) / 8)));
+    return static_cast<unsigned int>(std::min(g, 1ull << 22));
+}
+
+int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream) {
+    unsigned long long head = (16 - (dptr & 15)) & 15;
+    if (head > bytes) head = bytes;
+    unsigned long long n_vec = (bytes - head) / 16;
+    if (dev->capturing && stream == dev->stream) {
+        RecNode node;
+        node.type = RecNode::Fill;
+        node.ptrs = {dptr};
+        node.bytes = bytes;
+        node.head = head;
+        node.n_vec = n_vec;
+        node.acc = {{dptr, dptr + bytes, true}};
+        dev->recorded.push_back(std::move(node));
+        return CUSTOS_HIP_OK;
+    }
+    unsigned int grid = fill_grid(dev, n_vec);
+    hipLaunchKernelGGL(custos_fill_zero, dim3(grid), dim3(256), 0, stream,
+                       reinterpret_cast<unsigned char*>(dptr), static_cast<unsigned long long>(bytes),
+                       head, n_vec);
+    HIP_TRY(dev, hipGetLastError());
+    return CUSTOS_HIP_OK;
+}
+
+void* fill_zero_kernel() { return reinterpret_cast<void*>(custos_fill_zero); }
+
+}  // namespace custos_hip
+
+using namespace custos_hip;
+
+extern "C" {
+
+int32_t custos_hip_device_count(int32_t* count) {
+    if (!count) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "count is null");
+    int c = 0;
+    hipError_t e = hipGetDeviceCount(&c);
+    if (e != hipSuccess) {
+        *count = 0;
+        return hip_fail(nullptr, e, "hipGetDeviceCount");
+    }
+    *count = c;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_chosen_device_idx(void) {
+    const char* v = std::getenv("CUSTOS_HIP_DEVICE_IDX");
+    if (!v || !*v) return 0;
+    char* end = nullptr;
+    long idx = std::strtol(v, &end, 10);
+    if (*end != '\0' || idx < 0) return 0;
+    return static_cast<int32_t>(idx);
+}
+
+int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
+    if (!out) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "out handle is null");
+    *out = nullptr;
+    int count = 0;
+    HIP_TRY(nullptr, hipGetDeviceCount(&count));
+    if (idx < 0 || idx >= count)
+        return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_DEVICE_INDEX,
+                         "device index " + std::to_string(idx) + " out of range: " + std::to_string(count) + " device(s)");
+    std::unique_ptr<custos_hip_device> dev(new custos_hip_device);
+    dev->idx = idx;
+    HIP_TRY(nullptr, hipSetDevice(idx));
+    HIP_TRY(nullptr, hipGetDeviceProperties(&dev->props, idx));
+    dev->arch = dev->props.gcnArchName;
+    dev->tuning = normalize_tuning(0, 0, 0, 0);
+    HIP_TRY(nullptr, hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking));
+    HIP_TRY(nullptr, hipStreamCreateWithFlags(&dev->transfer, hipStreamNonBlocking));
+    HIP_TRY(nullptr, hipEventCreate(&dev->t0));
+    HIP_TRY(nullptr, hipEventCreate(&dev->t1));
+    *out = dev.release();
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_device_destroy(custos_hip_device* dev) {
+    if (!dev) return CUSTOS_HIP_OK;
+    (void)hipSetDevice(dev->idx);
+    (void)hipStreamSynchronize(dev->stream);
+    (void)hipStreamSynchronize(dev->transfer);
+    for (custos_hip_graph* g : dev->graphs) destroy_graph(g);
+    for (auto& bucket : dev->cache)
+        for (auto& k : bucket.second)
+            if (k->module) (void)hipModuleUnload(k->module);
+    (void)hipEventDestroy(dev->t0);
+    (void)hipEventDestroy(dev->t1);
+    (void)hipStreamDestroy(dev->stream);
+    (void)hipStreamDestroy(dev->transfer);
+    delete dev;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_get_device_info(custos_hip_device* dev, custos_hip_device_info* info) {
+    REQUIRE_DEV(dev);
+    if (!info) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "info is null");
+    std::memset(info, 0, sizeof *info);
+    std::snprintf(info->name, sizeof info->name, "%s", dev->props.name);
+    std::snprintf(info->arch, sizeof info->arch, "%s", dev->props.gcnArchName);
+    info->compute_units = dev->props.multiProcessorCount;
+    info->wavefront_size = dev->props.warpSize;
+    info->clock_khz = dev->props.clockRate;
+    info->memory_clock_khz = dev->props.memoryClockRate;
+    info->memory_bus_bits = dev->props.memoryBusWidth;
+    info->l2_bytes = dev->props.l2CacheSize;
+    info->total_memory = dev->props.totalGlobalMem;
+    return CUSTOS_HIP_OK;
+}
+
+const char* custos_hip_last_error(custos_hip_device* dev) {
+    return dev ? dev->last_error.c_str() : thread_last_error().c_str();
+}
+
+int32_t custos_hip_sync(custos_hip_device* dev) {
+    REQUIRE_DEV(dev);
+    if (dev->capturing)
+        return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot wait for a stream that is recording");
+    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_tuning(custos_hip_device* dev, const custos_hip_tuning* tuning) {
+    REQUIRE_DEV(dev);
+    dev->tuning = tuning_from_c(tuning);
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_get_tuning(custos_hip_device* dev, custos_hip_tuning* tuning) {
+    REQUIRE_DEV(dev);
+    if (!tuning) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "tuning is null");
+    tuning->block_threads = dev->tuning.block_threads;
+    tuning->unroll = dev->tuning.unroll;
+    tuning->blocks_per_cu = dev->tuning.blocks_per_cu;
+    tuning->nontemporal = dev->tuning.nontemporal;
+    return CUSTOS_HIP_OK;
+}
+
+// ---- memory ----
+
+int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, uint64_t* dptr) {
+    REQUIRE_DEV(dev);
+    if (!dptr) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "dptr is null");
+    *dptr = 0;
+    if (bytes == 0) return set_error(dev, CUSTOS_HIP_ERR_ZERO_LENGTH_BUFFER, "zero length buffers are not supported");
+    void* p = nullptr;
+    HIP_TRY(dev, hipMalloc(&p, bytes));
+    uint64_t addr = reinterpret_cast<uint64_t>(p);
+    if (flags != CUSTOS_HIP_ALLOC_UNINIT) {
+        // While recording, the fill must run now and not become part of the graph.
+        hipStream_t s = dev->capturing ? dev->transfer : dev->stream;
+        int32_t rc = launch_fill_zero(dev, addr, bytes, s);
+        if (rc == CUSTOS_HIP_OK && dev->capturing) {
+            hipError_t e = hipStreamSynchronize(dev->transfer);
+            if (e != hipSuccess) rc = hip_fail(dev, e, "hipStreamSynchronize(transfer)");
+        }
+        if (rc != CUSTOS_HIP_OK) {
+            (void)hipFree(p);
+            return rc;
+        }
+    }
+    *dptr = addr;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_free(custos_hip_device* dev, uint64_t dptr) {
+    REQUIRE_DEV(dev);
+    if (dptr == 0) return CUSTOS_HIP_OK;
+    // work that still uses the range must finish first
+    if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    HIP_TRY(dev, hipFree(reinterpret_cast<void*>(dptr)));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_write(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    if (dev->capturing) {
+        HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), src, bytes, hipMemcpyHostToDevice, dev->transfer));
+        HIP_TRY(dev, hipStreamSynchronize(dev->transfer));
+        return CUSTOS_HIP_OK;
+    }
+    HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), src, bytes, hipMemcpyHostToDevice, dev->stream));
+    // the caller may reuse `src` right away
+    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_read(custos_hip_device* dev, void* dst, uint64_t src, size_t bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    HIP_TRY(dev, hipMemcpyAsync(dst, reinterpret_cast<const void*>(src), bytes, hipMemcpyDeviceToHost, dev->transfer));
+    HIP_TRY(dev, hipStreamSynchronize(dev->transfer));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    if (dev->capturing) {
+        RecNode node;
+        node.type = RecNode::Copy;
+        node.ptrs = {dst, src};
+        node.bytes = bytes;
+        node.acc = {{dst, dst + bytes, true}, {src, src + bytes, false}};
+        dev->recorded.push_back(std::move(node));
+        return CUSTOS_HIP_OK;
+    }
+    HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src), bytes,
+                                hipMemcpyDeviceToDevice, dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_clear(custos_hip_device* dev, uint64_t dptr, size_t bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dptr) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    return launch_fill_zero(dev, dptr, bytes, dev->stream);
+}
+
+// ---- timing ----
+
+int32_t custos_hip_timer_begin(custos_hip_device* dev) {
+    REQUIRE_DEV(dev);
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot time a recording stream");
+    HIP_TRY(dev, hipEventRecord(dev->t0, dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_timer_end(custos_hip_device* dev, double* ms) {
+    REQUIRE_DEV(dev);
+    if (!ms) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "ms is null");
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot time a recording stream");
+    HIP_TRY(dev, hipEventRecord(dev->t1, dev->stream));
+    HIP_TRY(dev, hipEventSynchronize(dev->t1));
+    float f = 0.f;
+    HIP_TRY(dev, hipEventElapsedTime(&f, dev->t0, dev->t1));
+    *ms = f;
+    return CUSTOS_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,292 @@
+// Recording and graph construction: dependency levels from address-range
+// conflicts, merging of equal launches, explicit hipGraph nodes, replay
+// (include/custos_hip.h).
+#include <algorithm>
+
+#include "runtime.hpp"
+
+namespace custos_hip {
+
+namespace {
+
+// ---- building a graph from the recorded work ----
+//
+// The recorded list is not replayed launch by launch.  Every node gets a
+// dependency level: one more than the highest level among earlier nodes whose
+// memory it conflicts with (read-after-write, write-after-read or
+// write-after-write on overlapping address ranges).  Nodes of one level are
+// independent of each other, so they run side by side in the graph, and kernel
+// launches of one level that use the same kernel over the same length are
+// merged into ONE grid that walks a table of operand addresses.  1024 small
+// buffers with three operations each become three kernel nodes instead of
+// 3072.
+
+constexpr uint64_t kChunkShift = 21;  // conflict search buckets of 2 MiB
+
+void assign_levels(std::vector<RecNode>& nodes) {
+    struct Seen {
+        uint64_t begin, end;
+        bool write;
+        int level;
+    };
+    std::vector<Seen> seen;
+    std::unordered_map<uint64_t, std::vector<uint32_t>> buckets;
+    int highest = -1;  // highest level so far
+    int fence = -1;    // level of the last node with unknown memory use
+    for (RecNode& node : nodes) {
+        int level = fence + 1;
+        if (node.type == RecNode::Source) {
+            // unknown reads and writes: after everything before, before everything after
+            node.level = fence = highest = highest + 1;
+            continue;
+        }
+        for (const Access& a : node.acc) {
+            if (a.end <= a.begin) continue;
+            for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) {
+                auto it = buckets.find(c);
+                if (it == buckets.end()) continue;
+                for (uint32_t si : it->second) {
+                    const Seen& s = seen[si];
+                    if (s.level < level) continue;        // cannot raise the level any more
+                    if (!a.write && !s.write) continue;   // two reads never conflict
+                    if (a.begin < s.end && s.begin < a.end) level = s.level + 1;
+                }
+            }
+        }
+        node.level = level;
+        highest = std::max(highest, level);
+        for (const Access& a : node.acc) {
+            if (a.end <= a.begin) continue;
+            const uint32_t idx = static_cast<uint32_t>(seen.size());
+            seen.push_back({a.begin, a.end, a.write, level});
+            for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) buckets[c].push_back(idx);
+        }
+    }
+}
+
+bool batchable(const RecNode& n) {
+    if (n.type != RecNode::Kernel || n.head != 0 || !n.k->fn_batched) return false;
+    for (uint64_t p : n.ptrs)
+        if (p & 15) return false;
+    return true;
+}
+
+}  // namespace
+
+int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
+    std::vector<RecNode>& nodes = dev->recorded;
+    assign_levels(nodes);
+    int max_level = -1;
+    for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
+    g->recorded = nodes.size();
+    g->levels = static_cast<size_t>(max_level + 1);
+
+    // plan: per level, either single nodes or batches of node indices
+    struct Planned {
+        std::vector<size_t> members;  // indices into `nodes`; more than one = batched launch
+        size_t table_offset = 0;      // in u64 entries
+    };
+    std::vector<std::vector<Planned>> plan(static_cast<size_t>(max_level + 1));
+    std::vector<uint64_t> host_table;
+    for (int level = 0; level <= max_level; level++) {
+        std::vector<Planned>& out = plan[level];
+        // batches keyed by (kernel, n), in first-seen order
+        std::vector<std::pair<std::pair<custos_hip_kernel*, unsigned long long>, size_t>> keys;
+        for (size_t i = 0; i < nodes.size(); i++) {
+            if (nodes[i].level != level) continue;
+            if (dev->batching && batchable(nodes[i])) {
+                const auto key = std::make_pair(nodes[i].k, nodes[i].n);
+                size_t slot = out.size();
+                for (const auto& kv : keys)
+                    if (kv.first == key) slot = kv.second;
+                if (slot == out.size()) {
+                    keys.push_back({key, slot});
+                    out.emplace_back();
+                }
+                out[slot].members.push_back(i);
+            } else {
+                out.emplace_back();
+                out.back().members.push_back(i);
+            }
+        }
+        for (Planned& p : out) {
+            if (p.members.size() < 2) continue;
+            p.table_offset = host_table.size();
+            for (size_t i : p.members)
+                for (uint64_t ptr : nodes[i].ptrs) host_table.push_back(ptr);
+        }
+    }
+    if (!host_table.empty()) {
+        HIP_TRY(dev, hipMalloc(&g->table, host_table.size() * sizeof(uint64_t)));
+        HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
+    }
+
+    HIP_TRY(dev, hipGraphCreate(&g->graph, 0));
+    std::vector<hipGraphNode_t> prev;  // what the nodes of the current level wait for
+    for (int level = 0; level <= max_level; level++) {
+        std::vector<hipGraphNode_t> deps = prev;
+        if (deps.size() > 1) {  // one join node instead of |prev| x |level| edges
+            hipGraphNode_t join;
+            HIP_TRY(dev, hipGraphAddEmptyNode(&join, g->graph, deps.data(), deps.size()));
+            deps = {join};
+        }
+        std::vector<hipGraphNode_t> made;
+        for (const Planned& p : plan[level]) {
+            const RecNode& first = nodes[p.members[0]];
+            hipGraphNode_t node;
+            if (first.type == RecNode::Copy) {
+                HIP_TRY(dev, hipGraphAddMemcpyNode1D(&node, g->graph, deps.data(), deps.size(),
+                                                     reinterpret_cast<void*>(first.ptrs[0]),
+                                                     reinterpret_cast<const void*>(first.ptrs[1]), first.bytes,
+                                                     hipMemcpyDeviceToDevice));
+                made.push_back(node);
+                continue;
+            }
+            hipKernelNodeParams kp{};
+            kp.sharedMemBytes = 0;
+            kp.extra = nullptr;
+            std::vector<void*> args;
+            uint64_t ptrs[8];
+            unsigned long long a0, a1, a2, a3;
+            if (first.type == RecNode::Source) {
+                for (const auto& v : first.arg_values) args.push_back(const_cast<unsigned char*>(v.data()));
+                kp.func = reinterpret_cast<void*>(first.k->fn);
+                kp.gridDim = dim3(first.grid3[0], first.grid3[1], first.grid3[2]);
+                kp.blockDim = dim3(first.block3[0], first.block3[1], first.block3[2]);
+                kp.sharedMemBytes = first.shared_mem;
+            } else if (first.type == RecNode::Fill) {
+                ptrs[0] = first.ptrs[0];
+                a0 = first.bytes, a1 = first.head, a2 = first.n_vec;
+                args = {&ptrs[0], &a0, &a1, &a2};
+                kp.func = fill_zero_kernel();
+                kp.gridDim = dim3(fill_grid(dev, first.n_vec));
+                kp.blockDim = dim3(256);
+            } else if (p.members.size() == 1) {
+                for (size_t i = 0; i < first.ptrs.size(); i++) {
+                    ptrs[i] = first.ptrs[i];
+                    args.push_back(&ptrs[i]);
+                }
+                a0 = first.n, a1 = first.head, a2 = first.n_vec;
+                args.push_back(&a0);
+                args.push_back(&a1);
+                args.push_back(&a2);
+                kp.func = reinterpret_cast<void*>(first.k->fn);
+                kp.gridDim = dim3(first.grid);
+                kp.blockDim = dim3(static_cast<unsigned int>(first.k->spec.tuning.block_threads));
+            } else {
+                const Tuning& t = first.k->spec.tuning;
+                const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+                a3 = std::max(1ull, (first.n_vec + tile_vecs - 1) / tile_vecs);  // tiles per segment
+                const unsigned long long blocks = a3 * p.members.size();
+                if (blocks > (1ull << 31) - 1)
+                    return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a batched launch would need more than 2^31 workgroups");
+                ptrs[0] = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
+                a0 = first.n, a1 = first.n_vec;
+                args = {&ptrs[0], &a0, &a1, &a3};
+                kp.func = reinterpret_cast<void*>(first.k->fn_batched);
+                kp.gridDim = dim3(static_cast<unsigned int>(blocks));
+                kp.blockDim = dim3(static_cast<unsigned int>(t.block_threads));
+            }
+            kp.kernelParams = args.data();
+            HIP_TRY(dev, hipGraphAddKernelNode(&node, g->graph, deps.data(), deps.size(), &kp));
+            g->kernel_nodes++;
+            made.push_back(node);
+        }
+        prev = std::move(made);
+    }
+    HIP_TRY(dev, hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
+    return CUSTOS_HIP_OK;
+}
+
+void destroy_graph(custos_hip_graph* g) {
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    if (g->table) (void)hipFree(g->table);
+    delete g;
+}
+
+}  // namespace custos_hip
+
+using namespace custos_hip;
+
+extern "C" {
+
+// ---- capture / replay ----
+
+int32_t custos_hip_capture_begin(custos_hip_device* dev) {
+    REQUIRE_DEV(dev);
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the device is already recording");
+    // Earlier eager work must be complete before anything recorded can run, and
+    // the recorded list starts empty.  Allocation, reads and writes stay legal
+    // while recording: they execute at once and are not part of the graph.
+    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    dev->recorded.clear();
+    dev->capturing = true;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_capture_end(custos_hip_device* dev, custos_hip_graph** graph) {
+    REQUIRE_DEV(dev);
+    if (!graph) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph out pointer is null");
+    *graph = nullptr;
+    if (!dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the device is not recording");
+    dev->capturing = false;
+    custos_hip_graph* g = new custos_hip_graph;
+    int32_t rc = build_graph(dev, g);
+    dev->recorded.clear();
+    if (rc != CUSTOS_HIP_OK) {
+        destroy_graph(g);
+        return rc;
+    }
+    dev->graphs.push_back(g);
+    *graph = g;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_graph_batching(custos_hip_device* dev, int32_t enabled) {
+    REQUIRE_DEV(dev);
+    dev->batching = enabled != 0;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_is_capturing(custos_hip_device* dev, int32_t* capturing) {
+    REQUIRE_DEV(dev);
+    if (!capturing) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "capturing is null");
+    *capturing = dev->capturing ? 1 : 0;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_launch(custos_hip_device* dev, custos_hip_graph* graph) {
+    REQUIRE_DEV(dev);
+    if (!graph) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph is null");
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot replay while recording");
+    HIP_TRY(dev, hipGraphLaunch(graph->exec, dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_node_count(custos_hip_graph* graph, size_t* kernel_nodes) {
+    if (!graph || !kernel_nodes) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    *kernel_nodes = graph->kernel_nodes;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_stats(custos_hip_graph* graph, size_t* recorded, size_t* kernel_nodes, size_t* levels) {
+    if (!graph) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph is null");
+    if (recorded) *recorded = graph->recorded;
+    if (kernel_nodes) *kernel_nodes = graph->kernel_nodes;
+    if (levels) *levels = graph->levels;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_destroy(custos_hip_device* dev, custos_hip_graph* graph) {
+    REQUIRE_DEV(dev);
+    if (!graph) return CUSTOS_HIP_OK;
+    auto it = std::find(dev->graphs.begin(), dev->graphs.end(), graph);
+    if (it == dev->graphs.end()) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph does not belong to this device");
+    dev->graphs.erase(it);
+    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    destroy_graph(graph);
+    return CUSTOS_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,313 @@
+// Run-time compilation of kernels (hiprtc), the kernel caches in memory and on
+// disk, and the host-only expression helpers of the C ABI (include/custos_hip.h).
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+
+#include "runtime.hpp"
+
+namespace custos_hip {
+
+namespace {
+
+// ---- code objects on disk ----
+//
+// With CUSTOS_HIP_KERNEL_CACHE_DIR set, every compiled code object is stored as
+// <dir>/<key>-<arch>-<hiprtc version>.co together with the source it was built
+// from; a later process loads it instead of compiling when the stored source is
+// identical (the 64-bit key alone is not trusted).
+
+std::string cache_file(const KernelSpec& spec, const std::string& arch) {
+    const char* dir = std::getenv("CUSTOS_HIP_KERNEL_CACHE_DIR");
+    if (!dir || !*dir) return "";
+    int major = 0, minor = 0;
+    (void)hiprtcVersion(&major, &minor);
+    std::string a = arch;
+    for (char& c : a)
+        if (c == ':' || c == '/' || c == '+') c = '_';
+    char key[17];
+    std::snprintf(key, sizeof key, "%016llx", static_cast<unsigned long long>(spec.hash));
+    return std::string(dir) + "/" + key + "-" + a + "-" + std::to_string(major) + "." + std::to_string(minor) + ".co";
+}
+
+// the text hiprtc compiles: generated kernels start with a comment line that
+// spells the expression as the caller wrote it; it is not part of the identity
+std::string source_identity(const KernelSpec& spec) {
+    if (spec.kind == Kind::Source) return spec.name + "\n" + spec.source;
+    return spec.source.substr(spec.source.find('\n') + 1);
+}
+
+bool load_cached_code(const KernelSpec& spec, const std::string& arch, std::vector<char>* code) {
+    const std::string path = cache_file(spec, arch);
+    if (path.empty()) return false;
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return false;
+    char magic[8] = {0};
+    uint64_t src_len = 0, code_len = 0;
+    f.read(magic, 8);
+    f.read(reinterpret_cast<char*>(&src_len), 8);
+    if (!f || std::memcmp(magic, "CUSTOSC1", 8) != 0 || src_len > (1u << 26)) return false;
+    std::string src(src_len, '\0');
+    f.read(&src[0], static_cast<std::streamsize>(src_len));
+    f.read(reinterpret_cast<char*>(&code_len), 8);
+    if (!f || src != source_identity(spec) || code_len == 0 || code_len > (1u << 28)) return false;
+    code->resize(code_len);
+    f.read(code->data(), static_cast<std::streamsize>(code_len));
+    return static_cast<bool>(f);
+}
+
+void store_cached_code(const KernelSpec& spec, const std::string& arch, const std::vector<char>& code) {
+    const std::string path = cache_file(spec, arch);
+    if (path.empty()) return;
+    (void)mkdir(std::getenv("CUSTOS_HIP_KERNEL_CACHE_DIR"), 0777);
+    const std::string tmp = path + ".tmp" + std::to_string(static_cast<long>(getpid()));
+    {
+        std::ofstream f(tmp, std::ios::binary | std::ios::trunc);
+        if (!f) return;
+        const std::string src = source_identity(spec);
+        const uint64_t src_len = src.size(), code_len = code.size();
+        f.write("CUSTOSC1", 8);
+        f.write(reinterpret_cast<const char*>(&src_len), 8);
+        f.write(src.data(), static_cast<std::streamsize>(src_len));
+        f.write(reinterpret_cast<const char*>(&code_len), 8);
+        f.write(code.data(), static_cast<std::streamsize>(code_len));
+        if (!f) {
+            std::remove(tmp.c_str());
+            return;
+        }
+    }
+    if (std::rename(tmp.c_str(), path.c_str()) != 0) std::remove(tmp.c_str());
+}
+
+bool markers_from_c(const char* const* markers, int32_t n, std::vector<std::string>* out) {
+    if (!markers || n < 1 || n > 4) return false;
+    for (int i = 0; i < n; i++) {
+        if (!markers[i] || !markers[i][0]) return false;
+        out->push_back(markers[i]);
+    }
+    return true;
+}
+
+int32_t spec_from_c(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
+                    const char* const* markers, int32_t n_markers, const Tuning& tuning,
+                    KernelSpec* spec) {
+    if (!src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");
+    if (kind != CUSTOS_HIP_KIND_APPLY && kind != CUSTOS_HIP_KIND_UNARY_GRAD)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown kernel kind");
+    if (!dtype_valid(dtype)) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown element type");
+    std::vector<std::string> m;
+    if (!markers_from_c(markers, n_markers, &m))
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 4 non-empty markers are required");
+    ParseError err;
+    if (!build_kernel_spec(static_cast<Kind>(kind), static_cast<DType>(dtype), src, m, tuning, spec, &err))
+        return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+    return CUSTOS_HIP_OK;
+}
+
+int32_t copy_out_string(const std::string& s, char* buf, size_t cap, size_t* needed) {
+    if (needed) *needed = s.size() + 1;
+    if (buf && cap) {
+        size_t n = std::min(cap - 1, s.size());
+        std::memcpy(buf, s.data(), n);
+        buf[n] = '\0';
+    }
+    return CUSTOS_HIP_OK;
+}
+
+}  // namespace
+
+// ---- hiprtc ----
+
+int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec,
+                               const std::string& arch, std::vector<char>* code) {
+    hiprtcProgram prog = nullptr;
+    hiprtcResult r = hiprtcCreateProgram(&prog, spec.source.c_str(), "custos_kernel.hip", 0, nullptr, nullptr);
+    if (r != HIPRTC_SUCCESS)
+        return set_error(dev, CUSTOS_HIP_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
+    std::vector<std::string> opts = hiprtc_options(arch);
+    std::vector<const char*> copts;
+    for (const std::string& o : opts) copts.push_back(o.c_str());
+    r = hiprtcCompileProgram(prog, static_cast<int>(copts.size()), copts.data());
+    if (r != HIPRTC_SUCCESS) {
+        size_t log_size = 0;
+        hiprtcGetProgramLogSize(prog, &log_size);
+        std::string log(log_size, '\0');
+        if (log_size) hiprtcGetProgramLog(prog, &log[0]);
+        hiprtcDestroyProgram(&prog);
+        return set_error(dev, CUSTOS_HIP_ERR_COMPILE,
+                         std::string("hiprtcCompileProgram: ") + hiprtcGetErrorString(r) + "\n" + log +
+                             "\n--- source ---\n" + spec.source);
+    }
+    size_t size = 0;
+    hiprtcGetCodeSize(prog, &size);
+    code->resize(size);
+    hiprtcGetCode(prog, code->data());
+    hiprtcDestroyProgram(&prog);
+    return CUSTOS_HIP_OK;
+}
+
+// Code object from the disk cache or from hiprtc, loaded as a module; entry point looked up.
+int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k) {
+    std::vector<char> code;
+    bool from_disk = load_cached_code(k->spec, dev->arch, &code);
+    if (from_disk && hipModuleLoadData(&k->module, code.data()) != hipSuccess) {
+        (void)hipGetLastError();  // a stale or damaged file: compile instead
+        k->module = nullptr;
+        from_disk = false;
+    }
+    if (!from_disk) {
+        int32_t rc = compile_to_code_object(dev, k->spec, dev->arch, &code);
+        if (rc != CUSTOS_HIP_OK) return rc;
+        HIP_TRY(dev, hipModuleLoadData(&k->module, code.data()));
+        store_cached_code(k->spec, dev->arch, code);
+        dev->compiles++;
+    } else {
+        dev->disk_hits++;
+    }
+    hipError_t e = hipModuleGetFunction(&k->fn, k->module, k->spec.name.c_str());
+    if (e != hipSuccess) {
+        (void)hipModuleUnload(k->module);
+        k->module = nullptr;
+        return hip_fail(dev, e, "hipModuleGetFunction");
+    }
+    return CUSTOS_HIP_OK;
+}
+
+}  // namespace custos_hip
+
+using namespace custos_hip;
+
+extern "C" {
+
+// ---- expression kernels ----
+
+int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
+                                const char* const* markers, int32_t n_markers,
+                                custos_hip_kernel** kernel) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "kernel out pointer is null");
+    *kernel = nullptr;
+    std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
+    int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, dev->tuning, &k->spec);
+    if (rc != CUSTOS_HIP_OK) return rc;
+
+    auto& bucket = dev->cache[k->spec.hash];
+    for (auto& cached : bucket) {
+        // the generated text starts with the caller's spelling of the expression
+        // as a comment; compare what is compiled, i.e. everything after it
+        const std::string& a = cached->spec.source;
+        const std::string& b = k->spec.source;
+        if (a.compare(a.find('\n'), std::string::npos, b, b.find('\n'), std::string::npos) == 0) {
+            dev->hits++;
+            *kernel = cached.get();
+            return CUSTOS_HIP_OK;
+        }
+    }
+    rc = build_module(dev, k.get());
+    if (rc != CUSTOS_HIP_OK) return rc;
+    // the second entry point of the module: many equal launches in one grid
+    if (hipModuleGetFunction(&k->fn_batched, k->module, (k->spec.name + "_batched").c_str()) != hipSuccess) {
+        (void)hipGetLastError();
+        k->fn_batched = nullptr;
+    }
+    *kernel = k.get();
+    bucket.push_back(std::move(k));
+    return CUSTOS_HIP_OK;
+}
+
+// ---- caller-written kernels (src/devices/cuda/kernel_cache.rs:39-61, kernel_launch.rs:81-163) ----
+
+int32_t custos_hip_source_compile(custos_hip_device* dev, const char* src, const char* fn_name,
+                                  custos_hip_kernel** kernel) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "kernel out pointer is null");
+    *kernel = nullptr;
+    if (!src || !fn_name || !*fn_name) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "source or function name is null");
+    std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
+    k->spec.kind = Kind::Source;
+    k->spec.name = fn_name;
+    k->spec.source = src;
+    k->spec.hash = fnv1a64(fn_name, std::strlen(fn_name), fnv1a64(src, std::strlen(src), fnv1a64("custos-source-v1", 16)));
+    auto& bucket = dev->cache[k->spec.hash];
+    for (auto& cached : bucket) {
+        if (cached->spec.kind == Kind::Source && cached->spec.name == k->spec.name && cached->spec.source == k->spec.source) {
+            dev->hits++;
+            *kernel = cached.get();
+            return CUSTOS_HIP_OK;
+        }
+    }
+    int32_t rc = build_module(dev, k.get());
+    if (rc != CUSTOS_HIP_OK) return rc;
+    *kernel = k.get();
+    bucket.push_back(std::move(k));
+    return CUSTOS_HIP_OK;
+}
+
+const char* custos_hip_kernel_source(const custos_hip_kernel* kernel) {
+    return kernel ? kernel->spec.source.c_str() : "";
+}
+
+const char* custos_hip_kernel_name(const custos_hip_kernel* kernel) {
+    return kernel ? kernel->spec.name.c_str() : "";
+}
+
+uint64_t custos_hip_kernel_hash(const custos_hip_kernel* kernel) { return kernel ? kernel->spec.hash : 0; }
+
+int32_t custos_hip_kernel_arity(const custos_hip_kernel* kernel) {
+    return kernel ? kernel->spec.expr.n_vars : 0;
+}
+
+int32_t custos_hip_cache_stats(custos_hip_device* dev, uint64_t* compiles, uint64_t* hits) {
+    REQUIRE_DEV(dev);
+    if (compiles) *compiles = dev->compiles;
+    if (hits) *hits = dev->hits;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_cache_disk_hits(custos_hip_device* dev, uint64_t* disk_hits) {
+    REQUIRE_DEV(dev);
+    if (disk_hits) *disk_hits = dev->disk_hits;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_expr_emit(int32_t kind, int32_t dtype, const char* src, const char* const* markers,
+                             int32_t n_markers, const custos_hip_tuning* tuning, char* buf, size_t cap,
+                             size_t* needed, uint64_t* hash) {
+    KernelSpec spec;
+    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), &spec);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    if (hash) *hash = spec.hash;
+    return copy_out_string(spec.source, buf, cap, needed);
+}
+
+int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const char* src,
+                                          const char* const* markers, int32_t n_markers,
+                                          const custos_hip_tuning* tuning, size_t* code_size) {
+    KernelSpec spec;
+    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), &spec);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    std::vector<char> code;
+    rc = compile_to_code_object(nullptr, spec, "gfx950", &code);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    if (code_size) *code_size = code.size();
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_expr_canonical(const char* src, const char* const* markers, int32_t n_markers,
+                                  char* buf, size_t cap, size_t* needed) {
+    if (!src) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");
+    std::vector<std::string> m;
+    if (!markers_from_c(markers, n_markers, &m))
+        return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 4 non-empty markers are required");
+    Expr e;
+    ParseError err;
+    if (!parse_expr(src, m, &e, &err)) return set_error(nullptr, err.code, err.message);
+    return copy_out_string(to_cl_source(e, m), buf, cap, needed);
+}
+
+}  // extern "C"

@@ -1,0 +1,191 @@
+// Launches of generated and caller-written kernels: operand checks, the split
+// into scalar head / 16-byte vectors / scalar tail, and recording while the
+// device records (include/custos_hip.h).
+#include <algorithm>
+
+#include "runtime.hpp"
+
+namespace custos_hip {
+
+namespace {
+
+// Checks operand addresses and computes how the element range splits into a
+// scalar head, 16-byte vectors and a scalar tail.
+int32_t plan_launch(custos_hip_device* dev, const custos_hip_kernel* k, const std::vector<Range>& ops,
+                    size_t n, unsigned long long* head, unsigned long long* n_vec, unsigned int* grid) {
+    const size_t es = dtype_size(k->spec.dtype);
+    if (n > (1ull << 40)) return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "more than 2^40 elements");
+    const uint64_t bytes = static_cast<uint64_t>(n) * es;
+    for (const Range& r : ops) {
+        if (r.ptr == 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null device pointer");
+        if (r.ptr % es) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "device pointer is not aligned to the element size");
+    }
+    for (const Range& w : ops) {
+        if (!w.written) continue;
+        for (const Range& r : ops) {
+            if (&r == &w || r.ptr == w.ptr) continue;
+            if (r.ptr < w.ptr + bytes && w.ptr < r.ptr + bytes)
+                return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP,
+                                 "the output range partially overlaps an input range");
+        }
+    }
+    bool same_phase = true;
+    for (const Range& r : ops) same_phase = same_phase && (r.ptr & 15) == (ops[0].ptr & 15);
+    unsigned long long h = 0, nv = 0;
+    if (same_phase) {
+        h = ((16 - (ops[0].ptr & 15)) & 15) / es;
+        if (h > n) h = n;
+        nv = (n - h) / k->spec.vec_elems;
+    }
+    const Tuning& t = k->spec.tuning;
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+    unsigned long long tiles = (nv + tile_vecs - 1) / tile_vecs;
+    unsigned long long scalar = n - nv * k->spec.vec_elems;
+    const unsigned long long cus = static_cast<unsigned long long>(dev->props.multiProcessorCount);
+    unsigned long long scalar_blocks = std::min((scalar + t.block_threads - 1) / t.block_threads, cus * 32);
+    if (t.blocks_per_cu > 0) tiles = std::min(tiles, cus * t.blocks_per_cu);
+    unsigned long long g = std::max(1ull, std::max(tiles, scalar_blocks));
+    g = std::min(g, 1ull << 22);
+    *head = h;
+    *n_vec = nv;
+    *grid = static_cast<unsigned int>(g);
+    return CUSTOS_HIP_OK;
+}
+
+}  // namespace
+
+// Launches the kernel over one set of operands, or records the launch while
+// the device is recording.  `ops` are the operand addresses in the order of the
+// kernel's pointer parameters.
+int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n) {
+    unsigned long long head, n_vec, count = n;
+    unsigned int grid;
+    int32_t rc = plan_launch(dev, k, ops, n, &head, &n_vec, &grid);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    if (dev->capturing) {
+        RecNode node;
+        node.type = RecNode::Kernel;
+        node.k = k;
+        node.n = n;
+        node.head = head;
+        node.n_vec = n_vec;
+        node.grid = grid;
+        const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
+        for (const Range& r : ops) {
+            node.ptrs.push_back(r.ptr);
+            // (the gradient operand of a unary-gradient kernel is read and written;
+            // a write access already orders it against every other access)
+            node.acc.push_back({r.ptr, r.ptr + bytes, r.written});
+        }
+        dev->recorded.push_back(std::move(node));
+        return CUSTOS_HIP_OK;
+    }
+    uint64_t ptrs[8];
+    std::vector<void*> args;
+    for (size_t i = 0; i < ops.size(); i++) {
+        ptrs[i] = ops[i].ptr;
+        args.push_back(&ptrs[i]);
+    }
+    args.push_back(&count);
+    args.push_back(&head);
+    args.push_back(&n_vec);
+    HIP_TRY(dev, hipModuleLaunchKernel(k->fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
+                                       1, 1, 0, dev->stream, args.data(), nullptr));
+    return CUSTOS_HIP_OK;
+}
+
+}  // namespace custos_hip
+
+using namespace custos_hip;
+
+extern "C" {
+
+// ---- launches ----
+
+int32_t custos_hip_apply_fn_n(custos_hip_device* dev, custos_hip_kernel* kernel, const uint64_t* ins,
+                              int32_t n_ins, uint64_t out, size_t n) {
+    REQUIRE_DEV(dev);
+    if (!kernel || !ins) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel or operand list");
+    if (kernel->spec.kind != Kind::Apply)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled as an apply kernel");
+    if (n_ins != kernel->spec.expr.n_vars)
+        return set_error(dev, CUSTOS_HIP_ERR_ARITY_MISMATCH,
+                         "kernel takes " + std::to_string(kernel->spec.expr.n_vars) + " operand(s), got " + std::to_string(n_ins));
+    if (n == 0) return CUSTOS_HIP_OK;
+    std::vector<Range> ops;
+    for (int i = 0; i < n_ins; i++) ops.push_back({ins[i], false});
+    ops.push_back({out, true});
+    return launch_or_record(dev, kernel, ops, n);
+}
+
+int32_t custos_hip_apply_fn(custos_hip_device* dev, custos_hip_kernel* kernel, uint64_t x, uint64_t out, size_t n) {
+    return custos_hip_apply_fn_n(dev, kernel, &x, 1, out, n);
+}
+
+int32_t custos_hip_apply_fn2(custos_hip_device* dev, custos_hip_kernel* kernel, uint64_t lhs, uint64_t rhs,
+                             uint64_t out, size_t n) {
+    uint64_t ins[2] = {lhs, rhs};
+    return custos_hip_apply_fn_n(dev, kernel, ins, 2, out, n);
+}
+
+int32_t custos_hip_add_unary_grad(custos_hip_device* dev, custos_hip_kernel* kernel, uint64_t lhs,
+                                  uint64_t lhs_grad, uint64_t out_grad, size_t n) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel");
+    if (kernel->spec.kind != Kind::UnaryGrad)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled as a unary-gradient kernel");
+    if (n == 0) return CUSTOS_HIP_OK;
+    std::vector<Range> ops = {{lhs, false}, {lhs_grad, true}, {out_grad, false}};
+    return launch_or_record(dev, kernel, ops, n);
+}
+
+int32_t custos_hip_source_launch(custos_hip_device* dev, custos_hip_kernel* kernel, const uint32_t* grid,
+                                 const uint32_t* block, uint32_t shared_mem_bytes, void* const* params,
+                                 const size_t* param_sizes, int32_t n_params) {
+    REQUIRE_DEV(dev);
+    if (!kernel || !grid || !block || n_params < 0 || (n_params > 0 && (!params || !param_sizes)))
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    if (kernel->spec.kind != Kind::Source)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled from caller-written source");
+    for (int i = 0; i < 3; i++)
+        if (grid[i] == 0 || block[i] == 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "grid and block dimensions must be positive");
+    if (static_cast<uint64_t>(block[0]) * block[1] * block[2] > 1024)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "more than 1024 threads per workgroup");
+    if (dev->capturing) {
+        RecNode node;
+        node.type = RecNode::Source;
+        node.k = kernel;
+        for (int i = 0; i < 3; i++) node.grid3[i] = grid[i], node.block3[i] = block[i];
+        node.shared_mem = shared_mem_bytes;
+        for (int i = 0; i < n_params; i++) {
+            const unsigned char* p = static_cast<const unsigned char*>(params[i]);
+            node.arg_values.emplace_back(p, p + param_sizes[i]);
+        }
+        dev->recorded.push_back(std::move(node));
+        return CUSTOS_HIP_OK;
+    }
+    std::vector<void*> args(params, params + n_params);
+    HIP_TRY(dev, hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                       shared_mem_bytes, dev->stream, args.data(), nullptr));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_source_launch1d(custos_hip_device* dev, custos_hip_kernel* kernel, size_t len,
+                                   void* const* params, const size_t* param_sizes, int32_t n_params) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel");
+    if (kernel->spec.kind != Kind::Source)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel was not compiled from caller-written source");
+    if (len == 0) return CUSTOS_HIP_OK;
+    // block size from the occupancy calculator, grid = ceil(len / block) (kernel_launch.rs:141-151)
+    int min_grid = 0, block_size = 0;
+    HIP_TRY(dev, hipModuleOccupancyMaxPotentialBlockSize(&min_grid, &block_size, kernel->fn, 0, 0));
+    if (block_size <= 0) block_size = 256;
+    const uint64_t blocks = (len + static_cast<size_t>(block_size) - 1) / static_cast<size_t>(block_size);
+    if (blocks > 0x7fffffffull) return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "more workgroups than a one-dimensional grid holds");
+    const uint32_t grid[3] = {static_cast<uint32_t>(blocks), 1, 1};
+    const uint32_t block[3] = {static_cast<uint32_t>(block_size), 1, 1};
+    return custos_hip_source_launch(dev, kernel, grid, block, 0, params, param_sizes, n_params);
+}
+
+}  // extern "C"

@@ -1,0 +1,121 @@
+// Internal declarations shared by the translation units of libcustos_hip.so:
+// the handle types behind the C ABI, error helpers, and the functions that
+// cross file boundaries.  Interface and reference citations: include/custos_hip.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/custos_hip.h"
+#include "expr.hpp"
+#include "kernel_gen.hpp"
+
+struct custos_hip_kernel {
+    custos_hip::KernelSpec spec;
+    hipModule_t module = nullptr;
+    hipFunction_t fn = nullptr;
+    hipFunction_t fn_batched = nullptr;
+};
+
+struct custos_hip_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    void* table = nullptr;    // operand address tables of the batched nodes (device memory)
+    size_t kernel_nodes = 0;  // kernel nodes in the instantiated graph
+    size_t recorded = 0;      // launches, clears and copies that were recorded
+    size_t levels = 0;        // dependency levels
+};
+
+// One recorded piece of work (while the device is recording, nothing is launched).
+struct Access {
+    uint64_t begin, end;
+    bool write;
+};
+struct RecNode {
+    enum Type { Kernel, Fill, Copy, Source } type = Kernel;
+    custos_hip_kernel* k = nullptr;
+    std::vector<uint64_t> ptrs;  // kernel: operand addresses in parameter order; fill: {ptr}; copy: {dst, src}
+    unsigned long long n = 0, head = 0, n_vec = 0, bytes = 0;
+    unsigned int grid = 1;
+    std::vector<Access> acc;
+    int level = 0;
+    // Source: launch shape and a copy of the argument values.  What such a kernel
+    // reads and writes is unknown, so it orders itself against everything.
+    unsigned int grid3[3] = {1, 1, 1}, block3[3] = {1, 1, 1}, shared_mem = 0;
+    std::vector<std::vector<unsigned char>> arg_values;
+};
+
+struct custos_hip_device {
+    int idx = 0;
+    hipStream_t stream = nullptr;    // compute stream: every launch, in call order
+    hipStream_t transfer = nullptr;  // copies that must not be recorded while capturing
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    hipDeviceProp_t props{};
+    std::string arch;
+    custos_hip::Tuning tuning;
+    bool capturing = false;          // recording: launches, clears and copies go to `recorded`
+    bool batching = true;            // merge equal independent launches of a level into one grid
+    std::vector<RecNode> recorded;
+    uint64_t compiles = 0, hits = 0, disk_hits = 0;
+    std::string last_error;
+    std::unordered_map<uint64_t, std::vector<std::unique_ptr<custos_hip_kernel>>> cache;
+    std::vector<custos_hip_graph*> graphs;
+};
+
+namespace custos_hip {
+
+// Stores the message for custos_hip_last_error (per device, or per thread when
+// there is no device) and returns `code`.
+int32_t set_error(custos_hip_device* dev, int32_t code, const std::string& msg);
+// The same for a failed HIP runtime call; clears the runtime's sticky error.
+int32_t hip_fail(custos_hip_device* dev, hipError_t e, const char* what);
+const std::string& thread_last_error();
+
+#define HIP_TRY(dev, call)                                   \
+    do {                                                     \
+        hipError_t e__ = (call);                             \
+        if (e__ != hipSuccess) return hip_fail(dev, e__, #call); \
+    } while (0)
+
+#define REQUIRE_DEV(dev)                                                                    \
+    do {                                                                                    \
+        if (!(dev)) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "device handle is null"); \
+        HIP_TRY(dev, hipSetDevice((dev)->idx));                                             \
+    } while (0)
+
+// An operand of a launch: device address and whether the kernel writes it.
+struct Range {
+    uint64_t ptr;
+    bool written;
+};
+
+// launch shape from the C struct; unset fields take the defaults
+inline Tuning tuning_from_c(const custos_hip_tuning* t) {
+    if (!t) return normalize_tuning(0, 0, 0, 0);
+    return normalize_tuning(t->block_threads, t->unroll, t->blocks_per_cu, t->nontemporal);
+}
+
+// device.hip
+unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec);
+int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream);
+void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph kernel nodes
+
+// jit.cpp
+int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec, const std::string& arch,
+                               std::vector<char>* code);
+int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k);
+
+// launch.cpp
+int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
+
+// graph.cpp
+int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g);
+void destroy_graph(custos_hip_graph* g);
+
+}  // namespace custos_hip
