@@ -4,7 +4,8 @@
 Default workload (BASELINE.json configs[1]): the fused unary chain
 y = relu(sin(x)*2.0 + 1.0) - 0.5 (five unary ops fused into one kernel) over
 f32 N = 2^28, x uniform in [-pi, pi) from seed 0.  One "step" is one launch of
-the fused kernel over the whole buffer, inputs resident in HBM.
+the fused kernel over the whole buffer (replayed as the one-node graph a `Lazy`
+run holds), inputs resident in HBM.
 
 Prints ONE JSON line: metric/value (GB/s on the algorithmic 8 B per element),
 the roofline of the fused kernel (HIP-event timed on the compute stream) and a
@@ -110,8 +111,16 @@ def bench_c2(dev, args):
     def fused_step():
         capi.check(lib.custos_hip_apply_fn(h, kernel, xb.ptr, out.ptr, n), h)
 
-    ms, wall_ms = time_steps(dev, fused_step, args.steps, args.warmup)
+    # One step = what `Lazy::run` does from the second run on: replay the graph that holds the
+    # fused kernel.  (The first run records and instantiates it; that is outside the timed region.)
+    dev.capture_begin()
+    fused_step()
+    graph = dev.capture_end()
+    assert graph.kernel_nodes == 1
+    ms, wall_ms = time_steps(dev, graph.launch, args.steps, args.warmup)
     per_launch_ms = ms / args.steps
+    dms, _ = time_steps(dev, fused_step, args.steps, args.warmup)   # the same kernel launched directly
+    direct_ms = dms / args.steps
     algo_bytes = 8.0 * n
     gbs = algo_bytes / (per_launch_ms * 1e-3) / 1e9
 
@@ -161,6 +170,7 @@ def bench_c2(dev, args):
         "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "elements_per_s": round(n / (per_launch_ms * 1e-3), 1),
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
+        "direct_launch": {"ms_per_step": round(direct_ms, 5), "GBps": round(algo_bytes / (direct_ms * 1e-3) / 1e9, 2)},
         "unfused": {
             "ms_per_step": round(unfused_ms, 5),
             "effective_GBps_on_8B_basis": round(algo_bytes / (unfused_ms * 1e-3) / 1e9, 2),
@@ -341,6 +351,8 @@ def bench_others(dev, args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--direct-replay", type=int, default=None,
+                    help="longest recorded chain replayed as plain launches (library default 4; 0 = always a hipGraph)")
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c2", choices=["c2"])
@@ -361,6 +373,8 @@ def main():
     import custos_amd
 
     dev = custos_amd.HIP(0)
+    if args.direct_replay is not None:
+        dev.set_graph_direct_replay(args.direct_replay)
     if args.block or args.unroll or args.blocks_per_cu or args.nontemporal:
         dev.set_tuning(args.block, args.unroll, args.blocks_per_cu, args.nontemporal)
     info = dev.info()

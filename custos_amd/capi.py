@@ -125,6 +125,7 @@ PROTOTYPES = {
     "custos_hip_graph_node_count": (C.c_int32, [_P, C.POINTER(C.c_size_t)]),
     "custos_hip_graph_stats": (C.c_int32, [_P, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "custos_hip_set_graph_batching": (C.c_int32, [_P, C.c_int32]),
+    "custos_hip_set_graph_direct_replay": (C.c_int32, [_P, C.c_int32]),
     "custos_hip_graph_destroy": (C.c_int32, [_P, _P]),
     "custos_hip_timer_begin": (C.c_int32, [_P]),
     "custos_hip_timer_end": (C.c_int32, [_P, C.POINTER(C.c_double)]),

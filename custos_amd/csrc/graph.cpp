@@ -121,9 +121,74 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
         HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
     }
 
+    // lower every planned node to function + shape + argument values
+    auto value = [](const void* p, size_t n) {
+        const unsigned char* c = static_cast<const unsigned char*>(p);
+        return std::vector<unsigned char>(c, c + n);
+    };
+    std::vector<std::vector<LoweredNode>> lowered(plan.size());
+    size_t total = 0;
+    bool chain = true;
+    for (int level = 0; level <= max_level; level++) {
+        for (const Planned& p : plan[level]) {
+            const RecNode& first = nodes[p.members[0]];
+            LoweredNode ln;
+            if (first.type == RecNode::Copy) {
+                ln.is_copy = true;
+                ln.dst = first.ptrs[0];
+                ln.src = first.ptrs[1];
+                ln.bytes = first.bytes;
+            } else if (first.type == RecNode::Source) {
+                ln.args = first.arg_values;
+                ln.func = reinterpret_cast<void*>(first.k->fn);
+                ln.grid = dim3(first.grid3[0], first.grid3[1], first.grid3[2]);
+                ln.block = dim3(first.block3[0], first.block3[1], first.block3[2]);
+                ln.shared_mem = first.shared_mem;
+            } else if (first.type == RecNode::Fill) {
+                const unsigned long long a0 = first.bytes, a1 = first.head, a2 = first.n_vec;
+                ln.args = {value(&first.ptrs[0], 8), value(&a0, 8), value(&a1, 8), value(&a2, 8)};
+                ln.func = fill_zero_kernel();
+                ln.module_fn = false;
+                ln.grid = dim3(fill_grid(dev, first.n_vec));
+                ln.block = dim3(256);
+            } else if (p.members.size() == 1) {
+                for (uint64_t ptr : first.ptrs) ln.args.push_back(value(&ptr, 8));
+                const unsigned long long a0 = first.n, a1 = first.head, a2 = first.n_vec;
+                ln.args.push_back(value(&a0, 8));
+                ln.args.push_back(value(&a1, 8));
+                ln.args.push_back(value(&a2, 8));
+                ln.func = reinterpret_cast<void*>(first.k->fn);
+                ln.grid = dim3(first.grid);
+                ln.block = dim3(static_cast<unsigned int>(first.k->spec.tuning.block_threads));
+            } else {
+                const Tuning& t = first.k->spec.tuning;
+                const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+                const unsigned long long tiles_per_seg = std::max(1ull, (first.n_vec + tile_vecs - 1) / tile_vecs);
+                const unsigned long long blocks = tiles_per_seg * p.members.size();
+                if (blocks > (1ull << 31) - 1)
+                    return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a batched launch would need more than 2^31 workgroups");
+                const uint64_t table = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
+                const unsigned long long a0 = first.n, a1 = first.n_vec;
+                ln.args = {value(&table, 8), value(&a0, 8), value(&a1, 8), value(&tiles_per_seg, 8)};
+                ln.func = reinterpret_cast<void*>(first.k->fn_batched);
+                ln.grid = dim3(static_cast<unsigned int>(blocks));
+                ln.block = dim3(static_cast<unsigned int>(t.block_threads));
+            }
+            if (!ln.is_copy) g->kernel_nodes++;
+            lowered[level].push_back(std::move(ln));
+            total++;
+        }
+        chain = chain && lowered[level].size() == 1;
+    }
+
+    if (chain && total <= dev->direct_replay_max) {
+        for (auto& level : lowered) g->direct.push_back(std::move(level[0]));
+        return CUSTOS_HIP_OK;
+    }
+
     HIP_TRY(dev, hipGraphCreate(&g->graph, 0));
     std::vector<hipGraphNode_t> prev;  // what the nodes of the current level wait for
-    for (int level = 0; level <= max_level; level++) {
+    for (auto& level : lowered) {
         std::vector<hipGraphNode_t> deps = prev;
         if (deps.size() > 1) {  // one join node instead of |prev| x |level| edges
             hipGraphNode_t join;
@@ -131,70 +196,53 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
             deps = {join};
         }
         std::vector<hipGraphNode_t> made;
-        for (const Planned& p : plan[level]) {
-            const RecNode& first = nodes[p.members[0]];
+        for (LoweredNode& ln : level) {
             hipGraphNode_t node;
-            if (first.type == RecNode::Copy) {
+            if (ln.is_copy) {
                 HIP_TRY(dev, hipGraphAddMemcpyNode1D(&node, g->graph, deps.data(), deps.size(),
-                                                     reinterpret_cast<void*>(first.ptrs[0]),
-                                                     reinterpret_cast<const void*>(first.ptrs[1]), first.bytes,
+                                                     reinterpret_cast<void*>(ln.dst),
+                                                     reinterpret_cast<const void*>(ln.src), ln.bytes,
                                                      hipMemcpyDeviceToDevice));
-                made.push_back(node);
-                continue;
-            }
-            hipKernelNodeParams kp{};
-            kp.sharedMemBytes = 0;
-            kp.extra = nullptr;
-            std::vector<void*> args;
-            uint64_t ptrs[8];
-            unsigned long long a0, a1, a2, a3;
-            if (first.type == RecNode::Source) {
-                for (const auto& v : first.arg_values) args.push_back(const_cast<unsigned char*>(v.data()));
-                kp.func = reinterpret_cast<void*>(first.k->fn);
-                kp.gridDim = dim3(first.grid3[0], first.grid3[1], first.grid3[2]);
-                kp.blockDim = dim3(first.block3[0], first.block3[1], first.block3[2]);
-                kp.sharedMemBytes = first.shared_mem;
-            } else if (first.type == RecNode::Fill) {
-                ptrs[0] = first.ptrs[0];
-                a0 = first.bytes, a1 = first.head, a2 = first.n_vec;
-                args = {&ptrs[0], &a0, &a1, &a2};
-                kp.func = fill_zero_kernel();
-                kp.gridDim = dim3(fill_grid(dev, first.n_vec));
-                kp.blockDim = dim3(256);
-            } else if (p.members.size() == 1) {
-                for (size_t i = 0; i < first.ptrs.size(); i++) {
-                    ptrs[i] = first.ptrs[i];
-                    args.push_back(&ptrs[i]);
-                }
-                a0 = first.n, a1 = first.head, a2 = first.n_vec;
-                args.push_back(&a0);
-                args.push_back(&a1);
-                args.push_back(&a2);
-                kp.func = reinterpret_cast<void*>(first.k->fn);
-                kp.gridDim = dim3(first.grid);
-                kp.blockDim = dim3(static_cast<unsigned int>(first.k->spec.tuning.block_threads));
             } else {
-                const Tuning& t = first.k->spec.tuning;
-                const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
-                a3 = std::max(1ull, (first.n_vec + tile_vecs - 1) / tile_vecs);  // tiles per segment
-                const unsigned long long blocks = a3 * p.members.size();
-                if (blocks > (1ull << 31) - 1)
-                    return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a batched launch would need more than 2^31 workgroups");
-                ptrs[0] = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
-                a0 = first.n, a1 = first.n_vec;
-                args = {&ptrs[0], &a0, &a1, &a3};
-                kp.func = reinterpret_cast<void*>(first.k->fn_batched);
-                kp.gridDim = dim3(static_cast<unsigned int>(blocks));
-                kp.blockDim = dim3(static_cast<unsigned int>(t.block_threads));
+                std::vector<void*> args;
+                for (auto& v : ln.args) args.push_back(v.data());
+                hipKernelNodeParams kp{};
+                kp.func = ln.func;
+                kp.gridDim = ln.grid;
+                kp.blockDim = ln.block;
+                kp.sharedMemBytes = ln.shared_mem;
+                kp.kernelParams = args.data();
+                kp.extra = nullptr;
+                HIP_TRY(dev, hipGraphAddKernelNode(&node, g->graph, deps.data(), deps.size(), &kp));
             }
-            kp.kernelParams = args.data();
-            HIP_TRY(dev, hipGraphAddKernelNode(&node, g->graph, deps.data(), deps.size(), &kp));
-            g->kernel_nodes++;
             made.push_back(node);
         }
         prev = std::move(made);
     }
     HIP_TRY(dev, hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
+    if (g->exec) {
+        HIP_TRY(dev, hipGraphLaunch(g->exec, dev->stream));
+        return CUSTOS_HIP_OK;
+    }
+    for (LoweredNode& ln : g->direct) {
+        if (ln.is_copy) {
+            HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(ln.dst), reinterpret_cast<const void*>(ln.src), ln.bytes,
+                                        hipMemcpyDeviceToDevice, dev->stream));
+            continue;
+        }
+        std::vector<void*> argv(ln.args.size());
+        for (size_t i = 0; i < ln.args.size(); i++) argv[i] = ln.args[i].data();
+        void** args = argv.data();
+        if (ln.module_fn)
+            HIP_TRY(dev, hipModuleLaunchKernel(static_cast<hipFunction_t>(ln.func), ln.grid.x, ln.grid.y, ln.grid.z,
+                                               ln.block.x, ln.block.y, ln.block.z, ln.shared_mem, dev->stream, args, nullptr));
+        else
+            HIP_TRY(dev, hipLaunchKernel(ln.func, ln.grid, ln.block, args, ln.shared_mem, dev->stream));
+    }
     return CUSTOS_HIP_OK;
 }
 
@@ -249,6 +297,13 @@ int32_t custos_hip_set_graph_batching(custos_hip_device* dev, int32_t enabled) {
     return CUSTOS_HIP_OK;
 }
 
+int32_t custos_hip_set_graph_direct_replay(custos_hip_device* dev, int32_t max_nodes) {
+    REQUIRE_DEV(dev);
+    if (max_nodes < 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "max_nodes is negative");
+    dev->direct_replay_max = static_cast<size_t>(max_nodes);
+    return CUSTOS_HIP_OK;
+}
+
 int32_t custos_hip_is_capturing(custos_hip_device* dev, int32_t* capturing) {
     REQUIRE_DEV(dev);
     if (!capturing) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "capturing is null");
@@ -260,8 +315,7 @@ int32_t custos_hip_graph_launch(custos_hip_device* dev, custos_hip_graph* graph)
     REQUIRE_DEV(dev);
     if (!graph) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph is null");
     if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot replay while recording");
-    HIP_TRY(dev, hipGraphLaunch(graph->exec, dev->stream));
-    return CUSTOS_HIP_OK;
+    return replay_graph(dev, graph);
 }
 
 int32_t custos_hip_graph_node_count(custos_hip_graph* graph, size_t* kernel_nodes) {

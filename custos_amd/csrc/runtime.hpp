@@ -23,7 +23,24 @@ struct custos_hip_kernel {
     hipFunction_t fn_batched = nullptr;
 };
 
+// A graph node in launchable form: function, shape and a copy of the argument values.
+struct LoweredNode {
+    bool is_copy = false;
+    uint64_t dst = 0, src = 0;  // copy
+    size_t bytes = 0;
+    void* func = nullptr;       // kernel: hipFunction_t of a module, or the host handle of a library kernel
+    bool module_fn = true;
+    dim3 grid{1, 1, 1}, block{1, 1, 1};
+    unsigned int shared_mem = 0;
+    std::vector<std::vector<unsigned char>> args;
+};
+
 struct custos_hip_graph {
+    // A short chain (every level one node, at most direct_replay_max nodes) is
+    // replayed by issuing its nodes on the compute stream: stream order is exactly
+    // its dependency order, and a handful of launches cost less than a graph launch.
+    // Everything else is an instantiated hipGraph.
+    std::vector<LoweredNode> direct;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     void* table = nullptr;    // operand address tables of the batched nodes (device memory)
@@ -60,6 +77,7 @@ struct custos_hip_device {
     std::string arch;
     custos_hip::Tuning tuning;
     bool capturing = false;          // recording: launches, clears and copies go to `recorded`
+    size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     bool batching = true;            // merge equal independent launches of a level into one grid
     std::vector<RecNode> recorded;
     uint64_t compiles = 0, hits = 0, disk_hits = 0;
@@ -115,6 +133,7 @@ int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k);
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
 
 // graph.cpp
+int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g);
 int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g);
 void destroy_graph(custos_hip_graph* g);
 

@@ -288,6 +288,9 @@ class HIP:
     def set_graph_batching(self, enabled: bool) -> None:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 
+    def set_graph_direct_replay(self, max_nodes: int) -> None:
+        self._check(self.lib.custos_hip_set_graph_direct_replay(self.handle, max_nodes))
+
     def is_capturing(self) -> bool:
         v = C.c_int32(0)
         self._check(self.lib.custos_hip_is_capturing(self.handle, C.byref(v)))

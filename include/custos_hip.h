@@ -253,6 +253,11 @@ int32_t custos_hip_capture_end(custos_hip_device *dev, custos_hip_graph **graph)
 /* Switches the merging of equal independent launches off (0) or on (default):
  * with it off every recorded launch becomes its own kernel node. */
 int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
+/* A recording that comes out as a plain chain (every dependency level one node) of at
+ * most `max_nodes` nodes is replayed by issuing its nodes on the compute stream instead
+ * of launching an instantiated graph: for a handful of launches that is cheaper than a
+ * graph launch. Default 4; 0 always instantiates a graph. Applies to later capture_end calls. */
+int32_t custos_hip_set_graph_direct_replay(custos_hip_device *dev, int32_t max_nodes);
 int32_t custos_hip_is_capturing(custos_hip_device *dev, int32_t *capturing);
 /* LazyCudaGraph::launch on the compute stream (no wait; call custos_hip_sync). */
 int32_t custos_hip_graph_launch(custos_hip_device *dev, custos_hip_graph *graph);

@@ -223,3 +223,34 @@ def test_recorded_copy_nodes(hip):
     g.launch()
     hip.sync()
     assert_bits_equal(a.read(), (x * np.float32(4.0)).astype(np.float32))
+
+
+@pytest.mark.parametrize("direct_max", [0, 1, 4])
+def test_short_chain_replays_the_same_as_a_graph_or_as_plain_launches(hip, oracle, direct_max):
+    # A chain of at most `direct_max` nodes is replayed as plain launches on the compute
+    # stream, anything else as an instantiated graph: same results either way, replay after replay.
+    n = 70001
+    x = synth.uniform_f32(11, n, -2, 2)
+    a, b, c = hip.buffer(x), hip.alloc(n), hip.alloc(n)
+    scale = """extern "C" __global__ void scale3(float* p, unsigned long long n) {
+        unsigned long long i = blockIdx.x * (unsigned long long)blockDim.x + threadIdx.x;
+        if (i < n) p[i] = p[i] * 3.0f;
+    }"""
+    hip.set_graph_direct_replay(direct_max)
+    try:
+        hip.capture_begin()
+        b.clear()
+        hip.apply_fn(a, lambda v: v.mul(2.0).add(1.0), out=b)
+        hip.copy(c, b)
+        hip.launch_kernel(scale, "scale3", ((n + 255) // 256, 1, 1), (256, 1, 1), 0, [c, np.uint64(n)])
+        g = hip.capture_end()
+    finally:
+        hip.set_graph_direct_replay(4)
+    assert g.stats() == (4, 3, 4)
+    want = oracle.apply_fn(lambda v: v.mul(2.0).add(1.0), x) * np.float32(3.0)
+    for replay in range(3):
+        c.clear()
+        g.launch()
+        hip.sync()
+        assert_bits_equal(c.read(), want, f"direct_max={direct_max} replay {replay}")
+    g.destroy()
