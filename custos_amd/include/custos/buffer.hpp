@@ -59,6 +59,8 @@ class Buffer {
 
     // A non-owning copy of the handle (`ShallowCopy`).
     Buffer shallow() const { return from_parts(device_, ptr_, len_, id_, flag_ == AllocFlag::Lazy ? AllocFlag::Lazy : AllocFlag::Wrapper, requires_grad_); }
+    // `PtrType::set_flag` (src/devices/cuda/cuda_ptr.rs:51-61): who frees the memory.
+    void set_flag(AllocFlag flag) { flag_ = flag; }
 
     // `Read::read`: device -> host.
     std::vector<T> read() const { return device_->read(*this); }
@@ -125,6 +127,8 @@ class Buffer {
         if (device_ && flag_ == AllocFlag::None && ptr_ != 0) {
             device_->modules.on_drop_buffer(id_);
             device_->free_raw(ptr_);
+        } else if (device_ && flag_ == AllocFlag::Cached && ptr_ != 0) {
+            device_->modules.on_release_cached(ptr_);
         }
         device_ = nullptr;
         ptr_ = 0;

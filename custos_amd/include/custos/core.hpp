@@ -29,6 +29,7 @@ enum class DeviceError {
     DuplicateParent,         // "each parent (id) must be unique" (lazy_graph.rs:121-123)
     IdCollision,             // "IDs collided!" (src/modules/lazy.rs:354-357)
     TypeMismatch,            // a recorded buffer is used with another element type
+    CachedInUse,             // a cached allocation is replaced while a buffer handle still uses it
     Backend,                 // the device library reported an error (code in Error::code)
 };
 
@@ -44,6 +45,7 @@ inline const char* device_error_str(DeviceError e) {
         case DeviceError::DuplicateParent: return "each parent (id) must be unique";
         case DeviceError::IdCollision: return "IDs collided! Maybe a device address already occupies this id.";
         case DeviceError::TypeMismatch: return "Type data does not match";
+        case DeviceError::CachedInUse: return "A cached allocation is still in use by a buffer";
         case DeviceError::Backend: return "device library error";
     }
     return "";
@@ -71,6 +73,7 @@ enum class AllocFlag {
     None,     // the holder owns the allocation
     Wrapper,  // a shallow copy: never frees (src/flag.rs:24-26)
     Lazy,     // an id without memory yet
+    Cached,   // memory kept by a Cached module; the handle only reports its drop (src/flag.rs:14-16)
 };
 
 // Type-erased shallow copy of a buffer, what modules keep per id

@@ -200,6 +200,51 @@ class Device {
     // Fuses element-wise operations of any arity (unary chains included); needs `Graph`.
     void elementwise_fusing() { modules.elementwise_fusing(self(), nullptr, {}); }
 
+    // ---- cursor (src/features.rs:68-109, src/range.rs:9-62) ----
+
+    // `for epoch in device.range(begin..end)`: every epoch starts with the cursor
+    // where it was when the loop began, so the n-th retrieve of an epoch finds what
+    // the n-th retrieve of the epoch before allocated (with a `Cached` module).
+    class CursorRange {
+       public:
+        class Iter {
+           public:
+            Iter(Derived* dev, size_t at, size_t previous) : dev_(dev), at_(at), previous_(previous) {}
+            size_t operator*() const {
+                dev_->modules.set_cursor(previous_);
+                return at_;
+            }
+            Iter& operator++() {
+                at_++;
+                return *this;
+            }
+            bool operator!=(const Iter& o) const { return at_ < o.at_; }
+
+           private:
+            Derived* dev_;
+            size_t at_, previous_;
+        };
+        CursorRange(Derived* dev, size_t begin, size_t end) : dev_(dev), begin_(begin), end_(end), previous_(dev->modules.cursor()) {}
+        Iter begin() const { return Iter(dev_, begin_, previous_); }
+        Iter end() const { return Iter(dev_, end_, previous_); }
+
+       private:
+        Derived* dev_;
+        size_t begin_, end_, previous_;
+    };
+    CursorRange range(size_t begin, size_t end) { return CursorRange(&self(), begin, end); }
+    CursorRange range(size_t end) { return CursorRange(&self(), 0, end); }
+    size_t cursor() const { return modules.cursor(); }
+    void set_cursor(size_t c) { modules.set_cursor(c); }
+    // `device.cached(|| ...)`: runs `cb` and rewinds the cursor, so that the next call
+    // retrieves the same allocations again (src/features.rs:101-109).
+    template <class F>
+    void cached(F cb) {
+        const size_t previous = modules.cursor();
+        cb();
+        modules.set_cursor(previous);
+    }
+
     // ---- autograd ----
 
     // Gradient buffer of `id`, allocated zeroed on first use (autograd/gradients.rs:90-126).

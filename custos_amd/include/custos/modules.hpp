@@ -1,7 +1,7 @@
-// The module stack: Base, Lazy, Graph, Autograd.
+// The module stack: Base, Cached, Lazy, Graph, Autograd.
 //
 // Modules compose at compile time, `HIP<Autograd<Graph<Lazy<Base>>>>`, like the
-// reference's (src/modules/{base,lazy,graph,autograd}.rs).  Every module
+// reference's (src/modules/{base,cached,lazy,graph,autograd}.rs).  Every module
 // implements the same set of "features" and passes what it does not handle to
 // the module it wraps (`modules`), as the reference does with its pass-down
 // macros in src/features.rs.
@@ -86,6 +86,7 @@ struct Base {
     template <class T, class D>
     void on_new_buffer(D&, const Buffer<T, D>&) {}
     void on_drop_buffer(Id) {}
+    void on_release_cached(uint64_t) {}
 
     // Base never records (base.rs:53-62): the device calls the closure directly.
     template <class D>
@@ -177,6 +178,7 @@ struct Lazy {
         }
         modules.on_drop_buffer(id);
     }
+    void on_release_cached(uint64_t ptr) { modules.on_release_cached(ptr); }
 
     template <class D>
     void add_op(D& dev, Operation&& op) {
@@ -553,6 +555,161 @@ struct Lazy {
 };
 
 // ---------------------------------------------------------------------------
+// Cached: the n-th retrieve of an epoch returns the allocation the n-th
+// retrieve of the previous epoch made (src/modules/cached.rs:22-255).
+// ---------------------------------------------------------------------------
+// The key is the cursor, which counts retrieves and which the caller rewinds
+// with `device.range(..)` at the start of every epoch (src/range.rs:9-62).  The
+// module owns the allocations; a retrieved buffer is a handle with
+// `AllocFlag::Cached` that reports its drop, so that the module knows which
+// allocations are in use.  `optimize_mem_graph` lets all buffers of a cache
+// trace share the allocation of the trace's first buffer (cached.rs:415-446)
+// and frees the ones they had.
+template <class Mods>
+struct Cached {
+    Mods modules;
+
+    template <class D>
+    void setup(D& dev) {
+        modules.setup(dev);
+    }
+    template <class D>
+    void teardown(D& dev) {
+        std::unordered_set<uint64_t> freed;
+        for (auto& kv : cache_)
+            if (kv.second.ptr && freed.insert(kv.second.ptr).second) dev.free_raw(kv.second.ptr);
+        cache_.clear();
+        live_.clear();
+        modules.teardown(dev);
+    }
+
+    template <class U, class D>
+    Buffer<U, D> retrieve(D& dev, size_t len, const std::vector<Id>& parents, const std::vector<bool>& rg) {
+        const UniqueId key = static_cast<UniqueId>(cursor_);
+        auto it = cache_.find(key);
+        if (it == cache_.end()) {
+            Buffer<U, D> fresh = modules.template retrieve<U>(dev, len, parents, rg);
+            fresh.set_flag(AllocFlag::Cached);  // cached.rs:203: the module frees it, not the handle
+            it = cache_.emplace(key, AnyBuf{fresh.ptr(), len, std::type_index(typeid(U)), true, sizeof(U)}).first;
+            live_[fresh.ptr()]++;
+            cursor_++;
+            return fresh;
+        }
+        // The reference keys its default cache by the cursor alone and trusts the
+        // caller to repeat the same sequence of retrieves; here a retrieve that
+        // does not fit what the cursor position holds is an error.
+        if (it->second.type != std::type_index(typeid(U))) throw Error(DeviceError::TypeMismatch);
+        if (it->second.len != len) throw Error(DeviceError::ShapeLengthMismatch);
+        cursor_++;
+        live_[it->second.ptr]++;
+        return Buffer<U, D>::from_parts(&dev, it->second.ptr, len, Id{it->second.ptr, len}, AllocFlag::Cached);
+    }
+
+    template <class U, class D>
+    void on_new_buffer(D& dev, const Buffer<U, D>& b) {
+        modules.on_new_buffer(dev, b);
+    }
+    void on_drop_buffer(Id id) { modules.on_drop_buffer(id); }
+    void on_release_cached(uint64_t ptr) {
+        auto it = live_.find(ptr);
+        if (it != live_.end() && it->second > 0) it->second--;
+    }
+
+    template <class D>
+    void add_op(D& dev, Operation&& op) {
+        modules.add_op(dev, std::move(op));
+    }
+    size_t ops_count() const { return modules.ops_count(); }
+    void set_lazy_enabled(bool e) { modules.set_lazy_enabled(e); }
+    bool is_lazy_enabled() const { return modules.is_lazy_enabled(); }
+    void set_op_hint(AnyOpHint h) { modules.set_op_hint(std::move(h)); }
+    void set_expr_hint(AnyExprHint h) { modules.set_expr_hint(std::move(h)); }
+    template <class D>
+    void exec_now(D& dev, size_t b, size_t e) {
+        modules.exec_now(dev, b, e);
+    }
+    template <class D>
+    void run(D& dev) {
+        modules.run(dev);
+    }
+    template <class U, class D>
+    Buffer<U, D> replace_buf(D& dev, const Buffer<U, D>& b) {
+        return modules.template replace_buf<U>(dev, b);
+    }
+    void set_checkpoint_buffer(Id id) { modules.set_checkpoint_buffer(id); }
+
+    // cached.rs:415-446, on cursor positions instead of node indices
+    // (graph_translator.rs:45-57).  Buffers of another element type or length keep
+    // their own allocation.  Fails if a handle to an allocation that would be
+    // replaced is still alive.
+    template <class D>
+    void optimize_mem_graph(D& dev, const GraphTranslator* gt) {
+        if (!gt) throw Error(DeviceError::MissingCacheTraces);
+        const std::vector<CacheTrace> traces = gt->to_cursor_cache_traces(gt->opt_graph.cache_traces());
+        for (const CacheTrace& t : traces) {
+            auto head = cache_.find(static_cast<UniqueId>(t.cache_idx));
+            if (head == cache_.end()) throw Error(DeviceError::GraphOptimization);
+            for (size_t use : t.use_cache_idxs) {
+                auto u = cache_.find(static_cast<UniqueId>(use));
+                if (u == cache_.end()) throw Error(DeviceError::GraphOptimization);
+                if (u->second.ptr == head->second.ptr) continue;
+                if (u->second.type != head->second.type || u->second.len != head->second.len) continue;
+                if (live_[u->second.ptr] > 0) throw Error(DeviceError::CachedInUse);
+            }
+        }
+        for (const CacheTrace& t : traces) {
+            const AnyBuf shared = cache_.at(static_cast<UniqueId>(t.cache_idx));
+            for (size_t use : t.use_cache_idxs) {
+                AnyBuf& u = cache_.at(static_cast<UniqueId>(use));
+                if (u.ptr == shared.ptr || u.type != shared.type || u.len != shared.len) continue;
+                const uint64_t old = u.ptr;
+                u = shared;
+                bool still_used = false;
+                for (const auto& kv : cache_) still_used = still_used || kv.second.ptr == old;
+                if (!still_used) {
+                    dev.free_raw(old);
+                    live_.erase(old);
+                }
+            }
+        }
+        modules.optimize_mem_graph(dev, gt);
+    }
+    // cached.rs:448-455
+    template <class D>
+    void unary_fusing(D&, const GraphTranslator*) {
+        throw Error(DeviceError::UnaryFusingUnsupported);
+    }
+    template <class D>
+    void elementwise_fusing(D&, const GraphTranslator*, const std::vector<UniqueId>&) {
+        throw Error(DeviceError::UnaryFusingUnsupported);
+    }
+
+    void add_grad_fn(Operation&& op) { modules.add_grad_fn(std::move(op)); }
+    void set_grad_enabled(bool e) { modules.set_grad_enabled(e); }
+    bool is_grad_enabled() const { return modules.is_grad_enabled(); }
+    AutogradState* autograd() { return modules.autograd(); }
+    void set_requires_grad(Id id, bool v) { modules.set_requires_grad(id, v); }
+    bool requires_grad_of(Id id) const { return modules.requires_grad_of(id); }
+
+    // cached.rs:257-267: the module has a cursor of its own
+    size_t cursor() const { return cursor_; }
+    void set_cursor(size_t c) { cursor_ = c; }
+    Buffers* buffers() { return modules.buffers(); }
+    uint64_t lazy_version() const { return modules.lazy_version(); }
+
+    size_t cached_allocations() const {
+        std::unordered_set<uint64_t> distinct;
+        for (const auto& kv : cache_) distinct.insert(kv.second.ptr);
+        return distinct.size();
+    }
+
+   private:
+    std::unordered_map<UniqueId, AnyBuf> cache_;   // cursor position -> allocation
+    std::unordered_map<uint64_t, size_t> live_;    // address -> handles given out and not dropped yet
+    size_t cursor_ = 0;
+};
+
+// ---------------------------------------------------------------------------
 // Graph: dependency DAG built at every retrieve (src/modules/graph.rs)
 // ---------------------------------------------------------------------------
 template <class Mods, class T = float>
@@ -591,6 +748,7 @@ struct Graph {
         modules.on_new_buffer(dev, b);
     }
     void on_drop_buffer(Id id) { modules.on_drop_buffer(id); }
+    void on_release_cached(uint64_t ptr) { modules.on_release_cached(ptr); }
 
     template <class D>
     void add_op(D& dev, Operation&& op) {
@@ -699,6 +857,7 @@ struct Autograd {
         state.no_grads_pool.erase(id.id);
         modules.on_drop_buffer(id);
     }
+    void on_release_cached(uint64_t ptr) { modules.on_release_cached(ptr); }
 
     template <class D>
     void add_op(D& dev, Operation&& op) {

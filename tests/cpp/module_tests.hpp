@@ -706,6 +706,147 @@ void elementwise_fuse_random_programs() {
     }
 }
 
+// ---- Cached ----
+
+// tests/cache.rs:24-45 (test_caching_cpu)
+template <template <class> class DEV>
+void cached_same_allocation_every_epoch() {
+    DEV<Cached<Base>> device;
+    uint64_t old_ptr = 0;
+    for (size_t epoch : device.range(0, 100)) {
+        (void)epoch;
+        auto out = device.template retrieve<float>(10);
+        CHECK(old_ptr == 0 || out.ptr() == old_ptr);
+        CHECK(out.flag() == AllocFlag::Cached);
+        old_ptr = out.ptr();
+    }
+    CHECK_EQ(device.modules.cached_allocations(), size_t(1));
+    // outside a range the cursor keeps counting: a new position, a new allocation
+    auto next = device.template retrieve<float>(10);
+    CHECK(next.ptr() != old_ptr);
+    CHECK_EQ(device.modules.cached_allocations(), size_t(2));
+}
+
+// src/modules/cached.rs:544-569 (test_multi_level_retrieve): five retrieves, five positions
+template <template <class> class DEV>
+void cached_multi_level_retrieve() {
+    DEV<Cached<Base>> device;
+    std::vector<uint64_t> first;
+    for (size_t epoch : device.range(0, 3)) {
+        std::vector<uint64_t> ptrs;
+        auto a = device.template retrieve<float>(10);
+        ptrs.push_back(a.ptr());
+        for (int i = 0; i < 3; i++) {
+            auto b = device.template retrieve<float>(20);
+            CHECK_EQ(b.len(), size_t(20));
+            ptrs.push_back(b.ptr());
+        }
+        if (epoch == 0) {
+            first = ptrs;
+            for (size_t i = 0; i < ptrs.size(); i++)
+                for (size_t j = i + 1; j < ptrs.size(); j++) CHECK(ptrs[i] != ptrs[j]);
+        } else {
+            CHECK(ptrs == first);
+        }
+    }
+    CHECK_EQ(device.modules.cached_allocations(), size_t(4));
+}
+
+// src/modules/cached.rs:572-602 (test_add_cached_layer): operations on a cached device
+template <template <class> class DEV>
+void cached_apply_fn_and_unary_ew() {
+    DEV<Cached<Base>> device;
+    auto base = device.template buffer<float>({1.f, 2.f, 3.f, 4.f});
+    uint64_t first = 0;
+    for (size_t epoch : device.range(0, 10)) {
+        auto y = device.apply_fn(base, [](auto x) { return x.mul(2.f).add(1.f); });
+        CHECK_VEC_EQ(y.read(), (std::vector<float>{3.f, 5.f, 7.f, 9.f}));
+        if (epoch == 0) first = y.ptr();
+        CHECK_EQ(y.ptr(), first);
+        auto z = device.unary_ew(base, [](auto x) { return x.neg(); }, [](auto x) { return x.mul(0.f).sub(1.f); });
+        CHECK_VEC_EQ(z.read(), (std::vector<float>{-1.f, -2.f, -3.f, -4.f}));
+        CHECK(z.ptr() != y.ptr());
+    }
+    CHECK_EQ(device.modules.cached_allocations(), size_t(2));
+    // `device.cached(|| ..)` (src/features.rs:101-109): the closure's retrieves are replayed
+    uint64_t in_closure = 0;
+    for (int i = 0; i < 3; i++)
+        device.cached([&] {
+            auto w = device.apply_fn(base, [](auto x) { return x.add(1.f); });
+            CHECK(in_closure == 0 || w.ptr() == in_closure);
+            in_closure = w.ptr();
+            CHECK_VEC_EQ(w.read(), (std::vector<float>{2.f, 3.f, 4.f, 5.f}));
+        });
+    CHECK_EQ(device.modules.cached_allocations(), size_t(3));
+}
+
+// tests/graph/graph.rs:10-41 (test_graph) and :78-108 (test_graph_cu): after
+// `optimize_mem_graph` the three results of the chain share one allocation
+template <template <class> class DEV>
+void cached_graph_optimize_aliases() {
+    DEV<Graph<Cached<Base>>> device;
+    auto a = device.template buffer<int>({1, 2, 3, 4, 5, 6});
+    auto b = device.template buffer<int>({2, 3, 1, 4, 0, 5});
+    const size_t live_before = device.modules.modules.cached_allocations();
+    CHECK_EQ(live_before, size_t(0));
+    for (size_t epoch : device.range(0, 3)) {
+        {
+            auto c = device.apply_fn2(a, b, [](auto x, auto y) { return x.add(y); });
+            CHECK_VEC_EQ(c.read(), (std::vector<int>{3, 5, 4, 8, 5, 11}));
+            auto d = device.apply_fn(c, [](auto x) { return x.max(0); });
+            CHECK_VEC_EQ(d.read(), (std::vector<int>{3, 5, 4, 8, 5, 11}));
+            auto e = device.apply_fn2(d, b, [](auto x, auto y) { return x.add(y); });
+            CHECK_VEC_EQ(e.read(), (std::vector<int>{5, 8, 5, 12, 5, 16}));
+            if (epoch >= 1) {
+                CHECK_EQ(c.ptr(), d.ptr());
+                CHECK_EQ(c.ptr(), e.ptr());
+            } else {
+                CHECK(c.ptr() != d.ptr());
+                // replacing allocations that handles still use is refused
+                CHECK_THROWS_KIND(device.optimize_mem_graph(), DeviceError::CachedInUse);
+            }
+        }
+        device.optimize_mem_graph();
+        CHECK_EQ(device.modules.modules.cached_allocations(), size_t(1));
+    }
+    CHECK_VEC_EQ(a.read(), (std::vector<int>{1, 2, 3, 4, 5, 6}));
+    CHECK_VEC_EQ(b.read(), (std::vector<int>{2, 3, 1, 4, 0, 5}));
+}
+
+template <template <class> class DEV>
+void cached_errors() {
+    {
+        DEV<Cached<Base>> device;
+        for (size_t epoch : device.range(0, 2)) {
+            if (epoch == 0) {
+                auto x = device.template retrieve<float>(8);
+            } else {
+                // the same cursor position asked for another element type or length
+                CHECK_THROWS_KIND(device.template retrieve<int>(8), DeviceError::TypeMismatch);
+                CHECK_THROWS_KIND(device.template retrieve<float>(9), DeviceError::ShapeLengthMismatch);
+                auto x = device.template retrieve<float>(8);
+                CHECK_EQ(x.len(), size_t(8));
+            }
+        }
+        // src/modules/cached.rs:448-455; no Graph module, no cache traces
+        CHECK_THROWS_KIND(device.unary_fusing(), DeviceError::UnaryFusingUnsupported);
+        CHECK_THROWS_KIND(device.optimize_mem_graph(), DeviceError::MissingCacheTraces);
+    }
+    {
+        // buffers of another type in a trace keep their allocation (cached.rs:430-441)
+        DEV<Graph<Cached<Base>>> device;
+        auto a = device.template buffer<float>({1.f, 2.f});
+        {
+            auto c = device.template retrieve<float>(2, a);
+            auto d = device.template retrieve<int>(2, c);
+            auto e = device.template retrieve<float>(2, d);
+            (void)e;
+        }
+        device.optimize_mem_graph();
+        CHECK_EQ(device.modules.modules.cached_allocations(), size_t(2));
+    }
+}
+
 }  // namespace module_tests
 
 // Registers every generic case for one device template.
@@ -744,4 +885,9 @@ void elementwise_fuse_random_programs() {
     TEST_CASE(elementwise_fuse_binary_then_unary) { module_tests::elementwise_fuse_binary_then_unary<DEV>(); } \
     TEST_CASE(elementwise_fuse_respects_limits) { module_tests::elementwise_fuse_respects_limits<DEV>(); } \
     TEST_CASE(elementwise_fuse_keeps_tape_buffers) { module_tests::elementwise_fuse_keeps_tape_buffers<DEV>(TOL); } \
-    TEST_CASE(elementwise_fuse_random_programs) { module_tests::elementwise_fuse_random_programs<DEV>(); }
+    TEST_CASE(elementwise_fuse_random_programs) { module_tests::elementwise_fuse_random_programs<DEV>(); } \
+    TEST_CASE(cached_same_allocation_every_epoch) { module_tests::cached_same_allocation_every_epoch<DEV>(); } \
+    TEST_CASE(cached_multi_level_retrieve) { module_tests::cached_multi_level_retrieve<DEV>(); }  \
+    TEST_CASE(cached_apply_fn_and_unary_ew) { module_tests::cached_apply_fn_and_unary_ew<DEV>(); } \
+    TEST_CASE(cached_graph_optimize_aliases) { module_tests::cached_graph_optimize_aliases<DEV>(); } \
+    TEST_CASE(cached_errors) { module_tests::cached_errors<DEV>(); }
