@@ -95,6 +95,42 @@ class Device {
         self().copy_raw(dst.ptr(), src.ptr(), src.len() * sizeof(T));
     }
 
+    // `CopySlice::copy_slice_to` (src/op_traits.rs:68-75, src/devices/cuda/ops.rs:66-87):
+    // elements [src_begin, src_end) of `source` into `dest` from `dst_begin` on,
+    // device to device.  Ranges that leave either buffer are an error (the reference panics).
+    template <class T>
+    void copy_slice_to(const Buffer<T, Derived>& source, size_t src_begin, size_t src_end, Buffer<T, Derived>& dest,
+                       size_t dst_begin, size_t dst_end) {
+        if (!source.has_data() || !dest.has_data()) throw Error(DeviceError::InvalidLazyBuf);
+        if (src_begin > src_end || src_end > source.len() || dst_begin > dst_end || dst_end > dest.len() ||
+            src_end - src_begin != dst_end - dst_begin)
+            throw Error(DeviceError::ShapeLengthMismatch);
+        if (src_end == src_begin) return;
+        self().copy_raw(dest.ptr() + dst_begin * sizeof(T), source.ptr() + src_begin * sizeof(T),
+                        (src_end - src_begin) * sizeof(T));
+    }
+    // `CopySlice::copy_slice` (src/op_traits.rs:41-53): a new buffer holding the slice
+    template <class T>
+    Buffer<T, Derived> copy_slice(const Buffer<T, Derived>& buf, size_t begin, size_t end) {
+        if (begin > end || end > buf.len()) throw Error(DeviceError::ShapeLengthMismatch);
+        Buffer<T, Derived> copied = new_buffer<T>(end - begin);
+        copy_slice_to(buf, begin, end, copied, 0, end - begin);
+        return copied;
+    }
+    // `CopySlice::copy_slice_all` (src/devices/cuda/ops.rs:89-98): (source range, dest range) pairs
+    struct SlicePair {
+        size_t src_begin, src_end, dst_begin, dst_end;
+    };
+    template <class T>
+    void copy_slice_all(const Buffer<T, Derived>& source, Buffer<T, Derived>& dest, const std::vector<SlicePair>& ranges) {
+        for (const SlicePair& r : ranges) copy_slice_to(source, r.src_begin, r.src_end, dest, r.dst_begin, r.dst_end);
+    }
+    // `CloneBuf::clone_buf` (src/op_traits.rs:176-197)
+    template <class T>
+    Buffer<T, Derived> clone_buf(const Buffer<T, Derived>& buf) {
+        return copy_slice(buf, 0, buf.len());
+    }
+
     // ---- operations ----
 
     // `device.add_op((&mut out, buf), |(out, buf), dev| ...)`.

@@ -706,6 +706,33 @@ void elementwise_fuse_random_programs() {
     }
 }
 
+// ---- CopySlice / CloneBuf ----
+
+// tests/slice_buf.rs:5-84, tests/clone_buf.rs:5-49
+template <template <class> class DEV>
+void copy_slice_and_clone_buf() {
+    DEV<Base> device;
+    auto source = device.template buffer<float>({1.f, 2.f, 6.f, 2.f, 4.f});
+    auto actual = device.copy_slice(source, 1, 3);
+    CHECK_VEC_EQ(actual.read(), (std::vector<float>{2.f, 6.f}));
+    auto dest = device.template new_buffer<float>(10);
+    device.copy_slice_all(source, dest, {{2, 5, 7, 10}, {1, 3, 3, 5}});
+    CHECK_VEC_EQ(dest.read(), (std::vector<float>{0.f, 0.f, 0.f, 2.f, 6.f, 0.f, 0.f, 6.f, 2.f, 4.f}));
+    // out of bounds: the reference panics
+    CHECK_THROWS_KIND(device.copy_slice_all(source, dest, {{2, 5, 8, 11}, {1, 3, 3, 5}}), DeviceError::ShapeLengthMismatch);
+    CHECK_THROWS_KIND(device.copy_slice(source, 3, 6), DeviceError::ShapeLengthMismatch);
+    CHECK_THROWS_KIND(device.copy_slice_to(source, 0, 2, dest, 0, 3), DeviceError::ShapeLengthMismatch);
+    // src/op_traits.rs:60-66
+    auto dest2 = device.template buffer<float>({5.f, 4.f, 3.f, 2.f, 1.f});
+    device.copy_slice_to(source, 1, 3, dest2, 3, 5);
+    CHECK_VEC_EQ(dest2.read(), (std::vector<float>{5.f, 4.f, 3.f, 2.f, 6.f}));
+    auto cloned = device.clone_buf(source);
+    CHECK_VEC_EQ(cloned.read(), source.read());
+    CHECK(cloned.ptr() != source.ptr());
+    auto ints = device.template buffer<int>({7, 8, 9});
+    CHECK_VEC_EQ(device.clone_buf(ints).read(), (std::vector<int>{7, 8, 9}));
+}
+
 // ---- Cached ----
 
 // tests/cache.rs:24-45 (test_caching_cpu)
@@ -886,6 +913,7 @@ void cached_errors() {
     TEST_CASE(elementwise_fuse_respects_limits) { module_tests::elementwise_fuse_respects_limits<DEV>(); } \
     TEST_CASE(elementwise_fuse_keeps_tape_buffers) { module_tests::elementwise_fuse_keeps_tape_buffers<DEV>(TOL); } \
     TEST_CASE(elementwise_fuse_random_programs) { module_tests::elementwise_fuse_random_programs<DEV>(); } \
+    TEST_CASE(copy_slice_and_clone_buf) { module_tests::copy_slice_and_clone_buf<DEV>(); }        \
     TEST_CASE(cached_same_allocation_every_epoch) { module_tests::cached_same_allocation_every_epoch<DEV>(); } \
     TEST_CASE(cached_multi_level_retrieve) { module_tests::cached_multi_level_retrieve<DEV>(); }  \
     TEST_CASE(cached_apply_fn_and_unary_ew) { module_tests::cached_apply_fn_and_unary_ew<DEV>(); } \
