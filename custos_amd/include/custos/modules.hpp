@@ -274,6 +274,13 @@ struct Lazy {
                 for (size_t use : t.use_cache_idxs) {
                     auto use_id = gt->idx_to_buf_id.find(use);
                     if (use_id == gt->idx_to_buf_id.end()) throw Error(DeviceError::GraphOptimization);
+                    // a buffer of another element type keeps an allocation of its own, as in the
+                    // Cached module (cached.rs:430-441); the reference's Lazy aliases it anyway and
+                    // the run then fails (opt_graph/optimize.rs:659-690)
+                    bool same_type = true;
+                    for (const Pending& q : pending)
+                        if (q.id.id == use_id->second) same_type = q.type == p.type;
+                    if (!same_type) continue;
                     buffers_[use_id->second] = shared;
                     allocated_ids_.insert(use_id->second);
                 }

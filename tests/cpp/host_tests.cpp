@@ -113,6 +113,18 @@ TEST_CASE(cache_trace_break) {
     // the first unoptimizable node still joins the trace, then it ends
     CHECK_VEC_EQ(g.trace_cache_path_raw(g.node(c)), (std::vector<size_t>{3}));
 }
+// src/modules/graph/opt_graph/optimize.rs:248-275 (test_trace_all)
+TEST_CASE(cache_trace_all) {
+    OptGraph graph;
+    const size_t a = graph.add_leaf(10), b = graph.add_leaf(10);
+    const size_t c = graph.add_node(10, {a, b});
+    const size_t d = graph.add_node(10, {c, c});
+    graph.add_node(10, {d, b});
+    auto traces = graph.cache_traces();
+    CHECK_EQ(traces.size(), size_t(1));
+    CHECK(traces[0] == (CacheTrace{2, {3, 4}}));
+}
+
 TEST_CASE(cache_trace_leafed_diff_len) {
     OptGraph g;
     auto a = g.add_leaf(10);

@@ -706,6 +706,131 @@ void elementwise_fuse_random_programs() {
     }
 }
 
+// src/modules/lazy/lazy_graph.rs:253-370 (test_lazy_op_args, .._no_out_but_use, .._no_out_but_use_loop,
+// .._with_ew_fn): recorded operations get their arguments by id when the graph runs
+template <template <class> class DEV>
+void lazy_custom_operations() {
+    DEV<Lazy<Base>> device;
+    auto lhs = device.template buffer<float>({1.f, 2.f, 3.f, 4.f, 5.f});
+    auto rhs = device.template buffer<float>({1.f, 2.f, 6.f, 4.f, 5.f});
+    auto out = device.template retrieve<float>(lhs.len(), lhs, rhs);
+    int calls = 0;
+    using Buf = Buffer<float, DEV<Lazy<Base>>>;
+    for (int i = 0; i < 10; i++)
+        device.add_op(std::tie(lhs, rhs, out), [&calls](const Buf& l, const Buf& r, Buf& o, DEV<Lazy<Base>>&) {
+            CHECK_VEC_EQ(l.read(), (std::vector<float>{1.f, 2.f, 3.f, 4.f, 5.f}));
+            CHECK_VEC_EQ(r.read(), (std::vector<float>{1.f, 2.f, 6.f, 4.f, 5.f}));
+            CHECK(o.has_data());
+            calls++;
+        });
+    device.add_op(std::tie(lhs, rhs), [&calls](const Buf& l, const Buf& r, DEV<Lazy<Base>>&) {
+        CHECK_EQ(l.len(), r.len());
+        calls++;
+    });
+    // an operation that writes its output from the host (the reference's `ew_fn`)
+    device.add_op(std::tie(out, lhs), [](Buf& o, const Buf& l, DEV<Lazy<Base>>&) {
+        std::vector<float> v = l.read();
+        for (float& x : v) x += 10.f;
+        o.write(v);
+    });
+    CHECK_EQ(calls, 0);
+    CHECK_EQ(device.ops_count(), size_t(12));
+    device.run();
+    CHECK_EQ(calls, 11);
+    CHECK_VEC_EQ(out.replace().read(), (std::vector<float>{11.f, 12.f, 13.f, 14.f, 15.f}));
+}
+
+// src/modules/lazy.rs:842-856 (test_lazy_cached_two_producers): Lazy answers the retrieve itself
+template <template <class> class DEV>
+void lazy_over_cached() {
+    DEV<Lazy<Cached<Base>>> device;
+    auto lhs = device.template buffer<int>({1, 2, 3, 4});
+    auto rhs = device.template buffer<int>({1, 2, 3, 4});
+    auto out = device.template retrieve<int>(10, lhs, rhs);
+    CHECK(out.flag() == AllocFlag::Lazy);
+    CHECK_EQ(device.modules.modules.cached_allocations(), size_t(0));
+    auto sum = device.apply_fn2(lhs, rhs, [](auto x, auto y) { return x.add(y); });
+    device.run();
+    CHECK_VEC_EQ(sum.replace().read(), (std::vector<int>{2, 4, 6, 8}));
+}
+
+// src/modules/graph/opt_graph/optimize.rs:395-449 (test_from_retrieve_sine_neural_net)
+template <template <class> class DEV>
+void graph_cached_neural_net_traces() {
+    DEV<Graph<Cached<Base>>> device;
+    auto ones = [&](size_t n, int v = 1) { return device.template buffer<int>(std::vector<int>(n, v)); };
+    auto w1 = ones(10 * 64), b1 = ones(64), w2 = ones(64 * 64), b2 = ones(64), w3 = ones(64 * 64), b3 = ones(64);
+    auto w4 = ones(64), b4 = ones(1), inputs = ones(10 * 100), targets = ones(100, 2);
+    auto a1 = device.template retrieve<int>(100 * 64, inputs, w1);
+    auto a2 = device.template retrieve<int>(100 * 64, a1, b1);
+    auto a2b = device.template retrieve<int>(100 * 64, a2, a2);
+    auto a3 = device.template retrieve<int>(100 * 64, a2b, w2);
+    auto a4 = device.template retrieve<int>(100 * 64, a3, b2);
+    auto a4b = device.template retrieve<int>(100 * 64, a4, a4);
+    auto a5 = device.template retrieve<int>(100 * 64, a4b, w3);
+    auto a6 = device.template retrieve<int>(100 * 64, a5, b3);
+    auto a6b = device.template retrieve<int>(100 * 64, a6, a6);
+    auto a7 = device.template retrieve<int>(100, a6b, w4);
+    auto a8 = device.template retrieve<int>(100, a7, b4);
+    auto loss = device.template retrieve<int>(100, a8, targets);
+    auto traces = device.modules.graph_trans.opt_graph.cache_traces();
+    CHECK_EQ(traces.size(), size_t(2));
+    CHECK(traces[0] == (CacheTrace{10, {11, 12, 13, 14, 15, 16, 17, 18}}));
+    CHECK(traces[1] == (CacheTrace{19, {20, 21}}));
+}
+
+// src/modules/graph/opt_graph/optimize.rs:566-612 (.._optimize_cache) and :614-657
+// (test_mismatched_optimized_types_cached): ids after optimising the cached allocations
+template <template <class> class DEV>
+void cached_sliced_chained_optimize(bool mismatched) {
+    DEV<Graph<Cached<Base>>> device;
+    auto x = device.template buffer<float>(std::vector<float>(1000, 1.f));
+    auto b = device.template buffer<float>(std::vector<float>(1000, 1.1f));
+    for (size_t i : device.range(0, 2)) {
+        {
+            auto squared = device.template retrieve<float>(1000, x, x);
+            auto add = device.template retrieve<float>(1000, b, x);
+            Id mul_b_id;
+            // the reference retrieves `mul_b` as u8 in the mismatched case
+            auto mul_b_f = mismatched ? Buffer<float, DEV<Graph<Cached<Base>>>>() : device.template retrieve<float>(1000, add, b);
+            auto mul_b_u = mismatched ? device.template retrieve<unsigned char>(1000, add, b)
+                                      : Buffer<unsigned char, DEV<Graph<Cached<Base>>>>();
+            mul_b_id = mismatched ? mul_b_u.id() : mul_b_f.id();
+            auto mul = device.template retrieve<float>(1000, squared, x);
+            auto out = mismatched ? device.template retrieve<float>(1000, mul, mul_b_u)
+                                  : device.template retrieve<float>(1000, mul, mul_b_f);
+            if (i == 0) CHECK(squared.id() != mul.id());
+            if (i == 1) {
+                CHECK(squared.id() == mul.id());
+                CHECK(squared.id() == out.id());
+                if (mismatched) CHECK(add.id().id != mul_b_id.id);
+                else CHECK(add.id() == mul_b_id);
+            }
+        }
+        if (i == 0) device.optimize_mem_graph();
+    }
+}
+
+// src/modules/graph/opt_graph/optimize.rs:659-690 (test_mismatched_optimized_types_lazy, which
+// expects a panic): here the buffer of the other type keeps its own allocation and the run works
+template <template <class> class DEV>
+void lazy_mismatched_types_keep_their_allocation() {
+    DEV<Graph<Lazy<Base>>> device;
+    auto x = device.template buffer<float>(std::vector<float>(1000, 1.f));
+    auto b = device.template buffer<float>(std::vector<float>(1000, 1.1f));
+    auto squared = device.template retrieve<float>(1000, x, x);
+    auto add = device.template retrieve<float>(1000, b, x);
+    auto mul_b = device.template retrieve<unsigned char>(1000, add, b);
+    auto mul = device.template retrieve<float>(1000, squared, x);
+    auto out = device.template retrieve<float>(1000, mul, mul_b);
+    device.optimize_mem_graph();
+    device.run();
+    CHECK_EQ(squared.replace().ptr(), mul.replace().ptr());
+    CHECK_EQ(squared.replace().ptr(), out.replace().ptr());
+    CHECK(add.replace().ptr() != mul_b.replace().ptr());
+    CHECK_EQ(mul_b.replace().len(), size_t(1000));
+}
+
 // ---- CopySlice / CloneBuf ----
 
 // tests/slice_buf.rs:5-84, tests/clone_buf.rs:5-49
@@ -913,6 +1038,12 @@ void cached_errors() {
     TEST_CASE(elementwise_fuse_respects_limits) { module_tests::elementwise_fuse_respects_limits<DEV>(); } \
     TEST_CASE(elementwise_fuse_keeps_tape_buffers) { module_tests::elementwise_fuse_keeps_tape_buffers<DEV>(TOL); } \
     TEST_CASE(elementwise_fuse_random_programs) { module_tests::elementwise_fuse_random_programs<DEV>(); } \
+    TEST_CASE(lazy_custom_operations) { module_tests::lazy_custom_operations<DEV>(); }            \
+    TEST_CASE(lazy_over_cached) { module_tests::lazy_over_cached<DEV>(); }                        \
+    TEST_CASE(graph_cached_neural_net_traces) { module_tests::graph_cached_neural_net_traces<DEV>(); } \
+    TEST_CASE(cached_sliced_chained_optimize) { module_tests::cached_sliced_chained_optimize<DEV>(false); } \
+    TEST_CASE(cached_mismatched_types_optimize) { module_tests::cached_sliced_chained_optimize<DEV>(true); } \
+    TEST_CASE(lazy_mismatched_types_keep_their_allocation) { module_tests::lazy_mismatched_types_keep_their_allocation<DEV>(); } \
     TEST_CASE(copy_slice_and_clone_buf) { module_tests::copy_slice_and_clone_buf<DEV>(); }        \
     TEST_CASE(cached_same_allocation_every_epoch) { module_tests::cached_same_allocation_every_epoch<DEV>(); } \
     TEST_CASE(cached_multi_level_retrieve) { module_tests::cached_multi_level_retrieve<DEV>(); }  \
