@@ -831,6 +831,67 @@ void lazy_mismatched_types_keep_their_allocation() {
     CHECK_EQ(mul_b.replace().len(), size_t(1000));
 }
 
+// src/modules/autograd.rs:335-431: the pool of buffers by id that gradient functions look
+// their arguments up in when no Lazy module keeps one
+template <template <class> class DEV>
+void autograd_no_grads_pool() {
+    {
+        // test_buffer_creation_autograd_register_manual / _get_buf / _unregister
+        DEV<Autograd<Cached<Base>>> device;
+        Id id;
+        {
+            auto buf = device.template new_buffer<float>(10);
+            id = buf.id();
+            auto it = device.modules.state.no_grads_pool.find(id.id);
+            CHECK(it != device.modules.state.no_grads_pool.end());
+            if (it != device.modules.state.no_grads_pool.end()) {
+                CHECK_EQ(it->second.ptr, buf.ptr());
+                CHECK_EQ(it->second.len, size_t(10));
+                CHECK(it->second.type == std::type_index(typeid(float)));
+            }
+        }
+        CHECK(device.modules.state.no_grads_pool.find(id.id) == device.modules.state.no_grads_pool.end());
+    }
+    {
+        // test_buffer_new_and_retrieve
+        DEV<Autograd<Cached<Base>>> device;
+        auto lhs = device.template new_buffer<float>(10);
+        for (size_t epoch : device.range(0, 100)) {
+            (void)epoch;
+            auto x = device.template retrieve<float>(100);
+            CHECK_EQ(x.len(), size_t(100));
+        }
+        CHECK_EQ(device.modules.state.no_grads_pool.size(), size_t(2));
+    }
+    {
+        // test_cached_before_autograd
+        DEV<Cached<Autograd<Base>>> device;
+        auto lhs = device.template new_buffer<float>(10);
+        for (size_t epoch : device.range(0, 100)) {
+            (void)epoch;
+            auto x = device.template retrieve<float>(100);
+            CHECK_EQ(x.len(), size_t(100));
+        }
+        CHECK_EQ(device.modules.modules.state.no_grads_pool.size(), size_t(2));
+    }
+    {
+        // test_tape_return_without_autograd (panics in the reference), .._with_grad_allocation
+        DEV<Base> plain;
+        auto buf = plain.template new_buffer<float>(10);
+        bool threw = false;
+        try {
+            buf.grad();
+        } catch (const std::logic_error&) {
+            threw = true;
+        }
+        CHECK(threw);
+        DEV<Autograd<Base>> device;
+        auto buf2 = device.template new_buffer<float>(10);
+        auto g = buf2.grad();
+        CHECK_VEC_EQ(g.read(), std::vector<float>(10, 0.f));
+    }
+}
+
 // ---- CopySlice / CloneBuf ----
 
 // tests/slice_buf.rs:5-84, tests/clone_buf.rs:5-49
@@ -1044,6 +1105,7 @@ void cached_errors() {
     TEST_CASE(cached_sliced_chained_optimize) { module_tests::cached_sliced_chained_optimize<DEV>(false); } \
     TEST_CASE(cached_mismatched_types_optimize) { module_tests::cached_sliced_chained_optimize<DEV>(true); } \
     TEST_CASE(lazy_mismatched_types_keep_their_allocation) { module_tests::lazy_mismatched_types_keep_their_allocation<DEV>(); } \
+    TEST_CASE(autograd_no_grads_pool) { module_tests::autograd_no_grads_pool<DEV>(); }            \
     TEST_CASE(copy_slice_and_clone_buf) { module_tests::copy_slice_and_clone_buf<DEV>(); }        \
     TEST_CASE(cached_same_allocation_every_epoch) { module_tests::cached_same_allocation_every_epoch<DEV>(); } \
     TEST_CASE(cached_multi_level_retrieve) { module_tests::cached_multi_level_retrieve<DEV>(); }  \
