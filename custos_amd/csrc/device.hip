@@ -107,7 +107,15 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
     if (idx < 0 || idx >= count)
         return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_DEVICE_INDEX,
                          "device index " + std::to_string(idx) + " out of range: " + std::to_string(count) + " device(s)");
-    std::unique_ptr<custos_hip_device> dev(new custos_hip_device);
+    // the deleter also releases what was created before a later step failed
+    auto drop = [](custos_hip_device* d) {
+        if (d->t0) (void)hipEventDestroy(d->t0);
+        if (d->t1) (void)hipEventDestroy(d->t1);
+        if (d->stream) (void)hipStreamDestroy(d->stream);
+        if (d->transfer) (void)hipStreamDestroy(d->transfer);
+        delete d;
+    };
+    std::unique_ptr<custos_hip_device, decltype(drop)> dev(new custos_hip_device, drop);
     dev->idx = idx;
     HIP_TRY(nullptr, hipSetDevice(idx));
     HIP_TRY(nullptr, hipGetDeviceProperties(&dev->props, idx));

@@ -192,6 +192,20 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
     REQUIRE_DEV(dev);
     if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "kernel out pointer is null");
     *kernel = nullptr;
+    std::string text_key;
+    if (src && markers && n_markers >= 1 && n_markers <= 4) {
+        const Tuning& t = dev->tuning;
+        text_key = std::to_string(kind) + "," + std::to_string(dtype) + "," + std::to_string(t.block_threads) + "," +
+                   std::to_string(t.unroll) + "," + std::to_string(t.blocks_per_cu) + "," + std::to_string(t.nontemporal);
+        for (int i = 0; i < n_markers; i++) text_key.append(1, '\x1f').append(markers[i] ? markers[i] : "");
+        text_key.append(1, '\x1e').append(src);
+        auto known = dev->by_text.find(text_key);
+        if (known != dev->by_text.end()) {
+            dev->hits++;
+            *kernel = known->second;
+            return CUSTOS_HIP_OK;
+        }
+    }
     std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
     int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, dev->tuning, &k->spec);
     if (rc != CUSTOS_HIP_OK) return rc;
@@ -205,6 +219,7 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
         if (a.compare(a.find('\n'), std::string::npos, b, b.find('\n'), std::string::npos) == 0) {
             dev->hits++;
             *kernel = cached.get();
+            dev->by_text.emplace(std::move(text_key), cached.get());
             return CUSTOS_HIP_OK;
         }
     }
@@ -216,6 +231,7 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
         k->fn_batched = nullptr;
     }
     *kernel = k.get();
+    dev->by_text.emplace(std::move(text_key), k.get());
     bucket.push_back(std::move(k));
     return CUSTOS_HIP_OK;
 }

@@ -83,6 +83,10 @@ struct custos_hip_device {
     uint64_t compiles = 0, hits = 0, disk_hits = 0;
     std::string last_error;
     std::unordered_map<uint64_t, std::vector<std::unique_ptr<custos_hip_kernel>>> cache;
+    // expression exactly as the caller spelt it (with kind, type, markers, tuning) -> kernel:
+    // a repeated call is answered without parsing (what the (source, name) map of
+    // src/devices/cuda/kernel_cache.rs:45-49 does for the reference)
+    std::unordered_map<std::string, custos_hip_kernel*> by_text;
     std::vector<custos_hip_graph*> graphs;
 };
 
