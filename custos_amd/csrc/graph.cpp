@@ -16,12 +16,16 @@ namespace {
 // memory it conflicts with (read-after-write, write-after-read or
 // write-after-write on overlapping address ranges).  Nodes of one level are
 // independent of each other, so they run side by side in the graph, and kernel
-// launches of one level that use the same kernel over the same length are
-// merged into ONE grid that walks a table of operand addresses.  1024 small
-// buffers with three operations each become three kernel nodes instead of
-// 3072.
+// launches of one level that use the same kernel are merged into ONE grid that
+// walks a table of operand addresses (equal lengths: segment = block / tiles
+// per segment; different lengths: a block map names segment and tile of every
+// workgroup).  1024 small buffers with three operations each become three
+// kernel nodes instead of 3072.
 
 constexpr uint64_t kChunkShift = 21;  // conflict search buckets of 2 MiB
+// A launch of more tiles than this is not merged with launches of other lengths:
+// it fills the chip by itself, and the block map would grow with it.
+constexpr unsigned long long kRaggedMaxTiles = 16384;
 
 void assign_levels(std::vector<RecNode>& nodes) {
     struct Seen {
@@ -83,37 +87,85 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
 
     // plan: per level, either single nodes or batches of node indices
     struct Planned {
-        std::vector<size_t> members;  // indices into `nodes`; more than one = batched launch
+        std::vector<size_t> members;  // indices into `nodes`; more than one = one merged launch
+        bool ragged = false;          // members differ in length
         size_t table_offset = 0;      // in u64 entries
+        size_t map_offset = 0;        // ragged: start of the block map, in u64 entries
+        size_t blocks = 0;            // ragged: workgroups
+    };
+    auto tiles_of = [](const RecNode& n) {
+        const Tuning& t = n.k->spec.tuning;
+        const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+        return std::max(1ull, (n.n_vec + tile_vecs - 1) / tile_vecs);
     };
     std::vector<std::vector<Planned>> plan(static_cast<size_t>(max_level + 1));
     std::vector<uint64_t> host_table;
     for (int level = 0; level <= max_level; level++) {
         std::vector<Planned>& out = plan[level];
-        // batches keyed by (kernel, n), in first-seen order
-        std::vector<std::pair<std::pair<custos_hip_kernel*, unsigned long long>, size_t>> keys;
+        // candidates for merging, grouped by kernel in first-seen order
+        std::vector<std::pair<custos_hip_kernel*, std::vector<size_t>>> groups;
         for (size_t i = 0; i < nodes.size(); i++) {
             if (nodes[i].level != level) continue;
             if (dev->batching && batchable(nodes[i])) {
-                const auto key = std::make_pair(nodes[i].k, nodes[i].n);
-                size_t slot = out.size();
-                for (const auto& kv : keys)
-                    if (kv.first == key) slot = kv.second;
-                if (slot == out.size()) {
-                    keys.push_back({key, slot});
-                    out.emplace_back();
+                auto g = std::find_if(groups.begin(), groups.end(), [&](const auto& kv) { return kv.first == nodes[i].k; });
+                if (g == groups.end()) {
+                    groups.push_back({nodes[i].k, {}});
+                    g = groups.end() - 1;
                 }
-                out[slot].members.push_back(i);
+                g->second.push_back(i);
             } else {
                 out.emplace_back();
                 out.back().members.push_back(i);
             }
         }
+        for (auto& g : groups) {
+            bool uniform = true;
+            for (size_t i : g.second) uniform = uniform && nodes[i].n == nodes[g.second[0]].n;
+            Planned merged;
+            if (uniform || !g.first->fn_ragged) {
+                // equal lengths: one grid, segment = block / tiles per segment.  (Without the
+                // ragged entry point, different lengths fall back to one batch per length.)
+                std::vector<std::pair<unsigned long long, Planned>> by_n;
+                for (size_t i : g.second) {
+                    auto it = std::find_if(by_n.begin(), by_n.end(), [&](const auto& kv) { return kv.first == nodes[i].n; });
+                    if (it == by_n.end()) {
+                        by_n.push_back({nodes[i].n, Planned{}});
+                        it = by_n.end() - 1;
+                    }
+                    it->second.members.push_back(i);
+                }
+                for (auto& kv : by_n) out.push_back(std::move(kv.second));
+                continue;
+            }
+            // different lengths: one grid with a block map; a launch that fills the
+            // chip on its own stays a launch of its own
+            merged.ragged = true;
+            for (size_t i : g.second) {
+                if (tiles_of(nodes[i]) > kRaggedMaxTiles) {
+                    out.emplace_back();
+                    out.back().members.push_back(i);
+                } else {
+                    merged.members.push_back(i);
+                }
+            }
+            if (merged.members.size() == 1) merged.ragged = false;
+            if (!merged.members.empty()) out.push_back(std::move(merged));
+        }
         for (Planned& p : out) {
             if (p.members.size() < 2) continue;
             p.table_offset = host_table.size();
-            for (size_t i : p.members)
-                for (uint64_t ptr : nodes[i].ptrs) host_table.push_back(ptr);
+            for (size_t seg = 0; seg < p.members.size(); seg++) {
+                const RecNode& n = nodes[p.members[seg]];
+                for (uint64_t ptr : n.ptrs) host_table.push_back(ptr);
+                if (p.ragged) host_table.push_back(n.n);
+            }
+            if (!p.ragged) continue;
+            p.map_offset = host_table.size();
+            for (size_t seg = 0; seg < p.members.size(); seg++) {
+                const unsigned long long tiles = tiles_of(nodes[p.members[seg]]);
+                for (unsigned long long t = 0; t < tiles; t++) host_table.push_back(static_cast<uint64_t>(seg) << 32 | t);
+            }
+            p.blocks = host_table.size() - p.map_offset;
         }
     }
     if (!host_table.empty()) {
@@ -159,6 +211,15 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
                 ln.args.push_back(value(&a2, 8));
                 ln.func = reinterpret_cast<void*>(first.k->fn);
                 ln.grid = dim3(first.grid);
+                ln.block = dim3(static_cast<unsigned int>(first.k->spec.tuning.block_threads));
+            } else if (p.ragged) {
+                if (p.blocks > (1ull << 31) - 1)
+                    return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
+                const uint64_t table = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
+                const uint64_t map = reinterpret_cast<uint64_t>(g->table) + p.map_offset * sizeof(uint64_t);
+                ln.args = {value(&table, 8), value(&map, 8)};
+                ln.func = reinterpret_cast<void*>(first.k->fn_ragged);
+                ln.grid = dim3(static_cast<unsigned int>(p.blocks));
                 ln.block = dim3(static_cast<unsigned int>(first.k->spec.tuning.block_threads));
             } else {
                 const Tuning& t = first.k->spec.tuning;

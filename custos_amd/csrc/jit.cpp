@@ -230,6 +230,10 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
         (void)hipGetLastError();
         k->fn_batched = nullptr;
     }
+    if (hipModuleGetFunction(&k->fn_ragged, k->module, (k->spec.name + "_ragged").c_str()) != hipSuccess) {
+        (void)hipGetLastError();
+        k->fn_ragged = nullptr;
+    }
     *kernel = k.get();
     dev->by_text.emplace(std::move(text_key), k.get());
     bucket.push_back(std::move(k));

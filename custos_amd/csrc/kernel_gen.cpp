@@ -133,7 +133,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     uint64_t h;
     if (!hash_expr(k.expr, dtype, &h, err)) return false;
     int32_t tail[6] = {static_cast<int32_t>(kind), tuning.block_threads, tuning.unroll,
-                       tuning.blocks_per_cu, tuning.nontemporal, 4 /* template version */};
+                       tuning.blocks_per_cu, tuning.nontemporal, 5 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -272,6 +272,34 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     s += vec_ptrs;
     s += "    custos_tile(" + tile_args + "vout, tile * (u64)CUSTOS_BLOCK * CUSTOS_UNROLL + threadIdx.x, n_vec);\n";
     s += "    if (tile == tiles_per_seg - 1)\n";
+    s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
+         list("in", "[i]") + ");\n";
+    s += "    (void)head;\n}\n";
+
+    // Third entry point: launches of different lengths in one grid.  A table row
+    // holds the operand addresses (16-byte aligned) and the element count of its
+    // segment; `block_map[b]` = segment << 32 | tile tells workgroup b its work.
+    s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
+    s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map) {\n";
+    s += "    const u64 where = block_map[blockIdx.x];\n";
+    s += "    const u64 seg = where >> 32;\n";
+    s += "    const u64 tile = where & 0xffffffffull;\n";
+    s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + 1) + ";\n";
+    s += "    const u64 n = ptrs[" + std::to_string(n_ptrs) + "];\n";
+    s += "    const u64 n_vec = n / CUSTOS_VEC;\n";
+    s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
+    s += "    const u64 n_tiles = n_vec == 0 ? 1 : (n_vec + tile_vecs - 1) / tile_vecs;\n";
+    s += "    const u64 head = 0;\n";
+    if (kind == Kind::Apply) {
+        for (int i = 0; i < n_in; i++)
+            s += "    const S* in" + std::to_string(i) + " = (const S*)ptrs[" + std::to_string(i) + "];\n";
+        s += "    S* out = (S*)ptrs[" + std::to_string(n_in) + "];\n";
+    } else {
+        s += "    const S* in0 = (const S*)ptrs[0];\n    S* out = (S*)ptrs[1];\n    const S* in2 = (const S*)ptrs[2];\n";
+    }
+    s += vec_ptrs;
+    s += "    custos_tile(" + tile_args + "vout, tile * tile_vecs + threadIdx.x, n_vec);\n";
+    s += "    if (tile == n_tiles - 1)\n";
     s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
          list("in", "[i]") + ");\n";
     s += "    (void)head;\n}\n";

@@ -20,7 +20,8 @@ struct custos_hip_kernel {
     custos_hip::KernelSpec spec;
     hipModule_t module = nullptr;
     hipFunction_t fn = nullptr;
-    hipFunction_t fn_batched = nullptr;
+    hipFunction_t fn_batched = nullptr;  // equal launches in one grid
+    hipFunction_t fn_ragged = nullptr;   // launches of different lengths in one grid
 };
 
 // A graph node in launchable form: function, shape and a copy of the argument values.

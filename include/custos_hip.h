@@ -247,7 +247,7 @@ int32_t custos_hip_capture_begin(custos_hip_device *dev);
 /* Ends recording and instantiates an executable graph (LazyCudaGraph::new).
  * The graph is built from the recorded work, not replayed launch by launch:
  * work that does not touch the same memory runs side by side, and independent
- * launches of the same kernel over the same length are merged into one grid
+ * launches of the same kernel are merged into one grid, whatever their lengths
  * (1024 buffers x 3 operations replay as 3 kernel nodes). */
 int32_t custos_hip_capture_end(custos_hip_device *dev, custos_hip_graph **graph);
 /* Switches the merging of equal independent launches off (0) or on (default):

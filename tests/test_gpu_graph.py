@@ -118,8 +118,8 @@ def test_capture_state_errors(hip):
 
 
 def test_batched_launch_with_tails_and_mixed_lengths(hip, oracle):
-    """Independent launches of one kernel: equal lengths merge into one grid (including a
-    scalar tail per buffer), other lengths and unaligned views stay separate nodes."""
+    """Independent launches of one kernel merge into one grid, whatever their lengths
+    (a scalar tail per buffer included); unaligned views stay separate nodes."""
     f = lambda v: v.mul(1.5).add(0.25)
     lens = [1003] * 40 + [7] * 5 + [4096] * 3 + [1]
     xs = [synth.uniform_f32(100 + i, n, -2, 2) for i, n in enumerate(lens)]
@@ -134,7 +134,7 @@ def test_batched_launch_with_tails_and_mixed_lengths(hip, oracle):
     g = hip.capture_end()
     recorded, kernel_nodes, levels = g.stats()
     assert recorded == len(lens) + 1 and levels == 1
-    assert kernel_nodes == 3 + 1 + 1      # batches for 1003, 7, 4096; the single n=1; the unaligned view
+    assert kernel_nodes == 1 + 1          # one grid for all lengths; the unaligned view
     for _ in range(2):
         g.launch()
         hip.sync()
@@ -142,6 +142,70 @@ def test_batched_launch_with_tails_and_mixed_lengths(hip, oracle):
             assert_bits_equal(o.read(), oracle.apply_fn(f, x))
         assert_bits_equal(big_out.read()[3:], oracle.apply_fn(f, big.read()[3:]))
         assert not big_out.read()[:3].any()
+
+
+def test_merged_launches_of_different_lengths(hip, oracle):
+    """Launches of one kernel over many lengths (multi-tensor apply): one grid with a block
+    map; equal lengths alone keep the division-based grid; a launch that fills the chip on its
+    own is left out of the merge.  Unary-gradient kernels and 16-bit types merge the same way."""
+    f = lambda v: v.mul(0.75).sub(0.5)
+    rng = np.random.default_rng(5)
+    lens = [int(n) for n in rng.integers(1, 3000, size=200)] + [256, 257, 255, 1024, 1 << 16]
+    xs = [synth.uniform_f32(300 + i, n, -4, 4) for i, n in enumerate(lens)]
+    bufs = [hip.buffer(x) for x in xs]
+    outs = [hip.alloc(n) for n in lens]
+    huge_n = 16384 * 1024 + 4096          # more tiles than a merged launch takes
+    huge = hip.buffer(synth.uniform_f32(9, huge_n, -1, 1))
+    huge_out = hip.alloc(huge_n)
+    hip.capture_begin()
+    for b, o in zip(bufs, outs):
+        hip.apply_fn(b, f, out=o)
+    hip.apply_fn(huge, f, out=huge_out)
+    g = hip.capture_end()
+    assert g.stats() == (len(lens) + 1, 2, 1)
+    for _ in range(2):
+        for o in outs:
+            o.clear()
+        g.launch()
+        hip.sync()
+        for x, o in zip(xs, outs):
+            assert_bits_equal(o.read(), oracle.apply_fn(f, x))
+        assert_bits_equal(huge_out.read(), oracle.apply_fn(f, huge.read()))
+    g.destroy()
+
+    # equal lengths only: the uniform grid, still one node
+    hip.capture_begin()
+    same = [hip.alloc(lens[0]) for _ in range(8)]
+    for o in same:
+        hip.apply_fn(bufs[0], f, out=o)
+    g = hip.capture_end()
+    assert g.stats() == (8, 1, 1)
+    g.launch()
+    hip.sync()
+    for o in same:
+        assert_bits_equal(o.read(), oracle.apply_fn(f, xs[0]))
+    g.destroy()
+
+    # unary gradient, f16 storage, lengths with tails
+    d = lambda v: v.mul(2.0)
+    glens = [5, 64, 1000, 1001, 4099]
+    lhs = [synth.uniform_f32(40 + i, n, -2, 2).astype(np.float16) for i, n in enumerate(glens)]
+    og = [synth.uniform_f32(60 + i, n, -1, 1).astype(np.float16) for i, n in enumerate(glens)]
+    g0 = [np.full(n, 0.5, np.float16) for n in glens]
+    lb = [hip.buffer(a, "f16") for a in lhs]
+    ob = [hip.buffer(a, "f16") for a in og]
+    gb = [hip.buffer(a, "f16") for a in g0]
+    hip.capture_begin()
+    for l, gr, o in zip(lb, gb, ob):
+        hip.add_unary_grad(l, gr, o, d)
+    g = hip.capture_end()
+    assert g.stats() == (len(glens), 1, 1)
+    g.launch()
+    hip.sync()
+    for l, gr0, o, gr in zip(lhs, g0, og, gb):
+        want = oracle.add_unary_grad(d, l.view(np.uint16), gr0.view(np.uint16), o.view(np.uint16), dtype="f16")
+        assert_bits_equal(gr.read().view(np.uint16), want)
+    g.destroy()
 
 
 def test_recorded_dependencies_random(hip, oracle):
