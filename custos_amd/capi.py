@@ -25,6 +25,8 @@ DTYPES = {
     "u16": (9, "uint16"),
     "u32": (10, "uint32"),
     "u64": (11, "uint64"),
+    "f16_pernode": (12, "float16"),
+    "bf16_pernode": (13, "uint16"),
 }
 
 ERR_INVALID_ARGUMENT = 10001

@@ -14,7 +14,9 @@ namespace custos_hip {
 bool op_is_binary(Op op) { return op >= Op::Add && op <= Op::Eq; }
 bool op_is_unary(Op op) { return op >= Op::Sin && op <= Op::Sqrt; }
 
-bool dtype_valid(int32_t v) { return v >= 0 && v <= static_cast<int32_t>(DType::U64); }
+bool dtype_valid(int32_t v) { return v >= 0 && v <= static_cast<int32_t>(DType::BF16_PERNODE); }
+
+bool dtype_rounds_per_node(DType t) { return t == DType::F16_PERNODE || t == DType::BF16_PERNODE; }
 
 size_t dtype_size(DType t) {
     switch (t) {
@@ -26,6 +28,8 @@ size_t dtype_size(DType t) {
         case DType::U32: return 4;
         case DType::F16:
         case DType::BF16:
+        case DType::F16_PERNODE:
+        case DType::BF16_PERNODE:
         case DType::I16:
         case DType::U16: return 2;
         default: return 1;
@@ -33,7 +37,7 @@ size_t dtype_size(DType t) {
 }
 
 bool dtype_is_float(DType t) {
-    return t == DType::F32 || t == DType::F64 || t == DType::F16 || t == DType::BF16;
+    return t == DType::F32 || t == DType::F64 || t == DType::F16 || t == DType::BF16 || dtype_rounds_per_node(t);
 }
 
 bool dtype_is_signed(DType t) {
@@ -47,8 +51,10 @@ const char* dtype_storage_c(DType t) {
         case DType::F64: return "double";
         case DType::I32: return "int";
         case DType::I64: return "long long";
-        case DType::F16: return "_Float16";
-        case DType::BF16: return "unsigned short";
+        case DType::F16:
+        case DType::F16_PERNODE: return "_Float16";
+        case DType::BF16:
+        case DType::BF16_PERNODE: return "unsigned short";
         case DType::U8: return "unsigned char";
         case DType::I8: return "signed char";
         case DType::I16: return "short";
@@ -60,7 +66,7 @@ const char* dtype_storage_c(DType t) {
 }
 
 const char* dtype_compute_c(DType t) {
-    if (t == DType::F16 || t == DType::BF16) return "float";
+    if (t == DType::F16 || t == DType::BF16 || dtype_rounds_per_node(t)) return "float";
     return dtype_storage_c(t);
 }
 
@@ -634,6 +640,12 @@ bool emit_expr_body(const Expr& e, DType dtype, std::string* out, ParseError* er
                 else rhs = "(" + C + ")((" + U + ")0 - (" + U + ")" + t(n.a) + ")";
                 break;
         }
+        // Per-node rounding (what `half`'s f16 / bf16 arithmetic does, src/number.rs:487-676):
+        // every node that computes is rounded to the storage type.  Selects, comparisons,
+        // abs and neg are exact in the storage type already.
+        const bool computes = n.op == Op::Const || n.op == Op::Add || n.op == Op::Sub || n.op == Op::Mul ||
+                              n.op == Op::Div || n.op == Op::Pow || (op_is_unary(n.op) && n.op != Op::Abs && n.op != Op::Neg);
+        if (dtype_rounds_per_node(dtype) && computes) rhs = "custos_round(" + rhs + ")";
         body += "    const " + C + " " + t(static_cast<int>(i)) + " = " + rhs + ";\n";
     }
     body += "    return " + t(e.root) + ";\n";

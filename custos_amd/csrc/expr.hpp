@@ -72,12 +72,15 @@ enum class DType : int32_t {
     U16 = 9,
     U32 = 10,
     U64 = 11,
+    F16_PERNODE = 12,   // f16 storage, every node rounded to f16
+    BF16_PERNODE = 13,  // bf16 storage, every node rounded to bf16
 };
 
 bool dtype_valid(int32_t v);
 size_t dtype_size(DType t);
 bool dtype_is_float(DType t);
 bool dtype_is_signed(DType t);
+bool dtype_rounds_per_node(DType t);  // 16-bit float whose every node is rounded to the storage type
 const char* dtype_storage_c(DType t);  // C type of an element in memory
 const char* dtype_compute_c(DType t);  // C type the nodes are evaluated in
 

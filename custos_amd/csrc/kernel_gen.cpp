@@ -43,7 +43,7 @@ std::string prelude(DType dtype, int vec) {
     s += std::string("typedef ") + dtype_storage_c(dtype) + " S;\n";
     s += std::string("typedef ") + dtype_compute_c(dtype) + " C;\n";
     s += "typedef S vec_t __attribute__((ext_vector_type(" + std::to_string(vec) + ")));\n";
-    if (dtype == DType::BF16) {
+    if (dtype == DType::BF16 || dtype == DType::BF16_PERNODE) {
         s += R"(static __device__ __forceinline__ C custos_load(S s) {
     return __builtin_bit_cast(float, (unsigned int)s << 16);
 }
@@ -58,6 +58,8 @@ static __device__ __forceinline__ S custos_store(C c) {
         s += "static __device__ __forceinline__ C custos_load(S s) { return (C)s; }\n";
         s += "static __device__ __forceinline__ S custos_store(C c) { return (S)c; }\n";
     }
+    if (dtype_rounds_per_node(dtype))
+        s += "static __device__ __forceinline__ C custos_round(C c) { return custos_load(custos_store(c)); }\n";
     if (dtype == DType::F64) {
         s += R"(static __device__ __forceinline__ double custos_sin(double a) { return sin(a); }
 static __device__ __forceinline__ double custos_cos(double a) { return cos(a); }
@@ -77,7 +79,7 @@ static __device__ __forceinline__ double custos_sqrt(double a) { return sqrt(a);
         // tanh / log keep the full-precision routines: their results pass through
         // zero, where only a relative bound in f32 keeps the 16-bit result within
         // one ulp.
-        if (dtype == DType::F16 || dtype == DType::BF16)
+        if (dtype == DType::F16 || dtype == DType::BF16 || dtype_rounds_per_node(dtype))
             s += "static __device__ __forceinline__ float custos_exp(float a) {\n"
                  "    return __builtin_amdgcn_exp2f(a * 0x1.715476p+0f);\n}\n";
         else
@@ -106,6 +108,9 @@ std::string expr_fn(const KernelSpec& k, const std::string& body) {
 // lhs_grad + (out_grad * d): product rounded, then the sum rounded
 // (src/devices/cpu_stack_ops.rs:27-29); integers wrap.
 std::string grad_fn(DType dtype) {
+    if (dtype_rounds_per_node(dtype))
+        return "static __device__ __forceinline__ C custos_grad(const C g, const C o, const C d) {\n"
+               "    const C prod = custos_round(o * d);\n    const C sum = g + prod;\n    return sum;\n}\n";
     if (dtype_is_float(dtype))
         return "static __device__ __forceinline__ C custos_grad(const C g, const C o, const C d) {\n"
                "    const C prod = o * d;\n    const C sum = g + prod;\n    return sum;\n}\n";
@@ -138,7 +143,8 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
         static const char* const dtype_names[] = {"f32", "f64", "i32", "i64", "f16", "bf16",
-                                                  "u8",  "i8",  "i16", "u16", "u32", "u64"};
+                                                  "u8",  "i8",  "i16", "u16", "u32", "u64",
+                                                  "f16n", "bf16n"};
         char hex[17];
         std::snprintf(hex, sizeof hex, "%016llx", static_cast<unsigned long long>(k.hash));
         k.name = std::string(kind == Kind::Apply ? "custos_apply_" : "custos_unary_grad_") +

@@ -69,7 +69,13 @@ enum custos_hip_dtype {
     CUSTOS_HIP_I16 = 8,
     CUSTOS_HIP_U16 = 9,
     CUSTOS_HIP_U32 = 10,
-    CUSTOS_HIP_U64 = 11
+    CUSTOS_HIP_U64 = 11,
+    /* The same storage as F16 / BF16, but every node of the expression is rounded to the
+     * storage type (constants included), the product of the gradient kernel too: what the
+     * reference's `half` arithmetic computes on the CPU and native half arithmetic on a GPU
+     * (src/number.rs:487-676, src/devices/cdatatype.rs:53-62). */
+    CUSTOS_HIP_F16_PERNODE = 12,
+    CUSTOS_HIP_BF16_PERNODE = 13
 };
 
 /* Kernel kinds. */

@@ -29,7 +29,7 @@ DTYPES = {
     "f32": (0, np.float32), "f64": (1, np.float64), "i32": (2, np.int32), "i64": (3, np.int64),
     "f16": (4, np.uint16), "f16_pernode": (5, np.uint16), "u8": (6, np.uint8), "i8": (7, np.int8),
     "i16": (8, np.int16), "u16": (9, np.uint16), "u32": (10, np.uint32), "u64": (11, np.uint64),
-    "bf16": (12, np.uint16),
+    "bf16": (12, np.uint16), "bf16_pernode": (13, np.uint16),
 }
 
 
@@ -73,8 +73,8 @@ def compile_rpn(expr, dtype: str = "f32", eq_mode: str = "eq"):
 
     def const_value(v):
         if isinstance(v, str):
-            v = float(v) if dtype in ("f32", "f64", "f16", "bf16", "f16_pernode") else int(float(v))
-        if dtype in ("f32", "f16", "bf16", "f16_pernode"):
+            v = float(v) if dtype in ("f32", "f64", "f16", "bf16", "f16_pernode", "bf16_pernode") else int(float(v))
+        if dtype in ("f32", "f16", "bf16", "f16_pernode", "bf16_pernode"):
             return float(np.float32(v))
         if dtype == "f64":
             return float(v)

@@ -181,12 +181,24 @@ float oracle_bf16_to_f32(uint16_t h)
 
 #define NO_ROUND(v) (v)
 #define F16_ROUND(v) (oracle_f16_to_f32(oracle_f32_to_f16(v)))
+#define BF16_ROUND(v) (oracle_bf16_to_f32(oracle_f32_to_bf16(v)))
 
 DEFINE_FLOAT_EVAL(eval_f32, float, sinf, cosf, tanf, tanhf, expf, logf, powf, fabsf, sqrtf, NO_ROUND)
 DEFINE_FLOAT_EVAL(eval_f64, double, sin, cos, tan, tanh, exp, log, pow, fabs, sqrt, NO_ROUND)
 /* half crate semantics: convert to f32, f32 libm / f32 arithmetic, round to f16 (src/number.rs:543-608).
- * The reference's f16 `tan` calls `cos` (src/number.rs:575-577); not reproduced here (unpinned mode). */
+ * The reference's f16 `tan` calls `cos` (src/number.rs:575-577); not reproduced here. */
 DEFINE_FLOAT_EVAL(eval_f16_pernode, float, sinf, cosf, tanf, tanhf, expf, logf, powf, fabsf, sqrtf, F16_ROUND)
+/* the same for half::bf16 (src/number.rs:610-676) */
+DEFINE_FLOAT_EVAL(eval_bf16_pernode, float, sinf, cosf, tanf, tanhf, expf, logf, powf, fabsf, sqrtf, BF16_ROUND)
+
+static int eval_16(int dtype, const oracle_ins *prog, int n_prog, const float *vars, int n_vars, float *res)
+{
+    if (dtype == ORC_F16_PERNODE)
+        return eval_f16_pernode(prog, n_prog, vars, n_vars, res);
+    if (dtype == ORC_BF16_PERNODE)
+        return eval_bf16_pernode(prog, n_prog, vars, n_vars, res);
+    return eval_f32(prog, n_prog, vars, n_vars, res);
+}
 
 /* Integer interpreter: arithmetic wraps (Rust release mode), computed in the
  * unsigned counterpart U then cast back to T; transcendental nodes do not
@@ -287,17 +299,17 @@ int oracle_eval_i32(const oracle_ins *prog, int n_prog, const int32_t *vars, int
 static inline float load16(int dtype, const void *p, size_t i)
 {
     uint16_t h = ((const uint16_t *)p)[i];
-    return dtype == ORC_BF16_F32 ? oracle_bf16_to_f32(h) : oracle_f16_to_f32(h);
+    return (dtype == ORC_BF16_F32 || dtype == ORC_BF16_PERNODE) ? oracle_bf16_to_f32(h) : oracle_f16_to_f32(h);
 }
 
 static inline void store16(int dtype, void *p, size_t i, float v)
 {
-    ((uint16_t *)p)[i] = dtype == ORC_BF16_F32 ? oracle_f32_to_bf16(v) : oracle_f32_to_f16(v);
+    ((uint16_t *)p)[i] = (dtype == ORC_BF16_F32 || dtype == ORC_BF16_PERNODE) ? oracle_f32_to_bf16(v) : oracle_f32_to_f16(v);
 }
 
 static inline int is_16bit_float(int dtype)
 {
-    return dtype == ORC_F16_F32 || dtype == ORC_F16_PERNODE || dtype == ORC_BF16_F32;
+    return dtype == ORC_F16_F32 || dtype == ORC_F16_PERNODE || dtype == ORC_BF16_F32 || dtype == ORC_BF16_PERNODE;
 }
 
 #define MAX_IN 4
@@ -336,14 +348,14 @@ int oracle_apply_fn(int dtype, const oracle_ins *prog, int n_prog, const void *c
     case ORC_U64: TYPED_APPLY(uint64_t, eval_u64);
     case ORC_F16_F32:
     case ORC_BF16_F32:
+    case ORC_BF16_PERNODE:
     case ORC_F16_PERNODE: {
         float vars[MAX_IN];
         for (size_t i = 0; i < n; i++) {
             for (int k = 0; k < n_in; k++)
                 vars[k] = load16(dtype, ins[k], i);
             float r;
-            int rc = dtype == ORC_F16_PERNODE ? eval_f16_pernode(prog, n_prog, vars, n_in, &r)
-                                              : eval_f32(prog, n_prog, vars, n_in, &r);
+            int rc = eval_16(dtype, prog, n_prog, vars, n_in, &r);
             if (rc)
                 return rc;
             store16(dtype, out, i, r);
@@ -391,14 +403,14 @@ int oracle_fused_apply_fn(int dtype, const oracle_ins *progs, const int *prog_le
     case ORC_U64: TYPED_FUSED(uint64_t, eval_u64);
     case ORC_F16_F32:
     case ORC_BF16_F32:
+    case ORC_BF16_PERNODE:
     case ORC_F16_PERNODE: {
         for (size_t i = 0; i < n; i++) {
             float cur = load16(dtype, x, i);
             const oracle_ins *p = progs;
             for (int k = 0; k < n_progs; k++) {
                 float r;
-                int rc = dtype == ORC_F16_PERNODE ? eval_f16_pernode(p, prog_lens[k], &cur, 1, &r)
-                                                  : eval_f32(p, prog_lens[k], &cur, 1, &r);
+                int rc = eval_16(dtype, p, prog_lens[k], &cur, 1, &r);
                 if (rc)
                     return rc;
                 cur = r;
@@ -463,14 +475,15 @@ int oracle_add_unary_grad(int dtype, const oracle_ins *prog, int n_prog, const v
         }
         return 0;
     }
+    case ORC_BF16_PERNODE:
     case ORC_F16_PERNODE: {
         for (size_t i = 0; i < n; i++) {
             float v = load16(dtype, lhs, i), d;
-            int rc = eval_f16_pernode(prog, n_prog, &v, 1, &d);
+            int rc = eval_16(dtype, prog, n_prog, &v, 1, &d);
             if (rc)
                 return rc;
             float g = load16(dtype, lhs_grad, i), o = load16(dtype, out_grad, i);
-            float prod = F16_ROUND(o * d);
+            float prod = dtype == ORC_BF16_PERNODE ? BF16_ROUND(o * d) : F16_ROUND(o * d);
             store16(dtype, lhs_grad, i, g + prod);
         }
         return 0;

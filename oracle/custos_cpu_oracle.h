@@ -24,11 +24,19 @@
  *   - f16 <-> f32 conversion: brute force against numpy's float16 (an
  *     independent implementation) over all 65536 halves, all rounding
  *     midpoints and their neighbours.
- *   - OP_*  evaluated per node in f16 (oracle_*_f16_pernode): follows the
- *     third-party `half` crate (2.3) that the reference depends on and that is
- *     not vendored; the reference's tests never exercise f16 values on this
- *     path: PARITY UNPINNED.  The HIP path does not implement this mode; it
- *     implements f32 compute with one final rounding (oracle_*_f16_f32).
+ *   - nodes evaluated per node in f16 / bf16 (ORC_F16_PERNODE, ORC_BF16_PERNODE):
+ *     the third-party `half` crate (2.3) the reference depends on is not
+ *     vendored and the reference's tests never exercise 16-bit values on this
+ *     path.  Its published algorithm (widen to f32, f32 operation, round to
+ *     nearest even) and the reference's own `Float for f16` (`from_f32(
+ *     to_f32().sin())` ..., src/number.rs:543-676) are restated here; for
+ *     + - * / sqrt that equals the correctly rounded 16-bit operation, which
+ *     tests/test_oracle_kats.py checks bit for bit against numpy's float16
+ *     operators and, for bf16, against f32 steps rounded with the integer
+ *     formula.  Not pinned by a reference vector: PARITY UNPINNED for the
+ *     transcendental nodes of these two modes (they compose the pinned f32
+ *     routine with the pinned conversion).  The reference's f16 `tan` calls
+ *     `cos` (src/number.rs:575-577); that defect is not reproduced.
  */
 #ifndef CUSTOS_CPU_ORACLE_H
 #define CUSTOS_CPU_ORACLE_H
@@ -82,14 +90,15 @@ enum oracle_dtype {
     ORC_I32 = 2,
     ORC_I64 = 3,
     ORC_F16_F32 = 4,     /* f16 storage, f32 compute, one RNE rounding at the store */
-    ORC_F16_PERNODE = 5, /* f16 storage, every node rounded to f16 (half crate); parity unpinned */
+    ORC_F16_PERNODE = 5, /* f16 storage, every node rounded to f16 (half crate) */
     ORC_U8 = 6,
     ORC_I8 = 7,
     ORC_I16 = 8,
     ORC_U16 = 9,
     ORC_U32 = 10,
     ORC_U64 = 11,
-    ORC_BF16_F32 = 12    /* bf16 storage, f32 compute, one RNE rounding at the store */
+    ORC_BF16_F32 = 12,   /* bf16 storage, f32 compute, one RNE rounding at the store */
+    ORC_BF16_PERNODE = 13 /* bf16 storage, every node rounded to bf16 (half crate) */
 };
 
 /* out[i] = f(in0[i], in1[i], ...)   -- src/devices/cpu_stack_ops.rs:7-15.

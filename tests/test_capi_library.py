@@ -60,7 +60,8 @@ def test_no_device_means_error_not_fallback():
         custos_amd.HIP(0)
 
 
-@pytest.mark.parametrize("dtype", ["f32", "f64", "f16", "bf16", "i32", "i64", "u8", "i8", "i16", "u16", "u32", "u64"])
+@pytest.mark.parametrize("dtype", ["f32", "f64", "f16", "bf16", "i32", "i64", "u8", "i8", "i16", "u16", "u32", "u64",
+                                   "f16_pernode", "bf16_pernode"])
 def test_offline_compile_every_dtype(dtype):
     text = "((x * 2) + 1)" if dtype[0] in "iu" else "sqrt(abs(((x * 2.0) + 1.0)))"
     assert capi.expr_build_code_object(capi.KIND_APPLY, dtype, text, ["x"]) > 1000

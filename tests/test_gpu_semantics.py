@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 from custos_amd import Const, capi, synth
-from tests.helpers import assert_bits_equal, ulp_distance_f32
+from tests.helpers import assert_bits_equal, ulp_distance_f16, ulp_distance_f32
 
 pytestmark = pytest.mark.gpu
 
@@ -447,3 +447,46 @@ def test_more_than_2p32_bytes_and_elements(hip):
         assert_bits_equal(got, np.roll(want, -off), f"window at {start}")
     tail = out.slice(n - 77, n).read()
     assert_bits_equal(tail, np.roll(want, -((n - 77) % (1 << 20)))[:77])
+
+
+@pytest.mark.parametrize("dtype", ["f16_pernode", "bf16_pernode"])
+def test_per_node_rounding_of_16bit_floats(hip, oracle, dtype):
+    """Every node rounded to the storage type, what the reference's `half` arithmetic does
+    (src/number.rs:487-676).  + - * / sqrt of 16-bit operands computed in f32 and rounded once
+    are the correctly rounded 16-bit results, so these chains are bit-exact against the CPU
+    restatement; they differ from the f32-compute mode, which rounds only at the store."""
+    n = 50003
+    base = dtype.split("_")[0]
+    if base == "f16":
+        xb = synth.uniform_f16_bits(21, n, -3, 3)
+        yb = synth.uniform_f16_bits(22, n, 0.5, 2)
+    else:
+        xb = (synth.uniform_f32(21, n, -3, 3).view(np.uint32) >> 16).astype(np.uint16)
+        yb = (synth.uniform_f32(22, n, 0.5, 2).view(np.uint32) >> 16).astype(np.uint16)
+    view = (lambda a: a.view(np.float16)) if base == "f16" else (lambda a: a)
+    f = lambda a, b: a.mul(0.3).add(b).mul(a).div(b.add(1.7)).sub(0.1).abs().sqrt().max(0.25).neg()
+    x, y = hip.buffer(view(xb), dtype), hip.buffer(view(yb), dtype)
+    got = hip.apply_fn2(x, y, f).read().view(np.uint16)
+    assert_bits_equal(got, oracle.apply_fn(f, xb, yb, dtype=dtype))
+    once = hip.apply_fn2(hip.buffer(view(xb), base), hip.buffer(view(yb), base), f).read().view(np.uint16)
+    assert (once != got).mean() > 0.01          # the two modes really differ
+    assert_bits_equal(once, oracle.apply_fn(f, xb, yb, dtype=base))
+
+    # gradient: the product is rounded too, then the sum
+    d = lambda v: v.mul(v).mul(3.0).add(0.7)
+    g0 = (yb ^ 0x8000).astype(np.uint16)
+    gb = hip.buffer(view(g0), dtype)
+    hip.add_unary_grad(x, gb, y, d)
+    assert_bits_equal(gb.read().view(np.uint16), oracle.add_unary_grad(d, xb, g0, yb, dtype=dtype))
+
+    # transcendentals: f32 routine then one rounding; within one unit of the 16-bit type
+    t = lambda v: v.sin().mul(v.mul(0.25).exp()).add(v.tanh())
+    got = hip.apply_fn(x, t).read().view(np.uint16)
+    want = oracle.apply_fn(t, xb, dtype=dtype)
+    if base == "f16":
+        dist = ulp_distance_f16(got, want)
+    else:
+        key = lambda b: np.where(b & 0x8000, 0x8000 - (b & 0x7fff).astype(np.int32), 0x8000 + (b & 0x7fff).astype(np.int32))
+        dist = np.abs(key(got) - key(want))
+    # a chain of three rounded nodes: one unit of disagreement in a node can move the result
+    assert dist.max() <= 2 and (dist == 0).mean() > 0.98

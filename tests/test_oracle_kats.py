@@ -227,6 +227,54 @@ def test_bf16_conversion(oracle):
     assert l.oracle_f32_to_bf16(float(np.uint32(0x3F818000).view(np.float32))) == 0x3F82
 
 
+def test_per_node_rounding_against_independent_half_arithmetic(oracle):
+    """The per-node modes (every node rounded to the storage type, src/number.rs:487-676) against
+    arithmetic that does not go through the restatement: numpy's float16 operators are IEEE
+    binary16 operations, and for + - * / sqrt "f32 operation, then one rounding" IS the correctly
+    rounded 16-bit operation (24 >= 2*11 + 2 significand bits), so both must agree bit for bit.
+    bf16 has no numpy type: each step is done in f32 and rounded with the integer formula."""
+    from custos_amd import synth
+    n = 20011
+    xb = synth.uniform_f16_bits(31, n, -3, 3)
+    yb = synth.uniform_f16_bits(32, n, 0.5, 2)
+    f = lambda a, b: a.mul(0.3).add(b).mul(a).div(b.add(1.7)).sub(0.1).abs().sqrt().max(0.25).neg()
+    x, y = xb.view(np.float16), yb.view(np.float16)
+    h = np.float16
+    with np.errstate(all="ignore"):
+        r = np.sqrt(np.abs(((x * h(0.3) + y) * x) / (y + h(1.7)) - h(0.1)))
+        r = -np.where(r > h(0.25), r, h(0.25))
+    assert r.dtype == np.float16
+    assert_bits_equal(oracle.apply_fn(f, xb, yb, dtype="f16_pernode"), r.view(np.uint16))
+    # the f32-compute mode rounds once and gives other bits for a good part of the inputs
+    assert (oracle.apply_fn(f, xb, yb, dtype="f16") != r.view(np.uint16)).mean() > 0.01
+
+    def bf(v):  # f32 -> nearest-even bf16 -> f32 (finite values)
+        u = np.asarray(v, dtype=np.float32).view(np.uint32).astype(np.uint64)
+        u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16 << 16
+        return u.astype(np.uint32).view(np.float32)
+
+    xs = bf(synth.uniform_f32(33, n, -3, 3))
+    ys = bf(synth.uniform_f32(34, n, 0.5, 2))
+    f32 = np.float32
+    with np.errstate(all="ignore"):
+        t = bf(xs * bf(f32(0.3)))
+        t = bf(t + ys)
+        t = bf(t * xs)
+        t = bf(t / bf(ys + bf(f32(1.7))))
+        t = bf(t - bf(f32(0.1)))
+        t = bf(np.sqrt(np.abs(t)))
+        t = -np.where(t > f32(0.25), t, f32(0.25))
+    to_bits = lambda v: (v.view(np.uint32) >> 16).astype(np.uint16)
+    assert_bits_equal(oracle.apply_fn(f, to_bits(xs), to_bits(ys), dtype="bf16_pernode"), to_bits(t))
+
+    # gradient: g + round(o * d), both per-node (src/devices/cpu_stack_ops.rs:27-29 in 16-bit arithmetic)
+    d = lambda v: v.mul(v).mul(3.0).add(0.7)
+    g0 = synth.uniform_f16_bits(35, n, -1, 1)
+    with np.errstate(all="ignore"):
+        want = g0.view(np.float16) + y * ((x * x) * h(3.0) + h(0.7))
+    assert_bits_equal(oracle.add_unary_grad(d, xb, g0, yb, dtype="f16_pernode"), want.view(np.uint16))
+
+
 def test_integer_wrap(oracle):
     out = oracle.apply_fn(lambda x: x.mul(2), [2 ** 30, -(2 ** 30) - 1], dtype="i32")
     assert out.tolist() == [-(2 ** 31), 2 ** 31 - 2]
