@@ -169,3 +169,93 @@ def test_c2_full_size_properties(hip, oracle, log2n):
     for k in range(0, n // period, 37):
         bits ^= out.slice(k * period, (k + 1) * period).read().view(np.uint32) ^ first.view(np.uint32)
     assert not bits.any()
+
+
+def _replicate(hip, base, n, dtype="f32"):
+    """A device buffer of n elements holding `base` repeated (device-side doubling copies)."""
+    period = base.size
+    buf = hip.alloc(n, dtype, zeroed=False)
+    hip.copy(buf.slice(0, period), hip.buffer(base, dtype))
+    filled = period
+    while filled < n:
+        hip.copy(buf.slice(filled, 2 * filled), buf.slice(0, filled))
+        filled *= 2
+    return buf
+
+
+def _all_windows_equal(buf, period, first, stride=29):
+    """Every window of `period` elements holds the bits of `first` (sampled every `stride` windows
+    plus the last one)."""
+    bits = first.view(f"u{first.itemsize}")
+    windows = list(range(0, buf.len // period, stride)) + [buf.len // period - 1]
+    for k in windows:
+        got = buf.slice(k * period, (k + 1) * period).read().view(bits.dtype)
+        if not np.array_equal(got, bits):
+            return False
+    return True
+
+
+def test_c3_full_size_properties(hip, oracle):
+    """configs[2] at the full N = 2^26: forward and backward over a periodic input give a periodic
+    output whose first window matches the oracle; the gradient accumulates (a second backward
+    adds the same amount again)."""
+    n, period = 1 << 26, 1 << 18
+    x = synth.normal_f32(0, period)
+    yg = synth.uniform_f32(1, period, -1, 1)
+    xb, ygb = _replicate(hip, x, n), _replicate(hip, yg, n)
+    gb = _replicate(hip, np.full(period, 0.1, dtype=np.float32), n)
+    y = hip.apply_fn(xb, lambda v: v.tanh())
+    first = y.slice(0, period).read()
+    assert ulp_distance_f32(first, oracle.c3_tanh_fwd(x)).max() <= 4
+    assert _all_windows_equal(y, period, first)
+    hip.add_unary_grad(xb, gb, ygb, TANH_GRAD)
+    g1 = gb.slice(0, period).read()
+    want = oracle.c3_tanh_bwd(x, np.full(period, 0.1, dtype=np.float32), yg)
+    assert np.max(np.abs(g1.astype(np.float64) - want.astype(np.float64))) <= 12 * 2.0 ** -24
+    assert _all_windows_equal(gb, period, g1)
+    hip.add_unary_grad(xb, gb, ygb, TANH_GRAD)
+    g2 = gb.slice(0, period).read()
+    step = (g1 - np.float32(0.1)).astype(np.float32)
+    assert np.max(np.abs(g2.astype(np.float64) - (g1.astype(np.float64) + step))) <= 4 * 2.0 ** -24
+    assert _all_windows_equal(gb, period, g2)
+
+
+def test_c4_full_size_properties(hip, oracle):
+    """configs[3] at the full N = 2^28 (f16 storage): periodic input, periodic output, first
+    window within one f16 unit of the oracle."""
+    n, period = 1 << 28, 1 << 20
+    xbits = synth.uniform_f16_bits(0, period, -2, 2)
+    xb = _replicate(hip, xbits.view(np.float16), n, "f16")
+    out = hip.apply_fn(xb, C4)
+    first = out.slice(0, period).read()
+    d = ulp_distance_f16(first.view(np.uint16), oracle.c4_chain_f16(xbits))
+    assert d.max() <= 1 and (d == 0).mean() > 0.99
+    assert _all_windows_equal(out, period, first)
+
+
+def test_c5_full_size_graph(hip, oracle):
+    """configs[4] at its full shape, 1024 buffers of 4096 f32: three kernel nodes for 3072
+    recorded launches, 100 replays, bit-exact against the oracle after the first and the last."""
+    nbuf, m = 1024, 4096
+    a = synth.uniform_f32(1, nbuf * m, 0, 1)
+    b = synth.uniform_f32(2, nbuf * m, 0, 1)
+    c = synth.uniform_f32(3, nbuf * m, 0, 1)
+    A, B, Cc = hip.buffer(a), hip.buffer(b), hip.buffer(c)
+    T, U, Y = hip.alloc(nbuf * m), hip.alloc(nbuf * m), hip.alloc(nbuf * m)
+    hip.capture_begin()
+    for i in range(nbuf):
+        s = slice(i * m, (i + 1) * m)
+        hip.apply_fn2(A.slice(s.start, s.stop), B.slice(s.start, s.stop), lambda p, q: p.mul(q), out=T.slice(s.start, s.stop))
+        hip.apply_fn2(T.slice(s.start, s.stop), Cc.slice(s.start, s.stop), lambda p, q: p.add(q), out=U.slice(s.start, s.stop))
+        hip.fused_apply_fn(U.slice(s.start, s.stop), [lambda v: v.abs().sqrt(), lambda v: v.mul(0.3)], out=Y.slice(s.start, s.stop))
+    g = hip.capture_end()
+    assert g.stats() == (3 * nbuf, 3, 3)
+    _, _, want = oracle.c5_graph(a, b, c)
+    for replay in range(100):
+        if replay in (0, 99):
+            Y.clear()
+        g.launch()
+        if replay in (0, 99):
+            hip.sync()
+            assert_bits_equal(Y.read(), want, f"replay {replay}")
+    g.destroy()
