@@ -99,7 +99,7 @@ def bench_c2(dev, args):
     from custos_amd.expr import fused_source
 
     n = 1 << args.log2n
-    tuned = bool(args.block or args.unroll or args.blocks_per_cu or args.nontemporal)
+    tuned = bool(args.block or args.unroll or args.blocks_per_cu or args.nontemporal or args.direction)
     x = gen_chunked(lambda m, off: synth.uniform_f32(0, m, -np.pi, np.pi, off), n)
     xb = dev.buffer(x)
     out = dev.alloc(n, "f32")
@@ -111,18 +111,10 @@ def bench_c2(dev, args):
     def fused_step():
         capi.check(lib.custos_hip_apply_fn(h, kernel, xb.ptr, out.ptr, n), h)
 
-    # One step = what `Lazy::run` does from the second run on: replay the graph that holds the
-    # fused kernel.  (The first run records and instantiates it; that is outside the timed region.)
-    dev.capture_begin()
-    fused_step()
-    graph = dev.capture_end()
-    assert graph.kernel_nodes == 1
-    ms, wall_ms = time_steps(dev, graph.launch, args.steps, args.warmup)
-    per_launch_ms = ms / args.steps
-    dms, _ = time_steps(dev, fused_step, args.steps, args.warmup)   # the same kernel launched directly
-    direct_ms = dms / args.steps
     algo_bytes = 8.0 * n
-    gbs = algo_bytes / (per_launch_ms * 1e-3) / 1e9
+
+    # The comparisons run first (they also bring the device to its steady clocks: the first
+    # ~30 ms of back-to-back launches after start-up run up to 15 % slower), the headline last.
 
     # unfused comparison: five apply_fn launches through intermediates (40 B/elt moved)
     kernels = [dev.compile(capi.KIND_APPLY, "f32", custos_amd.expr._wrap(op(custos_amd.Resolve("x"))).to_cl_source("f32"), ("x",))
@@ -146,6 +138,39 @@ def bench_c2(dev, args):
 
     cms, _ = time_steps(dev, copy_step, max(1, args.steps // 2), max(1, args.warmup // 2))
     copy_ms = cms / max(1, args.steps // 2)
+
+    # The fused step with the launch shape pinned to plain HBM streaming: every launch walks the
+    # array from the first tile to the last, non-temporal accesses, two vectors per thread.  (By
+    # default every launch of this size walks the array against the direction of the launch
+    # before it and so starts on the last 256 MiB the memory-side cache still holds.)
+    streaming = None
+    if not tuned:
+        dev.set_tuning(0, 2, 0, 3, 1)
+        skernel = dev.compile(capi.KIND_APPLY, "f32", src, ("x",))
+        dev.capture_begin()
+        capi.check(lib.custos_hip_apply_fn(h, skernel, xb.ptr, out.ptr, n), h)
+        sgraph = dev.capture_end()
+        sms, _ = time_steps(dev, sgraph.launch, args.steps, args.warmup)
+        sgraph.destroy()
+        dev.set_tuning(0, 0, 0, 0, 0)
+        streaming = {"ms_per_step": round(sms / args.steps, 5),
+                     "GBps": round(algo_bytes / (sms / args.steps * 1e-3) / 1e9, 2),
+                     "kernel": dev.kernel_name(skernel),
+                     "shape": "tiles first to last, non-temporal loads and stores, 2 vectors per thread"}
+
+    dms, _ = time_steps(dev, fused_step, args.steps, args.warmup)   # the fused kernel launched directly
+    direct_ms = dms / args.steps
+
+    # Headline.  One step = what `Lazy::run` does from the second run on: replay the graph that
+    # holds the fused kernel.  (The first run records and builds it; that is outside the timed region.)
+    dev.capture_begin()
+    fused_step()
+    graph = dev.capture_end()
+    assert graph.kernel_nodes == 1
+    ms, wall_ms = time_steps(dev, graph.launch, args.steps, args.warmup)
+    per_launch_ms = ms / args.steps
+    graph.destroy()
+    gbs = algo_bytes / (per_launch_ms * 1e-3) / 1e9
 
     # parity of the very buffer that was timed, on the CPU sample
     fused_step()
@@ -171,6 +196,7 @@ def bench_c2(dev, args):
         "elements_per_s": round(n / (per_launch_ms * 1e-3), 1),
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
         "direct_launch": {"ms_per_step": round(direct_ms, 5), "GBps": round(algo_bytes / (direct_ms * 1e-3) / 1e9, 2)},
+        "hbm_streaming_only": streaming,
         "unfused": {
             "ms_per_step": round(unfused_ms, 5),
             "effective_GBps_on_8B_basis": round(algo_bytes / (unfused_ms * 1e-3) / 1e9, 2),
@@ -178,7 +204,7 @@ def bench_c2(dev, args):
             "speedup_fused": round(unfused_ms / per_launch_ms, 3),
         },
         "copy_kernel": {
-            "name": dev.kernel_name(copy_kernel),
+            "name": dev.kernel_name(copy_kernel, n),
             "ms_per_launch": round(copy_ms, 5),
             "GBps": round(algo_bytes / (copy_ms * 1e-3) / 1e9, 2),
             "bytes_per_launch": algo_bytes,
@@ -191,7 +217,7 @@ def bench_c2(dev, args):
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC_C2_N2P28 if (args.log2n == 28 and not tuned) else None,
-            "kernel": dev.kernel_name(kernel),
+            "kernel": dev.kernel_name(kernel, n),
             "algorithmic_bytes_per_launch": algo_bytes,
             "avg_launch_ms": round(per_launch_ms, 5),
         },
@@ -245,7 +271,7 @@ def bench_others(dev, args):
     got = ob.read()
     assert np.max(np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))) <= 4
     out["c1"] = _entry("c1: apply_fn(exp), f32 N=2^20, U[-4,4) seed 0", n, 8, ms / (steps * 4), cpu_s, n)
-    out["c1"]["kernel"] = dev.kernel_name(k)
+    out["c1"]["kernel"] = dev.kernel_name(k, n)
 
     # c3: unary_ew tanh forward + backward, f32 N = 2^26
     n = 1 << 26
@@ -269,9 +295,9 @@ def bench_others(dev, args):
     cpu_s, _ = _cpu_time(lambda: (cpu_oracle.c3_tanh_fwd(x[:cn]), cpu_oracle.c3_tanh_bwd(x[:cn], g0, yg[:cn])))
     e = _entry("c3: unary_ew tanh fwd + bwd (x_grad += y_grad*(1-tanh(x)^2)), f32 N=2^26", n, 24, ms / steps, cpu_s, cn)
     e["forward"] = {"ms": round(ms_f / steps, 5), "GBps": round(8 * n / (ms_f / steps * 1e-3) / 1e9, 2),
-                    "kernel": dev.kernel_name(kf)}
+                    "kernel": dev.kernel_name(kf, n)}
     e["backward"] = {"ms": round(ms_b / steps, 5), "GBps": round(16 * n / (ms_b / steps * 1e-3) / 1e9, 2),
-                     "kernel": dev.kernel_name(kb)}
+                     "kernel": dev.kernel_name(kb, n)}
     out["c3"] = e
     del xb, ygb, yb, gb
 
@@ -288,7 +314,7 @@ def bench_others(dev, args):
     d = np.abs(got.view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
     assert d.max() <= 1, "c4 differs from the CPU port by more than 1 f16 ulp"
     out["c4"] = _entry(f"c4: f16 chain exp(x*0.5)*x + x^2, f32 compute, N=2^{args.log2n}", n, 4, ms / steps, cpu_s, cn)
-    out["c4"]["kernel"] = dev.kernel_name(k)
+    out["c4"]["kernel"] = dev.kernel_name(k, n)
     del xb, ob
 
     # c5: 1024 buffers x 4096 f32: t=a*b; u=t+c; y=sqrt(abs(u))*0.3, one graph, 100 replays
@@ -320,7 +346,7 @@ def bench_others(dev, args):
     e["graph_kernel_nodes"] = graph.kernel_nodes
     e["recorded_launches"] = 3 * nbuf
     e["graph_build_ms"] = round(build_s * 1e3, 2)
-    e["kernels"] = [dev.kernel_name(q) + "_batched" for q in (kmul, kadd, kun)]
+    e["kernels"] = [dev.kernel_name(q, nbuf * m) + "_batched" for q in (kmul, kadd, kun)]
     graph.destroy()
 
     # the same work after element-wise fusing (what `Lazy::elementwise_fusing` of the host stack
@@ -341,7 +367,7 @@ def bench_others(dev, args):
         "GBps": round(16 * nbuf * m / (fms / replays * 1e-3) / 1e9, 2),
         "graph_kernel_nodes": fgraph.kernel_nodes,
         "expression": "(sqrt(abs(((a * b) + c))) * 0.3)",
-        "kernel": dev.kernel_name(kf) + "_batched",
+        "kernel": dev.kernel_name(kf, nbuf * m) + "_batched",
     }
     out["c5"] = e
     fgraph.destroy()
@@ -363,6 +389,8 @@ def main():
     ap.add_argument("--unroll", type=int, default=0)
     ap.add_argument("--blocks-per-cu", dest="blocks_per_cu", type=int, default=0)
     ap.add_argument("--nontemporal", type=int, default=0)
+    ap.add_argument("--direction", type=int, default=0,
+                    help="1: tiles first to last; 2: every launch the other way round; 0: library default")
     ap.add_argument("--no-others", dest="others", action="store_false",
                     help="skip the other BASELINE configurations (c1, c3, c4, c5)")
     args = ap.parse_args()
@@ -375,8 +403,8 @@ def main():
     dev = custos_amd.HIP(0)
     if args.direct_replay is not None:
         dev.set_graph_direct_replay(args.direct_replay)
-    if args.block or args.unroll or args.blocks_per_cu or args.nontemporal:
-        dev.set_tuning(args.block, args.unroll, args.blocks_per_cu, args.nontemporal)
+    if args.block or args.unroll or args.blocks_per_cu or args.nontemporal or args.direction:
+        dev.set_tuning(args.block, args.unroll, args.blocks_per_cu, args.nontemporal, args.direction)
     info = dev.info()
     res = {"c2": bench_c2}[args.workload](dev, args)
     if args.others:

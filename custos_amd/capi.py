@@ -70,6 +70,7 @@ class Tuning(C.Structure):
         ("unroll", C.c_int32),
         ("blocks_per_cu", C.c_int32),
         ("nontemporal", C.c_int32),
+        ("direction", C.c_int32),
     ]
 
 
@@ -103,6 +104,7 @@ PROTOTYPES = {
     "custos_hip_kernel_source": (C.c_char_p, [_P]),
     "custos_hip_kernel_name": (C.c_char_p, [_P]),
     "custos_hip_kernel_hash": (C.c_uint64, [_P]),
+    "custos_hip_kernel_launched_as": (C.c_int32, [_P, _P, C.c_size_t, C.POINTER(C.c_void_p)]),
     "custos_hip_kernel_arity": (C.c_int32, [_P]),
     "custos_hip_cache_stats": (C.c_int32, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "custos_hip_cache_disk_hits": (C.c_int32, [_P, C.POINTER(C.c_uint64)]),

@@ -120,7 +120,7 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
     HIP_TRY(nullptr, hipSetDevice(idx));
     HIP_TRY(nullptr, hipGetDeviceProperties(&dev->props, idx));
     dev->arch = dev->props.gcnArchName;
-    dev->tuning = normalize_tuning(0, 0, 0, 0);
+    dev->tuning = normalize_tuning(0, 0, 0, 0, 0);
     HIP_TRY(nullptr, hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking));
     HIP_TRY(nullptr, hipStreamCreateWithFlags(&dev->transfer, hipStreamNonBlocking));
     HIP_TRY(nullptr, hipEventCreate(&dev->t0));
@@ -186,7 +186,8 @@ int32_t custos_hip_get_tuning(custos_hip_device* dev, custos_hip_tuning* tuning)
     tuning->block_threads = dev->tuning.block_threads;
     tuning->unroll = dev->tuning.unroll;
     tuning->blocks_per_cu = dev->tuning.blocks_per_cu;
-    tuning->nontemporal = dev->tuning.nontemporal;
+    tuning->nontemporal = dev->tuning.nontemporal < 0 ? 0 : dev->tuning.nontemporal == 0 ? -1 : dev->tuning.nontemporal;
+    tuning->direction = dev->tuning.direction;
     return CUSTOS_HIP_OK;
 }
 

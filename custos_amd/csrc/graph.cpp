@@ -92,11 +92,23 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
         size_t table_offset = 0;      // in u64 entries
         size_t map_offset = 0;        // ragged: start of the block map, in u64 entries
         size_t blocks = 0;            // ragged: workgroups
+        custos_hip_kernel* kern = nullptr;  // kernels: the variant that suits the bytes the node touches
+        bool alternate = false;             // kernels: walks its tiles against the previous such node
     };
-    auto tiles_of = [](const RecNode& n) {
-        const Tuning& t = n.k->spec.tuning;
+    auto tiles_of = [](const custos_hip_kernel* k, const RecNode& n) {
+        const Tuning& t = k->spec.tuning;
         const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
         return std::max(1ull, (n.n_vec + tile_vecs - 1) / tile_vecs);
+    };
+    // the launch shape follows the bytes the (merged) launch touches
+    auto choose_kernel = [&](Planned& p) {
+        const RecNode& first = nodes[p.members[0]];
+        if (first.type != RecNode::Kernel) return;
+        unsigned long long footprint = 0;
+        for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
+        custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate);
+        const bool usable = p.members.size() == 1 || (p.ragged ? v->fn_ragged != nullptr : v->fn_batched != nullptr);
+        p.kern = usable ? v : first.k;
     };
     std::vector<std::vector<Planned>> plan(static_cast<size_t>(max_level + 1));
     std::vector<uint64_t> host_table;
@@ -141,7 +153,7 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
             // chip on its own stays a launch of its own
             merged.ragged = true;
             for (size_t i : g.second) {
-                if (tiles_of(nodes[i]) > kRaggedMaxTiles) {
+                if (tiles_of(nodes[i].k, nodes[i]) > kRaggedMaxTiles) {
                     out.emplace_back();
                     out.back().members.push_back(i);
                 } else {
@@ -152,6 +164,7 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
             if (!merged.members.empty()) out.push_back(std::move(merged));
         }
         for (Planned& p : out) {
+            choose_kernel(p);
             if (p.members.size() < 2) continue;
             p.table_offset = host_table.size();
             for (size_t seg = 0; seg < p.members.size(); seg++) {
@@ -162,7 +175,7 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
             if (!p.ragged) continue;
             p.map_offset = host_table.size();
             for (size_t seg = 0; seg < p.members.size(); seg++) {
-                const unsigned long long tiles = tiles_of(nodes[p.members[seg]]);
+                const unsigned long long tiles = tiles_of(p.kern, nodes[p.members[seg]]);
                 for (unsigned long long t = 0; t < tiles; t++) host_table.push_back(static_cast<uint64_t>(seg) << 32 | t);
             }
             p.blocks = host_table.size() - p.map_offset;
@@ -179,12 +192,15 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
         return std::vector<unsigned char>(c, c + n);
     };
     std::vector<std::vector<LoweredNode>> lowered(plan.size());
+    unsigned long long parity = 0;
     size_t total = 0;
     bool chain = true;
     for (int level = 0; level <= max_level; level++) {
         for (const Planned& p : plan[level]) {
             const RecNode& first = nodes[p.members[0]];
             LoweredNode ln;
+            // a node that alternates runs against the direction of the one before it
+            const unsigned long long rev = (first.type == RecNode::Kernel && p.alternate) ? (parity ^= 1) : 0;
             if (first.type == RecNode::Copy) {
                 ln.is_copy = true;
                 ln.dst = first.ptrs[0];
@@ -209,20 +225,21 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
                 ln.args.push_back(value(&a0, 8));
                 ln.args.push_back(value(&a1, 8));
                 ln.args.push_back(value(&a2, 8));
-                ln.func = reinterpret_cast<void*>(first.k->fn);
-                ln.grid = dim3(first.grid);
-                ln.block = dim3(static_cast<unsigned int>(first.k->spec.tuning.block_threads));
+                ln.args.push_back(value(&rev, 8));
+                ln.func = reinterpret_cast<void*>(p.kern->fn);
+                ln.grid = dim3(launch_grid(dev, p.kern, first.n, first.n_vec));
+                ln.block = dim3(static_cast<unsigned int>(p.kern->spec.tuning.block_threads));
             } else if (p.ragged) {
                 if (p.blocks > (1ull << 31) - 1)
                     return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
                 const uint64_t table = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
                 const uint64_t map = reinterpret_cast<uint64_t>(g->table) + p.map_offset * sizeof(uint64_t);
-                ln.args = {value(&table, 8), value(&map, 8)};
-                ln.func = reinterpret_cast<void*>(first.k->fn_ragged);
+                ln.args = {value(&table, 8), value(&map, 8), value(&rev, 8)};
+                ln.func = reinterpret_cast<void*>(p.kern->fn_ragged);
                 ln.grid = dim3(static_cast<unsigned int>(p.blocks));
-                ln.block = dim3(static_cast<unsigned int>(first.k->spec.tuning.block_threads));
+                ln.block = dim3(static_cast<unsigned int>(p.kern->spec.tuning.block_threads));
             } else {
-                const Tuning& t = first.k->spec.tuning;
+                const Tuning& t = p.kern->spec.tuning;
                 const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
                 const unsigned long long tiles_per_seg = std::max(1ull, (first.n_vec + tile_vecs - 1) / tile_vecs);
                 const unsigned long long blocks = tiles_per_seg * p.members.size();
@@ -230,11 +247,12 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
                     return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a batched launch would need more than 2^31 workgroups");
                 const uint64_t table = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
                 const unsigned long long a0 = first.n, a1 = first.n_vec;
-                ln.args = {value(&table, 8), value(&a0, 8), value(&a1, 8), value(&tiles_per_seg, 8)};
-                ln.func = reinterpret_cast<void*>(first.k->fn_batched);
+                ln.args = {value(&table, 8), value(&a0, 8), value(&a1, 8), value(&tiles_per_seg, 8), value(&rev, 8)};
+                ln.func = reinterpret_cast<void*>(p.kern->fn_batched);
                 ln.grid = dim3(static_cast<unsigned int>(blocks));
                 ln.block = dim3(static_cast<unsigned int>(t.block_threads));
             }
+            if (first.type == RecNode::Kernel && p.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
             if (!ln.is_copy) g->kernel_nodes++;
             lowered[level].push_back(std::move(ln));
             total++;
@@ -244,6 +262,11 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
 
     if (chain && total <= dev->direct_replay_max) {
         for (auto& level : lowered) g->direct.push_back(std::move(level[0]));
+        // With an odd number of alternating nodes the first one of the next replay would
+        // run in the direction of the last one of this replay: flip them all every replay.
+        size_t alternating = 0;
+        for (const LoweredNode& ln : g->direct) alternating += ln.rev_arg >= 0;
+        g->flip_each_replay = alternating % 2 == 1;
         return CUSTOS_HIP_OK;
     }
 
@@ -295,6 +318,7 @@ int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
                                         hipMemcpyDeviceToDevice, dev->stream));
             continue;
         }
+        if (ln.rev_arg >= 0 && g->flip_each_replay) ln.args[ln.rev_arg][0] ^= 1;
         std::vector<void*> argv(ln.args.size());
         for (size_t i = 0; i < ln.args.size(); i++) argv[i] = ln.args[i].data();
         void** args = argv.data();

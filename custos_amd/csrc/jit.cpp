@@ -178,6 +178,71 @@ int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k) {
     return CUSTOS_HIP_OK;
 }
 
+// Parses, looks the structural key up in the cache, compiles on a miss.
+static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
+                            const char* const* markers, int32_t n_markers, const Tuning& tuning,
+                            custos_hip_kernel** out) {
+    std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
+    int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, &k->spec);
+    if (rc != CUSTOS_HIP_OK) return rc;
+
+    auto& bucket = dev->cache[k->spec.hash];
+    for (auto& cached : bucket) {
+        // the generated text starts with the caller's spelling of the expression
+        // as a comment; compare what is compiled, i.e. everything after it
+        const std::string& a = cached->spec.source;
+        const std::string& b = k->spec.source;
+        if (a.compare(a.find('\n'), std::string::npos, b, b.find('\n'), std::string::npos) == 0) {
+            dev->hits++;
+            *out = cached.get();
+            return CUSTOS_HIP_OK;
+        }
+    }
+    rc = build_module(dev, k.get());
+    if (rc != CUSTOS_HIP_OK) return rc;
+    // further entry points of the module: many launches in one grid
+    if (hipModuleGetFunction(&k->fn_batched, k->module, (k->spec.name + "_batched").c_str()) != hipSuccess) {
+        (void)hipGetLastError();
+        k->fn_batched = nullptr;
+    }
+    if (hipModuleGetFunction(&k->fn_ragged, k->module, (k->spec.name + "_ragged").c_str()) != hipSuccess) {
+        (void)hipGetLastError();
+        k->fn_ragged = nullptr;
+    }
+    k->expr_src = src;
+    for (int i = 0; i < n_markers; i++) k->markers.push_back(markers[i]);
+    *out = k.get();
+    bucket.push_back(std::move(k));
+    return CUSTOS_HIP_OK;
+}
+
+custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
+                                  bool* alternate) {
+    const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;
+    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands);
+    const int direction = dev->tuning.direction;
+    *alternate = direction == 2 || (direction == 0 && shape.alternate);
+    if (k->spec.kind == Kind::Source || (!k->spec.auto_unroll && !k->spec.auto_nt)) return k;
+    Tuning t = k->spec.tuning;
+    if (k->spec.auto_unroll) t.unroll = shape.unroll;
+    if (k->spec.auto_nt) t.nontemporal = shape.nontemporal;
+    if (t.unroll == k->spec.tuning.unroll && t.nontemporal == k->spec.tuning.nontemporal) return k;
+    const int key = t.unroll * 8 + t.nontemporal;
+    for (const auto& v : k->variants)
+        if (v.first == key) return v.second ? v.second : k;
+    std::vector<const char*> m;
+    for (const std::string& s : k->markers) m.push_back(s.c_str());
+    const std::string keep = dev->last_error;
+    custos_hip_kernel* made = nullptr;
+    if (compile_expr(dev, static_cast<int32_t>(k->spec.kind), static_cast<int32_t>(k->spec.dtype), k->expr_src.c_str(),
+                     m.data(), static_cast<int32_t>(m.size()), t, &made) != CUSTOS_HIP_OK) {
+        made = nullptr;  // the first kernel serves this size too
+        dev->last_error = keep;
+    }
+    k->variants.push_back({key, made});
+    return made ? made : k;
+}
+
 }  // namespace custos_hip
 
 using namespace custos_hip;
@@ -206,37 +271,11 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
             return CUSTOS_HIP_OK;
         }
     }
-    std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
-    int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, dev->tuning, &k->spec);
+    custos_hip_kernel* k = nullptr;
+    int32_t rc = compile_expr(dev, kind, dtype, src, markers, n_markers, dev->tuning, &k);
     if (rc != CUSTOS_HIP_OK) return rc;
-
-    auto& bucket = dev->cache[k->spec.hash];
-    for (auto& cached : bucket) {
-        // the generated text starts with the caller's spelling of the expression
-        // as a comment; compare what is compiled, i.e. everything after it
-        const std::string& a = cached->spec.source;
-        const std::string& b = k->spec.source;
-        if (a.compare(a.find('\n'), std::string::npos, b, b.find('\n'), std::string::npos) == 0) {
-            dev->hits++;
-            *kernel = cached.get();
-            dev->by_text.emplace(std::move(text_key), cached.get());
-            return CUSTOS_HIP_OK;
-        }
-    }
-    rc = build_module(dev, k.get());
-    if (rc != CUSTOS_HIP_OK) return rc;
-    // the second entry point of the module: many equal launches in one grid
-    if (hipModuleGetFunction(&k->fn_batched, k->module, (k->spec.name + "_batched").c_str()) != hipSuccess) {
-        (void)hipGetLastError();
-        k->fn_batched = nullptr;
-    }
-    if (hipModuleGetFunction(&k->fn_ragged, k->module, (k->spec.name + "_ragged").c_str()) != hipSuccess) {
-        (void)hipGetLastError();
-        k->fn_ragged = nullptr;
-    }
-    *kernel = k.get();
-    dev->by_text.emplace(std::move(text_key), k.get());
-    bucket.push_back(std::move(k));
+    *kernel = k;
+    dev->by_text.emplace(std::move(text_key), k);
     return CUSTOS_HIP_OK;
 }
 
@@ -280,6 +319,18 @@ uint64_t custos_hip_kernel_hash(const custos_hip_kernel* kernel) { return kernel
 
 int32_t custos_hip_kernel_arity(const custos_hip_kernel* kernel) {
     return kernel ? kernel->spec.expr.n_vars : 0;
+}
+
+int32_t custos_hip_kernel_launched_as(custos_hip_device* dev, custos_hip_kernel* kernel, size_t n,
+                                      custos_hip_kernel** variant) {
+    REQUIRE_DEV(dev);
+    if (!kernel || !variant) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    const unsigned long long operands = kernel->spec.kind == Kind::UnaryGrad ? 3 : kernel->spec.expr.n_vars + 1;
+    bool alternate = false;
+    *variant = kernel->spec.kind == Kind::Source
+                   ? kernel
+                   : kernel_variant(dev, kernel, operands * n * dtype_size(kernel->spec.dtype), &alternate);
+    return CUSTOS_HIP_OK;
 }
 
 int32_t custos_hip_cache_stats(custos_hip_device* dev, uint64_t* compiles, uint64_t* hits) {

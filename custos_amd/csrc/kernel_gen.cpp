@@ -7,7 +7,7 @@
 
 namespace custos_hip {
 
-Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int nontemporal) {
+Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int nontemporal, int direction) {
     Tuning t;
     if (block_threads > 0) {
         block_threads = std::max(64, std::min(1024, block_threads));
@@ -16,7 +16,42 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
     if (unroll > 0) t.unroll = std::min(16, unroll);
     t.blocks_per_cu = blocks_per_cu > 0 ? std::min(64, blocks_per_cu) : 0;
     if (nontemporal != 0) t.nontemporal = nontemporal < 0 ? 0 : (nontemporal & 3);
+    if (direction == 1 || direction == 2) t.direction = direction;
     return t;
+}
+
+// Launch shape by the bytes a launch touches, measured on MI355X (8 x 4 MiB L2,
+// 256 MiB memory-side cache, HBM3E).  Abbreviations: vectors per thread (u1 /
+// u2), temporal or non-temporal accesses (T / N), tiles always first to last or
+// every launch the other way round (f / a).
+//
+// Small launches (under 64 MiB): a chain whose working set fits the memory-side
+// cache runs 4 % faster with temporal accesses (a non-temporal store pushes what
+// the next kernel reads out to HBM): 1024 x (a*b; +c; sqrt(abs)*0.3) over 16 KiB
+// buffers replays in 23.5 us with u2 T, 24.4 with u2 N, 27.3 with u1 N.
+//
+// Large launches stream from HBM; temporal accesses then cost up to 10 % (the
+// same chain over 256 MiB arrays: u2 T 5846, u2 N 6409, u1 N 7051 GB/s).  Kernels
+// that read through three or more pointers sustain most with one vector per
+// thread, kernels with one input with two, in isolation and in sequence
+// (tanh forward 1R+1W + backward 3R+1W at 2^26 elements, GB/s on 24 B/element:
+// forward u2 / backward u1 7100-7350, u2 / u2 6400, u1 / u2 6500, u1 / u1 5700-5870,
+// the same for four placements of the buffers and both directions).
+//
+// Alternating the direction costs nothing in such sequences and lets a launch
+// that repeats over the same buffers (a graph replay, a consumer after its
+// producer) start on the last 256 MiB the memory-side cache still holds; with it
+// one vector per thread is best for one-input kernels too once they touch more
+// than three cache sizes (1 R + 1 W, GB/s, u1Na / u2Na / u2Nf / u1Nf:
+// 768 MiB 6755 / 6440 / 6476 / 6258, 1 GiB 6979 / 6444 / 6473 / 6310,
+// 2 GiB 6711 / 6401 / 6378 / 6293; 2 R + 1 W at 1.5 GiB 7178 / 6536 / 6455 / 6396;
+// 3 R + 1 W at 2 GiB 6845 / 6316 / 6294 / 6137).
+LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands) {
+    constexpr unsigned long long MiB = 1ull << 20;
+    if (footprint_bytes < 64 * MiB) return {2, 0, false};
+    if (footprint_bytes <= 256 * MiB) return {2, 3, false};
+    const bool one_vector = n_operands >= 3 || footprint_bytes >= 768 * MiB;
+    return {one_vector ? 1 : 2, 3, true};
 }
 
 std::vector<std::string> hiprtc_options(const std::string& arch) {
@@ -135,10 +170,18 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
         err->message = "a unary gradient expression takes exactly one marker";
         return false;
     }
+    // Open knobs: the kernel is first compiled for small launches; another size compiles
+    // its variant when it first occurs.
+    const LaunchShape small = preferred_shape(0, kind == Kind::UnaryGrad ? 3 : k.expr.n_vars + 1);
+    k.auto_unroll = tuning.unroll <= 0;
+    if (k.auto_unroll) k.tuning.unroll = small.unroll;
+    k.auto_nt = tuning.nontemporal < 0;
+    if (k.auto_nt) k.tuning.nontemporal = small.nontemporal;
     uint64_t h;
     if (!hash_expr(k.expr, dtype, &h, err)) return false;
-    int32_t tail[6] = {static_cast<int32_t>(kind), tuning.block_threads, tuning.unroll,
-                       tuning.blocks_per_cu, tuning.nontemporal, 5 /* template version */};
+    // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
+    int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
+                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 6 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -155,12 +198,12 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     if (!emit_expr_body(k.expr, dtype, &body, err)) return false;
 
     const int n_in = k.expr.n_vars;
-    const bool nt_load = tuning.nontemporal & 1, nt_store = tuning.nontemporal & 2;
+    const bool nt_load = k.tuning.nontemporal & 1, nt_store = k.tuning.nontemporal & 2;
 
     std::string s;
     s += "// generated by custos-hip: " + to_cl_source(k.expr, markers) + "\n";
-    s += "#define CUSTOS_BLOCK " + std::to_string(tuning.block_threads) + "\n";
-    s += "#define CUSTOS_UNROLL " + std::to_string(tuning.unroll) + "\n";
+    s += "#define CUSTOS_BLOCK " + std::to_string(k.tuning.block_threads) + "\n";
+    s += "#define CUSTOS_UNROLL " + std::to_string(k.tuning.unroll) + "\n";
     s += "#define CUSTOS_VEC " + std::to_string(k.vec_elems) + "\n";
     s += nt_load ? "#define CUSTOS_LD(p) __builtin_nontemporal_load(p)\n" : "#define CUSTOS_LD(p) (*(p))\n";
     s += nt_store ? "#define CUSTOS_ST(p, v) __builtin_nontemporal_store(v, p)\n"
@@ -241,12 +284,13 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
 
     // Entry point for one launch over one set of operands.
     s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-    s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec) {\n";
+    // `rev` != 0 walks the tiles from the last to the first (see Tuning::direction).
+    s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec, const u64 rev) {\n";
     s += vec_ptrs;
     s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
     s += "    const u64 n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;\n";
     s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x)\n";
-    s += "        custos_tile(" + tile_args + "vout, tile * tile_vecs + threadIdx.x, n_vec);\n";
+    s += "        custos_tile(" + tile_args + "vout, (rev ? n_tiles - 1 - tile : tile) * tile_vecs + threadIdx.x, n_vec);\n";
     // Elements outside the 16-byte aligned body: `head` leading ones and the
     // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
     s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
@@ -263,9 +307,10 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     // of segment b / tiles_per_seg; the last tile of a segment also does the tail.
     const int n_ptrs = kind == Kind::Apply ? n_in + 1 : 3;
     s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-    s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg) {\n";
-    s += "    const u64 seg = blockIdx.x / tiles_per_seg;\n";
-    s += "    const u64 tile = blockIdx.x - seg * tiles_per_seg;\n";
+    s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, const u64 rev) {\n";
+    s += "    const u64 blk = rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
+    s += "    const u64 seg = blk / tiles_per_seg;\n";
+    s += "    const u64 tile = blk - seg * tiles_per_seg;\n";
     s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs) + ";\n";
     s += "    const u64 head = 0;\n";
     if (kind == Kind::Apply) {
@@ -286,8 +331,8 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     // holds the operand addresses (16-byte aligned) and the element count of its
     // segment; `block_map[b]` = segment << 32 | tile tells workgroup b its work.
     s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-    s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map) {\n";
-    s += "    const u64 where = block_map[blockIdx.x];\n";
+    s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, const u64 rev) {\n";
+    s += "    const u64 where = block_map[rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x];\n";
     s += "    const u64 seg = where >> 32;\n";
     s += "    const u64 tile = where & 0xffffffffull;\n";
     s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + 1) + ";\n";

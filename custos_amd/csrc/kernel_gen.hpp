@@ -18,26 +18,39 @@ namespace custos_hip {
 enum class Kind : int32_t { Apply = 0, UnaryGrad = 1, Source = 2 /* caller-written kernel source */ };
 
 struct Tuning {
-    // Defaults from interleaved, repeated timing of the fused f32 chain at 2^28
-    // elements on MI355X: workgroups of 64 or 128 threads with 2 vectors per
-    // thread sustain 3-5 % more than 256..1024-thread workgroups or other unroll
-    // factors (many small workgroups keep the memory channels evenly loaded);
-    // streaming (non-temporal) loads and stores add another 1-2 %; persistent
-    // grids were 5-20 % slower.
+    // Launch shape of the generated kernels.  Workgroups of 64 or 128 threads
+    // sustain 3-5 % more than 256..1024-thread workgroups in interleaved,
+    // repeated timing on MI355X (many small workgroups keep the memory channels
+    // evenly loaded); persistent grids were 5-20 % slower.  The other three
+    // knobs are chosen per launch from the bytes it touches (preferred_shape)
+    // unless the caller fixes them.
     int block_threads = 128;
-    int unroll = 2;
+    int unroll = 0;         // 16-byte vectors per thread and tile; 0: chosen per launch
     int blocks_per_cu = 0;  // <= 0: one tile per workgroup
-    int nontemporal = 3;    // bit 0 loads, bit 1 stores
+    int nontemporal = -1;   // bit 0 loads, bit 1 stores; -1: chosen per launch
+    int direction = 0;      // 1: tiles first to last; 2: every launch the other way round; 0: chosen per launch
 };
 
-// Fills unset (zero) fields with the defaults and clamps to legal values.
-Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int nontemporal);
+// What suits a launch that touches `footprint_bytes` (all operands together)
+// through `n_operands` pointers.
+struct LaunchShape {
+    int unroll;
+    int nontemporal;
+    bool alternate;  // walk the tiles in the direction opposite to the previous launch
+};
+LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands);
+
+// Fills unset (zero) fields with the defaults and clamps to legal values
+// (`nontemporal` and `direction` as in custos_hip_tuning).
+Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int nontemporal, int direction);
 
 struct KernelSpec {
     Kind kind = Kind::Apply;
     DType dtype = DType::F32;
     Expr expr;
-    Tuning tuning;
+    Tuning tuning;             // as compiled (unroll resolved)
+    bool auto_unroll = false;  // the caller left the unroll factor / the cache policy open:
+    bool auto_nt = false;      // launches may use a variant compiled with another choice
     uint64_t hash = 0;   // cache key: expression, dtype, kind, tuning
     std::string name;    // entry point: custos_<kind>_<dtype>_<hash>, unique per kernel so
                          // that profiler output tells the kernels apart

@@ -12,7 +12,7 @@ namespace {
 // Checks operand addresses and computes how the element range splits into a
 // scalar head, 16-byte vectors and a scalar tail.
 int32_t plan_launch(custos_hip_device* dev, const custos_hip_kernel* k, const std::vector<Range>& ops,
-                    size_t n, unsigned long long* head, unsigned long long* n_vec, unsigned int* grid) {
+                    size_t n, unsigned long long* head, unsigned long long* n_vec) {
     const size_t es = dtype_size(k->spec.dtype);
     if (n > (1ull << 40)) return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "more than 2^40 elements");
     const uint64_t bytes = static_cast<uint64_t>(n) * es;
@@ -37,30 +37,32 @@ int32_t plan_launch(custos_hip_device* dev, const custos_hip_kernel* k, const st
         if (h > n) h = n;
         nv = (n - h) / k->spec.vec_elems;
     }
-    const Tuning& t = k->spec.tuning;
-    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
-    unsigned long long tiles = (nv + tile_vecs - 1) / tile_vecs;
-    unsigned long long scalar = n - nv * k->spec.vec_elems;
-    const unsigned long long cus = static_cast<unsigned long long>(dev->props.multiProcessorCount);
-    unsigned long long scalar_blocks = std::min((scalar + t.block_threads - 1) / t.block_threads, cus * 32);
-    if (t.blocks_per_cu > 0) tiles = std::min(tiles, cus * t.blocks_per_cu);
-    unsigned long long g = std::max(1ull, std::max(tiles, scalar_blocks));
-    g = std::min(g, 1ull << 22);
     *head = h;
     *n_vec = nv;
-    *grid = static_cast<unsigned int>(g);
     return CUSTOS_HIP_OK;
 }
 
 }  // namespace
+
+unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
+                         unsigned long long n_vec) {
+    const Tuning& t = k->spec.tuning;
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+    unsigned long long tiles = (n_vec + tile_vecs - 1) / tile_vecs;
+    const unsigned long long scalar = n - n_vec * k->spec.vec_elems;
+    const unsigned long long cus = static_cast<unsigned long long>(dev->props.multiProcessorCount);
+    const unsigned long long scalar_blocks = std::min((scalar + t.block_threads - 1) / t.block_threads, cus * 32);
+    if (t.blocks_per_cu > 0) tiles = std::min(tiles, cus * t.blocks_per_cu);
+    unsigned long long g = std::max(1ull, std::max(tiles, scalar_blocks));
+    return static_cast<unsigned int>(std::min(g, 1ull << 22));
+}
 
 // Launches the kernel over one set of operands, or records the launch while
 // the device is recording.  `ops` are the operand addresses in the order of the
 // kernel's pointer parameters.
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n) {
     unsigned long long head, n_vec, count = n;
-    unsigned int grid;
-    int32_t rc = plan_launch(dev, k, ops, n, &head, &n_vec, &grid);
+    int32_t rc = plan_launch(dev, k, ops, n, &head, &n_vec);
     if (rc != CUSTOS_HIP_OK) return rc;
     if (dev->capturing) {
         RecNode node;
@@ -69,7 +71,6 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
         node.n = n;
         node.head = head;
         node.n_vec = n_vec;
-        node.grid = grid;
         const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
         for (const Range& r : ops) {
             node.ptrs.push_back(r.ptr);
@@ -80,6 +81,11 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
         dev->recorded.push_back(std::move(node));
         return CUSTOS_HIP_OK;
     }
+    // the launch shape that suits the bytes this launch touches
+    bool alternate = false;
+    k = kernel_variant(dev, k, static_cast<unsigned long long>(ops.size()) * n * dtype_size(k->spec.dtype), &alternate);
+    const unsigned int grid = launch_grid(dev, k, n, n_vec);
+    unsigned long long rev = alternate ? (dev->launch_parity ^= 1) : 0;
     uint64_t ptrs[8];
     std::vector<void*> args;
     for (size_t i = 0; i < ops.size(); i++) {
@@ -89,6 +95,7 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     args.push_back(&count);
     args.push_back(&head);
     args.push_back(&n_vec);
+    args.push_back(&rev);
     HIP_TRY(dev, hipModuleLaunchKernel(k->fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
                                        1, 1, 0, dev->stream, args.data(), nullptr));
     return CUSTOS_HIP_OK;

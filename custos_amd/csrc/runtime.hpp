@@ -22,6 +22,12 @@ struct custos_hip_kernel {
     hipFunction_t fn = nullptr;
     hipFunction_t fn_batched = nullptr;  // equal launches in one grid
     hipFunction_t fn_ragged = nullptr;   // launches of different lengths in one grid
+    // To compile the same expression with another launch shape on demand:
+    std::string expr_src;
+    std::vector<std::string> markers;
+    // same expression compiled with another (unroll, cache policy); owned by the cache.
+    // key = unroll * 8 + nontemporal; a null entry is a variant that failed to compile
+    std::vector<std::pair<int, custos_hip_kernel*>> variants;
 };
 
 // A graph node in launchable form: function, shape and a copy of the argument values.
@@ -34,6 +40,7 @@ struct LoweredNode {
     dim3 grid{1, 1, 1}, block{1, 1, 1};
     unsigned int shared_mem = 0;
     std::vector<std::vector<unsigned char>> args;
+    int rev_arg = -1;  // index of the direction argument of a node that alternates, else -1
 };
 
 struct custos_hip_graph {
@@ -42,6 +49,7 @@ struct custos_hip_graph {
     // its dependency order, and a handful of launches cost less than a graph launch.
     // Everything else is an instantiated hipGraph.
     std::vector<LoweredNode> direct;
+    bool flip_each_replay = false;  // direct replay: alternating nodes change direction every replay
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     void* table = nullptr;    // operand address tables of the batched nodes (device memory)
@@ -60,7 +68,6 @@ struct RecNode {
     custos_hip_kernel* k = nullptr;
     std::vector<uint64_t> ptrs;  // kernel: operand addresses in parameter order; fill: {ptr}; copy: {dst, src}
     unsigned long long n = 0, head = 0, n_vec = 0, bytes = 0;
-    unsigned int grid = 1;
     std::vector<Access> acc;
     int level = 0;
     // Source: launch shape and a copy of the argument values.  What such a kernel
@@ -79,6 +86,7 @@ struct custos_hip_device {
     custos_hip::Tuning tuning;
     bool capturing = false;          // recording: launches, clears and copies go to `recorded`
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
+    unsigned long long launch_parity = 0;  // direction of the last launch that alternates
     bool batching = true;            // merge equal independent launches of a level into one grid
     std::vector<RecNode> recorded;
     uint64_t compiles = 0, hits = 0, disk_hits = 0;
@@ -120,8 +128,8 @@ struct Range {
 
 // launch shape from the C struct; unset fields take the defaults
 inline Tuning tuning_from_c(const custos_hip_tuning* t) {
-    if (!t) return normalize_tuning(0, 0, 0, 0);
-    return normalize_tuning(t->block_threads, t->unroll, t->blocks_per_cu, t->nontemporal);
+    if (!t) return normalize_tuning(0, 0, 0, 0, 0);
+    return normalize_tuning(t->block_threads, t->unroll, t->blocks_per_cu, t->nontemporal, t->direction);
 }
 
 // device.hip
@@ -133,9 +141,19 @@ void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph ker
 int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec, const std::string& arch,
                                std::vector<char>* code);
 int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k);
+// The kernel to launch for `footprint_bytes` touched: `k` itself, or a variant
+// compiled with the unroll factor and cache policy that suit the size (where the
+// caller left them open).  Never fails: without a variant it returns `k`.
+// `alternate` tells whether the launch should walk the tiles in the direction
+// opposite to the previous launch.
+custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
+                                  bool* alternate);
 
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
+// Workgroups of a single launch of `k` over n_vec vectors and n elements.
+unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
+                         unsigned long long n_vec);
 
 // graph.cpp
 int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g);

@@ -134,8 +134,9 @@ class HIP:
     def sync(self) -> None:
         self._check(self.lib.custos_hip_sync(self.handle))
 
-    def set_tuning(self, block_threads=0, unroll=0, blocks_per_cu=0, nontemporal=0) -> None:
-        t = capi.Tuning(block_threads, unroll, blocks_per_cu, nontemporal)
+    def set_tuning(self, block_threads=0, unroll=0, blocks_per_cu=0, nontemporal=0, direction=0) -> None:
+        """Launch shape of generated kernels; 0 leaves a knob to the library (`custos_hip_tuning`)."""
+        t = capi.Tuning(block_threads, unroll, blocks_per_cu, nontemporal, direction)
         self._check(self.lib.custos_hip_set_tuning(self.handle, C.byref(t)))
 
     def cache_stats(self):
@@ -187,7 +188,12 @@ class HIP:
     def kernel_source(self, kernel) -> str:
         return self.lib.custos_hip_kernel_source(kernel).decode()
 
-    def kernel_name(self, kernel) -> str:
+    def kernel_name(self, kernel, n: int | None = None) -> str:
+        """Entry point name; with `n`, of the variant a launch over n elements runs."""
+        if n is not None:
+            v = C.c_void_p()
+            self._check(self.lib.custos_hip_kernel_launched_as(self.handle, kernel, n, C.byref(v)))
+            kernel = v
         return self.lib.custos_hip_kernel_name(kernel).decode()
 
     def apply_fn(self, buf: Buffer, f, out: Buffer | None = None) -> Buffer:

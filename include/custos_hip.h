@@ -113,11 +113,15 @@ typedef struct custos_hip_device_info {
  * They are part of the kernel cache key. */
 typedef struct custos_hip_tuning {
     int32_t block_threads;   /* threads per workgroup (multiple of 64), default 128 */
-    int32_t unroll;          /* 16-byte vectors per thread per tile, default 2 */
+    int32_t unroll;          /* 16-byte vectors per thread per tile; 0 (default): 2 for kernels
+                                with one input operand, 1 for kernels that read several */
     int32_t blocks_per_cu;   /* > 0: persistent grid of CUs*blocks_per_cu workgroups that
                                 stride over the tiles; <= 0 (default): one tile per workgroup */
-    int32_t nontemporal;     /* bit 0: non-temporal loads, bit 1: non-temporal stores;
-                                0 = default (3: both), -1 = off */
+    int32_t nontemporal;     /* bit 0: non-temporal loads, bit 1: non-temporal stores; -1 = off;
+                                0 (default): chosen per launch from the bytes it touches */
+    int32_t direction;       /* 1: tiles from the first to the last; 2: every launch walks them the
+                                other way round than the launch before, so that it starts on what
+                                the caches still hold; 0 (default): chosen per launch */
 } custos_hip_tuning;
 
 /* ---- device (src/devices/cuda/cuda.rs:53-67, cuda_device.rs:31-128) ---- */
@@ -184,6 +188,12 @@ const char *custos_hip_kernel_source(const custos_hip_kernel *kernel);
 const char *custos_hip_kernel_name(const custos_hip_kernel *kernel);
 uint64_t custos_hip_kernel_hash(const custos_hip_kernel *kernel);
 int32_t custos_hip_kernel_arity(const custos_hip_kernel *kernel);
+/* The kernel a launch of `kernel` over `n` elements really runs: `kernel` itself, or the
+ * variant of the same expression whose launch shape (vectors per thread, cache policy)
+ * suits the bytes such a launch touches, compiled on first use.  Its name is what a
+ * profiler shows.  Only knobs that custos_hip_set_tuning left at 0 vary. */
+int32_t custos_hip_kernel_launched_as(custos_hip_device *dev, custos_hip_kernel *kernel, size_t n,
+                                      custos_hip_kernel **variant);
 /* Number of hiprtc compilations / cache hits since the device was created. */
 int32_t custos_hip_cache_stats(custos_hip_device *dev, uint64_t *compiles, uint64_t *hits);
 

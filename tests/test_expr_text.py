@@ -132,9 +132,16 @@ def test_tuning_is_part_of_the_key_and_source():
     src, h1 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], t)
     assert "#define CUSTOS_BLOCK 256" in src and "#define CUSTOS_UNROLL 4" in src
     assert "__builtin_nontemporal" not in src
+    # knobs left open: the text is the shape for small launches (temporal accesses, two vectors
+    # per thread); other sizes compile a variant when launched
     src2, h2 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"])
-    assert "#define CUSTOS_BLOCK 128" in src2 and "__builtin_nontemporal_load" in src2
-    assert h1 != h2
+    assert "#define CUSTOS_BLOCK 128" in src2 and "#define CUSTOS_UNROLL 2" in src2
+    assert "__builtin_nontemporal" not in src2
+    src4, h4 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], capi.Tuning(0, 0, 0, 3))
+    assert "__builtin_nontemporal_load" in src4 and "__builtin_nontemporal_store" in src4
+    src5, h5 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], capi.Tuning(0, 2, 0, -1))
+    assert len({h1, h2, h4, h5}) == 4            # "open" and "fixed to the same value" are different keys
+    assert "const u64 rev" in src2
 
 
 def test_integer_rejects_transcendentals_and_fractions():
