@@ -318,3 +318,35 @@ def test_short_chain_replays_the_same_as_a_graph_or_as_plain_launches(hip, oracl
         hip.sync()
         assert_bits_equal(c.read(), want, f"direct_max={direct_max} replay {replay}")
     g.destroy()
+
+
+def test_alternating_direction_in_replayed_graphs(hip, oracle):
+    """Nodes that alternate their direction (here forced for every size): a directly replayed
+    chain with an odd number of them flips on every replay, an instantiated graph keeps the
+    directions it was built with; results are the same bits on every replay."""
+    n = 40001
+    x = synth.uniform_f32(13, n, -2, 2)
+    f = lambda v: v.mul(1.5).sub(0.25)
+    want1 = oracle.apply_fn(f, x)
+    want3 = oracle.apply_fn(f, oracle.apply_fn(f, want1))
+    try:
+        hip.set_tuning(0, 0, 0, 0, 2)
+        for direct_max, steps in ((4, 1), (4, 3), (0, 3)):
+            hip.set_graph_direct_replay(direct_max)
+            a, b, c, d = hip.buffer(x), hip.alloc(n), hip.alloc(n), hip.alloc(n)
+            hip.capture_begin()
+            hip.apply_fn(a, f, out=b)
+            if steps == 3:
+                hip.apply_fn(b, f, out=c)
+                hip.apply_fn(c, f, out=d)
+            g = hip.capture_end()
+            last = b if steps == 1 else d
+            for replay in range(4):
+                last.clear()
+                g.launch()
+                hip.sync()
+                assert_bits_equal(last.read(), want1 if steps == 1 else want3, f"direct_max={direct_max} steps={steps} replay={replay}")
+            g.destroy()
+    finally:
+        hip.set_tuning()
+        hip.set_graph_direct_replay(4)

@@ -277,6 +277,72 @@ def test_tuning_variants_agree(hip, oracle):
         hip.set_tuning()
 
 
+def test_both_traversal_directions_and_all_shapes(hip, oracle):
+    """Every launch shape the library can pick (vectors per thread x cache policy x direction)
+    computes the same bits: views with heads and tails, a unary gradient, a persistent grid."""
+    n = 100003
+    x = synth.uniform_f32(7, n + 5, -2, 2)
+    y = synth.uniform_f32(8, n + 5, 0.5, 2)
+    f = lambda a, b: a.mul(b).add(0.25).max(0.0)
+    d = lambda v: v.mul(2.0).add(1.0)
+    xb, yb = hip.buffer(x), hip.buffer(y)
+    try:
+        for unroll in (1, 2, 3):
+            for nt in (-1, 3):
+                for bpc in (0, 1):
+                    hip.set_tuning(0, unroll, bpc, nt, 2)          # every launch the other way round
+                    for launch in range(2):                        # so: both directions
+                        for off in (0, 1, 3):                      # aligned, and views with a scalar head
+                            xs, ys = xb.slice(off, off + n), yb.slice(off, off + n)
+                            got = hip.apply_fn2(xs, ys, f).read()
+                            assert_bits_equal(got, oracle.apply_fn(f, x[off:off + n], y[off:off + n]),
+                                              f"unroll={unroll} nt={nt} bpc={bpc} launch={launch} off={off}")
+                        g0 = np.full(n, 0.5, dtype=np.float32)
+                        gb = hip.buffer(g0)
+                        hip.add_unary_grad(xb.slice(0, n), gb, yb.slice(0, n), d)
+                        assert_bits_equal(gb.read(), oracle.add_unary_grad(d, x[:n], g0, y[:n]))
+    finally:
+        hip.set_tuning()
+
+
+def test_launch_shape_follows_the_bytes_touched(hip):
+    """With the knobs left open, small launches run the kernel as first compiled and a large
+    launch runs a variant of the same expression; a pinned knob pins the kernel."""
+    src = "((x * 3.0) - 1.0)"
+    k = hip.compile(capi.KIND_APPLY, "f32", src, ("x",))
+    small = hip.kernel_name(k, 1000)
+    assert small == hip.kernel_name(k) == hip.kernel_name(k, 1 << 20)
+    assert "__builtin_nontemporal" not in hip.kernel_source(k)
+    big = hip.kernel_name(k, 1 << 28)
+    assert big != small
+    c0, _ = hip.cache_stats()
+    assert hip.kernel_name(k, 1 << 28) == big               # compiled once
+    assert hip.cache_stats()[0] == c0
+    try:
+        hip.set_tuning(0, 2, 0, 3, 1)
+        pinned = hip.compile(capi.KIND_APPLY, "f32", src, ("x",))
+        assert hip.kernel_name(pinned, 1000) == hip.kernel_name(pinned, 1 << 28) == hip.kernel_name(pinned)
+        assert "__builtin_nontemporal_store" in hip.kernel_source(pinned)
+    finally:
+        hip.set_tuning()
+    # results do not depend on the variant: a 2^25-element launch (256 MiB touched) and its head
+    n = 1 << 25
+    xb = hip.alloc(n, zeroed=False)
+    base = synth.uniform_f32(3, 1 << 16, -1, 1)
+    hip.copy(xb.slice(0, 1 << 16), hip.buffer(base))
+    filled = 1 << 16
+    while filled < n:
+        hip.copy(xb.slice(filled, 2 * filled), xb.slice(0, filled))
+        filled *= 2
+    want = (base * np.float32(3.0) - np.float32(1.0)).astype(np.float32)
+    for launch in range(2):
+        out = hip.apply_fn(xb, lambda v: v.mul(3.0).sub(1.0))
+        for start in (0, n // 2, n - (1 << 16)):
+            assert_bits_equal(out.slice(start, start + (1 << 16)).read(), want, f"launch {launch} window {start}")
+    big_launch = hip.apply_fn(hip.alloc(1 << 27), lambda v: v.mul(3.0).sub(1.0))   # 1 GiB touched, zeros in
+    assert np.all(big_launch.slice((1 << 27) - 4096, 1 << 27).read() == np.float32(-1.0))
+
+
 def test_kernel_cache(hip):
     c0, h0 = hip.cache_stats()
     k1 = hip.compile(capi.KIND_APPLY, "f32", "((x * 41.0) + 0.125)", ("x",))
