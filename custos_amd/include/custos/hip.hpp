@@ -223,6 +223,12 @@ class HIP : public Device<HIP<Mods>, Mods> {
         return n;
     }
 
+    // Launch shape of the generated kernels; zero fields are left to the library, which
+    // chooses them per launch from the bytes it touches.
+    void set_tuning(const custos_hip_tuning& tuning) { check(custos_hip_set_tuning(dev_, &tuning)); }
+    // Longest recorded chain that is replayed as plain launches instead of a graph launch.
+    void set_graph_direct_replay(int32_t max_nodes) { check(custos_hip_set_graph_direct_replay(dev_, max_nodes)); }
+
     custos_hip_kernel* compile(int32_t kind, int32_t dtype, const std::string& src,
                                std::initializer_list<const char*> markers) {
         std::vector<const char*> m(markers);
