@@ -21,9 +21,10 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 }
 
 // Launch shape by the bytes a launch touches, measured on MI355X (8 x 4 MiB L2,
-// 256 MiB memory-side cache, HBM3E).  Abbreviations: vectors per thread (u1 /
-// u2), temporal or non-temporal accesses (T / N), tiles always first to last or
-// every launch the other way round (f / a).
+// 256 MiB memory-side cache, HBM3E) over buffers of random data (buffers of
+// zeros run 5-10 % faster and hide differences).  Abbreviations: vectors per
+// thread (u1 / u2), temporal or non-temporal accesses (T / N), tiles always
+// first to last or every launch the other way round (f / a).
 //
 // Small launches (under 64 MiB): a chain whose working set fits the memory-side
 // cache runs 4 % faster with temporal accesses (a non-temporal store pushes what
@@ -33,24 +34,27 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // Large launches stream from HBM; temporal accesses then cost up to 10 % (the
 // same chain over 256 MiB arrays: u2 T 5846, u2 N 6409, u1 N 7051 GB/s).  Kernels
 // that read through three or more pointers sustain most with one vector per
-// thread, kernels with one input with two, in isolation and in sequence
-// (tanh forward 1R+1W + backward 3R+1W at 2^26 elements, GB/s on 24 B/element:
-// forward u2 / backward u1 7100-7350, u2 / u2 6400, u1 / u2 6500, u1 / u1 5700-5870,
-// the same for four placements of the buffers and both directions).
+// thread from about 512 MiB on, kernels with one input with two, in isolation
+// and in sequence (tanh forward 1R+1W + backward 3R+1W at 2^26 elements, GB/s on
+// 24 B/element: forward u2 / backward u1 6920, u2 / u2 6400, u1 / u2 6350,
+// u1 / u1 5860, whatever the direction).
 //
 // Alternating the direction costs nothing in such sequences and lets a launch
 // that repeats over the same buffers (a graph replay, a consumer after its
 // producer) start on the last 256 MiB the memory-side cache still holds; with it
-// one vector per thread is best for one-input kernels too once they touch more
-// than three cache sizes (1 R + 1 W, GB/s, u1Na / u2Na / u2Nf / u1Nf:
-// 768 MiB 6755 / 6440 / 6476 / 6258, 1 GiB 6979 / 6444 / 6473 / 6310,
-// 2 GiB 6711 / 6401 / 6378 / 6293; 2 R + 1 W at 1.5 GiB 7178 / 6536 / 6455 / 6396;
-// 3 R + 1 W at 2 GiB 6845 / 6316 / 6294 / 6137).
+// one vector per thread is best for every arity from 768 MiB on.  GB/s, same
+// kernel launched back to back, u1Na / u2Na / u2Nf / u1Nf:
+//   1R+1W   768 MiB 6861 / 6452 / 6482 / 6286    2 GiB 6759 / 6427 / 6406 / 6326
+//   2R+1W   576 MiB 6873 / 6590 / 6701 / 6908  1.5 GiB 6810 / 6555 / 6598 / 6212
+//   3R+1W     1 GiB 6986 / 6375 / 6412 / 7019    2 GiB 6646 / 6298 / 6313 / 6115
+// Between 64 and 256 MiB temporal accesses win 5-9 % when one kernel repeats over
+// the same buffers but nothing in a chain of kernels, and lose once the chain's
+// working set leaves the cache, which a single launch cannot know: non-temporal.
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands) {
     constexpr unsigned long long MiB = 1ull << 20;
     if (footprint_bytes < 64 * MiB) return {2, 0, false};
     if (footprint_bytes <= 256 * MiB) return {2, 3, false};
-    const bool one_vector = n_operands >= 3 || footprint_bytes >= 768 * MiB;
+    const bool one_vector = footprint_bytes >= 768 * MiB || (n_operands >= 3 && footprint_bytes >= 512 * MiB);
     return {one_vector ? 1 : 2, 3, true};
 }
 
