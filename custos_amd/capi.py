@@ -104,6 +104,7 @@ PROTOTYPES = {
     "custos_hip_kernel_source": (C.c_char_p, [_P]),
     "custos_hip_kernel_name": (C.c_char_p, [_P]),
     "custos_hip_kernel_hash": (C.c_uint64, [_P]),
+    "custos_hip_preferred_shape": (C.c_int32, [C.c_uint64, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "custos_hip_kernel_launched_as": (C.c_int32, [_P, _P, C.c_size_t, C.POINTER(C.c_void_p)]),
     "custos_hip_kernel_arity": (C.c_int32, [_P]),
     "custos_hip_cache_stats": (C.c_int32, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
@@ -172,6 +173,13 @@ def last_error(dev_handle) -> str:
 def check(rc: int, dev_handle=None):
     if rc != 0:
         raise CustosHipError(rc, last_error(dev_handle))
+
+
+def preferred_shape(footprint_bytes: int, n_operands: int):
+    """(vectors per thread, nontemporal bits, alternates direction) for such a launch."""
+    u, nt, alt = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+    check(load_library().custos_hip_preferred_shape(footprint_bytes, n_operands, C.byref(u), C.byref(nt), C.byref(alt)))
+    return u.value, nt.value, bool(alt.value)
 
 
 def expr_emit(kind: int, dtype: str, src: str, markers, tuning: Tuning | None = None):

@@ -369,6 +369,16 @@ int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const cha
     return CUSTOS_HIP_OK;
 }
 
+int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t* unroll,
+                                   int32_t* nontemporal, int32_t* alternate) {
+    if (n_operands < 1) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "n_operands must be positive");
+    const LaunchShape s = preferred_shape(footprint_bytes, n_operands);
+    if (unroll) *unroll = s.unroll;
+    if (nontemporal) *nontemporal = s.nontemporal;
+    if (alternate) *alternate = s.alternate ? 1 : 0;
+    return CUSTOS_HIP_OK;
+}
+
 int32_t custos_hip_expr_canonical(const char* src, const char* const* markers, int32_t n_markers,
                                   char* buf, size_t cap, size_t* needed) {
     if (!src) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");

@@ -235,6 +235,12 @@ int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const cha
                                           const char *const *markers, int32_t n_markers,
                                           const custos_hip_tuning *tuning, size_t *code_size);
 /* Canonical re-print of an expression in the reference's ToCLSource format. */
+/* Host-only: the launch shape the library picks for a launch that touches `footprint_bytes`
+ * (all operands together) through `n_operands` pointers, for the knobs left at 0 in
+ * custos_hip_tuning: vectors per thread, the `nontemporal` bits, and whether the launch
+ * walks its tiles against the direction of the previous one. */
+int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t *unroll,
+                                   int32_t *nontemporal, int32_t *alternate);
 int32_t custos_hip_expr_canonical(const char *src, const char *const *markers, int32_t n_markers,
                                   char *buf, size_t cap, size_t *needed);
 

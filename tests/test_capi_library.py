@@ -94,3 +94,22 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".cpp", ".hpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f), errors="replace").read()
                 assert "cpu_oracle" not in text and "custos_cpu_oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_launch_shape_by_bytes_touched():
+    """The shape for the knobs a caller leaves open: temporal accesses for what fits the caches,
+    non-temporal streaming beyond, one vector per thread and alternating direction for the
+    large launches."""
+    MiB = 1 << 20
+    shape = capi.preferred_shape
+    assert shape(8 * MiB, 2) == (2, 0, False)              # config 1: 2^20 f32 in, out
+    assert shape(48 * MiB, 3) == (2, 0, False)             # config 5, one recorded level merged
+    assert shape(64 * MiB, 4) == (2, 3, False)             # config 5 after element-wise fusing
+    assert shape(256 * MiB, 2) == (2, 3, False)
+    assert shape(512 * MiB, 2) == (2, 3, True)             # config 3 forward
+    assert shape(768 * MiB, 3) == (1, 3, True)             # config 3 backward
+    assert shape(512 * MiB, 3) == (1, 3, True) and shape(511 * MiB, 3) == (2, 3, True)
+    assert shape(1024 * MiB, 2) == (1, 3, True)            # config 4
+    assert shape(2048 * MiB, 2) == (1, 3, True)            # config 2
+    with pytest.raises(capi.CustosHipError):
+        shape(1, 0)
