@@ -26,6 +26,8 @@ constexpr uint64_t kChunkShift = 21;  // conflict search buckets of 2 MiB
 // A launch of more tiles than this is not merged with launches of other lengths:
 // it fills the chip by itself, and the block map would grow with it.
 constexpr unsigned long long kRaggedMaxTiles = 16384;
+// A recorded graph that touches no more than this keeps its data in the memory-side cache.
+constexpr unsigned long long kCacheWorkingSet = 320ull << 20;
 
 void assign_levels(std::vector<RecNode>& nodes) {
     struct Seen {
@@ -100,13 +102,36 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
         const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
         return std::max(1ull, (n.n_vec + tile_vecs - 1) / tile_vecs);
     };
+    // Everything the graph touches, as the union of the recorded address ranges.  While it
+    // fits the memory-side cache (256 MiB, with some slack: a chain over 288 MiB still gains
+    // 4 %, over 192 MiB 9.5 %, over 384 MiB nothing, over 1.5 GiB it loses 10 %), every kernel
+    // of the graph uses temporal accesses: the next kernel, and the next replay, find the data
+    // in the cache.  Caller-written kernels are not counted.
+    bool fits_cache = false;
+    {
+        std::vector<std::pair<uint64_t, uint64_t>> ranges;
+        for (const RecNode& n : nodes)
+            for (const Access& a : n.acc)
+                if (a.end > a.begin) ranges.push_back({a.begin, a.end});
+        std::sort(ranges.begin(), ranges.end());
+        unsigned long long working_set = 0;
+        uint64_t covered = 0;
+        for (const auto& r : ranges) {
+            const uint64_t from = std::max(r.first, covered);
+            if (r.second > from) working_set += r.second - from;
+            covered = std::max(covered, r.second);
+        }
+        // (only a graph with consumers after producers: more than one dependency level)
+        fits_cache = max_level >= 1 && working_set <= kCacheWorkingSet;
+    }
+
     // the launch shape follows the bytes the (merged) launch touches
     auto choose_kernel = [&](Planned& p) {
         const RecNode& first = nodes[p.members[0]];
         if (first.type != RecNode::Kernel) return;
         unsigned long long footprint = 0;
         for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
-        custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate);
+        custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, fits_cache);
         const bool usable = p.members.size() == 1 || (p.ragged ? v->fn_ragged != nullptr : v->fn_batched != nullptr);
         p.kern = usable ? v : first.k;
     };

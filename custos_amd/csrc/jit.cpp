@@ -217,9 +217,10 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
 }
 
 custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
-                                  bool* alternate) {
+                                  bool* alternate, bool working_set_fits_cache) {
     const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;
-    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands);
+    LaunchShape shape = preferred_shape(footprint_bytes, n_operands);
+    if (working_set_fits_cache) shape = {2, 0, false};
     const int direction = dev->tuning.direction;
     *alternate = direction == 2 || (direction == 0 && shape.alternate);
     if (k->spec.kind == Kind::Source || (!k->spec.auto_unroll && !k->spec.auto_nt)) return k;

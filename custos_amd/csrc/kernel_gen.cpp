@@ -47,13 +47,17 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 //   1R+1W   768 MiB 6861 / 6452 / 6482 / 6286    2 GiB 6759 / 6427 / 6406 / 6326
 //   2R+1W   576 MiB 6873 / 6590 / 6701 / 6908  1.5 GiB 6810 / 6555 / 6598 / 6212
 //   3R+1W     1 GiB 6986 / 6375 / 6412 / 7019    2 GiB 6646 / 6298 / 6313 / 6115
-// Between 64 and 256 MiB temporal accesses win 5-9 % when one kernel repeats over
-// the same buffers but nothing in a chain of kernels, and lose once the chain's
-// working set leaves the cache, which a single launch cannot know: non-temporal.
+// Up to 256 MiB a launch fits the memory-side cache and temporal accesses win
+// 3-9 % when the kernel repeats over the same buffers (1R+1W at 192 MiB: 6959
+// against 6383 GB/s) and in chains over arrays of that size; the exception is the
+// range just above the L2 capacity, 64 to 128 MiB, where non-temporal accesses
+// are ahead (3R+1W at 64 MiB: 6883 against 6343) unless a chain reuses the data
+// (build_graph knows that and overrides).
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands) {
     constexpr unsigned long long MiB = 1ull << 20;
     if (footprint_bytes < 64 * MiB) return {2, 0, false};
-    if (footprint_bytes <= 256 * MiB) return {2, 3, false};
+    if (footprint_bytes < 128 * MiB) return {2, 3, false};
+    if (footprint_bytes <= 256 * MiB) return {2, 0, false};
     const bool one_vector = footprint_bytes >= 768 * MiB || (n_operands >= 3 && footprint_bytes >= 512 * MiB);
     return {one_vector ? 1 : 2, 3, true};
 }

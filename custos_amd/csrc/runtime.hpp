@@ -146,8 +146,11 @@ int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k);
 // caller left them open).  Never fails: without a variant it returns `k`.
 // `alternate` tells whether the launch should walk the tiles in the direction
 // opposite to the previous launch.
+// `working_set_fits_cache`: the caller knows that everything the surrounding graph touches
+// stays in the memory-side cache between its kernels (temporal accesses then, whatever the
+// size of the single launch).
 custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
-                                  bool* alternate);
+                                  bool* alternate, bool working_set_fits_cache = false);
 
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);

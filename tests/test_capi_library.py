@@ -105,7 +105,9 @@ def test_launch_shape_by_bytes_touched():
     assert shape(8 * MiB, 2) == (2, 0, False)              # config 1: 2^20 f32 in, out
     assert shape(48 * MiB, 3) == (2, 0, False)             # config 5, one recorded level merged
     assert shape(64 * MiB, 4) == (2, 3, False)             # config 5 after element-wise fusing
-    assert shape(256 * MiB, 2) == (2, 3, False)
+    assert shape(96 * MiB, 3) == (2, 3, False)             # just above the L2 capacity
+    assert shape(128 * MiB, 2) == (2, 0, False) and shape(256 * MiB, 2) == (2, 0, False)
+    assert shape(257 * MiB, 2) == (2, 3, True)
     assert shape(512 * MiB, 2) == (2, 3, True)             # config 3 forward
     assert shape(768 * MiB, 3) == (1, 3, True)             # config 3 backward
     assert shape(512 * MiB, 3) == (1, 3, True) and shape(511 * MiB, 3) == (2, 3, True)
