@@ -165,3 +165,47 @@ def test_marker_arguments_validated():
         with pytest.raises(capi.CustosHipError) as e:
             capi.expr_emit(capi.KIND_APPLY, "f32", "x", markers)
         assert e.value.code == capi.ERR_INVALID_ARGUMENT
+
+
+def test_parser_survives_malformed_input():
+    """Random token soup and mutated valid expressions: every input is either compiled to text
+    or rejected with a message; nothing crashes, nesting is bounded."""
+    import random
+    rng = random.Random(7)
+    atoms = ["x", "y", "(", ")", " ", "+", "-", "*", "/", ",", "sin", "cos", "tan", "tanh", "exp", "log", "abs",
+             "sqrt", "pow", "min", "max", ">=", "<=", "==", "1.0", "2", "0.5e3", "inf", "NaN", "1e400", "=", ";",
+             "\n", "x = ", "z", "1.", ".5", "0x10", "-(", "((", "))", "\x00", "\xff"]
+    good = ["(x + y)", "pow((x * 3.0), (y + 1.0))", "x = sin(x);\nx = -(x);\nx = cos(x);\n", "((x >= 0) * x)",
+            "-(tan(x))", "max(x, 0.0)"]
+    accepted = rejected = 0
+    for it in range(6000):
+        if it % 3 == 0:
+            s = list(rng.choice(good))
+            for _ in range(rng.randint(1, 3)):
+                pos = rng.randrange(len(s)) if s else 0
+                kind = rng.randrange(3)
+                if kind == 0 and s:
+                    del s[pos:pos + rng.randint(1, 3)]
+                elif kind == 1:
+                    s.insert(pos, rng.choice(atoms))
+                elif s:
+                    s[pos] = chr(rng.randrange(1, 128))
+            s = "".join(s)
+        else:
+            s = "".join(rng.choice(atoms) for _ in range(rng.randint(1, 24)))
+        s = s.replace("\x00", "")          # C strings end at NUL
+        for dtype in rng.sample(list(capi.DTYPES), 2):
+            try:
+                src, _ = capi.expr_emit(rng.choice([capi.KIND_APPLY, capi.KIND_UNARY_GRAD]), dtype, s, ["x", "y"])
+                assert "custos_expr" in src
+                accepted += 1
+            except capi.CustosHipError as e:
+                assert str(e)
+                rejected += 1
+    assert accepted > 20 and rejected > 1000
+    for depth in (300, 100000):
+        with pytest.raises(capi.CustosHipError) as e:
+            capi.expr_emit(capi.KIND_APPLY, "f32", "(" * depth + "x" + ")" * depth, ["x"])
+        assert "nested too deeply" in str(e.value)
+        with pytest.raises(capi.CustosHipError):
+            capi.expr_emit(capi.KIND_APPLY, "f32", "sin(" * depth + "x" + ")" * depth, ["x"])
