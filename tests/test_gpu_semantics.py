@@ -556,3 +556,62 @@ def test_per_node_rounding_of_16bit_floats(hip, oracle, dtype):
         dist = np.abs(key(got) - key(want))
     # a chain of three rounded nodes: one unit of disagreement in a node can move the result
     assert dist.max() <= 2 and (dist == 0).mean() > 0.98
+
+
+def _random_tree(rng, leaves, depth, integer, unsigned=False):
+    """A random expression over `leaves` built from the nodes whose results are exact."""
+    if depth == 0 or rng.random() < 0.15:
+        if rng.random() < 0.25:
+            if integer:
+                return Const(int(rng.integers(0 if unsigned else -5, 6)))
+            return Const(float(np.float32(rng.uniform(-4, 4))))
+        return leaves[int(rng.integers(len(leaves)))]
+    a = _random_tree(rng, leaves, depth - 1, integer, unsigned)
+    # (`abs` needs `Float` in the reference's CPU evaluation, src/two_way_ops/ops/unary.rs:246)
+    ops1 = ["neg", "identity"] + ([] if integer else ["abs", "sqrtabs"])
+    ops2 = ["add", "sub", "mul", "min", "max", "geq", "leq", "eq"] + ([] if integer else ["div"])
+    if rng.random() < 0.25:
+        op = ops1[int(rng.integers(len(ops1)))]
+        return a.abs().sqrt() if op == "sqrtabs" else getattr(a, op)()
+    b = _random_tree(rng, leaves, depth - 1, integer, unsigned)
+    return getattr(a, ops2[int(rng.integers(len(ops2)))])(b)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u16", "f16_pernode"])
+def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
+    """Random trees of up to 31 nodes over one to four operands, built from the nodes whose
+    results are exact: parser, operand order, literal typing and emitted code against the CPU
+    restatement evaluating the same tree, bit for bit (NaNs compare as NaN)."""
+    from custos_amd.expr import Resolve
+    rng = np.random.default_rng(sum(map(ord, dtype)))
+    integer = dtype[0] in "iu"
+    n = 4099
+    for trial in range(10):
+        k = int(rng.integers(1, 5))
+        seed = int(rng.integers(1 << 30))
+        build = lambda *leaves: _random_tree(np.random.default_rng(seed), list(leaves), 4, integer, dtype[0] == "u")
+        tree = build(*[Resolve(nm, i) for i, nm in enumerate(("a", "b", "c", "d")[:k])])
+        if isinstance(tree, (Const, Resolve)):
+            continue
+        if dtype == "f16_pernode":
+            arrs = [synth.uniform_f16_bits(200 + trial * 4 + i, n, -3, 3) for i in range(k)]
+            bufs = [hip.buffer(a.view(np.float16), dtype) for a in arrs]
+        else:
+            npdt = np.dtype(capi.DTYPES[dtype][1])
+            if integer:
+                lo, hi = (0, 60000) if dtype == "u16" else (-70000, 70000)
+                arrs = [rng.integers(lo, hi, size=n).astype(npdt) for _ in range(k)]
+            else:
+                arrs = [synth.uniform_f32(200 + trial * 4 + i, n, -3, 3).astype(npdt) for i in range(k)]
+                arrs[0][:SPECIALS.size] = SPECIALS.astype(npdt)
+            bufs = [hip.buffer(a, dtype) for a in arrs]
+        got = hip.apply_fn_n(bufs, build).read()
+        want = oracle.apply_fn(build, *arrs, dtype=dtype)
+        what = f"trial {trial}: {tree.to_cl_source(dtype)}"
+        if dtype == "f16_pernode":
+            got = got.view(np.uint16)
+            nan = lambda b: (b & 0x7fff) > 0x7c00
+            same = (got == want) | (nan(got) & nan(want))
+            assert same.all(), f"{what} differs at {np.flatnonzero(~same)[:5]}"
+        else:
+            assert_bits_equal(got, want, what)
