@@ -9,12 +9,13 @@ import subprocess
 import pytest
 
 HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp")
+EXAMPLES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "examples")
 
 
-def _binary(name):
-    path = os.path.join(HERE, name)
+def _binary(name, where=HERE):
+    path = os.path.join(where, name)
     if not os.path.exists(path):
-        subprocess.run(["make", "-C", HERE, name], check=True, capture_output=True)
+        subprocess.run(["make", "-C", where, name], check=True, capture_output=True)
     return path
 
 
@@ -39,3 +40,12 @@ def test_hip_module_stack():
     for case in ("hip_lazy_run_replays_one_graph", "hip_fused_chain_is_one_kernel", "graph_fuse_chain_optimized",
                  "autograd_tanh_config"):
         assert f"[  OK  ] {case}" in out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["lazy_and_fusing", "unary_autograd"])
+def test_examples_run(name):
+    proc = subprocess.run([_binary(name, EXAMPLES)], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    if name == "lazy_and_fusing":
+        assert "1 kernel node(s)" in proc.stdout and "1 graph build(s)" in proc.stdout
