@@ -95,6 +95,9 @@ PROTOTYPES = {
     "custos_hip_set_tuning": (C.c_int32, [_P, C.POINTER(Tuning)]),
     "custos_hip_get_tuning": (C.c_int32, [_P, C.POINTER(Tuning)]),
     "custos_hip_alloc": (C.c_int32, [_P, C.c_size_t, C.c_int32, C.POINTER(C.c_uint64)]),
+    "custos_hip_set_pool_limit": (C.c_int32, [_P, C.c_size_t]),
+    "custos_hip_pool_trim": (C.c_int32, [_P]),
+    "custos_hip_pool_stats": (C.c_int32, [_P, C.POINTER(C.c_size_t), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "custos_hip_free": (C.c_int32, [_P, C.c_uint64]),
     "custos_hip_write": (C.c_int32, [_P, C.c_uint64, C.c_void_p, C.c_size_t]),
     "custos_hip_read": (C.c_int32, [_P, C.c_void_p, C.c_uint64, C.c_size_t]),

@@ -125,6 +125,7 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
     HIP_TRY(nullptr, hipStreamCreateWithFlags(&dev->transfer, hipStreamNonBlocking));
     HIP_TRY(nullptr, hipEventCreate(&dev->t0));
     HIP_TRY(nullptr, hipEventCreate(&dev->t1));
+    dev->pool_limit = dev->props.totalGlobalMem / 4;
     *out = dev.release();
     return CUSTOS_HIP_OK;
 }
@@ -135,6 +136,8 @@ int32_t custos_hip_device_destroy(custos_hip_device* dev) {
     (void)hipStreamSynchronize(dev->stream);
     (void)hipStreamSynchronize(dev->transfer);
     for (custos_hip_graph* g : dev->graphs) destroy_graph(g);
+    for (auto& kv : dev->pool)
+        for (void* p : kv.second) (void)hipFree(p);
     for (auto& bucket : dev->cache)
         for (auto& k : bucket.second)
             if (k->module) (void)hipModuleUnload(k->module);
@@ -193,13 +196,49 @@ int32_t custos_hip_get_tuning(custos_hip_device* dev, custos_hip_tuning* tuning)
 
 // ---- memory ----
 
+// Sizes are rounded so that buffers of similar length share pool entries:
+// 512 B steps below 1 MiB, 2 MiB steps above (hipMalloc hands out 2 MiB
+// granules for large blocks anyway).
+static size_t pool_size_class(size_t bytes) {
+    const size_t step = bytes < (1u << 20) ? 512 : (2u << 20);
+    return (bytes + step - 1) / step * step;
+}
+
+static void release_pool(custos_hip_device* dev) {
+    (void)hipStreamSynchronize(dev->stream);
+    for (auto& kv : dev->pool)
+        for (void* p : kv.second) {
+            dev->block_bytes.erase(reinterpret_cast<uint64_t>(p));
+            (void)hipFree(p);
+        }
+    dev->pool.clear();
+    dev->pooled_bytes = 0;
+}
+
 int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, uint64_t* dptr) {
     REQUIRE_DEV(dev);
     if (!dptr) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "dptr is null");
     *dptr = 0;
     if (bytes == 0) return set_error(dev, CUSTOS_HIP_ERR_ZERO_LENGTH_BUFFER, "zero length buffers are not supported");
+    const size_t rounded = pool_size_class(bytes);
     void* p = nullptr;
-    HIP_TRY(dev, hipMalloc(&p, bytes));
+    auto pooled = dev->pool.find(rounded);
+    if (pooled != dev->pool.end() && !pooled->second.empty()) {
+        p = pooled->second.back();
+        pooled->second.pop_back();
+        dev->pooled_bytes -= rounded;
+        dev->pool_reused++;
+    } else {
+        hipError_t e = hipMalloc(&p, rounded);
+        if (e != hipSuccess && dev->pooled_bytes > 0) {
+            (void)hipGetLastError();
+            release_pool(dev);  // the pool may hold what this allocation needs
+            e = hipMalloc(&p, rounded);
+        }
+        if (e != hipSuccess) return hip_fail(dev, e, "hipMalloc");
+        dev->block_bytes[reinterpret_cast<uint64_t>(p)] = rounded;
+        dev->pool_allocated++;
+    }
     uint64_t addr = reinterpret_cast<uint64_t>(p);
     if (flags != CUSTOS_HIP_ALLOC_UNINIT) {
         // While recording, the fill must run now and not become part of the graph.
@@ -210,6 +249,7 @@ int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, ui
             if (e != hipSuccess) rc = hip_fail(dev, e, "hipStreamSynchronize(transfer)");
         }
         if (rc != CUSTOS_HIP_OK) {
+            dev->block_bytes.erase(addr);
             (void)hipFree(p);
             return rc;
         }
@@ -221,9 +261,40 @@ int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, ui
 int32_t custos_hip_free(custos_hip_device* dev, uint64_t dptr) {
     REQUIRE_DEV(dev);
     if (dptr == 0) return CUSTOS_HIP_OK;
+    auto known = dev->block_bytes.find(dptr);
+    if (known != dev->block_bytes.end() && dev->pooled_bytes + known->second <= dev->pool_limit) {
+        // Reuse is ordered on the compute stream behind whatever still uses the block.
+        // (A recorded graph that names the address must not be replayed after this,
+        // exactly as after a real free.)
+        dev->pool[known->second].push_back(reinterpret_cast<void*>(dptr));
+        dev->pooled_bytes += known->second;
+        return CUSTOS_HIP_OK;
+    }
+    if (known != dev->block_bytes.end()) dev->block_bytes.erase(known);
     // work that still uses the range must finish first
     if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
     HIP_TRY(dev, hipFree(reinterpret_cast<void*>(dptr)));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_pool_limit(custos_hip_device* dev, size_t limit_bytes) {
+    REQUIRE_DEV(dev);
+    dev->pool_limit = limit_bytes;
+    if (dev->pooled_bytes > limit_bytes) release_pool(dev);
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_pool_trim(custos_hip_device* dev) {
+    REQUIRE_DEV(dev);
+    release_pool(dev);
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_pool_stats(custos_hip_device* dev, size_t* pooled_bytes, uint64_t* reused, uint64_t* allocated) {
+    REQUIRE_DEV(dev);
+    if (pooled_bytes) *pooled_bytes = dev->pooled_bytes;
+    if (reused) *reused = dev->pool_reused;
+    if (allocated) *allocated = dev->pool_allocated;
     return CUSTOS_HIP_OK;
 }
 

@@ -86,6 +86,11 @@ struct custos_hip_device {
     custos_hip::Tuning tuning;
     bool capturing = false;          // recording: launches, clears and copies go to `recorded`
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
+    // allocation pool: freed blocks by rounded size; every block this handle allocated, by address
+    std::unordered_map<size_t, std::vector<void*>> pool;
+    std::unordered_map<uint64_t, size_t> block_bytes;
+    size_t pooled_bytes = 0, pool_limit = 0;
+    uint64_t pool_reused = 0, pool_allocated = 0;
     unsigned long long launch_parity = 0;  // direction of the last launch that alternates
     bool batching = true;            // merge equal independent launches of a level into one grid
     std::vector<RecNode> recorded;

@@ -139,6 +139,19 @@ class HIP:
         t = capi.Tuning(block_threads, unroll, blocks_per_cu, nontemporal, direction)
         self._check(self.lib.custos_hip_set_tuning(self.handle, C.byref(t)))
 
+    def set_pool_limit(self, limit_bytes: int) -> None:
+        """Bytes of freed blocks the device keeps for reuse (0 switches the pool off)."""
+        self._check(self.lib.custos_hip_set_pool_limit(self.handle, limit_bytes))
+
+    def pool_trim(self) -> None:
+        self._check(self.lib.custos_hip_pool_trim(self.handle))
+
+    def pool_stats(self):
+        """(bytes held in the pool, allocations served from it, allocations that went to hipMalloc)"""
+        a, b, c = C.c_size_t(0), C.c_uint64(0), C.c_uint64(0)
+        self._check(self.lib.custos_hip_pool_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
     def cache_stats(self):
         a, b = C.c_uint64(0), C.c_uint64(0)
         self._check(self.lib.custos_hip_cache_stats(self.handle, C.byref(a), C.byref(b)))

@@ -147,8 +147,23 @@ int32_t custos_hip_get_tuning(custos_hip_device *dev, custos_hip_tuning *tuning)
 
 /* Alloc::alloc.  bytes == 0 fails with ZERO_LENGTH_BUFFER. */
 int32_t custos_hip_alloc(custos_hip_device *dev, size_t bytes, int32_t flags, uint64_t *dptr);
-/* Drop of an owning CUDAPtr (src/devices/cuda/cuda_ptr.rs:64-77). 0 is ignored. */
+/* Drop of an owning CUDAPtr (src/devices/cuda/cuda_ptr.rs:64-77). 0 is ignored.
+ * The block goes back to the device's pool (below) without waiting for the
+ * stream: every later use of the address is ordered behind the work that still
+ * reads or writes it, because all device work of a handle runs on one stream. */
 int32_t custos_hip_free(custos_hip_device *dev, uint64_t dptr);
+/* Freed blocks are kept, by rounded size, and handed out again by custos_hip_alloc
+ * instead of going through hipFree / hipMalloc (tens of microseconds and a device-wide
+ * wait each; the reference's CUDA device pays cuMemAlloc / cuMemFree per buffer,
+ * src/devices/cuda/api/cuda.rs:60-78).  `limit_bytes` bounds what the pool holds; 0
+ * switches pooling off and releases what is held.  Default: a quarter of the device's
+ * memory.  When hipMalloc fails the pool is released and the allocation retried. */
+int32_t custos_hip_set_pool_limit(custos_hip_device *dev, size_t limit_bytes);
+/* Releases every pooled block to the driver (waits for the stream). */
+int32_t custos_hip_pool_trim(custos_hip_device *dev);
+/* Bytes held in the pool, allocations served from it, allocations that went to hipMalloc. */
+int32_t custos_hip_pool_stats(custos_hip_device *dev, size_t *pooled_bytes, uint64_t *reused,
+                              uint64_t *allocated);
 /* WriteBuf::write: host -> device, ordered on the compute stream; the host
  * range may be reused as soon as the call returns. */
 int32_t custos_hip_write(custos_hip_device *dev, uint64_t dst, const void *src, size_t bytes);

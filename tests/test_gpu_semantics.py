@@ -615,3 +615,46 @@ def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
             assert same.all(), f"{what} differs at {np.flatnonzero(~same)[:5]}"
         else:
             assert_bits_equal(got, want, what)
+
+
+def test_allocation_pool():
+    """Freed blocks are handed out again: same address, zero-filled again, ordered behind the
+    work that still used them; limit 0 switches the pool off; trim gives everything back."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        n = 300000
+        x = synth.uniform_f32(1, n, -1, 1)
+        a = dev.buffer(x)
+        held0, reused0, allocated0 = dev.pool_stats()
+        out = dev.apply_fn(a, lambda v: v.mul(2.0))
+        addr = out.ptr
+        want = (x * np.float32(2.0)).astype(np.float32)
+        out.free()                                   # the kernel may still be running: no wait here
+        held1, _, _ = dev.pool_stats()
+        assert held1 >= n * 4
+        again = dev.alloc(n)                         # same size class: the same block, zero-filled behind the kernel
+        assert again.ptr == addr
+        assert dev.pool_stats()[1] == reused0 + 1
+        assert not again.read().any()
+        again.free()
+        smaller = dev.alloc(n - 100)                 # rounds to the same class
+        assert smaller.ptr == addr
+        dirty = dev.apply_fn(a, lambda v: v.mul(2.0), out=smaller.slice(0, n - 100))
+        assert_bits_equal(smaller.read(), want[: n - 100])
+        smaller.free()
+        dev.pool_trim()
+        assert dev.pool_stats()[0] == 0
+        dev.set_pool_limit(0)
+        b = dev.alloc(n)
+        b.free()
+        assert dev.pool_stats()[0] == 0              # went back to the driver
+        dev.set_pool_limit(1 << 30)
+        # many eager operations reuse two blocks instead of allocating each time
+        _, reused, allocated = dev.pool_stats()
+        for _ in range(50):
+            dev.apply_fn(a, lambda v: v.add(1.0)).free()
+        _, reused2, allocated2 = dev.pool_stats()
+        assert allocated2 - allocated <= 1 and reused2 - reused >= 49
+    finally:
+        dev.close()
