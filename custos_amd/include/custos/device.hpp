@@ -70,6 +70,21 @@ class Device {
         return modules.template retrieve<T>(self(), len, ids, rg);
     }
 
+    // `retrieve` for the output of an operation that writes every element: when the
+    // operation runs at once (no Lazy module) the allocation need not be zero-filled
+    // first -- one memory pass less per eager operation.  Lazily retrieved buffers are
+    // zero-filled as always (a fused-away intermediate keeps its zeros).
+    template <class T, class... P>
+    Buffer<T, Derived> retrieve_output(size_t len, const P&... parents) {
+        struct Scope {
+            bool& flag;
+            explicit Scope(bool& f) : flag(f) { flag = true; }
+            ~Scope() { flag = false; }
+        } scope(output_hint_);
+        return retrieve<T>(len, parents...);
+    }
+    bool output_hint() const { return output_hint_; }
+
     template <class T>
     std::vector<T> read(const Buffer<T, Derived>& buf) {
         if (!buf.has_data()) throw Error(DeviceError::InvalidLazyBuf);
@@ -172,7 +187,7 @@ class Device {
     // `device.apply_fn(&buf, |x| ...)`: retrieve out, add the op, tag it with the unary hint.
     template <class T, class F>
     Buffer<T, Derived> apply_fn(const Buffer<T, Derived>& buf, F f) {
-        Buffer<T, Derived> out = retrieve<T>(buf.len(), buf);
+        Buffer<T, Derived> out = retrieve_output<T>(buf.len(), buf);
         add_op(std::tie(out, buf), [f](Buffer<T, Derived>& o, const Buffer<T, Derived>& x, Derived& dev) {
             dev.apply_fn_impl(x, o, f);
         });
@@ -186,7 +201,7 @@ class Device {
     // expression written in the `Combiner` vocabulary: out[i] = f(lhs[i], rhs[i]).
     template <class T, class F>
     Buffer<T, Derived> apply_fn2(const Buffer<T, Derived>& lhs, const Buffer<T, Derived>& rhs, F f) {
-        Buffer<T, Derived> out = retrieve<T>(lhs.len(), lhs, rhs);
+        Buffer<T, Derived> out = retrieve_output<T>(lhs.len(), lhs, rhs);
         add_op(std::tie(lhs, rhs, out),
                [f](const Buffer<T, Derived>& l, const Buffer<T, Derived>& r, Buffer<T, Derived>& o, Derived& dev) {
                    dev.apply_fn2_impl(l, r, o, f);
@@ -337,6 +352,8 @@ class Device {
     void disable_grad() { modules.set_grad_enabled(false); }
 
    private:
+    bool output_hint_ = false;
+
     template <class BufT>
     static BufT view_of(Derived& dev, Buffers& bufs, Id id) {
         using B = std::remove_const_t<BufT>;

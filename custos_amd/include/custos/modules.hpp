@@ -76,11 +76,12 @@ struct Base {
     template <class D>
     void teardown(D&) {}
 
-    // `Retrieve::retrieve`: a fresh zeroed allocation (base.rs:103-130)
+    // `Retrieve::retrieve`: a fresh zeroed allocation (base.rs:103-130); not zero-filled
+    // when the caller is an operation that overwrites all of it right away
     template <class T, class D>
     Buffer<T, D> retrieve(D& dev, size_t len, const std::vector<Id>&, const std::vector<bool>&) {
         cursor_++;
-        uint64_t ptr = dev.alloc_raw(len * sizeof(T), /*zeroed=*/true, len);
+        uint64_t ptr = dev.alloc_raw(len * sizeof(T), /*zeroed=*/!dev.output_hint(), len);
         return Buffer<T, D>::from_parts(&dev, ptr, len, Id{ptr, len}, AllocFlag::None);
     }
     template <class T, class D>

@@ -223,4 +223,29 @@ TEST_CASE(host_device_frees_everything) {
     // the device's destructor ran teardown; buffers freed themselves before
 }
 
+// Outputs of operations that run at once are not zero-filled first; lazily retrieved ones are.
+TEST_CASE(eager_outputs_skip_the_zero_fill) {
+    {
+        TestCPU<Base> dev;
+        auto buf = dev.buffer<float>({1.f, 2.f, 3.f});
+        const size_t before = dev.unzeroed_allocations;
+        auto out = dev.apply_fn(buf, [](auto x) { return x.mul(2.f); });
+        auto sum = dev.apply_fn2(buf, out, [](auto x, auto y) { return x.add(y); });
+        CHECK_EQ(dev.unzeroed_allocations, before + 2);
+        CHECK_VEC_EQ(sum.read(), (std::vector<float>{3.f, 6.f, 9.f}));
+        auto plain = dev.retrieve<float>(3, buf);       // a plain retrieve stays zeroed
+        CHECK_EQ(dev.unzeroed_allocations, before + 2);
+        CHECK_VEC_EQ(plain.read(), (std::vector<float>{0.f, 0.f, 0.f}));
+    }
+    {
+        TestCPU<Lazy<Base>> dev;
+        auto buf = dev.buffer<float>({1.f, 2.f, 3.f});
+        const size_t before = dev.unzeroed_allocations;
+        auto out = dev.apply_fn(buf, [](auto x) { return x.mul(2.f); });
+        dev.run();
+        CHECK_EQ(dev.unzeroed_allocations, before);
+        CHECK_VEC_EQ(out.replace().read(), (std::vector<float>{2.f, 4.f, 6.f}));
+    }
+}
+
 int main(int argc, char** argv) { return check::run(argc, argv); }

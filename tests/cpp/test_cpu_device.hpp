@@ -26,8 +26,16 @@ class TestCPU : public Device<TestCPU<Mods>, Mods> {
     size_t live_allocations = 0;
     size_t lazy_runs = 0;
 
-    uint64_t alloc_raw(size_t bytes, bool, size_t) {
+    size_t unzeroed_allocations = 0;
+
+    uint64_t alloc_raw(size_t bytes, bool zeroed, size_t) {
         void* p = std::calloc(bytes, 1);  // CPU alloc is zero-initialised (cpu_ptr.rs:74-85)
+        // an allocation the caller promised to overwrite: poison it, so that a test sees
+        // any element the operation leaves out
+        if (!zeroed) {
+            std::memset(p, 0xCD, bytes);
+            unzeroed_allocations++;
+        }
         live_allocations++;
         return reinterpret_cast<uint64_t>(p);
     }
