@@ -91,6 +91,9 @@ struct custos_hip_device {
     std::unordered_map<uint64_t, size_t> block_bytes;
     size_t pooled_bytes = 0, pool_limit = 0;
     uint64_t pool_reused = 0, pool_allocated = 0;
+    uint32_t* done_flag = nullptr;  // pinned host word the compute stream writes sequence numbers to
+    void* done_flag_dev = nullptr;  // its device address
+    uint32_t done_seq = 0;
     unsigned long long launch_parity = 0;  // direction of the last launch that alternates
     bool batching = true;            // merge equal independent launches of a level into one grid
     std::vector<RecNode> recorded;
@@ -138,6 +141,7 @@ inline Tuning tuning_from_c(const custos_hip_tuning* t) {
 }
 
 // device.hip
+hipError_t wait_compute_stream(custos_hip_device* dev);
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec);
 int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream);
 void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph kernel nodes
