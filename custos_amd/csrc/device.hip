@@ -357,9 +357,12 @@ int32_t custos_hip_read(custos_hip_device* dev, void* dst, uint64_t src, size_t 
     REQUIRE_DEV(dev);
     if (bytes == 0) return CUSTOS_HIP_OK;
     if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
-    if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
-    HIP_TRY(dev, hipMemcpyAsync(dst, reinterpret_cast<const void*>(src), bytes, hipMemcpyDeviceToHost, dev->transfer));
-    HIP_TRY(dev, hipStreamSynchronize(dev->transfer));
+    // Not recording: the copy is ordered on the compute stream behind the work that produces
+    // the data, one wait in all.  While recording nothing is in flight there, and the copy must
+    // not become part of the recording: it goes through the transfer stream.
+    hipStream_t s = dev->capturing ? dev->transfer : dev->stream;
+    HIP_TRY(dev, hipMemcpyAsync(dst, reinterpret_cast<const void*>(src), bytes, hipMemcpyDeviceToHost, s));
+    HIP_TRY(dev, hipStreamSynchronize(s));
     return CUSTOS_HIP_OK;
 }
 
