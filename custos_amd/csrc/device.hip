@@ -48,26 +48,40 @@ hipError_t wait_compute_stream(custos_hip_device* dev) {
 }
 
 // ---- zero fill: 16-byte stores over the aligned body, bytes at the edges ----
+//
+// Tiles of 128 threads x 2 vectors, one tile per workgroup: 6.56 TB/s over 1 GiB and
+// 6.66 over 64 MiB on MI355X, against 5.6 / 6.5 for 256-thread workgroups that loop
+// over 8 vectors per thread, 5.9-6.0 for one vector per thread, and 6.4-6.6 for
+// hipMemsetAsync (which may not be recorded into graphs here).
 
-__global__ void __launch_bounds__(256) custos_fill_zero(unsigned char* p, unsigned long long bytes,
-                                                        unsigned long long head,
-                                                        unsigned long long n_vec) {
+constexpr unsigned int kFillBlock = 128, kFillUnroll = 2;
+
+__global__ void __launch_bounds__(kFillBlock) custos_fill_zero(unsigned char* p, unsigned long long bytes,
+                                                               unsigned long long head,
+                                                               unsigned long long n_vec) {
     typedef unsigned int u4 __attribute__((ext_vector_type(4)));
     u4* v = reinterpret_cast<u4*>(p + head);
-    const unsigned long long gid = (unsigned long long)blockIdx.x * 256 + threadIdx.x;
-    const unsigned long long n_threads = (unsigned long long)gridDim.x * 256;
     const u4 z = {0u, 0u, 0u, 0u};
-    for (unsigned long long i = gid; i < n_vec; i += n_threads) v[i] = z;
+    const unsigned long long tile_vecs = (unsigned long long)kFillBlock * kFillUnroll;
+    const unsigned long long n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;
+    for (unsigned long long tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+#pragma unroll
+        for (unsigned int u = 0; u < kFillUnroll; u++) {
+            const unsigned long long i = tile * tile_vecs + (unsigned long long)u * kFillBlock + threadIdx.x;
+            if (i < n_vec) v[i] = z;
+        }
+    }
+    const unsigned long long gid = (unsigned long long)blockIdx.x * kFillBlock + threadIdx.x;
+    const unsigned long long n_threads = (unsigned long long)gridDim.x * kFillBlock;
     if (gid < head) p[gid] = 0;
     for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads) p[i] = 0;
 }
 
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec) {
-    unsigned long long want = (n_vec + 255) / 256;
-    // 8 vectors per thread at most: enough workgroups to fill the chip, not one per 4 KiB
-    unsigned long long cap = static_cast<unsigned long long>(dev->props.multiProcessorCount) * 64;
-    unsigned long long g = std::max(1ull, std::min(want, std::max(cap, (want + 7) / 8)));
-    return static_cast<unsigned int>(std::min(g, 1ull << 22));
+    (void)dev;
+    const unsigned long long tile_vecs = (unsigned long long)kFillBlock * kFillUnroll;
+    const unsigned long long tiles = (n_vec + tile_vecs - 1) / tile_vecs;
+    return static_cast<unsigned int>(std::max(1ull, std::min(tiles, 1ull << 22)));
 }
 
 int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream) {
@@ -86,7 +100,7 @@ int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hi
         return CUSTOS_HIP_OK;
     }
     unsigned int grid = fill_grid(dev, n_vec);
-    hipLaunchKernelGGL(custos_fill_zero, dim3(grid), dim3(256), 0, stream,
+    hipLaunchKernelGGL(custos_fill_zero, dim3(grid), dim3(kFillBlock), 0, stream,
                        reinterpret_cast<unsigned char*>(dptr), static_cast<unsigned long long>(bytes),
                        head, n_vec);
     HIP_TRY(dev, hipGetLastError());
@@ -94,6 +108,7 @@ int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hi
 }
 
 void* fill_zero_kernel() { return reinterpret_cast<void*>(custos_fill_zero); }
+unsigned int fill_block() { return kFillBlock; }
 
 }  // namespace custos_hip
 

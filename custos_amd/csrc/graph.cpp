@@ -243,7 +243,7 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
                 ln.func = fill_zero_kernel();
                 ln.module_fn = false;
                 ln.grid = dim3(fill_grid(dev, first.n_vec));
-                ln.block = dim3(256);
+                ln.block = dim3(fill_block());
             } else if (p.members.size() == 1) {
                 for (uint64_t ptr : first.ptrs) ln.args.push_back(value(&ptr, 8));
                 const unsigned long long a0 = first.n, a1 = first.head, a2 = first.n_vec;

@@ -143,6 +143,7 @@ inline Tuning tuning_from_c(const custos_hip_tuning* t) {
 // device.hip
 hipError_t wait_compute_stream(custos_hip_device* dev);
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec);
+unsigned int fill_block();  // threads per workgroup of the zero-fill kernel
 int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream);
 void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph kernel nodes
 
