@@ -143,7 +143,12 @@ inline Tuning tuning_from_c(const custos_hip_tuning* t) {
 // device.hip
 hipError_t wait_compute_stream(custos_hip_device* dev);
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec);
-unsigned int fill_block();  // threads per workgroup of the zero-fill kernel
+unsigned int fill_block();
+// device-to-device copies: a kernel for 16-byte aligned ranges, the runtime otherwise
+bool copy_uses_kernel(uint64_t dst, uint64_t src, size_t bytes);
+void* copy_kernel();  // host handle, for graph kernel nodes: (src, dst, n_vec, stream_hint)
+unsigned long long copy_stream_hint(size_t bytes);
+int32_t launch_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t bytes);  // threads per workgroup of the zero-fill kernel
 int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream);
 void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph kernel nodes
 

@@ -272,15 +272,18 @@ def test_recorded_dependencies_random(hip, oracle):
         g.destroy()
 
 
-def test_recorded_copy_nodes(hip):
-    x = synth.uniform_f32(3, 5000, -1, 1)
-    a, b, c = hip.buffer(x), hip.alloc(5000), hip.alloc(5000)
+@pytest.mark.parametrize("n,copy_kernels", [(5000, 2), (5001, 0)])
+def test_recorded_copy_nodes(hip, n, copy_kernels):
+    """Recorded device-to-device copies: 16-byte aligned ranges become nodes of the library's
+    copy kernel, others memcpy nodes of the runtime."""
+    x = synth.uniform_f32(3, n, -1, 1)
+    a, b, c = hip.buffer(x), hip.alloc(n), hip.alloc(n)
     hip.capture_begin()
     hip.copy(b, a)
     hip.apply_fn(b, lambda v: v.mul(2.0), out=c)
     hip.copy(a, c)
     g = hip.capture_end()
-    assert g.stats() == (3, 1, 3)
+    assert g.stats() == (3, 1 + copy_kernels, 3)
     g.launch()
     hip.sync()
     assert_bits_equal(a.read(), (x * np.float32(2.0)).astype(np.float32))
