@@ -84,54 +84,34 @@ unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec) {
     return static_cast<unsigned int>(std::max(1ull, std::min(tiles, 1ull << 22)));
 }
 
-// ---- device-to-device copy of 16-byte aligned ranges ----
+// ---- device-to-device copy ----
 //
-// The same tile shape as the generated kernels; the runtime's hipMemcpyAsync moves
-// 1 GiB at 5.06 TB/s on MI355X, this kernel at the 6.4-6.8 TB/s of the identity
-// expression.  Ranges that are not 16-byte aligned go through the runtime.
-
-__global__ void __launch_bounds__(kFillBlock) custos_copy16(const unsigned char* src, unsigned char* dst,
-                                                            unsigned long long n_vec, unsigned long long stream_hint) {
-    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
-    const u4* s = reinterpret_cast<const u4*>(src);
-    u4* d = reinterpret_cast<u4*>(dst);
-    const unsigned long long tile_vecs = (unsigned long long)kFillBlock * kFillUnroll;
-    const unsigned long long n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;
-    for (unsigned long long tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        u4 a[kFillUnroll];
-#pragma unroll
-        for (unsigned int u = 0; u < kFillUnroll; u++) {
-            const unsigned long long i = tile * tile_vecs + (unsigned long long)u * kFillBlock + threadIdx.x;
-            if (i < n_vec) a[u] = stream_hint ? __builtin_nontemporal_load(s + i) : s[i];
-        }
-#pragma unroll
-        for (unsigned int u = 0; u < kFillUnroll; u++) {
-            const unsigned long long i = tile * tile_vecs + (unsigned long long)u * kFillBlock + threadIdx.x;
-            if (i < n_vec) {
-                if (stream_hint) __builtin_nontemporal_store(a[u], d + i);
-                else d[i] = a[u];
-            }
-        }
-    }
-}
-
-bool copy_uses_kernel(uint64_t dst, uint64_t src, size_t bytes) { return ((dst | src | bytes) & 15) == 0; }
-void* copy_kernel() { return reinterpret_cast<void*>(custos_copy16); }
-// non-temporal accesses once the copy does not fit the memory-side cache
-unsigned long long copy_stream_hint(size_t bytes) { return 2ull * bytes > (256ull << 20) ? 1 : 0; }
+// A copy is the identity expression: it runs through the generated kernel for `x`
+// over 4-byte (or 1-byte) elements and so gets the launch shape, the recording and the
+// merging of every other launch; the runtime's hipMemcpyAsync moves 1 GiB at 5.06 TB/s
+// on MI355X, the identity kernel at 6.4-6.8 TB/s.  Only byte-granular ranges whose
+// source and destination sit at different 16-byte phases go through the runtime.
 
 int32_t launch_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t bytes) {
-    if (!copy_uses_kernel(dst, src, bytes)) {
+    const bool words = ((dst | src | bytes) & 3) == 0;
+    if (!words && ((dst ^ src) & 15) != 0) {
+        if (dev->capturing) {
+            RecNode node;
+            node.type = RecNode::Copy;
+            node.ptrs = {dst, src};
+            node.bytes = bytes;
+            node.acc = {{dst, dst + bytes, true}, {src, src + bytes, false}};
+            dev->recorded.push_back(std::move(node));
+            return CUSTOS_HIP_OK;
+        }
         HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src), bytes,
                                     hipMemcpyDeviceToDevice, dev->stream));
         return CUSTOS_HIP_OK;
     }
-    const unsigned long long n_vec = bytes / 16;
-    hipLaunchKernelGGL(custos_copy16, dim3(fill_grid(dev, n_vec)), dim3(kFillBlock), 0, dev->stream,
-                       reinterpret_cast<const unsigned char*>(src), reinterpret_cast<unsigned char*>(dst), n_vec,
-                       copy_stream_hint(bytes));
-    HIP_TRY(dev, hipGetLastError());
-    return CUSTOS_HIP_OK;
+    custos_hip_kernel* k = nullptr;
+    int32_t rc = identity_kernel(dev, words ? DType::U32 : DType::U8, &k);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    return launch_or_record(dev, k, {{src, false}, {dst, true}}, words ? bytes / 4 : bytes);
 }
 
 int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream) {
@@ -435,15 +415,6 @@ int32_t custos_hip_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size
     REQUIRE_DEV(dev);
     if (bytes == 0) return CUSTOS_HIP_OK;
     if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
-    if (dev->capturing) {
-        RecNode node;
-        node.type = RecNode::Copy;
-        node.ptrs = {dst, src};
-        node.bytes = bytes;
-        node.acc = {{dst, dst + bytes, true}, {src, src + bytes, false}};
-        dev->recorded.push_back(std::move(node));
-        return CUSTOS_HIP_OK;
-    }
     return launch_copy(dev, dst, src, bytes);
 }
 

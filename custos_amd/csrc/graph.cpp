@@ -226,14 +226,7 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
             LoweredNode ln;
             // a node that alternates runs against the direction of the one before it
             const unsigned long long rev = (first.type == RecNode::Kernel && p.alternate) ? (parity ^= 1) : 0;
-            if (first.type == RecNode::Copy && copy_uses_kernel(first.ptrs[0], first.ptrs[1], first.bytes)) {
-                const unsigned long long n_vec = first.bytes / 16, hint = copy_stream_hint(first.bytes);
-                ln.args = {value(&first.ptrs[1], 8), value(&first.ptrs[0], 8), value(&n_vec, 8), value(&hint, 8)};
-                ln.func = copy_kernel();
-                ln.module_fn = false;
-                ln.grid = dim3(fill_grid(dev, n_vec));
-                ln.block = dim3(fill_block());
-            } else if (first.type == RecNode::Copy) {
+            if (first.type == RecNode::Copy) {
                 ln.is_copy = true;
                 ln.dst = first.ptrs[0];
                 ln.src = first.ptrs[1];

@@ -216,6 +216,17 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
     return CUSTOS_HIP_OK;
 }
 
+int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel** out) {
+    custos_hip_kernel*& slot = dtype == DType::U32 ? dev->identity_u32 : dev->identity_u8;
+    if (!slot) {
+        const char* markers[] = {"x"};
+        int32_t rc = compile_expr(dev, CUSTOS_HIP_KIND_APPLY, static_cast<int32_t>(dtype), "x", markers, 1, dev->tuning, &slot);
+        if (rc != CUSTOS_HIP_OK) return rc;
+    }
+    *out = slot;
+    return CUSTOS_HIP_OK;
+}
+
 custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
                                   bool* alternate, bool working_set_fits_cache) {
     const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;

@@ -91,6 +91,8 @@ struct custos_hip_device {
     std::unordered_map<uint64_t, size_t> block_bytes;
     size_t pooled_bytes = 0, pool_limit = 0;
     uint64_t pool_reused = 0, pool_allocated = 0;
+    custos_hip_kernel* identity_u32 = nullptr;  // copies run through these
+    custos_hip_kernel* identity_u8 = nullptr;
     uint32_t* done_flag = nullptr;  // pinned host word the compute stream writes sequence numbers to
     void* done_flag_dev = nullptr;  // its device address
     uint32_t done_seq = 0;
@@ -144,10 +146,7 @@ inline Tuning tuning_from_c(const custos_hip_tuning* t) {
 hipError_t wait_compute_stream(custos_hip_device* dev);
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec);
 unsigned int fill_block();
-// device-to-device copies: a kernel for 16-byte aligned ranges, the runtime otherwise
-bool copy_uses_kernel(uint64_t dst, uint64_t src, size_t bytes);
-void* copy_kernel();  // host handle, for graph kernel nodes: (src, dst, n_vec, stream_hint)
-unsigned long long copy_stream_hint(size_t bytes);
+// device-to-device copy, launched or recorded: the identity kernel, or the runtime's copy
 int32_t launch_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t bytes);  // threads per workgroup of the zero-fill kernel
 int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream);
 void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph kernel nodes
@@ -156,6 +155,8 @@ void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph ker
 int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec, const std::string& arch,
                                std::vector<char>* code);
 int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k);
+// The kernel of the expression `x` over `dtype` elements (compiled once per device).
+int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel** out);
 // The kernel to launch for `footprint_bytes` touched: `k` itself, or a variant
 // compiled with the unroll factor and cache policy that suit the size (where the
 // caller left them open).  Never fails: without a variant it returns `k`.

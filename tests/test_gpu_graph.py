@@ -272,10 +272,11 @@ def test_recorded_dependencies_random(hip, oracle):
         g.destroy()
 
 
-@pytest.mark.parametrize("n,copy_kernels", [(5000, 2), (5001, 0)])
-def test_recorded_copy_nodes(hip, n, copy_kernels):
-    """Recorded device-to-device copies: 16-byte aligned ranges become nodes of the library's
-    copy kernel, others memcpy nodes of the runtime."""
+@pytest.mark.parametrize("n", [5000, 5001])
+def test_recorded_copy_nodes(hip, n):
+    """Recorded device-to-device copies are launches of the identity kernel (kernel nodes that
+    merge and alternate like any other launch); only byte-granular ranges at different 16-byte
+    phases stay memcpy nodes of the runtime."""
     x = synth.uniform_f32(3, n, -1, 1)
     a, b, c = hip.buffer(x), hip.alloc(n), hip.alloc(n)
     hip.capture_begin()
@@ -283,13 +284,29 @@ def test_recorded_copy_nodes(hip, n, copy_kernels):
     hip.apply_fn(b, lambda v: v.mul(2.0), out=c)
     hip.copy(a, c)
     g = hip.capture_end()
-    assert g.stats() == (3, 1 + copy_kernels, 3)
+    assert g.stats() == (3, 3, 3)
     g.launch()
     hip.sync()
     assert_bits_equal(a.read(), (x * np.float32(2.0)).astype(np.float32))
     g.launch()
     hip.sync()
     assert_bits_equal(a.read(), (x * np.float32(4.0)).astype(np.float32))
+    g.destroy()
+
+    raw = (np.arange(4099, dtype=np.uint32) * 37 % 251).astype(np.uint8)
+    p, q = hip.buffer(raw, "u8"), hip.alloc(4099 + 16, "u8")
+    hip.capture_begin()
+    hip.copy(q.slice(3, 3 + 4096), p.slice(1, 1 + 4096))      # phases 3 and 1: the runtime's copy
+    hip.copy(q.slice(4100, 4100 + 9), p.slice(4, 4 + 9))      # both at phase 4: the identity kernel over bytes
+    g = hip.capture_end()
+    assert g.stats()[:2] == (2, 1)
+    g.launch()
+    hip.sync()
+    got = q.read()
+    assert_bits_equal(got[3:3 + 4096], raw[1:1 + 4096])
+    assert_bits_equal(got[4100:4109], raw[4:13])
+    assert not got[:3].any() and not got[4099:4100].any() and not got[4109:].any()
+    g.destroy()
 
 
 @pytest.mark.parametrize("direct_max", [0, 1, 4])
@@ -313,7 +330,7 @@ def test_short_chain_replays_the_same_as_a_graph_or_as_plain_launches(hip, oracl
         g = hip.capture_end()
     finally:
         hip.set_graph_direct_replay(4)
-    assert g.stats() == (4, 3, 4)
+    assert g.stats() == (4, 4, 4)          # clear, kernel, copy (the identity kernel), caller-written kernel
     want = oracle.apply_fn(lambda v: v.mul(2.0).add(1.0), x) * np.float32(3.0)
     for replay in range(3):
         c.clear()
