@@ -170,7 +170,9 @@ int32_t custos_hip_write(custos_hip_device *dev, uint64_t dst, const void *src, 
 /* Read::read: waits for the compute stream unless it is capturing, then copies
  * device -> host and waits for the copy (src/devices/cuda/ops.rs:32-48). */
 int32_t custos_hip_read(custos_hip_device *dev, void *dst, uint64_t src, size_t bytes);
-/* WriteBuf::write_buf / CopySlice / CloneBuf: device -> device. */
+/* WriteBuf::write_buf / CopySlice / CloneBuf: device -> device
+ * (src/devices/cuda/ops.rs:66-117).  Runs as the identity expression through the
+ * generated kernels; ranges that overlap partly are rejected (CUSTOS_HIP_ERR_BAD_OVERLAP). */
 int32_t custos_hip_copy(custos_hip_device *dev, uint64_t dst, uint64_t src, size_t bytes);
 /* ClearBuf::clear / ZeroGrad::zero_grad (`cu_clear`, src/devices/cuda/mod.rs:59-74).
  * Implemented as a fill kernel, so it may be captured into a graph. */
