@@ -15,6 +15,8 @@
 #include <string>
 #include <type_traits>
 
+#include "half.hpp"
+
 namespace custos {
 
 template <class Derived>
@@ -50,7 +52,7 @@ struct Wrapped {
     using type = R;
 };
 template <class R>
-struct Wrapped<R, std::enable_if_t<std::is_arithmetic_v<R>>> {
+struct Wrapped<R, std::enable_if_t<std::is_arithmetic_v<R> || is_half16<R>::value>> {
     using type = Scalar<R>;
 };
 template <class R>
@@ -105,6 +107,8 @@ std::string scalar_source(N v) {
         std::string s(buf, res.ptr);
         if (s.find_first_of(".en") == std::string::npos) s += ".0";
         return s;
+    } else if constexpr (is_half16<N>::value) {
+        return scalar_source(static_cast<float>(v));
     } else if constexpr (std::is_same_v<N, bool>) {
         return v ? "true" : "false";
     } else {
@@ -140,7 +144,7 @@ struct Text : Combiner<Text> {
 namespace detail {
 template <class R>
 wrapped_t<R> wrap_operand(R r) {
-    if constexpr (std::is_arithmetic_v<R>) return Scalar<R>(r);
+    if constexpr (std::is_arithmetic_v<R> || is_half16<R>::value) return Scalar<R>(r);
     else if constexpr (std::is_convertible_v<R, const char*>) return Text(std::string(r));
     else return r;
 }

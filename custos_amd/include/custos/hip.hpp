@@ -41,20 +41,23 @@ CUSTOS_HIP_DTYPE(uint32_t, CUSTOS_HIP_U32)
 CUSTOS_HIP_DTYPE(uint64_t, CUSTOS_HIP_U64)
 #undef CUSTOS_HIP_DTYPE
 
-// f16 storage (f32 compute in the kernels); a plain 16-bit pattern on the host.
-struct f16 {
-    uint16_t bits = 0;
-};
+// 16-bit floats (custos/half.hpp): f32 compute and one rounding in the kernels for
+// f16 / bf16, every node rounded for the *_pernode types.
 template <>
 struct HipDType<f16> {
     static constexpr int32_t value = CUSTOS_HIP_F16;
 };
-struct bf16 {
-    uint16_t bits = 0;
-};
 template <>
 struct HipDType<bf16> {
     static constexpr int32_t value = CUSTOS_HIP_BF16;
+};
+template <>
+struct HipDType<f16_pernode> {
+    static constexpr int32_t value = CUSTOS_HIP_F16_PERNODE;
+};
+template <>
+struct HipDType<bf16_pernode> {
+    static constexpr int32_t value = CUSTOS_HIP_BF16_PERNODE;
 };
 
 template <class Mods>

@@ -195,4 +195,25 @@ TEST_CASE(hip_backend_errors_surface) {
     CHECK(threw);
 }
 
+// BASELINE configuration 4 through the C++ device: f16 storage, the expression computed in f32
+// and rounded once at the store -- within one unit of the last place of the host's value
+TEST_CASE(hip_f16_chain_f32_compute) {
+    HIP<Base> device;
+    const size_t n = 100003;
+    std::vector<f16> xs(n);
+    for (size_t i = 0; i < n; i++) xs[i] = f16(-2.f + 4.f * static_cast<float>((i * 7919) % n) / n);
+    auto out = device.apply_fn(device.buffer(xs), [](auto x) { return x.mul(0.5f).exp().mul(x).add(x.mul(x)); });
+    const std::vector<f16> got = out.read();
+    size_t exact = 0, off_by_more = 0;
+    for (size_t i = 0; i < n; i++) {
+        const float x = xs[i];
+        const uint16_t want = f16(std::exp(x * 0.5f) * x + x * x).bits;
+        const int dist = std::abs(static_cast<int>(got[i].bits) - static_cast<int>(want));
+        exact += dist == 0;
+        off_by_more += dist > 1;
+    }
+    CHECK_EQ(off_by_more, size_t(0));
+    CHECK(exact > n * 99 / 100);
+}
+
 int main(int argc, char** argv) { return check::run(argc, argv); }

@@ -248,4 +248,61 @@ TEST_CASE(eager_outputs_skip_the_zero_fill) {
     }
 }
 
+// f32 -> f16 against the definition: the nearest representable value, ties to the even
+// significand, found by search over the table of all finite halves (no formula shared with
+// the conversion under test).
+TEST_CASE(half_conversions_round_to_nearest_even) {
+    std::vector<double> table;  // all non-negative finite halves, ascending; index = bit pattern
+    for (uint32_t b = 0; b < 0x7c00u; b++) table.push_back(static_cast<double>(detail::f16_bits_to_f32(static_cast<uint16_t>(b))));
+    for (size_t i = 1; i < table.size(); i++) CHECK(table[i] > table[i - 1]);
+    CHECK_EQ(table[1], std::ldexp(1.0, -24));
+    CHECK_EQ(table[0x3c00], 1.0);
+    CHECK_EQ(table[0x7bff], 65504.0);
+    auto nearest = [&](double v) -> uint16_t {  // v >= 0, finite
+        if (v >= 65520.0) return 0x7c00;
+        size_t hi = std::lower_bound(table.begin(), table.end(), v) - table.begin();
+        if (hi == 0) return 0;
+        if (hi == table.size()) return 0x7bff;
+        const size_t lo = hi - 1;
+        const double dl = v - table[lo], dh = table[hi] - v;
+        if (dl < dh) return static_cast<uint16_t>(lo);
+        if (dh < dl) return static_cast<uint16_t>(hi);
+        return static_cast<uint16_t>((lo & 1) ? hi : lo);
+    };
+    std::vector<float> cases;
+    for (size_t i = 0; i + 1 < table.size(); i++) {  // every midpoint and its f32 neighbours
+        const float mid = static_cast<float>((table[i] + table[i + 1]) / 2);
+        cases.push_back(mid);
+        cases.push_back(std::nextafter(mid, 1e30f));
+        cases.push_back(std::nextafter(mid, 0.f));
+    }
+    uint64_t state = 42;
+    for (int i = 0; i < 200000; i++) {  // random bit patterns of finite floats
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        const uint32_t u = static_cast<uint32_t>(state >> 33) % 0x7f800000u;
+        cases.push_back(detail::f32_from_bits(u));
+    }
+    for (float extra : {0.f, 65504.f, 65519.996f, 65520.f, 65536.f, 1e-8f, 2.9802322e-8f, 2.9802326e-8f, 5.9604645e-8f, 3.4e38f})
+        cases.push_back(extra);
+    size_t wrong = 0;
+    for (float c : cases) {
+        const uint16_t want = nearest(static_cast<double>(c));
+        if (detail::f32_to_f16_bits(c) != want || detail::f32_to_f16_bits(-c) != (want | 0x8000u)) wrong++;
+    }
+    CHECK_EQ(wrong, size_t(0));
+    CHECK_EQ(detail::f32_to_f16_bits(INFINITY), uint16_t(0x7c00));
+    CHECK((detail::f32_to_f16_bits(NAN) & 0x7c00) == 0x7c00 && (detail::f32_to_f16_bits(NAN) & 0x3ff) != 0);
+    // bf16: ties to even on the 16 dropped bits
+    CHECK_EQ(detail::f32_to_bf16_bits(detail::f32_from_bits(0x3F808000u)), uint16_t(0x3F80));
+    CHECK_EQ(detail::f32_to_bf16_bits(detail::f32_from_bits(0x3F818000u)), uint16_t(0x3F82));
+    CHECK_EQ(detail::f32_to_bf16_bits(detail::f32_from_bits(0x3F808001u)), uint16_t(0x3F81));
+    // arithmetic rounds at every operation (src/number.rs:487-676)
+    const f16 a(0.1f), b(0.2f);
+    CHECK_EQ((a + b).bits, detail::f32_to_f16_bits(float(a) + float(b)));
+    CHECK_EQ((a * b).bits, detail::f32_to_f16_bits(float(a) * float(b)));
+    CHECK_EQ((-a).bits, uint16_t(a.bits ^ 0x8000));
+    CHECK_EQ(eval<f16>(Resolve<f16>::with_val(f16(1.5f)).mul(f16(1.5f)).add(2.f)).bits, f16(4.25f).bits);
+    CHECK_EQ(to_cl_source(Resolve<f16>::with_marker("x").mul(f16(0.5f)).exp()), std::string("exp((x * 0.5))"));
+}
+
 int main(int argc, char** argv) { return check::run(argc, argv); }

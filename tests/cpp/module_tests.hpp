@@ -892,6 +892,37 @@ void autograd_no_grads_pool() {
     }
 }
 
+// ---- 16-bit floats ----
+
+// `half::f16` / `half::bf16` as element types (src/number.rs:487-676, src/devices/cdatatype.rs:53-62):
+// the per-node types give the same bits on the device as the host evaluation of the expression
+template <template <class> class DEV, class H>
+void half_per_node_type() {
+    DEV<Base> device;
+    const size_t n = 2003;
+    std::vector<H> xs(n), ys(n);
+    for (size_t i = 0; i < n; i++) {
+        xs[i] = H(-3.f + 6.f * static_cast<float>((i * 7919) % n) / n);
+        ys[i] = H(0.5f + 1.5f * static_cast<float>((i * 104729) % n) / n);
+    }
+    auto f = [](auto a, auto b) { return a.mul(0.3f).add(b).mul(a).div(b.add(1.7f)).sub(0.1f).abs().sqrt().max(0.25f).neg(); };
+    auto bx = device.buffer(xs), by = device.buffer(ys);
+    const std::vector<H> got = device.apply_fn2(bx, by, f).read();
+    size_t wrong = 0;
+    for (size_t i = 0; i < n; i++)
+        wrong += got[i].bits != eval<H>(f(Resolve<H>::with_val(xs[i]), Resolve<H>::with_val(ys[i]))).bits;
+    CHECK_EQ(wrong, size_t(0));
+    // gradient: g + round(o * d), both rounded
+    auto d = [](auto v) { return v.mul(v).mul(3.f).add(0.7f); };
+    std::vector<H> g0(n, H(0.5f));
+    auto bg = device.buffer(g0);
+    device.add_unary_grad(bx, bg, by, d);
+    const std::vector<H> g1 = bg.read();
+    wrong = 0;
+    for (size_t i = 0; i < n; i++) wrong += g1[i].bits != (g0[i] + ys[i] * eval<H>(d(Resolve<H>::with_val(xs[i])))).bits;
+    CHECK_EQ(wrong, size_t(0));
+}
+
 // ---- CopySlice / CloneBuf ----
 
 // tests/slice_buf.rs:5-84, tests/clone_buf.rs:5-49
@@ -1106,6 +1137,8 @@ void cached_errors() {
     TEST_CASE(cached_mismatched_types_optimize) { module_tests::cached_sliced_chained_optimize<DEV>(true); } \
     TEST_CASE(lazy_mismatched_types_keep_their_allocation) { module_tests::lazy_mismatched_types_keep_their_allocation<DEV>(); } \
     TEST_CASE(autograd_no_grads_pool) { module_tests::autograd_no_grads_pool<DEV>(); }            \
+    TEST_CASE(half_f16_per_node) { module_tests::half_per_node_type<DEV, f16_pernode>(); }        \
+    TEST_CASE(half_bf16_per_node) { module_tests::half_per_node_type<DEV, bf16_pernode>(); }      \
     TEST_CASE(copy_slice_and_clone_buf) { module_tests::copy_slice_and_clone_buf<DEV>(); }        \
     TEST_CASE(cached_same_allocation_every_epoch) { module_tests::cached_same_allocation_every_epoch<DEV>(); } \
     TEST_CASE(cached_multi_level_retrieve) { module_tests::cached_multi_level_retrieve<DEV>(); }  \
