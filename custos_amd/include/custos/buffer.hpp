@@ -108,6 +108,8 @@ class Buffer {
         return device.template try_grad_of<T>(id_);
     }
 
+    // `impl Clone for Buffer` (src/buffer.rs:598-606): a new buffer with the same contents.
+    Buffer clone() const { return device_->clone_buf(*this); }
     // `buf.empty_like()`: a new zeroed buffer of the same length.
     Buffer empty_like() const { return device_->template new_buffer<T>(len_); }
 

@@ -943,6 +943,8 @@ void copy_slice_and_clone_buf() {
     auto dest2 = device.template buffer<float>({5.f, 4.f, 3.f, 2.f, 1.f});
     device.copy_slice_to(source, 1, 3, dest2, 3, 5);
     CHECK_VEC_EQ(dest2.read(), (std::vector<float>{5.f, 4.f, 3.f, 2.f, 6.f}));
+    auto self_cloned = source.clone();   // tests/clone_buf.rs:17-23 (test_self_buf_clone)
+    CHECK_VEC_EQ(self_cloned.read(), source.read());
     auto cloned = device.clone_buf(source);
     CHECK_VEC_EQ(cloned.read(), source.read());
     CHECK(cloned.ptr() != source.ptr());
