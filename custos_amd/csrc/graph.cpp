@@ -77,229 +77,201 @@ bool batchable(const RecNode& n) {
     return true;
 }
 
-}  // namespace
+// One node of the graph to be: a recorded piece of work, or several launches merged.
+struct Planned {
+    std::vector<size_t> members;  // indices into the recorded list; more than one = one merged launch
+    bool ragged = false;          // members differ in length
+    size_t table_offset = 0;      // in u64 entries
+    size_t map_offset = 0;        // ragged: start of the block map, in u64 entries
+    size_t blocks = 0;            // ragged: workgroups
+    custos_hip_kernel* kern = nullptr;  // kernels: the variant that suits the bytes the node touches
+    bool alternate = false;             // kernels: walks its tiles against the previous such node
+};
 
-int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
-    std::vector<RecNode>& nodes = dev->recorded;
-    assign_levels(nodes);
-    int max_level = -1;
-    for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
-    g->recorded = nodes.size();
-    g->levels = static_cast<size_t>(max_level + 1);
+unsigned long long tiles_of(const custos_hip_kernel* k, const RecNode& n) {
+    const Tuning& t = k->spec.tuning;
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+    return std::max(1ull, (n.n_vec + tile_vecs - 1) / tile_vecs);
+}
 
-    // plan: per level, either single nodes or batches of node indices
-    struct Planned {
-        std::vector<size_t> members;  // indices into `nodes`; more than one = one merged launch
-        bool ragged = false;          // members differ in length
-        size_t table_offset = 0;      // in u64 entries
-        size_t map_offset = 0;        // ragged: start of the block map, in u64 entries
-        size_t blocks = 0;            // ragged: workgroups
-        custos_hip_kernel* kern = nullptr;  // kernels: the variant that suits the bytes the node touches
-        bool alternate = false;             // kernels: walks its tiles against the previous such node
-    };
-    auto tiles_of = [](const custos_hip_kernel* k, const RecNode& n) {
-        const Tuning& t = k->spec.tuning;
-        const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
-        return std::max(1ull, (n.n_vec + tile_vecs - 1) / tile_vecs);
-    };
-    // Everything the graph touches, as the union of the recorded address ranges.  While it
-    // fits the memory-side cache (256 MiB, with some slack: a chain over 288 MiB still gains
-    // 4 %, over 192 MiB 9.5 %, over 384 MiB nothing, over 1.5 GiB it loses 10 %), every kernel
-    // of the graph uses temporal accesses: the next kernel, and the next replay, find the data
-    // in the cache.  Caller-written kernels are not counted.
-    bool fits_cache = false;
-    {
-        std::vector<std::pair<uint64_t, uint64_t>> ranges;
-        for (const RecNode& n : nodes)
-            for (const Access& a : n.acc)
-                if (a.end > a.begin) ranges.push_back({a.begin, a.end});
-        std::sort(ranges.begin(), ranges.end());
-        unsigned long long working_set = 0;
-        uint64_t covered = 0;
-        for (const auto& r : ranges) {
-            const uint64_t from = std::max(r.first, covered);
-            if (r.second > from) working_set += r.second - from;
-            covered = std::max(covered, r.second);
-        }
-        // (only a graph with consumers after producers: more than one dependency level)
-        fits_cache = max_level >= 1 && working_set <= kCacheWorkingSet;
+// Everything the graph touches, as the union of the recorded address ranges.  While it
+// fits the memory-side cache (256 MiB, with some slack: a chain over 288 MiB still gains
+// 4 %, over 192 MiB 9.5 %, over 384 MiB nothing, over 1.5 GiB it loses 10 %) and the graph
+// has consumers after producers, every kernel of the graph uses temporal accesses: the next
+// kernel, and the next replay, find the data in the cache.  Caller-written kernels are not
+// counted.
+bool working_set_fits_cache(const std::vector<RecNode>& nodes, int max_level) {
+    if (max_level < 1) return false;
+    std::vector<std::pair<uint64_t, uint64_t>> ranges;
+    for (const RecNode& n : nodes)
+        for (const Access& a : n.acc)
+            if (a.end > a.begin) ranges.push_back({a.begin, a.end});
+    std::sort(ranges.begin(), ranges.end());
+    unsigned long long working_set = 0;
+    uint64_t covered = 0;
+    for (const auto& r : ranges) {
+        const uint64_t from = std::max(r.first, covered);
+        if (r.second > from) working_set += r.second - from;
+        covered = std::max(covered, r.second);
     }
+    return working_set <= kCacheWorkingSet;
+}
 
-    // the launch shape follows the bytes the (merged) launch touches
-    auto choose_kernel = [&](Planned& p) {
-        const RecNode& first = nodes[p.members[0]];
-        if (first.type != RecNode::Kernel) return;
-        unsigned long long footprint = 0;
-        for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
-        custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, fits_cache);
-        const bool usable = p.members.size() == 1 || (p.ragged ? v->fn_ragged != nullptr : v->fn_batched != nullptr);
-        p.kern = usable ? v : first.k;
-    };
-    std::vector<std::vector<Planned>> plan(static_cast<size_t>(max_level + 1));
-    std::vector<uint64_t> host_table;
-    for (int level = 0; level <= max_level; level++) {
-        std::vector<Planned>& out = plan[level];
-        // candidates for merging, grouped by kernel in first-seen order
-        std::vector<std::pair<custos_hip_kernel*, std::vector<size_t>>> groups;
-        for (size_t i = 0; i < nodes.size(); i++) {
-            if (nodes[i].level != level) continue;
-            if (dev->batching && batchable(nodes[i])) {
-                auto g = std::find_if(groups.begin(), groups.end(), [&](const auto& kv) { return kv.first == nodes[i].k; });
-                if (g == groups.end()) {
-                    groups.push_back({nodes[i].k, {}});
-                    g = groups.end() - 1;
+// The nodes of one dependency level: launches of one kernel are merged (equal lengths into a
+// `_batched` grid, different lengths into a `_ragged` one), everything else stays single.
+// Operand tables and block maps of the merged launches are appended to `host_table`.
+std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNode>& nodes, int level,
+                                bool fits_cache, std::vector<uint64_t>* host_table) {
+    std::vector<Planned> out;
+    // candidates for merging, grouped by kernel in first-seen order
+    std::vector<std::pair<custos_hip_kernel*, std::vector<size_t>>> groups;
+    for (size_t i = 0; i < nodes.size(); i++) {
+        if (nodes[i].level != level) continue;
+        if (dev->batching && batchable(nodes[i])) {
+            auto g = std::find_if(groups.begin(), groups.end(), [&](const auto& kv) { return kv.first == nodes[i].k; });
+            if (g == groups.end()) {
+                groups.push_back({nodes[i].k, {}});
+                g = groups.end() - 1;
+            }
+            g->second.push_back(i);
+        } else {
+            out.emplace_back();
+            out.back().members.push_back(i);
+        }
+    }
+    for (auto& g : groups) {
+        bool uniform = true;
+        for (size_t i : g.second) uniform = uniform && nodes[i].n == nodes[g.second[0]].n;
+        if (uniform || !g.first->fn_ragged) {
+            // equal lengths: one grid, segment = block / tiles per segment.  (Without the
+            // ragged entry point, different lengths fall back to one batch per length.)
+            std::vector<std::pair<unsigned long long, Planned>> by_n;
+            for (size_t i : g.second) {
+                auto it = std::find_if(by_n.begin(), by_n.end(), [&](const auto& kv) { return kv.first == nodes[i].n; });
+                if (it == by_n.end()) {
+                    by_n.push_back({nodes[i].n, Planned{}});
+                    it = by_n.end() - 1;
                 }
-                g->second.push_back(i);
-            } else {
+                it->second.members.push_back(i);
+            }
+            for (auto& kv : by_n) out.push_back(std::move(kv.second));
+            continue;
+        }
+        // different lengths: one grid with a block map; a launch that fills the chip on its
+        // own stays a launch of its own
+        Planned merged;
+        for (size_t i : g.second) {
+            if (tiles_of(nodes[i].k, nodes[i]) > kRaggedMaxTiles) {
                 out.emplace_back();
                 out.back().members.push_back(i);
-            }
-        }
-        for (auto& g : groups) {
-            bool uniform = true;
-            for (size_t i : g.second) uniform = uniform && nodes[i].n == nodes[g.second[0]].n;
-            Planned merged;
-            if (uniform || !g.first->fn_ragged) {
-                // equal lengths: one grid, segment = block / tiles per segment.  (Without the
-                // ragged entry point, different lengths fall back to one batch per length.)
-                std::vector<std::pair<unsigned long long, Planned>> by_n;
-                for (size_t i : g.second) {
-                    auto it = std::find_if(by_n.begin(), by_n.end(), [&](const auto& kv) { return kv.first == nodes[i].n; });
-                    if (it == by_n.end()) {
-                        by_n.push_back({nodes[i].n, Planned{}});
-                        it = by_n.end() - 1;
-                    }
-                    it->second.members.push_back(i);
-                }
-                for (auto& kv : by_n) out.push_back(std::move(kv.second));
-                continue;
-            }
-            // different lengths: one grid with a block map; a launch that fills the
-            // chip on its own stays a launch of its own
-            merged.ragged = true;
-            for (size_t i : g.second) {
-                if (tiles_of(nodes[i].k, nodes[i]) > kRaggedMaxTiles) {
-                    out.emplace_back();
-                    out.back().members.push_back(i);
-                } else {
-                    merged.members.push_back(i);
-                }
-            }
-            if (merged.members.size() == 1) merged.ragged = false;
-            if (!merged.members.empty()) out.push_back(std::move(merged));
-        }
-        for (Planned& p : out) {
-            choose_kernel(p);
-            if (p.members.size() < 2) continue;
-            p.table_offset = host_table.size();
-            for (size_t seg = 0; seg < p.members.size(); seg++) {
-                const RecNode& n = nodes[p.members[seg]];
-                for (uint64_t ptr : n.ptrs) host_table.push_back(ptr);
-                if (p.ragged) host_table.push_back(n.n);
-            }
-            if (!p.ragged) continue;
-            p.map_offset = host_table.size();
-            for (size_t seg = 0; seg < p.members.size(); seg++) {
-                const unsigned long long tiles = tiles_of(p.kern, nodes[p.members[seg]]);
-                for (unsigned long long t = 0; t < tiles; t++) host_table.push_back(static_cast<uint64_t>(seg) << 32 | t);
-            }
-            p.blocks = host_table.size() - p.map_offset;
-        }
-    }
-    if (!host_table.empty()) {
-        HIP_TRY(dev, hipMalloc(&g->table, host_table.size() * sizeof(uint64_t)));
-        HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
-    }
-
-    // lower every planned node to function + shape + argument values
-    auto value = [](const void* p, size_t n) {
-        const unsigned char* c = static_cast<const unsigned char*>(p);
-        return std::vector<unsigned char>(c, c + n);
-    };
-    std::vector<std::vector<LoweredNode>> lowered(plan.size());
-    unsigned long long parity = 0;
-    size_t total = 0;
-    bool chain = true;
-    for (int level = 0; level <= max_level; level++) {
-        for (const Planned& p : plan[level]) {
-            const RecNode& first = nodes[p.members[0]];
-            LoweredNode ln;
-            // a node that alternates runs against the direction of the one before it
-            const unsigned long long rev = (first.type == RecNode::Kernel && p.alternate) ? (parity ^= 1) : 0;
-            if (first.type == RecNode::Copy) {
-                ln.is_copy = true;
-                ln.dst = first.ptrs[0];
-                ln.src = first.ptrs[1];
-                ln.bytes = first.bytes;
-            } else if (first.type == RecNode::Source) {
-                ln.args = first.arg_values;
-                ln.func = reinterpret_cast<void*>(first.k->fn);
-                ln.grid = dim3(first.grid3[0], first.grid3[1], first.grid3[2]);
-                ln.block = dim3(first.block3[0], first.block3[1], first.block3[2]);
-                ln.shared_mem = first.shared_mem;
-            } else if (first.type == RecNode::Fill) {
-                const unsigned long long a0 = first.bytes, a1 = first.head, a2 = first.n_vec;
-                ln.args = {value(&first.ptrs[0], 8), value(&a0, 8), value(&a1, 8), value(&a2, 8)};
-                ln.func = fill_zero_kernel();
-                ln.module_fn = false;
-                ln.grid = dim3(fill_grid(dev, first.n_vec));
-                ln.block = dim3(fill_block());
-            } else if (p.members.size() == 1) {
-                for (uint64_t ptr : first.ptrs) ln.args.push_back(value(&ptr, 8));
-                const unsigned long long a0 = first.n, a1 = first.head, a2 = first.n_vec;
-                ln.args.push_back(value(&a0, 8));
-                ln.args.push_back(value(&a1, 8));
-                ln.args.push_back(value(&a2, 8));
-                ln.args.push_back(value(&rev, 8));
-                ln.func = reinterpret_cast<void*>(p.kern->fn);
-                ln.grid = dim3(launch_grid(dev, p.kern, first.n, first.n_vec));
-                ln.block = dim3(static_cast<unsigned int>(p.kern->spec.tuning.block_threads));
-            } else if (p.ragged) {
-                if (p.blocks > (1ull << 31) - 1)
-                    return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
-                const uint64_t table = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
-                const uint64_t map = reinterpret_cast<uint64_t>(g->table) + p.map_offset * sizeof(uint64_t);
-                ln.args = {value(&table, 8), value(&map, 8), value(&rev, 8)};
-                ln.func = reinterpret_cast<void*>(p.kern->fn_ragged);
-                ln.grid = dim3(static_cast<unsigned int>(p.blocks));
-                ln.block = dim3(static_cast<unsigned int>(p.kern->spec.tuning.block_threads));
             } else {
-                const Tuning& t = p.kern->spec.tuning;
-                const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
-                const unsigned long long tiles_per_seg = std::max(1ull, (first.n_vec + tile_vecs - 1) / tile_vecs);
-                const unsigned long long blocks = tiles_per_seg * p.members.size();
-                if (blocks > (1ull << 31) - 1)
-                    return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a batched launch would need more than 2^31 workgroups");
-                const uint64_t table = reinterpret_cast<uint64_t>(g->table) + p.table_offset * sizeof(uint64_t);
-                const unsigned long long a0 = first.n, a1 = first.n_vec;
-                ln.args = {value(&table, 8), value(&a0, 8), value(&a1, 8), value(&tiles_per_seg, 8), value(&rev, 8)};
-                ln.func = reinterpret_cast<void*>(p.kern->fn_batched);
-                ln.grid = dim3(static_cast<unsigned int>(blocks));
-                ln.block = dim3(static_cast<unsigned int>(t.block_threads));
+                merged.members.push_back(i);
             }
-            if (first.type == RecNode::Kernel && p.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
-            if (!ln.is_copy) g->kernel_nodes++;
-            lowered[level].push_back(std::move(ln));
-            total++;
         }
-        chain = chain && lowered[level].size() == 1;
+        merged.ragged = merged.members.size() > 1;
+        if (!merged.members.empty()) out.push_back(std::move(merged));
     }
-
-    if (chain && total <= dev->direct_replay_max) {
-        for (auto& level : lowered) g->direct.push_back(std::move(level[0]));
-        // With an odd number of alternating nodes the first one of the next replay would
-        // run in the direction of the last one of this replay: flip them all every replay.
-        size_t alternating = 0;
-        for (const LoweredNode& ln : g->direct) alternating += ln.rev_arg >= 0;
-        g->flip_each_replay = alternating % 2 == 1;
-        return CUSTOS_HIP_OK;
+    for (Planned& p : out) {
+        const RecNode& first = nodes[p.members[0]];
+        if (first.type == RecNode::Kernel) {
+            // the launch shape follows the bytes the (merged) launch touches
+            unsigned long long footprint = 0;
+            for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
+            custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, fits_cache);
+            const bool usable = p.members.size() == 1 || (p.ragged ? v->fn_ragged != nullptr : v->fn_batched != nullptr);
+            p.kern = usable ? v : first.k;
+        }
+        if (p.members.size() < 2) continue;
+        p.table_offset = host_table->size();
+        for (size_t member : p.members) {
+            for (uint64_t ptr : nodes[member].ptrs) host_table->push_back(ptr);
+            if (p.ragged) host_table->push_back(nodes[member].n);
+        }
+        if (!p.ragged) continue;
+        p.map_offset = host_table->size();
+        for (size_t seg = 0; seg < p.members.size(); seg++) {
+            const unsigned long long tiles = tiles_of(p.kern, nodes[p.members[seg]]);
+            for (unsigned long long t = 0; t < tiles; t++) host_table->push_back(static_cast<uint64_t>(seg) << 32 | t);
+        }
+        p.blocks = host_table->size() - p.map_offset;
     }
+    return out;
+}
 
+std::vector<unsigned char> value(const void* p, size_t n) {
+    const unsigned char* c = static_cast<const unsigned char*>(p);
+    return std::vector<unsigned char>(c, c + n);
+}
+
+// A planned node in launchable form: function, launch shape, argument values.  `rev` is the
+// direction argument of a generated kernel; `table` the device address of the graph's tables.
+int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, const Planned& p, uint64_t table,
+                   unsigned long long rev, LoweredNode* out) {
+    const RecNode& first = nodes[p.members[0]];
+    LoweredNode ln;
+    if (first.type == RecNode::Copy) {
+        ln.is_copy = true;
+        ln.dst = first.ptrs[0];
+        ln.src = first.ptrs[1];
+        ln.bytes = first.bytes;
+    } else if (first.type == RecNode::Source) {
+        ln.args = first.arg_values;
+        ln.func = reinterpret_cast<void*>(first.k->fn);
+        ln.grid = dim3(first.grid3[0], first.grid3[1], first.grid3[2]);
+        ln.block = dim3(first.block3[0], first.block3[1], first.block3[2]);
+        ln.shared_mem = first.shared_mem;
+    } else if (first.type == RecNode::Fill) {
+        const unsigned long long a0 = first.bytes, a1 = first.head, a2 = first.n_vec;
+        ln.args = {value(&first.ptrs[0], 8), value(&a0, 8), value(&a1, 8), value(&a2, 8)};
+        ln.func = fill_zero_kernel();
+        ln.module_fn = false;
+        ln.grid = dim3(fill_grid(dev, first.n_vec));
+        ln.block = dim3(fill_block());
+    } else {
+        const Tuning& t = p.kern->spec.tuning;
+        ln.block = dim3(static_cast<unsigned int>(t.block_threads));
+        if (p.members.size() == 1) {
+            for (uint64_t ptr : first.ptrs) ln.args.push_back(value(&ptr, 8));
+            const unsigned long long a0 = first.n, a1 = first.head, a2 = first.n_vec;
+            ln.args.push_back(value(&a0, 8));
+            ln.args.push_back(value(&a1, 8));
+            ln.args.push_back(value(&a2, 8));
+            ln.func = reinterpret_cast<void*>(p.kern->fn);
+            ln.grid = dim3(launch_grid(dev, p.kern, first.n, first.n_vec));
+        } else if (p.ragged) {
+            if (p.blocks > (1ull << 31) - 1)
+                return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
+            const uint64_t rows = table + p.table_offset * sizeof(uint64_t);
+            const uint64_t map = table + p.map_offset * sizeof(uint64_t);
+            ln.args = {value(&rows, 8), value(&map, 8)};
+            ln.func = reinterpret_cast<void*>(p.kern->fn_ragged);
+            ln.grid = dim3(static_cast<unsigned int>(p.blocks));
+        } else {
+            const unsigned long long tiles_per_seg = tiles_of(p.kern, first);
+            const unsigned long long blocks = tiles_per_seg * p.members.size();
+            if (blocks > (1ull << 31) - 1)
+                return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a batched launch would need more than 2^31 workgroups");
+            const uint64_t rows = table + p.table_offset * sizeof(uint64_t);
+            const unsigned long long a0 = first.n, a1 = first.n_vec;
+            ln.args = {value(&rows, 8), value(&a0, 8), value(&a1, 8), value(&tiles_per_seg, 8)};
+            ln.func = reinterpret_cast<void*>(p.kern->fn_batched);
+            ln.grid = dim3(static_cast<unsigned int>(blocks));
+        }
+        ln.args.push_back(value(&rev, 8));  // every generated entry point ends with the direction
+        if (p.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
+    }
+    *out = std::move(ln);
+    return CUSTOS_HIP_OK;
+}
+
+// The levels as an instantiated hipGraph: the nodes of a level side by side, one empty join
+// node between levels instead of |previous| x |level| edges.
+int32_t instantiate(custos_hip_device* dev, custos_hip_graph* g, std::vector<std::vector<LoweredNode>>& lowered) {
     HIP_TRY(dev, hipGraphCreate(&g->graph, 0));
     std::vector<hipGraphNode_t> prev;  // what the nodes of the current level wait for
     for (auto& level : lowered) {
         std::vector<hipGraphNode_t> deps = prev;
-        if (deps.size() > 1) {  // one join node instead of |prev| x |level| edges
+        if (deps.size() > 1) {
             hipGraphNode_t join;
             HIP_TRY(dev, hipGraphAddEmptyNode(&join, g->graph, deps.data(), deps.size()));
             deps = {join};
@@ -330,6 +302,55 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     }
     HIP_TRY(dev, hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
     return CUSTOS_HIP_OK;
+}
+
+}  // namespace
+
+int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
+    std::vector<RecNode>& nodes = dev->recorded;
+    assign_levels(nodes);
+    int max_level = -1;
+    for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
+    g->recorded = nodes.size();
+    g->levels = static_cast<size_t>(max_level + 1);
+
+    const bool fits_cache = working_set_fits_cache(nodes, max_level);
+    std::vector<std::vector<Planned>> plan;
+    std::vector<uint64_t> host_table;
+    for (int level = 0; level <= max_level; level++) plan.push_back(plan_level(dev, nodes, level, fits_cache, &host_table));
+    if (!host_table.empty()) {
+        HIP_TRY(dev, hipMalloc(&g->table, host_table.size() * sizeof(uint64_t)));
+        HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
+    }
+
+    std::vector<std::vector<LoweredNode>> lowered(plan.size());
+    unsigned long long parity = 0;
+    size_t total = 0;
+    bool chain = true;
+    for (size_t level = 0; level < plan.size(); level++) {
+        for (const Planned& p : plan[level]) {
+            // a node that alternates runs against the direction of the one before it
+            const unsigned long long rev = p.alternate ? (parity ^= 1) : 0;
+            LoweredNode ln;
+            int32_t rc = lower_node(dev, nodes, p, reinterpret_cast<uint64_t>(g->table), rev, &ln);
+            if (rc != CUSTOS_HIP_OK) return rc;
+            if (!ln.is_copy) g->kernel_nodes++;
+            lowered[level].push_back(std::move(ln));
+            total++;
+        }
+        chain = chain && lowered[level].size() == 1;
+    }
+
+    if (chain && total <= dev->direct_replay_max) {
+        for (auto& level : lowered) g->direct.push_back(std::move(level[0]));
+        // With an odd number of alternating nodes the first one of the next replay would
+        // run in the direction of the last one of this replay: flip them all every replay.
+        size_t alternating = 0;
+        for (const LoweredNode& ln : g->direct) alternating += ln.rev_arg >= 0;
+        g->flip_each_replay = alternating % 2 == 1;
+        return CUSTOS_HIP_OK;
+    }
+    return instantiate(dev, g, lowered);
 }
 
 int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
