@@ -163,6 +163,195 @@ std::string grad_fn(DType dtype) {
            "    return (C)((" + U + ")g + (" + U + ")prod);\n}\n";
 }
 
+// Text of the per-element function, the tile function and the three entry points of one
+// kernel.  Operand naming inside a kernel: in0.. are the inputs, `out` the output; for a unary
+// gradient 0 = lhs, 1 = lhs_grad (also the output), 2 = out_grad.
+struct KernelText {
+    const KernelSpec& k;
+    const int n_in;    // inputs of the expression
+    const int n_ops;   // values custos_elem takes
+    const int n_ptrs;  // pointers per operand set (table row of a merged launch)
+    std::string params;     // pointer parameters of the single-launch entry point
+    std::string vec_ptrs;   // declarations of the vector views of the operands
+    std::string tile_args;  // the views custos_tile takes
+
+    explicit KernelText(const KernelSpec& spec)
+        : k(spec),
+          n_in(spec.expr.n_vars),
+          n_ops(spec.kind == Kind::Apply ? spec.expr.n_vars : 3),
+          n_ptrs(spec.kind == Kind::Apply ? spec.expr.n_vars + 1 : 3) {
+        if (k.kind == Kind::Apply) {
+            for (int i = 0; i < n_in; i++) {
+                const std::string id = std::to_string(i);
+                params += "const S* in" + id + ", ";
+                vec_ptrs += "    const vec_t* vin" + id + " = (const vec_t*)(in" + id + " + head);\n";
+            }
+            params += "S* out";
+            vec_ptrs += "    vec_t* vout = (vec_t*)(out + head);\n";
+        } else {
+            params = "const S* in0, S* out, const S* in2";
+            vec_ptrs = "    const vec_t* vin0 = (const vec_t*)(in0 + head);\n"
+                       "    const vec_t* vin2 = (const vec_t*)(in2 + head);\n"
+                       "    vec_t* vout = (vec_t*)(out + head);\n"
+                       "    const vec_t* vin1 = vout;\n"
+                       "    const S* in1 = out;\n";
+        }
+        for (int i = 0; i < n_ops; i++) {
+            if (k.kind == Kind::UnaryGrad && i == 1) continue;  // vin1 is vout
+            tile_args += "vin" + std::to_string(i) + ", ";
+        }
+    }
+
+    // "pre0post, pre1post, ..." over the values custos_elem takes
+    std::string list(const std::string& pre, const std::string& post) const {
+        std::string r;
+        for (int i = 0; i < n_ops; i++) r += std::string(i ? ", " : "") + pre + std::to_string(i) + post;
+        return r;
+    }
+
+    // Per-element function on storage values: `custos_elem(in0.., [g])`.
+    std::string elem_fn() const {
+        std::string s;
+        if (k.kind == Kind::Apply) {
+            s += "static __device__ __forceinline__ S custos_elem(";
+            for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "const S s" + std::to_string(i);
+            s += ") {\n    return custos_store(custos_expr(";
+            for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "custos_load(s" + std::to_string(i) + ")";
+            s += "));\n}\n";
+        } else {
+            s += grad_fn(k.dtype);
+            s += "static __device__ __forceinline__ S custos_elem(const S s0, const S s1, const S s2) {\n"
+                 "    return custos_store(custos_grad(custos_load(s1), custos_load(s2), custos_expr(custos_load(s0))));\n}\n";
+        }
+        return s;
+    }
+
+    // One tile: every lane loads all its vectors, then computes and stores.  `base` is the
+    // lane's first vector; a partial last tile takes the masked path.  Pointers that are read
+    // and written (`out`, `lhs_grad`) carry no __restrict__: the output may be exactly one of
+    // the inputs.
+    std::string tile_fn() const {
+        std::string tile_params;
+        for (int i = 0; i < n_ops; i++) {
+            if (k.kind == Kind::UnaryGrad && i == 1) continue;
+            tile_params += "const vec_t* vin" + std::to_string(i) + ", ";
+        }
+        std::string s;
+        s += "static __device__ __forceinline__ void custos_tile(" + tile_params + "vec_t* vout, const u64 base, const u64 n_vec) {\n";
+        if (k.kind == Kind::UnaryGrad) s += "    const vec_t* vin1 = vout;\n";
+        s += "    if (base + (u64)(CUSTOS_UNROLL - 1) * CUSTOS_BLOCK < n_vec) {\n";
+        for (int i = 0; i < n_ops; i++) s += "        vec_t a" + std::to_string(i) + "[CUSTOS_UNROLL];\n";
+        s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+        for (int i = 0; i < n_ops; i++) {
+            const std::string id = std::to_string(i);
+            s += "            a" + id + "[u] = CUSTOS_LD(vin" + id + " + base + (u64)u * CUSTOS_BLOCK);\n";
+        }
+        s += "        }\n";
+        s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+        s += "            vec_t r;\n#pragma unroll\n            for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
+             list("a", "[u][k]") + ");\n";
+        s += "            CUSTOS_ST(vout + base + (u64)u * CUSTOS_BLOCK, r);\n        }\n";
+        s += "    } else {\n";
+        s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+        s += "            const u64 idx = base + (u64)u * CUSTOS_BLOCK;\n";
+        s += "            if (idx < n_vec) {\n";
+        for (int i = 0; i < n_ops; i++) {
+            const std::string id = std::to_string(i);
+            s += "                const vec_t b" + id + " = CUSTOS_LD(vin" + id + " + idx);\n";
+        }
+        s += "                vec_t r;\n#pragma unroll\n                for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
+             list("b", "[k]") + ");\n";
+        s += "                CUSTOS_ST(vout + idx, r);\n            }\n        }\n";
+        s += "    }\n}\n";
+        return s;
+    }
+
+    // Entry point for one launch over one set of operands.  `rev` != 0 walks the tiles from
+    // the last to the first (see Tuning::direction).
+    std::string single_entry() const {
+        std::string s;
+        s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
+        s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec, const u64 rev) {\n";
+        s += vec_ptrs;
+        s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
+        s += "    const u64 n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;\n";
+        s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x)\n";
+        s += "        custos_tile(" + tile_args + "vout, (rev ? n_tiles - 1 - tile : tile) * tile_vecs + threadIdx.x, n_vec);\n";
+        // Elements outside the 16-byte aligned body: `head` leading ones and the
+        // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
+        s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
+        s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BLOCK;\n";
+        s += "    if (gid < head) out[gid] = custos_elem(" + list("in", "[gid]") + ");\n";
+        s += "    for (u64 i = head + n_vec * CUSTOS_VEC + gid; i < n; i += n_threads) out[i] = custos_elem(" +
+             list("in", "[i]") + ");\n";
+        s += "}\n";
+        return s;
+    }
+
+    // operand pointers of a merged launch, read from the table row `ptrs`
+    std::string table_operands() const {
+        std::string s;
+        if (k.kind == Kind::Apply) {
+            for (int i = 0; i < n_in; i++)
+                s += "    const S* in" + std::to_string(i) + " = (const S*)ptrs[" + std::to_string(i) + "];\n";
+            s += "    S* out = (S*)ptrs[" + std::to_string(n_in) + "];\n";
+        } else {
+            s += "    const S* in0 = (const S*)ptrs[0];\n    S* out = (S*)ptrs[1];\n    const S* in2 = (const S*)ptrs[2];\n";
+        }
+        return s;
+    }
+
+    // Entry point for many independent launches of equal length in one grid (graph replay of
+    // many small buffers).  `table` holds, per segment, the operand addresses in the order of
+    // the single-launch parameters; every address is 16-byte aligned.  Workgroup b works on
+    // tile b % tiles_per_seg of segment b / tiles_per_seg; the last tile of a segment also
+    // does the tail.
+    std::string batched_entry() const {
+        std::string s;
+        s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
+        s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, const u64 rev) {\n";
+        s += "    const u64 blk = rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
+        s += "    const u64 seg = blk / tiles_per_seg;\n";
+        s += "    const u64 tile = blk - seg * tiles_per_seg;\n";
+        s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs) + ";\n";
+        s += "    const u64 head = 0;\n";
+        s += table_operands();
+        s += vec_ptrs;
+        s += "    custos_tile(" + tile_args + "vout, tile * (u64)CUSTOS_BLOCK * CUSTOS_UNROLL + threadIdx.x, n_vec);\n";
+        s += "    if (tile == tiles_per_seg - 1)\n";
+        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
+             list("in", "[i]") + ");\n";
+        s += "    (void)head;\n}\n";
+        return s;
+    }
+
+    // Entry point for launches of different lengths in one grid.  A table row holds the
+    // operand addresses (16-byte aligned) and the element count of its segment;
+    // `block_map[b]` = segment << 32 | tile tells workgroup b its work.
+    std::string ragged_entry() const {
+        std::string s;
+        s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
+        s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, const u64 rev) {\n";
+        s += "    const u64 where = block_map[rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x];\n";
+        s += "    const u64 seg = where >> 32;\n";
+        s += "    const u64 tile = where & 0xffffffffull;\n";
+        s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + 1) + ";\n";
+        s += "    const u64 n = ptrs[" + std::to_string(n_ptrs) + "];\n";
+        s += "    const u64 n_vec = n / CUSTOS_VEC;\n";
+        s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
+        s += "    const u64 n_tiles = n_vec == 0 ? 1 : (n_vec + tile_vecs - 1) / tile_vecs;\n";
+        s += "    const u64 head = 0;\n";
+        s += table_operands();
+        s += vec_ptrs;
+        s += "    custos_tile(" + tile_args + "vout, tile * tile_vecs + threadIdx.x, n_vec);\n";
+        s += "    if (tile == n_tiles - 1)\n";
+        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
+             list("in", "[i]") + ");\n";
+        s += "    (void)head;\n}\n";
+        return s;
+    }
+};
+
 }  // namespace
 
 bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
@@ -205,7 +394,6 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     std::string body;
     if (!emit_expr_body(k.expr, dtype, &body, err)) return false;
 
-    const int n_in = k.expr.n_vars;
     const bool nt_load = k.tuning.nontemporal & 1, nt_store = k.tuning.nontemporal & 2;
 
     std::string s;
@@ -219,149 +407,12 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     s += prelude(dtype, k.vec_elems);
     s += expr_fn(k, body);
 
-    // Per-element function on storage values: `custos_elem(in0.., [g])`.
-    // Pointers that are read and written (`out`, `lhs_grad`) carry no
-    // __restrict__: the output may be exactly one of the inputs.
-    std::string params, vec_ptrs;
-    if (kind == Kind::Apply) {
-        s += "static __device__ __forceinline__ S custos_elem(";
-        for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "const S s" + std::to_string(i);
-        s += ") {\n    return custos_store(custos_expr(";
-        for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "custos_load(s" + std::to_string(i) + ")";
-        s += "));\n}\n";
-        for (int i = 0; i < n_in; i++) {
-            std::string id = std::to_string(i);
-            params += "const S* in" + id + ", ";
-            vec_ptrs += "    const vec_t* vin" + id + " = (const vec_t*)(in" + id + " + head);\n";
-        }
-        params += "S* out";
-        vec_ptrs += "    vec_t* vout = (vec_t*)(out + head);\n";
-    } else {
-        s += grad_fn(dtype);
-        s += "static __device__ __forceinline__ S custos_elem(const S s0, const S s1, const S s2) {\n"
-             "    return custos_store(custos_grad(custos_load(s1), custos_load(s2), custos_expr(custos_load(s0))));\n}\n";
-        // operand order inside the kernel: 0 = lhs, 1 = lhs_grad (also the output), 2 = out_grad
-        params = "const S* in0, S* out, const S* in2";
-        vec_ptrs = "    const vec_t* vin0 = (const vec_t*)(in0 + head);\n"
-                   "    const vec_t* vin2 = (const vec_t*)(in2 + head);\n"
-                   "    vec_t* vout = (vec_t*)(out + head);\n"
-                   "    const vec_t* vin1 = vout;\n"
-                   "    const S* in1 = out;\n";
-    }
-    const int n_ops = kind == Kind::Apply ? n_in : 3;
-    auto list = [&](const std::string& pre, const std::string& post) {
-        std::string r;
-        for (int i = 0; i < n_ops; i++) r += std::string(i ? ", " : "") + pre + std::to_string(i) + post;
-        return r;
-    };
-
-    // One tile: every lane loads all its vectors, then computes and stores.
-    // `base` is the lane's first vector; a partial last tile takes the masked path.
-    std::string tile_params, tile_args;
-    for (int i = 0; i < n_ops; i++) {
-        if (kind == Kind::UnaryGrad && i == 1) continue;  // vin1 is vout
-        tile_params += "const vec_t* vin" + std::to_string(i) + ", ";
-        tile_args += "vin" + std::to_string(i) + ", ";
-    }
-    s += "static __device__ __forceinline__ void custos_tile(" + tile_params + "vec_t* vout, const u64 base, const u64 n_vec) {\n";
-    if (kind == Kind::UnaryGrad) s += "    const vec_t* vin1 = vout;\n";
-    s += "    if (base + (u64)(CUSTOS_UNROLL - 1) * CUSTOS_BLOCK < n_vec) {\n";
-    for (int i = 0; i < n_ops; i++) s += "        vec_t a" + std::to_string(i) + "[CUSTOS_UNROLL];\n";
-    s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
-    for (int i = 0; i < n_ops; i++) {
-        std::string id = std::to_string(i);
-        s += "            a" + id + "[u] = CUSTOS_LD(vin" + id + " + base + (u64)u * CUSTOS_BLOCK);\n";
-    }
-    s += "        }\n";
-    s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
-    s += "            vec_t r;\n#pragma unroll\n            for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
-         list("a", "[u][k]") + ");\n";
-    s += "            CUSTOS_ST(vout + base + (u64)u * CUSTOS_BLOCK, r);\n        }\n";
-    s += "    } else {\n";
-    s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
-    s += "            const u64 idx = base + (u64)u * CUSTOS_BLOCK;\n";
-    s += "            if (idx < n_vec) {\n";
-    for (int i = 0; i < n_ops; i++) {
-        std::string id = std::to_string(i);
-        s += "                const vec_t b" + id + " = CUSTOS_LD(vin" + id + " + idx);\n";
-    }
-    s += "                vec_t r;\n#pragma unroll\n                for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
-         list("b", "[k]") + ");\n";
-    s += "                CUSTOS_ST(vout + idx, r);\n            }\n        }\n";
-    s += "    }\n}\n";
-
-    // Entry point for one launch over one set of operands.
-    s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-    // `rev` != 0 walks the tiles from the last to the first (see Tuning::direction).
-    s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec, const u64 rev) {\n";
-    s += vec_ptrs;
-    s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
-    s += "    const u64 n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;\n";
-    s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x)\n";
-    s += "        custos_tile(" + tile_args + "vout, (rev ? n_tiles - 1 - tile : tile) * tile_vecs + threadIdx.x, n_vec);\n";
-    // Elements outside the 16-byte aligned body: `head` leading ones and the
-    // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
-    s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
-    s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BLOCK;\n";
-    s += "    if (gid < head) out[gid] = custos_elem(" + list("in", "[gid]") + ");\n";
-    s += "    for (u64 i = head + n_vec * CUSTOS_VEC + gid; i < n; i += n_threads) out[i] = custos_elem(" +
-         list("in", "[i]") + ");\n";
-    s += "}\n";
-
-    // Entry point for many independent launches of equal length in one grid
-    // (graph replay of many small buffers).  `table` holds, per segment, the
-    // operand addresses in the order of the single-launch parameters; every
-    // address is 16-byte aligned.  Workgroup b works on tile b % tiles_per_seg
-    // of segment b / tiles_per_seg; the last tile of a segment also does the tail.
-    const int n_ptrs = kind == Kind::Apply ? n_in + 1 : 3;
-    s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-    s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, const u64 rev) {\n";
-    s += "    const u64 blk = rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
-    s += "    const u64 seg = blk / tiles_per_seg;\n";
-    s += "    const u64 tile = blk - seg * tiles_per_seg;\n";
-    s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs) + ";\n";
-    s += "    const u64 head = 0;\n";
-    if (kind == Kind::Apply) {
-        for (int i = 0; i < n_in; i++)
-            s += "    const S* in" + std::to_string(i) + " = (const S*)ptrs[" + std::to_string(i) + "];\n";
-        s += "    S* out = (S*)ptrs[" + std::to_string(n_in) + "];\n";
-    } else {
-        s += "    const S* in0 = (const S*)ptrs[0];\n    S* out = (S*)ptrs[1];\n    const S* in2 = (const S*)ptrs[2];\n";
-    }
-    s += vec_ptrs;
-    s += "    custos_tile(" + tile_args + "vout, tile * (u64)CUSTOS_BLOCK * CUSTOS_UNROLL + threadIdx.x, n_vec);\n";
-    s += "    if (tile == tiles_per_seg - 1)\n";
-    s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
-         list("in", "[i]") + ");\n";
-    s += "    (void)head;\n}\n";
-
-    // Third entry point: launches of different lengths in one grid.  A table row
-    // holds the operand addresses (16-byte aligned) and the element count of its
-    // segment; `block_map[b]` = segment << 32 | tile tells workgroup b its work.
-    s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-    s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, const u64 rev) {\n";
-    s += "    const u64 where = block_map[rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x];\n";
-    s += "    const u64 seg = where >> 32;\n";
-    s += "    const u64 tile = where & 0xffffffffull;\n";
-    s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + 1) + ";\n";
-    s += "    const u64 n = ptrs[" + std::to_string(n_ptrs) + "];\n";
-    s += "    const u64 n_vec = n / CUSTOS_VEC;\n";
-    s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
-    s += "    const u64 n_tiles = n_vec == 0 ? 1 : (n_vec + tile_vecs - 1) / tile_vecs;\n";
-    s += "    const u64 head = 0;\n";
-    if (kind == Kind::Apply) {
-        for (int i = 0; i < n_in; i++)
-            s += "    const S* in" + std::to_string(i) + " = (const S*)ptrs[" + std::to_string(i) + "];\n";
-        s += "    S* out = (S*)ptrs[" + std::to_string(n_in) + "];\n";
-    } else {
-        s += "    const S* in0 = (const S*)ptrs[0];\n    S* out = (S*)ptrs[1];\n    const S* in2 = (const S*)ptrs[2];\n";
-    }
-    s += vec_ptrs;
-    s += "    custos_tile(" + tile_args + "vout, tile * tile_vecs + threadIdx.x, n_vec);\n";
-    s += "    if (tile == n_tiles - 1)\n";
-    s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
-         list("in", "[i]") + ");\n";
-    s += "    (void)head;\n}\n";
+    const KernelText text(k);
+    s += text.elem_fn();
+    s += text.tile_fn();
+    s += text.single_entry();
+    s += text.batched_entry();
+    s += text.ragged_entry();
 
     k.source = std::move(s);
     *out = std::move(k);
