@@ -215,8 +215,16 @@ class HIP : public Device<HIP<Mods>, Mods> {
             graph_builds_++;
         }
         check(custos_hip_graph_launch(dev_, graph_));
-        check(custos_hip_sync(dev_));
+        if (run_waits_) check(custos_hip_sync(dev_));
     }
+
+    // The reference's run returns after the stream has drained
+    // (src/devices/cuda/lazy.rs:42-43).  A caller that runs the same graph many times
+    // and reads results only at the end can switch the wait off: runs then queue behind
+    // each other on the stream, and `read`, `sync` and every copy to the host still wait
+    // for them.
+    void set_run_waits(bool waits) { run_waits_ = waits; }
+    bool run_waits() const { return run_waits_; }
 
     // how often a run had to (re)record its graph, and the kernels in it
     uint64_t graph_builds() const { return graph_builds_; }
@@ -275,6 +283,7 @@ class HIP : public Device<HIP<Mods>, Mods> {
     custos_hip_graph* graph_ = nullptr;
     uint64_t graph_version_ = 0;
     uint64_t graph_builds_ = 0;
+    bool run_waits_ = true;
 };
 
 }  // namespace custos

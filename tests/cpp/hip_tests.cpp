@@ -44,6 +44,26 @@ TEST_CASE(hip_lazy_run_replays_one_graph) {
     CHECK_VEC_EQ(extra.replace().read(), (std::vector<int32_t>{3, 5, 7, 9, 11, 13}));
 }
 
+// Runs that do not wait queue behind each other on the stream; a read still sees all of
+// them (the reference's run always waits: src/devices/cuda/lazy.rs:42-43)
+TEST_CASE(hip_runs_without_wait_queue_in_order) {
+    using D = HIP<Lazy<Base, int32_t>>;
+    D device;
+    const size_t n = (size_t(1) << 20) + 3;
+    auto acc = device.buffer(std::vector<int32_t>(n, 0));
+    auto one = device.buffer(std::vector<int32_t>(n, 1));
+    auto add = [](auto a, auto b) { return a.add(b); };
+    device.add_op(std::tie(acc, one), [add](Buffer<int32_t, D>& a, Buffer<int32_t, D>& o, D& d) { d.apply_fn2_impl(a, o, a, add); });
+    CHECK(device.run_waits());
+    device.set_run_waits(false);
+    for (int i = 0; i < 25; i++) device.run();
+    CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(n, 25)));
+    device.set_run_waits(true);
+    device.run();
+    CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(n, 26)));
+    CHECK_EQ(device.graph_builds(), uint64_t(1));
+}
+
 // BASELINE configs[1] in miniature, through the whole stack: five apply_fn calls on
 // Graph<Lazy<Base>>, fused into one kernel node, bit-identical to the unfused device result
 TEST_CASE(hip_fused_chain_is_one_kernel) {
