@@ -29,13 +29,28 @@ constexpr unsigned long long kRaggedMaxTiles = 16384;
 // A recorded graph that touches no more than this keeps its data in the memory-side cache.
 constexpr unsigned long long kCacheWorkingSet = 320ull << 20;
 
+// Earlier accesses are kept once per distinct (range, mode) with the highest level seen, so
+// a program that runs over the same buffers many times keeps the search lists as short as
+// a single pass does; the lists hang off the 2 MiB address chunks a range touches.
 void assign_levels(std::vector<RecNode>& nodes) {
     struct Seen {
         uint64_t begin, end;
         bool write;
         int level;
     };
+    struct Key {
+        uint64_t begin, end;
+        bool write;
+        bool operator==(const Key& o) const { return begin == o.begin && end == o.end && write == o.write; }
+    };
+    struct KeyHash {
+        size_t operator()(const Key& k) const {
+            uint64_t h = (k.begin * 0x9e3779b97f4a7c15ull) ^ (k.end + (k.write ? 0x7f4a7c15ull : 0));
+            return static_cast<size_t>(h ^ (h >> 29));
+        }
+    };
     std::vector<Seen> seen;
+    std::unordered_map<Key, uint32_t, KeyHash> known;
     std::unordered_map<uint64_t, std::vector<uint32_t>> buckets;
     int highest = -1;  // highest level so far
     int fence = -1;    // level of the last node with unknown memory use
@@ -63,9 +78,13 @@ void assign_levels(std::vector<RecNode>& nodes) {
         highest = std::max(highest, level);
         for (const Access& a : node.acc) {
             if (a.end <= a.begin) continue;
-            const uint32_t idx = static_cast<uint32_t>(seen.size());
+            auto [slot, fresh] = known.try_emplace(Key{a.begin, a.end, a.write}, static_cast<uint32_t>(seen.size()));
+            if (!fresh) {
+                seen[slot->second].level = std::max(seen[slot->second].level, level);
+                continue;
+            }
             seen.push_back({a.begin, a.end, a.write, level});
-            for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) buckets[c].push_back(idx);
+            for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) buckets[c].push_back(slot->second);
         }
     }
 }
@@ -120,13 +139,12 @@ bool working_set_fits_cache(const std::vector<RecNode>& nodes, int max_level) {
 // The nodes of one dependency level: launches of one kernel are merged (equal lengths into a
 // `_batched` grid, different lengths into a `_ragged` one), everything else stays single.
 // Operand tables and block maps of the merged launches are appended to `host_table`.
-std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNode>& nodes, int level,
-                                bool fits_cache, std::vector<uint64_t>* host_table) {
+std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNode>& nodes,
+                                const std::vector<size_t>& of_level, bool fits_cache, std::vector<uint64_t>* host_table) {
     std::vector<Planned> out;
     // candidates for merging, grouped by kernel in first-seen order
     std::vector<std::pair<custos_hip_kernel*, std::vector<size_t>>> groups;
-    for (size_t i = 0; i < nodes.size(); i++) {
-        if (nodes[i].level != level) continue;
+    for (size_t i : of_level) {
         if (dev->batching && batchable(nodes[i])) {
             auto g = std::find_if(groups.begin(), groups.end(), [&](const auto& kv) { return kv.first == nodes[i].k; });
             if (g == groups.end()) {
@@ -317,7 +335,9 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     const bool fits_cache = working_set_fits_cache(nodes, max_level);
     std::vector<std::vector<Planned>> plan;
     std::vector<uint64_t> host_table;
-    for (int level = 0; level <= max_level; level++) plan.push_back(plan_level(dev, nodes, level, fits_cache, &host_table));
+    std::vector<std::vector<size_t>> by_level(static_cast<size_t>(max_level + 1));
+    for (size_t i = 0; i < nodes.size(); i++) by_level[static_cast<size_t>(nodes[i].level)].push_back(i);
+    for (const auto& of_level : by_level) plan.push_back(plan_level(dev, nodes, of_level, fits_cache, &host_table));
     if (!host_table.empty()) {
         HIP_TRY(dev, hipMalloc(&g->table, host_table.size() * sizeof(uint64_t)));
         HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
