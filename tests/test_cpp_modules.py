@@ -43,9 +43,11 @@ def test_hip_module_stack():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["lazy_and_fusing", "unary_autograd"])
+@pytest.mark.parametrize("name", ["lazy_and_fusing", "unary_autograd", "modules_usage"])
 def test_examples_run(name):
     proc = subprocess.run([_binary(name, EXAMPLES)], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     if name == "lazy_and_fusing":
         assert "1 kernel node(s)" in proc.stdout and "1 graph build(s)" in proc.stdout
+    if name == "modules_usage":
+        assert proc.stdout.count(" ok\n") == 6 and "FAILED" not in proc.stdout
