@@ -1,5 +1,8 @@
 // The module-stack tests on the HIP device (needs an MI355X), plus what only a
 // GPU device has: graph capture/replay behind `run()`.
+#include <atomic>
+#include <thread>
+
 #include "check.hpp"
 #include "custos/custos.hpp"
 #include "module_tests.hpp"
@@ -62,6 +65,44 @@ TEST_CASE(hip_runs_without_wait_queue_in_order) {
     device.run();
     CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(n, 26)));
     CHECK_EQ(device.graph_builds(), uint64_t(1));
+}
+
+// One device per thread (tests/threading/threads.rs:5-25; the reference's devices are not
+// shared between threads either): three threads, each with a device handle of its own on the
+// same GPU, compile, launch, record and read at the same time.
+TEST_CASE(hip_one_device_per_thread) {
+    std::atomic<int> wrong{0};
+    auto eager = [&wrong](int seed) {
+        HIP<Base> device(0);
+        std::vector<float> xs(50000 + 17 * seed);
+        for (size_t i = 0; i < xs.size(); i++) xs[i] = static_cast<float>(i % 1000) * 0.25f + static_cast<float>(seed);
+        auto buf = device.buffer(xs);
+        for (int round = 0; round < 50; round++) {
+            const float k = static_cast<float>(seed * 100 + round);  // a new constant: a new kernel every round
+            auto out = device.apply_fn(buf, [k](auto x) { return x.mul(2.f).add(k); });
+            const std::vector<float> got = out.read();
+            for (size_t i = 0; i < xs.size(); i++) wrong += got[i] != xs[i] * 2.f + k;
+        }
+    };
+    auto lazy = [&wrong]() {
+        HIP<Graph<Lazy<Base>>> device(0);
+        std::vector<float> xs(30011, 1.5f);
+        auto buf = device.buffer(xs);
+        auto a = device.apply_fn(buf, [](auto x) { return x.add(1.f); });
+        auto b = device.apply_fn(a, [](auto x) { return x.mul(3.f); });
+        device.unary_fusing();
+        for (int round = 0; round < 50; round++) {
+            buf.write(std::vector<float>(xs.size(), static_cast<float>(round)));
+            device.run();
+            const std::vector<float> got = b.replace().read();
+            for (float v : got) wrong += v != (static_cast<float>(round) + 1.f) * 3.f;
+        }
+    };
+    std::thread t1(eager, 1), t2(eager, 2), t3(lazy);
+    t1.join();
+    t2.join();
+    t3.join();
+    CHECK_EQ(wrong.load(), 0);
 }
 
 // BASELINE configs[1] in miniature, through the whole stack: five apply_fn calls on

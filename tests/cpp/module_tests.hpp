@@ -923,6 +923,36 @@ void half_per_node_type() {
     CHECK_EQ(wrong, size_t(0));
 }
 
+// ---- Read / WriteBuf / ClearBuf ----
+
+// tests/write.rs:6-87, tests/read.rs:4-13, tests/clear.rs:7-43
+template <template <class> class DEV>
+void write_read_clear() {
+    DEV<Base> device;
+    auto buf = device.template new_buffer<double>(5);
+    buf.write({1., 2., 3., 4., 5.});
+    CHECK_VEC_EQ(buf.read(), (std::vector<double>{1., 2., 3., 4., 5.}));
+    auto dst = device.template new_buffer<int32_t>(4);
+    auto src = device.template buffer<int32_t>({1, 2, -5, 4});
+    device.write_buf(dst, src);
+    CHECK_VEC_EQ(dst.read(), (std::vector<int32_t>{1, 2, -5, 4}));
+    CHECK_VEC_EQ(src.read(), (std::vector<int32_t>{1, 2, -5, 4}));
+    auto shorter = device.template new_buffer<int32_t>(3);
+    CHECK_THROWS_KIND(device.write_buf(shorter, src), DeviceError::ShapeLengthMismatch);
+    auto a = device.template buffer<double>({3., 1., 3., 4.});
+    CHECK_VEC_EQ(a.read(), (std::vector<double>{3., 1., 3., 4.}));
+    auto c = device.template buffer<double>({1., 2., 3., 4., 5., 6.});
+    CHECK_VEC_EQ(c.read(), (std::vector<double>{1., 2., 3., 4., 5., 6.}));
+    c.clear();
+    CHECK_VEC_EQ(c.read(), (std::vector<double>(6, 0.)));
+    // an odd number of narrow elements: the clear stops at the buffer's last byte
+    auto bytes = device.template buffer<uint8_t>(std::vector<uint8_t>(37, 9));
+    auto next = device.template buffer<uint8_t>(std::vector<uint8_t>(37, 7));
+    bytes.clear();
+    CHECK_VEC_EQ(bytes.read(), (std::vector<uint8_t>(37, 0)));
+    CHECK_VEC_EQ(next.read(), (std::vector<uint8_t>(37, 7)));
+}
+
 // ---- CopySlice / CloneBuf ----
 
 // tests/slice_buf.rs:5-84, tests/clone_buf.rs:5-49
@@ -1141,6 +1171,7 @@ void cached_errors() {
     TEST_CASE(autograd_no_grads_pool) { module_tests::autograd_no_grads_pool<DEV>(); }            \
     TEST_CASE(half_f16_per_node) { module_tests::half_per_node_type<DEV, f16_pernode>(); }        \
     TEST_CASE(half_bf16_per_node) { module_tests::half_per_node_type<DEV, bf16_pernode>(); }      \
+    TEST_CASE(write_read_clear) { module_tests::write_read_clear<DEV>(); }                        \
     TEST_CASE(copy_slice_and_clone_buf) { module_tests::copy_slice_and_clone_buf<DEV>(); }        \
     TEST_CASE(cached_same_allocation_every_epoch) { module_tests::cached_same_allocation_every_epoch<DEV>(); } \
     TEST_CASE(cached_multi_level_retrieve) { module_tests::cached_multi_level_retrieve<DEV>(); }  \
