@@ -118,10 +118,15 @@ PROTOTYPES = {
     "custos_hip_source_launch1d": (C.c_int32, [_P, _P, C.c_size_t, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t), C.c_int32]),
     "custos_hip_expr_emit": (C.c_int32, [C.c_int32, C.c_int32, C.c_char_p, _STRS, C.c_int32, C.POINTER(Tuning),
                                          C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint64)]),
+    "custos_hip_expr_emit_shared": (C.c_int32, [C.c_int32, C.c_int32, C.c_char_p, _STRS, C.c_int32, C.POINTER(Tuning),
+                                                C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint64)]),
+    "custos_hip_set_literal_policy": (C.c_int32, [_P, C.c_int32]),
     "custos_hip_expr_build_code_object": (C.c_int32, [C.c_int32, C.c_int32, C.c_char_p, _STRS, C.c_int32,
                                                       C.POINTER(Tuning), C.POINTER(C.c_size_t)]),
     "custos_hip_expr_canonical": (C.c_int32, [C.c_char_p, _STRS, C.c_int32, C.c_char_p, C.c_size_t,
                                               C.POINTER(C.c_size_t)]),
+    "custos_hip_expr_constants": (C.c_int32, [C.c_int32, C.c_char_p, _STRS, C.c_int32, C.c_void_p, C.c_size_t,
+                                              C.POINTER(C.c_size_t), C.POINTER(C.c_int32)]),
     "custos_hip_apply_fn": (C.c_int32, [_P, _P, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_apply_fn2": (C.c_int32, [_P, _P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_apply_fn_n": (C.c_int32, [_P, _P, C.POINTER(C.c_uint64), C.c_int32, C.c_uint64, C.c_size_t]),
@@ -185,16 +190,21 @@ def preferred_shape(footprint_bytes: int, n_operands: int):
     return u.value, nt.value, bool(alt.value)
 
 
-def expr_emit(kind: int, dtype: str, src: str, markers, tuning: Tuning | None = None):
-    """Host-only: generated HIP source and cache key of a kernel."""
+LITERALS_ADAPTIVE, LITERALS_IN_CODE, LITERALS_AS_PARAMETERS = 0, 1, 2
+
+
+def expr_emit(kind: int, dtype: str, src: str, markers, tuning: Tuning | None = None, shared: bool = False):
+    """Host-only: generated HIP source and cache key of a kernel: the one for exactly these
+    literal values, or (`shared`) the form that takes the literals as launch parameters."""
     lib = load_library()
+    emit = lib.custos_hip_expr_emit_shared if shared else lib.custos_hip_expr_emit
     arr, n = c_markers(markers)
     needed = C.c_size_t(0)
     h = C.c_uint64(0)
     t = C.byref(tuning) if tuning is not None else None
-    check(lib.custos_hip_expr_emit(kind, DTYPES[dtype][0], src.encode(), arr, n, t, None, 0, C.byref(needed), C.byref(h)))
+    check(emit(kind, DTYPES[dtype][0], src.encode(), arr, n, t, None, 0, C.byref(needed), C.byref(h)))
     buf = C.create_string_buffer(needed.value)
-    check(lib.custos_hip_expr_emit(kind, DTYPES[dtype][0], src.encode(), arr, n, t, buf, needed.value, None, None))
+    check(emit(kind, DTYPES[dtype][0], src.encode(), arr, n, t, buf, needed.value, None, None))
     return buf.value.decode(), h.value
 
 
@@ -206,6 +216,23 @@ def expr_build_code_object(kind: int, dtype: str, src: str, markers, tuning: Tun
     t = C.byref(tuning) if tuning is not None else None
     check(lib.custos_hip_expr_build_code_object(kind, DTYPES[dtype][0], src.encode(), arr, n, t, C.byref(size)))
     return size.value
+
+
+def expr_constants(dtype: str, src: str, markers):
+    """The literals of `src` that its kernel takes as launch parameters (c0, c1, ...), as a
+    numpy array of the type the expression is computed in."""
+    import numpy as np
+    lib = load_library()
+    arr, n = c_markers(markers)
+    needed, count = C.c_size_t(0), C.c_int32(0)
+    check(lib.custos_hip_expr_constants(DTYPES[dtype][0], src.encode(), arr, n, None, 0, C.byref(needed), C.byref(count)))
+    compute = {"f16": "f32", "bf16": "f32", "f16_pernode": "f32", "bf16_pernode": "f32"}.get(dtype, dtype)
+    np_type = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "i64": np.int64, "u8": np.uint8, "i8": np.int8,
+               "i16": np.int16, "u16": np.uint16, "u32": np.uint32, "u64": np.uint64}[compute]
+    out = np.zeros(count.value, dtype=np_type)
+    if needed.value:
+        check(lib.custos_hip_expr_constants(DTYPES[dtype][0], src.encode(), arr, n, out.ctypes.data, out.nbytes, None, None))
+    return out
 
 
 def expr_canonical(src: str, markers) -> str:

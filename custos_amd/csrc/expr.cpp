@@ -472,10 +472,10 @@ bool parse_expr(const std::string& src, const std::vector<std::string>& markers,
 // printing in the reference's format
 // ---------------------------------------------------------------------------
 
-static void print_node(const Expr& e, int idx, const std::vector<std::string>& markers,
+static void print_node(const Expr& e, int idx, const std::vector<std::string>& markers, const ConstPlan* plan,
                        std::string* out) {
     const Node& n = e.nodes[idx];
-    auto rec = [&](int k) { print_node(e, k, markers, out); };
+    auto rec = [&](int k) { print_node(e, k, markers, plan, out); };
     auto infix = [&](const char* op) {
         *out += "(";
         rec(n.a);
@@ -499,7 +499,10 @@ static void print_node(const Expr& e, int idx, const std::vector<std::string>& m
     };
     switch (n.op) {
         case Op::Var: *out += markers[n.var]; break;
-        case Op::Const: *out += n.lit; break;
+        case Op::Const:
+            if (plan && plan->slot[static_cast<size_t>(idx)] >= 0) *out += "c" + std::to_string(plan->slot[static_cast<size_t>(idx)]);
+            else *out += n.lit;
+            break;
         case Op::Add: infix(" + "); break;
         case Op::Sub: infix(" - "); break;
         case Op::Mul: infix(" * "); break;
@@ -522,24 +525,78 @@ static void print_node(const Expr& e, int idx, const std::vector<std::string>& m
     }
 }
 
-std::string to_cl_source(const Expr& e, const std::vector<std::string>& markers) {
+std::string to_cl_source(const Expr& e, const std::vector<std::string>& markers, const ConstPlan* plan) {
     std::string out;
-    if (e.root >= 0) print_node(e, e.root, markers, &out);
+    if (e.root >= 0) print_node(e, e.root, markers, plan, &out);
     return out;
+}
+
+// ---------------------------------------------------------------------------
+// literals as launch parameters
+// ---------------------------------------------------------------------------
+
+namespace {
+
+// The bytes of a literal in the compute type, as the compiler would materialise `literal_c`.
+void append_literal_bytes(const Literal& l, DType dtype, std::vector<unsigned char>* out) {
+    unsigned char raw[8];
+    size_t n;
+    if (dtype == DType::F64) {
+        uint64_t bits;
+        std::memcpy(&bits, &l.f, 8);
+        if (l.is_nan) bits = 0x7ff8000000000000ull;
+        std::memcpy(raw, &bits, n = 8);
+    } else if (dtype_is_float(dtype)) {
+        const float f = static_cast<float>(l.f);  // exact: already rounded to f32
+        uint32_t bits;
+        std::memcpy(&bits, &f, 4);
+        if (l.is_nan) bits = 0x7fc00000u;
+        std::memcpy(raw, &bits, n = 4);
+    } else {
+        const uint64_t v = dtype_is_signed(dtype) ? static_cast<uint64_t>(l.i) : l.u;
+        std::memcpy(raw, &v, 8);  // little endian: the low bytes are the narrower value
+        n = dtype_size(dtype);
+    }
+    out->insert(out->end(), raw, raw + n);
+}
+
+}  // namespace
+
+bool plan_constants(const Expr& e, DType dtype, bool all_in_code, ConstPlan* plan, ParseError* err) {
+    plan->slot.assign(e.nodes.size(), -1);
+    plan->n_params = 0;
+    plan->bytes.clear();
+    if (all_in_code) return true;
+    std::vector<bool> in_code(e.nodes.size(), false);
+    if (!dtype_is_float(dtype))
+        for (const Node& n : e.nodes)
+            if (n.op == Op::Div && n.b >= 0 && e.nodes[static_cast<size_t>(n.b)].op == Op::Const) in_code[static_cast<size_t>(n.b)] = true;
+    int wanted = 0;
+    for (size_t i = 0; i < e.nodes.size(); i++) wanted += e.nodes[i].op == Op::Const && !in_code[i];
+    if (wanted > kMaxConstParams) return true;
+    for (size_t i = 0; i < e.nodes.size(); i++) {
+        if (e.nodes[i].op != Op::Const || in_code[i]) continue;
+        Literal l;
+        if (!convert_literal(e.nodes[i].lit, dtype, &l, err)) return false;
+        plan->slot[i] = plan->n_params++;
+        append_literal_bytes(l, dtype, &plan->bytes);
+    }
+    return true;
 }
 
 // ---------------------------------------------------------------------------
 // hashing
 // ---------------------------------------------------------------------------
 
-bool hash_expr(const Expr& e, DType dtype, uint64_t* hash, ParseError* err) {
-    uint64_t h = fnv1a64("custos-expr-v1", 14);
+bool hash_expr(const Expr& e, DType dtype, const ConstPlan& plan, uint64_t* hash, ParseError* err) {
+    uint64_t h = fnv1a64("custos-expr-v2", 14);
     int32_t head[3] = {static_cast<int32_t>(dtype), e.n_vars, e.root};
     h = fnv1a64(head, sizeof head, h);
-    for (const Node& n : e.nodes) {
-        int32_t rec[4] = {static_cast<int32_t>(n.op), n.a, n.b, n.var};
+    for (size_t i = 0; i < e.nodes.size(); i++) {
+        const Node& n = e.nodes[i];
+        int32_t rec[5] = {static_cast<int32_t>(n.op), n.a, n.b, n.var, plan.slot[i]};
         h = fnv1a64(rec, sizeof rec, h);
-        if (n.op == Op::Const) {
+        if (n.op == Op::Const && plan.slot[i] < 0) {
             Literal l;
             if (!convert_literal(n.lit, dtype, &l, err)) return false;
             if (dtype_is_float(dtype)) {
@@ -561,7 +618,7 @@ bool hash_expr(const Expr& e, DType dtype, uint64_t* hash, ParseError* err) {
 // HIP C emission
 // ---------------------------------------------------------------------------
 
-bool emit_expr_body(const Expr& e, DType dtype, std::string* out, ParseError* err) {
+bool emit_expr_body(const Expr& e, DType dtype, const ConstPlan& plan, std::string* out, ParseError* err) {
     auto fail = [&](const std::string& m) {
         if (err && err->code == 0) {
             err->code = CUSTOS_HIP_ERR_EXPR_UNSUPPORTED;
@@ -591,6 +648,10 @@ bool emit_expr_body(const Expr& e, DType dtype, std::string* out, ParseError* er
         switch (n.op) {
             case Op::Var: rhs = "v" + std::to_string(n.var); break;
             case Op::Const: {
+                if (plan.slot[i] >= 0) {
+                    rhs = "kc.c[" + std::to_string(plan.slot[i]) + "]";
+                    break;
+                }
                 Literal l;
                 if (!convert_literal(n.lit, dtype, &l, err)) return false;
                 rhs = literal_c(l, dtype);

@@ -94,16 +94,34 @@ struct ParseError {
 bool parse_expr(const std::string& src, const std::vector<std::string>& markers, Expr* out,
                 ParseError* err);
 
-// Re-prints a tree in the reference's ToCLSource format (literals as given).
-std::string to_cl_source(const Expr& e, const std::vector<std::string>& markers);
+// Which literals of an expression are launch parameters.  A closure like `|x| x.mul(lr)`
+// prints a new text for every value of `lr` (src/two_way_ops/resolve.rs:131-141); compiled
+// in, every value would be a kernel of its own.  In the shared form of a kernel a literal
+// is slot `slot[node]` of a block of scalars the kernel takes by value, and kernels that
+// differ only in such values share their code.  Kept in the code even then: divisors of
+// integer divisions (the compiler turns a division by a known value into a multiplication),
+// and every literal of an expression with more than kMaxConstParams of them.  With
+// `all_in_code` no literal is a parameter (the form compiled for one set of values).
+constexpr int kMaxConstParams = 32;
+struct ConstPlan {
+    std::vector<int> slot;             // per node: parameter slot, or -1
+    int n_params = 0;
+    std::vector<unsigned char> bytes;  // the values, n_params elements of the compute type
+};
+bool plan_constants(const Expr& e, DType dtype, bool all_in_code, ConstPlan* plan, ParseError* err);
 
-// Structural 64-bit hash: node kinds, operand wiring and the literal *values*
-// after conversion to the element type ("2", "2.0" and "2.00" hash alike).
-bool hash_expr(const Expr& e, DType dtype, uint64_t* hash, ParseError* err);
+// Re-prints a tree in the reference's ToCLSource format (literals as given; with a plan,
+// parameters print as c0, c1, ...).
+std::string to_cl_source(const Expr& e, const std::vector<std::string>& markers, const ConstPlan* plan = nullptr);
+
+// Structural 64-bit hash: node kinds, operand wiring, which literals are parameters, and
+// the *values* of the literals that stay in the code after conversion to the element type
+// ("2", "2.0" and "2.00" hash alike).
+bool hash_expr(const Expr& e, DType dtype, const ConstPlan& plan, uint64_t* hash, ParseError* err);
 
 // Emits the body of `custos_expr`: SSA statements over v0..v{n-1} of the
-// compute type and a final `return`.
-bool emit_expr_body(const Expr& e, DType dtype, std::string* out, ParseError* err);
+// compute type (parameters read `kc.c[slot]`) and a final `return`.
+bool emit_expr_body(const Expr& e, DType dtype, const ConstPlan& plan, std::string* out, ParseError* err);
 
 uint64_t fnv1a64(const void* data, size_t n, uint64_t seed = 0xcbf29ce484222325ull);
 

@@ -275,7 +275,11 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
             ln.func = reinterpret_cast<void*>(p.kern->fn_batched);
             ln.grid = dim3(static_cast<unsigned int>(blocks));
         }
-        ln.args.push_back(value(&rev, 8));  // every generated entry point ends with the direction
+        // every generated entry point ends with the block of literal parameters (if the
+        // expression has any) and the direction
+        const ConstPlan& consts = p.kern->spec.consts;
+        if (consts.n_params > 0) ln.args.push_back(consts.bytes);
+        ln.args.push_back(value(&rev, 8));
         if (p.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
     }
     *out = std::move(ln);

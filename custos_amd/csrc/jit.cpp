@@ -95,7 +95,7 @@ bool markers_from_c(const char* const* markers, int32_t n, std::vector<std::stri
 
 int32_t spec_from_c(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
                     const char* const* markers, int32_t n_markers, const Tuning& tuning,
-                    KernelSpec* spec) {
+                    bool literals_in_code, KernelSpec* spec) {
     if (!src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");
     if (kind != CUSTOS_HIP_KIND_APPLY && kind != CUSTOS_HIP_KIND_UNARY_GRAD)
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown kernel kind");
@@ -104,7 +104,7 @@ int32_t spec_from_c(custos_hip_device* dev, int32_t kind, int32_t dtype, const c
     if (!markers_from_c(markers, n_markers, &m))
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 4 non-empty markers are required");
     ParseError err;
-    if (!build_kernel_spec(static_cast<Kind>(kind), static_cast<DType>(dtype), src, m, tuning, spec, &err))
+    if (!build_kernel_spec(static_cast<Kind>(kind), static_cast<DType>(dtype), src, m, tuning, literals_in_code, spec, &err))
         return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
     return CUSTOS_HIP_OK;
 }
@@ -178,24 +178,73 @@ int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k) {
     return CUSTOS_HIP_OK;
 }
 
-// Parses, looks the structural key up in the cache, compiles on a miss.
+// The cached kernel that was compiled from the same text as `spec` (apart from the first
+// line, a comment in which literals that stay in the code keep the caller's spelling).
+static custos_hip_kernel* find_code(custos_hip_device* dev, const KernelSpec& spec) {
+    auto bucket = dev->cache.find(spec.hash);
+    if (bucket == dev->cache.end()) return nullptr;
+    for (auto& cached : bucket->second) {
+        const std::string& a = cached->spec.source;
+        const std::string& b = spec.source;
+        if (cached->spec.kind != Kind::Source &&
+            a.compare(a.find('\n'), std::string::npos, b, b.find('\n'), std::string::npos) == 0)
+            return cached.get();
+    }
+    return nullptr;
+}
+
+// Parses, looks the key up in the cache, compiles on a miss.
+//
+// Literal values: the first set of values an expression is seen with is compiled into the
+// code (the compiler folds them: a fused chain that sits at the edge of being ALU-bound
+// runs 4 % faster than with the values in registers).  When the same expression arrives
+// with other values, the form that takes them as launch parameters is compiled once, and
+// every further set of values is a handle on that code (`prefer_shared`: go there at once,
+// for the launch-shape variants of such a handle).  custos_hip_set_literal_policy pins
+// either behaviour.
 static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
                             const char* const* markers, int32_t n_markers, const Tuning& tuning,
-                            custos_hip_kernel** out) {
+                            bool prefer_shared, custos_hip_kernel** out) {
     std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
-    int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, &k->spec);
+    int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, /*literals_in_code=*/true, &k->spec);
     if (rc != CUSTOS_HIP_OK) return rc;
-
-    auto& bucket = dev->cache[k->spec.hash];
-    for (auto& cached : bucket) {
-        // the generated text starts with the caller's spelling of the expression
-        // as a comment; compare what is compiled, i.e. everything after it
-        const std::string& a = cached->spec.source;
-        const std::string& b = k->spec.source;
-        if (a.compare(a.find('\n'), std::string::npos, b, b.find('\n'), std::string::npos) == 0) {
-            dev->hits++;
-            *out = cached.get();
-            return CUSTOS_HIP_OK;
+    if (custos_hip_kernel* known = find_code(dev, k->spec)) {
+        dev->hits++;
+        *out = known;
+        return CUSTOS_HIP_OK;
+    }
+    if (k->spec.n_literals > 0 && dev->literal_policy != CUSTOS_HIP_LITERALS_IN_CODE) {
+        std::unique_ptr<custos_hip_kernel> shared(new custos_hip_kernel);
+        rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, /*literals_in_code=*/false, &shared->spec);
+        if (rc != CUSTOS_HIP_OK) return rc;
+        if (shared->spec.consts.n_params > 0) {
+            custos_hip_kernel* owner = find_code(dev, shared->spec);
+            uint32_t& value_sets = dev->value_sets_seen[shared->spec.hash];
+            const bool first_values = value_sets++ == 0;
+            if (owner || dev->literal_policy == CUSTOS_HIP_LITERALS_AS_PARAMETERS || prefer_shared || !first_values)
+                k = std::move(shared);
+            if (owner) {
+                dev->hits++;
+                if (owner->spec.consts.bytes == k->spec.consts.bytes) {
+                    *out = owner;
+                    return CUSTOS_HIP_OK;
+                }
+                // the same code with other values: a handle of its own that shares the module
+                const std::string values(k->spec.consts.bytes.begin(), k->spec.consts.bytes.end());
+                auto sibling = owner->siblings.find(values);
+                if (sibling == owner->siblings.end()) {
+                    k->spec.source.clear();  // the owner holds the text
+                    k->code = owner;
+                    k->fn = owner->fn;
+                    k->fn_batched = owner->fn_batched;
+                    k->fn_ragged = owner->fn_ragged;
+                    k->expr_src = src;
+                    for (int i = 0; i < n_markers; i++) k->markers.push_back(markers[i]);
+                    sibling = owner->siblings.emplace(values, std::move(k)).first;
+                }
+                *out = sibling->second.get();
+                return CUSTOS_HIP_OK;
+            }
         }
     }
     rc = build_module(dev, k.get());
@@ -211,8 +260,9 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
     }
     k->expr_src = src;
     for (int i = 0; i < n_markers; i++) k->markers.push_back(markers[i]);
+    k->code = k.get();
     *out = k.get();
-    bucket.push_back(std::move(k));
+    dev->cache[k->spec.hash].push_back(std::move(k));
     return CUSTOS_HIP_OK;
 }
 
@@ -220,7 +270,7 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
     custos_hip_kernel*& slot = dtype == DType::U32 ? dev->identity_u32 : dev->identity_u8;
     if (!slot) {
         const char* markers[] = {"x"};
-        int32_t rc = compile_expr(dev, CUSTOS_HIP_KIND_APPLY, static_cast<int32_t>(dtype), "x", markers, 1, dev->tuning, &slot);
+        int32_t rc = compile_expr(dev, CUSTOS_HIP_KIND_APPLY, static_cast<int32_t>(dtype), "x", markers, 1, dev->tuning, false, &slot);
         if (rc != CUSTOS_HIP_OK) return rc;
     }
     *out = slot;
@@ -247,7 +297,8 @@ custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, 
     const std::string keep = dev->last_error;
     custos_hip_kernel* made = nullptr;
     if (compile_expr(dev, static_cast<int32_t>(k->spec.kind), static_cast<int32_t>(k->spec.dtype), k->expr_src.c_str(),
-                     m.data(), static_cast<int32_t>(m.size()), t, &made) != CUSTOS_HIP_OK) {
+                     m.data(), static_cast<int32_t>(m.size()), t, /*prefer_shared=*/k->spec.consts.n_params > 0, &made) !=
+        CUSTOS_HIP_OK) {
         made = nullptr;  // the first kernel serves this size too
         dev->last_error = keep;
     }
@@ -284,7 +335,7 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
         }
     }
     custos_hip_kernel* k = nullptr;
-    int32_t rc = compile_expr(dev, kind, dtype, src, markers, n_markers, dev->tuning, &k);
+    int32_t rc = compile_expr(dev, kind, dtype, src, markers, n_markers, dev->tuning, false, &k);
     if (rc != CUSTOS_HIP_OK) return rc;
     *kernel = k;
     dev->by_text.emplace(std::move(text_key), k);
@@ -320,7 +371,8 @@ int32_t custos_hip_source_compile(custos_hip_device* dev, const char* src, const
 }
 
 const char* custos_hip_kernel_source(const custos_hip_kernel* kernel) {
-    return kernel ? kernel->spec.source.c_str() : "";
+    if (!kernel) return "";
+    return (kernel->code ? kernel->code : kernel)->spec.source.c_str();
 }
 
 const char* custos_hip_kernel_name(const custos_hip_kernel* kernel) {
@@ -362,17 +414,37 @@ int32_t custos_hip_expr_emit(int32_t kind, int32_t dtype, const char* src, const
                              int32_t n_markers, const custos_hip_tuning* tuning, char* buf, size_t cap,
                              size_t* needed, uint64_t* hash) {
     KernelSpec spec;
-    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), &spec);
+    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), true, &spec);
     if (rc != CUSTOS_HIP_OK) return rc;
     if (hash) *hash = spec.hash;
     return copy_out_string(spec.source, buf, cap, needed);
+}
+
+int32_t custos_hip_expr_emit_shared(int32_t kind, int32_t dtype, const char* src, const char* const* markers,
+                                    int32_t n_markers, const custos_hip_tuning* tuning, char* buf, size_t cap,
+                                    size_t* needed, uint64_t* hash) {
+    KernelSpec spec;
+    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), false, &spec);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    if (hash) *hash = spec.hash;
+    return copy_out_string(spec.source, buf, cap, needed);
+}
+
+int32_t custos_hip_set_literal_policy(custos_hip_device* dev, int32_t policy) {
+    REQUIRE_DEV(dev);
+    if (policy != CUSTOS_HIP_LITERALS_ADAPTIVE && policy != CUSTOS_HIP_LITERALS_IN_CODE &&
+        policy != CUSTOS_HIP_LITERALS_AS_PARAMETERS)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown literal policy");
+    dev->literal_policy = policy;
+    dev->by_text.clear();  // the same text may now map to another kernel
+    return CUSTOS_HIP_OK;
 }
 
 int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const char* src,
                                           const char* const* markers, int32_t n_markers,
                                           const custos_hip_tuning* tuning, size_t* code_size) {
     KernelSpec spec;
-    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), &spec);
+    int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), true, &spec);
     if (rc != CUSTOS_HIP_OK) return rc;
     std::vector<char> code;
     rc = compile_to_code_object(nullptr, spec, "gfx950", &code);
@@ -401,6 +473,24 @@ int32_t custos_hip_expr_canonical(const char* src, const char* const* markers, i
     ParseError err;
     if (!parse_expr(src, m, &e, &err)) return set_error(nullptr, err.code, err.message);
     return copy_out_string(to_cl_source(e, m), buf, cap, needed);
+}
+
+int32_t custos_hip_expr_constants(int32_t dtype, const char* src, const char* const* markers, int32_t n_markers,
+                                  void* buf, size_t cap, size_t* needed, int32_t* n_params) {
+    if (!src) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");
+    if (!dtype_valid(dtype)) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown element type");
+    std::vector<std::string> m;
+    if (!markers_from_c(markers, n_markers, &m))
+        return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 4 non-empty markers are required");
+    Expr e;
+    ParseError err;
+    ConstPlan plan;
+    if (!parse_expr(src, m, &e, &err) || !plan_constants(e, static_cast<DType>(dtype), false, &plan, &err))
+        return set_error(nullptr, err.code, err.message);
+    if (needed) *needed = plan.bytes.size();
+    if (n_params) *n_params = plan.n_params;
+    if (buf && cap >= plan.bytes.size() && !plan.bytes.empty()) std::memcpy(buf, plan.bytes.data(), plan.bytes.size());
+    return CUSTOS_HIP_OK;
 }
 
 }  // extern "C"

@@ -80,12 +80,23 @@ namespace {
 
 // Conversions between the storage and the compute type, and the math wrappers
 // the emitted expression calls.
-std::string prelude(DType dtype, int vec) {
+std::string prelude(DType dtype, int vec, int n_consts) {
     std::string s;
     s += "typedef unsigned long long u64;\n";
     s += std::string("typedef ") + dtype_storage_c(dtype) + " S;\n";
     s += std::string("typedef ") + dtype_compute_c(dtype) + " C;\n";
     s += "typedef S vec_t __attribute__((ext_vector_type(" + std::to_string(vec) + ")));\n";
+    // The literals of the expression that are launch parameters: one block of scalars, an
+    // argument by value of every entry point (it sits in the kernel argument segment, every
+    // read of it is a scalar load).  KC_PARAM / KC_ARG thread it through the helper functions.
+    if (n_consts > 0) {
+        s += "struct CustosConsts { C c[" + std::to_string(n_consts) + "]; };\n";
+        s += "#define CUSTOS_KC_ENTRY const CustosConsts kc,\n";
+        s += "#define CUSTOS_KC_PARAM , const CustosConsts& kc\n";
+        s += "#define CUSTOS_KC_ARG , kc\n";
+    } else {
+        s += "#define CUSTOS_KC_ENTRY\n#define CUSTOS_KC_PARAM\n#define CUSTOS_KC_ARG\n";
+    }
     if (dtype == DType::BF16 || dtype == DType::BF16_PERNODE) {
         s += R"(static __device__ __forceinline__ C custos_load(S s) {
     return __builtin_bit_cast(float, (unsigned int)s << 16);
@@ -144,7 +155,7 @@ std::string expr_fn(const KernelSpec& k, const std::string& body) {
         if (i) s += ", ";
         s += "const C v" + std::to_string(i);
     }
-    s += ") {\n" + body + "}\n";
+    s += " CUSTOS_KC_PARAM) {\n" + body + "}\n";
     return s;
 }
 
@@ -215,13 +226,13 @@ struct KernelText {
         if (k.kind == Kind::Apply) {
             s += "static __device__ __forceinline__ S custos_elem(";
             for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "const S s" + std::to_string(i);
-            s += ") {\n    return custos_store(custos_expr(";
+            s += " CUSTOS_KC_PARAM) {\n    return custos_store(custos_expr(";
             for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "custos_load(s" + std::to_string(i) + ")";
-            s += "));\n}\n";
+            s += " CUSTOS_KC_ARG));\n}\n";
         } else {
             s += grad_fn(k.dtype);
-            s += "static __device__ __forceinline__ S custos_elem(const S s0, const S s1, const S s2) {\n"
-                 "    return custos_store(custos_grad(custos_load(s1), custos_load(s2), custos_expr(custos_load(s0))));\n}\n";
+            s += "static __device__ __forceinline__ S custos_elem(const S s0, const S s1, const S s2 CUSTOS_KC_PARAM) {\n"
+                 "    return custos_store(custos_grad(custos_load(s1), custos_load(s2), custos_expr(custos_load(s0) CUSTOS_KC_ARG)));\n}\n";
         }
         return s;
     }
@@ -237,7 +248,7 @@ struct KernelText {
             tile_params += "const vec_t* vin" + std::to_string(i) + ", ";
         }
         std::string s;
-        s += "static __device__ __forceinline__ void custos_tile(" + tile_params + "vec_t* vout, const u64 base, const u64 n_vec) {\n";
+        s += "static __device__ __forceinline__ void custos_tile(" + tile_params + "vec_t* vout, const u64 base, const u64 n_vec CUSTOS_KC_PARAM) {\n";
         if (k.kind == Kind::UnaryGrad) s += "    const vec_t* vin1 = vout;\n";
         s += "    if (base + (u64)(CUSTOS_UNROLL - 1) * CUSTOS_BLOCK < n_vec) {\n";
         for (int i = 0; i < n_ops; i++) s += "        vec_t a" + std::to_string(i) + "[CUSTOS_UNROLL];\n";
@@ -249,7 +260,7 @@ struct KernelText {
         s += "        }\n";
         s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
         s += "            vec_t r;\n#pragma unroll\n            for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
-             list("a", "[u][k]") + ");\n";
+             list("a", "[u][k]") + " CUSTOS_KC_ARG);\n";
         s += "            CUSTOS_ST(vout + base + (u64)u * CUSTOS_BLOCK, r);\n        }\n";
         s += "    } else {\n";
         s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
@@ -260,7 +271,7 @@ struct KernelText {
             s += "                const vec_t b" + id + " = CUSTOS_LD(vin" + id + " + idx);\n";
         }
         s += "                vec_t r;\n#pragma unroll\n                for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
-             list("b", "[k]") + ");\n";
+             list("b", "[k]") + " CUSTOS_KC_ARG);\n";
         s += "                CUSTOS_ST(vout + idx, r);\n            }\n        }\n";
         s += "    }\n}\n";
         return s;
@@ -271,19 +282,19 @@ struct KernelText {
     std::string single_entry() const {
         std::string s;
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-        s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec, const u64 rev) {\n";
+        s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec, CUSTOS_KC_ENTRY const u64 rev) {\n";
         s += vec_ptrs;
         s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
         s += "    const u64 n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;\n";
         s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x)\n";
-        s += "        custos_tile(" + tile_args + "vout, (rev ? n_tiles - 1 - tile : tile) * tile_vecs + threadIdx.x, n_vec);\n";
+        s += "        custos_tile(" + tile_args + "vout, (rev ? n_tiles - 1 - tile : tile) * tile_vecs + threadIdx.x, n_vec CUSTOS_KC_ARG);\n";
         // Elements outside the 16-byte aligned body: `head` leading ones and the
         // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
         s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
         s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BLOCK;\n";
-        s += "    if (gid < head) out[gid] = custos_elem(" + list("in", "[gid]") + ");\n";
+        s += "    if (gid < head) out[gid] = custos_elem(" + list("in", "[gid]") + " CUSTOS_KC_ARG);\n";
         s += "    for (u64 i = head + n_vec * CUSTOS_VEC + gid; i < n; i += n_threads) out[i] = custos_elem(" +
-             list("in", "[i]") + ");\n";
+             list("in", "[i]") + " CUSTOS_KC_ARG);\n";
         s += "}\n";
         return s;
     }
@@ -309,7 +320,7 @@ struct KernelText {
     std::string batched_entry() const {
         std::string s;
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-        s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, const u64 rev) {\n";
+        s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, CUSTOS_KC_ENTRY const u64 rev) {\n";
         s += "    const u64 blk = rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
         s += "    const u64 seg = blk / tiles_per_seg;\n";
         s += "    const u64 tile = blk - seg * tiles_per_seg;\n";
@@ -317,10 +328,10 @@ struct KernelText {
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
-        s += "    custos_tile(" + tile_args + "vout, tile * (u64)CUSTOS_BLOCK * CUSTOS_UNROLL + threadIdx.x, n_vec);\n";
+        s += "    custos_tile(" + tile_args + "vout, tile * (u64)CUSTOS_BLOCK * CUSTOS_UNROLL + threadIdx.x, n_vec CUSTOS_KC_ARG);\n";
         s += "    if (tile == tiles_per_seg - 1)\n";
         s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
-             list("in", "[i]") + ");\n";
+             list("in", "[i]") + " CUSTOS_KC_ARG);\n";
         s += "    (void)head;\n}\n";
         return s;
     }
@@ -331,7 +342,7 @@ struct KernelText {
     std::string ragged_entry() const {
         std::string s;
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-        s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, const u64 rev) {\n";
+        s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, CUSTOS_KC_ENTRY const u64 rev) {\n";
         s += "    const u64 where = block_map[rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x];\n";
         s += "    const u64 seg = where >> 32;\n";
         s += "    const u64 tile = where & 0xffffffffull;\n";
@@ -343,10 +354,10 @@ struct KernelText {
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
-        s += "    custos_tile(" + tile_args + "vout, tile * tile_vecs + threadIdx.x, n_vec);\n";
+        s += "    custos_tile(" + tile_args + "vout, tile * tile_vecs + threadIdx.x, n_vec CUSTOS_KC_ARG);\n";
         s += "    if (tile == n_tiles - 1)\n";
         s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
-             list("in", "[i]") + ");\n";
+             list("in", "[i]") + " CUSTOS_KC_ARG);\n";
         s += "    (void)head;\n}\n";
         return s;
     }
@@ -356,7 +367,7 @@ struct KernelText {
 
 bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
                        const std::vector<std::string>& markers, const Tuning& tuning,
-                       KernelSpec* out, ParseError* err) {
+                       bool literals_in_code, KernelSpec* out, ParseError* err) {
     KernelSpec k;
     k.kind = kind;
     k.dtype = dtype;
@@ -374,11 +385,13 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     if (k.auto_unroll) k.tuning.unroll = small.unroll;
     k.auto_nt = tuning.nontemporal < 0;
     if (k.auto_nt) k.tuning.nontemporal = small.nontemporal;
+    if (!plan_constants(k.expr, dtype, literals_in_code, &k.consts, err)) return false;
+    for (const Node& n : k.expr.nodes) k.n_literals += n.op == Op::Const;
     uint64_t h;
-    if (!hash_expr(k.expr, dtype, &h, err)) return false;
+    if (!hash_expr(k.expr, dtype, k.consts, &h, err)) return false;
     // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
     int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 6 /* template version */};
+                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 7 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -392,19 +405,19 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     }
 
     std::string body;
-    if (!emit_expr_body(k.expr, dtype, &body, err)) return false;
+    if (!emit_expr_body(k.expr, dtype, k.consts, &body, err)) return false;
 
     const bool nt_load = k.tuning.nontemporal & 1, nt_store = k.tuning.nontemporal & 2;
 
     std::string s;
-    s += "// generated by custos-hip: " + to_cl_source(k.expr, markers) + "\n";
+    s += "// generated by custos-hip: " + to_cl_source(k.expr, markers, &k.consts) + "\n";
     s += "#define CUSTOS_BLOCK " + std::to_string(k.tuning.block_threads) + "\n";
     s += "#define CUSTOS_UNROLL " + std::to_string(k.tuning.unroll) + "\n";
     s += "#define CUSTOS_VEC " + std::to_string(k.vec_elems) + "\n";
     s += nt_load ? "#define CUSTOS_LD(p) __builtin_nontemporal_load(p)\n" : "#define CUSTOS_LD(p) (*(p))\n";
     s += nt_store ? "#define CUSTOS_ST(p, v) __builtin_nontemporal_store(v, p)\n"
                   : "#define CUSTOS_ST(p, v) (*(p) = (v))\n";
-    s += prelude(dtype, k.vec_elems);
+    s += prelude(dtype, k.vec_elems, k.consts.n_params);
     s += expr_fn(k, body);
 
     const KernelText text(k);

@@ -51,7 +51,9 @@ struct KernelSpec {
     Tuning tuning;             // as compiled (unroll resolved)
     bool auto_unroll = false;  // the caller left the unroll factor / the cache policy open:
     bool auto_nt = false;      // launches may use a variant compiled with another choice
-    uint64_t hash = 0;   // cache key: expression, dtype, kind, tuning
+    ConstPlan consts;          // literals that are launch parameters, and this text's values for them
+    int n_literals = 0;        // literals in the expression, parameters or not
+    uint64_t hash = 0;   // cache key: expression without the parameter values, dtype, kind, tuning
     std::string name;    // entry point: custos_<kind>_<dtype>_<hash>, unique per kernel so
                          // that profiler output tells the kernels apart
     std::string source;  // complete translation unit
@@ -59,9 +61,12 @@ struct KernelSpec {
 };
 
 // Parses, hashes and emits. On failure returns false and fills `err`.
+// `literals_in_code`: the kernel for exactly these literal values (the compiler sees them);
+// else the form shared by all expressions that differ only in literal values, which takes
+// them as launch parameters (ConstPlan).
 bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
                        const std::vector<std::string>& markers, const Tuning& tuning,
-                       KernelSpec* out, ParseError* err);
+                       bool literals_in_code, KernelSpec* out, ParseError* err);
 
 // Options handed to hiprtc for every kernel.
 std::vector<std::string> hiprtc_options(const std::string& arch);

@@ -95,6 +95,8 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     args.push_back(&count);
     args.push_back(&head);
     args.push_back(&n_vec);
+    // the expression's literals that are launch parameters: one block by value
+    if (k->spec.consts.n_params > 0) args.push_back(k->spec.consts.bytes.data());
     args.push_back(&rev);
     HIP_TRY(dev, hipModuleLaunchKernel(k->fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
                                        1, 1, 0, dev->stream, args.data(), nullptr));

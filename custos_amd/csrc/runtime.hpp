@@ -7,6 +7,7 @@
 #include <hip/hiprtc.h>
 
 #include <cstdint>
+#include <map>
 #include <memory>
 #include <string>
 #include <unordered_map>
@@ -28,6 +29,12 @@ struct custos_hip_kernel {
     // same expression compiled with another (unroll, cache policy); owned by the cache.
     // key = unroll * 8 + nontemporal; a null entry is a variant that failed to compile
     std::vector<std::pair<int, custos_hip_kernel*>> variants;
+    // Handles for the same code with other values of the literal parameters, by those
+    // values: they share this kernel's module (their own `module` stays null) and differ
+    // in `spec.consts.bytes`, `spec.expr` and `expr_src`.  `code` points at the kernel that
+    // owns the module (itself for the owner).
+    std::map<std::string, std::unique_ptr<custos_hip_kernel>> siblings;
+    custos_hip_kernel* code = nullptr;
 };
 
 // A graph node in launchable form: function, shape and a copy of the argument values.
@@ -85,6 +92,9 @@ struct custos_hip_device {
     std::string arch;
     custos_hip::Tuning tuning;
     bool capturing = false;          // recording: launches, clears and copies go to `recorded`
+    int32_t literal_policy = 0;      // CUSTOS_HIP_LITERALS_*
+    // per shared-form key: how many distinct texts of that structure were compiled or looked up
+    std::unordered_map<uint64_t, uint32_t> value_sets_seen;
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     // allocation pool: freed blocks by rounded size; every block this handle allocated, by address
     std::unordered_map<size_t, std::vector<void*>> pool;

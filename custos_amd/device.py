@@ -307,6 +307,10 @@ class HIP:
     def set_graph_batching(self, enabled: bool) -> None:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 
+    def set_literal_policy(self, policy: int) -> None:
+        """How literal values reach kernels: capi.LITERALS_ADAPTIVE (default), _IN_CODE, _AS_PARAMETERS."""
+        self._check(self.lib.custos_hip_set_literal_policy(self.handle, policy))
+
     def set_graph_direct_replay(self, max_nodes: int) -> None:
         self._check(self.lib.custos_hip_set_graph_direct_replay(self.handle, max_nodes))
 

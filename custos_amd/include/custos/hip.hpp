@@ -237,6 +237,15 @@ class HIP : public Device<HIP<Mods>, Mods> {
     // Launch shape of the generated kernels; zero fields are left to the library, which
     // chooses them per launch from the bytes it touches.
     void set_tuning(const custos_hip_tuning& tuning) { check(custos_hip_set_tuning(dev_, &tuning)); }
+    // How literal values reach kernels (CUSTOS_HIP_LITERALS_*): by default the first set of values of an
+    // expression is compiled in, later sets are launch parameters of one shared kernel.
+    void set_literal_policy(int32_t policy) { check(custos_hip_set_literal_policy(dev_, policy)); }
+    // (hiprtc compilations, cache hits) so far
+    std::pair<uint64_t, uint64_t> cache_stats() const {
+        uint64_t compiles = 0, hits = 0;
+        custos_hip_cache_stats(dev_, &compiles, &hits);
+        return {compiles, hits};
+    }
     // Longest recorded chain that is replayed as plain launches instead of a graph launch.
     void set_graph_direct_replay(int32_t max_nodes) { check(custos_hip_set_graph_direct_replay(dev_, max_nodes)); }
 

@@ -194,7 +194,19 @@ int32_t custos_hip_clear(custos_hip_device *dev, uint64_t dptr, size_t bytes);
  * + - * / compare min max abs neg are bit-identical to the CPU device.
  * Kernels are cached per device by (expression structure, dtype, kind,
  * tuning): the same expression is compiled once.
- * The kernel handle stays valid until the device is destroyed.
+ * Literal values need not cost a compilation each: a closure such as
+ * `|x| x.mul(lr)` prints a new text for every value of `lr`
+ * (src/two_way_ops/resolve.rs:131-141), and the reference compiles every distinct
+ * text (src/devices/cuda/kernel_cache.rs:45-61).  Here the first set of values an
+ * expression is seen with is compiled into the code; when the same expression
+ * arrives with other values, a form that takes the literals as launch parameters
+ * ("(x * c0)") is compiled once, and every further set of values is a handle on that
+ * code carrying its own values.  Literals that always stay in the code: the divisor
+ * of an integer division, and every literal of an expression with more than 32 of
+ * them.  Results do not depend on which way a literal travels
+ * (custos_hip_set_literal_policy pins one).
+ * The kernel handle stays valid until the device is destroyed; a handle per distinct
+ * set of values is kept (about 1 KiB each).
  */
 int32_t custos_hip_expr_compile(custos_hip_device *dev, int32_t kind, int32_t dtype,
                                 const char *src, const char *const *markers, int32_t n_markers,
@@ -211,6 +223,11 @@ int32_t custos_hip_kernel_arity(const custos_hip_kernel *kernel);
  * profiler shows.  Only knobs that custos_hip_set_tuning left at 0 vary. */
 int32_t custos_hip_kernel_launched_as(custos_hip_device *dev, custos_hip_kernel *kernel, size_t n,
                                       custos_hip_kernel **variant);
+/* How literal values reach a kernel (see custos_hip_expr_compile). */
+#define CUSTOS_HIP_LITERALS_ADAPTIVE 0      /* in the code for the first set of values, parameters after */
+#define CUSTOS_HIP_LITERALS_IN_CODE 1       /* every distinct set of values is compiled (the reference's way) */
+#define CUSTOS_HIP_LITERALS_AS_PARAMETERS 2 /* always the shared form */
+int32_t custos_hip_set_literal_policy(custos_hip_device *dev, int32_t policy);
 /* Number of hiprtc compilations / cache hits since the device was created. */
 int32_t custos_hip_cache_stats(custos_hip_device *dev, uint64_t *compiles, uint64_t *hits);
 
@@ -248,18 +265,31 @@ int32_t custos_hip_expr_emit(int32_t kind, int32_t dtype, const char *src,
                              const char *const *markers, int32_t n_markers,
                              const custos_hip_tuning *tuning, char *buf, size_t cap,
                              size_t *needed, uint64_t *hash);
+/* The same for the form shared by all expressions that differ from `src` only in literal
+ * values (literals as launch parameters, see custos_hip_expr_constants). */
+int32_t custos_hip_expr_emit_shared(int32_t kind, int32_t dtype, const char *src,
+                                    const char *const *markers, int32_t n_markers,
+                                    const custos_hip_tuning *tuning, char *buf, size_t cap,
+                                    size_t *needed, uint64_t *hash);
 int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const char *src,
                                           const char *const *markers, int32_t n_markers,
                                           const custos_hip_tuning *tuning, size_t *code_size);
-/* Canonical re-print of an expression in the reference's ToCLSource format. */
 /* Host-only: the launch shape the library picks for a launch that touches `footprint_bytes`
  * (all operands together) through `n_operands` pointers, for the knobs left at 0 in
  * custos_hip_tuning: vectors per thread, the `nontemporal` bits, and whether the launch
  * walks its tiles against the direction of the previous one. */
 int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t *unroll,
                                    int32_t *nontemporal, int32_t *alternate);
+/* Canonical re-print of an expression in the reference's ToCLSource format. */
 int32_t custos_hip_expr_canonical(const char *src, const char *const *markers, int32_t n_markers,
                                   char *buf, size_t cap, size_t *needed);
+/* Host-only: the values of the literals of `src` that the shared form of its kernel takes
+ * as launch parameters, in the order c0, c1, ... of the generated text, each in the type the
+ * expression is computed in (f32 for the 16-bit float types, else the element type).
+ * `*n_params` = how many, `*needed` = their bytes; copied to `buf` if `cap` suffices. */
+int32_t custos_hip_expr_constants(int32_t dtype, const char *src, const char *const *markers,
+                                  int32_t n_markers, void *buf, size_t cap, size_t *needed,
+                                  int32_t *n_params);
 
 /* ---- launches ---- */
 

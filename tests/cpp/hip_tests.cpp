@@ -105,6 +105,48 @@ TEST_CASE(hip_one_device_per_thread) {
     CHECK_EQ(wrong.load(), 0);
 }
 
+// A closure that captures a scalar prints a new text for every value
+// (src/two_way_ops/resolve.rs:131-141); the reference compiles each text
+// (src/devices/cuda/kernel_cache.rs:45-61).  Here: one compilation for the first value,
+// one for the form that takes the value as a launch parameter, none after that --
+// eager, recorded into graphs, and merged into one grid.
+TEST_CASE(hip_captured_scalars_share_one_kernel) {
+    HIP<Base> device;
+    std::vector<float> xs(4099);
+    for (size_t i = 0; i < xs.size(); i++) xs[i] = static_cast<float>(i) * 0.125f - 200.f;
+    auto x = device.buffer(xs);
+    const uint64_t before = device.cache_stats().first;
+    for (int step = 0; step < 30; step++) {
+        const float lr = 0.01f * static_cast<float>(step + 1), eps = 1.f / static_cast<float>(step + 3);
+        auto out = device.apply_fn(x, [lr, eps](auto v) { return v.mul(lr).add(eps).abs().min(lr); });
+        const std::vector<float> got = out.read();
+        for (size_t i = 0; i < xs.size(); i++) {
+            const float t = std::fabs(xs[i] * lr + eps);
+            CHECK_EQ(got[i], t < lr ? t : lr);
+        }
+    }
+    CHECK_EQ(device.cache_stats().first - before, uint64_t(2));
+
+    // recorded: 64 buffers, each scaled by its own factor, replayed as a graph
+    using D = HIP<Lazy<Base>>;
+    D lazy;
+    std::vector<Buffer<float, D>> ins, outs;
+    for (int b = 0; b < 64; b++) ins.push_back(lazy.buffer(std::vector<float>(1000 + 8 * b, static_cast<float>(b))));
+    for (int b = 0; b < 64; b++) {
+        const float k = 0.5f + static_cast<float>(b % 4);   // four distinct factors
+        outs.push_back(lazy.apply_fn(ins[static_cast<size_t>(b)], [k](auto v) { return v.mul(k).sub(1.f); }));
+    }
+    const uint64_t compiled_before = lazy.cache_stats().first;
+    lazy.run();
+    CHECK(lazy.cache_stats().first - compiled_before <= uint64_t(2));
+    // launches with the same factor share a handle and are merged: four ragged grids
+    CHECK_EQ(lazy.graph_kernel_nodes(), size_t(4));
+    for (int b = 0; b < 64; b++) {
+        const float k = 0.5f + static_cast<float>(b % 4);
+        CHECK_VEC_EQ(outs[static_cast<size_t>(b)].replace().read(), (std::vector<float>(1000 + 8 * b, static_cast<float>(b) * k - 1.f)));
+    }
+}
+
 // BASELINE configs[1] in miniature, through the whole stack: five apply_fn calls on
 // Graph<Lazy<Base>>, fused into one kernel node, bit-identical to the unfused device result
 TEST_CASE(hip_fused_chain_is_one_kernel) {

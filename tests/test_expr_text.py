@@ -3,6 +3,8 @@ reference asserts for `to_cl_source`, and the library's parser must accept
 them, re-print them unchanged and emit typed HIP C for them.  CPU only."""
 import re
 
+import numpy as np
+
 import pytest
 
 from custos_amd import Const, Resolve, capi, to_marker, to_val
@@ -100,6 +102,7 @@ def test_emit_types_literals_and_no_contraction():
     assert not re.search(r"[^x0-9a-f.p+]2\.0[^f]", src.split("\n", 1)[1])
     assert "fma" not in src.lower()
     assert "const float t2 = (float)(t0 * t1);" in src     # one statement per node
+    assert "CustosConsts" not in src
     src64, _ = capi.expr_emit(capi.KIND_APPLY, "f64", "((x * 2.0) + 1.0)", ["x"])
     assert "typedef double S;" in src64 and "0x1p+1;" in src64
     srci, _ = capi.expr_emit(capi.KIND_APPLY, "i32", "((x >= 0) * x)", ["x"])
@@ -107,6 +110,48 @@ def test_emit_types_literals_and_no_contraction():
     srch, _ = capi.expr_emit(capi.KIND_APPLY, "f16", "(exp((x * 0.5)) * x)", ["x"])
     assert "typedef _Float16 S;" in srch and "typedef float C;" in srch
     assert "ext_vector_type(8)" in srch                     # 16-byte vectors of halves
+
+
+def test_shared_form_takes_literals_as_launch_parameters():
+    """The form compiled once an expression has been seen with a second set of literal values."""
+    src, _ = capi.expr_emit(capi.KIND_APPLY, "f32", "((x * 2.0) + 1.0)", ["x"], shared=True)
+    assert "struct CustosConsts { C c[2]; };" in src and "const float t1 = kc.c[0];" in src
+    assert "0x1p+1f" not in src
+    assert src.startswith("// generated by custos-hip: ((x * c0) + c1)\n")
+    assert "CUSTOS_KC_ENTRY const u64 rev)" in src          # the block is an argument by value of every entry point
+    consts = capi.expr_constants("f32", "((x * 2.0) + 1.0)", ["x"])
+    assert consts.dtype == np.float32 and consts.tolist() == [2.0, 1.0]
+    src64, _ = capi.expr_emit(capi.KIND_APPLY, "f64", "((x * 2.0) + 1.0)", ["x"], shared=True)
+    assert "const double t1 = kc.c[0];" in src64
+    assert capi.expr_constants("f64", "((x * 0.1) + 1.0)", ["x"]).tolist() == [0.1, 1.0]
+    assert capi.expr_constants("f16", "(exp((x * 0.5)) * x)", ["x"]).dtype == np.float32   # the compute type
+    assert capi.expr_constants("i8", "(x + -3)", ["x"]).tolist() == [-3]
+    nan_inf = capi.expr_constants("f32", "min(max(x, -inf), NaN)", ["x"])
+    assert nan_inf[0] == -np.inf and np.isnan(nan_inf[1])
+    # no literal: no parameter block, and the shared form is the only form
+    plain, h = capi.expr_emit(capi.KIND_APPLY, "f32", "sin(x)", ["x"], shared=True)
+    assert "CustosConsts" not in plain and len(capi.expr_constants("f32", "sin(x)", ["x"])) == 0
+    assert (plain, h) == capi.expr_emit(capi.KIND_APPLY, "f32", "sin(x)", ["x"])
+    # the divisor of an integer division stays in the code: the compiler turns it into a multiplication
+    src, h3 = capi.expr_emit(capi.KIND_APPLY, "i32", "((x / 3) + 2)", ["x"], shared=True)
+    assert "((int)3LL)" in src and "struct CustosConsts { C c[1]; };" in src
+    assert capi.expr_constants("i32", "((x / 3) + 2)", ["x"]).tolist() == [2]
+    assert capi.expr_emit(capi.KIND_APPLY, "i32", "((x / 4) + 2)", ["x"], shared=True)[1] != h3
+    assert capi.expr_emit(capi.KIND_APPLY, "i32", "((x / 3) + 7)", ["x"], shared=True)[1] == h3
+    # a float division by a literal is a parameter like any other
+    assert "kc.c[0]" in capi.expr_emit(capi.KIND_APPLY, "f32", "(x / 3.0)", ["x"], shared=True)[0]
+    # more than 32 literals: all of them stay
+    many = "x"
+    for i in range(33):
+        many = f"({many} + {i + 1}.0)"
+    src, _ = capi.expr_emit(capi.KIND_APPLY, "f32", many, ["x"], shared=True)
+    assert "CustosConsts" not in src and "0x1p+1f" in src
+    assert len(capi.expr_constants("f32", many, ["x"])) == 0
+    # every element type compiles in the shared form
+    for dtype in capi.DTYPES:
+        text = "((x * 3) + 1)" if dtype[0] in "iu" else "(exp((x * 0.5)) + 1.5)"
+        for kind in (capi.KIND_APPLY, capi.KIND_UNARY_GRAD):
+            assert "kc.c[1]" in capi.expr_emit(kind, dtype, text, ["x"], shared=True)[0]
 
 
 def test_min_max_emitted_as_selects():
@@ -125,6 +170,20 @@ def test_hash_ignores_literal_spelling_but_not_value_or_type():
     # f32 rounding of the literal decides, not the text
     assert h("(x * 0.1)") == h("(x * 0.100000001)")
     assert h("(x * 0.1)", "f64") != h("(x * 0.100000001)", "f64")
+
+
+def test_shared_hash_ignores_literal_values_but_not_structure_or_type():
+    h = lambda text, dt="f32", kind=capi.KIND_APPLY: capi.expr_emit(kind, dt, text, ["x"], shared=True)[1]
+    c = lambda text, dt="f32": capi.expr_constants(dt, text, ["x"]).tolist()
+    assert h("(x * 2.0)") == h("(x * 2)") == h("(x * 2.5)") == h("(x * -1e9)")
+    assert c("(x * 2.0)") == c("(x * 2)") == c("(x * 2.00)") == [2.0] and c("(x * 2.5)") == [2.5]
+    assert h("(x * 2.0)") != capi.expr_emit(capi.KIND_APPLY, "f32", "(x * 2.0)", ["x"])[1]
+    assert h("(x * 2.0)") != h("(x * 2.0)", "f64")
+    assert h("(x * 2.0)") != h("(x * 2.0)", "f32", capi.KIND_UNARY_GRAD)
+    assert h("(x * 2.0)") != h("(2.0 * x)")
+    assert h("(x * 2.0)") != h("(x + 2.0)")
+    assert c("(x * 0.1)") == c("(x * 0.100000001)")
+    assert c("(x * 0.1)", "f64") != c("(x * 0.100000001)", "f64")
 
 
 def test_tuning_is_part_of_the_key_and_source():

@@ -345,16 +345,83 @@ def test_launch_shape_follows_the_bytes_touched(hip):
 
 def test_kernel_cache(hip):
     c0, h0 = hip.cache_stats()
-    k1 = hip.compile(capi.KIND_APPLY, "f32", "((x * 41.0) + 0.125)", ("x",))
-    k2 = hip.compile(capi.KIND_APPLY, "f32", "((x*41) + 0.1250)", ("x",))
-    k3 = hip.compile(capi.KIND_APPLY, "f32", "((y * 41.0) + 0.125)", ("y",))
+    k1 = hip.compile(capi.KIND_APPLY, "f32", "tan(cos(((x * 41.0) + 0.125)))", ("x",))
+    k2 = hip.compile(capi.KIND_APPLY, "f32", "tan(cos(((x*41) + 0.1250)))", ("x",))
+    k3 = hip.compile(capi.KIND_APPLY, "f32", "tan(cos(((y * 41.0) + 0.125)))", ("y",))
     c1, h1 = hip.cache_stats()
     assert k1.value == k2.value == k3.value
     assert c1 - c0 == 1 and h1 - h0 == 2
-    k4 = hip.compile(capi.KIND_UNARY_GRAD, "f32", "((x * 41.0) + 0.125)", ("x",))
+    k4 = hip.compile(capi.KIND_UNARY_GRAD, "f32", "tan(cos(((x * 41.0) + 0.125)))", ("x",))
     assert k4.value != k1.value
     assert hip.kernel_name(k1).startswith("custos_apply_f32_") and hip.kernel_name(k1) in hip.kernel_source(k1)
     assert hip.kernel_name(k4).startswith("custos_unary_grad_f32_")
+
+
+def test_literals_are_launch_parameters(hip, oracle):
+    """The first set of literal values of an expression is compiled into the code; the second
+    compiles the form that takes them as launch parameters, and every later set of values is a
+    handle on that code (the reference compiles each distinct text,
+    src/devices/cuda/kernel_cache.rs:45-61)."""
+    rng = np.random.default_rng(77)
+    x = rng.uniform(-3, 3, 100003).astype(np.float32)
+    xb = hip.buffer(x)
+    first = hip.compile(capi.KIND_APPLY, "f32", "max(cos(((x * 1.5) - 0.25)), -0.75)", ("x",))
+    assert "CustosConsts" not in hip.kernel_source(first) and "0x1.8p+0f" in hip.kernel_source(first)
+    c0, _ = hip.cache_stats()
+    for step in range(40):
+        a, b, c = np.float32(1.0 + step * 0.37), np.float32(step * 0.11 - 2.0), np.float32(-0.05 * step)
+        f = lambda v: v.mul(float(a)).sub(float(b)).cos().max(float(c))
+        out = hip.apply_fn(xb, f)
+        assert ulp_distance_f32(out.read(), oracle.apply_fn(f, x)).max() <= 4, f"step {step}"
+        exact = hip.apply_fn(xb, lambda v: v.mul(float(a)).sub(float(b)).max(float(c)))
+        assert_bits_equal(exact.read(), np.maximum(x * a - b, c), f"exact step {step}")
+    c1, _ = hip.cache_stats()
+    # the shared form of the first expression; the second expression once for its first values, once shared
+    assert c1 - c0 == 3
+    k_a = hip.compile(capi.KIND_APPLY, "f32", "max(cos(((x * 2.5) - 0.25)), -0.75)", ("x",))
+    k_b = hip.compile(capi.KIND_APPLY, "f32", "max(cos(((x*2.50) - 0.250)), -0.75)", ("x",))
+    k_c = hip.compile(capi.KIND_APPLY, "f32", "max(cos(((x * 3.5) - 0.25)), -0.75)", ("x",))
+    assert k_a.value == k_b.value and k_a.value != k_c.value            # same values: same handle
+    assert hip.kernel_name(k_a) == hip.kernel_name(k_c) != hip.kernel_name(first)   # same code, other values
+    assert hip.kernel_source(k_a) == hip.kernel_source(k_c) and "struct CustosConsts { C c[3]; };" in hip.kernel_source(k_a)
+    again = hip.compile(capi.KIND_APPLY, "f32", "max(cos(((x * 1.5) - 0.25)), -0.75)", ("x",))
+    assert again.value == first.value                                   # the first values keep their kernel
+    assert hip.cache_stats()[0] == c1
+    # the shared code and the one with the values compiled in give the same bits
+    f15 = lambda v: v.mul(1.5).sub(0.25).cos().max(-0.75)
+    in_code = hip.apply_fn(xb, f15).read()
+    try:
+        hip.set_literal_policy(capi.LITERALS_AS_PARAMETERS)
+        as_parameters = hip.apply_fn(xb, f15).read()
+        fresh = hip.compile(capi.KIND_APPLY, "f32", "tanh(((x * 1.25) + 7.0))", ("x",))
+        assert "kc.c[1]" in hip.kernel_source(fresh)                    # shared form at once
+        hip.set_literal_policy(capi.LITERALS_IN_CODE)
+        before = hip.cache_stats()[0]
+        for k in (1.0, 2.0, 3.0):
+            got = hip.apply_fn(xb, lambda v: v.mul(k).add(k).abs().mul(k)).read()
+            assert_bits_equal(got, np.abs(x * np.float32(k) + np.float32(k)) * np.float32(k), f"in code {k}")
+        assert hip.cache_stats()[0] - before == 3                       # the reference's behaviour: one per text
+    finally:
+        hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
+    assert_bits_equal(as_parameters, in_code, "policy")
+    # integer types, a two-operand expression, the gradient kind, special values
+    xi = rng.integers(-1000, 1000, 5001).astype(np.int32)
+    for k in (3, -7, 2**31 - 1, -2**31):
+        got = hip.apply_fn(hip.buffer(xi, "i32"), lambda v: v.mul(k).add(k)).read()
+        assert_bits_equal(got, (xi.astype(np.int64) * k + k).astype(np.int32), f"i32 {k}")
+    xd = rng.uniform(-2, 2, 4099)
+    for k in (0.1, 1e300, -0.0, float("inf")):
+        got = hip.apply_fn(hip.buffer(xd, "f64"), lambda v: v.mul(k).min(k)).read()
+        prod = xd * k
+        assert_bits_equal(got, np.where(prod < k, prod, k), f"f64 {k}")
+    y = rng.uniform(-1, 1, x.size).astype(np.float32)
+    g = rng.uniform(-1, 1, x.size).astype(np.float32)
+    for k in (0.5, 4.0):
+        got = hip.apply_fn2(xb, hip.buffer(y), lambda l, r: l.mul(k).add(r.mul(k + 1))).read()
+        assert_bits_equal(got, x * np.float32(k) + y * np.float32(k + 1), f"two operands {k}")
+        lhs_grad = hip.buffer(g)
+        hip.add_unary_grad(xb, lhs_grad, hip.buffer(y), lambda v: v.mul(k))
+        assert_bits_equal(lhs_grad.read(), g + y * (x * np.float32(k)), f"gradient {k}")
 
 
 def test_error_paths(hip):
