@@ -159,7 +159,7 @@ def bench_c2(dev, args):
         dev.capture_begin()
         capi.check(lib.custos_hip_apply_fn(h, skernel, xb.ptr, out.ptr, n), h)
         sgraph = dev.capture_end()
-        sms, _ = time_steps(dev, sgraph.launch, args.steps, args.warmup)
+        sms, _ = time_steps(dev, sgraph.launch, args.steps, args.warmup, settle_ms=100)
         sgraph.destroy()
         dev.set_tuning(0, 0, 0, 0, 0)
         streaming = {"ms_per_step": round(sms / args.steps, 5),
@@ -167,7 +167,7 @@ def bench_c2(dev, args):
                      "kernel": dev.kernel_name(skernel),
                      "shape": "tiles first to last, non-temporal loads and stores, 2 vectors per thread"}
 
-    dms, _ = time_steps(dev, fused_step, args.steps, args.warmup)   # the fused kernel launched directly
+    dms, _ = time_steps(dev, fused_step, args.steps, args.warmup, settle_ms=100)   # the fused kernel launched directly
     direct_ms = dms / args.steps
 
     # Headline.  One step = what `Lazy::run` does from the second run on: replay the graph that
@@ -176,7 +176,7 @@ def bench_c2(dev, args):
     fused_step()
     graph = dev.capture_end()
     assert graph.kernel_nodes == 1
-    ms, wall_ms = time_steps(dev, graph.launch, args.steps, args.warmup)
+    ms, wall_ms = time_steps(dev, graph.launch, args.steps, args.warmup, settle_ms=100)
     per_launch_ms = ms / args.steps
     graph.destroy()
     gbs = algo_bytes / (per_launch_ms * 1e-3) / 1e9
