@@ -424,6 +424,34 @@ def test_literals_are_launch_parameters(hip, oracle):
         assert_bits_equal(lhs_grad.read(), g + y * (x * np.float32(k)), f"gradient {k}")
 
 
+def test_launch_shape_variants_of_shared_code(hip):
+    """A launch large enough for another launch shape compiles that variant once per form, not
+    once per set of literal values -- launched directly and from a recorded graph."""
+    n = 1 << 23                                   # 32 MiB per array: the 64 MiB launch takes non-temporal accesses
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-8, 8, n).astype(np.float32)
+    xb, out = hip.buffer(x), hip.alloc(n)
+    c0, _ = hip.cache_stats()
+    names = set()
+    for step, (a, b) in enumerate([(1.25, 0.5), (2.5, 0.75), (3.75, 1.0), (5.0, 1.25), (6.25, 1.5)]):
+        src = f"min(((x * {a}) - {b}), (x * {b}))"
+        k = hip.compile(capi.KIND_APPLY, "f32", src, ("x",))
+        names.add(hip.kernel_name(k, n))
+        want = np.minimum(x * np.float32(a) - np.float32(b), x * np.float32(b))
+        capi.check(hip.lib.custos_hip_apply_fn(hip.handle, k, xb.ptr, out.ptr, n), hip.handle)
+        assert_bits_equal(out.read(), want, f"direct {step}")
+        out.clear()
+        hip.capture_begin()
+        capi.check(hip.lib.custos_hip_apply_fn(hip.handle, k, xb.ptr, out.ptr, n), hip.handle)
+        graph = hip.capture_end()
+        for _ in range(3):
+            graph.launch()
+        assert_bits_equal(out.read(), want, f"graph {step}")
+        graph.destroy()
+    c1, _ = hip.cache_stats()
+    assert c1 - c0 == 4 and len(names) == 2       # (values in the code, shared form) x (small shape, this shape)
+
+
 def test_error_paths(hip):
     with pytest.raises(capi.CustosHipError) as e:
         hip.alloc(0)
