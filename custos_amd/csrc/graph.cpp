@@ -2,6 +2,7 @@
 // conflicts, merging of equal launches, explicit hipGraph nodes, replay
 // (include/custos_hip.h).
 #include <algorithm>
+#include <cstring>
 
 #include "runtime.hpp"
 
@@ -146,9 +147,10 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
     std::vector<std::pair<custos_hip_kernel*, std::vector<size_t>>> groups;
     for (size_t i : of_level) {
         if (dev->batching && batchable(nodes[i])) {
-            auto g = std::find_if(groups.begin(), groups.end(), [&](const auto& kv) { return kv.first == nodes[i].k; });
+            // (handles that differ only in the values of their literal parameters share `code`)
+            auto g = std::find_if(groups.begin(), groups.end(), [&](const auto& kv) { return kv.first == nodes[i].k->code; });
             if (g == groups.end()) {
-                groups.push_back({nodes[i].k, {}});
+                groups.push_back({nodes[i].k->code, {}});
                 g = groups.end() - 1;
             }
             g->second.push_back(i);
@@ -204,6 +206,13 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
         for (size_t member : p.members) {
             for (uint64_t ptr : nodes[member].ptrs) host_table->push_back(ptr);
             if (p.ragged) host_table->push_back(nodes[member].n);
+            // the member's literal parameters, padded to whole words
+            const std::vector<unsigned char>& values = nodes[member].k->spec.consts.bytes;
+            for (size_t at = 0; at < values.size(); at += 8) {
+                uint64_t word = 0;
+                std::memcpy(&word, values.data() + at, std::min<size_t>(8, values.size() - at));
+                host_table->push_back(word);
+            }
         }
         if (!p.ragged) continue;
         p.map_offset = host_table->size();
@@ -275,10 +284,11 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
             ln.func = reinterpret_cast<void*>(p.kern->fn_batched);
             ln.grid = dim3(static_cast<unsigned int>(blocks));
         }
-        // every generated entry point ends with the block of literal parameters (if the
+        // a generated entry point ends with the block of literal parameters (if the
         // expression has any) and the direction
-        const ConstPlan& consts = p.kern->spec.consts;
-        if (consts.n_params > 0) ln.args.push_back(consts.bytes);
+        // (a merged launch reads them from its table rows instead)
+        const ConstPlan& consts = first.k->spec.consts;
+        if (consts.n_params > 0 && p.members.size() == 1) ln.args.push_back(consts.bytes);
         ln.args.push_back(value(&rev, 8));
         if (p.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
     }

@@ -182,6 +182,7 @@ struct KernelText {
     const int n_in;    // inputs of the expression
     const int n_ops;   // values custos_elem takes
     const int n_ptrs;  // pointers per operand set (table row of a merged launch)
+    const int const_words;  // 8-byte words of a table row that hold the literal parameters
     std::string params;     // pointer parameters of the single-launch entry point
     std::string vec_ptrs;   // declarations of the vector views of the operands
     std::string tile_args;  // the views custos_tile takes
@@ -190,7 +191,8 @@ struct KernelText {
         : k(spec),
           n_in(spec.expr.n_vars),
           n_ops(spec.kind == Kind::Apply ? spec.expr.n_vars : 3),
-          n_ptrs(spec.kind == Kind::Apply ? spec.expr.n_vars + 1 : 3) {
+          n_ptrs(spec.kind == Kind::Apply ? spec.expr.n_vars + 1 : 3),
+          const_words(static_cast<int>((spec.consts.bytes.size() + 7) / 8)) {
         if (k.kind == Kind::Apply) {
             for (int i = 0; i < n_in; i++) {
                 const std::string id = std::to_string(i);
@@ -299,6 +301,14 @@ struct KernelText {
         return s;
     }
 
+    // In a merged launch every segment brings its own literal parameters: they follow the
+    // operand addresses (and the length) in its table row, so launches of one kernel merge
+    // whatever their values.  The row is the same for the whole workgroup: scalar loads.
+    std::string row_consts(int first_word) const {
+        if (const_words == 0) return "";
+        return "    CustosConsts kc;\n    __builtin_memcpy(&kc, ptrs + " + std::to_string(first_word) + ", sizeof(kc));\n";
+    }
+
     // operand pointers of a merged launch, read from the table row `ptrs`
     std::string table_operands() const {
         std::string s;
@@ -320,11 +330,12 @@ struct KernelText {
     std::string batched_entry() const {
         std::string s;
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-        s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, CUSTOS_KC_ENTRY const u64 rev) {\n";
+        s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, const u64 rev) {\n";
         s += "    const u64 blk = rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
         s += "    const u64 seg = blk / tiles_per_seg;\n";
         s += "    const u64 tile = blk - seg * tiles_per_seg;\n";
-        s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs) + ";\n";
+        s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + const_words) + ";\n";
+        s += row_consts(n_ptrs);
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
@@ -342,12 +353,13 @@ struct KernelText {
     std::string ragged_entry() const {
         std::string s;
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-        s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, CUSTOS_KC_ENTRY const u64 rev) {\n";
+        s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, const u64 rev) {\n";
         s += "    const u64 where = block_map[rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x];\n";
         s += "    const u64 seg = where >> 32;\n";
         s += "    const u64 tile = where & 0xffffffffull;\n";
-        s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + 1) + ";\n";
+        s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + 1 + const_words) + ";\n";
         s += "    const u64 n = ptrs[" + std::to_string(n_ptrs) + "];\n";
+        s += row_consts(n_ptrs + 1);
         s += "    const u64 n_vec = n / CUSTOS_VEC;\n";
         s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
         s += "    const u64 n_tiles = n_vec == 0 ? 1 : (n_vec + tile_vecs - 1) / tile_vecs;\n";
@@ -391,7 +403,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     if (!hash_expr(k.expr, dtype, k.consts, &h, err)) return false;
     // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
     int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 7 /* template version */};
+                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 8 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {

@@ -370,3 +370,45 @@ def test_alternating_direction_in_replayed_graphs(hip, oracle):
     finally:
         hip.set_tuning()
         hip.set_graph_direct_replay(4)
+
+
+def test_merged_launches_carry_their_own_literals(hip):
+    """Launches of one expression with different literal values are merged into one grid; every
+    segment reads its own values from its table row (equal and different lengths, several dtypes)."""
+    rng = np.random.default_rng(21)
+    for dtype, np_t, lengths in (("f32", np.float32, [4096] * 48), ("f32", np.float32, [1000 + 37 * i for i in range(48)]),
+                                 ("f64", np.float64, [515 + 8 * i for i in range(20)]), ("i16", np.int16, [4096 + 8 * i for i in range(20)]),
+                                 ("f16", np.float16, [2048] * 24)):
+        hip.set_literal_policy(capi.LITERALS_AS_PARAMETERS)
+        try:
+            ins, outs, wants = [], [], []
+            for i, length in enumerate(lengths):
+                if dtype[0] == "i":
+                    data = rng.integers(-100, 100, length).astype(np_t)
+                    a, b = int(i - 7), int(3 * i + 1)
+                    wants.append((data.astype(np.int64) * a + b).astype(np_t))
+                else:
+                    data = rng.uniform(-2, 2, length).astype(np_t)
+                    a, b = float(i) * 0.25 - 3.0, 1.0 / (i + 1)
+                    if dtype == "f16":
+                        wide = data.astype(np.float32)
+                        wants.append(np.maximum(wide * np.float32(a), np.float32(b)).astype(np.float16))
+                    else:
+                        wants.append(np.maximum(data * np_t(a), np_t(b)))
+                ins.append((hip.buffer(data, dtype), a, b))
+            hip.capture_begin()
+            for buf, a, b in ins:
+                if dtype[0] == "i":
+                    outs.append(hip.apply_fn(buf, lambda v: v.mul(a).add(b)))
+                else:
+                    outs.append(hip.apply_fn(buf, lambda v: v.mul(a).max(b)))
+            graph = hip.capture_end()
+            assert graph.kernel_nodes == 1, (dtype, graph.kernel_nodes)
+            for _ in range(2):
+                graph.launch()
+            for out, want in zip(outs, wants):
+                got = out.read()
+                assert got.view(np.uint8).tobytes() == np.ascontiguousarray(want).view(np.uint8).tobytes(), dtype
+            graph.destroy()
+        finally:
+            hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
