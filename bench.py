@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per launch of the fused chain at N = 2^28 with the default launch shape, from two
 # `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE) scaled by the identity-copy kernel of
 # known size; commands and raw counter values: profiles/fused_chain_f32_n2p28_hbm_traffic.md
-MEASURED_TRAFFIC_C2_N2P28 = 2147557902
+MEASURED_TRAFFIC_C2_N2P28 = 2147557720
 
 C2_OPS = [
     lambda v: v.sin(),
