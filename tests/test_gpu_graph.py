@@ -412,3 +412,27 @@ def test_merged_launches_carry_their_own_literals(hip):
             graph.destroy()
         finally:
             hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
+
+
+def test_merged_gradient_launches_carry_their_own_literals(hip):
+    """The same for the unary-gradient kind: g += o * (x * k_i), one grid for all k_i."""
+    rng = np.random.default_rng(22)
+    hip.set_literal_policy(capi.LITERALS_AS_PARAMETERS)
+    try:
+        sets = []
+        for i in range(40):
+            length = 700 + 64 * i
+            x, g, o = (rng.uniform(-1, 1, length).astype(np.float32) for _ in range(3))
+            k = 0.5 + i
+            sets.append((hip.buffer(x), hip.buffer(g), hip.buffer(o), k, g + o * (x * np.float32(k))))
+        hip.capture_begin()
+        for xb, gb, ob, k, _ in sets:
+            hip.add_unary_grad(xb, gb, ob, lambda v: v.mul(k))
+        graph = hip.capture_end()
+        assert graph.kernel_nodes == 1
+        graph.launch()
+        for _, gb, _, _, want in sets:
+            assert_bits_equal(gb.read(), want, "gradient")
+        graph.destroy()
+    finally:
+        hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
