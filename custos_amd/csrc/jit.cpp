@@ -193,6 +193,26 @@ static custos_hip_kernel* find_code(custos_hip_device* dev, const KernelSpec& sp
     return nullptr;
 }
 
+// The handle on `owner`'s code that carries the literal values of `k`: the owner itself if
+// they are its own, else a handle that shares the owner's module (made on first use).
+static custos_hip_kernel* handle_for_values(custos_hip_kernel* owner, std::unique_ptr<custos_hip_kernel> k,
+                                            const char* src, const char* const* markers, int32_t n_markers) {
+    if (owner->spec.consts.bytes == k->spec.consts.bytes) return owner;
+    const std::string values(k->spec.consts.bytes.begin(), k->spec.consts.bytes.end());
+    auto sibling = owner->siblings.find(values);
+    if (sibling == owner->siblings.end()) {
+        k->spec.source.clear();  // the owner holds the text
+        k->code = owner;
+        k->fn = owner->fn;
+        k->fn_batched = owner->fn_batched;
+        k->fn_ragged = owner->fn_ragged;
+        k->expr_src = src;
+        for (int i = 0; i < n_markers; i++) k->markers.push_back(markers[i]);
+        sibling = owner->siblings.emplace(values, std::move(k)).first;
+    }
+    return sibling->second.get();
+}
+
 // Parses, looks the key up in the cache, compiles on a miss.
 //
 // Literal values: the first set of values an expression is seen with is compiled into the
@@ -225,24 +245,7 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
                 k = std::move(shared);
             if (owner) {
                 dev->hits++;
-                if (owner->spec.consts.bytes == k->spec.consts.bytes) {
-                    *out = owner;
-                    return CUSTOS_HIP_OK;
-                }
-                // the same code with other values: a handle of its own that shares the module
-                const std::string values(k->spec.consts.bytes.begin(), k->spec.consts.bytes.end());
-                auto sibling = owner->siblings.find(values);
-                if (sibling == owner->siblings.end()) {
-                    k->spec.source.clear();  // the owner holds the text
-                    k->code = owner;
-                    k->fn = owner->fn;
-                    k->fn_batched = owner->fn_batched;
-                    k->fn_ragged = owner->fn_ragged;
-                    k->expr_src = src;
-                    for (int i = 0; i < n_markers; i++) k->markers.push_back(markers[i]);
-                    sibling = owner->siblings.emplace(values, std::move(k)).first;
-                }
-                *out = sibling->second.get();
+                *out = handle_for_values(owner, std::move(k), src, markers, n_markers);
                 return CUSTOS_HIP_OK;
             }
         }
