@@ -436,3 +436,26 @@ def test_merged_gradient_launches_carry_their_own_literals(hip):
         graph.destroy()
     finally:
         hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
+
+
+def test_unmerged_graph_nodes_take_literals_by_value(hip):
+    """With merging off every launch is a kernel node of its own in an instantiated hipGraph and
+    takes its literal values as an argument by value."""
+    rng = np.random.default_rng(23)
+    hip.set_literal_policy(capi.LITERALS_AS_PARAMETERS)
+    hip.set_graph_batching(False)
+    try:
+        data = [rng.uniform(-2, 2, 3000 + 16 * i).astype(np.float32) for i in range(12)]
+        bufs = [hip.buffer(d) for d in data]
+        hip.capture_begin()
+        outs = [hip.apply_fn(b, lambda v: v.mul(float(i) + 0.5).sub(1.0 / (i + 2))) for i, b in enumerate(bufs)]
+        graph = hip.capture_end()
+        assert graph.kernel_nodes == len(bufs)
+        for _ in range(3):
+            graph.launch()
+        for i, (d, out) in enumerate(zip(data, outs)):
+            assert_bits_equal(out.read(), d * np.float32(i + 0.5) - np.float32(1.0 / (i + 2)), f"node {i}")
+        graph.destroy()
+    finally:
+        hip.set_graph_batching(True)
+        hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
