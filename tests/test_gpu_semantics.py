@@ -676,12 +676,14 @@ def _random_tree(rng, leaves, depth, integer, unsigned=False):
 def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
     """Random trees of up to 31 nodes over one to four operands, built from the nodes whose
     results are exact: parser, operand order, literal typing and emitted code against the CPU
-    restatement evaluating the same tree, bit for bit (NaNs compare as NaN)."""
+    restatement evaluating the same tree, bit for bit (NaNs compare as NaN); and with the
+    literals compiled in against the literals as launch parameters."""
     from custos_amd.expr import Resolve
     rng = np.random.default_rng(sum(map(ord, dtype)))
     integer = dtype[0] in "iu"
     n = 4099
-    for trial in range(10):
+    import os
+    for trial in range(int(os.environ.get("CUSTOS_RANDOM_TREES", "10"))):   # more for a longer run
         k = int(rng.integers(1, 5))
         seed = int(rng.integers(1 << 30))
         build = lambda *leaves: _random_tree(np.random.default_rng(seed), list(leaves), 4, integer, dtype[0] == "u")
@@ -703,6 +705,13 @@ def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
         got = hip.apply_fn_n(bufs, build).read()
         want = oracle.apply_fn(build, *arrs, dtype=dtype)
         what = f"trial {trial}: {tree.to_cl_source(dtype)}"
+        # the form that takes the literals as launch parameters gives the same bits
+        hip.set_literal_policy(capi.LITERALS_AS_PARAMETERS)
+        try:
+            shared = hip.apply_fn_n(bufs, build).read()
+        finally:
+            hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
+        assert shared.view(np.uint8).tobytes() == got.view(np.uint8).tobytes(), f"literal parameters, {what}"
         if dtype == "f16_pernode":
             got = got.view(np.uint16)
             nan = lambda b: (b & 0x7fff) > 0x7c00
