@@ -73,6 +73,11 @@ std::vector<std::string> hiprtc_options(const std::string& arch) {
         "-fhip-fp32-correctly-rounded-divide-sqrt",
         // keep f32 arithmetic on the scalar-per-lane instructions
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        // No v_fma_mix*: hipcc folds `(_Float16)(a * b)` into v_fma_mixlo_f16 a, b, +0, and
+        // adding +0 turns a product of -0 into +0 (the CPU device keeps the sign).  Costs
+        // nothing measurable on the f16 chain; keeping the product apart from the rounding
+        // with an empty asm instead cost 5 %.
+        "-Xclang", "-target-feature", "-Xclang", "-fma-mix-insts",
     };
 }
 
@@ -403,7 +408,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     if (!hash_expr(k.expr, dtype, k.consts, &h, err)) return false;
     // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
     int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 8 /* template version */};
+                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 9 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {

@@ -610,6 +610,44 @@ def test_more_than_2p32_bytes_and_elements(hip):
     assert_bits_equal(tail, np.roll(want, -((n - 77) % (1 << 20)))[:77])
 
 
+@pytest.mark.parametrize("dtype", ["f16", "f16_pernode", "bf16", "bf16_pernode", "f32"])
+def test_products_keep_the_sign_of_zero(hip, oracle, dtype):
+    """0 * negative = -0, also where the product is rounded to a 16-bit type next: a compiler
+    that folds product and rounding into one fused multiply-add with a +0 addend loses the
+    sign.  Vector body, partial tile and scalar tail (n is not a multiple of the vector)."""
+    n = 4099
+    base = dtype.split("_")[0]
+    if base == "f16":
+        xb = synth.uniform_f16_bits(31, n, -3, 3)
+        xb[5::7] = 0x8000
+        view = lambda a: a.view(np.float16)
+    elif base == "bf16":
+        xb = (synth.uniform_f32(31, n, -3, 3).view(np.uint32) >> 16).astype(np.uint16)
+        xb[5::7] = 0x8000
+        view = lambda a: a
+    else:
+        xb = synth.uniform_f32(31, n, -3, 3)
+        xb[5::7] = -0.0
+        view = lambda a: a
+    x = hip.buffer(view(xb), dtype)
+    for name, f in (("x * 0", lambda v: v.mul(0.0)), ("(x >= 9) * (x + x)", lambda v: v.geq(9.0).mul(v.add(v))),
+                    ("-(x * 0)", lambda v: v.mul(0.0).neg()), ("(x * 0) * 5", lambda v: v.mul(0.0).mul(5.0)),
+                    ("x * (x - x)", lambda v: v.mul(v.sub(v)))):
+        got = hip.apply_fn(x, f).read()
+        want = oracle.apply_fn(f, xb, dtype=dtype)
+        if base != "f32":
+            got = got.view(np.uint16)
+        assert_bits_equal(got, want, f"{dtype}: {name}")
+        bits = got.view(np.uint32) if base == "f32" else got
+        assert ((bits << 1) == 0).all() and (bits != 0).any() and (bits == 0).any(), name   # zeros of both signs
+    g0 = xb.copy()
+    gb = hip.buffer(view(g0), dtype)
+    hip.add_unary_grad(x, gb, x, lambda v: v.mul(0.0))          # g + x * (x * 0)
+    got = gb.read()
+    assert_bits_equal(got.view(np.uint16) if base != "f32" else got,
+                      oracle.add_unary_grad(lambda v: v.mul(0.0), xb, g0, xb, dtype=dtype), f"{dtype}: gradient")
+
+
 @pytest.mark.parametrize("dtype", ["f16_pernode", "bf16_pernode"])
 def test_per_node_rounding_of_16bit_floats(hip, oracle, dtype):
     """Every node rounded to the storage type, what the reference's `half` arithmetic does
