@@ -78,6 +78,11 @@ std::vector<std::string> hiprtc_options(const std::string& arch) {
         // nothing measurable on the f16 chain; keeping the product apart from the rounding
         // with an empty asm instead cost 5 %.
         "-Xclang", "-target-feature", "-Xclang", "-fma-mix-insts",
+        // No SLP vectorizer: without the packed f32 instructions the backend cannot select the
+        // two-element f32 negation the vectorizer forms in front of a packed f32 -> f16
+        // conversion ("Cannot select: v2f32 = bitcast", which ends the process); the kernels
+        // are written in 16-byte vectors already and gain nothing from it.
+        "-fno-slp-vectorize",
     };
 }
 
@@ -408,7 +413,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     if (!hash_expr(k.expr, dtype, k.consts, &h, err)) return false;
     // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
     int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 9 /* template version */};
+                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 10 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {

@@ -154,6 +154,18 @@ def test_shared_form_takes_literals_as_launch_parameters():
             assert "kc.c[1]" in capi.expr_emit(kind, dtype, text, ["x"], shared=True)[0]
 
 
+def test_expressions_that_ended_the_compiler_do_compile():
+    """With the packed f32 instructions off, the backend could not select a two-element f32
+    negation that the SLP vectorizer formed in front of a packed f32 -> f16 conversion; the
+    compiler's fatal error ends the process, so these would not even fail."""
+    for dtype, text, markers in (("f16_pernode", "-(((min(a, c) <= -1.0535643) / a))", ["a", "b", "c"]),
+                                 ("f16_pernode", "(a + ((min(b, a) * (a <= a)) + -3.632779))", ["a", "b"]),
+                                 ("f16", "-((a / b))", ["a", "b"]),
+                                 ("f16_pernode", "-((a - max(b, 1.9355469)))", ["a", "b"])):
+        for kind in (capi.KIND_APPLY,) + ((capi.KIND_UNARY_GRAD,) if len(markers) == 1 else ()):
+            assert capi.expr_build_code_object(kind, dtype, text, markers) > 0
+
+
 def test_min_max_emitted_as_selects():
     src, _ = capi.expr_emit(capi.KIND_APPLY, "f32", "min(max(x, 0.0), 6.0)", ["x"])
     assert "fmax" not in src and "fmin" not in src
