@@ -710,36 +710,51 @@ def _random_tree(rng, leaves, depth, integer, unsigned=False):
     return getattr(a, ops2[int(rng.integers(len(ops2)))])(b)
 
 
-@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u16", "f16_pernode"])
+_INT_RANGES = {"i8": (-128, 128), "u8": (0, 256), "i16": (-32768, 32768), "u16": (0, 60000), "i32": (-70000, 70000),
+               "u32": (0, 1 << 32), "i64": (-(1 << 40), 1 << 40), "u64": (0, 1 << 63)}
+
+
+def _random_tree_cases(dtype, trials):
+    """(trial, build, tree, input arrays) of the random-tree test for one element type."""
+    from custos_amd.expr import Resolve
+    rng = np.random.default_rng(sum(map(ord, dtype)))
+    integer = dtype[0] in "iu"
+    n = 4099
+    for trial in range(trials):
+        k = int(rng.integers(1, 5))
+        seed = int(rng.integers(1 << 30))
+        build = lambda *leaves, seed=seed: _random_tree(np.random.default_rng(seed), list(leaves), 4, integer, dtype[0] == "u")
+        tree = build(*[Resolve(nm, i) for i, nm in enumerate(("a", "b", "c", "d")[:k])])
+        if isinstance(tree, (Const, Resolve)):
+            continue
+        if dtype.startswith("f16"):
+            arrs = [synth.uniform_f16_bits(200 + trial * 4 + i, n, -3, 3) for i in range(k)]
+            arrs[0][:8] = [0x0000, 0x8000, 0x7c00, 0xfc00, 0x7e00, 0x0001, 0x8001, 0x7bff]
+        elif dtype.startswith("bf16"):
+            arrs = [(synth.uniform_f32(200 + trial * 4 + i, n, -3, 3).view(np.uint32) >> 16).astype(np.uint16) for i in range(k)]
+            arrs[0][:8] = [0x0000, 0x8000, 0x7f80, 0xff80, 0x7fc0, 0x0001, 0x8001, 0x7f7f]
+        elif integer:
+            lo, hi = _INT_RANGES[dtype]
+            npdt = np.dtype(capi.DTYPES[dtype][1])
+            arrs = [rng.integers(lo, hi, size=n, dtype=np.uint64 if dtype == "u64" else np.int64).astype(npdt) for _ in range(k)]
+        else:
+            npdt = np.dtype(capi.DTYPES[dtype][1])
+            arrs = [synth.uniform_f32(200 + trial * 4 + i, n, -3, 3).astype(npdt) for i in range(k)]
+            arrs[0][:SPECIALS.size] = SPECIALS.astype(npdt)
+        yield trial, build, tree, arrs
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u16", "f16_pernode", "f16", "bf16", "bf16_pernode",
+                                   "i8", "u8", "i16", "i64", "u32", "u64"])
 def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
     """Random trees of up to 31 nodes over one to four operands, built from the nodes whose
     results are exact: parser, operand order, literal typing and emitted code against the CPU
     restatement evaluating the same tree, bit for bit (NaNs compare as NaN); and with the
     literals compiled in against the literals as launch parameters."""
-    from custos_amd.expr import Resolve
-    rng = np.random.default_rng(sum(map(ord, dtype)))
-    integer = dtype[0] in "iu"
-    n = 4099
     import os
-    for trial in range(int(os.environ.get("CUSTOS_RANDOM_TREES", "10"))):   # more for a longer run
-        k = int(rng.integers(1, 5))
-        seed = int(rng.integers(1 << 30))
-        build = lambda *leaves: _random_tree(np.random.default_rng(seed), list(leaves), 4, integer, dtype[0] == "u")
-        tree = build(*[Resolve(nm, i) for i, nm in enumerate(("a", "b", "c", "d")[:k])])
-        if isinstance(tree, (Const, Resolve)):
-            continue
-        if dtype == "f16_pernode":
-            arrs = [synth.uniform_f16_bits(200 + trial * 4 + i, n, -3, 3) for i in range(k)]
-            bufs = [hip.buffer(a.view(np.float16), dtype) for a in arrs]
-        else:
-            npdt = np.dtype(capi.DTYPES[dtype][1])
-            if integer:
-                lo, hi = (0, 60000) if dtype == "u16" else (-70000, 70000)
-                arrs = [rng.integers(lo, hi, size=n).astype(npdt) for _ in range(k)]
-            else:
-                arrs = [synth.uniform_f32(200 + trial * 4 + i, n, -3, 3).astype(npdt) for i in range(k)]
-                arrs[0][:SPECIALS.size] = SPECIALS.astype(npdt)
-            bufs = [hip.buffer(a, dtype) for a in arrs]
+    half = dtype.split("_")[0] in ("f16", "bf16")
+    for trial, build, tree, arrs in _random_tree_cases(dtype, int(os.environ.get("CUSTOS_RANDOM_TREES", "10"))):
+        bufs = [hip.buffer(a.view(np.float16) if dtype.startswith("f16") else a, dtype) for a in arrs]
         got = hip.apply_fn_n(bufs, build).read()
         want = oracle.apply_fn(build, *arrs, dtype=dtype)
         what = f"trial {trial}: {tree.to_cl_source(dtype)}"
@@ -750,9 +765,12 @@ def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
         finally:
             hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
         assert shared.view(np.uint8).tobytes() == got.view(np.uint8).tobytes(), f"literal parameters, {what}"
-        if dtype == "f16_pernode":
+        if half:
             got = got.view(np.uint16)
-            nan = lambda b: (b & 0x7fff) > 0x7c00
+            if dtype.startswith("f16"):
+                nan = lambda b: (b & 0x7fff) > 0x7c00
+            else:
+                nan = lambda b: (b & 0x7fff) > 0x7f80
             same = (got == want) | (nan(got) & nan(want))
             assert same.all(), f"{what} differs at {np.flatnonzero(~same)[:5]}"
         else:
