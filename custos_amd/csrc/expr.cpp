@@ -667,8 +667,29 @@ bool emit_expr_body(const Expr& e, DType dtype, const ConstPlan& plan, std::stri
                 break;
             // Number::min / Number::max: a select on < and > (src/number.rs:201-209),
             // not fmin/fmax: NaN and signed-zero behaviour differ.
-            case Op::Min: rhs = "(" + t(n.a) + " < " + t(n.b) + ") ? " + t(n.a) + " : " + t(n.b); break;
-            case Op::Max: rhs = "(" + t(n.a) + " > " + t(n.b) + ") ? " + t(n.a) + " : " + t(n.b); break;
+            case Op::Min:
+            case Op::Max: {
+                const char* cmp = n.op == Op::Min ? " < " : " > ";
+                // hipcc turns the select into v_min / v_max where it can prove that a NaN
+                // cannot change the outcome (a constant second operand, operands that are
+                // comparison results, ...).  For two zeros of different sign those return -0
+                // (min) and +0 (max), the select returns the second operand.  So unless the
+                // second operand is a literal for which both agree, it reaches the select
+                // through custos_pick, and the compiler sees no min / max pattern.
+                bool plain = !flt;
+                const Node& second = e.nodes[static_cast<size_t>(n.b)];
+                if (flt && second.op == Op::Const) {
+                    Literal l;
+                    if (!convert_literal(second.lit, dtype, &l, err)) return false;
+                    const bool zero = !l.is_nan && l.f == 0.0;
+                    const bool negative_zero = zero && std::signbit(l.f);
+                    plain = plan.slot[static_cast<size_t>(n.b)] >= 0 || !zero ||
+                            (n.op == Op::Min ? negative_zero : !negative_zero);
+                }
+                if (plain) rhs = "(" + t(n.a) + cmp + t(n.b) + ") ? " + t(n.a) + " : " + t(n.b);
+                else rhs = "custos_pick(" + t(n.a) + cmp + t(n.b) + ", " + t(n.a) + ", " + t(n.b) + ")";
+                break;
+            }
             case Op::GEq: rhs = "(" + C + ")(" + t(n.a) + " >= " + t(n.b) + ")"; break;
             case Op::LEq: rhs = "(" + C + ")(" + t(n.a) + " <= " + t(n.b) + ")"; break;
             case Op::Eq: rhs = "(" + C + ")(" + t(n.a) + " == " + t(n.b) + ")"; break;

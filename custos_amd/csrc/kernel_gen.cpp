@@ -124,6 +124,12 @@ static __device__ __forceinline__ S custos_store(C c) {
     }
     if (dtype_rounds_per_node(dtype))
         s += "static __device__ __forceinline__ C custos_round(C c) { return custos_load(custos_store(c)); }\n";
+    // `first ? a : b` with b passed through an empty asm (no instruction) on its way into the
+    // select, so that the compiler cannot turn it into v_min / v_max; see the min / max nodes
+    // in emit_expr_body.  (The asm sits outside the conditional, else it becomes a branch.)
+    if (dtype_is_float(dtype))
+        s += "static __device__ __forceinline__ C custos_pick(bool first, C a, C b) {\n"
+             "    __asm__(\"\" : \"+v\"(b));\n    return first ? a : b;\n}\n";
     if (dtype == DType::F64) {
         s += R"(static __device__ __forceinline__ double custos_sin(double a) { return sin(a); }
 static __device__ __forceinline__ double custos_cos(double a) { return cos(a); }
@@ -413,7 +419,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     if (!hash_expr(k.expr, dtype, k.consts, &h, err)) return false;
     // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
     int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 10 /* template version */};
+                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 11 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {

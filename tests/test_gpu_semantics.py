@@ -610,6 +610,40 @@ def test_more_than_2p32_bytes_and_elements(hip):
     assert_bits_equal(tail, np.roll(want, -((n - 77) % (1 << 20)))[:77])
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64", "f16", "f16_pernode", "bf16"])
+def test_min_max_of_zeros_return_the_second_operand(hip, oracle, dtype):
+    """`Number::min` / `max` are selects (src/number.rs:201-209): for two zeros of different sign
+    they return the second operand, where the hardware's min / max return -0 / +0.  The compiler
+    swaps the select for the instruction when it can rule NaNs out: a literal operand, operands
+    that are comparison results."""
+    n = 4099
+    base = dtype.split("_")[0]
+    if base == "f16":
+        xb = synth.uniform_f16_bits(41, n, -3, 3)
+        xb[3::5], xb[4::5] = 0x8000, 0x0000
+        view = lambda a: a.view(np.float16)
+    elif base == "bf16":
+        xb = (synth.uniform_f32(41, n, -3, 3).view(np.uint32) >> 16).astype(np.uint16)
+        xb[3::5], xb[4::5] = 0x8000, 0x0000
+        view = lambda a: a
+    else:
+        xb = synth.uniform_f32(41, n, -3, 3).astype(np.float32 if dtype == "f32" else np.float64)
+        xb[3::5], xb[4::5] = -0.0, 0.0
+        view = lambda a: a
+    x = hip.buffer(view(xb), dtype)
+    cases = (("min(x, 0)", lambda v: v.min(0.0)), ("max(x, 0)", lambda v: v.max(0.0)),
+             ("min(x, -0)", lambda v: v.min(-0.0)), ("max(x, -0)", lambda v: v.max(-0.0)),
+             ("min(0, x)", lambda v: Const(0.0).min(v)), ("max(0, x)", lambda v: Const(0.0).max(v)),
+             ("min(-0, x)", lambda v: Const(-0.0).min(v)), ("max(-0, x)", lambda v: Const(-0.0).max(v)),
+             ("min(x, x >= 9)", lambda v: v.min(v.geq(9.0))), ("max(x >= 9, -(x >= 9))", lambda v: v.geq(9.0).max(v.geq(9.0).neg())),
+             ("min(-(x >= 9), x >= 9)", lambda v: v.geq(9.0).neg().min(v.geq(9.0))), ("max(x, x * 0)", lambda v: v.max(v.mul(0.0))),
+             ("min(|x|, -(|x| * 0))", lambda v: v.abs().min(v.abs().mul(0.0).neg())))
+    for name, f in cases:
+        got = hip.apply_fn(x, f).read()
+        want = oracle.apply_fn(f, xb, dtype=dtype)
+        assert_bits_equal(got.view(np.uint16) if base in ("f16", "bf16") else got, want, f"{dtype}: {name}")
+
+
 @pytest.mark.parametrize("dtype", ["f16", "f16_pernode", "bf16", "bf16_pernode", "f32"])
 def test_products_keep_the_sign_of_zero(hip, oracle, dtype):
     """0 * negative = -0, also where the product is rounded to a 16-bit type next: a compiler
