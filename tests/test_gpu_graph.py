@@ -211,49 +211,51 @@ def test_merged_launches_of_different_lengths(hip, oracle):
 def test_recorded_dependencies_random(hip, oracle):
     """Random programs over a small pool of buffers, with in-place updates, views and clears:
     replaying the built graph (levels, side-by-side nodes, merged launches) must equal running
-    the same calls eagerly, bit for bit."""
+    the same calls eagerly, bit for bit.  Even trials use aligned half-buffer views, odd trials
+    views of any offset and length (partial overlaps between operations, scalar launches)."""
+    import os
     rng = np.random.default_rng(1234)
     n = 2048
     fns1 = [lambda v: v.mul(1.25).add(0.5), lambda v: v.neg().max(-3.0), lambda v: v.abs().sqrt(), lambda v: v.mul(v).min(9.0)]
     fns2 = [lambda p, q: p.add(q), lambda p, q: p.mul(q).sub(0.125), lambda p, q: p.max(q)]
-    for trial in range(6):
+    for trial in range(int(os.environ.get("CUSTOS_RANDOM_PROGRAMS", "6"))):   # more for a longer run
         nbuf = 6
         init = [synth.uniform_f32(trial * 10 + i, n, -2, 2) for i in range(nbuf)]
         program = []
         for _ in range(40):
             kind = rng.integers(0, 5)
-            lo = int(rng.integers(0, 3)) * 512          # views: [lo, lo + 1024) keeps 16-byte phases equal
+            if trial % 2:
+                lo = int(rng.integers(0, 1500))
+                ln = int(rng.integers(1, n - lo + 1))
+            else:
+                lo, ln = int(rng.integers(0, 3)) * 512, 1024     # [lo, lo + 1024) keeps 16-byte phases equal
             if kind == 0:
-                program.append(("u", int(rng.integers(len(fns1))), int(rng.integers(nbuf)), int(rng.integers(nbuf)), lo))
+                program.append(("u", int(rng.integers(len(fns1))), int(rng.integers(nbuf)), int(rng.integers(nbuf)), lo, ln))
             elif kind in (1, 2):
                 a, b, o = (int(v) for v in rng.integers(nbuf, size=3))
-                program.append(("b", int(rng.integers(len(fns2))), a, b, o, lo))
+                program.append(("b", int(rng.integers(len(fns2))), a, b, o, lo, ln))
             elif kind == 3:
-                program.append(("g", int(rng.integers(len(fns1))), *(int(v) for v in rng.choice(nbuf, size=3, replace=False)), lo))
+                program.append(("g", int(rng.integers(len(fns1))), *(int(v) for v in rng.choice(nbuf, size=3, replace=False)), lo, ln))
             else:
-                program.append(("c", int(rng.integers(nbuf)), lo))
+                program.append(("c", int(rng.integers(nbuf)), lo, ln))
 
         def run(bufs):
             for op in program:
+                lo, ln = op[-2], op[-1]
+                view = lambda i: bufs[i].slice(lo, lo + ln)
                 if op[0] == "u":
-                    _, fi, src, dst, lo = op
-                    if src == dst:
-                        hip.apply_fn(bufs[src].slice(lo, lo + 1024), fns1[fi], out=bufs[dst].slice(lo, lo + 1024))
-                    else:
-                        hip.apply_fn(bufs[src].slice(lo, lo + 1024), fns1[fi], out=bufs[dst].slice(lo, lo + 1024))
+                    _, fi, src, dst = op[:4]
+                    hip.apply_fn(view(src), fns1[fi], out=view(dst))
                 elif op[0] == "b":
-                    _, fi, a, b, o, lo = op
-                    if a == b or (o in (a, b) and False):
+                    _, fi, a, b, o = op[:5]
+                    if a == b:
                         continue
-                    hip.apply_fn2(bufs[a].slice(lo, lo + 1024), bufs[b].slice(lo, lo + 1024), fns2[fi],
-                                  out=bufs[o].slice(lo, lo + 1024))
+                    hip.apply_fn2(view(a), view(b), fns2[fi], out=view(o))
                 elif op[0] == "g":
-                    _, fi, x, g, o, lo = op
-                    hip.add_unary_grad(bufs[x].slice(lo, lo + 1024), bufs[g].slice(lo, lo + 1024),
-                                       bufs[o].slice(lo, lo + 1024), fns1[fi])
+                    _, fi, x, g, o = op[:5]
+                    hip.add_unary_grad(view(x), view(g), view(o), fns1[fi])
                 else:
-                    _, b, lo = op
-                    bufs[b].slice(lo, lo + 1024).clear()
+                    view(op[1]).clear()
 
         eager = [hip.buffer(x) for x in init]
         run(eager)
@@ -269,6 +271,11 @@ def test_recorded_dependencies_random(hip, oracle):
         hip.sync()
         for i, b in enumerate(lazy):
             assert_bits_equal(b.read(), want[i], f"trial {trial} buffer {i} (levels {g.stats()})")
+        g.launch()          # a second replay continues from the first one's results, like a second eager run
+        run(eager)
+        hip.sync()
+        for i, b in enumerate(lazy):
+            assert_bits_equal(b.read(), eager[i].read(), f"trial {trial} second replay, buffer {i}")
         g.destroy()
 
 
