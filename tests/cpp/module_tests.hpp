@@ -5,6 +5,7 @@
 #pragma once
 
 #include <cmath>
+#include <cstdlib>
 #include <vector>
 
 #include "check.hpp"
@@ -660,7 +661,9 @@ void elementwise_fuse_random_programs() {
         rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
         return rng % m;
     };
-    for (int trial = 0; trial < 12; trial++) {
+    const char* more = std::getenv("CUSTOS_RANDOM_PROGRAMS");   // more trials for a longer run
+    const int trials = more ? std::atoi(more) : 12;
+    for (int trial = 0; trial < trials; trial++) {
         std::vector<std::vector<int>> prog;  // {kind, fn, in0, in1}
         const int n_leaf = 3, n_ops = 10;
         for (int i = 0; i < n_ops; i++) {
