@@ -808,7 +808,23 @@ def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
             same = (got == want) | (nan(got) & nan(want))
             assert same.all(), f"{what} differs at {np.flatnonzero(~same)[:5]}"
         else:
+            nan = None
             assert_bits_equal(got, want, what)
+        if len(arrs) == 1:
+            # the same tree as the derivative of a unary gradient: g + o * f(x), the buffer's own
+            # values rotated serve as g and o
+            g0, o = np.roll(arrs[0], 1), np.roll(arrs[0], 2)
+            as_buf = lambda a: hip.buffer(a.view(np.float16) if dtype.startswith("f16") else a, dtype)
+            gb = as_buf(g0)
+            hip.add_unary_grad(bufs[0], gb, as_buf(o), build)
+            got_g = gb.read()
+            want_g = oracle.add_unary_grad(build, arrs[0], g0, o, dtype=dtype)
+            if half:
+                got_g = got_g.view(np.uint16)
+                same = (got_g == want_g) | (nan(got_g) & nan(want_g))
+                assert same.all(), f"gradient, {what} differs at {np.flatnonzero(~same)[:5]}"
+            else:
+                assert_bits_equal(got_g, want_g, f"gradient, {what}")
 
 
 def test_allocation_pool():
