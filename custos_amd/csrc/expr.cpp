@@ -588,7 +588,8 @@ bool plan_constants(const Expr& e, DType dtype, bool all_in_code, ConstPlan* pla
 // hashing
 // ---------------------------------------------------------------------------
 
-bool hash_expr(const Expr& e, DType dtype, const ConstPlan& plan, uint64_t* hash, ParseError* err) {
+bool hash_expr(const Expr& e, DType dtype, const ConstPlan& plan, uint64_t* hash, ParseError* err,
+               std::vector<uint64_t>* code_literals) {
     uint64_t h = fnv1a64("custos-expr-v2", 14);
     int32_t head[3] = {static_cast<int32_t>(dtype), e.n_vars, e.root};
     h = fnv1a64(head, sizeof head, h);
@@ -605,8 +606,10 @@ bool hash_expr(const Expr& e, DType dtype, const ConstPlan& plan, uint64_t* hash
                 std::memcpy(&bits, &v, 8);
                 if (l.is_nan) bits = 0x7ff8000000000000ull;
                 h = fnv1a64(&bits, 8, h);
+                if (code_literals) code_literals->push_back(bits);
             } else {
                 h = fnv1a64(&l.u, 8, h);
+                if (code_literals) code_literals->push_back(l.u);
             }
         }
     }

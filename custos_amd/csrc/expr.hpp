@@ -117,7 +117,9 @@ std::string to_cl_source(const Expr& e, const std::vector<std::string>& markers,
 // Structural 64-bit hash: node kinds, operand wiring, which literals are parameters, and
 // the *values* of the literals that stay in the code after conversion to the element type
 // ("2", "2.0" and "2.00" hash alike).
-bool hash_expr(const Expr& e, DType dtype, const ConstPlan& plan, uint64_t* hash, ParseError* err);
+// `code_literals` (optional) receives those values' bits in node order.
+bool hash_expr(const Expr& e, DType dtype, const ConstPlan& plan, uint64_t* hash, ParseError* err,
+               std::vector<uint64_t>* code_literals = nullptr);
 
 // Emits the body of `custos_expr`: SSA statements over v0..v{n-1} of the
 // compute type (parameters read `kc.c[slot]`) and a final `return`.

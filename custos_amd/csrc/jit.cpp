@@ -95,7 +95,7 @@ bool markers_from_c(const char* const* markers, int32_t n, std::vector<std::stri
 
 int32_t spec_from_c(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
                     const char* const* markers, int32_t n_markers, const Tuning& tuning,
-                    bool literals_in_code, KernelSpec* spec) {
+                    bool literals_in_code, KernelSpec* spec, bool with_source = true) {
     if (!src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");
     if (kind != CUSTOS_HIP_KIND_APPLY && kind != CUSTOS_HIP_KIND_UNARY_GRAD)
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown kernel kind");
@@ -104,7 +104,8 @@ int32_t spec_from_c(custos_hip_device* dev, int32_t kind, int32_t dtype, const c
     if (!markers_from_c(markers, n_markers, &m))
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 4 non-empty markers are required");
     ParseError err;
-    if (!build_kernel_spec(static_cast<Kind>(kind), static_cast<DType>(dtype), src, m, tuning, literals_in_code, spec, &err))
+    if (!build_kernel_spec(static_cast<Kind>(kind), static_cast<DType>(dtype), src, m, tuning, literals_in_code, spec, &err,
+                           with_source))
         return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
     return CUSTOS_HIP_OK;
 }
@@ -178,18 +179,13 @@ int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k) {
     return CUSTOS_HIP_OK;
 }
 
-// The cached kernel that was compiled from the same text as `spec` (apart from the first
-// line, a comment in which literals that stay in the code keep the caller's spelling).
+// The cached kernel for the same translation unit as `spec` (compared by structure: `spec`
+// need not have its text yet).
 static custos_hip_kernel* find_code(custos_hip_device* dev, const KernelSpec& spec) {
     auto bucket = dev->cache.find(spec.hash);
     if (bucket == dev->cache.end()) return nullptr;
-    for (auto& cached : bucket->second) {
-        const std::string& a = cached->spec.source;
-        const std::string& b = spec.source;
-        if (cached->spec.kind != Kind::Source &&
-            a.compare(a.find('\n'), std::string::npos, b, b.find('\n'), std::string::npos) == 0)
-            return cached.get();
-    }
+    for (auto& cached : bucket->second)
+        if (cached->spec.kind != Kind::Source && same_code(cached->spec, spec)) return cached.get();
     return nullptr;
 }
 
@@ -201,8 +197,7 @@ static custos_hip_kernel* handle_for_values(custos_hip_kernel* owner, std::uniqu
     const std::string values(k->spec.consts.bytes.begin(), k->spec.consts.bytes.end());
     auto sibling = owner->siblings.find(values);
     if (sibling == owner->siblings.end()) {
-        k->spec.source.clear();  // the owner holds the text
-        k->code = owner;
+        k->code = owner;  // (which also holds the text)
         k->fn = owner->fn;
         k->fn_batched = owner->fn_batched;
         k->fn_ragged = owner->fn_ragged;
@@ -226,7 +221,8 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
                             const char* const* markers, int32_t n_markers, const Tuning& tuning,
                             bool prefer_shared, custos_hip_kernel** out) {
     std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
-    int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, /*literals_in_code=*/true, &k->spec);
+    // (specs without their text: it is generated only for what is compiled)
+    int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, /*literals_in_code=*/true, &k->spec, false);
     if (rc != CUSTOS_HIP_OK) return rc;
     if (custos_hip_kernel* known = find_code(dev, k->spec)) {
         dev->hits++;
@@ -235,7 +231,7 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
     }
     if (k->spec.n_literals > 0 && dev->literal_policy != CUSTOS_HIP_LITERALS_IN_CODE) {
         std::unique_ptr<custos_hip_kernel> shared(new custos_hip_kernel);
-        rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, /*literals_in_code=*/false, &shared->spec);
+        rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, /*literals_in_code=*/false, &shared->spec, false);
         if (rc != CUSTOS_HIP_OK) return rc;
         if (shared->spec.consts.n_params > 0) {
             custos_hip_kernel* owner = find_code(dev, shared->spec);
@@ -250,6 +246,8 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
             }
         }
     }
+    ParseError err;
+    if (!emit_kernel_source(&k->spec, &err)) return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
     rc = build_module(dev, k.get());
     if (rc != CUSTOS_HIP_OK) return rc;
     // further entry points of the module: many launches in one grid

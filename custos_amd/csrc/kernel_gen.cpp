@@ -395,7 +395,7 @@ struct KernelText {
 
 bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
                        const std::vector<std::string>& markers, const Tuning& tuning,
-                       bool literals_in_code, KernelSpec* out, ParseError* err) {
+                       bool literals_in_code, KernelSpec* out, ParseError* err, bool with_source) {
     KernelSpec k;
     k.kind = kind;
     k.dtype = dtype;
@@ -416,7 +416,8 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     if (!plan_constants(k.expr, dtype, literals_in_code, &k.consts, err)) return false;
     for (const Node& n : k.expr.nodes) k.n_literals += n.op == Op::Const;
     uint64_t h;
-    if (!hash_expr(k.expr, dtype, k.consts, &h, err)) return false;
+    if (!hash_expr(k.expr, dtype, k.consts, &h, err, &k.code_literals)) return false;
+    k.markers = markers;
     // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
     int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
                        k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 11 /* template version */};
@@ -432,20 +433,27 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
                  dtype_names[static_cast<int>(dtype)] + "_" + hex;
     }
 
+    if (with_source && !emit_kernel_source(&k, err)) return false;
+    *out = std::move(k);
+    return true;
+}
+
+bool emit_kernel_source(KernelSpec* spec, ParseError* err) {
+    KernelSpec& k = *spec;
     std::string body;
-    if (!emit_expr_body(k.expr, dtype, k.consts, &body, err)) return false;
+    if (!emit_expr_body(k.expr, k.dtype, k.consts, &body, err)) return false;
 
     const bool nt_load = k.tuning.nontemporal & 1, nt_store = k.tuning.nontemporal & 2;
 
     std::string s;
-    s += "// generated by custos-hip: " + to_cl_source(k.expr, markers, &k.consts) + "\n";
+    s += "// generated by custos-hip: " + to_cl_source(k.expr, k.markers, &k.consts) + "\n";
     s += "#define CUSTOS_BLOCK " + std::to_string(k.tuning.block_threads) + "\n";
     s += "#define CUSTOS_UNROLL " + std::to_string(k.tuning.unroll) + "\n";
     s += "#define CUSTOS_VEC " + std::to_string(k.vec_elems) + "\n";
     s += nt_load ? "#define CUSTOS_LD(p) __builtin_nontemporal_load(p)\n" : "#define CUSTOS_LD(p) (*(p))\n";
     s += nt_store ? "#define CUSTOS_ST(p, v) __builtin_nontemporal_store(v, p)\n"
                   : "#define CUSTOS_ST(p, v) (*(p) = (v))\n";
-    s += prelude(dtype, k.vec_elems, k.consts.n_params);
+    s += prelude(k.dtype, k.vec_elems, k.consts.n_params);
     s += expr_fn(k, body);
 
     const KernelText text(k);
@@ -456,8 +464,22 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     s += text.ragged_entry();
 
     k.source = std::move(s);
-    *out = std::move(k);
     return true;
+}
+
+bool same_code(const KernelSpec& a, const KernelSpec& b) {
+    if (a.kind != b.kind || a.dtype != b.dtype || a.hash != b.hash) return false;
+    if (a.tuning.block_threads != b.tuning.block_threads || a.tuning.unroll != b.tuning.unroll ||
+        a.tuning.blocks_per_cu != b.tuning.blocks_per_cu || a.tuning.nontemporal != b.tuning.nontemporal ||
+        a.auto_unroll != b.auto_unroll || a.auto_nt != b.auto_nt)
+        return false;
+    if (a.expr.n_vars != b.expr.n_vars || a.expr.root != b.expr.root || a.expr.nodes.size() != b.expr.nodes.size()) return false;
+    for (size_t i = 0; i < a.expr.nodes.size(); i++) {
+        const Node& x = a.expr.nodes[i];
+        const Node& y = b.expr.nodes[i];
+        if (x.op != y.op || x.a != y.a || x.b != y.b || x.var != y.var) return false;
+    }
+    return a.consts.slot == b.consts.slot && a.code_literals == b.code_literals;
 }
 
 }  // namespace custos_hip

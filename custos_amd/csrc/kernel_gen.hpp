@@ -53,10 +53,12 @@ struct KernelSpec {
     bool auto_nt = false;      // launches may use a variant compiled with another choice
     ConstPlan consts;          // literals that are launch parameters, and this text's values for them
     int n_literals = 0;        // literals in the expression, parameters or not
+    std::vector<uint64_t> code_literals;  // values of the literals that stay in the code, in node order
+    std::vector<std::string> markers;     // operand names, for the text
     uint64_t hash = 0;   // cache key: expression without the parameter values, dtype, kind, tuning
     std::string name;    // entry point: custos_<kind>_<dtype>_<hash>, unique per kernel so
                          // that profiler output tells the kernels apart
-    std::string source;  // complete translation unit
+    std::string source;  // complete translation unit (empty until emit_kernel_source)
     int vec_elems = 4;   // elements per 16-byte vector
 };
 
@@ -64,9 +66,16 @@ struct KernelSpec {
 // `literals_in_code`: the kernel for exactly these literal values (the compiler sees them);
 // else the form shared by all expressions that differ only in literal values, which takes
 // them as launch parameters (ConstPlan).
+// `with_source = false` stops before the text is generated (enough for a cache lookup).
 bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
                        const std::vector<std::string>& markers, const Tuning& tuning,
-                       bool literals_in_code, KernelSpec* out, ParseError* err);
+                       bool literals_in_code, KernelSpec* out, ParseError* err, bool with_source = true);
+// Generates `k->source` (which also finds node / element type combinations that cannot be
+// compiled, such as a transcendental node over integers).
+bool emit_kernel_source(KernelSpec* k, ParseError* err);
+// Whether two specs describe the same translation unit, without looking at the text: kind,
+// element type, launch shape, expression structure and the literals that stay in the code.
+bool same_code(const KernelSpec& a, const KernelSpec& b);
 
 // Options handed to hiprtc for every kernel.
 std::vector<std::string> hiprtc_options(const std::string& arch);
