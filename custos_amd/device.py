@@ -14,7 +14,7 @@ import ctypes as C
 import numpy as np
 
 from . import capi
-from .expr import Expr, Resolve, _wrap, fused_source
+from .expr import Resolve, _wrap, fused_source
 
 
 def _np_dtype(dtype: str):

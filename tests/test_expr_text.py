@@ -7,7 +7,7 @@ import numpy as np
 
 import pytest
 
-from custos_amd import Const, Resolve, capi, to_marker, to_val
+from custos_amd import Resolve, capi, to_marker, to_val
 from custos_amd.expr import format_float, fused_source
 
 
