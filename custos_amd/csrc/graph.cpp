@@ -27,8 +27,8 @@ constexpr uint64_t kChunkShift = 21;  // conflict search buckets of 2 MiB
 // A launch of more tiles than this is not merged with launches of other lengths:
 // it fills the chip by itself, and the block map would grow with it.
 constexpr unsigned long long kRaggedMaxTiles = 16384;
-// A recorded graph that touches no more than this keeps its data in the memory-side cache.
-constexpr unsigned long long kCacheWorkingSet = 320ull << 20;
+// A node counts as a producer if one of this many levels after it reads what it writes.
+constexpr size_t kLookAheadLevels = 8;
 
 // Earlier accesses are kept once per distinct (range, mode) with the highest level seen, so
 // a program that runs over the same buffers many times keeps the search lists as short as
@@ -114,34 +114,29 @@ unsigned long long tiles_of(const custos_hip_kernel* k, const RecNode& n) {
     return std::max(1ull, (n.n_vec + tile_vecs - 1) / tile_vecs);
 }
 
-// Everything the graph touches, as the union of the recorded address ranges.  While it
-// fits the memory-side cache (256 MiB, with some slack: a chain over 288 MiB still gains
-// 4 %, over 192 MiB 9.5 %, over 384 MiB nothing, over 1.5 GiB it loses 10 %) and the graph
-// has consumers after producers, every kernel of the graph uses temporal accesses: the next
-// kernel, and the next replay, find the data in the cache.  Caller-written kernels are not
-// counted.
-bool working_set_fits_cache(const std::vector<RecNode>& nodes, int max_level) {
-    if (max_level < 1) return false;
-    std::vector<std::pair<uint64_t, uint64_t>> ranges;
-    for (const RecNode& n : nodes)
-        for (const Access& a : n.acc)
-            if (a.end > a.begin) ranges.push_back({a.begin, a.end});
-    std::sort(ranges.begin(), ranges.end());
-    unsigned long long working_set = 0;
-    uint64_t covered = 0;
-    for (const auto& r : ranges) {
-        const uint64_t from = std::max(r.first, covered);
-        if (r.second > from) working_set += r.second - from;
-        covered = std::max(covered, r.second);
-    }
-    return working_set <= kCacheWorkingSet;
+// Whether a recorded piece of work reads the operand behind one of its accesses (the gradient
+// operand of a unary-gradient kernel is read and written).
+bool reads_operand(const RecNode& n, const Access& a) {
+    return !a.write || (n.type == RecNode::Kernel && n.k->spec.kind == Kind::UnaryGrad);
+}
+
+// The traffic of one level's nodes, for the launch shapes of the levels after it.
+void record_level(const std::vector<RecNode>& nodes, const std::vector<size_t>& of_level, RecentTraffic* history) {
+    std::vector<Access> all;
+    for (size_t i : of_level)
+        if (nodes[i].type != RecNode::Source) all.insert(all.end(), nodes[i].acc.begin(), nodes[i].acc.end());
+    unsigned long long bytes = 0;
+    for (const Access& a : all) bytes += a.end - a.begin;
+    if (bytes >= kTrafficFromBytes) history->record(all);
 }
 
 // The nodes of one dependency level: launches of one kernel are merged (equal lengths into a
 // `_batched` grid, different lengths into a `_ragged` one), everything else stays single.
 // Operand tables and block maps of the merged launches are appended to `host_table`.
 std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNode>& nodes,
-                                const std::vector<size_t>& of_level, bool fits_cache, std::vector<uint64_t>* host_table) {
+                                const std::vector<size_t>& of_level, RecentTraffic* history,
+                                const std::vector<const std::vector<Access>*>& later_reads,
+                                std::vector<uint64_t>* host_table) {
     std::vector<Planned> out;
     // candidates for merging, grouped by kernel in first-seen order
     std::vector<std::pair<custos_hip_kernel*, std::vector<size_t>>> groups;
@@ -197,7 +192,25 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
             // the launch shape follows the bytes the (merged) launch touches
             unsigned long long footprint = 0;
             for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
-            custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, fits_cache);
+            // ... and what the nodes of the levels before left in the memory-side cache
+            // ... and on the launches around it: the levels before, and whether one of the
+            // levels after reads what it writes
+            CacheHint hint = CacheHint::Unknown;
+            if (footprint >= kHintFromBytes) {
+                std::vector<Access> all, reads;
+                bool feeds_later = false;
+                for (size_t i : p.members)
+                    for (const Access& a : nodes[i].acc) {
+                        all.push_back(a);
+                        if (reads_operand(nodes[i], a)) reads.push_back(a);
+                        if (!a.write) continue;
+                        for (const std::vector<Access>* level : later_reads)
+                            for (const Access& r : *level) feeds_later = feeds_later || (r.begin < a.end && a.begin < r.end);
+                    }
+                hint = history->classify(reads, all, feeds_later);
+                dev->hinted[static_cast<int>(hint)]++;
+            }
+            custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, hint);
             const bool usable = p.members.size() == 1 || (p.ragged ? v->fn_ragged != nullptr : v->fn_batched != nullptr);
             p.kern = usable ? v : first.k;
         }
@@ -222,6 +235,7 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
         }
         p.blocks = host_table->size() - p.map_offset;
     }
+    record_level(nodes, of_level, history);
     return out;
 }
 
@@ -346,12 +360,27 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     g->recorded = nodes.size();
     g->levels = static_cast<size_t>(max_level + 1);
 
-    const bool fits_cache = working_set_fits_cache(nodes, max_level);
     std::vector<std::vector<Planned>> plan;
     std::vector<uint64_t> host_table;
     std::vector<std::vector<size_t>> by_level(static_cast<size_t>(max_level + 1));
     for (size_t i = 0; i < nodes.size(); i++) by_level[static_cast<size_t>(nodes[i].level)].push_back(i);
-    for (const auto& of_level : by_level) plan.push_back(plan_level(dev, nodes, of_level, fits_cache, &host_table));
+    // A graph is built to be replayed: its first levels follow its last ones, so the traffic
+    // history starts with one pass over the whole graph.
+    RecentTraffic history;
+    for (const auto& of_level : by_level) record_level(nodes, of_level, &history);
+    // what every level reads, for the producers in the levels before it (the levels after the
+    // last one are the first ones of the next replay)
+    std::vector<std::vector<Access>> level_reads(by_level.size());
+    for (size_t level = 0; level < by_level.size(); level++)
+        for (size_t i : by_level[level])
+            for (const Access& a : nodes[i].acc)
+                if (nodes[i].type != RecNode::Source && reads_operand(nodes[i], a)) level_reads[level].push_back(a);
+    for (size_t level = 0; level < by_level.size(); level++) {
+        std::vector<const std::vector<Access>*> later_reads;
+        for (size_t ahead = 1; ahead <= kLookAheadLevels && ahead <= by_level.size(); ahead++)
+            later_reads.push_back(&level_reads[(level + ahead) % by_level.size()]);
+        plan.push_back(plan_level(dev, nodes, by_level[level], &history, later_reads, &host_table));
+    }
     if (!host_table.empty()) {
         HIP_TRY(dev, hipMalloc(&g->table, host_table.size() * sizeof(uint64_t)));
         HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));

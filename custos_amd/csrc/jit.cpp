@@ -279,10 +279,9 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 }
 
 custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
-                                  bool* alternate, bool working_set_fits_cache) {
+                                  bool* alternate, CacheHint hint) {
     const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;
-    LaunchShape shape = preferred_shape(footprint_bytes, n_operands);
-    if (working_set_fits_cache) shape = {2, 0, false};
+    LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint);
     const int direction = dev->tuning.direction;
     *alternate = direction == 2 || (direction == 0 && shape.alternate);
     if (k->spec.kind == Kind::Source || (!k->spec.auto_unroll && !k->spec.auto_nt)) return k;

@@ -51,11 +51,24 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // 3-9 % when the kernel repeats over the same buffers (1R+1W at 192 MiB: 6959
 // against 6383 GB/s) and in chains over arrays of that size; the exception is the
 // range just above the L2 capacity, 64 to 128 MiB, where non-temporal accesses
-// are ahead (3R+1W at 64 MiB: 6883 against 6343) unless a chain reuses the data
-// (build_graph knows that and overrides).
-LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands) {
+// are ahead (3R+1W at 64 MiB: 6883 against 6343) unless the launch reads what a
+// launch just before it wrote.
+//
+// Chains (a launch reads what the launch before it wrote; 1R+1W kernels, GB/s on 8
+// bytes per element) differ from repeats of one launch: while everything the
+// chain touches fits the memory-side cache, temporal accesses win at every launch
+// size, beyond that one vector per thread with non-temporal accesses does,
+// whatever the direction.  Eager cycle over three arrays of A MiB, u2T / u1T /
+// u2N / u1N: A = 32: 6487 / 6184 / 5348 / 5936; 64: 6777 / 6843 / 5874 / 6686;
+// 100: 6159 / 5955 / 6131 / 6960; 128: 6393 / 6301 / 6219 / 7069; 256: 5957 / 6082 /
+// 6388 / 7294.  Replayed graph of five kernels over six arrays: A = 32 (192 MiB
+// in all): 5887 / 5694 / 4941 / 5363; 64 (384 MiB): 5684 / 5841 / 5607 / 6270;
+// 128: 5597 / 5856 / 6057 / 6776; 256: 5885 / 6032 / 6307 / 6956.
+LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint) {
     constexpr unsigned long long MiB = 1ull << 20;
     if (footprint_bytes < 64 * MiB) return {2, 0, false};
+    if (hint == CacheHint::Resident) return {2, 0, false};
+    if (hint == CacheHint::Streams) return {1, 3, footprint_bytes > 256 * MiB};
     if (footprint_bytes < 128 * MiB) return {2, 3, false};
     if (footprint_bytes <= 256 * MiB) return {2, 0, false};
     const bool one_vector = footprint_bytes >= 768 * MiB || (n_operands >= 3 && footprint_bytes >= 512 * MiB);

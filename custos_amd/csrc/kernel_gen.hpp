@@ -38,7 +38,17 @@ struct LaunchShape {
     int nontemporal;
     bool alternate;  // walk the tiles in the direction opposite to the previous launch
 };
-LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands);
+// What is known about a launch from the address ranges of the launches around it.  A launch
+// that reads what one of the last few launches wrote (or whose output one of the next few
+// reads) is part of a chain; what suits it depends on whether everything those launches touch
+// stays in the memory-side cache (256 MiB).
+enum class CacheHint {
+    Unknown,   // not part of a chain: the launch shape follows the bytes the launch touches
+    Resident,  // the chain's working set fits the cache: temporal accesses
+    Streams,   // it does not: stream past the cache
+};
+constexpr unsigned long long kCacheWorkingSet = 256ull << 20;
+LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint = CacheHint::Unknown);
 
 // Fills unset (zero) fields with the defaults and clamps to legal values
 // (`nontemporal` and `direction` as in custos_hip_tuning).

@@ -5,6 +5,70 @@
 
 #include "runtime.hpp"
 
+// ---- RecentTraffic ----
+
+namespace {
+
+constexpr size_t kTrafficDepth = 8;  // launches looked back at
+
+// Sorted, non-overlapping ranges covering the same addresses; `write` = any writer.
+std::vector<Access> merged(std::vector<Access> ranges) {
+    std::sort(ranges.begin(), ranges.end(), [](const Access& a, const Access& b) { return a.begin < b.begin; });
+    std::vector<Access> out;
+    for (const Access& r : ranges) {
+        if (r.end <= r.begin) continue;
+        if (!out.empty() && r.begin <= out.back().end) {
+            out.back().end = std::max(out.back().end, r.end);
+            out.back().write = out.back().write || r.write;
+        } else {
+            out.push_back(r);
+        }
+    }
+    return out;
+}
+
+unsigned long long total_bytes(const std::vector<Access>& sorted_disjoint) {
+    unsigned long long bytes = 0;
+    for (const Access& r : sorted_disjoint) bytes += r.end - r.begin;
+    return bytes;
+}
+
+}  // namespace
+
+bool RecentTraffic::wrote_any_of(const std::vector<Access>& reads) const {
+    for (const std::vector<Access>& launch : launches_)
+        for (const Access& w : launch) {
+            if (!w.write) continue;
+            for (const Access& r : reads)
+                if (r.begin < w.end && w.begin < r.end) return true;
+        }
+    return false;
+}
+
+unsigned long long RecentTraffic::working_set_with(const std::vector<Access>& all) const {
+    std::vector<Access> touched = all;
+    for (const std::vector<Access>& launch : launches_) touched.insert(touched.end(), launch.begin(), launch.end());
+    return total_bytes(merged(std::move(touched)));
+}
+
+custos_hip::CacheHint RecentTraffic::classify(const std::vector<Access>& reads, const std::vector<Access>& all,
+                                              bool feeds_later) const {
+    if (!feeds_later && !wrote_any_of(reads)) return custos_hip::CacheHint::Unknown;
+    return working_set_with(all) <= custos_hip::kCacheWorkingSet ? custos_hip::CacheHint::Resident
+                                                                  : custos_hip::CacheHint::Streams;
+}
+
+void RecentTraffic::record(const std::vector<Access>& all) {
+    if (launches_.size() == kTrafficDepth) launches_.erase(launches_.begin());
+    // written and read ranges are merged separately, so that the writer flag stays exact
+    std::vector<Access> reads, writes;
+    for (const Access& a : all) (a.write ? writes : reads).push_back(a);
+    std::vector<Access> launch = merged(std::move(writes));
+    const std::vector<Access> r = merged(std::move(reads));
+    launch.insert(launch.end(), r.begin(), r.end());
+    launches_.push_back(std::move(launch));
+}
+
 namespace custos_hip {
 
 namespace {
@@ -81,9 +145,21 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
         dev->recorded.push_back(std::move(node));
         return CUSTOS_HIP_OK;
     }
-    // the launch shape that suits the bytes this launch touches
+    // the launch shape that suits the bytes this launch touches and what the launches just
+    // before it left in the memory-side cache
+    std::vector<Access> all, reads;
+    const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
+    for (const Range& r : ops) {
+        all.push_back({r.ptr, r.ptr + bytes, r.written});
+        // (the gradient operand of a unary-gradient kernel is read and written)
+        if (!r.written || k->spec.kind == Kind::UnaryGrad) reads.push_back(all.back());
+    }
+    const unsigned long long footprint = static_cast<unsigned long long>(ops.size()) * bytes;
+    const CacheHint hint = footprint >= kHintFromBytes ? dev->recent.classify(reads, all) : CacheHint::Unknown;
+    if (footprint >= kTrafficFromBytes) dev->recent.record(all);
+    if (footprint >= kHintFromBytes) dev->hinted[static_cast<int>(hint)]++;
     bool alternate = false;
-    k = kernel_variant(dev, k, static_cast<unsigned long long>(ops.size()) * n * dtype_size(k->spec.dtype), &alternate);
+    k = kernel_variant(dev, k, footprint, &alternate, hint);
     const unsigned int grid = launch_grid(dev, k, n, n_vec);
     unsigned long long rev = alternate ? (dev->launch_parity ^= 1) : 0;
     uint64_t ptrs[8];
@@ -125,6 +201,14 @@ int32_t custos_hip_apply_fn_n(custos_hip_device* dev, custos_hip_kernel* kernel,
     for (int i = 0; i < n_ins; i++) ops.push_back({ins[i], false});
     ops.push_back({out, true});
     return launch_or_record(dev, kernel, ops, n);
+}
+
+int32_t custos_hip_launch_hint_stats(custos_hip_device* dev, uint64_t* unrelated, uint64_t* resident, uint64_t* streaming) {
+    REQUIRE_DEV(dev);
+    if (unrelated) *unrelated = dev->hinted[static_cast<int>(CacheHint::Unknown)];
+    if (resident) *resident = dev->hinted[static_cast<int>(CacheHint::Resident)];
+    if (streaming) *streaming = dev->hinted[static_cast<int>(CacheHint::Streams)];
+    return CUSTOS_HIP_OK;
 }
 
 int32_t custos_hip_apply_fn(custos_hip_device* dev, custos_hip_kernel* kernel, uint64_t x, uint64_t out, size_t n) {

@@ -83,6 +83,28 @@ struct RecNode {
     std::vector<std::vector<unsigned char>> arg_values;
 };
 
+// The address ranges of the last few launches, from which a launch learns whether it reads
+// what one of them wrote and how much was touched since (see CacheHint).
+// Launches below kHintFromBytes take the small-launch shape whatever the cache holds; launches
+// below kTrafficFromBytes are not worth tracking (their kernels are shorter than a launch call).
+constexpr unsigned long long kHintFromBytes = 64ull << 20;
+constexpr unsigned long long kTrafficFromBytes = 8ull << 20;
+class RecentTraffic {
+   public:
+    // Whether one of the recorded launches wrote something in `reads`.
+    bool wrote_any_of(const std::vector<Access>& reads) const;
+    // Distinct bytes touched by the recorded launches and by `all` together.
+    unsigned long long working_set_with(const std::vector<Access>& all) const;
+    void record(const std::vector<Access>& all);
+    // The hint for a launch that reads `reads` and touches `all`; `feeds_later`: it is known
+    // that a launch soon after it reads what it writes.
+    custos_hip::CacheHint classify(const std::vector<Access>& reads, const std::vector<Access>& all,
+                                   bool feeds_later = false) const;
+
+   private:
+    std::vector<std::vector<Access>> launches_;  // oldest first, at most 8, each merged and sorted
+};
+
 struct custos_hip_device {
     int idx = 0;
     hipStream_t stream = nullptr;    // compute stream: every launch, in call order
@@ -95,6 +117,8 @@ struct custos_hip_device {
     int32_t literal_policy = 0;      // CUSTOS_HIP_LITERALS_*
     // per shared-form key: how many distinct texts of that structure were compiled or looked up
     std::unordered_map<uint64_t, uint32_t> value_sets_seen;
+    RecentTraffic recent;            // of the launches issued directly (not recorded)
+    uint64_t hinted[3] = {0, 0, 0};  // launches and graph nodes of at least kHintFromBytes by CacheHint
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     // allocation pool: freed blocks by rounded size; every block this handle allocated, by address
     std::unordered_map<size_t, std::vector<void*>> pool;
@@ -172,11 +196,9 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 // caller left them open).  Never fails: without a variant it returns `k`.
 // `alternate` tells whether the launch should walk the tiles in the direction
 // opposite to the previous launch.
-// `working_set_fits_cache`: the caller knows that everything the surrounding graph touches
-// stays in the memory-side cache between its kernels (temporal accesses then, whatever the
-// size of the single launch).
+// `hint`: what is known about the data the launch reads (see CacheHint).
 custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
-                                  bool* alternate, bool working_set_fits_cache = false);
+                                  bool* alternate, CacheHint hint = CacheHint::Unknown);
 
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);

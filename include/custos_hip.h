@@ -274,10 +274,20 @@ int32_t custos_hip_expr_emit_shared(int32_t kind, int32_t dtype, const char *src
 int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const char *src,
                                           const char *const *markers, int32_t n_markers,
                                           const custos_hip_tuning *tuning, size_t *code_size);
+/* Launches of 64 MiB and more (issued directly, or nodes of built graphs) so far, by what the
+ * address ranges of the launches around them told: not part of a chain (the launch shape
+ * then follows the bytes the launch touches, custos_hip_preferred_shape); part of a chain
+ * -- it reads what one of the last eight launches wrote, or in a graph one of the next
+ * levels reads what it writes -- whose working set stays in the 256 MiB memory-side cache
+ * (temporal accesses, two vectors per thread); part of a chain whose working set does not
+ * (non-temporal accesses, one vector per thread). */
+int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated, uint64_t *resident,
+                                     uint64_t *streaming);
 /* Host-only: the launch shape the library picks for a launch that touches `footprint_bytes`
  * (all operands together) through `n_operands` pointers, for the knobs left at 0 in
  * custos_hip_tuning: vectors per thread, the `nontemporal` bits, and whether the launch
- * walks its tiles against the direction of the previous one. */
+ * walks its tiles against the direction of the previous one -- for a launch that is not part
+ * of a chain (see custos_hip_launch_hint_stats). */
 int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t *unroll,
                                    int32_t *nontemporal, int32_t *alternate);
 /* Canonical re-print of an expression in the reference's ToCLSource format. */

@@ -827,6 +827,52 @@ def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
                 assert_bits_equal(got_g, want_g, f"gradient, {what}")
 
 
+def test_launch_shape_follows_the_launches_around_it(oracle):
+    """A launch of 64 MiB and more that reads what one of the last launches wrote is part of a
+    chain: temporal accesses while the chain's working set stays in the 256 MiB memory-side cache,
+    streaming with one vector per thread beyond that.  Results are the same either way."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        n = 1 << 23                                   # 32 MiB per array
+        x = synth.uniform_f32(3, n, -2, 2)
+        f = lambda v: v.mul(1.5).sub(0.25)
+        g = lambda v: v.abs().add(1.0)
+        a, b, c = dev.buffer(x), dev.alloc(n), dev.alloc(n)
+        base = dev.launch_hint_stats()
+        dev.apply_fn(a, f, out=b)                     # reads what no launch wrote
+        dev.apply_fn(b, g, out=c)                     # consumer after producer, 96 MiB in all
+        dev.apply_fn(c, f, out=b)
+        s1 = dev.launch_hint_stats()
+        assert (s1[0] - base[0], s1[1] - base[1], s1[2] - base[2]) == (1, 2, 0)
+        want = (np.abs(x * np.float32(1.5) - np.float32(0.25)) + np.float32(1.0)) * np.float32(1.5) - np.float32(0.25)
+        assert_bits_equal(b.read(), want)
+        # the same chain over arrays that do not fit: 3 x 128 MiB
+        big = 1 << 25
+        xb = synth.uniform_f32(4, big, -2, 2)
+        p, q, r = dev.buffer(xb), dev.alloc(big), dev.alloc(big)
+        dev.apply_fn(p, f, out=q)
+        dev.apply_fn(q, g, out=r)
+        dev.apply_fn(r, f, out=q)
+        s2 = dev.launch_hint_stats()
+        assert (s2[0] - s1[0], s2[1] - s1[1], s2[2] - s1[2]) == (1, 0, 2)
+        wantb = (np.abs(xb * np.float32(1.5) - np.float32(0.25)) + np.float32(1.0)) * np.float32(1.5) - np.float32(0.25)
+        assert_bits_equal(q.read(), wantb)
+        # in a recorded graph the first kernel counts as part of the chain too: a later level reads its output
+        dev.capture_begin()
+        dev.apply_fn(a, f, out=b)
+        dev.apply_fn(b, g, out=c)
+        graph = dev.capture_end()
+        s3 = dev.launch_hint_stats()
+        assert (s3[0] - s2[0], s3[1] - s2[1], s3[2] - s2[2]) == (0, 2, 0)
+        for _ in range(3):
+            graph.launch()
+        assert_bits_equal(c.read(), np.abs(x * np.float32(1.5) - np.float32(0.25)) + np.float32(1.0))
+        graph.destroy()
+    finally:
+        dev.close()
+
+
 def test_allocation_pool():
     """Freed blocks are handed out again: same address, zero-filled again, ordered behind the
     work that still used them; limit 0 switches the pool off; trim gives everything back."""
