@@ -44,6 +44,7 @@ struct LaunchShape {
 // stays in the memory-side cache (256 MiB).
 enum class CacheHint {
     Unknown,   // not part of a chain: the launch shape follows the bytes the launch touches
+    Crowded,   // not part of a chain, but the launches around it touch more than the cache holds
     Resident,  // the chain's working set fits the cache: temporal accesses
     Streams,   // it does not: stream past the cache
 };

@@ -53,9 +53,9 @@ unsigned long long RecentTraffic::working_set_with(const std::vector<Access>& al
 
 custos_hip::CacheHint RecentTraffic::classify(const std::vector<Access>& reads, const std::vector<Access>& all,
                                               bool feeds_later) const {
-    if (!feeds_later && !wrote_any_of(reads)) return custos_hip::CacheHint::Unknown;
-    return working_set_with(all) <= custos_hip::kCacheWorkingSet ? custos_hip::CacheHint::Resident
-                                                                  : custos_hip::CacheHint::Streams;
+    const bool fits = working_set_with(all) <= custos_hip::kCacheWorkingSet;
+    if (!feeds_later && !wrote_any_of(reads)) return fits ? custos_hip::CacheHint::Unknown : custos_hip::CacheHint::Crowded;
+    return fits ? custos_hip::CacheHint::Resident : custos_hip::CacheHint::Streams;
 }
 
 void RecentTraffic::record(const std::vector<Access>& all) {
@@ -205,7 +205,7 @@ int32_t custos_hip_apply_fn_n(custos_hip_device* dev, custos_hip_kernel* kernel,
 
 int32_t custos_hip_launch_hint_stats(custos_hip_device* dev, uint64_t* unrelated, uint64_t* resident, uint64_t* streaming) {
     REQUIRE_DEV(dev);
-    if (unrelated) *unrelated = dev->hinted[static_cast<int>(CacheHint::Unknown)];
+    if (unrelated) *unrelated = dev->hinted[static_cast<int>(CacheHint::Unknown)] + dev->hinted[static_cast<int>(CacheHint::Crowded)];
     if (resident) *resident = dev->hinted[static_cast<int>(CacheHint::Resident)];
     if (streaming) *streaming = dev->hinted[static_cast<int>(CacheHint::Streams)];
     return CUSTOS_HIP_OK;

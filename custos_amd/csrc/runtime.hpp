@@ -118,7 +118,7 @@ struct custos_hip_device {
     // per shared-form key: how many distinct texts of that structure were compiled or looked up
     std::unordered_map<uint64_t, uint32_t> value_sets_seen;
     RecentTraffic recent;            // of the launches issued directly (not recorded)
-    uint64_t hinted[3] = {0, 0, 0};  // launches and graph nodes of at least kHintFromBytes by CacheHint
+    uint64_t hinted[4] = {0, 0, 0, 0};  // launches and graph nodes of at least kHintFromBytes by CacheHint
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     // allocation pool: freed blocks by rounded size; every block this handle allocated, by address
     std::unordered_map<size_t, std::vector<void*>> pool;
