@@ -147,17 +147,22 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     }
     // the launch shape that suits the bytes this launch touches and what the launches just
     // before it left in the memory-side cache
-    std::vector<Access> all, reads;
     const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
-    for (const Range& r : ops) {
-        all.push_back({r.ptr, r.ptr + bytes, r.written});
-        // (the gradient operand of a unary-gradient kernel is read and written)
-        if (!r.written || k->spec.kind == Kind::UnaryGrad) reads.push_back(all.back());
-    }
     const unsigned long long footprint = static_cast<unsigned long long>(ops.size()) * bytes;
-    const CacheHint hint = footprint >= kHintFromBytes ? dev->recent.classify(reads, all) : CacheHint::Unknown;
-    if (footprint >= kTrafficFromBytes) dev->recent.record(all);
-    if (footprint >= kHintFromBytes) dev->hinted[static_cast<int>(hint)]++;
+    CacheHint hint = CacheHint::Unknown;
+    if (footprint >= kTrafficFromBytes) {
+        std::vector<Access> all, reads;
+        for (const Range& r : ops) {
+            all.push_back({r.ptr, r.ptr + bytes, r.written});
+            // (the gradient operand of a unary-gradient kernel is read and written)
+            if (!r.written || k->spec.kind == Kind::UnaryGrad) reads.push_back(all.back());
+        }
+        if (footprint >= kHintFromBytes) {
+            hint = dev->recent.classify(reads, all);
+            dev->hinted[static_cast<int>(hint)]++;
+        }
+        dev->recent.record(all);
+    }
     bool alternate = false;
     k = kernel_variant(dev, k, footprint, &alternate, hint);
     const unsigned int grid = launch_grid(dev, k, n, n_vec);

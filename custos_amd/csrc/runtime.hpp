@@ -88,7 +88,7 @@ struct RecNode {
 // Launches below kHintFromBytes take the small-launch shape whatever the cache holds; launches
 // below kTrafficFromBytes are not worth tracking (their kernels are shorter than a launch call).
 constexpr unsigned long long kHintFromBytes = 64ull << 20;
-constexpr unsigned long long kTrafficFromBytes = 8ull << 20;
+constexpr unsigned long long kTrafficFromBytes = 32ull << 20;
 class RecentTraffic {
    public:
     // Whether one of the recorded launches wrote something in `reads`.
