@@ -130,19 +130,16 @@ void record_level(const std::vector<RecNode>& nodes, const std::vector<size_t>& 
     if (bytes >= kTrafficFromBytes) history->record(all);
 }
 
-// The nodes of one dependency level: launches of one kernel are merged (equal lengths into a
-// `_batched` grid, different lengths into a `_ragged` one), everything else stays single.
-// Operand tables and block maps of the merged launches are appended to `host_table`.
-std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNode>& nodes,
-                                const std::vector<size_t>& of_level, RecentTraffic* history,
-                                const std::vector<const std::vector<Access>*>& later_reads,
-                                std::vector<uint64_t>* host_table) {
+// The nodes of one dependency level: launches of one kernel (or of one code with different
+// literal values) are merged -- equal lengths into a `_batched` grid, different lengths into a
+// `_ragged` one --, everything else stays single.
+std::vector<Planned> group_level(const custos_hip_device* dev, const std::vector<RecNode>& nodes,
+                                 const std::vector<size_t>& of_level) {
     std::vector<Planned> out;
-    // candidates for merging, grouped by kernel in first-seen order
+    // candidates for merging, grouped by code in first-seen order
     std::vector<std::pair<custos_hip_kernel*, std::vector<size_t>>> groups;
     for (size_t i : of_level) {
         if (dev->batching && batchable(nodes[i])) {
-            // (handles that differ only in the values of their literal parameters share `code`)
             auto g = std::find_if(groups.begin(), groups.end(), [&](const auto& kv) { return kv.first == nodes[i].k->code; });
             if (g == groups.end()) {
                 groups.push_back({nodes[i].k->code, {}});
@@ -186,54 +183,73 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
         merged.ragged = merged.members.size() > 1;
         if (!merged.members.empty()) out.push_back(std::move(merged));
     }
+    return out;
+}
+
+// What the launches around a (merged) kernel node say about it: the levels before it (`history`),
+// and whether one of the levels after it reads what it writes (`later_reads`).
+CacheHint hint_for(const std::vector<RecNode>& nodes, const Planned& p, const RecentTraffic& history,
+                   const std::vector<const std::vector<Access>*>& later_reads) {
+    std::vector<Access> all, reads;
+    bool feeds_later = false;
+    for (size_t i : p.members)
+        for (const Access& a : nodes[i].acc) {
+            all.push_back(a);
+            if (reads_operand(nodes[i], a)) reads.push_back(a);
+            if (!a.write) continue;
+            for (const std::vector<Access>* level : later_reads)
+                for (const Access& r : *level) feeds_later = feeds_later || (r.begin < a.end && a.begin < r.end);
+        }
+    return history.classify(reads, all, feeds_later);
+}
+
+// Table rows of a merged launch: per member its operand addresses, for a ragged launch its
+// length, then its literal parameters padded to whole words; after the rows of a ragged
+// launch the block map (segment << 32 | tile per workgroup).
+void append_tables(const std::vector<RecNode>& nodes, Planned* p, std::vector<uint64_t>* host_table) {
+    p->table_offset = host_table->size();
+    for (size_t member : p->members) {
+        for (uint64_t ptr : nodes[member].ptrs) host_table->push_back(ptr);
+        if (p->ragged) host_table->push_back(nodes[member].n);
+        const std::vector<unsigned char>& values = nodes[member].k->spec.consts.bytes;
+        for (size_t at = 0; at < values.size(); at += 8) {
+            uint64_t word = 0;
+            std::memcpy(&word, values.data() + at, std::min<size_t>(8, values.size() - at));
+            host_table->push_back(word);
+        }
+    }
+    if (!p->ragged) return;
+    p->map_offset = host_table->size();
+    for (size_t seg = 0; seg < p->members.size(); seg++) {
+        const unsigned long long tiles = tiles_of(p->kern, nodes[p->members[seg]]);
+        for (unsigned long long t = 0; t < tiles; t++) host_table->push_back(static_cast<uint64_t>(seg) << 32 | t);
+    }
+    p->blocks = host_table->size() - p->map_offset;
+}
+
+// Plans one level: merging, the kernel variant of every kernel node, the tables of the merged
+// launches (appended to `host_table`); then the level's traffic joins `history`.
+std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNode>& nodes,
+                                const std::vector<size_t>& of_level, RecentTraffic* history,
+                                const std::vector<const std::vector<Access>*>& later_reads,
+                                std::vector<uint64_t>* host_table) {
+    std::vector<Planned> out = group_level(dev, nodes, of_level);
     for (Planned& p : out) {
         const RecNode& first = nodes[p.members[0]];
         if (first.type == RecNode::Kernel) {
-            // the launch shape follows the bytes the (merged) launch touches
+            // the launch shape follows the bytes the (merged) launch touches and the launches around it
             unsigned long long footprint = 0;
             for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
-            // ... and what the nodes of the levels before left in the memory-side cache
-            // ... and on the launches around it: the levels before, and whether one of the
-            // levels after reads what it writes
             CacheHint hint = CacheHint::Unknown;
             if (footprint >= kHintFromBytes) {
-                std::vector<Access> all, reads;
-                bool feeds_later = false;
-                for (size_t i : p.members)
-                    for (const Access& a : nodes[i].acc) {
-                        all.push_back(a);
-                        if (reads_operand(nodes[i], a)) reads.push_back(a);
-                        if (!a.write) continue;
-                        for (const std::vector<Access>* level : later_reads)
-                            for (const Access& r : *level) feeds_later = feeds_later || (r.begin < a.end && a.begin < r.end);
-                    }
-                hint = history->classify(reads, all, feeds_later);
+                hint = hint_for(nodes, p, *history, later_reads);
                 dev->hinted[static_cast<int>(hint)]++;
             }
             custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, hint);
             const bool usable = p.members.size() == 1 || (p.ragged ? v->fn_ragged != nullptr : v->fn_batched != nullptr);
             p.kern = usable ? v : first.k;
         }
-        if (p.members.size() < 2) continue;
-        p.table_offset = host_table->size();
-        for (size_t member : p.members) {
-            for (uint64_t ptr : nodes[member].ptrs) host_table->push_back(ptr);
-            if (p.ragged) host_table->push_back(nodes[member].n);
-            // the member's literal parameters, padded to whole words
-            const std::vector<unsigned char>& values = nodes[member].k->spec.consts.bytes;
-            for (size_t at = 0; at < values.size(); at += 8) {
-                uint64_t word = 0;
-                std::memcpy(&word, values.data() + at, std::min<size_t>(8, values.size() - at));
-                host_table->push_back(word);
-            }
-        }
-        if (!p.ragged) continue;
-        p.map_offset = host_table->size();
-        for (size_t seg = 0; seg < p.members.size(); seg++) {
-            const unsigned long long tiles = tiles_of(p.kern, nodes[p.members[seg]]);
-            for (unsigned long long t = 0; t < tiles; t++) host_table->push_back(static_cast<uint64_t>(seg) << 32 | t);
-        }
-        p.blocks = host_table->size() - p.map_offset;
+        if (p.members.size() > 1) append_tables(nodes, &p, host_table);
     }
     record_level(nodes, of_level, history);
     return out;
