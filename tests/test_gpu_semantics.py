@@ -873,6 +873,31 @@ def test_launch_shape_follows_the_launches_around_it(oracle):
         dev.close()
 
 
+def test_more_than_two_to_the_32_elements(hip):
+    """Indices are 64-bit throughout: 2^32 + 5 one-byte elements (4 GiB in, 4 GiB out), launched
+    directly and from a replayed graph; windows around 2^31, 2^32 and the scalar tail."""
+    n = (1 << 32) + 5
+    x = hip.alloc(n, "u8")
+    pat = (np.arange(1 << 20, dtype=np.uint32) * 7 % 251).astype(np.uint8)
+    starts = (0, (1 << 31) - 4096, (1 << 32) - (3 << 20), n - (1 << 20))
+    for start in starts:
+        x.slice(start, start + (1 << 20)).write(pat)
+    want = (pat.astype(np.uint32) * 3 + 1).astype(np.uint8)
+    f = lambda v: v.mul(3).add(1)
+    out = hip.apply_fn(x, f)
+    for start in starts:
+        assert_bits_equal(out.slice(start, start + (1 << 20)).read(), want, f"window at {start}")
+    assert np.all(out.slice(3 << 30, (3 << 30) + 4096).read() == 1)
+    out.slice(n - 4096, n).clear()
+    hip.capture_begin()
+    hip.apply_fn(x, f, out=out)
+    graph = hip.capture_end()
+    graph.launch()
+    graph.launch()                       # the second replay walks the tiles the other way round
+    assert_bits_equal(out.slice(n - (1 << 20), n).read(), want, "tail after replays")
+    graph.destroy()
+
+
 def test_allocation_pool():
     """Freed blocks are handed out again: same address, zero-filled again, ordered behind the
     work that still used them; limit 0 switches the pool off; trim gives everything back."""
