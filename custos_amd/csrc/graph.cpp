@@ -241,11 +241,14 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
             unsigned long long footprint = 0;
             for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
             CacheHint hint = CacheHint::Unknown;
+            int keep_loads = 0;
             if (footprint >= kHintFromBytes) {
                 hint = hint_for(nodes, p, *history, later_reads);
                 dev->hinted[static_cast<int>(hint)]++;
+                if (p.members.size() == 1) keep_loads = hot_operands(*history, first.acc, hint);
+                dev->kept_loads += keep_loads != 0;
             }
-            custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, hint);
+            custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, hint, keep_loads);
             const bool usable = p.members.size() == 1 || (p.ragged ? v->fn_ragged != nullptr : v->fn_batched != nullptr);
             p.kern = usable ? v : first.k;
         }

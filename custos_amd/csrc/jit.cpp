@@ -279,7 +279,7 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 }
 
 custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
-                                  bool* alternate, CacheHint hint) {
+                                  bool* alternate, CacheHint hint, int keep_loads) {
     const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;
     LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint);
     const int direction = dev->tuning.direction;
@@ -287,9 +287,9 @@ custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, 
     if (k->spec.kind == Kind::Source || (!k->spec.auto_unroll && !k->spec.auto_nt)) return k;
     Tuning t = k->spec.tuning;
     if (k->spec.auto_unroll) t.unroll = shape.unroll;
-    if (k->spec.auto_nt) t.nontemporal = shape.nontemporal;
+    if (k->spec.auto_nt) t.nontemporal = shape.nontemporal | ((shape.nontemporal & 1) ? (keep_loads & 15) << 2 : 0);
     if (t.unroll == k->spec.tuning.unroll && t.nontemporal == k->spec.tuning.nontemporal) return k;
-    const int key = t.unroll * 8 + t.nontemporal;
+    const int key = t.unroll * 64 + t.nontemporal;
     for (const auto& v : k->variants)
         if (v.first == key) return v.second ? v.second : k;
     std::vector<const char*> m;

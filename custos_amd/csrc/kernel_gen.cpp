@@ -64,6 +64,11 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // 6388 / 7294.  Replayed graph of five kernels over six arrays: A = 32 (192 MiB
 // in all): 5887 / 5694 / 4941 / 5363; 64 (384 MiB): 5684 / 5841 / 5607 / 6270;
 // 128: 5597 / 5856 / 6057 / 6776; 256: 5885 / 6032 / 6307 / 6956.
+// An operand that every kernel of a streaming chain reads again (and nobody
+// writes) keeps temporal loads while the rest streams (bits 2.. of the policy,
+// launch.cpp hot_operands): five 2R+1W kernels with one shared operand over
+// arrays of 64 / 100 MiB 6626 / 6848 against 6082 / 6457 without, and against
+// 6607 / 6501 for the best uniform shape.
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint) {
     constexpr unsigned long long MiB = 1ull << 20;
     if (footprint_bytes < 64 * MiB) return {2, 0, false};
@@ -289,7 +294,7 @@ struct KernelText {
         s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
         for (int i = 0; i < n_ops; i++) {
             const std::string id = std::to_string(i);
-            s += "            a" + id + "[u] = CUSTOS_LD(vin" + id + " + base + (u64)u * CUSTOS_BLOCK);\n";
+            s += "            a" + id + "[u] = CUSTOS_LD" + id + "(vin" + id + " + base + (u64)u * CUSTOS_BLOCK);\n";
         }
         s += "        }\n";
         s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
@@ -302,7 +307,7 @@ struct KernelText {
         s += "            if (idx < n_vec) {\n";
         for (int i = 0; i < n_ops; i++) {
             const std::string id = std::to_string(i);
-            s += "                const vec_t b" + id + " = CUSTOS_LD(vin" + id + " + idx);\n";
+            s += "                const vec_t b" + id + " = CUSTOS_LD" + id + "(vin" + id + " + idx);\n";
         }
         s += "                vec_t r;\n#pragma unroll\n                for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
              list("b", "[k]") + " CUSTOS_KC_ARG);\n";
@@ -436,7 +441,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
     int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 11 /* template version */};
+                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 12 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -466,7 +471,13 @@ bool emit_kernel_source(KernelSpec* spec, ParseError* err) {
     s += "#define CUSTOS_BLOCK " + std::to_string(k.tuning.block_threads) + "\n";
     s += "#define CUSTOS_UNROLL " + std::to_string(k.tuning.unroll) + "\n";
     s += "#define CUSTOS_VEC " + std::to_string(k.vec_elems) + "\n";
-    s += nt_load ? "#define CUSTOS_LD(p) __builtin_nontemporal_load(p)\n" : "#define CUSTOS_LD(p) (*(p))\n";
+    // one load macro per operand: with non-temporal loads, the operands named in bits 2.. of
+    // the policy are still loaded temporally (an operand that the launches around this one
+    // read again and again stays cached while the rest streams)
+    for (int i = 0; i < 4; i++) {
+        const bool nt = nt_load && !((k.tuning.nontemporal >> (2 + i)) & 1);
+        s += "#define CUSTOS_LD" + std::to_string(i) + (nt ? "(p) __builtin_nontemporal_load(p)\n" : "(p) (*(p))\n");
+    }
     s += nt_store ? "#define CUSTOS_ST(p, v) __builtin_nontemporal_store(v, p)\n"
                   : "#define CUSTOS_ST(p, v) (*(p) = (v))\n";
     s += prelude(k.dtype, k.vec_elems, k.consts.n_params);

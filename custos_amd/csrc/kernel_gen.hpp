@@ -27,7 +27,8 @@ struct Tuning {
     int block_threads = 128;
     int unroll = 0;         // 16-byte vectors per thread and tile; 0: chosen per launch
     int blocks_per_cu = 0;  // <= 0: one tile per workgroup
-    int nontemporal = -1;   // bit 0 loads, bit 1 stores; -1: chosen per launch
+    int nontemporal = -1;   // bit 0 loads, bit 1 stores; -1: chosen per launch.  Bits 2..5 (set by the
+                            // library only): operand 0..3 is loaded temporally although bit 0 is set
     int direction = 0;      // 1: tiles first to last; 2: every launch the other way round; 0: chosen per launch
 };
 

@@ -100,6 +100,8 @@ class RecentTraffic {
     // that a launch soon after it reads what it writes.
     custos_hip::CacheHint classify(const std::vector<Access>& reads, const std::vector<Access>& all,
                                    bool feeds_later = false) const;
+    // Whether the recorded launches only ever read `range`, and at least `times` of them do.
+    bool read_only_by(const Access& range, int times) const;
 
    private:
     std::vector<std::vector<Access>> launches_;  // oldest first, at most 8, each merged and sorted
@@ -118,7 +120,8 @@ struct custos_hip_device {
     // per shared-form key: how many distinct texts of that structure were compiled or looked up
     std::unordered_map<uint64_t, uint32_t> value_sets_seen;
     RecentTraffic recent;            // of the launches issued directly (not recorded)
-    uint64_t hinted[4] = {0, 0, 0, 0};  // launches and graph nodes of at least kHintFromBytes by CacheHint
+    uint64_t hinted[4] = {0, 0, 0, 0};
+    uint64_t kept_loads = 0;         // of those, launches that keep an operand's loads temporal while streaming  // launches and graph nodes of at least kHintFromBytes by CacheHint
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     // allocation pool: freed blocks by rounded size; every block this handle allocated, by address
     std::unordered_map<size_t, std::vector<void*>> pool;
@@ -197,11 +200,16 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 // `alternate` tells whether the launch should walk the tiles in the direction
 // opposite to the previous launch.
 // `hint`: what is known about the data the launch reads (see CacheHint).
+// `keep_loads`: bit i = operand i is read by the launches around this one again and again;
+// where the launch streams, that operand is still loaded temporally.
 custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
-                                  bool* alternate, CacheHint hint = CacheHint::Unknown);
+                                  bool* alternate, CacheHint hint = CacheHint::Unknown, int keep_loads = 0);
 
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
+// The operands of a launch (in pointer-parameter order, `all`) that `kernel_variant` should keep
+// loading temporally, given what the launches before it did with them.
+int hot_operands(const RecentTraffic& recent, const std::vector<Access>& all, CacheHint hint);
 // Workgroups of a single launch of `k` over n_vec vectors and n elements.
 unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
                          unsigned long long n_vec);

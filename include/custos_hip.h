@@ -280,9 +280,12 @@ int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const cha
  * -- it reads what one of the last eight launches wrote, or in a graph one of the next
  * levels reads what it writes -- whose working set stays in the 256 MiB memory-side cache
  * (temporal accesses, two vectors per thread); part of a chain whose working set does not
- * (non-temporal accesses, one vector per thread). */
+ * (non-temporal accesses, one vector per thread).  `*kept_operand`: how many of the streaming
+ * ones still load one of their operands temporally, because the launches before them read
+ * that operand again and again and never wrote it (a weight that every kernel of a chain
+ * multiplies by stays cached while the activations stream). */
 int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated, uint64_t *resident,
-                                     uint64_t *streaming);
+                                     uint64_t *streaming, uint64_t *kept_operand);
 /* Host-only: the launch shape the library picks for a launch that touches `footprint_bytes`
  * (all operands together) through `n_operands` pointers, for the knobs left at 0 in
  * custos_hip_tuning: vectors per thread, the `nontemporal` bits, and whether the launch

@@ -449,7 +449,9 @@ def test_launch_shape_variants_of_shared_code(hip):
         assert_bits_equal(out.read(), want, f"graph {step}")
         graph.destroy()
     c1, _ = hip.cache_stats()
-    assert c1 - c0 == 4 and len(names) == 2       # (values in the code, shared form) x (small shape, this shape)
+    # (values in the code, shared form) x (small shape, this size's shape, and the shape that keeps
+    # loading x temporally once the launches before have read it twice) -- not one per set of values
+    assert 4 <= c1 - c0 <= 6 and len(names) == 2
 
 
 def test_error_paths(hip):
@@ -844,7 +846,7 @@ def test_launch_shape_follows_the_launches_around_it(oracle):
         dev.apply_fn(b, g, out=c)                     # consumer after producer, 96 MiB in all
         dev.apply_fn(c, f, out=b)
         s1 = dev.launch_hint_stats()
-        assert (s1[0] - base[0], s1[1] - base[1], s1[2] - base[2]) == (1, 2, 0)
+        assert (s1[0] - base[0], s1[1] - base[1], s1[2] - base[2], s1[3] - base[3]) == (1, 2, 0, 0)
         want = (np.abs(x * np.float32(1.5) - np.float32(0.25)) + np.float32(1.0)) * np.float32(1.5) - np.float32(0.25)
         assert_bits_equal(b.read(), want)
         # the same chain over arrays that do not fit: 3 x 128 MiB
@@ -858,6 +860,17 @@ def test_launch_shape_follows_the_launches_around_it(oracle):
         assert (s2[0] - s1[0], s2[1] - s1[1], s2[2] - s1[2]) == (1, 0, 2)
         wantb = (np.abs(xb * np.float32(1.5) - np.float32(0.25)) + np.float32(1.0)) * np.float32(1.5) - np.float32(0.25)
         assert_bits_equal(q.read(), wantb)
+        # a streaming chain whose kernels all read one more array: that operand stays cached
+        w = dev.buffer(synth.uniform_f32(5, big, 0.5, 1.5))
+        mul = lambda u, v: u.mul(v)
+        for _ in range(2):
+            dev.apply_fn2(q, w, mul, out=r)
+            dev.apply_fn2(r, w, mul, out=q)
+        s2b = dev.launch_hint_stats()
+        assert s2b[2] - s2[2] == 4 and s2b[3] - s2[3] == 2            # from the third launch on, w has been read twice
+        wb = synth.uniform_f32(5, big, 0.5, 1.5)
+        assert_bits_equal(q.read(), ((((wantb * wb) * wb) * wb) * wb))
+        s2 = s2b
         # in a recorded graph the first kernel counts as part of the chain too: a later level reads its output
         dev.capture_begin()
         dev.apply_fn(a, f, out=b)
