@@ -8,6 +8,7 @@
 // computes happens in the library; nothing is evaluated on the host.
 #pragma once
 
+#include <array>
 #include <cstdint>
 #include <cstring>
 #include <functional>
@@ -245,6 +246,13 @@ class HIP : public Device<HIP<Mods>, Mods> {
         uint64_t compiles = 0, hits = 0;
         custos_hip_cache_stats(dev_, &compiles, &hits);
         return {compiles, hits};
+    }
+    // Launches and graph nodes of 64 MiB and more so far: {not part of a chain, chain that stays in the
+    // memory-side cache, chain that streams, streaming with one operand kept cached}.
+    std::array<uint64_t, 4> launch_hint_stats() const {
+        std::array<uint64_t, 4> s{};
+        custos_hip_launch_hint_stats(dev_, &s[0], &s[1], &s[2], &s[3]);
+        return s;
     }
     // Longest recorded chain that is replayed as plain launches instead of a graph launch.
     void set_graph_direct_replay(int32_t max_nodes) { check(custos_hip_set_graph_direct_replay(dev_, max_nodes)); }
