@@ -245,7 +245,9 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
             if (footprint >= kHintFromBytes) {
                 hint = hint_for(nodes, p, *history, later_reads);
                 dev->hinted[static_cast<int>(hint)]++;
-                if (p.members.size() == 1) keep_loads = hot_operands(*history, first.acc, hint);
+                std::vector<const std::vector<Access>*> member_accesses;
+                for (size_t i : p.members) member_accesses.push_back(&nodes[i].acc);
+                keep_loads = hot_operands(*history, member_accesses, hint);
                 dev->kept_loads += keep_loads != 0;
             }
             custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, hint, keep_loads);

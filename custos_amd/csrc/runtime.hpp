@@ -207,9 +207,10 @@ custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, 
 
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
-// The operands of a launch (in pointer-parameter order, `all`) that `kernel_variant` should keep
-// loading temporally, given what the launches before it did with them.
-int hot_operands(const RecentTraffic& recent, const std::vector<Access>& all, CacheHint hint);
+// The operands (bit i = i-th pointer parameter) that `kernel_variant` should keep loading
+// temporally, given what the launches before did with them; `members`: the access lists of the
+// launches merged into this one, each in parameter order.
+int hot_operands(const RecentTraffic& recent, const std::vector<const std::vector<Access>*>& members, CacheHint hint);
 // Workgroups of a single launch of `k` over n_vec vectors and n elements.
 unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
                          unsigned long long n_vec);
