@@ -39,8 +39,11 @@ ERR_COMPILE = 10020
 ERR_KIND_MISMATCH = 10030
 ERR_ARITY_MISMATCH = 10031
 ERR_CAPTURE_STATE = 10040
+ERR_GRAPH_ORDER = 10041
 ERR_BAD_OVERLAP = 10050
 ERR_TOO_LARGE = 10060
+
+GRAPH_EDGES_LEVEL_JOINS, GRAPH_EDGES_PER_NODE, GRAPH_EDGES_CHAIN = 0, 1, 2
 
 
 class CustosHipError(RuntimeError):
@@ -141,6 +144,9 @@ PROTOTYPES = {
     "custos_hip_graph_stats": (C.c_int32, [_P, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "custos_hip_set_graph_batching": (C.c_int32, [_P, C.c_int32]),
     "custos_hip_set_graph_direct_replay": (C.c_int32, [_P, C.c_int32]),
+    "custos_hip_set_graph_edges": (C.c_int32, [_P, C.c_int32]),
+    "custos_hip_set_graph_verify": (C.c_int32, [_P, C.c_int32]),
+    "custos_hip_graph_edge_count": (C.c_int32, [_P, C.POINTER(C.c_size_t)]),
     "custos_hip_graph_destroy": (C.c_int32, [_P, _P]),
     "custos_hip_timer_begin": (C.c_int32, [_P]),
     "custos_hip_timer_end": (C.c_int32, [_P, C.POINTER(C.c_double)]),

@@ -16,12 +16,15 @@ namespace {
 // dependency level: one more than the highest level among earlier nodes whose
 // memory it conflicts with (read-after-write, write-after-read or
 // write-after-write on overlapping address ranges).  Nodes of one level are
-// independent of each other, so they run side by side in the graph, and kernel
-// launches of one level that use the same kernel are merged into ONE grid that
-// walks a table of operand addresses (equal lengths: segment = block / tiles
-// per segment; different lengths: a block map names segment and tile of every
-// workgroup).  1024 small buffers with three operations each become three
-// kernel nodes instead of 3072.
+// independent of each other, so kernel launches of one level that use the same
+// kernel are merged into ONE grid that walks a table of operand addresses
+// (equal lengths: segment = block / tiles per segment; different lengths: a
+// block map names segment and tile of every workgroup).  1024 small buffers
+// with three operations each become three kernel nodes instead of 3072.  The
+// merged nodes are then ordered as one chain in level order (the default: a
+// dependency between branches of a graph costs several times what a node of a
+// chain costs, and an element-wise launch of any size fills the chip alone), by
+// an edge per dependency, or by joins between levels.
 
 constexpr uint64_t kChunkShift = 21;  // conflict search buckets of 2 MiB
 // A launch of more tiles than this is not merged with launches of other lengths:
@@ -33,11 +36,18 @@ constexpr size_t kLookAheadLevels = 8;
 // Earlier accesses are kept once per distinct (range, mode) with the highest level seen, so
 // a program that runs over the same buffers many times keeps the search lists as short as
 // a single pass does; the lists hang off the 2 MiB address chunks a range touches.
-void assign_levels(std::vector<RecNode>& nodes) {
+//
+// With `edges`, every node also gets the recorded nodes it has to wait for (`deps`).  An entry
+// then names the nodes a later conflicting access must follow: for a written range its last
+// writer (earlier writers of the same range precede it already), for a read range the readers
+// since the last write that covered it.  A write that covers an entry entirely takes over from
+// it: whatever conflicts with the entry later conflicts with that write too.
+void assign_levels(std::vector<RecNode>& nodes, bool edges) {
     struct Seen {
         uint64_t begin, end;
         bool write;
         int level;
+        std::vector<uint32_t> users;
     };
     struct Key {
         uint64_t begin, end;
@@ -53,15 +63,19 @@ void assign_levels(std::vector<RecNode>& nodes) {
     std::vector<Seen> seen;
     std::unordered_map<Key, uint32_t, KeyHash> known;
     std::unordered_map<uint64_t, std::vector<uint32_t>> buckets;
+    std::vector<uint32_t> covered;
     int highest = -1;  // highest level so far
     int fence = -1;    // level of the last node with unknown memory use
-    for (RecNode& node : nodes) {
+    for (size_t index = 0; index < nodes.size(); index++) {
+        RecNode& node = nodes[index];
+        node.deps.clear();
         int level = fence + 1;
         if (node.type == RecNode::Source) {
             // unknown reads and writes: after everything before, before everything after
             node.level = fence = highest = highest + 1;
             continue;
         }
+        covered.clear();
         for (const Access& a : node.acc) {
             if (a.end <= a.begin) continue;
             for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) {
@@ -69,22 +83,34 @@ void assign_levels(std::vector<RecNode>& nodes) {
                 if (it == buckets.end()) continue;
                 for (uint32_t si : it->second) {
                     const Seen& s = seen[si];
-                    if (s.level < level) continue;        // cannot raise the level any more
-                    if (!a.write && !s.write) continue;   // two reads never conflict
-                    if (a.begin < s.end && s.begin < a.end) level = s.level + 1;
+                    if (!edges && s.level < level) continue;  // cannot raise the level any more
+                    if (!a.write && !s.write) continue;       // two reads never conflict
+                    if (!(a.begin < s.end && s.begin < a.end)) continue;
+                    level = std::max(level, s.level + 1);
+                    if (!edges) continue;
+                    node.deps.insert(node.deps.end(), s.users.begin(), s.users.end());
+                    if (a.write && a.begin <= s.begin && s.end <= a.end && !s.users.empty()) covered.push_back(si);
                 }
             }
         }
         node.level = level;
         highest = std::max(highest, level);
+        if (edges) {
+            std::sort(node.deps.begin(), node.deps.end());
+            node.deps.erase(std::unique(node.deps.begin(), node.deps.end()), node.deps.end());
+            for (uint32_t si : covered) seen[si].users.clear();
+        }
         for (const Access& a : node.acc) {
             if (a.end <= a.begin) continue;
             auto [slot, fresh] = known.try_emplace(Key{a.begin, a.end, a.write}, static_cast<uint32_t>(seen.size()));
             if (!fresh) {
-                seen[slot->second].level = std::max(seen[slot->second].level, level);
+                Seen& s = seen[slot->second];
+                s.level = std::max(s.level, level);
+                if (edges && (s.users.empty() || s.users.back() != index)) s.users.push_back(static_cast<uint32_t>(index));
                 continue;
             }
-            seen.push_back({a.begin, a.end, a.write, level});
+            seen.push_back({a.begin, a.end, a.write, level, {}});
+            if (edges) seen.back().users.push_back(static_cast<uint32_t>(index));
             for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) buckets[c].push_back(slot->second);
         }
     }
@@ -331,20 +357,119 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
     return CUSTOS_HIP_OK;
 }
 
-// The levels as an instantiated hipGraph: the nodes of a level side by side, one empty join
-// node between levels instead of |previous| x |level| edges.
-int32_t instantiate(custos_hip_device* dev, custos_hip_graph* g, std::vector<std::vector<LoweredNode>>& lowered) {
+// What every node of the graph to be waits for, as indices into the nodes in level order.
+// Level joins: a node waits for the whole level before it (`join_levels`).  Per-node edges: a
+// node waits for the nodes that hold the recorded work its members conflict with; a node with
+// unknown memory use waits for everything before it that nothing waits for yet, and everything
+// after it waits for it, directly or through a node that does.
+std::vector<std::vector<uint32_t>> node_edges(const std::vector<RecNode>& nodes, const std::vector<std::vector<Planned>>& plan) {
+    std::vector<uint32_t> planned_of(nodes.size(), 0);
+    uint32_t id = 0;
+    for (const auto& level : plan)
+        for (const Planned& p : level) {
+            for (size_t m : p.members) planned_of[m] = id;
+            id++;
+        }
+    std::vector<std::vector<uint32_t>> waits(id);
+    std::vector<char> waited_for(id, 0);
+    int64_t fence = -1;  // the last node with unknown memory use
+    id = 0;
+    for (const auto& level : plan)
+        for (const Planned& p : level) {
+            std::vector<uint32_t>& w = waits[id];
+            if (nodes[p.members[0]].type == RecNode::Source) {
+                for (uint32_t q = fence < 0 ? 0 : static_cast<uint32_t>(fence); q < id; q++)
+                    if (!waited_for[q]) w.push_back(q);
+                fence = id;
+            } else {
+                for (size_t m : p.members)
+                    for (uint32_t d : nodes[m].deps) w.push_back(planned_of[d]);
+                std::sort(w.begin(), w.end());
+                w.erase(std::unique(w.begin(), w.end()), w.end());
+                if (fence >= 0) {
+                    // everything before the fence precedes it; the fence itself is waited for
+                    // unless a node that follows it is
+                    w.erase(w.begin(), std::lower_bound(w.begin(), w.end(), static_cast<uint32_t>(fence)));
+                    if (w.empty()) w.push_back(static_cast<uint32_t>(fence));
+                }
+            }
+            for (uint32_t q : w) waited_for[q] = 1;
+            id++;
+        }
+    return waits;
+}
+
+// Brute-force check of a built graph's ordering, independent of how the edges were found: every
+// two recorded pieces of work that touch overlapping memory, one of them writing (or one of
+// them with unknown memory use), must sit in different nodes with a path from the earlier one's
+// node to the later one's.  Quadratic in the recorded work; for tests.
+bool ordering_holds(const std::vector<RecNode>& nodes, const std::vector<std::vector<Planned>>& plan,
+                    const std::vector<std::vector<uint32_t>>& waits) {
+    std::vector<uint32_t> planned_of(nodes.size(), 0);
+    uint32_t count = 0;
+    for (const auto& level : plan)
+        for (const Planned& p : level) {
+            for (size_t m : p.members) planned_of[m] = count;
+            count++;
+        }
+    // reach[b][a]: node a runs before node b.  Nodes only wait for nodes made before them.
+    std::vector<std::vector<char>> reach(count, std::vector<char>(count, 0));
+    for (uint32_t b = 0; b < count; b++)
+        for (uint32_t a : waits[b]) {
+            if (a >= b) return false;
+            reach[b][a] = 1;
+            for (uint32_t c = 0; c < a; c++) reach[b][c] = reach[b][c] | reach[a][c];
+        }
+    auto conflict = [](const RecNode& x, const RecNode& y) {
+        if (x.type == RecNode::Source || y.type == RecNode::Source) return true;
+        for (const Access& a : x.acc)
+            for (const Access& b : y.acc)
+                if ((a.write || b.write) && a.begin < b.end && b.begin < a.end && a.begin < a.end && b.begin < b.end) return true;
+        return false;
+    };
+    for (size_t j = 0; j < nodes.size(); j++)
+        for (size_t i = 0; i < j; i++)
+            if (conflict(nodes[i], nodes[j]) && !reach[planned_of[j]][planned_of[i]]) return false;
+    return true;
+}
+
+// The waits of level joins, in the form node_edges gives: everything of the level before.
+std::vector<std::vector<uint32_t>> level_waits(const std::vector<std::vector<Planned>>& plan) {
+    std::vector<std::vector<uint32_t>> waits;
+    uint32_t first_of_previous = 0, first_of_this = 0;
+    for (const auto& level : plan) {
+        for (size_t k = 0; k < level.size(); k++) {
+            waits.emplace_back();
+            for (uint32_t q = first_of_previous; q < first_of_this; q++) waits.back().push_back(q);
+        }
+        first_of_previous = first_of_this;
+        first_of_this += static_cast<uint32_t>(level.size());
+    }
+    return waits;
+}
+
+// The plan as an instantiated hipGraph.  With level joins the nodes of a level sit side by side
+// behind one empty node that waits for the level before (instead of |previous| x |level|
+// edges); with per-node edges (`waits`) every node follows exactly what it conflicts with.
+int32_t instantiate(custos_hip_device* dev, custos_hip_graph* g, std::vector<std::vector<LoweredNode>>& lowered,
+                    const std::vector<std::vector<uint32_t>>* waits) {
     HIP_TRY(dev, hipGraphCreate(&g->graph, 0));
-    std::vector<hipGraphNode_t> prev;  // what the nodes of the current level wait for
+    std::vector<hipGraphNode_t> prev;  // level joins: what the nodes of the current level wait for
+    std::vector<hipGraphNode_t> all;   // per-node edges: every node made so far
     for (auto& level : lowered) {
         std::vector<hipGraphNode_t> deps = prev;
-        if (deps.size() > 1) {
+        if (!waits && deps.size() > 1) {
             hipGraphNode_t join;
             HIP_TRY(dev, hipGraphAddEmptyNode(&join, g->graph, deps.data(), deps.size()));
+            g->edges += deps.size();
             deps = {join};
         }
         std::vector<hipGraphNode_t> made;
         for (LoweredNode& ln : level) {
+            if (waits) {
+                deps.clear();
+                for (uint32_t q : (*waits)[all.size()]) deps.push_back(all[q]);
+            }
             hipGraphNode_t node;
             if (ln.is_copy) {
                 HIP_TRY(dev, hipGraphAddMemcpyNode1D(&node, g->graph, deps.data(), deps.size(),
@@ -363,7 +488,9 @@ int32_t instantiate(custos_hip_device* dev, custos_hip_graph* g, std::vector<std
                 kp.extra = nullptr;
                 HIP_TRY(dev, hipGraphAddKernelNode(&node, g->graph, deps.data(), deps.size(), &kp));
             }
+            g->edges += deps.size();
             made.push_back(node);
+            all.push_back(node);
         }
         prev = std::move(made);
     }
@@ -375,7 +502,7 @@ int32_t instantiate(custos_hip_device* dev, custos_hip_graph* g, std::vector<std
 
 int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     std::vector<RecNode>& nodes = dev->recorded;
-    assign_levels(nodes);
+    assign_levels(nodes, dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_PER_NODE);
     int max_level = -1;
     for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
     g->recorded = nodes.size();
@@ -425,8 +552,12 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
         chain = chain && lowered[level].size() == 1;
     }
 
-    if (chain && total <= dev->direct_replay_max) {
-        for (auto& level : lowered) g->direct.push_back(std::move(level[0]));
+    // In one chain every order that follows the levels is a valid one, so a short graph of any
+    // shape can be replayed as plain launches.
+    const bool serial = dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN;
+    if ((chain || serial) && total <= dev->direct_replay_max) {
+        for (auto& level : lowered)
+            for (LoweredNode& ln : level) g->direct.push_back(std::move(ln));
         // With an odd number of alternating nodes the first one of the next replay would
         // run in the direction of the last one of this replay: flip them all every replay.
         size_t alternating = 0;
@@ -434,7 +565,21 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
         g->flip_each_replay = alternating % 2 == 1;
         return CUSTOS_HIP_OK;
     }
-    return instantiate(dev, g, lowered);
+    std::vector<std::vector<uint32_t>> waits;
+    if (dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_PER_NODE) {
+        waits = node_edges(nodes, plan);
+    } else if (serial) {
+        waits.resize(total);
+        for (uint32_t id = 1; id < total; id++) waits[id].push_back(id - 1);
+    } else {
+        waits = level_waits(plan);
+    }
+    if (dev->graph_verify) {
+        if (nodes.size() > 8192) return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "recording too long for the brute-force ordering check");
+        if (!ordering_holds(nodes, plan, waits))
+            return set_error(dev, CUSTOS_HIP_ERR_GRAPH_ORDER, "built graph does not order two conflicting pieces of recorded work");
+    }
+    return instantiate(dev, g, lowered, dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS ? nullptr : &waits);
 }
 
 int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
@@ -516,6 +661,26 @@ int32_t custos_hip_set_graph_direct_replay(custos_hip_device* dev, int32_t max_n
     REQUIRE_DEV(dev);
     if (max_nodes < 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "max_nodes is negative");
     dev->direct_replay_max = static_cast<size_t>(max_nodes);
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_graph_edges(custos_hip_device* dev, int32_t mode) {
+    REQUIRE_DEV(dev);
+    if (mode < CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS || mode > CUSTOS_HIP_GRAPH_EDGES_CHAIN)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown graph edge mode");
+    dev->graph_edges = mode;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_graph_verify(custos_hip_device* dev, int32_t enabled) {
+    REQUIRE_DEV(dev);
+    dev->graph_verify = enabled != 0;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_edge_count(custos_hip_graph* graph, size_t* edges) {
+    if (!graph || !edges) return CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+    *edges = graph->edges;
     return CUSTOS_HIP_OK;
 }
 

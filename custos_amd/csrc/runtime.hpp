@@ -63,6 +63,7 @@ struct custos_hip_graph {
     size_t kernel_nodes = 0;  // kernel nodes in the instantiated graph
     size_t recorded = 0;      // launches, clears and copies that were recorded
     size_t levels = 0;        // dependency levels
+    size_t edges = 0;         // dependency edges of the instantiated graph (joins included)
 };
 
 // One recorded piece of work (while the device is recording, nothing is launched).
@@ -77,6 +78,7 @@ struct RecNode {
     unsigned long long n = 0, head = 0, n_vec = 0, bytes = 0;
     std::vector<Access> acc;
     int level = 0;
+    std::vector<uint32_t> deps;  // recorded nodes this one has to follow (filled when a graph is built with per-node edges)
     // Source: launch shape and a copy of the argument values.  What such a kernel
     // reads and writes is unknown, so it orders itself against everything.
     unsigned int grid3[3] = {1, 1, 1}, block3[3] = {1, 1, 1}, shared_mem = 0;
@@ -123,6 +125,8 @@ struct custos_hip_device {
     uint64_t hinted[4] = {0, 0, 0, 0};
     uint64_t kept_loads = 0;         // of those, launches that keep an operand's loads temporal while streaming  // launches and graph nodes of at least kHintFromBytes by CacheHint
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
+    bool graph_verify = false;       // built graphs are checked by brute force against the recorded conflicts
+    int32_t graph_edges = CUSTOS_HIP_GRAPH_EDGES_CHAIN;  // how built graphs order their nodes
     // allocation pool: freed blocks by rounded size; every block this handle allocated, by address
     std::unordered_map<size_t, std::vector<void*>> pool;
     std::unordered_map<uint64_t, size_t> block_bytes;

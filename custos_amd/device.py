@@ -93,6 +93,12 @@ class Graph:
         self.device._check(self.device.lib.custos_hip_graph_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
         return a.value, b.value, c.value
 
+    def edge_count(self) -> int:
+        """Dependency edges of the instantiated graph, joins included (0 for a directly replayed chain)."""
+        e = C.c_size_t(0)
+        self.device._check(self.device.lib.custos_hip_graph_edge_count(self.handle, C.byref(e)))
+        return e.value
+
     def destroy(self) -> None:
         if self.handle and self.device.handle:
             self.device._check(self.device.lib.custos_hip_graph_destroy(self.device.handle, self.handle))
@@ -320,6 +326,14 @@ class HIP:
 
     def set_graph_direct_replay(self, max_nodes: int) -> None:
         self._check(self.lib.custos_hip_set_graph_direct_replay(self.handle, max_nodes))
+
+    def set_graph_edges(self, mode: int) -> None:
+        """How built graphs order their nodes: capi.GRAPH_EDGES_LEVEL_JOINS, _PER_NODE or _CHAIN."""
+        self._check(self.lib.custos_hip_set_graph_edges(self.handle, int(mode)))
+
+    def set_graph_verify(self, enabled: bool) -> None:
+        """capture_end checks the ordering of every graph it builds by brute force (for tests)."""
+        self._check(self.lib.custos_hip_set_graph_verify(self.handle, 1 if enabled else 0))
 
     def is_capturing(self) -> bool:
         v = C.c_int32(0)

@@ -256,6 +256,8 @@ class HIP : public Device<HIP<Mods>, Mods> {
     }
     // Longest recorded chain that is replayed as plain launches instead of a graph launch.
     void set_graph_direct_replay(int32_t max_nodes) { check(custos_hip_set_graph_direct_replay(dev_, max_nodes)); }
+    // How built graphs order their nodes: CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS, _PER_NODE or _CHAIN.
+    void set_graph_edges(int32_t mode) { check(custos_hip_set_graph_edges(dev_, mode)); }
 
     custos_hip_kernel* compile(int32_t kind, int32_t dtype, const std::string& src,
                                std::initializer_list<const char*> markers) {

@@ -208,12 +208,28 @@ def test_merged_launches_of_different_lengths(hip, oracle):
     g.destroy()
 
 
-def test_recorded_dependencies_random(hip, oracle):
+@pytest.fixture
+def checked_graphs(hip):
+    """Every graph built inside the test is checked by brute force against the recorded conflicts."""
+    hip.set_graph_verify(True)
+    yield hip
+    hip.set_graph_verify(False)
+    hip.set_graph_edges(capi.GRAPH_EDGES_CHAIN)
+
+
+EDGE_MODES = {"level joins": capi.GRAPH_EDGES_LEVEL_JOINS, "per node": capi.GRAPH_EDGES_PER_NODE, "chain": capi.GRAPH_EDGES_CHAIN}
+
+
+@pytest.mark.parametrize("edges", list(EDGE_MODES))
+def test_recorded_dependencies_random(checked_graphs, oracle, edges):
     """Random programs over a small pool of buffers, with in-place updates, views and clears:
-    replaying the built graph (levels, side-by-side nodes, merged launches) must equal running
-    the same calls eagerly, bit for bit.  Even trials use aligned half-buffer views, odd trials
-    views of any offset and length (partial overlaps between operations, scalar launches)."""
+    replaying the built graph (ordered by level joins, per-node edges or as one chain; merged launches)
+    must equal running the same calls eagerly, bit for bit.  Even trials use aligned half-buffer
+    views, odd trials views of any offset and length (partial overlaps between operations,
+    scalar launches).  The library also checks each graph's ordering by brute force."""
     import os
+    hip = checked_graphs
+    hip.set_graph_edges(EDGE_MODES[edges])
     rng = np.random.default_rng(1234)
     n = 2048
     fns1 = [lambda v: v.mul(1.25).add(0.5), lambda v: v.neg().max(-3.0), lambda v: v.abs().sqrt(), lambda v: v.mul(v).min(9.0)]
@@ -276,6 +292,85 @@ def test_recorded_dependencies_random(hip, oracle):
         hip.sync()
         for i, b in enumerate(lazy):
             assert_bits_equal(b.read(), eager[i].read(), f"trial {trial} second replay, buffer {i}")
+        g.destroy()
+
+
+def test_per_node_edges_let_independent_chains_run_apart(checked_graphs, oracle):
+    """Two chains over different buffers with different kernels, one twice as long as the other,
+    then a caller-written kernel (unknown memory use: ordered against everything) and one more
+    launch per chain.  With an edge per dependency no node waits for the other chain (fewer edges
+    than level joins need); as one chain the nodes follow each other in level order.  The same
+    bits in every mode, replay after replay."""
+    hip = checked_graphs
+    n = 30011
+    x, y = synth.uniform_f32(31, n, -2, 2), synth.uniform_f32(32, n, -2, 2)
+    f = lambda v: v.mul(1.5).sub(0.25)
+    h = lambda v: v.abs().add(0.5)
+    scale = """extern "C" __global__ void halve(float* p, unsigned long long n) {
+        unsigned long long i = blockIdx.x * (unsigned long long)blockDim.x + threadIdx.x;
+        if (i < n) p[i] = p[i] * 0.5f;
+    }"""
+
+    def program(a, b):
+        for _ in range(4):
+            hip.apply_fn(a, f, out=a)
+        for _ in range(2):
+            hip.apply_fn(b, h, out=b)
+        hip.launch_kernel(scale, "halve", ((n + 255) // 256, 1, 1), (256, 1, 1), 0, [a, np.uint64(n)])
+        hip.apply_fn(a, h, out=a)
+        hip.apply_fn(b, f, out=b)
+
+    ea, eb = hip.buffer(x), hip.buffer(y)
+    edges = {}
+    hip.set_graph_direct_replay(0)
+    try:
+        for per_node, mode in EDGE_MODES.items():
+            hip.set_graph_edges(mode)
+            a, b = hip.buffer(x), hip.buffer(y)
+            hip.capture_begin()
+            program(a, b)
+            g = hip.capture_end()
+            assert g.stats() == (9, 9, 6)
+            edges[per_node] = g.edge_count()
+            ca, cb = hip.buffer(x), hip.buffer(y)
+            for replay in range(3):
+                g.launch()
+                program(ca, cb)
+                hip.sync()
+                assert_bits_equal(a.read(), ca.read(), f"per_node={per_node} replay {replay}, first chain")
+                assert_bits_equal(b.read(), cb.read(), f"per_node={per_node} replay {replay}, second chain")
+            g.destroy()
+    finally:
+        hip.set_graph_direct_replay(4)
+    # per-node: 3 edges inside the first chain, 1 inside the second, 2 into the caller-written kernel, 2 out of it
+    assert edges["per node"] == 8
+    assert edges["chain"] == 8          # nine nodes one after the other
+    assert edges["level joins"] == 11
+    want = x
+    for _ in range(4):
+        want = oracle.apply_fn(f, want)
+    want = oracle.apply_fn(h, want * np.float32(0.5))
+    program(ea, eb)
+    hip.sync()
+    assert_bits_equal(ea.read(), want)
+
+
+def test_ordering_check_accepts_merged_and_fenced_graphs(checked_graphs):
+    """The brute-force check runs on a graph of merged launches in every edge mode."""
+    hip = checked_graphs
+    n, count = 4096, 64
+    xs = [hip.buffer(synth.uniform_f32(100 + i, n, 0, 1)) for i in range(count)]
+    ts = [hip.alloc(n) for _ in range(count)]
+    for mode in EDGE_MODES.values():
+        hip.set_graph_edges(mode)
+        hip.capture_begin()
+        for x, t in zip(xs, ts):
+            hip.apply_fn(x, lambda v: v.mul(2.0), out=t)
+            hip.apply_fn(t, lambda v: v.add(1.0), out=x)
+        g = hip.capture_end()
+        assert g.stats() == (2 * count, 2, 2)
+        g.launch()
+        hip.sync()
         g.destroy()
 
 
