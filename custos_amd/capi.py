@@ -138,6 +138,7 @@ PROTOTYPES = {
     "custos_hip_add_unary_grad": (C.c_int32, [_P, _P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_capture_begin": (C.c_int32, [_P]),
     "custos_hip_capture_end": (C.c_int32, [_P, _PP]),
+    "custos_hip_capture_end_reuse": (C.c_int32, [_P, _P, _PP]),
     "custos_hip_is_capturing": (C.c_int32, [_P, C.POINTER(C.c_int32)]),
     "custos_hip_graph_launch": (C.c_int32, [_P, _P]),
     "custos_hip_graph_node_count": (C.c_int32, [_P, C.POINTER(C.c_size_t)]),

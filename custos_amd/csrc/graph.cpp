@@ -2,6 +2,7 @@
 // conflicts, merging of equal launches, explicit hipGraph nodes, replay
 // (include/custos_hip.h).
 #include <algorithm>
+#include <array>
 #include <cstring>
 
 #include "runtime.hpp"
@@ -357,6 +358,32 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
     return CUSTOS_HIP_OK;
 }
 
+// Everything that decides what a recording does, word by word: two recordings with equal
+// signatures build equal graphs.  (A kernel handle stands for its code and its literal values.)
+std::vector<uint64_t> signature(const std::vector<RecNode>& nodes) {
+    std::vector<uint64_t> sig;
+    sig.reserve(nodes.size() * 10);
+    for (const RecNode& n : nodes) {
+        sig.push_back(static_cast<uint64_t>(n.type));
+        sig.push_back(reinterpret_cast<uint64_t>(n.k));
+        sig.insert(sig.end(), {n.n, n.head, n.n_vec, n.bytes, static_cast<uint64_t>(n.ptrs.size())});
+        sig.insert(sig.end(), n.ptrs.begin(), n.ptrs.end());
+        if (n.type != RecNode::Source) continue;
+        for (int d = 0; d < 3; d++) sig.push_back(static_cast<uint64_t>(n.grid3[d]) << 32 | n.block3[d]);
+        sig.push_back(n.shared_mem);
+        sig.push_back(n.arg_values.size());
+        for (const auto& value : n.arg_values) {
+            sig.push_back(value.size());
+            for (size_t at = 0; at < value.size(); at += 8) {
+                uint64_t word = 0;
+                std::memcpy(&word, value.data() + at, std::min<size_t>(8, value.size() - at));
+                sig.push_back(word);
+            }
+        }
+    }
+    return sig;
+}
+
 // What every node of the graph to be waits for, as indices into the nodes in level order.
 // Level joins: a node waits for the whole level before it (`join_levels`).  Per-node edges: a
 // node waits for the nodes that hold the recorded work its members conflict with; a node with
@@ -507,6 +534,8 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
     g->recorded = nodes.size();
     g->levels = static_cast<size_t>(max_level + 1);
+    g->signature = signature(nodes);
+    g->built_with = {dev->batching ? 1u : 0u, static_cast<uint64_t>(dev->graph_edges), dev->direct_replay_max};
 
     std::vector<std::vector<Planned>> plan;
     std::vector<uint64_t> host_table;
@@ -649,6 +678,24 @@ int32_t custos_hip_capture_end(custos_hip_device* dev, custos_hip_graph** graph)
     dev->graphs.push_back(g);
     *graph = g;
     return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_capture_end_reuse(custos_hip_device* dev, custos_hip_graph* previous, custos_hip_graph** graph) {
+    REQUIRE_DEV(dev);
+    if (!graph) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph out pointer is null");
+    *graph = nullptr;
+    if (!dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the device is not recording");
+    if (previous && std::find(dev->graphs.begin(), dev->graphs.end(), previous) == dev->graphs.end())
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "the previous graph does not belong to this device");
+    const std::array<uint64_t, 3> settings = {dev->batching ? 1u : 0u, static_cast<uint64_t>(dev->graph_edges),
+                                              dev->direct_replay_max};
+    if (previous && previous->built_with == settings && previous->signature == signature(dev->recorded)) {
+        dev->capturing = false;
+        dev->recorded.clear();
+        *graph = previous;
+        return CUSTOS_HIP_OK;
+    }
+    return custos_hip_capture_end(dev, graph);
 }
 
 int32_t custos_hip_set_graph_batching(custos_hip_device* dev, int32_t enabled) {

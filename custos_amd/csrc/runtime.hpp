@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <array>
 #include <cstdint>
 #include <map>
 #include <memory>
@@ -64,6 +65,10 @@ struct custos_hip_graph {
     size_t recorded = 0;      // launches, clears and copies that were recorded
     size_t levels = 0;        // dependency levels
     size_t edges = 0;         // dependency edges of the instantiated graph (joins included)
+    // what the graph was built from: the recording, word by word, and the device's graph settings
+    // (merging, edge mode, direct replay limit) -- see custos_hip_capture_end_reuse
+    std::vector<uint64_t> signature;
+    std::array<uint64_t, 3> built_with{};
 };
 
 // One recorded piece of work (while the device is recording, nothing is launched).

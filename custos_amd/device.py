@@ -310,6 +310,14 @@ class HIP:
         self._check(self.lib.custos_hip_capture_end(self.handle, C.byref(g)))
         return Graph(self, g)
 
+    def capture_end_reuse(self, previous: Graph | None) -> Graph:
+        """capture_end that hands back `previous` itself when the recording is the one it was built from."""
+        g = C.c_void_p()
+        self._check(self.lib.custos_hip_capture_end_reuse(self.handle, previous.handle if previous else None, C.byref(g)))
+        if previous is not None and g.value == previous.handle.value:
+            return previous
+        return Graph(self, g)
+
     def set_graph_batching(self, enabled: bool) -> None:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 

@@ -334,6 +334,14 @@ int32_t custos_hip_capture_begin(custos_hip_device *dev);
  * grid, whatever their lengths (1024 buffers x 3 operations replay as 3 kernel
  * nodes). How the nodes are ordered: custos_hip_set_graph_edges. */
 int32_t custos_hip_capture_end(custos_hip_device *dev, custos_hip_graph **graph);
+/* capture_end for a caller that records the same program before every run (the reference's
+ * Lazy::run calls every recorded operation again before each launch of its graph,
+ * src/modules/lazy.rs:190-197, src/devices/cuda/lazy.rs:31-49): ends recording, and if the
+ * recording is, launch for launch and address for address, the one `previous` was built from
+ * (and the graph settings have not changed), hands back `previous` itself and builds nothing.
+ * Otherwise a new graph is built as by capture_end; `previous` (may be null) is left alone and
+ * stays the caller's to destroy. */
+int32_t custos_hip_capture_end_reuse(custos_hip_device *dev, custos_hip_graph *previous, custos_hip_graph **graph);
 /* Switches the merging of equal independent launches off (0) or on (default):
  * with it off every recorded launch becomes its own kernel node. */
 int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);

@@ -374,6 +374,58 @@ def test_ordering_check_accepts_merged_and_fenced_graphs(checked_graphs):
         g.destroy()
 
 
+def test_a_repeated_recording_reuses_its_graph(hip, oracle):
+    """A caller that records its program again before every run (the reference's Lazy::run does)
+    gets the graph it already has as long as the recording is the same; another length, another
+    buffer, another literal or another graph setting builds a new one."""
+    n = 9000
+    x = synth.uniform_f32(41, n, -2, 2)
+    a, b, c = hip.buffer(x), hip.alloc(n), hip.alloc(n)
+    f = lambda v: v.mul(1.5).sub(0.25)
+
+    def record(src=a, dst=c, length=n, fn=f):
+        hip.capture_begin()
+        hip.apply_fn(src.slice(0, length), lambda v: v.abs(), out=b.slice(0, length))
+        hip.apply_fn(b.slice(0, length), fn, out=dst.slice(0, length))
+
+    record()
+    g = hip.capture_end_reuse(None)
+    want = oracle.apply_fn(f, np.abs(x))
+    for run in range(3):
+        c.clear()
+        record()
+        again = hip.capture_end_reuse(g)
+        assert again is g, f"run {run}: the same recording built a new graph"
+        assert not hip.is_capturing()
+        again.launch()
+        hip.sync()
+        assert_bits_equal(c.read(), want)
+    d = hip.alloc(n)
+    changes = {"shorter": dict(length=n - 1), "other output": dict(dst=d), "other literal": dict(fn=lambda v: v.mul(1.5).sub(0.5))}
+    for what, change in changes.items():
+        record(**change)
+        other = hip.capture_end_reuse(g)
+        assert other is not g, what
+        other.launch()
+        hip.sync()
+        other.destroy()
+    try:
+        hip.set_graph_direct_replay(0)
+        record()
+        other = hip.capture_end_reuse(g)
+        assert other is not g, "graph settings changed"
+        other.destroy()
+    finally:
+        hip.set_graph_direct_replay(4)
+    c.clear()
+    record()
+    assert hip.capture_end_reuse(g) is g
+    g.launch()
+    hip.sync()
+    assert_bits_equal(c.read(), want)
+    g.destroy()
+
+
 @pytest.mark.parametrize("n", [5000, 5001])
 def test_recorded_copy_nodes(hip, n):
     """Recorded device-to-device copies are launches of the identity kernel (kernel nodes that
