@@ -426,6 +426,31 @@ def test_a_repeated_recording_reuses_its_graph(hip, oracle):
     g.destroy()
 
 
+def test_lazy_run_sequence_of_an_unmodified_lazy_module(hip, oracle):
+    """The call sequence of a device under the reference's own Lazy module (src/modules/lazy.rs:190-197,
+    src/devices/cuda/lazy.rs:31-72): recording starts when the device is set up, buffers are allocated and
+    written while it records, every run calls all operations again and then the device's run, results are
+    read while the next recording is already open.  Every operation must run exactly once per run."""
+    n = 5000
+    x = synth.uniform_f32(51, n, 0.5, 2)
+    hip.capture_begin()                                  # lazy_setup
+    try:
+        a, acc = hip.buffer(x), hip.alloc(n)             # allocation and writes execute at once
+        graph = None
+        for run in range(1, 5):
+            hip.apply_fn2(acc, a, lambda p, q: p.add(q), out=acc)      # call_lazily: recorded, not run
+            new = hip.capture_end_reuse(graph)                          # LazyRun::run
+            assert graph is None or new is graph
+            graph = new
+            graph.launch()
+            hip.sync()
+            hip.capture_begin()
+            assert_bits_equal(acc.read(), (x * np.float32(run)).astype(np.float32), f"run {run}")   # read while recording
+    finally:
+        hip.capture_end().destroy()
+    graph.destroy()
+
+
 @pytest.mark.parametrize("n", [5000, 5001])
 def test_recorded_copy_nodes(hip, n):
     """Recorded device-to-device copies are launches of the identity kernel (kernel nodes that
