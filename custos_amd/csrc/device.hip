@@ -77,6 +77,40 @@ __global__ void __launch_bounds__(kFillBlock) custos_fill_zero(unsigned char* p,
     for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads) p[i] = 0;
 }
 
+// The same walk with a 16-byte pattern instead of zeros (a value of 1, 2, 4, 8 or 16 bytes
+// repeated): byte k of the pattern belongs at addresses that are k modulo 16, which is what
+// the aligned body stores; the bytes at the edges pick theirs by address.
+__device__ __forceinline__ unsigned char pattern_byte(unsigned int w0, unsigned int w1, unsigned int w2, unsigned int w3,
+                                                      unsigned long long address) {
+    const unsigned int k = static_cast<unsigned int>(address & 15);
+    const unsigned int word = k < 4 ? w0 : k < 8 ? w1 : k < 12 ? w2 : w3;
+    return static_cast<unsigned char>(word >> ((k & 3) * 8));
+}
+
+__global__ void __launch_bounds__(kFillBlock) custos_fill_pattern(unsigned char* p, unsigned long long bytes,
+                                                                  unsigned long long head, unsigned long long n_vec,
+                                                                  unsigned int w0, unsigned int w1, unsigned int w2,
+                                                                  unsigned int w3) {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    u4* v = reinterpret_cast<u4*>(p + head);
+    const u4 pattern = {w0, w1, w2, w3};
+    const unsigned long long tile_vecs = (unsigned long long)kFillBlock * kFillUnroll;
+    const unsigned long long n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;
+    for (unsigned long long tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+#pragma unroll
+        for (unsigned int u = 0; u < kFillUnroll; u++) {
+            const unsigned long long i = tile * tile_vecs + (unsigned long long)u * kFillBlock + threadIdx.x;
+            if (i < n_vec) v[i] = pattern;
+        }
+    }
+    const unsigned long long gid = (unsigned long long)blockIdx.x * kFillBlock + threadIdx.x;
+    const unsigned long long n_threads = (unsigned long long)gridDim.x * kFillBlock;
+    const unsigned long long base = reinterpret_cast<unsigned long long>(p);
+    if (gid < head) p[gid] = pattern_byte(w0, w1, w2, w3, base + gid);
+    for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads)
+        p[i] = pattern_byte(w0, w1, w2, w3, base + i);
+}
+
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec) {
     (void)dev;
     const unsigned long long tile_vecs = (unsigned long long)kFillBlock * kFillUnroll;
@@ -114,7 +148,8 @@ int32_t launch_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t b
     return launch_or_record(dev, k, {{src, false}, {dst, true}}, words ? bytes / 4 : bytes);
 }
 
-int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream) {
+// `pattern`: null for zeros, else the 16 bytes that repeat from any 16-byte boundary on.
+int32_t launch_fill(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream, const uint32_t* pattern) {
     unsigned long long head = (16 - (dptr & 15)) & 15;
     if (head > bytes) head = bytes;
     unsigned long long n_vec = (bytes - head) / 16;
@@ -125,19 +160,30 @@ int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hi
         node.bytes = bytes;
         node.head = head;
         node.n_vec = n_vec;
+        if (pattern) node.pattern.assign(pattern, pattern + 4);
         node.acc = {{dptr, dptr + bytes, true}};
         dev->recorded.push_back(std::move(node));
         return CUSTOS_HIP_OK;
     }
     unsigned int grid = fill_grid(dev, n_vec);
-    hipLaunchKernelGGL(custos_fill_zero, dim3(grid), dim3(kFillBlock), 0, stream,
-                       reinterpret_cast<unsigned char*>(dptr), static_cast<unsigned long long>(bytes),
-                       head, n_vec);
+    if (pattern)
+        hipLaunchKernelGGL(custos_fill_pattern, dim3(grid), dim3(kFillBlock), 0, stream,
+                           reinterpret_cast<unsigned char*>(dptr), static_cast<unsigned long long>(bytes), head, n_vec,
+                           pattern[0], pattern[1], pattern[2], pattern[3]);
+    else
+        hipLaunchKernelGGL(custos_fill_zero, dim3(grid), dim3(kFillBlock), 0, stream,
+                           reinterpret_cast<unsigned char*>(dptr), static_cast<unsigned long long>(bytes),
+                           head, n_vec);
     HIP_TRY(dev, hipGetLastError());
     return CUSTOS_HIP_OK;
 }
 
+int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream) {
+    return launch_fill(dev, dptr, bytes, stream, nullptr);
+}
+
 void* fill_zero_kernel() { return reinterpret_cast<void*>(custos_fill_zero); }
+void* fill_pattern_kernel() { return reinterpret_cast<void*>(custos_fill_pattern); }
 unsigned int fill_block() { return kFillBlock; }
 
 }  // namespace custos_hip
@@ -423,6 +469,22 @@ int32_t custos_hip_clear(custos_hip_device* dev, uint64_t dptr, size_t bytes) {
     if (bytes == 0) return CUSTOS_HIP_OK;
     if (!dptr) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
     return launch_fill_zero(dev, dptr, bytes, dev->stream);
+}
+
+int32_t custos_hip_fill(custos_hip_device* dev, uint64_t dptr, size_t bytes, const void* value, size_t value_bytes) {
+    REQUIRE_DEV(dev);
+    if (bytes == 0) return CUSTOS_HIP_OK;
+    if (!dptr || !value) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
+    if (value_bytes == 0 || value_bytes > 16 || (value_bytes & (value_bytes - 1)) != 0)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "a fill value has 1, 2, 4, 8 or 16 bytes");
+    if (dptr % value_bytes != 0 || bytes % value_bytes != 0)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "address and length of a fill are multiples of the value's size");
+    unsigned char repeated[16];
+    for (size_t k = 0; k < 16; k++) repeated[k] = static_cast<const unsigned char*>(value)[k % value_bytes];
+    uint32_t pattern[4];
+    std::memcpy(pattern, repeated, 16);
+    const bool zeros = (pattern[0] | pattern[1] | pattern[2] | pattern[3]) == 0;
+    return launch_fill(dev, dptr, bytes, dev->stream, zeros ? nullptr : pattern);
 }
 
 // ---- timing ----

@@ -312,7 +312,8 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
     } else if (first.type == RecNode::Fill) {
         const unsigned long long a0 = first.bytes, a1 = first.head, a2 = first.n_vec;
         ln.args = {value(&first.ptrs[0], 8), value(&a0, 8), value(&a1, 8), value(&a2, 8)};
-        ln.func = fill_zero_kernel();
+        for (uint32_t word : first.pattern) ln.args.push_back(value(&word, 4));
+        ln.func = first.pattern.empty() ? fill_zero_kernel() : fill_pattern_kernel();
         ln.module_fn = false;
         ln.grid = dim3(fill_grid(dev, first.n_vec));
         ln.block = dim3(fill_block());
@@ -368,6 +369,8 @@ std::vector<uint64_t> signature(const std::vector<RecNode>& nodes) {
         sig.push_back(reinterpret_cast<uint64_t>(n.k));
         sig.insert(sig.end(), {n.n, n.head, n.n_vec, n.bytes, static_cast<uint64_t>(n.ptrs.size())});
         sig.insert(sig.end(), n.ptrs.begin(), n.ptrs.end());
+        sig.push_back(n.pattern.size());
+        sig.insert(sig.end(), n.pattern.begin(), n.pattern.end());
         if (n.type != RecNode::Source) continue;
         for (int d = 0; d < 3; d++) sig.push_back(static_cast<uint64_t>(n.grid3[d]) << 32 | n.block3[d]);
         sig.push_back(n.shared_mem);

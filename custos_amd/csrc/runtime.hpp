@@ -81,6 +81,7 @@ struct RecNode {
     custos_hip_kernel* k = nullptr;
     std::vector<uint64_t> ptrs;  // kernel: operand addresses in parameter order; fill: {ptr}; copy: {dst, src}
     unsigned long long n = 0, head = 0, n_vec = 0, bytes = 0;
+    std::vector<uint32_t> pattern;  // fill: the 16 bytes that repeat; empty = zeros
     std::vector<Access> acc;
     int level = 0;
     std::vector<uint32_t> deps;  // recorded nodes this one has to follow (filled when a graph is built with per-node edges)
@@ -195,6 +196,7 @@ unsigned int fill_block();
 // device-to-device copy, launched or recorded: the identity kernel, or the runtime's copy
 int32_t launch_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t bytes);  // threads per workgroup of the zero-fill kernel
 int32_t launch_fill_zero(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStream_t stream);
+void* fill_pattern_kernel();  // the same for a fill with a repeated value
 void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph kernel nodes
 
 // jit.cpp

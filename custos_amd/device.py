@@ -192,6 +192,11 @@ class HIP:
     def clear(self, buf: Buffer) -> None:
         self._check(self.lib.custos_hip_clear(self.handle, buf.ptr, buf.nbytes))
 
+    def fill(self, buf: Buffer, value) -> None:
+        """Every element of `buf` set to `value` on the device."""
+        item = np.asarray(value, dtype=_np_dtype(buf.dtype)).reshape(1)
+        self._check(self.lib.custos_hip_fill(self.handle, buf.ptr, buf.nbytes, item.ctypes.data_as(C.c_void_p), item.itemsize))
+
     def copy(self, dst: Buffer, src: Buffer) -> None:
         if dst.nbytes != src.nbytes:
             raise ValueError("size mismatch")

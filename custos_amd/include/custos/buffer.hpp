@@ -94,7 +94,7 @@ class Buffer {
     }
 
     // src/buffer/impl_autograd.rs:20-56
-    void backward() const { backward_with(std::vector<T>(len_, T(1))); }
+    void backward() const { device_->backward_ones(*this); }
     void backward_with(const std::vector<T>& seed) const { device_->backward_seeded(*this, seed); }
 
     // Gradient of this buffer, allocated (zeroed) on first use

@@ -103,6 +103,12 @@ class Device {
         if (!buf.has_data()) throw Error(DeviceError::InvalidLazyBuf);
         self().clear_raw(buf.ptr(), buf.len() * sizeof(T));
     }
+    // Every element set to `value`, on the device (no host array, no transfer).
+    template <class T>
+    void fill(Buffer<T, Derived>& buf, T value) {
+        if (!buf.has_data()) throw Error(DeviceError::InvalidLazyBuf);
+        self().fill_raw(buf.ptr(), buf.len() * sizeof(T), &value, sizeof(T));
+    }
     // `WriteBuf::write_buf`
     template <class T>
     void write_buf(Buffer<T, Derived>& dst, const Buffer<T, Derived>& src) {
@@ -335,10 +341,21 @@ class Device {
     // kept when lazy recording is on (tape.rs:39-83, impl_autograd.rs:37-56).
     template <class T>
     void backward_seeded(const Buffer<T, Derived>& buf, const std::vector<T>& seed) {
+        backward_from(buf, [&](Buffer<T, Derived>& g) { write(g, seed); });
+    }
+    // `Buffer::backward`: a seed of ones.  The reference builds `vec![T::one(); len]` on the host
+    // and writes it to the device (impl_autograd.rs:20-34, tape.rs:53-64); here the gradient is
+    // filled on the device.
+    template <class T>
+    void backward_ones(const Buffer<T, Derived>& buf) {
+        backward_from(buf, [&](Buffer<T, Derived>& g) { fill(g, T(1)); });
+    }
+    template <class T, class Seed>
+    void backward_from(const Buffer<T, Derived>& buf, Seed seed) {
         AutogradState* ag = modules.autograd();
         if (!ag) return;
         Buffer<T, Derived> g = grad_of<T>(buf.id());
-        write(g, seed);
+        seed(g);
         const bool lazy_enabled = modules.is_lazy_enabled();
         Buffers* buffers = modules.buffers();
         eagerly([&] {

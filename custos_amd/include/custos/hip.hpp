@@ -97,6 +97,9 @@ class HIP : public Device<HIP<Mods>, Mods> {
     void read_raw(void* dst, uint64_t src, size_t bytes) { check(custos_hip_read(dev_, dst, src, bytes)); }
     void write_raw(uint64_t dst, const void* src, size_t bytes) { check(custos_hip_write(dev_, dst, src, bytes)); }
     void clear_raw(uint64_t ptr, size_t bytes) { check(custos_hip_clear(dev_, ptr, bytes)); }
+    void fill_raw(uint64_t ptr, size_t bytes, const void* value, size_t value_bytes) {
+        check(custos_hip_fill(dev_, ptr, bytes, value, value_bytes));
+    }
     void copy_raw(uint64_t dst, uint64_t src, size_t bytes) { check(custos_hip_copy(dev_, dst, src, bytes)); }
 
     // ---- launches ----

@@ -51,6 +51,8 @@ extern "C" {
     pub fn custos_hip_read(dev: *mut HipDeviceHandle, dst: *mut c_void, src: u64, bytes: usize) -> i32;
     pub fn custos_hip_copy(dev: *mut HipDeviceHandle, dst: u64, src: u64, bytes: usize) -> i32;
     pub fn custos_hip_clear(dev: *mut HipDeviceHandle, dptr: u64, bytes: usize) -> i32;
+    pub fn custos_hip_fill(dev: *mut HipDeviceHandle, dptr: u64, bytes: usize, value: *const c_void,
+                           value_bytes: usize) -> i32;
     pub fn custos_hip_expr_compile(dev: *mut HipDeviceHandle, kind: i32, dtype: i32, src: *const c_char,
                                    markers: *const *const c_char, n_markers: i32, kernel: *mut *mut HipKernel) -> i32;
     pub fn custos_hip_kernel_source(kernel: *const HipKernel) -> *const c_char;

@@ -178,6 +178,13 @@ int32_t custos_hip_copy(custos_hip_device *dev, uint64_t dst, uint64_t src, size
 /* ClearBuf::clear / ZeroGrad::zero_grad (`cu_clear`, src/devices/cuda/mod.rs:59-74).
  * Implemented as a fill kernel, so it may be captured into a graph. */
 int32_t custos_hip_clear(custos_hip_device *dev, uint64_t dptr, size_t bytes);
+/* Fills `bytes` bytes with one value of `value_bytes` (1, 2, 4, 8 or 16) bytes repeated;
+ * address and length are multiples of `value_bytes`. What `Buffer::backward` needs for its
+ * seed of ones: the reference builds the ones on the host and writes them to the device
+ * (src/buffer/impl_autograd.rs:37-56, src/modules/autograd/tape.rs:67-83), N elements over
+ * the host link for every backward pass; this is one store-only kernel at memory speed,
+ * and it can be recorded like a clear. */
+int32_t custos_hip_fill(custos_hip_device *dev, uint64_t dptr, size_t bytes, const void *value, size_t value_bytes);
 
 /* ---- expression kernels (src/devices/cuda/kernel_cache.rs:10-73, source.rs:21-66) ---- */
 

@@ -46,6 +46,9 @@ class TestCPU : public Device<TestCPU<Mods>, Mods> {
     void read_raw(void* dst, uint64_t src, size_t bytes) { std::memcpy(dst, reinterpret_cast<void*>(src), bytes); }
     void write_raw(uint64_t dst, const void* src, size_t bytes) { std::memcpy(reinterpret_cast<void*>(dst), src, bytes); }
     void clear_raw(uint64_t ptr, size_t bytes) { std::memset(reinterpret_cast<void*>(ptr), 0, bytes); }
+    void fill_raw(uint64_t ptr, size_t bytes, const void* value, size_t value_bytes) {
+        for (size_t at = 0; at < bytes; at += value_bytes) std::memcpy(reinterpret_cast<char*>(ptr) + at, value, value_bytes);
+    }
     void copy_raw(uint64_t dst, uint64_t src, size_t bytes) {
         std::memmove(reinterpret_cast<void*>(dst), reinterpret_cast<void*>(src), bytes);
     }

@@ -1,4 +1,6 @@
 """GPU parity for node semantics, element types, addressing and error paths."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -502,6 +504,52 @@ def test_alloc_is_zeroed_and_clear_write_copy(hip):
     u = hip.buffer([1, 2, 3, 4, 5, 6], "u32")                    # src/devices/cuda/ops.rs:242-247
     u.clear()
     assert u.read().tolist() == [0] * 6
+
+
+@pytest.mark.parametrize("dtype,value", [("f32", 1.0), ("f32", -0.0), ("f64", 0.1), ("i32", -7), ("u8", 200), ("i16", -300),
+                                         ("u64", 2**63 + 5), ("f16", 1.0), ("f32", 0.0)])
+def test_fill_sets_every_element_and_nothing_else(hip, dtype, value):
+    """custos_hip_fill over views of every offset phase and length class: the bytes at the unaligned
+    edges, the 16-byte body and the neighbours of the view."""
+    np_type = np.dtype(capi.DTYPES[dtype][1])
+    item = np_type.itemsize
+    n = 5000
+    rng = np.random.default_rng(3)
+    background = rng.integers(0, 256, n * item, dtype=np.uint8).view(np_type)
+    for lo, length in ((0, n), (1, n - 2), (3, 1), (5, 16 // item + 1), (7, 1000), (2, 0), (16 // item, 333)):
+        buf = hip.buffer(background, dtype)
+        hip.fill(buf.slice(lo, lo + length), value)
+        want = background.copy()
+        want[lo:lo + length] = np.asarray(value, dtype=np_type)
+        assert_bits_equal(buf.read().view(np.uint8), want.view(np.uint8), f"{dtype} fill of [{lo}, {lo + length})")
+
+
+def test_fill_is_recorded_like_a_clear(hip):
+    n = 3001
+    a, b = hip.alloc(n), hip.alloc(n)
+    hip.capture_begin()
+    hip.fill(a, 2.5)
+    hip.apply_fn(a, lambda v: v.mul(2.0), out=b)
+    hip.fill(a, -1.0)
+    g = hip.capture_end()
+    assert not a.read().any(), "nothing may run while recording"
+    for _ in range(2):
+        g.launch()
+        hip.sync()
+        assert_bits_equal(b.read(), np.full(n, 5.0, np.float32))
+        assert_bits_equal(a.read(), np.full(n, -1.0, np.float32))
+        b.clear()
+    g.destroy()
+
+
+def test_fill_rejects_what_it_cannot_do(hip):
+    buf = hip.alloc(64, "u8")
+    value = (C.c_ubyte * 16)(*range(16))
+    for ptr, nbytes, size in ((buf.ptr + 1, 8, 4), (buf.ptr, 6, 4), (buf.ptr, 12, 3), (buf.ptr, 32, 32), (buf.ptr, 8, 0)):
+        rc = hip.lib.custos_hip_fill(hip.handle, ptr, nbytes, value, size)
+        assert rc == capi.ERR_INVALID_ARGUMENT, (ptr - buf.ptr, nbytes, size)
+    assert hip.lib.custos_hip_fill(hip.handle, buf.ptr, 32, value, 16) == 0          # a 16-byte value
+    assert buf.read()[:32].tolist() == list(range(16)) * 2
 
 
 RELU_SRC = """extern "C" __global__ void relu(float* lhs, float* out, int numElements) {
