@@ -25,12 +25,15 @@ int32_t hip_fail(custos_hip_device* dev, hipError_t e, const char* what) {
 
 const std::string& thread_last_error() { return g_last_error; }
 
+constexpr size_t kStagedReadMax = 64u << 10;  // reads and writes up to this size go through pinned staging memory
+constexpr size_t kWriteSlots = 16;            // staging slots of short writes (the first slot of the block is the read's)
+
 // Waits for the compute stream.  The blocking wait of the runtime takes about 9 us to
 // notice that a short job has finished -- three times the job itself for a small replayed
 // graph.  So the stream writes a sequence number into pinned host memory behind the
 // work, and the host polls that word for a short while before it falls back to the
 // blocking wait.
-hipError_t wait_compute_stream(custos_hip_device* dev) {
+static hipError_t wait_compute_stream_now(custos_hip_device* dev) {
     if (!dev->done_flag) return hipStreamSynchronize(dev->stream);
     const uint32_t seq = ++dev->done_seq;
     hipError_t e = hipStreamWriteValue32(dev->stream, dev->done_flag_dev, seq, 0);
@@ -45,6 +48,15 @@ hipError_t wait_compute_stream(custos_hip_device* dev) {
         if ((spins & 255) == 255 && std::chrono::steady_clock::now() - start > std::chrono::microseconds(200))
             return hipStreamSynchronize(dev->stream);
     }
+}
+
+// `waits_begun` / `waits_done` number the waits: work issued while `waits_begun` was w has
+// finished once `waits_done` is above w (what the staging slots of short writes go by).
+hipError_t wait_compute_stream(custos_hip_device* dev) {
+    const uint64_t mine = ++dev->waits_begun;
+    hipError_t e = wait_compute_stream_now(dev);
+    if (e == hipSuccess) dev->waits_done = mine;
+    return e;
 }
 
 // ---- zero fill: 16-byte stores over the aligned body, bytes at the edges ----
@@ -109,6 +121,36 @@ __global__ void __launch_bounds__(kFillBlock) custos_fill_pattern(unsigned char*
     if (gid < head) p[gid] = pattern_byte(w0, w1, w2, w3, base + gid);
     for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads)
         p[i] = pattern_byte(w0, w1, w2, w3, base + i);
+}
+
+// Short copies between device memory and pinned host memory (the staging of short reads and
+// writes): source and destination at the same 16-byte phase, 16-byte vectors over the aligned
+// body, bytes at the edges.  Compiled with the library, so that a first read or write does
+// not wait for a run-time compilation.
+__global__ void __launch_bounds__(kFillBlock) custos_stage_copy(unsigned char* dst, const unsigned char* src,
+                                                                unsigned long long bytes, unsigned long long head,
+                                                                unsigned long long n_vec) {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    u4* d = reinterpret_cast<u4*>(dst + head);
+    const u4* s = reinterpret_cast<const u4*>(src + head);
+    const unsigned long long gid = (unsigned long long)blockIdx.x * kFillBlock + threadIdx.x;
+    const unsigned long long n_threads = (unsigned long long)gridDim.x * kFillBlock;
+    for (unsigned long long i = gid; i < n_vec; i += n_threads) d[i] = s[i];
+    if (gid < head) dst[gid] = src[gid];
+    for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads) dst[i] = src[i];
+}
+
+// `dst` and `src` at the same 16-byte phase; runs on the compute stream, never recorded.
+static int32_t launch_stage_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t bytes) {
+    unsigned long long head = (16 - (dst & 15)) & 15;
+    if (head > bytes) head = bytes;
+    const unsigned long long n_vec = (bytes - head) / 16;
+    const unsigned int grid = static_cast<unsigned int>(std::max(1ull, (n_vec + kFillBlock - 1) / kFillBlock));
+    hipLaunchKernelGGL(custos_stage_copy, dim3(grid), dim3(kFillBlock), 0, dev->stream,
+                       reinterpret_cast<unsigned char*>(dst), reinterpret_cast<const unsigned char*>(src),
+                       static_cast<unsigned long long>(bytes), head, n_vec);
+    HIP_TRY(dev, hipGetLastError());
+    return CUSTOS_HIP_OK;
 }
 
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec) {
@@ -249,6 +291,20 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
             dev->done_flag = static_cast<uint32_t*>(flag);
             dev->done_flag_dev = flag_dev;
             *dev->done_flag = 0;
+            // staging for short reads, next to it (optional as well)
+            void* stage = nullptr;
+            void* stage_dev = nullptr;
+            if (hipHostMalloc(&stage, (kStagedReadMax + 16) * (1 + kWriteSlots), hipHostMallocMapped) == hipSuccess) {
+                if (hipHostGetDevicePointer(&stage_dev, stage, 0) == hipSuccess) {
+                    dev->read_stage = static_cast<unsigned char*>(stage);
+                    dev->read_stage_dev = reinterpret_cast<uint64_t>(stage_dev);
+                } else {
+                    (void)hipGetLastError();
+                    (void)hipHostFree(stage);
+                }
+            } else {
+                (void)hipGetLastError();
+            }
         } else {
             (void)hipGetLastError();
             (void)hipHostFree(flag);
@@ -276,6 +332,7 @@ int32_t custos_hip_device_destroy(custos_hip_device* dev) {
     (void)hipStreamDestroy(dev->stream);
     (void)hipStreamDestroy(dev->transfer);
     if (dev->done_flag) (void)hipHostFree(dev->done_flag);
+    if (dev->read_stage) (void)hipHostFree(dev->read_stage);
     delete dev;
     return CUSTOS_HIP_OK;
 }
@@ -438,6 +495,26 @@ int32_t custos_hip_write(custos_hip_device* dev, uint64_t dst, const void* src, 
         HIP_TRY(dev, hipStreamSynchronize(dev->transfer));
         return CUSTOS_HIP_OK;
     }
+    // A short write costs the runtime about 14 us, most of it the wait that lets the caller
+    // reuse `src`.  Up to 64 KiB the data is copied into a pinned staging slot (at the
+    // destination's 16-byte phase) and a copy kernel moves it from there, in stream
+    // order and without a wait; a slot is reused once a wait that began after its launch has
+    // finished, and a seventeenth write in a row without one waits first.
+    if (dev->read_stage && bytes <= kStagedReadMax) {
+        const size_t slot = dev->write_slot;
+        static_assert(kWriteSlots == std::tuple_size<decltype(dev->write_slot_issued)>::value, "one entry per slot");
+        if (dev->write_slot_used[slot] && dev->waits_done <= dev->write_slot_issued[slot])
+            HIP_TRY(dev, wait_compute_stream(dev));
+        const uint64_t phase = dst & 15;
+        const size_t offset = (kStagedReadMax + 16) * (1 + slot) + phase;
+        std::memcpy(dev->read_stage + offset, src, bytes);
+        int32_t rc = launch_stage_copy(dev, dst, dev->read_stage_dev + offset, bytes);
+        if (rc != CUSTOS_HIP_OK) return rc;
+        dev->write_slot_issued[slot] = dev->waits_begun;
+        dev->write_slot_used[slot] = true;
+        dev->write_slot = (slot + 1) % kWriteSlots;
+        return CUSTOS_HIP_OK;
+    }
     HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), src, bytes, hipMemcpyHostToDevice, dev->stream));
     // the caller may reuse `src` right away
     HIP_TRY(dev, hipStreamSynchronize(dev->stream));
@@ -451,6 +528,18 @@ int32_t custos_hip_read(custos_hip_device* dev, void* dst, uint64_t src, size_t 
     // Not recording: the copy is ordered on the compute stream behind the work that produces
     // the data, one wait in all.  While recording nothing is in flight there, and the copy must
     // not become part of the recording: it goes through the transfer stream.
+    // A short read costs the runtime about 20 us whatever its size.  Up to 64 KiB a copy
+    // kernel stores the data into pinned host memory instead (at the source's 16-byte phase, so
+    // that it moves whole vectors), and the host waits on the completion word: 4 bytes in
+    // about 8 us.
+    if (!dev->capturing && dev->read_stage && bytes <= kStagedReadMax) {
+        const uint64_t phase = src & 15;
+        int32_t rc = launch_stage_copy(dev, dev->read_stage_dev + phase, src, bytes);
+        if (rc != CUSTOS_HIP_OK) return rc;
+        HIP_TRY(dev, wait_compute_stream(dev));
+        std::memcpy(dst, dev->read_stage + phase, bytes);
+        return CUSTOS_HIP_OK;
+    }
     hipStream_t s = dev->capturing ? dev->transfer : dev->stream;
     HIP_TRY(dev, hipMemcpyAsync(dst, reinterpret_cast<const void*>(src), bytes, hipMemcpyDeviceToHost, s));
     HIP_TRY(dev, hipStreamSynchronize(s));

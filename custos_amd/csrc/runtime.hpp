@@ -143,6 +143,12 @@ struct custos_hip_device {
     uint32_t* done_flag = nullptr;  // pinned host word the compute stream writes sequence numbers to
     void* done_flag_dev = nullptr;  // its device address
     uint32_t done_seq = 0;
+    unsigned char* read_stage = nullptr;  // pinned host memory short reads (first slot) and writes are staged in
+    uint64_t read_stage_dev = 0;          // its device address
+    uint64_t waits_begun = 0, waits_done = 0;  // waits for the compute stream, numbered
+    size_t write_slot = 0;                     // next staging slot of a short write
+    std::array<uint64_t, 16> write_slot_issued{};  // per slot: `waits_begun` when its last launch was issued
+    std::array<bool, 16> write_slot_used{};
     unsigned long long launch_parity = 0;  // direction of the last launch that alternates
     bool batching = true;            // merge equal independent launches of a level into one grid
     std::vector<RecNode> recorded;

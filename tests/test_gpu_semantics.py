@@ -524,6 +524,55 @@ def test_fill_sets_every_element_and_nothing_else(hip, dtype, value):
         assert_bits_equal(buf.read().view(np.uint8), want.view(np.uint8), f"{dtype} fill of [{lo}, {lo + length})")
 
 
+def test_short_reads_at_every_phase_and_length(hip):
+    """Reads of up to 64 KiB are staged through pinned memory by the identity kernel; longer ones and
+    reads while recording go through the runtime's copy.  Same bytes at every offset phase, for
+    byte-granular and word-granular lengths, on both sides of the limit."""
+    n = (64 << 10) + 4096
+    data = np.random.default_rng(9).integers(0, 256, n, dtype=np.uint8)
+    buf = hip.buffer(data, "u8")
+    for lo in (0, 1, 3, 4, 13, 16, 4095):
+        for length in (1, 2, 3, 4, 15, 16, 17, 1000, 4096, (64 << 10) - 1, 64 << 10, (64 << 10) + 1):
+            got = buf.slice(lo, lo + length).read()
+            assert_bits_equal(got, data[lo:lo + length], f"read of [{lo}, {lo + length})")
+    words = hip.buffer(np.arange(5000, dtype=np.uint32), "u32")
+    hip.apply_fn(words, lambda v: v.add(1), out=words)                 # a read waits for the work before it
+    assert words.slice(7, 4000).read().tolist() == list(range(8, 4001))
+    hip.capture_begin()
+    try:
+        assert_bits_equal(buf.slice(5, 300).read(), data[5:300], "read while recording")
+    finally:
+        hip.capture_end().destroy()
+
+
+def test_short_writes_in_a_row_keep_their_own_data(hip):
+    """Writes of up to 64 KiB go through a ring of 16 pinned staging slots without a wait; the host
+    array may change right after the call, and more writes in a row than there are slots must not
+    overwrite data a launch has still to read."""
+    rng = np.random.default_rng(10)
+    n = (64 << 10) + 64
+    target = hip.alloc(n * 40, "u8")
+    want = np.zeros(n * 40, np.uint8)
+    scratch = np.empty(n, np.uint8)
+    lengths = [1, 3, 4, 16, 17, 1000, 4096, (64 << 10) - 1, 64 << 10, (64 << 10) + 1]
+    for i in range(40):                                    # no read, no sync in between
+        length = lengths[i % len(lengths)]
+        lo = i * n + int(rng.integers(0, 32))
+        scratch[:length] = rng.integers(0, 256, length, dtype=np.uint8)
+        want[lo:lo + length] = scratch[:length]
+        target.slice(lo, lo + length).write(scratch[:length])
+        scratch[:length] = 0xEE                            # the caller reuses its array at once
+    assert_bits_equal(target.read(), want)
+    # stream order: a write, a kernel on what was written, a write over the kernel's input
+    a, b = hip.alloc(1000), hip.alloc(1000)
+    for step in range(20):
+        a.write(np.full(1000, float(step), np.float32))
+        hip.apply_fn(a, lambda v: v.add(0.5), out=b)
+        a.write(np.full(1000, -1.0, np.float32))
+        assert b.read()[::333].tolist() == [step + 0.5] * 4
+        assert a.read()[0] == -1.0
+
+
 def test_fill_is_recorded_like_a_clear(hip):
     n = 3001
     a, b = hip.alloc(n), hip.alloc(n)
