@@ -60,6 +60,29 @@ def test_no_device_means_error_not_fallback():
         custos_amd.HIP(0)
 
 
+def test_entry_points_reject_a_null_device():
+    """Every entry point that takes a device handle answers a null one with an error code, not a crash."""
+    import ctypes as C
+    lib = custos_amd.load_library()
+    out = C.c_void_p()
+    value = C.c_float(1.0)
+    calls = [
+        lambda: lib.custos_hip_sync(None),
+        lambda: lib.custos_hip_capture_begin(None),
+        lambda: lib.custos_hip_capture_end(None, C.byref(out)),
+        lambda: lib.custos_hip_capture_end_reuse(None, None, C.byref(out)),
+        lambda: lib.custos_hip_set_graph_edges(None, capi.GRAPH_EDGES_CHAIN),
+        lambda: lib.custos_hip_set_graph_verify(None, 1),
+        lambda: lib.custos_hip_fill(None, 256, 4, C.byref(value), 4),
+        lambda: lib.custos_hip_clear(None, 256, 4),
+        lambda: lib.custos_hip_read(None, C.byref(value), 256, 4),
+        lambda: lib.custos_hip_write(None, 256, C.byref(value), 4),
+        lambda: lib.custos_hip_graph_edge_count(None, None),
+    ]
+    for number, call in enumerate(calls):
+        assert call() == capi.ERR_INVALID_ARGUMENT, number
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64", "f16", "bf16", "i32", "i64", "u8", "i8", "i16", "u16", "u32", "u64",
                                    "f16_pernode", "bf16_pernode"])
 def test_offline_compile_every_dtype(dtype):

@@ -2,6 +2,7 @@
 import numpy as np
 import pytest
 
+import custos_amd
 from custos_amd import capi, synth
 from tests.helpers import assert_bits_equal
 
@@ -424,6 +425,28 @@ def test_a_repeated_recording_reuses_its_graph(hip, oracle):
     hip.sync()
     assert_bits_equal(c.read(), want)
     g.destroy()
+
+
+def test_graph_settings_and_reuse_reject_bad_calls(hip):
+    import ctypes as C
+    out = C.c_void_p()
+    assert hip.lib.custos_hip_capture_end_reuse(hip.handle, None, C.byref(out)) == capi.ERR_CAPTURE_STATE   # not recording
+    assert hip.lib.custos_hip_set_graph_edges(hip.handle, 3) == capi.ERR_INVALID_ARGUMENT
+    assert hip.lib.custos_hip_set_graph_edges(hip.handle, -1) == capi.ERR_INVALID_ARGUMENT
+    other = custos_amd.HIP(0)
+    try:
+        other.capture_begin()
+        theirs = other.capture_end()
+        hip.capture_begin()
+        try:
+            rc = hip.lib.custos_hip_capture_end_reuse(hip.handle, theirs.handle, C.byref(out))
+            assert rc == capi.ERR_INVALID_ARGUMENT          # a graph of another device
+            assert hip.is_capturing()                        # and the recording is still open
+        finally:
+            hip.capture_end().destroy()
+        theirs.destroy()
+    finally:
+        other.close()
 
 
 def test_lazy_run_sequence_of_an_unmodified_lazy_module(hip, oracle):
