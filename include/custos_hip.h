@@ -386,9 +386,11 @@ int32_t custos_hip_set_graph_edges(custos_hip_device *dev, int32_t mode);
 /* With `enabled`, capture_end checks every graph it builds by brute force before instantiating it:
  * any two recorded pieces of work that touch overlapping memory, one of them writing, must be in
  * different nodes joined by a path; otherwise CUSTOS_HIP_ERR_GRAPH_ORDER. Quadratic in the
- * recorded work (at most 4096 nodes); meant for tests. */
+ * recorded work (at most 8192 recorded pieces); meant for tests. No counterpart in the
+ * reference, whose captured graphs are serial by construction. */
 int32_t custos_hip_set_graph_verify(custos_hip_device *dev, int32_t enabled);
-/* Dependency edges of an instantiated graph, joins included (0 for a directly replayed chain). */
+/* Dependency edges of an instantiated graph, joins included (0 for a directly replayed chain).
+ * No counterpart in the reference. */
 int32_t custos_hip_graph_edge_count(custos_hip_graph *graph, size_t *edges);
 int32_t custos_hip_is_capturing(custos_hip_device *dev, int32_t *capturing);
 /* LazyCudaGraph::launch on the compute stream (no wait; call custos_hip_sync). */
