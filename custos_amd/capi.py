@@ -43,7 +43,7 @@ ERR_GRAPH_ORDER = 10041
 ERR_BAD_OVERLAP = 10050
 ERR_TOO_LARGE = 10060
 
-GRAPH_EDGES_LEVEL_JOINS, GRAPH_EDGES_PER_NODE, GRAPH_EDGES_CHAIN = 0, 1, 2
+GRAPH_EDGES_LEVEL_JOINS, GRAPH_EDGES_PER_NODE, GRAPH_EDGES_CHAIN, GRAPH_EDGES_CHAIN_BY_LEVEL = 0, 1, 2, 3
 
 
 class CustosHipError(RuntimeError):

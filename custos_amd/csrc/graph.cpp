@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <array>
 #include <cstring>
+#include <queue>
 
 #include "runtime.hpp"
 
@@ -33,6 +34,8 @@ constexpr uint64_t kChunkShift = 21;  // conflict search buckets of 2 MiB
 constexpr unsigned long long kRaggedMaxTiles = 16384;
 // A node counts as a producer if one of this many levels after it reads what it writes.
 constexpr size_t kLookAheadLevels = 8;
+// A chain follows the recording (instead of the levels) if one of its launches touches this much.
+constexpr unsigned long long kFollowRecordingFromBytes = 8ull << 20;
 
 // Earlier accesses are kept once per distinct (range, mode) with the highest level seen, so
 // a program that runs over the same buffers many times keeps the search lists as short as
@@ -429,6 +432,43 @@ std::vector<std::vector<uint32_t>> node_edges(const std::vector<RecNode>& nodes,
     return waits;
 }
 
+// One chain has to put the nodes in SOME order that respects their dependencies.  Level by
+// level is one; it interleaves independent chains, so that a chain over large buffers finds
+// nothing of its own left in the caches when its next launch comes.  This order follows the
+// recording instead: among the nodes whose dependencies are out, the one whose first launch
+// was recorded first.  A program recorded chain by chain replays chain by chain, one recorded
+// level by level stays as it is, and so do merged launches (their first members were recorded
+// in level order).  Returns the recorded work of every node, in that order.
+std::vector<std::vector<size_t>> stages_in_recording_order(const custos_hip_device* dev, const std::vector<RecNode>& nodes,
+                                                           const std::vector<std::vector<size_t>>& by_level) {
+    std::vector<std::vector<Planned>> groups;
+    for (const auto& of_level : by_level) groups.push_back(group_level(dev, nodes, of_level));
+    const std::vector<std::vector<uint32_t>> waits = node_edges(nodes, groups);
+    std::vector<const Planned*> flat;
+    for (const auto& level : groups)
+        for (const Planned& p : level) flat.push_back(&p);
+    std::vector<std::vector<uint32_t>> followers(flat.size());
+    std::vector<uint32_t> pending(flat.size(), 0);
+    for (uint32_t id = 0; id < flat.size(); id++) {
+        pending[id] = static_cast<uint32_t>(waits[id].size());
+        for (uint32_t q : waits[id]) followers[q].push_back(id);
+    }
+    auto first_recorded = [&](uint32_t id) { return *std::min_element(flat[id]->members.begin(), flat[id]->members.end()); };
+    typedef std::pair<size_t, uint32_t> Ready;  // (first recorded member, node)
+    std::priority_queue<Ready, std::vector<Ready>, std::greater<Ready>> ready;
+    for (uint32_t id = 0; id < flat.size(); id++)
+        if (pending[id] == 0) ready.push({first_recorded(id), id});
+    std::vector<std::vector<size_t>> stages;
+    while (!ready.empty()) {
+        const uint32_t id = ready.top().second;
+        ready.pop();
+        stages.push_back(flat[id]->members);
+        for (uint32_t f : followers[id])
+            if (--pending[f] == 0) ready.push({first_recorded(f), f});
+    }
+    return stages;
+}
+
 // Brute-force check of a built graph's ordering, independent of how the edges were found: every
 // two recorded pieces of work that touch overlapping memory, one of them writing (or one of
 // them with unknown memory use), must sit in different nodes with a path from the earlier one's
@@ -532,7 +572,17 @@ int32_t instantiate(custos_hip_device* dev, custos_hip_graph* g, std::vector<std
 
 int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     std::vector<RecNode>& nodes = dev->recorded;
-    assign_levels(nodes, dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_PER_NODE);
+    const bool serial = dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN || dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN_BY_LEVEL;
+    // The order of a chain only matters where a launch is large enough for the caches to matter;
+    // a recording of small launches keeps the level order and the cheaper analysis.
+    bool follow_recording = false;
+    if (dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN)
+        for (const RecNode& n : nodes) {
+            unsigned long long touched = 0;
+            for (const Access& a : n.acc) touched += a.end - a.begin;
+            follow_recording = follow_recording || touched >= kFollowRecordingFromBytes;
+        }
+    assign_levels(nodes, dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_PER_NODE || follow_recording);
     int max_level = -1;
     for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
     g->recorded = nodes.size();
@@ -544,6 +594,8 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     std::vector<uint64_t> host_table;
     std::vector<std::vector<size_t>> by_level(static_cast<size_t>(max_level + 1));
     for (size_t i = 0; i < nodes.size(); i++) by_level[static_cast<size_t>(nodes[i].level)].push_back(i);
+    // One chain: from here on a "level" is one node, in the order the chain will have.
+    if (follow_recording) by_level = stages_in_recording_order(dev, nodes, by_level);
     // A graph is built to be replayed: its first levels follow its last ones, so the traffic
     // history starts with one pass over the whole graph.
     RecentTraffic history;
@@ -586,7 +638,6 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
 
     // In one chain every order that follows the levels is a valid one, so a short graph of any
     // shape can be replayed as plain launches.
-    const bool serial = dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN;
     if ((chain || serial) && total <= dev->direct_replay_max) {
         for (auto& level : lowered)
             for (LoweredNode& ln : level) g->direct.push_back(std::move(ln));
@@ -716,7 +767,7 @@ int32_t custos_hip_set_graph_direct_replay(custos_hip_device* dev, int32_t max_n
 
 int32_t custos_hip_set_graph_edges(custos_hip_device* dev, int32_t mode) {
     REQUIRE_DEV(dev);
-    if (mode < CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS || mode > CUSTOS_HIP_GRAPH_EDGES_CHAIN)
+    if (mode < CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS || mode > CUSTOS_HIP_GRAPH_EDGES_CHAIN_BY_LEVEL)
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown graph edge mode");
     dev->graph_edges = mode;
     return CUSTOS_HIP_OK;

@@ -29,6 +29,7 @@ pub const LITERALS_AS_PARAMETERS: i32 = 2;
 pub const GRAPH_EDGES_LEVEL_JOINS: i32 = 0;
 pub const GRAPH_EDGES_PER_NODE: i32 = 1;
 pub const GRAPH_EDGES_CHAIN: i32 = 2;
+pub const GRAPH_EDGES_CHAIN_BY_LEVEL: i32 = 3;
 
 #[link(name = "custos_hip")]
 extern "C" {

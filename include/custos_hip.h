@@ -370,17 +370,23 @@ int32_t custos_hip_set_graph_direct_replay(custos_hip_device *dev, int32_t max_n
  * PER_NODE: every node waits only for the nodes whose memory it conflicts with (read-after-write,
  *   write-after-read, write-after-write on overlapping ranges), so independent chains do not wait
  *   for each other; a caller-written kernel still orders itself against everything.
- * CHAIN (default): the (merged) nodes form one chain in level order; nothing runs side by side.
+ * CHAIN (default): the (merged) nodes form one chain; nothing runs side by side.
  *   An element-wise launch of any size worth it fills the chip by itself, and on this runtime a
  *   dependency between branches of a graph costs several times what a node of a chain costs:
  *   measured 1.3 to 4.7 times faster than LEVEL_JOINS and up to 2.2 times faster than PER_NODE
  *   on graphs of 16 to 768 nodes; only independent chains of launches that stream hundreds of
  *   MiB each replayed 3 % faster with PER_NODE. A graph of at most
- *   custos_hip_set_graph_direct_replay nodes is then replayed as plain launches. */
+ *   custos_hip_set_graph_direct_replay nodes is then replayed as plain launches.
+ * CHAIN_BY_LEVEL: one chain, always level by level. CHAIN differs from it only for recordings
+ *   with launches of 8 MiB and more: there the chain follows the recording where the
+ *   dependencies allow (among the nodes that are ready, the one recorded first), so that a
+ *   program recorded chain by chain over large buffers also replays chain by chain and finds its
+ *   data in the caches, instead of streaming every buffer from memory at every level. */
 enum custos_hip_graph_edges {
     CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS = 0,
     CUSTOS_HIP_GRAPH_EDGES_PER_NODE = 1,
-    CUSTOS_HIP_GRAPH_EDGES_CHAIN = 2
+    CUSTOS_HIP_GRAPH_EDGES_CHAIN = 2,
+    CUSTOS_HIP_GRAPH_EDGES_CHAIN_BY_LEVEL = 3
 };
 int32_t custos_hip_set_graph_edges(custos_hip_device *dev, int32_t mode);
 /* With `enabled`, capture_end checks every graph it builds by brute force before instantiating it:

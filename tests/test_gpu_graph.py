@@ -218,7 +218,8 @@ def checked_graphs(hip):
     hip.set_graph_edges(capi.GRAPH_EDGES_CHAIN)
 
 
-EDGE_MODES = {"level joins": capi.GRAPH_EDGES_LEVEL_JOINS, "per node": capi.GRAPH_EDGES_PER_NODE, "chain": capi.GRAPH_EDGES_CHAIN}
+EDGE_MODES = {"level joins": capi.GRAPH_EDGES_LEVEL_JOINS, "per node": capi.GRAPH_EDGES_PER_NODE, "chain": capi.GRAPH_EDGES_CHAIN,
+              "chain by level": capi.GRAPH_EDGES_CHAIN_BY_LEVEL}
 
 
 @pytest.mark.parametrize("edges", list(EDGE_MODES))
@@ -346,6 +347,7 @@ def test_per_node_edges_let_independent_chains_run_apart(checked_graphs, oracle)
     # per-node: 3 edges inside the first chain, 1 inside the second, 2 into the caller-written kernel, 2 out of it
     assert edges["per node"] == 8
     assert edges["chain"] == 8          # nine nodes one after the other
+    assert edges["chain by level"] == 8
     assert edges["level joins"] == 11
     want = x
     for _ in range(4):
@@ -354,6 +356,64 @@ def test_per_node_edges_let_independent_chains_run_apart(checked_graphs, oracle)
     program(ea, eb)
     hip.sync()
     assert_bits_equal(ea.read(), want)
+
+
+@pytest.mark.parametrize("edges", ["chain", "chain by level", "per node"])
+def test_large_launches_in_recording_order(checked_graphs, oracle, edges):
+    """Recordings with launches of 8 MiB and more: one chain follows the recording where the
+    dependencies allow.  Random programs over four buffers of 2^20 elements (in-place updates, two-operand
+    launches between buffers, clears, a caller-written kernel), every graph checked by the library's ordering
+    check, replays compared with eager execution bit for bit."""
+    hip = checked_graphs
+    hip.set_graph_edges(EDGE_MODES[edges])
+    hip.set_graph_direct_replay(0)
+    n = 1 << 20
+    rng = np.random.default_rng(77)
+    fns1 = [lambda v: v.mul(1.25).add(0.5), lambda v: v.neg().max(-3.0), lambda v: v.abs().sqrt()]
+    fns2 = [lambda p, q: p.add(q), lambda p, q: p.mul(q).sub(0.125)]
+    halve = """extern "C" __global__ void halve(float* p, unsigned long long n) {
+        unsigned long long i = blockIdx.x * (unsigned long long)blockDim.x + threadIdx.x;
+        if (i < n) p[i] = p[i] * 0.5f;
+    }"""
+    try:
+        for trial in range(4):
+            init = [synth.uniform_f32(200 + trial * 4 + i, n, -2, 2) for i in range(4)]
+            program = []
+            for chain in rng.permutation(4):                      # chain by chain, as user code records
+                for _ in range(int(rng.integers(1, 4))):
+                    program.append(("u", int(rng.integers(len(fns1))), int(chain)))
+            for _ in range(3):                                     # then work across the chains
+                a, b, o = (int(v) for v in rng.choice(4, size=3, replace=False))
+                program.append(("b", int(rng.integers(len(fns2))), a, b, o))
+            program.insert(int(rng.integers(len(program))), ("k", int(rng.integers(4))))
+            program.append(("c", int(rng.integers(4))))
+            program.append(("u", 0, int(rng.integers(4))))
+
+            def run(bufs):
+                for op in program:
+                    if op[0] == "u":
+                        hip.apply_fn(bufs[op[2]], fns1[op[1]], out=bufs[op[2]])
+                    elif op[0] == "b":
+                        hip.apply_fn2(bufs[op[2]], bufs[op[3]], fns2[op[1]], out=bufs[op[4]])
+                    elif op[0] == "k":
+                        hip.launch_kernel(halve, "halve", ((n + 255) // 256, 1, 1), (256, 1, 1), 0, [bufs[op[1]], np.uint64(n)])
+                    else:
+                        bufs[op[1]].clear()
+
+            eager = [hip.buffer(x) for x in init]
+            lazy = [hip.buffer(x) for x in init]
+            hip.capture_begin()
+            run(lazy)
+            g = hip.capture_end()
+            for replay in range(2):
+                run(eager)
+                g.launch()
+                hip.sync()
+                for i in range(4):
+                    assert_bits_equal(lazy[i].read(), eager[i].read(), f"{edges}, trial {trial}, replay {replay}, buffer {i}")
+            g.destroy()
+    finally:
+        hip.set_graph_direct_replay(4)
 
 
 def test_ordering_check_accepts_merged_and_fenced_graphs(checked_graphs):
@@ -431,7 +491,7 @@ def test_graph_settings_and_reuse_reject_bad_calls(hip):
     import ctypes as C
     out = C.c_void_p()
     assert hip.lib.custos_hip_capture_end_reuse(hip.handle, None, C.byref(out)) == capi.ERR_CAPTURE_STATE   # not recording
-    assert hip.lib.custos_hip_set_graph_edges(hip.handle, 3) == capi.ERR_INVALID_ARGUMENT
+    assert hip.lib.custos_hip_set_graph_edges(hip.handle, 4) == capi.ERR_INVALID_ARGUMENT
     assert hip.lib.custos_hip_set_graph_edges(hip.handle, -1) == capi.ERR_INVALID_ARGUMENT
     other = custos_amd.HIP(0)
     try:
