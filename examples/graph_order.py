@@ -1,5 +1,6 @@
-"""How a recorded program replays under the three node orders of a built graph
-(`custos_hip_set_graph_edges`): joins between dependency levels, an edge per dependency, one chain.
+"""How a recorded program replays under the node orders of a built graph (`custos_hip_set_graph_edges`):
+joins between dependency levels, an edge per dependency, one chain level by level, and one chain that
+follows the recording where launches are large (the default).
 
     python3 examples/graph_order.py            # needs an AMD GPU; prints microseconds per replay
 
@@ -14,7 +15,8 @@ import numpy as np
 from custos_amd import capi
 from custos_amd.device import HIP
 
-ORDERS = (("level joins", capi.GRAPH_EDGES_LEVEL_JOINS), ("per node", capi.GRAPH_EDGES_PER_NODE), ("chain", capi.GRAPH_EDGES_CHAIN))
+ORDERS = (("level joins", capi.GRAPH_EDGES_LEVEL_JOINS), ("per node", capi.GRAPH_EDGES_PER_NODE),
+          ("chain by level", capi.GRAPH_EDGES_CHAIN_BY_LEVEL), ("chain", capi.GRAPH_EDGES_CHAIN))
 SOURCES = ("((x * 1.0001) + 0.5)", "max(x, -3.0)", "(x - 0.25)", "abs(x)", "(x * 0.999)", "(x + 0.125)", "min(x, 7.0)", "-(x)")
 
 
@@ -26,11 +28,17 @@ def main():
     def launch(k, buf):
         capi.check(dev.lib.custos_hip_apply_fn(dev.handle, kernels[k], buf.ptr, buf.ptr, buf.len), dev.handle)
 
-    def chains(lengths, elements, kernel_of=lambda chain, depth: chain):
-        """One in-place chain of launches per buffer; recorded level by level like interleaved user code."""
+    def chains(lengths, elements, kernel_of=lambda chain, depth: chain, chain_by_chain=False):
+        """One in-place chain of launches per buffer; recorded level by level like interleaved user code,
+        or chain by chain."""
         bufs = [dev.alloc(n) for n in elements]
 
         def record():
+            if chain_by_chain:
+                for chain, buf in enumerate(bufs):
+                    for depth in range(lengths[chain]):
+                        launch(kernel_of(chain, depth) % len(kernels), buf)
+                return
             for depth in range(max(lengths)):
                 for chain, buf in enumerate(bufs):
                     if depth < lengths[chain]:
@@ -43,6 +51,8 @@ def main():
         ("8 chains of 2..16 launches, 256 KiB buffers", chains([2 * (c + 1) for c in range(8)], [1 << 16] * 8)),
         ("8 chains of 4 launches, another kernel at every level, 1 MiB buffers", chains([4] * 8, [1 << 18] * 8, lambda c, d: c + d)),
         ("4 chains of 4 launches, 64 MiB buffers", chains([4] * 4, [1 << 24] * 4, lambda c, d: c + d)),
+        ("16 chains of 4 launches, 16 MiB buffers, recorded chain by chain",
+         chains([4] * 16, [1 << 22] * 16, lambda c, d: c + d, chain_by_chain=True)),
     ]
     print(f"{'program':70s} {'nodes':>5s} " + " ".join(f"{name:>14s}" for name, _ in ORDERS))
     for title, (bufs, record) in programs:
