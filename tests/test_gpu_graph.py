@@ -376,7 +376,8 @@ def test_large_launches_in_recording_order(checked_graphs, oracle, edges):
         if (i < n) p[i] = p[i] * 0.5f;
     }"""
     try:
-        for trial in range(4):
+        import os
+        for trial in range(int(os.environ.get("CUSTOS_LARGE_RANDOM_PROGRAMS", "4"))):   # more for a longer run
             init = [synth.uniform_f32(200 + trial * 4 + i, n, -2, 2) for i in range(4)]
             program = []
             for chain in rng.permutation(4):                      # chain by chain, as user code records
