@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <thread>
 
 #include "runtime.hpp"
 
@@ -29,10 +30,23 @@ constexpr size_t kStagedReadMax = 64u << 10;  // reads and writes up to this siz
 constexpr size_t kWriteSlots = 16;            // staging slots of short writes (the first slot of the block is the read's)
 
 // Waits for the compute stream.  The blocking wait of the runtime takes about 9 us to
-// notice that a short job has finished -- three times the job itself for a small replayed
-// graph.  So the stream writes a sequence number into pinned host memory behind the
-// work, and the host polls that word for a short while before it falls back to the
-// blocking wait.
+// notice that a job has finished -- three times the job itself for a small replayed
+// graph, and a gap in front of the next launch for a large one.  So the stream writes a
+// sequence number into pinned host memory behind the work, and the host polls that word.
+// How long it polls follows the work: the wait remembers how long the last wait for the
+// same work took (per graph when exactly the launch of a graph is waited for, else per
+// stream).  A graph launch predicted to take milliseconds is slept through up to half a
+// millisecond before its predicted end; the rest is polled with a pause instruction, for at least 2 ms
+// and at least twice the prediction.  Only work that outlasts that window -- work nothing
+// predicted -- ends in the blocking wait, where 9 us no longer matter.
+static inline void cpu_pause() {
+#if defined(__x86_64__) || defined(__i386__)
+    __builtin_ia32_pause();
+#else
+    std::this_thread::yield();
+#endif
+}
+
 static hipError_t wait_compute_stream_now(custos_hip_device* dev) {
     if (!dev->done_flag) return hipStreamSynchronize(dev->stream);
     const uint32_t seq = ++dev->done_seq;
@@ -41,13 +55,38 @@ static hipError_t wait_compute_stream_now(custos_hip_device* dev) {
         (void)hipGetLastError();
         return hipStreamSynchronize(dev->stream);
     }
-    const auto start = std::chrono::steady_clock::now();
+    using clock = std::chrono::steady_clock;
+    using std::chrono::nanoseconds;
+    custos_hip_graph* const graph = dev->graphs_since_wait == 1 && !dev->launches_since_wait ? dev->graph_since_wait : nullptr;
+    const uint64_t predicted_ns = graph && graph->last_wait_ns ? graph->last_wait_ns : dev->last_wait_ns;
+    const uint64_t window_ns = std::min<uint64_t>(std::max<uint64_t>(2000000, 2 * predicted_ns), 50000000);
+    const auto start = clock::now();
     volatile uint32_t* flag = dev->done_flag;
-    for (unsigned spins = 0;; spins++) {
-        if (*flag == seq) return hipSuccess;
-        if ((spins & 255) == 255 && std::chrono::steady_clock::now() - start > std::chrono::microseconds(200))
-            return hipStreamSynchronize(dev->stream);
+    hipError_t result = hipSuccess;
+    bool done = *flag == seq;
+    // (only a prediction for exactly this work is slept on: a wrong one would add latency)
+    if (graph && graph->last_wait_ns > 2000000) {
+        const auto sleep_until = start + nanoseconds(graph->last_wait_ns - 500000);
+        while (!done && clock::now() < sleep_until) {
+            std::this_thread::sleep_for(std::min<nanoseconds>(nanoseconds(1000000), sleep_until - clock::now()));
+            done = *flag == seq;
+        }
     }
+    for (unsigned spins = 0; !done; spins++) {
+        cpu_pause();
+        done = *flag == seq;
+        if (!done && (spins & 63) == 63 && clock::now() - start > nanoseconds(window_ns)) {
+            result = hipStreamSynchronize(dev->stream);
+            break;
+        }
+    }
+    const uint64_t took = static_cast<uint64_t>(std::chrono::duration_cast<nanoseconds>(clock::now() - start).count());
+    dev->last_wait_ns = took;
+    if (graph) graph->last_wait_ns = took;
+    dev->graph_since_wait = nullptr;
+    dev->graphs_since_wait = 0;
+    dev->launches_since_wait = false;
+    return result;
 }
 
 // `waits_begun` / `waits_done` number the waits: work issued while `waits_begun` was w has
@@ -146,10 +185,33 @@ static int32_t launch_stage_copy(custos_hip_device* dev, uint64_t dst, uint64_t 
     if (head > bytes) head = bytes;
     const unsigned long long n_vec = (bytes - head) / 16;
     const unsigned int grid = static_cast<unsigned int>(std::max(1ull, (n_vec + kFillBlock - 1) / kFillBlock));
+    dev->launches_since_wait = true;
     hipLaunchKernelGGL(custos_stage_copy, dim3(grid), dim3(kFillBlock), 0, dev->stream,
                        reinterpret_cast<unsigned char*>(dst), reinterpret_cast<const unsigned char*>(src),
                        static_cast<unsigned long long>(bytes), head, n_vec);
     HIP_TRY(dev, hipGetLastError());
+    return CUSTOS_HIP_OK;
+}
+
+// A short write costs the runtime about 14 us, most of it the wait that lets the caller
+// reuse `src`.  Up to 64 KiB the data is copied into a pinned staging slot (at the
+// destination's 16-byte phase) and a copy kernel moves it from there, in stream
+// order and without a wait; a slot is reused once a wait that began after its launch has
+// finished, and a seventeenth write in a row without one waits first.
+// Needs the staging memory, at most kStagedReadMax bytes, and a device that is not recording.
+static int32_t staged_write(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes) {
+    const size_t slot = dev->write_slot;
+    static_assert(kWriteSlots == std::tuple_size<decltype(dev->write_slot_issued)>::value, "one entry per slot");
+    if (dev->write_slot_used[slot] && dev->waits_done <= dev->write_slot_issued[slot])
+        HIP_TRY(dev, wait_compute_stream(dev));
+    const uint64_t phase = dst & 15;
+    const size_t offset = (kStagedReadMax + 16) * (1 + slot) + phase;
+    std::memcpy(dev->read_stage + offset, src, bytes);
+    int32_t rc = launch_stage_copy(dev, dst, dev->read_stage_dev + offset, bytes);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    dev->write_slot_issued[slot] = dev->waits_begun;
+    dev->write_slot_used[slot] = true;
+    dev->write_slot = (slot + 1) % kWriteSlots;
     return CUSTOS_HIP_OK;
 }
 
@@ -180,6 +242,7 @@ int32_t launch_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t b
             dev->recorded.push_back(std::move(node));
             return CUSTOS_HIP_OK;
         }
+        dev->launches_since_wait = true;
         HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src), bytes,
                                     hipMemcpyDeviceToDevice, dev->stream));
         return CUSTOS_HIP_OK;
@@ -208,6 +271,7 @@ int32_t launch_fill(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStre
         return CUSTOS_HIP_OK;
     }
     unsigned int grid = fill_grid(dev, n_vec);
+    if (stream == dev->stream) dev->launches_since_wait = true;
     if (pattern)
         hipLaunchKernelGGL(custos_fill_pattern, dim3(grid), dim3(kFillBlock), 0, stream,
                            reinterpret_cast<unsigned char*>(dptr), static_cast<unsigned long long>(bytes), head, n_vec,
@@ -495,26 +559,7 @@ int32_t custos_hip_write(custos_hip_device* dev, uint64_t dst, const void* src, 
         HIP_TRY(dev, hipStreamSynchronize(dev->transfer));
         return CUSTOS_HIP_OK;
     }
-    // A short write costs the runtime about 14 us, most of it the wait that lets the caller
-    // reuse `src`.  Up to 64 KiB the data is copied into a pinned staging slot (at the
-    // destination's 16-byte phase) and a copy kernel moves it from there, in stream
-    // order and without a wait; a slot is reused once a wait that began after its launch has
-    // finished, and a seventeenth write in a row without one waits first.
-    if (dev->read_stage && bytes <= kStagedReadMax) {
-        const size_t slot = dev->write_slot;
-        static_assert(kWriteSlots == std::tuple_size<decltype(dev->write_slot_issued)>::value, "one entry per slot");
-        if (dev->write_slot_used[slot] && dev->waits_done <= dev->write_slot_issued[slot])
-            HIP_TRY(dev, wait_compute_stream(dev));
-        const uint64_t phase = dst & 15;
-        const size_t offset = (kStagedReadMax + 16) * (1 + slot) + phase;
-        std::memcpy(dev->read_stage + offset, src, bytes);
-        int32_t rc = launch_stage_copy(dev, dst, dev->read_stage_dev + offset, bytes);
-        if (rc != CUSTOS_HIP_OK) return rc;
-        dev->write_slot_issued[slot] = dev->waits_begun;
-        dev->write_slot_used[slot] = true;
-        dev->write_slot = (slot + 1) % kWriteSlots;
-        return CUSTOS_HIP_OK;
-    }
+    if (dev->read_stage && bytes <= kStagedReadMax) return staged_write(dev, dst, src, bytes);
     HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), src, bytes, hipMemcpyHostToDevice, dev->stream));
     // the caller may reuse `src` right away
     HIP_TRY(dev, hipStreamSynchronize(dev->stream));

@@ -666,6 +666,8 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
 }
 
 int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
+    dev->graph_since_wait = g;
+    dev->graphs_since_wait++;
     if (g->exec) {
         HIP_TRY(dev, hipGraphLaunch(g->exec, dev->stream));
         return CUSTOS_HIP_OK;
@@ -819,6 +821,10 @@ int32_t custos_hip_graph_destroy(custos_hip_device* dev, custos_hip_graph* graph
     auto it = std::find(dev->graphs.begin(), dev->graphs.end(), graph);
     if (it == dev->graphs.end()) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph does not belong to this device");
     dev->graphs.erase(it);
+    if (dev->graph_since_wait == graph) {
+        dev->graph_since_wait = nullptr;
+        dev->launches_since_wait = true;  // the pending work is no longer that of one known graph
+    }
     HIP_TRY(dev, hipStreamSynchronize(dev->stream));
     destroy_graph(graph);
     return CUSTOS_HIP_OK;

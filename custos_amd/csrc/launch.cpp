@@ -222,6 +222,7 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     // the expression's literals that are launch parameters: one block by value
     if (k->spec.consts.n_params > 0) args.push_back(k->spec.consts.bytes.data());
     args.push_back(&rev);
+    dev->launches_since_wait = true;
     HIP_TRY(dev, hipModuleLaunchKernel(k->fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
                                        1, 1, 0, dev->stream, args.data(), nullptr));
     return CUSTOS_HIP_OK;
@@ -308,6 +309,7 @@ int32_t custos_hip_source_launch(custos_hip_device* dev, custos_hip_kernel* kern
         return CUSTOS_HIP_OK;
     }
     std::vector<void*> args(params, params + n_params);
+    dev->launches_since_wait = true;
     HIP_TRY(dev, hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
                                        shared_mem_bytes, dev->stream, args.data(), nullptr));
     return CUSTOS_HIP_OK;

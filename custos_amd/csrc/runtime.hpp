@@ -69,6 +69,8 @@ struct custos_hip_graph {
     // (merging, edge mode, direct replay limit) -- see custos_hip_capture_end_reuse
     std::vector<uint64_t> signature;
     std::array<uint64_t, 3> built_with{};
+    // how long the last wait took that waited for one launch of this graph and nothing else
+    uint64_t last_wait_ns = 0;
 };
 
 // One recorded piece of work (while the device is recording, nothing is launched).
@@ -143,6 +145,13 @@ struct custos_hip_device {
     uint32_t* done_flag = nullptr;  // pinned host word the compute stream writes sequence numbers to
     void* done_flag_dev = nullptr;  // its device address
     uint32_t done_seq = 0;
+    // What the next wait waits for, and how long the last one took (the poll window of a wait
+    // follows the work, see wait_compute_stream_now in device.hip): graph launches and other
+    // work issued on the compute stream since the last wait.
+    uint64_t last_wait_ns = 0;
+    custos_hip_graph* graph_since_wait = nullptr;
+    uint32_t graphs_since_wait = 0;
+    bool launches_since_wait = false;
     unsigned char* read_stage = nullptr;  // pinned host memory short reads (first slot) and writes are staged in
     uint64_t read_stage_dev = 0;          // its device address
     uint64_t waits_begun = 0, waits_done = 0;  // waits for the compute stream, numbered
