@@ -135,6 +135,7 @@ PROTOTYPES = {
     "custos_hip_apply_fn": (C.c_int32, [_P, _P, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_apply_fn2": (C.c_int32, [_P, _P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_apply_fn_n": (C.c_int32, [_P, _P, C.POINTER(C.c_uint64), C.c_int32, C.c_uint64, C.c_size_t]),
+    "custos_hip_apply_fn_many_noalloc": (C.c_int32, [_P, _P, C.POINTER(C.c_uint64), C.c_int32, C.c_size_t, C.c_size_t]),
     "custos_hip_fill": (C.c_int32, [_P, C.c_uint64, C.c_size_t, C.c_void_p, C.c_size_t]),
     "custos_hip_add_unary_grad": (C.c_int32, [_P, _P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_capture_begin": (C.c_int32, [_P]),

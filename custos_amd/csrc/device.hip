@@ -29,6 +29,30 @@ const std::string& thread_last_error() { return g_last_error; }
 constexpr size_t kStagedReadMax = 64u << 10;  // reads and writes up to this size go through pinned staging memory
 constexpr size_t kWriteSlots = 16;            // staging slots of short writes (the first slot of the block is the read's)
 
+// Operand table of custos_hip_apply_fn_many_noalloc: device memory that belongs to the
+// library's code object, so the entry point never allocates.  Every GPU the library runs on
+// holds its own copy (64 KiB) at its own address until the process ends; `scratch` itself is
+// only the host-side name of the symbol, the address on device d is g_scratch_ptr[d], looked
+// up once per device when the first handle on that device is created.
+constexpr size_t kScratchWords = 8192;
+static __device__ __align__(256) unsigned long long scratch[kScratchWords];
+constexpr int kMaxDevices = 64;
+static unsigned long long* g_scratch_ptr[kMaxDevices];
+static_assert(kScratchWords * sizeof(unsigned long long) <= kStagedReadMax, "the table travels through one staging slot");
+
+// With device `idx` current: the address of that device's copy of `scratch`.
+static hipError_t scratch_address(int idx, unsigned long long** out) {
+    if (idx < 0 || idx >= kMaxDevices) return hipErrorInvalidDevice;
+    if (!g_scratch_ptr[idx]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        g_scratch_ptr[idx] = static_cast<unsigned long long*>(p);
+    }
+    *out = g_scratch_ptr[idx];
+    return hipSuccess;
+}
+
 // Waits for the compute stream.  The blocking wait of the runtime takes about 9 us to
 // notice that a job has finished -- three times the job itself for a small replayed
 // graph, and a gap in front of the next launch for a large one.  So the stream writes a
@@ -347,6 +371,7 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
     HIP_TRY(nullptr, hipEventCreate(&dev->t0));
     HIP_TRY(nullptr, hipEventCreate(&dev->t1));
     dev->pool_limit = dev->props.totalGlobalMem / 4;
+    HIP_TRY(nullptr, scratch_address(idx, &dev->scratch_table));
     // completion word for short waits (pinned, mapped host memory); optional
     void* flag = nullptr;
     if (hipHostMalloc(&flag, 64, hipHostMallocMapped) == hipSuccess) {
@@ -619,6 +644,109 @@ int32_t custos_hip_fill(custos_hip_device* dev, uint64_t dptr, size_t bytes, con
     std::memcpy(pattern, repeated, 16);
     const bool zeros = (pattern[0] | pattern[1] | pattern[2] | pattern[3]) == 0;
     return launch_fill(dev, dptr, bytes, dev->stream, zeros ? nullptr : pattern);
+}
+
+// ---- many launches of one kernel in one grid, without any allocation ----
+
+int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kernel* kernel, const uint64_t* operands,
+                                         int32_t operands_per_set, size_t n_sets, size_t n) {
+    REQUIRE_DEV(dev);
+    if (!kernel || !operands) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel or operand table");
+    if (kernel->spec.kind == Kind::Source || !kernel->fn_batched)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel has no entry point for merged launches");
+    if (dev->capturing)
+        return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the allocation-free merged launch cannot be recorded");
+    const int n_ptrs = kernel->spec.kind == Kind::UnaryGrad ? 3 : kernel->spec.expr.n_vars + 1;
+    if (operands_per_set != n_ptrs)
+        return set_error(dev, CUSTOS_HIP_ERR_ARITY_MISMATCH,
+                         "kernel takes " + std::to_string(n_ptrs) + " addresses per operand set, got " + std::to_string(operands_per_set));
+    if (n_sets == 0 || n == 0) return CUSTOS_HIP_OK;
+    if (!dev->read_stage || !dev->scratch_table)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "the device handle has no staging memory for the operand table");
+    if (n > (1ull << 40)) return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "more than 2^40 elements");
+    const std::vector<unsigned char>& values = kernel->spec.consts.bytes;
+    const size_t const_words = (values.size() + 7) / 8;
+    const size_t row_words = static_cast<size_t>(n_ptrs) + const_words;
+    if (n_sets > kScratchWords / row_words)
+        return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE,
+                         "the static operand table holds " + std::to_string(kScratchWords / row_words) + " operand sets of this kernel (" +
+                             std::to_string(kScratchWords * 8) + " bytes), got " + std::to_string(n_sets));
+    // Operand checks on the host, before anything is launched: aligned, no partial overlap
+    // inside a set (`out == in` exactly is fine), and no set writes what another set touches.
+    const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(kernel->spec.dtype);
+    const int written = kernel->spec.kind == Kind::UnaryGrad ? 1 : n_ptrs - 1;
+    struct Span {
+        uint64_t begin;
+        uint32_t set;
+        bool write;
+    };
+    std::vector<Span> spans;
+    spans.reserve(n_sets * static_cast<size_t>(n_ptrs));
+    for (size_t s = 0; s < n_sets; s++) {
+        const uint64_t* row = operands + s * static_cast<size_t>(n_ptrs);
+        for (int i = 0; i < n_ptrs; i++) {
+            if (row[i] == 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null device pointer");
+            if (row[i] & 15)
+                return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "operands of a merged launch are 16-byte aligned");
+            if (i != written && row[i] != row[written] && row[i] < row[written] + bytes && row[written] < row[i] + bytes)
+                return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP, "the output range partially overlaps an input range");
+            spans.push_back({row[i], static_cast<uint32_t>(s), i == written});
+        }
+    }
+    std::sort(spans.begin(), spans.end(), [](const Span& a, const Span& b) { return a.begin < b.begin; });
+    // sweep by start address: the furthest-reaching earlier span of any kind and the furthest
+    // written one, each with a runner-up from another set
+    struct Reach {
+        uint64_t end[2] = {0, 0};
+        uint32_t set[2] = {0xffffffffu, 0xffffffffu};
+        void add(uint64_t e, uint32_t s) {
+            if (s == set[0]) {
+                end[0] = std::max(end[0], e);
+            } else if (e > end[0]) {
+                end[1] = end[0], set[1] = set[0];
+                end[0] = e, set[0] = s;
+            } else if (e > end[1]) {
+                end[1] = e, set[1] = s;
+            }
+        }
+        uint64_t other_than(uint32_t s) const { return set[0] != s ? end[0] : end[1]; }
+    } any, writes;
+    for (const Span& sp : spans) {
+        if ((sp.write && any.other_than(sp.set) > sp.begin) || writes.other_than(sp.set) > sp.begin)
+            return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP, "an operand set writes memory that another operand set uses");
+        any.add(sp.begin + bytes, sp.set);
+        if (sp.write) writes.add(sp.begin + bytes, sp.set);
+    }
+    const Tuning& t = kernel->spec.tuning;
+    const unsigned long long count = n, n_vec = n / static_cast<unsigned long long>(kernel->spec.vec_elems);
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+    unsigned long long tiles_per_seg = std::max(1ull, (n_vec + tile_vecs - 1) / tile_vecs);
+    if (tiles_per_seg * n_sets > (1ull << 31) - 1)
+        return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
+    // table rows as the `_batched` entry point reads them: addresses, then the literal parameters
+    std::vector<uint64_t> table(n_sets * row_words);
+    for (size_t s = 0; s < n_sets; s++) {
+        uint64_t* row = table.data() + s * row_words;
+        std::memcpy(row, operands + s * static_cast<size_t>(n_ptrs), static_cast<size_t>(n_ptrs) * 8);
+        for (size_t w = 0; w < const_words; w++) {
+            uint64_t word = 0;
+            std::memcpy(&word, values.data() + w * 8, std::min<size_t>(8, values.size() - w * 8));
+            row[n_ptrs + w] = word;
+        }
+    }
+    // The table goes through a pinned staging slot and a copy kernel on the compute stream: it
+    // lands behind the previous call's launch, which still reads the table.
+    const uint64_t table_dev = reinterpret_cast<uint64_t>(dev->scratch_table);
+    int32_t rc = staged_write(dev, table_dev, table.data(), table.size() * 8);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    unsigned long long rev = 0;
+    uint64_t table_arg = table_dev;
+    unsigned long long count_arg = count, n_vec_arg = n_vec;
+    void* args[] = {&table_arg, &count_arg, &n_vec_arg, &tiles_per_seg, &rev};
+    dev->launches_since_wait = true;
+    HIP_TRY(dev, hipModuleLaunchKernel(kernel->fn_batched, static_cast<unsigned int>(tiles_per_seg * n_sets), 1, 1,
+                                       static_cast<unsigned int>(t.block_threads), 1, 1, 0, dev->stream, args, nullptr));
+    return CUSTOS_HIP_OK;
 }
 
 // ---- timing ----

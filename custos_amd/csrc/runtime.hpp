@@ -152,6 +152,7 @@ struct custos_hip_device {
     custos_hip_graph* graph_since_wait = nullptr;
     uint32_t graphs_since_wait = 0;
     bool launches_since_wait = false;
+    unsigned long long* scratch_table = nullptr;  // this device's copy of the library's static operand table
     unsigned char* read_stage = nullptr;  // pinned host memory short reads (first slot) and writes are staged in
     uint64_t read_stage_dev = 0;          // its device address
     uint64_t waits_begun = 0, waits_done = 0;  // waits for the compute stream, numbered

@@ -251,6 +251,21 @@ class HIP:
         self._check(self.lib.custos_hip_apply_fn_n(self.handle, kernel, ptrs, len(ins), out.ptr, ins[0].len))
         return out
 
+    def apply_fn_many_noalloc(self, kernel, operand_sets, n: int) -> None:
+        """One grid over many operand sets of `n` elements each, the operand table in the library's
+        static device array: no allocation anywhere on the way.  `operand_sets`: per set the
+        buffers (or addresses) in the order of the kernel's pointer parameters."""
+        rows = [[b.ptr if isinstance(b, Buffer) else int(b) for b in row] for row in operand_sets]
+        per_set = len(rows[0]) if rows else 0
+        if any(len(r) != per_set for r in rows):
+            raise ValueError("operand sets differ in their number of operands")
+        for row, given in zip(rows, operand_sets):
+            for b in given:
+                if isinstance(b, Buffer) and b.len < n:
+                    raise ValueError(f"operand of {b.len} elements in a launch over {n}")
+        flat = (C.c_uint64 * max(1, len(rows) * per_set))(*[p for r in rows for p in r])
+        self._check(self.lib.custos_hip_apply_fn_many_noalloc(self.handle, kernel, flat, per_set, len(rows), n))
+
     def fused_apply_fn(self, buf: Buffer, ops, out: Buffer | None = None) -> Buffer:
         """The op `unary_fuse_op` returns: all `ops` applied in sequence in one kernel."""
         src = fused_source(ops, buf.dtype)

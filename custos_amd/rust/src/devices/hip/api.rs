@@ -94,6 +94,8 @@ extern "C" {
                                 n: usize) -> i32;
     pub fn custos_hip_apply_fn_n(dev: *mut HipDeviceHandle, kernel: *mut HipKernel, ins: *const u64, n_ins: i32,
                                  out: u64, n: usize) -> i32;
+    pub fn custos_hip_apply_fn_many_noalloc(dev: *mut HipDeviceHandle, kernel: *mut HipKernel, operands: *const u64,
+                                            operands_per_set: i32, n_sets: usize, n: usize) -> i32;
     pub fn custos_hip_add_unary_grad(dev: *mut HipDeviceHandle, kernel: *mut HipKernel, lhs: u64, lhs_grad: u64,
                                      out_grad: u64, n: usize) -> i32;
     pub fn custos_hip_capture_begin(dev: *mut HipDeviceHandle) -> i32;

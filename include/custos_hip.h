@@ -334,6 +334,30 @@ int32_t custos_hip_apply_fn_n(custos_hip_device *dev, custos_hip_kernel *kernel,
 int32_t custos_hip_add_unary_grad(custos_hip_device *dev, custos_hip_kernel *kernel, uint64_t lhs,
                                   uint64_t lhs_grad, uint64_t out_grad, size_t n);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory where they
+ * launch: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * What it does is what a recording of `n_sets` independent launches of `kernel` does when it is
+ * built and replayed (custos_hip_capture_end merges them into one grid whose operand addresses
+ * sit in a device table that the graph allocates): ONE grid over `n_sets` operand sets of `n`
+ * elements each, but with the table in a static device array of the library (64 KiB per GPU,
+ * held until the process ends) instead of an allocation.  This call never calls hipMalloc,
+ * hipFree, or compiles or loads code: `kernel` runs exactly as custos_hip_expr_compile built it.
+ * `operands`: `n_sets` rows of `operands_per_set` device addresses in the order of the
+ * kernel's pointer parameters (apply kernel: the inputs, then the output; unary-gradient kernel:
+ * lhs, lhs_grad, out_grad), every address 16-byte aligned.  A row may name its output as one of
+ * its inputs (exact alias); partial overlap inside a row, and a row that writes what another row
+ * uses, are rejected (CUSTOS_HIP_ERR_BAD_OVERLAP).
+ * Limit: n_sets * (operands_per_set + ceil(bytes of the kernel's literal parameters / 8)) <= 8192
+ * table words, else CUSTOS_HIP_ERR_TOO_LARGE (2048 sets of a three-operand kernel).  Not legal
+ * while the device records (CUSTOS_HIP_ERR_CAPTURE_STATE).
+ * All calls on one GPU share that GPU's table, which keeps the rows of the last call (nothing in
+ * it has to start at zero: every row a launch reads is rewritten by its call).  Calls through one
+ * device handle are ordered by its compute stream; calls through two handles on the same GPU that
+ * overlap in time race on the table. */
+int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device *dev, custos_hip_kernel *kernel,
+                                         const uint64_t *operands, int32_t operands_per_set,
+                                         size_t n_sets, size_t n);
+
 /* ---- lazy run: capture once, replay (src/devices/cuda/lazy.rs:10-72) ---- */
 
 /* LazySetup::lazy_setup: from here on launches/clears/copies are recorded, not run.
