@@ -718,8 +718,9 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
         if (sp.write) writes.add(sp.begin + bytes, sp.set);
     }
     const Tuning& t = kernel->spec.tuning;
+    const ResolvedShape shape = resolve_shape(dev, kernel, static_cast<unsigned long long>(n_sets) * n_ptrs * bytes);
     const unsigned long long count = n, n_vec = n / static_cast<unsigned long long>(kernel->spec.vec_elems);
-    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * shape.unroll;
     unsigned long long tiles_per_seg = std::max(1ull, (n_vec + tile_vecs - 1) / tile_vecs);
     if (tiles_per_seg * n_sets > (1ull << 31) - 1)
         return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
@@ -739,10 +740,10 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
     const uint64_t table_dev = reinterpret_cast<uint64_t>(dev->scratch_table);
     int32_t rc = staged_write(dev, table_dev, table.data(), table.size() * 8);
     if (rc != CUSTOS_HIP_OK) return rc;
-    unsigned long long rev = 0;
+    unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, false);
     uint64_t table_arg = table_dev;
     unsigned long long count_arg = count, n_vec_arg = n_vec;
-    void* args[] = {&table_arg, &count_arg, &n_vec_arg, &tiles_per_seg, &rev};
+    void* args[] = {&table_arg, &count_arg, &n_vec_arg, &tiles_per_seg, &mode};
     dev->launches_since_wait = true;
     HIP_TRY(dev, hipModuleLaunchKernel(kernel->fn_batched, static_cast<unsigned int>(tiles_per_seg * n_sets), 1, 1,
                                        static_cast<unsigned int>(t.block_threads), 1, 1, 0, dev->stream, args, nullptr));

@@ -134,13 +134,13 @@ struct Planned {
     size_t table_offset = 0;      // in u64 entries
     size_t map_offset = 0;        // ragged: start of the block map, in u64 entries
     size_t blocks = 0;            // ragged: workgroups
-    custos_hip_kernel* kern = nullptr;  // kernels: the variant that suits the bytes the node touches
-    bool alternate = false;             // kernels: walks its tiles against the previous such node
+    custos_hip_kernel* kern = nullptr;  // kernels: the kernel of the (first) member
+    ResolvedShape shape;                // kernels: vectors per thread and cache policy that suit the bytes the
+                                        // node touches; whether it walks its tiles against the previous such node
 };
 
-unsigned long long tiles_of(const custos_hip_kernel* k, const RecNode& n) {
-    const Tuning& t = k->spec.tuning;
-    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+unsigned long long tiles_of(const custos_hip_kernel* k, const RecNode& n, int unroll) {
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(k->spec.tuning.block_threads) * unroll;
     return std::max(1ull, (n.n_vec + tile_vecs - 1) / tile_vecs);
 }
 
@@ -203,7 +203,7 @@ std::vector<Planned> group_level(const custos_hip_device* dev, const std::vector
         // own stays a launch of its own
         Planned merged;
         for (size_t i : g.second) {
-            if (tiles_of(nodes[i].k, nodes[i]) > kRaggedMaxTiles) {
+            if (tiles_of(nodes[i].k, nodes[i], 2) > kRaggedMaxTiles) {
                 out.emplace_back();
                 out.back().members.push_back(i);
             } else {
@@ -251,13 +251,13 @@ void append_tables(const std::vector<RecNode>& nodes, Planned* p, std::vector<ui
     if (!p->ragged) return;
     p->map_offset = host_table->size();
     for (size_t seg = 0; seg < p->members.size(); seg++) {
-        const unsigned long long tiles = tiles_of(p->kern, nodes[p->members[seg]]);
+        const unsigned long long tiles = tiles_of(p->kern, nodes[p->members[seg]], p->shape.unroll);
         for (unsigned long long t = 0; t < tiles; t++) host_table->push_back(static_cast<uint64_t>(seg) << 32 | t);
     }
     p->blocks = host_table->size() - p->map_offset;
 }
 
-// Plans one level: merging, the kernel variant of every kernel node, the tables of the merged
+// Plans one level: merging, the launch shape of every kernel node, the tables of the merged
 // launches (appended to `host_table`); then the level's traffic joins `history`.
 std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNode>& nodes,
                                 const std::vector<size_t>& of_level, RecentTraffic* history,
@@ -280,9 +280,8 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
                 keep_loads = hot_operands(*history, member_accesses, hint);
                 dev->kept_loads += keep_loads != 0;
             }
-            custos_hip_kernel* v = kernel_variant(dev, first.k, footprint, &p.alternate, hint, keep_loads);
-            const bool usable = p.members.size() == 1 || (p.ragged ? v->fn_ragged != nullptr : v->fn_batched != nullptr);
-            p.kern = usable ? v : first.k;
+            p.kern = first.k;
+            p.shape = resolve_shape(dev, first.k, footprint, hint, keep_loads);
         }
         if (p.members.size() > 1) append_tables(nodes, &p, host_table);
     }
@@ -296,7 +295,7 @@ std::vector<unsigned char> value(const void* p, size_t n) {
 }
 
 // A planned node in launchable form: function, launch shape, argument values.  `rev` is the
-// direction argument of a generated kernel; `table` the device address of the graph's tables.
+// direction bit of a generated kernel's mode word; `table` the device address of the graph's tables.
 int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, const Planned& p, uint64_t table,
                    unsigned long long rev, LoweredNode* out) {
     const RecNode& first = nodes[p.members[0]];
@@ -330,7 +329,7 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
             ln.args.push_back(value(&a1, 8));
             ln.args.push_back(value(&a2, 8));
             ln.func = reinterpret_cast<void*>(p.kern->fn);
-            ln.grid = dim3(launch_grid(dev, p.kern, first.n, first.n_vec));
+            ln.grid = dim3(launch_grid(dev, p.kern, first.n, first.n_vec, p.shape.unroll));
         } else if (p.ragged) {
             if (p.blocks > (1ull << 31) - 1)
                 return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
@@ -340,7 +339,7 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
             ln.func = reinterpret_cast<void*>(p.kern->fn_ragged);
             ln.grid = dim3(static_cast<unsigned int>(p.blocks));
         } else {
-            const unsigned long long tiles_per_seg = tiles_of(p.kern, first);
+            const unsigned long long tiles_per_seg = tiles_of(p.kern, first, p.shape.unroll);
             const unsigned long long blocks = tiles_per_seg * p.members.size();
             if (blocks > (1ull << 31) - 1)
                 return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a batched launch would need more than 2^31 workgroups");
@@ -355,8 +354,9 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
         // (a merged launch reads them from its table rows instead)
         const ConstPlan& consts = first.k->spec.consts;
         if (consts.n_params > 0 && p.members.size() == 1) ln.args.push_back(consts.bytes);
-        ln.args.push_back(value(&rev, 8));
-        if (p.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
+        const unsigned long long mode = launch_mode(p.shape.unroll, p.shape.nontemporal, rev != 0);
+        ln.args.push_back(value(&mode, 8));
+        if (p.shape.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
     }
     *out = std::move(ln);
     return CUSTOS_HIP_OK;
@@ -625,7 +625,7 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     for (size_t level = 0; level < plan.size(); level++) {
         for (const Planned& p : plan[level]) {
             // a node that alternates runs against the direction of the one before it
-            const unsigned long long rev = p.alternate ? (parity ^= 1) : 0;
+            const unsigned long long rev = p.shape.alternate ? (parity ^= 1) : 0;
             LoweredNode ln;
             int32_t rc = lower_node(dev, nodes, p, reinterpret_cast<uint64_t>(g->table), rev, &ln);
             if (rc != CUSTOS_HIP_OK) return rc;

@@ -214,12 +214,11 @@ static custos_hip_kernel* handle_for_values(custos_hip_kernel* owner, std::uniqu
 // code (the compiler folds them: a fused chain that sits at the edge of being ALU-bound
 // runs 4 % faster than with the values in registers).  When the same expression arrives
 // with other values, the form that takes them as launch parameters is compiled once, and
-// every further set of values is a handle on that code (`prefer_shared`: go there at once,
-// for the launch-shape variants of such a handle).  custos_hip_set_literal_policy pins
+// every further set of values is a handle on that code.  custos_hip_set_literal_policy pins
 // either behaviour.
 static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
                             const char* const* markers, int32_t n_markers, const Tuning& tuning,
-                            bool prefer_shared, custos_hip_kernel** out) {
+                            custos_hip_kernel** out) {
     std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
     // (specs without their text: it is generated only for what is compiled)
     int32_t rc = spec_from_c(dev, kind, dtype, src, markers, n_markers, tuning, /*literals_in_code=*/true, &k->spec, false);
@@ -237,7 +236,7 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
             custos_hip_kernel* owner = find_code(dev, shared->spec);
             uint32_t& value_sets = dev->value_sets_seen[shared->spec.hash];
             const bool first_values = value_sets++ == 0;
-            if (owner || dev->literal_policy == CUSTOS_HIP_LITERALS_AS_PARAMETERS || prefer_shared || !first_values)
+            if (owner || dev->literal_policy == CUSTOS_HIP_LITERALS_AS_PARAMETERS || !first_values)
                 k = std::move(shared);
             if (owner) {
                 dev->hits++;
@@ -271,39 +270,25 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
     custos_hip_kernel*& slot = dtype == DType::U32 ? dev->identity_u32 : dev->identity_u8;
     if (!slot) {
         const char* markers[] = {"x"};
-        int32_t rc = compile_expr(dev, CUSTOS_HIP_KIND_APPLY, static_cast<int32_t>(dtype), "x", markers, 1, dev->tuning, false, &slot);
+        int32_t rc = compile_expr(dev, CUSTOS_HIP_KIND_APPLY, static_cast<int32_t>(dtype), "x", markers, 1, dev->tuning, &slot);
         if (rc != CUSTOS_HIP_OK) return rc;
     }
     *out = slot;
     return CUSTOS_HIP_OK;
 }
 
-custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
-                                  bool* alternate, CacheHint hint, int keep_loads) {
+ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
+                            CacheHint hint, int keep_loads) {
     const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;
-    LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint);
+    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint);
+    ResolvedShape r;
     const int direction = dev->tuning.direction;
-    *alternate = direction == 2 || (direction == 0 && shape.alternate);
-    if (k->spec.kind == Kind::Source || (!k->spec.auto_unroll && !k->spec.auto_nt)) return k;
-    Tuning t = k->spec.tuning;
-    if (k->spec.auto_unroll) t.unroll = shape.unroll;
-    if (k->spec.auto_nt) t.nontemporal = shape.nontemporal | ((shape.nontemporal & 1) ? (keep_loads & 15) << 2 : 0);
-    if (t.unroll == k->spec.tuning.unroll && t.nontemporal == k->spec.tuning.nontemporal) return k;
-    const int key = t.unroll * 64 + t.nontemporal;
-    for (const auto& v : k->variants)
-        if (v.first == key) return v.second ? v.second : k;
-    std::vector<const char*> m;
-    for (const std::string& s : k->markers) m.push_back(s.c_str());
-    const std::string keep = dev->last_error;
-    custos_hip_kernel* made = nullptr;
-    if (compile_expr(dev, static_cast<int32_t>(k->spec.kind), static_cast<int32_t>(k->spec.dtype), k->expr_src.c_str(),
-                     m.data(), static_cast<int32_t>(m.size()), t, /*prefer_shared=*/k->spec.consts.n_params > 0, &made) !=
-        CUSTOS_HIP_OK) {
-        made = nullptr;  // the first kernel serves this size too
-        dev->last_error = keep;
-    }
-    k->variants.push_back({key, made});
-    return made ? made : k;
+    r.alternate = direction == 2 || (direction == 0 && shape.alternate);
+    r.unroll = k->spec.auto_unroll ? shape.unroll : k->spec.tuning.unroll;
+    r.nontemporal = dev->tuning.nontemporal >= 0
+                        ? dev->tuning.nontemporal & 3
+                        : shape.nontemporal | ((shape.nontemporal & 1) ? (keep_loads & 15) << 2 : 0);
+    return r;
 }
 
 }  // namespace custos_hip
@@ -335,7 +320,7 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
         }
     }
     custos_hip_kernel* k = nullptr;
-    int32_t rc = compile_expr(dev, kind, dtype, src, markers, n_markers, dev->tuning, false, &k);
+    int32_t rc = compile_expr(dev, kind, dtype, src, markers, n_markers, dev->tuning, &k);
     if (rc != CUSTOS_HIP_OK) return rc;
     *kernel = k;
     dev->by_text.emplace(std::move(text_key), k);
@@ -389,11 +374,8 @@ int32_t custos_hip_kernel_launched_as(custos_hip_device* dev, custos_hip_kernel*
                                       custos_hip_kernel** variant) {
     REQUIRE_DEV(dev);
     if (!kernel || !variant) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
-    const unsigned long long operands = kernel->spec.kind == Kind::UnaryGrad ? 3 : kernel->spec.expr.n_vars + 1;
-    bool alternate = false;
-    *variant = kernel->spec.kind == Kind::Source
-                   ? kernel
-                   : kernel_variant(dev, kernel, operands * n * dtype_size(kernel->spec.dtype), &alternate);
+    (void)n;
+    *variant = kernel;  // one kernel per expression: the launch shape is an argument of the launch
     return CUSTOS_HIP_OK;
 }
 

@@ -71,16 +71,15 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // 6607 / 6501 for the best uniform shape.
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint) {
     constexpr unsigned long long MiB = 1ull << 20;
+    constexpr int kLoads = 1, kBoth = 3;  // non-temporal loads only / loads and stores
     if (footprint_bytes < 64 * MiB) return {2, 0, false};
     if (hint == CacheHint::Resident) return {2, 0, false};
-    if (hint == CacheHint::Streams) return {1, 3, footprint_bytes > 256 * MiB};
-    if (footprint_bytes < 128 * MiB) return {2, 3, false};
-    // (a launch that would fit the cache by itself gains nothing from temporal accesses
-    // when the launches around it push its data out: tanh forward + backward over 128 MiB
-    // arrays 6.44 -> 6.6 TB/s)
-    if (footprint_bytes <= 256 * MiB) return {2, hint == CacheHint::Crowded ? 3 : 0, false};
+    if (hint == CacheHint::Streams) return {2, kLoads, footprint_bytes > 256 * MiB};
+    if (footprint_bytes < 128 * MiB) return {2, kBoth, false};
+    if (footprint_bytes <= 256 * MiB) return {2, hint == CacheHint::Crowded ? kBoth : 0, false};
     const bool one_vector = footprint_bytes >= 768 * MiB || (n_operands >= 3 && footprint_bytes >= 512 * MiB);
-    return {one_vector ? 1 : 2, 3, true};
+    if (one_vector) return {n_operands < 3 ? 2 : 1, kLoads, true};
+    return {2, kBoth, true};
 }
 
 std::vector<std::string> hiprtc_options(const std::string& arch) {
@@ -276,57 +275,102 @@ struct KernelText {
         return s;
     }
 
-    // One tile: every lane loads all its vectors, then computes and stores.  `base` is the
-    // lane's first vector; a partial last tile takes the masked path.  Pointers that are read
-    // and written (`out`, `lhs_grad`) carry no __restrict__: the output may be exactly one of
-    // the inputs.
-    std::string tile_fn() const {
-        std::string tile_params;
+    // The numbers of vectors per thread this kernel has a tile function for: the caller's
+    // choice, or both shapes the library picks from per launch.
+    std::vector<int> unrolls() const {
+        if (k.auto_unroll) return {2, 1};
+        return {k.tuning.unroll};
+    }
+
+    // `custos_tile<U>(args)` for the launch's number of vectors per thread `U`.
+    std::string tile_call(const std::string& indent, const std::string& args) const {
+        const std::vector<int> us = unrolls();
+        if (us.size() == 1) return indent + "custos_tile" + std::to_string(us[0]) + "(" + args + ");\n";
+        return indent + "if (U == 2) custos_tile2(" + args + ");\n" + indent + "else custos_tile1(" + args + ");\n";
+    }
+
+    // Tiles of a range of `n_vec` vectors, as an expression over constant divisors (a division by
+    // the launch's own `U` would cost every wavefront a 64-bit division routine).
+    std::string n_tiles_expr() const {
+        auto tiles = [](int unroll) {
+            const std::string tv = "((u64)CUSTOS_BLOCK * " + std::to_string(unroll) + ")";
+            return "(n_vec + " + tv + " - 1) / " + tv;
+        };
+        const std::vector<int> us = unrolls();
+        if (us.size() == 1) return tiles(us[0]);
+        return "(U == 2 ? " + tiles(2) + " : " + tiles(1) + ")";
+    }
+
+    // `const u64 U = ...;`: vectors per thread of this launch, from the mode word
+    std::string unroll_of_mode() const {
+        if (!k.auto_unroll) return "    const u64 U = " + std::to_string(k.tuning.unroll) + ";\n";
+        return "    const u64 U = (mode >> 8) & 15;\n";
+    }
+
+    // One tile of `unroll` vectors per thread, starting at vector `first` of the operands (the
+    // same for the whole workgroup): every lane loads all its vectors, then computes and stores.
+    // The operands are addressed through buffer descriptors whose base is the tile's first
+    // vector and whose size is what is left of the vector range from there on: the hardware
+    // returns zeros for a load beyond it and drops a store, so a partial last tile runs the
+    // same instructions as a full one, and the cache policy of the launch (uniform: a scalar
+    // branch around the instruction) is an immediate operand of each load and store.  An output
+    // may be exactly one of the inputs: every lane has loaded all its vectors before its first
+    // store.
+    std::string tile_fn(int unroll) const {
+        const std::string U = std::to_string(unroll);
+        std::string ptr_params;
         for (int i = 0; i < n_ops; i++) {
             if (k.kind == Kind::UnaryGrad && i == 1) continue;
-            tile_params += "const vec_t* vin" + std::to_string(i) + ", ";
+            ptr_params += "const vec_t* vin" + std::to_string(i) + ", ";
         }
         std::string s;
-        s += "static __device__ __forceinline__ void custos_tile(" + tile_params + "vec_t* vout, const u64 base, const u64 n_vec CUSTOS_KC_PARAM) {\n";
-        if (k.kind == Kind::UnaryGrad) s += "    const vec_t* vin1 = vout;\n";
-        s += "    if (base + (u64)(CUSTOS_UNROLL - 1) * CUSTOS_BLOCK < n_vec) {\n";
-        for (int i = 0; i < n_ops; i++) s += "        vec_t a" + std::to_string(i) + "[CUSTOS_UNROLL];\n";
-        s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
+        s += "static __device__ __forceinline__ void custos_tile" + U + "(" + ptr_params +
+             "vec_t* vout, const u64 first, const u64 n_vec, const u64 mode CUSTOS_KC_PARAM) {\n";
+        s += "    const u64 left = (n_vec - first) * 16;\n";
+        s += "    const int bound = left > 0x7ffffff0ull ? 0x7ffffff0 : (int)left;\n";
         for (int i = 0; i < n_ops; i++) {
             const std::string id = std::to_string(i);
-            s += "            a" + id + "[u] = CUSTOS_LD" + id + "(vin" + id + " + base + (u64)u * CUSTOS_BLOCK);\n";
+            if (k.kind == Kind::UnaryGrad && i == 1) {
+                s += "    const custos_rsrc rs1 = custos_make_rsrc(vout + first, bound);\n";
+                s += "    const bool nt1 = (mode & 2) && !(mode & 16);\n";
+                continue;
+            }
+            s += "    const custos_rsrc rs" + id + " = custos_make_rsrc(vin" + id + " + first, bound);\n";
+            s += "    const bool nt" + id + " = (mode & 2) && !(mode & " + std::to_string(8 << i) + ");\n";
         }
-        s += "        }\n";
-        s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
-        s += "            vec_t r;\n#pragma unroll\n            for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
+        s += k.kind == Kind::UnaryGrad ? "    const custos_rsrc rso = rs1;\n" : "    const custos_rsrc rso = custos_make_rsrc(vout + first, bound);\n";
+        s += "    const bool nts = mode & 4;\n";
+        s += "    const unsigned int lane = threadIdx.x * 16u;\n";
+        for (int i = 0; i < n_ops; i++) s += "    vec_t a" + std::to_string(i) + "[" + U + "];\n";
+        s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
+        for (int i = 0; i < n_ops; i++) {
+            const std::string id = std::to_string(i);
+            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), nt" + id + ");\n";
+        }
+        s += "    }\n";
+        s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
+        s += "        vec_t r;\n#pragma unroll\n        for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
              list("a", "[u][k]") + " CUSTOS_KC_ARG);\n";
-        s += "            CUSTOS_ST(vout + base + (u64)u * CUSTOS_BLOCK, r);\n        }\n";
-        s += "    } else {\n";
-        s += "#pragma unroll\n        for (int u = 0; u < CUSTOS_UNROLL; u++) {\n";
-        s += "            const u64 idx = base + (u64)u * CUSTOS_BLOCK;\n";
-        s += "            if (idx < n_vec) {\n";
-        for (int i = 0; i < n_ops; i++) {
-            const std::string id = std::to_string(i);
-            s += "                const vec_t b" + id + " = CUSTOS_LD" + id + "(vin" + id + " + idx);\n";
-        }
-        s += "                vec_t r;\n#pragma unroll\n                for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
-             list("b", "[k]") + " CUSTOS_KC_ARG);\n";
-        s += "                CUSTOS_ST(vout + idx, r);\n            }\n        }\n";
-        s += "    }\n}\n";
+        s += "        custos_st(rso, lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), r, nts);\n    }\n";
+        s += "}\n";
         return s;
     }
 
-    // Entry point for one launch over one set of operands.  `rev` != 0 walks the tiles from
-    // the last to the first (see Tuning::direction).
+    // Entry point for one launch over one set of operands.  `mode`: bit 0 walks the tiles from
+    // the last to the first (see Tuning::direction), bits 1..6 the cache policy, bits 8..11 the
+    // vectors per thread (kernel_gen.hpp, launch_mode).
     std::string single_entry() const {
         std::string s;
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-        s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec, CUSTOS_KC_ENTRY const u64 rev) {\n";
+        s += k.name + "(" + params + ", const u64 n, const u64 head, const u64 n_vec, CUSTOS_KC_ENTRY const u64 mode) {\n";
         s += vec_ptrs;
-        s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
-        s += "    const u64 n_tiles = (n_vec + tile_vecs - 1) / tile_vecs;\n";
-        s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x)\n";
-        s += "        custos_tile(" + tile_args + "vout, (rev ? n_tiles - 1 - tile : tile) * tile_vecs + threadIdx.x, n_vec CUSTOS_KC_ARG);\n";
+        s += "    const u64 rev = mode & 1;\n";
+        s += unroll_of_mode();
+        s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * U;\n";
+        s += "    const u64 n_tiles = " + n_tiles_expr() + ";\n";
+        s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {\n";
+        s += tile_call("        ", tile_args + "vout, (rev ? n_tiles - 1 - tile : tile) * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
+        s += "    }\n";
         // Elements outside the 16-byte aligned body: `head` leading ones and the
         // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
         s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
@@ -367,8 +411,9 @@ struct KernelText {
     std::string batched_entry() const {
         std::string s;
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-        s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, const u64 rev) {\n";
-        s += "    const u64 blk = rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
+        s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, const u64 mode) {\n";
+        s += unroll_of_mode();
+        s += "    const u64 blk = (mode & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
         s += "    const u64 seg = blk / tiles_per_seg;\n";
         s += "    const u64 tile = blk - seg * tiles_per_seg;\n";
         s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + const_words) + ";\n";
@@ -376,7 +421,7 @@ struct KernelText {
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
-        s += "    custos_tile(" + tile_args + "vout, tile * (u64)CUSTOS_BLOCK * CUSTOS_UNROLL + threadIdx.x, n_vec CUSTOS_KC_ARG);\n";
+        s += tile_call("    ", tile_args + "vout, tile * (u64)CUSTOS_BLOCK * U, n_vec, mode CUSTOS_KC_ARG");
         s += "    if (tile == tiles_per_seg - 1)\n";
         s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
              list("in", "[i]") + " CUSTOS_KC_ARG);\n";
@@ -390,20 +435,21 @@ struct KernelText {
     std::string ragged_entry() const {
         std::string s;
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
-        s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, const u64 rev) {\n";
-        s += "    const u64 where = block_map[rev ? gridDim.x - 1 - blockIdx.x : blockIdx.x];\n";
+        s += k.name + "_ragged(const u64* __restrict__ table, const u64* __restrict__ block_map, const u64 mode) {\n";
+        s += unroll_of_mode();
+        s += "    const u64 where = block_map[(mode & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x];\n";
         s += "    const u64 seg = where >> 32;\n";
         s += "    const u64 tile = where & 0xffffffffull;\n";
         s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + 1 + const_words) + ";\n";
         s += "    const u64 n = ptrs[" + std::to_string(n_ptrs) + "];\n";
         s += row_consts(n_ptrs + 1);
         s += "    const u64 n_vec = n / CUSTOS_VEC;\n";
-        s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * CUSTOS_UNROLL;\n";
-        s += "    const u64 n_tiles = n_vec == 0 ? 1 : (n_vec + tile_vecs - 1) / tile_vecs;\n";
+        s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * U;\n";
+        s += "    const u64 n_tiles = n_vec == 0 ? 1 : " + n_tiles_expr() + ";\n";
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
-        s += "    custos_tile(" + tile_args + "vout, tile * tile_vecs + threadIdx.x, n_vec CUSTOS_KC_ARG);\n";
+        s += tile_call("    ", tile_args + "vout, tile * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
         s += "    if (tile == n_tiles - 1)\n";
         s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
              list("in", "[i]") + " CUSTOS_KC_ARG);\n";
@@ -427,21 +473,21 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
         err->message = "a unary gradient expression takes exactly one marker";
         return false;
     }
-    // Open knobs: the kernel is first compiled for small launches; another size compiles
-    // its variant when it first occurs.
-    const LaunchShape small = preferred_shape(0, kind == Kind::UnaryGrad ? 3 : k.expr.n_vars + 1);
+    // Vectors per thread left open: the kernel holds a tile function for two and for one, and
+    // every launch names the one it takes.  The cache policy is never part of the code: it is a
+    // field of the mode word of every launch.
     k.auto_unroll = tuning.unroll <= 0;
-    if (k.auto_unroll) k.tuning.unroll = small.unroll;
-    k.auto_nt = tuning.nontemporal < 0;
-    if (k.auto_nt) k.tuning.nontemporal = small.nontemporal;
+    if (k.auto_unroll) k.tuning.unroll = 2;
+    k.tuning.nontemporal = -1;
+    k.tuning.direction = 0;
     if (!plan_constants(k.expr, dtype, literals_in_code, &k.consts, err)) return false;
     for (const Node& n : k.expr.nodes) k.n_literals += n.op == Op::Const;
     uint64_t h;
     if (!hash_expr(k.expr, dtype, k.consts, &h, err, &k.code_literals)) return false;
     k.markers = markers;
-    // (the key holds unroll factor and cache policy as requested: 0 / -1 = chosen per launch)
-    int32_t tail[6] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, k.auto_nt ? -1 : k.tuning.nontemporal, 12 /* template version */};
+    // (the key holds the vectors per thread as requested: 0 = chosen per launch)
+    int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
+                       k.tuning.blocks_per_cu, 13 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -464,28 +510,35 @@ bool emit_kernel_source(KernelSpec* spec, ParseError* err) {
     std::string body;
     if (!emit_expr_body(k.expr, k.dtype, k.consts, &body, err)) return false;
 
-    const bool nt_load = k.tuning.nontemporal & 1, nt_store = k.tuning.nontemporal & 2;
-
     std::string s;
     s += "// generated by custos-hip: " + to_cl_source(k.expr, k.markers, &k.consts) + "\n";
     s += "#define CUSTOS_BLOCK " + std::to_string(k.tuning.block_threads) + "\n";
-    s += "#define CUSTOS_UNROLL " + std::to_string(k.tuning.unroll) + "\n";
     s += "#define CUSTOS_VEC " + std::to_string(k.vec_elems) + "\n";
-    // one load macro per operand: with non-temporal loads, the operands named in bits 2.. of
-    // the policy are still loaded temporally (an operand that the launches around this one
-    // read again and again stays cached while the rest streams)
-    for (int i = 0; i < 4; i++) {
-        const bool nt = nt_load && !((k.tuning.nontemporal >> (2 + i)) & 1);
-        s += "#define CUSTOS_LD" + std::to_string(i) + (nt ? "(p) __builtin_nontemporal_load(p)\n" : "(p) (*(p))\n");
-    }
-    s += nt_store ? "#define CUSTOS_ST(p, v) __builtin_nontemporal_store(v, p)\n"
-                  : "#define CUSTOS_ST(p, v) (*(p) = (v))\n";
     s += prelude(k.dtype, k.vec_elems, k.consts.n_params);
+    // Loads and stores of one 16-byte vector through a buffer descriptor, with the cache policy
+    // of the launch as the instruction's immediate operand: temporal, or non-temporal (2) for
+    // what streams past the caches.
+    s += R"(typedef unsigned int custos_u4 __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t custos_rsrc;
+static __device__ __forceinline__ custos_rsrc custos_make_rsrc(const vec_t* p, const int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, bytes, 0x00020000);
+}
+static __device__ __forceinline__ vec_t custos_ld(const custos_rsrc rs, const unsigned int offset, const bool nt) {
+    custos_u4 v;
+    if (nt) v = __builtin_amdgcn_raw_buffer_load_b128(rs, offset, 0, 2);
+    else v = __builtin_amdgcn_raw_buffer_load_b128(rs, offset, 0, 0);
+    return __builtin_bit_cast(vec_t, v);
+}
+static __device__ __forceinline__ void custos_st(const custos_rsrc rs, const unsigned int offset, const vec_t v, const bool nt) {
+    if (nt) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(custos_u4, v), rs, offset, 0, 2);
+    else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(custos_u4, v), rs, offset, 0, 0);
+}
+)";
     s += expr_fn(k, body);
 
     const KernelText text(k);
     s += text.elem_fn();
-    s += text.tile_fn();
+    for (int unroll : text.unrolls()) s += text.tile_fn(unroll);
     s += text.single_entry();
     s += text.batched_entry();
     s += text.ragged_entry();
@@ -497,8 +550,7 @@ bool emit_kernel_source(KernelSpec* spec, ParseError* err) {
 bool same_code(const KernelSpec& a, const KernelSpec& b) {
     if (a.kind != b.kind || a.dtype != b.dtype || a.hash != b.hash) return false;
     if (a.tuning.block_threads != b.tuning.block_threads || a.tuning.unroll != b.tuning.unroll ||
-        a.tuning.blocks_per_cu != b.tuning.blocks_per_cu || a.tuning.nontemporal != b.tuning.nontemporal ||
-        a.auto_unroll != b.auto_unroll || a.auto_nt != b.auto_nt)
+        a.tuning.blocks_per_cu != b.tuning.blocks_per_cu || a.auto_unroll != b.auto_unroll)
         return false;
     if (a.expr.n_vars != b.expr.n_vars || a.expr.root != b.expr.root || a.expr.nodes.size() != b.expr.nodes.size()) return false;
     for (size_t i = 0; i < a.expr.nodes.size(); i++) {

@@ -25,10 +25,11 @@ struct Tuning {
     // knobs are chosen per launch from the bytes it touches (preferred_shape)
     // unless the caller fixes them.
     int block_threads = 128;
-    int unroll = 0;         // 16-byte vectors per thread and tile; 0: chosen per launch
+    int unroll = 0;         // 16-byte vectors per thread and tile; 0: chosen per launch (2 or 1)
     int blocks_per_cu = 0;  // <= 0: one tile per workgroup
     int nontemporal = -1;   // bit 0 loads, bit 1 stores; -1: chosen per launch.  Bits 2..5 (set by the
-                            // library only): operand 0..3 is loaded temporally although bit 0 is set
+                            // library only): operand 0..3 is loaded temporally although bit 0 is set.
+                            // Read from the device's tuning when a launch is issued or a graph built.
     int direction = 0;      // 1: tiles first to last; 2: every launch the other way round; 0: chosen per launch
 };
 
@@ -52,6 +53,17 @@ enum class CacheHint {
 constexpr unsigned long long kCacheWorkingSet = 256ull << 20;
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint = CacheHint::Unknown);
 
+// The last argument of every generated entry point: how this launch runs the kernel.  Nothing
+// of it is compiled in, so one kernel per expression serves every launch size.
+//   bit 0      the tiles are walked from the last to the first
+//   bit 1, 2   non-temporal loads, non-temporal stores
+//   bits 3..6  operand 0..3 is loaded temporally although bit 1 is set
+//   bits 8..11 vectors per thread (only read by kernels whose unroll factor was left open)
+inline uint64_t launch_mode(int unroll, int nontemporal, bool rev) {
+    return (rev ? 1u : 0u) | static_cast<uint64_t>(nontemporal & 3) << 1 | static_cast<uint64_t>((nontemporal >> 2) & 15) << 3 |
+           static_cast<uint64_t>(unroll & 15) << 8;
+}
+
 // Fills unset (zero) fields with the defaults and clamps to legal values
 // (`nontemporal` and `direction` as in custos_hip_tuning).
 Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int nontemporal, int direction);
@@ -60,9 +72,9 @@ struct KernelSpec {
     Kind kind = Kind::Apply;
     DType dtype = DType::F32;
     Expr expr;
-    Tuning tuning;             // as compiled (unroll resolved)
-    bool auto_unroll = false;  // the caller left the unroll factor / the cache policy open:
-    bool auto_nt = false;      // launches may use a variant compiled with another choice
+    Tuning tuning;             // as compiled: workgroup size, grid kind, most vectors per thread
+    bool auto_unroll = false;  // the caller left the vectors per thread open: the kernel holds the
+                               // tile functions for 2 and for 1, and every launch picks one
     ConstPlan consts;          // literals that are launch parameters, and this text's values for them
     int n_literals = 0;        // literals in the expression, parameters or not
     std::vector<uint64_t> code_literals;  // values of the literals that stay in the code, in node order

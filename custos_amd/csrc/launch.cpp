@@ -123,9 +123,9 @@ int32_t plan_launch(custos_hip_device* dev, const custos_hip_kernel* k, const st
 }  // namespace
 
 unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
-                         unsigned long long n_vec) {
+                         unsigned long long n_vec, int unroll) {
     const Tuning& t = k->spec.tuning;
-    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * t.unroll;
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * unroll;
     unsigned long long tiles = (n_vec + tile_vecs - 1) / tile_vecs;
     const unsigned long long scalar = n - n_vec * k->spec.vec_elems;
     const unsigned long long cus = static_cast<unsigned long long>(dev->props.multiProcessorCount);
@@ -206,10 +206,9 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
         }
         dev->recent.record(all);
     }
-    bool alternate = false;
-    k = kernel_variant(dev, k, footprint, &alternate, hint, keep_loads);
-    const unsigned int grid = launch_grid(dev, k, n, n_vec);
-    unsigned long long rev = alternate ? (dev->launch_parity ^= 1) : 0;
+    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, keep_loads);
+    const unsigned int grid = launch_grid(dev, k, n, n_vec, shape.unroll);
+    unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, shape.alternate && (dev->launch_parity ^= 1));
     uint64_t ptrs[8];
     std::vector<void*> args;
     for (size_t i = 0; i < ops.size(); i++) {
@@ -221,7 +220,7 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     args.push_back(&n_vec);
     // the expression's literals that are launch parameters: one block by value
     if (k->spec.consts.n_params > 0) args.push_back(k->spec.consts.bytes.data());
-    args.push_back(&rev);
+    args.push_back(&mode);
     dev->launches_since_wait = true;
     HIP_TRY(dev, hipModuleLaunchKernel(k->fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
                                        1, 1, 0, dev->stream, args.data(), nullptr));

@@ -24,12 +24,8 @@ struct custos_hip_kernel {
     hipFunction_t fn = nullptr;
     hipFunction_t fn_batched = nullptr;  // equal launches in one grid
     hipFunction_t fn_ragged = nullptr;   // launches of different lengths in one grid
-    // To compile the same expression with another launch shape on demand:
-    std::string expr_src;
+    std::string expr_src;  // the expression as the caller spelt it
     std::vector<std::string> markers;
-    // same expression compiled with another (unroll, cache policy); owned by the cache.
-    // key = unroll * 8 + nontemporal; a null entry is a variant that failed to compile
-    std::vector<std::pair<int, custos_hip_kernel*>> variants;
     // Handles for the same code with other values of the literal parameters, by those
     // values: they share this kernel's module (their own `module` stays null) and differ
     // in `spec.consts.bytes`, `spec.expr` and `expr_src`.  `code` points at the kernel that
@@ -48,7 +44,7 @@ struct LoweredNode {
     dim3 grid{1, 1, 1}, block{1, 1, 1};
     unsigned int shared_mem = 0;
     std::vector<std::vector<unsigned char>> args;
-    int rev_arg = -1;  // index of the direction argument of a node that alternates, else -1
+    int rev_arg = -1;  // index of the mode word (bit 0 = direction) of a node that alternates, else -1
 };
 
 struct custos_hip_graph {
@@ -221,26 +217,29 @@ int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec, c
 int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k);
 // The kernel of the expression `x` over `dtype` elements (compiled once per device).
 int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel** out);
-// The kernel to launch for `footprint_bytes` touched: `k` itself, or a variant
-// compiled with the unroll factor and cache policy that suit the size (where the
-// caller left them open).  Never fails: without a variant it returns `k`.
-// `alternate` tells whether the launch should walk the tiles in the direction
-// opposite to the previous launch.
-// `hint`: what is known about the data the launch reads (see CacheHint).
-// `keep_loads`: bit i = operand i is read by the launches around this one again and again;
-// where the launch streams, that operand is still loaded temporally.
-custos_hip_kernel* kernel_variant(custos_hip_device* dev, custos_hip_kernel* k, unsigned long long footprint_bytes,
-                                  bool* alternate, CacheHint hint = CacheHint::Unknown, int keep_loads = 0);
+// How a launch of `k` that touches `footprint_bytes` runs: vectors per thread and cache policy
+// from the bytes touched and from what is known about the launches around it (`hint`,
+// `keep_loads`: bit i = operand i is read by those launches again and again, and is still
+// loaded temporally where the launch streams), unless the caller pinned them (the vectors per
+// thread when the kernel was compiled, cache policy and direction in the device's tuning now).
+// `alternate`: the launch walks its tiles against the direction of the previous such launch.
+struct ResolvedShape {
+    int unroll = 2;
+    int nontemporal = 0;
+    bool alternate = false;
+};
+ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
+                            CacheHint hint = CacheHint::Unknown, int keep_loads = 0);
 
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
-// The operands (bit i = i-th pointer parameter) that `kernel_variant` should keep loading
+// The operands (bit i = i-th pointer parameter) that a streaming launch should keep loading
 // temporally, given what the launches before did with them; `members`: the access lists of the
 // launches merged into this one, each in parameter order.
 int hot_operands(const RecentTraffic& recent, const std::vector<const std::vector<Access>*>& members, CacheHint hint);
-// Workgroups of a single launch of `k` over n_vec vectors and n elements.
+// Workgroups of a single launch of `k` over n_vec vectors and n elements with `unroll` vectors per thread.
 unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
-                         unsigned long long n_vec);
+                         unsigned long long n_vec, int unroll);
 
 // graph.cpp
 int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g);

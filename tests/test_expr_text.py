@@ -118,7 +118,7 @@ def test_shared_form_takes_literals_as_launch_parameters():
     assert "struct CustosConsts { C c[2]; };" in src and "const float t1 = kc.c[0];" in src
     assert "0x1p+1f" not in src
     assert src.startswith("// generated by custos-hip: ((x * c0) + c1)\n")
-    assert "CUSTOS_KC_ENTRY const u64 rev)" in src          # the block is an argument by value of every entry point
+    assert "CUSTOS_KC_ENTRY const u64 mode)" in src         # the block is an argument by value of every entry point
     consts = capi.expr_constants("f32", "((x * 2.0) + 1.0)", ["x"])
     assert consts.dtype == np.float32 and consts.tolist() == [2.0, 1.0]
     src64, _ = capi.expr_emit(capi.KIND_APPLY, "f64", "((x * 2.0) + 1.0)", ["x"], shared=True)
@@ -201,18 +201,21 @@ def test_shared_hash_ignores_literal_values_but_not_structure_or_type():
 def test_tuning_is_part_of_the_key_and_source():
     t = capi.Tuning(256, 4, 0, -1)
     src, h1 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], t)
-    assert "#define CUSTOS_BLOCK 256" in src and "#define CUSTOS_UNROLL 4" in src
-    assert "__builtin_nontemporal" not in src
-    # knobs left open: the text is the shape for small launches (temporal accesses, two vectors
-    # per thread); other sizes compile a variant when launched
+    assert "#define CUSTOS_BLOCK 256" in src and "custos_tile4(" in src and "custos_tile2(" not in src
+    # vectors per thread left open: the kernel holds the tile functions for two and for one, and
+    # every launch names the one it takes in its mode word
     src2, h2 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"])
-    assert "#define CUSTOS_BLOCK 128" in src2 and "#define CUSTOS_UNROLL 2" in src2
-    assert "__builtin_nontemporal" not in src2
+    assert "#define CUSTOS_BLOCK 128" in src2 and "custos_tile2(" in src2 and "custos_tile1(" in src2
+    assert "const u64 U = (mode >> 8) & 15;" in src2
+    # the cache policy is never compiled in: it is an operand of the launch, so one kernel per
+    # expression serves every launch size
     src4, h4 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], capi.Tuning(0, 0, 0, 3))
-    assert "__builtin_nontemporal_load" in src4 and "__builtin_nontemporal_store" in src4
+    assert src4 == src2 and h4 == h2
+    assert "__builtin_amdgcn_raw_buffer_load_b128(rs, offset, 0, 2)" in src2
     src5, h5 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], capi.Tuning(0, 2, 0, -1))
-    assert len({h1, h2, h4, h5}) == 4            # "open" and "fixed to the same value" are different keys
-    assert "const u64 rev" in src2
+    assert len({h1, h2, h5}) == 3                # "open" and "fixed to the same value" are different keys
+    assert "custos_tile1(" not in src5
+    assert "const u64 mode" in src2
 
 
 def test_integer_rejects_transcendentals_and_fractions():

@@ -308,23 +308,39 @@ def test_both_traversal_directions_and_all_shapes(hip, oracle):
 
 
 def test_launch_shape_follows_the_bytes_touched(hip):
-    """With the knobs left open, small launches run the kernel as first compiled and a large
-    launch runs a variant of the same expression; a pinned knob pins the kernel."""
+    """One kernel per expression: the launch shape (vectors per thread, cache policy, direction) is
+    an operand of every launch, so no launch of any size compiles anything after `expr_compile`
+    has returned (the reference compiles once per text too: src/devices/cuda/kernel_cache.rs:39-61)."""
     src = "((x * 3.0) - 1.0)"
     k = hip.compile(capi.KIND_APPLY, "f32", src, ("x",))
-    small = hip.kernel_name(k, 1000)
-    assert small == hip.kernel_name(k) == hip.kernel_name(k, 1 << 20)
-    assert "__builtin_nontemporal" not in hip.kernel_source(k)
-    big = hip.kernel_name(k, 1 << 28)
-    assert big != small
+    kg = hip.compile(capi.KIND_UNARY_GRAD, "f32", "(x * 2.0)", ("x",))
+    identity = hip.alloc(16)
+    hip.copy(identity, hip.alloc(16))             # the library's own copy kernel is compiled on first use
     c0, _ = hip.cache_stats()
-    assert hip.kernel_name(k, 1 << 28) == big               # compiled once
-    assert hip.cache_stats()[0] == c0
+    big = hip.alloc(1 << 29, zeroed=False)        # 2 GiB
+    xs = synth.uniform_f32(21, 1 << 12, -1, 1)
+    hip.write(big.slice(0, 1 << 12), xs)
+    for log2n in range(10, 29, 3):                # 4 KiB ... 1 GiB per operand
+        n = 1 << log2n
+        src_buf, dst_buf = big.slice(0, n), big.slice(1 << 28, (1 << 28) + n)
+        capi.check(hip.lib.custos_hip_apply_fn(hip.handle, k, src_buf.ptr, dst_buf.ptr, n), hip.handle)
+        capi.check(hip.lib.custos_hip_add_unary_grad(hip.handle, kg, src_buf.ptr, dst_buf.ptr, src_buf.ptr, n), hip.handle)
+        assert hip.kernel_name(k, n) == hip.kernel_name(k)
+        hip.capture_begin()
+        capi.check(hip.lib.custos_hip_apply_fn(hip.handle, k, src_buf.ptr, dst_buf.ptr, n), hip.handle)
+        graph = hip.capture_end()
+        graph.launch()
+        hip.sync()
+        graph.destroy()
+        assert hip.cache_stats()[0] == c0, f"a launch over 2^{log2n} elements compiled something"
+    want = xs * np.float32(3.0) - np.float32(1.0)
+    assert_bits_equal(big.slice(1 << 28, (1 << 28) + (1 << 12)).read(), want)
+    del big
     try:
         hip.set_tuning(0, 2, 0, 3, 1)
         pinned = hip.compile(capi.KIND_APPLY, "f32", src, ("x",))
-        assert hip.kernel_name(pinned, 1000) == hip.kernel_name(pinned, 1 << 28) == hip.kernel_name(pinned)
-        assert "__builtin_nontemporal_store" in hip.kernel_source(pinned)
+        assert hip.kernel_name(pinned) != hip.kernel_name(k)     # vectors per thread pinned: another kernel
+        assert "custos_tile1(" not in hip.kernel_source(pinned)
     finally:
         hip.set_tuning()
     # results do not depend on the variant: a 2^25-element launch (256 MiB touched) and its head
@@ -426,9 +442,10 @@ def test_literals_are_launch_parameters(hip, oracle):
         assert_bits_equal(lhs_grad.read(), g + y * (x * np.float32(k)), f"gradient {k}")
 
 
-def test_launch_shape_variants_of_shared_code(hip):
-    """A launch large enough for another launch shape compiles that variant once per form, not
-    once per set of literal values -- launched directly and from a recorded graph."""
+def test_launch_shapes_of_shared_code(hip):
+    """A launch large enough for another launch shape runs the same code: one compilation per form
+    (values in the code, values as parameters), not one per shape or per set of literal values --
+    launched directly and from a recorded graph."""
     n = 1 << 23                                   # 32 MiB per array: the 64 MiB launch takes non-temporal accesses
     rng = np.random.default_rng(5)
     x = rng.uniform(-8, 8, n).astype(np.float32)
@@ -451,9 +468,7 @@ def test_launch_shape_variants_of_shared_code(hip):
         assert_bits_equal(out.read(), want, f"graph {step}")
         graph.destroy()
     c1, _ = hip.cache_stats()
-    # (values in the code, shared form) x (small shape, this size's shape, and the shape that keeps
-    # loading x temporally once the launches before have read it twice) -- not one per set of values
-    assert 4 <= c1 - c0 <= 6 and len(names) == 2
+    assert c1 - c0 == 2 and len(names) == 2
 
 
 def test_error_paths(hip):
