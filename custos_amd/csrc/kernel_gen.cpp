@@ -23,52 +23,46 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // Launch shape by the bytes a launch touches, measured on MI355X (8 x 4 MiB L2,
 // 256 MiB memory-side cache, HBM3E) over buffers of random data (buffers of
 // zeros run 5-10 % faster and hide differences).  Abbreviations: vectors per
-// thread (u1 / u2), temporal or non-temporal accesses (T / N), tiles always
-// first to last or every launch the other way round (f / a).
+// thread (u1 / u2); cache policy T (all temporal), L (non-temporal loads,
+// temporal stores), S (temporal loads, non-temporal stores), N (both
+// non-temporal); tiles always first to last (f) or every launch the other way
+// round (a).  GB/s on the algorithmic bytes.
 //
-// Small launches (under 64 MiB): a chain whose working set fits the memory-side
-// cache runs 4 % faster with temporal accesses (a non-temporal store pushes what
-// the next kernel reads out to HBM): 1024 x (a*b; +c; sqrt(abs)*0.3) over 16 KiB
-// buffers replays in 23.5 us with u2 T, 24.4 with u2 N, 27.3 with u1 N.
+// What fits the memory-side cache (up to 256 MiB touched): temporal accesses,
+// two vectors per thread; a chain whose working set fits runs 4 % faster with
+// them (a non-temporal store pushes what the next kernel reads out to HBM).  The
+// exception is the range just above the L2 capacity, 64 to 128 MiB, where N is
+// ahead for a launch that does not read what a launch just before it wrote
+// (1R+1W at 64 MiB: u2N 7074, u2T 6454; 3R+1W at 64 MiB: u2N 6874, u2T 6588).
 //
-// Large launches stream from HBM; temporal accesses then cost up to 10 % (the
-// same chain over 256 MiB arrays: u2 T 5846, u2 N 6409, u1 N 7051 GB/s).  Kernels
-// that read through three or more pointers sustain most with one vector per
-// thread from about 512 MiB on, kernels with one input with two, in isolation
-// and in sequence (tanh forward 1R+1W + backward 3R+1W at 2^26 elements, GB/s on
-// 24 B/element: forward u2 / backward u1 6920, u2 / u2 6400, u1 / u2 6350,
-// u1 / u1 5860, whatever the direction).
+// What does not fit streams, and the policy that streams best is L, not N: loads
+// pass the caches by, while the stores stay in the memory-side cache, so that the
+// 256 MiB written last are still there when the next launch over the same
+// buffers starts at that end (direction a), and a consumer finds them.  The same
+// launch repeated, u2La / u1La / u2Nf / u1Nf / u2Tf:
+//   1R+1W   768 MiB 7115 / 6583 / 6580 / 6514 / 6112   1 GiB 7333 / 7045 / 6536 / 6476 / 6124
+//           2 GiB   6896 / 6737 / 6418 / 6518 / 6169
+//   2R+1W   768 MiB 6998 / 6763 / 6576 / 6708 / 5792   1 GiB 6810 / 6710 / 6521 / 6684 / 5917
+//   3R+1W (gradient kernel, in place)
+//           768 MiB 7135 / 7091 / 6257 / 6824 / 5492   1 GiB 6874 / 7086 / 6389 / 6792 / 5668
+// Launches through three or more pointers keep one vector per thread from 512 MiB
+// on (3R+1W at 1 GiB above, and in sequence: tanh forward 1R+1W over 512 MiB with
+// u2N followed by backward 3R+1W over 768 MiB with u1L sustains 6830 on 24 bytes per
+// element, more than any single shape for both: u1N 6636, u2L 5895, u2T 5712).
+// Between 256 and 768 MiB a launch through two pointers keeps N (in that very
+// sequence L for the forward kernel alone is faster, 7147 against 6451, and the
+// sequence slower, 5918 against 6742: its stores push out what the backward kernel
+// could have kept).
 //
-// Alternating the direction costs nothing in such sequences and lets a launch
-// that repeats over the same buffers (a graph replay, a consumer after its
-// producer) start on the last 256 MiB the memory-side cache still holds; with it
-// one vector per thread is best for every arity from 768 MiB on.  GB/s, same
-// kernel launched back to back, u1Na / u2Na / u2Nf / u1Nf:
-//   1R+1W   768 MiB 6861 / 6452 / 6482 / 6286    2 GiB 6759 / 6427 / 6406 / 6326
-//   2R+1W   576 MiB 6873 / 6590 / 6701 / 6908  1.5 GiB 6810 / 6555 / 6598 / 6212
-//   3R+1W     1 GiB 6986 / 6375 / 6412 / 7019    2 GiB 6646 / 6298 / 6313 / 6115
-// Up to 256 MiB a launch fits the memory-side cache and temporal accesses win
-// 3-9 % when the kernel repeats over the same buffers (1R+1W at 192 MiB: 6959
-// against 6383 GB/s) and in chains over arrays of that size; the exception is the
-// range just above the L2 capacity, 64 to 128 MiB, where non-temporal accesses
-// are ahead (3R+1W at 64 MiB: 6883 against 6343) unless the launch reads what a
-// launch just before it wrote.
-//
-// Chains (a launch reads what the launch before it wrote; 1R+1W kernels, GB/s on 8
-// bytes per element) differ from repeats of one launch: while everything the
-// chain touches fits the memory-side cache, temporal accesses win at every launch
-// size, beyond that one vector per thread with non-temporal accesses does,
-// whatever the direction.  Eager cycle over three arrays of A MiB, u2T / u1T /
-// u2N / u1N: A = 32: 6487 / 6184 / 5348 / 5936; 64: 6777 / 6843 / 5874 / 6686;
-// 100: 6159 / 5955 / 6131 / 6960; 128: 6393 / 6301 / 6219 / 7069; 256: 5957 / 6082 /
-// 6388 / 7294.  Replayed graph of five kernels over six arrays: A = 32 (192 MiB
-// in all): 5887 / 5694 / 4941 / 5363; 64 (384 MiB): 5684 / 5841 / 5607 / 6270;
-// 128: 5597 / 5856 / 6057 / 6776; 256: 5885 / 6032 / 6307 / 6956.
+// Chains (a launch reads what the launch before it wrote; 1R+1W kernels, eager
+// cycle over three arrays, by the bytes one launch touches): while everything the
+// chain touches fits the memory-side cache, temporal accesses win (64 MiB: u2T
+// 6507, u2L 6271, u2N 5802); beyond, L with two vectors per thread, whatever the
+// direction (192 MiB: u2L 6956, u2T 6229, u2N 6153; 256 MiB: 7081 / 5653 / 6340;
+// 512 MiB: 7142 / 5993 / 6467; 768 MiB: 6970 / 6075 / 6475).
 // An operand that every kernel of a streaming chain reads again (and nobody
 // writes) keeps temporal loads while the rest streams (bits 2.. of the policy,
-// launch.cpp hot_operands): five 2R+1W kernels with one shared operand over
-// arrays of 64 / 100 MiB 6626 / 6848 against 6082 / 6457 without, and against
-// 6607 / 6501 for the best uniform shape.
+// launch.cpp hot_operands).
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint) {
     constexpr unsigned long long MiB = 1ull << 20;
     constexpr int kLoads = 1, kBoth = 3;  // non-temporal loads only / loads and stores

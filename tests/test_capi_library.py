@@ -121,8 +121,8 @@ def test_product_never_imports_the_oracle():
 
 def test_launch_shape_by_bytes_touched():
     """The shape for the knobs a caller leaves open: temporal accesses for what fits the caches,
-    non-temporal streaming beyond, one vector per thread and alternating direction for the
-    large launches."""
+    non-temporal streaming beyond; the largest launches load non-temporally, store temporally and
+    alternate their direction (what they wrote last is what the next launch starts on)."""
     MiB = 1 << 20
     shape = capi.preferred_shape
     assert shape(8 * MiB, 2) == (2, 0, False)              # config 1: 2^20 f32 in, out
@@ -132,9 +132,9 @@ def test_launch_shape_by_bytes_touched():
     assert shape(128 * MiB, 2) == (2, 0, False) and shape(256 * MiB, 2) == (2, 0, False)
     assert shape(257 * MiB, 2) == (2, 3, True)
     assert shape(512 * MiB, 2) == (2, 3, True)             # config 3 forward
-    assert shape(768 * MiB, 3) == (1, 3, True)             # config 3 backward
-    assert shape(512 * MiB, 3) == (1, 3, True) and shape(511 * MiB, 3) == (2, 3, True)
-    assert shape(1024 * MiB, 2) == (1, 3, True)            # config 4
-    assert shape(2048 * MiB, 2) == (1, 3, True)            # config 2
+    assert shape(768 * MiB, 3) == (1, 1, True)             # config 3 backward
+    assert shape(512 * MiB, 3) == (1, 1, True) and shape(511 * MiB, 3) == (2, 3, True)
+    assert shape(1024 * MiB, 2) == (2, 1, True)            # config 4
+    assert shape(2048 * MiB, 2) == (2, 1, True)            # config 2
     with pytest.raises(capi.CustosHipError):
         shape(1, 0)
