@@ -1,19 +1,28 @@
 #!/usr/bin/env python3
 """Benchmark of the element-wise hot path on one MI355X.
 
-Default workload (BASELINE.json configs[1]): the fused unary chain
-y = relu(sin(x)*2.0 + 1.0) - 0.5 (five unary ops fused into one kernel) over
-f32 N = 2^28, x uniform in [-pi, pi) from seed 0.  One "step" is one launch of
-the fused kernel over the whole buffer (replayed as the one-node graph a `Lazy`
-run holds), inputs resident in HBM.
+Default workload (BASELINE.json configs[1]): y = relu(sin(x)*2.0 + 1.0) - 0.5, five unary
+operations fused into ONE kernel, over f32 N = 2^28, x uniform in [-pi, pi) from seed 0, inputs
+resident in HBM.  What is timed, and where:
 
-Prints ONE JSON line: metric/value (GB/s on the algorithmic 8 B per element),
-the roofline of the fused kernel (HIP-event timed on the compute stream) and a
-CPU baseline (the oracle's compiled loop, one thread, on a stated sample).
+  value / ms_per_step   this process, through the C ABI: one step = one replay of the one-node
+                        recording that holds the fused kernel (what a lazy run holds from its
+                        second run on); exactly --steps replays between two events on the
+                        library's compute stream, no wait between steps.  By default such a
+                        launch walks the array against the direction of the launch before it and
+                        so starts on the 256 MiB the memory-side cache still holds.
+  per_step              the same replays with an event between every two (>= 50): median and min.
+  roofline              the same kernel pinned to plain HBM streaming (every launch first tile to
+                        last, non-temporal accesses): no help from the memory-side cache.
+  module_stack          a child process started before this one touches the GPU: the C++ module
+                        stack HIP<Graph<Lazy<Base>>>, five apply_fn calls, optimize_mem_graph,
+                        unary_fusing, then run() with the reference's wait after every run.
+  cpu_baseline          the oracle's compiled loop for the same chain, one thread.
 
-The same line carries `other_configs`: the other four BASELINE configurations
-(c1 exp, c3 tanh forward+backward, c4 f16 chain, c5 graph replay), each with
-elements/s, GB/s and the CPU port timed beside it (skip with --no-others).
+`other_configs` carries the other four BASELINE configurations (c1 exp, c3 tanh forward +
+backward, c4 f16 chain, c5 graph replay), each with elements/s, GB/s and the CPU port beside it
+(skip with --no-others).  Phases other than the headline run at least 50 launches and 50 ms of
+device time whatever --steps says.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--log2n L] [--no-others]
 """
@@ -23,7 +32,10 @@ import argparse
 import ctypes as C
 import json
 import os
+import re
+import subprocess
 import sys
+import tempfile
 import time
 
 import numpy as np
@@ -33,10 +45,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the fused chain at N = 2^28 with the default launch shape, from two
-# `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE) scaled by the identity-copy kernel of
-# known size; commands and raw counter values: profiles/fused_chain_f32_n2p28_hbm_traffic.md
-MEASURED_TRAFFIC_C2_N2P28 = 2147557720
+# HBM bytes per launch of the streaming-pinned fused chain at N = 2^28, from two `rocprofv3 --pmc`
+# runs (FETCH_SIZE, then WRITE_SIZE) scaled by the identity-copy kernel of known size: the number
+# is read from the summary of those runs, which also holds the commands and the raw counters.
+TRAFFIC_PROFILE = "profiles/fused_chain_f32_n2p28_hbm_traffic.md"
+
+MIN_LAUNCHES = 50      # floor of every timed phase except the headline's --steps
+MIN_DEVICE_MS = 50.0
 
 C2_OPS = [
     lambda v: v.sin(),
@@ -58,16 +73,35 @@ def gen_chunked(fn, n, chunk=1 << 24):
     return out
 
 
-def time_steps(dev, step, steps, warmup, settle_ms=0.0):
-    """`warmup` untimed steps, then `steps` timed ones.  `settle_ms` > 0 first repeats the step
-    untimed until that much time has passed: after an idle period (host-side data generation,
-    the CPU baseline) the device needs about 30 ms of work to return to its steady clocks."""
-    if settle_ms > 0:
-        t_end = time.perf_counter() + settle_ms * 1e-3
-        while time.perf_counter() < t_end:
-            for _ in range(8):
-                step()
-            dev.sync()
+def launcher(dev, fn, *args):
+    """A step that calls one entry point of the library with fixed arguments."""
+    h = dev.handle
+
+    def step():
+        rc = fn(h, *args)
+        if rc:
+            from custos_amd import capi
+            capi.check(rc, h)
+    return step
+
+
+def settle(dev, step, settle_ms):
+    """Runs `step` untimed: once with a wait (whatever a first call costs stays outside), then
+    for `settle_ms` of back-to-back work.  After an idle period (host-side data generation, the
+    CPU baseline) the device needs some tens of milliseconds of work to return to its steady clocks."""
+    step()
+    dev.sync()
+    t_end = time.perf_counter() + settle_ms * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(8):
+            step()
+        dev.sync()
+
+
+def time_exactly(dev, step, steps, warmup, settle_ms=100.0):
+    """`warmup` untimed steps, then EXACTLY `steps` timed ones between two events on the compute
+    stream, bracketed by waits.  Returns (event ms, wall ms)."""
+    settle(dev, step, settle_ms)
     for _ in range(warmup):
         step()
     dev.sync()
@@ -77,8 +111,67 @@ def time_steps(dev, step, steps, warmup, settle_ms=0.0):
         step()
     ms_events = dev.timer_end()
     dev.sync()
-    wall_ms = (time.perf_counter() - t_wall) * 1e3
-    return ms_events, wall_ms
+    return ms_events, (time.perf_counter() - t_wall) * 1e3
+
+
+def time_floor(dev, step, launches_per_step=1, settle_ms=60.0):
+    """Mean ms per step over at least MIN_LAUNCHES launches and MIN_DEVICE_MS of device time."""
+    settle(dev, step, settle_ms)
+    dev.timer_begin()
+    for _ in range(8):
+        step()
+    guess = max(dev.timer_end() / 8, 1e-4)
+    steps = int(max(-(-MIN_LAUNCHES // launches_per_step), -(-MIN_DEVICE_MS // guess)))
+    dev.sync()
+    dev.timer_begin()
+    for _ in range(steps):
+        step()
+    return dev.timer_end() / steps, steps
+
+
+def per_step_stats(dev, step, steps):
+    """Every step's own duration: a mark on the compute stream between every two steps."""
+    steps = min(max(steps, MIN_LAUNCHES), 4000)
+    dev.sync()
+    dev.timer_mark(0)
+    for i in range(steps):
+        step()
+        dev.timer_mark(i + 1)
+    ms = np.array([dev.timer_between(i, i + 1) for i in range(steps)])
+    return {"steps": steps, "mean_ms": round(float(ms.mean()), 5), "median_ms": round(float(np.median(ms)), 5),
+            "min_ms": round(float(ms.min()), 5), "max_ms": round(float(ms.max()), 5)}
+
+
+def module_stack(config, steps, warmup, log2n=None, fuse=False, dump=None):
+    """Runs examples/bench_module_stack as a child process and returns its JSON line."""
+    exe = os.path.join(ROOT, "examples", "bench_module_stack")
+    if not os.path.exists(exe):
+        return {"error": f"{exe} is not built (make -C examples)"}
+    cmd = [exe, "--config", config, "--steps", str(max(steps, MIN_LAUNCHES)), "--warmup", str(warmup)]
+    if log2n is not None:
+        cmd += ["--log2n", str(log2n)]
+    if fuse:
+        cmd += ["--fuse"]
+    if dump:
+        cmd += ["--dump", str(dump[0]), dump[1]]
+    try:
+        proc = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
+    except subprocess.TimeoutExpired:
+        return {"error": "timed out"}
+    if proc.returncode != 0:
+        return {"error": (proc.stderr or proc.stdout)[-400:]}
+    return json.loads(proc.stdout.strip().splitlines()[-1])
+
+
+def measured_traffic(kernel_label):
+    """(bytes per launch, source) for the kernel the roofline is quoted on, from the committed
+    summary of the rocprofv3 counter runs; (None, None) when the summary does not hold it."""
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+    except OSError:
+        return None, None
+    m = re.search(rf"^traffic_bytes_per_launch\[{re.escape(kernel_label)}\]\s*=\s*(\d+)", text, flags=re.M)
+    return (int(m.group(1)), TRAFFIC_PROFILE) if m else (None, None)
 
 
 def cpu_baseline_c2(x, sample_elems):
@@ -102,7 +195,16 @@ def cpu_baseline_c2(x, sample_elems):
     }, out
 
 
-def bench_c2(dev, args):
+def check_chain(got, want, what):
+    m = min(got.size, want.size)
+    diff = float(np.max(np.abs(got[:m] - want[:m])))
+    tol = 8 * float(np.spacing(np.float32(1.0)))
+    if not diff <= tol:
+        raise SystemExit(f"bench: {what} differs from the CPU oracle: max abs diff {diff} > {tol}")
+    return diff
+
+
+def bench_c2(dev, args, stack):
     import custos_amd
     from custos_amd import capi, synth
     from custos_amd.expr import fused_source
@@ -115,123 +217,135 @@ def bench_c2(dev, args):
 
     src = fused_source(C2_OPS, "f32")
     kernel = dev.compile(capi.KIND_APPLY, "f32", src, ("x",))
-    lib, h = dev.lib, dev.handle
-
-    def fused_step():
-        capi.check(lib.custos_hip_apply_fn(h, kernel, xb.ptr, out.ptr, n), h)
-
+    lib = dev.lib
+    fused_step = launcher(dev, lib.custos_hip_apply_fn, kernel, xb.ptr, out.ptr, n)
     algo_bytes = 8.0 * n
+    gbs_of = lambda ms: algo_bytes / (ms * 1e-3) / 1e9
 
-    # The comparisons run first (they also bring the device to its steady clocks: the first
-    # ~30 ms of back-to-back launches after start-up run up to 15 % slower), the headline last.
+    # The comparisons run first, the headline last.
 
     # unfused comparison: five apply_fn launches through intermediates (40 B/elt moved)
     kernels = [dev.compile(capi.KIND_APPLY, "f32", custos_amd.expr._wrap(op(custos_amd.Resolve("x"))).to_cl_source("f32"), ("x",))
                for op in C2_OPS]
     tmp_a, tmp_b = dev.alloc(n, "f32"), dev.alloc(n, "f32")
     chain = [(xb, tmp_a), (tmp_a, tmp_b), (tmp_b, tmp_a), (tmp_a, tmp_b), (tmp_b, out)]
+    unfused_steps = [launcher(dev, lib.custos_hip_apply_fn, k, s.ptr, d.ptr, n) for k, (s, d) in zip(kernels, chain)]
 
     def unfused_step():
-        for k, (src_b, dst_b) in zip(kernels, chain):
-            capi.check(lib.custos_hip_apply_fn(h, k, src_b.ptr, dst_b.ptr, n), h)
+        for one in unfused_steps:
+            one()
 
-    ums, _ = time_steps(dev, unfused_step, max(1, args.steps // 4), max(1, args.warmup // 2), settle_ms=50)
-    unfused_ms = ums / max(1, args.steps // 4)
+    unfused_ms, unfused_n = time_floor(dev, unfused_step, launches_per_step=5)
 
     # plain copy (identity expression) over the same buffers: the achievable 1R+1W rate on
     # this box, and the known-size dispatch the profiler counters are scaled by
     copy_kernel = dev.compile(capi.KIND_APPLY, "f32", "x", ("x",))
+    copy_ms, copy_n = time_floor(dev, launcher(dev, lib.custos_hip_apply_fn, copy_kernel, xb.ptr, tmp_a.ptr, n))
 
-    def copy_step():
-        capi.check(lib.custos_hip_apply_fn(h, copy_kernel, xb.ptr, tmp_a.ptr, n), h)
-
-    cms, _ = time_steps(dev, copy_step, max(1, args.steps // 2), max(1, args.warmup // 2))
-    copy_ms = cms / max(1, args.steps // 2)
-
-    # The fused step with the launch shape pinned to plain HBM streaming: every launch walks the
-    # array from the first tile to the last, non-temporal accesses, two vectors per thread.  (By
-    # default every launch of this size walks the array against the direction of the launch
-    # before it and so starts on the last 256 MiB the memory-side cache still holds.)
+    # The fused step pinned to plain HBM streaming: every launch walks the array from the first tile
+    # to the last, non-temporal loads and stores, so nothing of the previous launch is found in the
+    # memory-side cache.  This is the figure the roofline fraction is quoted on.
     streaming = None
     if not tuned:
         dev.set_tuning(0, 2, 0, 3, 1)
         skernel = dev.compile(capi.KIND_APPLY, "f32", src, ("x",))
         dev.capture_begin()
-        capi.check(lib.custos_hip_apply_fn(h, skernel, xb.ptr, out.ptr, n), h)
+        capi.check(lib.custos_hip_apply_fn(dev.handle, skernel, xb.ptr, out.ptr, n), dev.handle)
         sgraph = dev.capture_end()
-        sms, _ = time_steps(dev, sgraph.launch, args.steps, args.warmup, settle_ms=100)
-        sgraph.destroy()
         dev.set_tuning(0, 0, 0, 0, 0)
-        streaming = {"ms_per_step": round(sms / args.steps, 5),
-                     "GBps": round(algo_bytes / (sms / args.steps * 1e-3) / 1e9, 2),
+        sms, _ = time_exactly(dev, sgraph.launch, max(args.steps, MIN_LAUNCHES), args.warmup)
+        sms /= max(args.steps, MIN_LAUNCHES)
+        streaming = {"ms_per_step": round(sms, 5), "GBps": round(gbs_of(sms), 2),
+                     "per_step": per_step_stats(dev, sgraph.launch, args.steps),
                      "kernel": dev.kernel_name(skernel),
                      "shape": "tiles first to last, non-temporal loads and stores, 2 vectors per thread"}
+        check_chain(out.slice(0, 1 << 20).read(), cpu_oracle_chain(x[: 1 << 20]), "the streaming-pinned fused chain")
+        sgraph.destroy()
 
-    dms, _ = time_steps(dev, fused_step, args.steps, args.warmup, settle_ms=100)   # the fused kernel launched directly
-    direct_ms = dms / args.steps
+    direct_ms, direct_n = time_floor(dev, fused_step)   # the fused kernel launched directly, not replayed
 
-    # Headline.  One step = what `Lazy::run` does from the second run on: replay the graph that
+    # Headline.  One step = what a lazy run does from its second run on: replay the recording that
     # holds the fused kernel.  (The first run records and builds it; that is outside the timed region.)
     dev.capture_begin()
     fused_step()
     graph = dev.capture_end()
     assert graph.kernel_nodes == 1
-    ms, wall_ms = time_steps(dev, graph.launch, args.steps, args.warmup, settle_ms=100)
+    ms, wall_ms = time_exactly(dev, graph.launch, args.steps, args.warmup)
     per_launch_ms = ms / args.steps
+    per_step = per_step_stats(dev, graph.launch, args.steps)
     graph.destroy()
-    gbs = algo_bytes / (per_launch_ms * 1e-3) / 1e9
+    gbs = gbs_of(per_launch_ms)
 
     # parity of the very buffer that was timed, on the CPU sample
     fused_step()
     got = out.read()
     base, want = cpu_baseline_c2(x, min(n, 1 << args.cpu_log2n))
-    diff = float(np.max(np.abs(got[: want.size] - want)))
-    tol = 8 * float(np.spacing(np.float32(1.0)))
-    if not diff <= tol:
-        raise SystemExit(f"bench: fused chain differs from the CPU oracle: max abs diff {diff} > {tol}")
+    diff = check_chain(got, want, "the fused chain")
+    if stack.get("dump") is not None:
+        stack["max_abs_diff_vs_cpu_oracle"] = check_chain(stack.pop("dump"), want, "the module stack's fused chain")
 
+    roof_ms = streaming["ms_per_step"] if streaming else per_launch_ms
+    roof_kernel = streaming["kernel"] if streaming else dev.kernel_name(kernel)
+    traffic, traffic_source = measured_traffic("c2 streaming") if (streaming and args.log2n == 28) else (None, None)
     return {
         "metric": "fused unary-chain GB/s and % of HBM peak, f32 N=2^28, 1xMI355X",
         "value": round(gbs, 2),
         "unit": "GB/s",
         "ms_per_step": round(per_launch_ms, 5),
         "config": {
-            "workload": f"c2: fused relu(sin(x)*2+1)-0.5, f32, N=2^{args.log2n}, x~U[-pi,pi) seed 0, "
-                        "Lazy+Graph unary fusion -> 1 kernel",
+            "workload": f"c2: y = relu(sin(x)*2+1)-0.5 as ONE fused kernel (the text that unary fusing of the five recorded "
+                        f"apply_fn operations emits), f32, N=2^{args.log2n}, x~U[-pi,pi) seed 0; one step = one replay of the "
+                        "one-node recording through custos_hip_graph_launch (C ABI), launches alternate their direction, no "
+                        "wait between steps; the same workload through the C++ module stack with a wait per run: module_stack",
             "elements": n,
             "algorithmic_bytes_per_element": 8,
         },
         "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "elements_per_s": round(n / (per_launch_ms * 1e-3), 1),
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
-        "direct_launch": {"ms_per_step": round(direct_ms, 5), "GBps": round(algo_bytes / (direct_ms * 1e-3) / 1e9, 2)},
+        "per_step": per_step,
+        "module_stack": stack,
+        "direct_launch": {"ms_per_step": round(direct_ms, 5), "GBps": round(gbs_of(direct_ms), 2), "launches": direct_n},
         "hbm_streaming_only": streaming,
         "unfused": {
             "ms_per_step": round(unfused_ms, 5),
-            "effective_GBps_on_8B_basis": round(algo_bytes / (unfused_ms * 1e-3) / 1e9, 2),
-            "moved_GBps_on_40B_basis": round(5 * algo_bytes / (unfused_ms * 1e-3) / 1e9, 2),
+            "steps": unfused_n,
+            "effective_GBps_on_8B_basis": round(gbs_of(unfused_ms), 2),
+            "moved_GBps_on_40B_basis": round(5 * gbs_of(unfused_ms), 2),
             "speedup_fused": round(unfused_ms / per_launch_ms, 3),
         },
         "copy_kernel": {
-            "name": dev.kernel_name(copy_kernel, n),
+            "name": dev.kernel_name(copy_kernel),
             "ms_per_launch": round(copy_ms, 5),
-            "GBps": round(algo_bytes / (copy_ms * 1e-3) / 1e9, 2),
+            "launches": copy_n,
+            "GBps": round(gbs_of(copy_ms), 2),
             "bytes_per_launch": algo_bytes,
         },
         "max_abs_diff_vs_cpu_oracle": diff,
         "roofline": {
             "bound": "hbm",
-            "achieved": round(gbs, 2),
+            "achieved": round(gbs_of(roof_ms), 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_C2_N2P28 if (args.log2n == 28 and not tuned) else None,
-            "kernel": dev.kernel_name(kernel, n),
+            "frac": round(gbs_of(roof_ms) / HBM_PEAK_GBS, 4),
+            "traffic": traffic,
+            "traffic_source": traffic_source,
+            "kernel": roof_kernel,
             "algorithmic_bytes_per_launch": algo_bytes,
-            "avg_launch_ms": round(per_launch_ms, 5),
+            "avg_launch_ms": round(roof_ms, 5),
+            "what": ("the fused kernel pinned to first-to-last streaming (hbm_streaming_only): HBM only" if streaming
+                     else "the fused kernel with the launch shape given on the command line"),
+            "with_memory_side_cache": {"achieved": round(gbs, 2), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                                       "what": "the headline replay: launches alternate their direction and start on "
+                                               "the 256 MiB the memory-side cache still holds"},
         },
         "cpu_baseline": base,
     }
+
+
+def cpu_oracle_chain(x):
+    from oracle import cpu_oracle
+    return cpu_oracle.c2_chain_fused(np.ascontiguousarray(x))
 
 
 def _cpu_time(fn, *a):
@@ -259,7 +373,7 @@ def _entry(name, n, bytes_per_elt, ms, cpu_s, cpu_n, note=""):
     }
 
 
-def bench_others(dev, args):
+def bench_others(dev, args, stack_c5):
     """The other BASELINE configurations (c1, c3, c4, c5), each with its CPU port beside it."""
     import custos_amd
     from custos_amd import Const, capi, synth
@@ -267,7 +381,6 @@ def bench_others(dev, args):
     from oracle import cpu_oracle
 
     lib, h = dev.lib, dev.handle
-    steps, warm = max(5, args.steps // 2), max(2, args.warmup // 2)
     out = {}
 
     # c1: apply_fn(exp), f32 N = 2^20 (latency-bound: 8 MiB of traffic)
@@ -275,12 +388,26 @@ def bench_others(dev, args):
     x = synth.uniform_f32(0, n, -4, 4)
     xb, ob = dev.buffer(x), dev.alloc(n)
     k = dev.compile(capi.KIND_APPLY, "f32", "exp(x)", ("x",))
-    ms, _ = time_steps(dev, lambda: capi.check(lib.custos_hip_apply_fn(h, k, xb.ptr, ob.ptr, n), h), steps * 4, warm, settle_ms=50)
+    step = launcher(dev, lib.custos_hip_apply_fn, k, xb.ptr, ob.ptr, n)
+    ms, launches = time_floor(dev, step)
     cpu_s, want = _cpu_time(cpu_oracle.c1_exp, x)
     got = ob.read()
     assert np.max(np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))) <= 4
-    out["c1"] = _entry("c1: apply_fn(exp), f32 N=2^20, U[-4,4) seed 0", n, 8, ms / (steps * 4), cpu_s, n)
-    out["c1"]["kernel"] = dev.kernel_name(k, n)
+    out["c1"] = _entry("c1: apply_fn(exp), f32 N=2^20, U[-4,4) seed 0", n, 8, ms, cpu_s, n,
+                       note="back-to-back launches through the C ABI from Python: the larger of the kernel's time "
+                            "and the host's time per launch")
+    out["c1"]["launches"] = launches
+    out["c1"]["kernel"] = dev.kernel_name(k)
+    # the same launch recorded 64 times into one graph (every launch writes the same output, so
+    # the graph is a chain of 64 nodes): the device's time per launch, without the host's
+    dev.capture_begin()
+    for i in range(64):
+        capi.check(lib.custos_hip_apply_fn(h, k, xb.ptr, ob.ptr, n), h)
+    g = dev.capture_end()
+    gms, _ = time_floor(dev, g.launch, launches_per_step=g.kernel_nodes)
+    out["c1"]["in_a_graph"] = {"us_per_launch": round(gms / g.kernel_nodes * 1e3, 3), "kernel_nodes": g.kernel_nodes,
+                               "what": "64 such launches into the same output recorded as one hipGraph (a chain of 64 nodes)"}
+    g.destroy()
 
     # c3: unary_ew tanh forward + backward, f32 N = 2^26
     n = 1 << 26
@@ -291,22 +418,23 @@ def bench_others(dev, args):
     kf = dev.compile(capi.KIND_APPLY, "f32", "tanh(x)", ("x",))
     grad_src = Const(1.0).sub(custos_amd.Resolve("x").tanh().mul(custos_amd.Resolve("x").tanh())).to_cl_source("f32")
     kb = dev.compile(capi.KIND_UNARY_GRAD, "f32", grad_src, ("x",))
+    fwd = launcher(dev, lib.custos_hip_apply_fn, kf, xb.ptr, yb.ptr, n)
+    bwd = launcher(dev, lib.custos_hip_add_unary_grad, kb, xb.ptr, gb.ptr, ygb.ptr, n)
 
     def c3_step():
-        capi.check(lib.custos_hip_apply_fn(h, kf, xb.ptr, yb.ptr, n), h)
-        capi.check(lib.custos_hip_add_unary_grad(h, kb, xb.ptr, gb.ptr, ygb.ptr, n), h)
+        fwd()
+        bwd()
 
-    ms, _ = time_steps(dev, c3_step, steps, warm, settle_ms=50)
-    ms_f, _ = time_steps(dev, lambda: capi.check(lib.custos_hip_apply_fn(h, kf, xb.ptr, yb.ptr, n), h), steps, warm, settle_ms=50)
-    ms_b, _ = time_steps(dev, lambda: capi.check(lib.custos_hip_add_unary_grad(h, kb, xb.ptr, gb.ptr, ygb.ptr, n), h), steps, warm, settle_ms=50)
+    ms, c3_steps = time_floor(dev, c3_step, launches_per_step=2)
+    ms_f, _ = time_floor(dev, fwd)
+    ms_b, _ = time_floor(dev, bwd)
     cn = min(n, 1 << 24)
     g0 = np.full(cn, 0.1, dtype=np.float32)
     cpu_s, _ = _cpu_time(lambda: (cpu_oracle.c3_tanh_fwd(x[:cn]), cpu_oracle.c3_tanh_bwd(x[:cn], g0, yg[:cn])))
-    e = _entry("c3: unary_ew tanh fwd + bwd (x_grad += y_grad*(1-tanh(x)^2)), f32 N=2^26", n, 24, ms / steps, cpu_s, cn)
-    e["forward"] = {"ms": round(ms_f / steps, 5), "GBps": round(8 * n / (ms_f / steps * 1e-3) / 1e9, 2),
-                    "kernel": dev.kernel_name(kf, n)}
-    e["backward"] = {"ms": round(ms_b / steps, 5), "GBps": round(16 * n / (ms_b / steps * 1e-3) / 1e9, 2),
-                     "kernel": dev.kernel_name(kb, n)}
+    e = _entry("c3: unary_ew tanh fwd + bwd (x_grad += y_grad*(1-tanh(x)^2)), f32 N=2^26", n, 24, ms, cpu_s, cn)
+    e["steps"] = c3_steps
+    e["forward"] = {"ms": round(ms_f, 5), "GBps": round(8 * n / (ms_f * 1e-3) / 1e9, 2), "kernel": dev.kernel_name(kf)}
+    e["backward"] = {"ms": round(ms_b, 5), "GBps": round(16 * n / (ms_b * 1e-3) / 1e9, 2), "kernel": dev.kernel_name(kb)}
     out["c3"] = e
     del xb, ygb, yb, gb
 
@@ -316,17 +444,18 @@ def bench_others(dev, args):
     xb, ob = dev.buffer(xh.view(np.float16), "f16"), dev.alloc(n, "f16")
     c4 = lambda v: v.mul(0.5).exp().mul(v).add(v.mul(v))
     k = dev.compile(capi.KIND_APPLY, "f16", c4(custos_amd.Resolve("x")).to_cl_source("f16"), ("x",))
-    ms, _ = time_steps(dev, lambda: capi.check(lib.custos_hip_apply_fn(h, k, xb.ptr, ob.ptr, n), h), steps, warm, settle_ms=50)
+    ms, c4_steps = time_floor(dev, launcher(dev, lib.custos_hip_apply_fn, k, xb.ptr, ob.ptr, n))
     cn = min(n, 1 << 24)
     cpu_s, want = _cpu_time(cpu_oracle.c4_chain_f16, np.ascontiguousarray(xh[:cn]))
     got = ob.slice(0, cn).read().view(np.uint16)
     d = np.abs(got.view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
     assert d.max() <= 1, "c4 differs from the CPU port by more than 1 f16 ulp"
-    out["c4"] = _entry(f"c4: f16 chain exp(x*0.5)*x + x^2, f32 compute, N=2^{args.log2n}", n, 4, ms / steps, cpu_s, cn)
-    out["c4"]["kernel"] = dev.kernel_name(k, n)
+    out["c4"] = _entry(f"c4: f16 chain exp(x*0.5)*x + x^2, f32 compute, N=2^{args.log2n}", n, 4, ms, cpu_s, cn)
+    out["c4"]["launches"] = c4_steps
+    out["c4"]["kernel"] = dev.kernel_name(k)
     del xb, ob
 
-    # c5: 1024 buffers x 4096 f32: t=a*b; u=t+c; y=sqrt(abs(u))*0.3, one graph, 100 replays
+    # c5: 1024 buffers x 4096 f32: t=a*b; u=t+c; y=sqrt(abs(u))*0.3, recorded once, replayed
     nbuf, m = 1024, 4096
     mk = lambda seed: dev.buffer(gen_chunked(lambda q, off: synth.uniform_f32(seed, q, 0, 1, off), nbuf * m))
     A, B, Cc = mk(1), mk(2), mk(3)
@@ -334,52 +463,65 @@ def bench_others(dev, args):
     kmul = dev.compile(capi.KIND_APPLY, "f32", "(x * y)", ("x", "y"))
     kadd = dev.compile(capi.KIND_APPLY, "f32", "(x + y)", ("x", "y"))
     kun = dev.compile(capi.KIND_APPLY, "f32", fused_source([lambda v: v.abs().sqrt(), lambda v: v.mul(0.3)]), ("x",))
-    dev.capture_begin()
-    for i in range(nbuf):
-        o = i * m * 4
-        capi.check(lib.custos_hip_apply_fn2(h, kmul, A.ptr + o, B.ptr + o, T.ptr + o, m), h)
-        capi.check(lib.custos_hip_apply_fn2(h, kadd, T.ptr + o, Cc.ptr + o, U.ptr + o, m), h)
-        capi.check(lib.custos_hip_apply_fn(h, kun, U.ptr + o, Y.ptr + o, m), h)
-    t0 = time.perf_counter()
-    graph = dev.capture_end()
-    build_s = time.perf_counter() - t0
-    replays = 100
-    ms, wall = time_steps(dev, graph.launch, replays, 3, settle_ms=50)
     a, b, c = A.read(), B.read(), Cc.read()
     cpu_s, (_, _, want) = _cpu_time(cpu_oracle.c5_graph, a, b, c)
-    assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), "c5 replay differs from the CPU port"
-    e = _entry("c5: 1024 x f32[4096], t=a*b; u=t+c; y=sqrt(abs(u))*0.3, one hipGraph, 100 replays", nbuf * m, 16,
-               ms / replays, cpu_s, nbuf * m, note="GB/s on the minimal 16 B/element; the recorded 3-kernel form moves 32 B/element")
-    e["us_per_replay"] = round(ms / replays * 1e3, 2)
-    e["wall_us_per_replay"] = round(wall / replays * 1e3, 2)
+
+    def record_c5(fused_kernel=None):
+        dev.capture_begin()
+        for i in range(nbuf):
+            o = i * m * 4
+            if fused_kernel is None:
+                capi.check(lib.custos_hip_apply_fn2(h, kmul, A.ptr + o, B.ptr + o, T.ptr + o, m), h)
+                capi.check(lib.custos_hip_apply_fn2(h, kadd, T.ptr + o, Cc.ptr + o, U.ptr + o, m), h)
+                capi.check(lib.custos_hip_apply_fn(h, kun, U.ptr + o, Y.ptr + o, m), h)
+            else:
+                ptrs = (C.c_uint64 * 3)(A.ptr + o, B.ptr + o, Cc.ptr + o)
+                capi.check(lib.custos_hip_apply_fn_n(h, fused_kernel, ptrs, 3, Y.ptr + o, m), h)
+        t0 = time.perf_counter()
+        graph = dev.capture_end()
+        return graph, time.perf_counter() - t0
+
+    def timed_c5(graph, what):
+        Y.clear()
+        ms_, replays = time_floor(dev, graph.launch, launches_per_step=max(1, graph.kernel_nodes))
+        assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), f"c5 {what} differs from the CPU port"
+        return {"us_per_replay": round(ms_ * 1e3, 2), "replays": replays, "GBps_on_16B": round(16 * nbuf * m / (ms_ * 1e-3) / 1e9, 2),
+                "kernel_nodes": graph.kernel_nodes, "replayed_as": what}
+
+    default_direct = args.direct_replay if args.direct_replay is not None else 4
+    graph, build_s = record_c5()
+    plain = timed_c5(graph, f"{graph.kernel_nodes} plain launches on the compute stream (a recording of at most "
+                            f"{default_direct} nodes is not instantiated as a hipGraph)" if default_direct >= graph.kernel_nodes
+                     else "one hipGraphLaunch")
+    e = _entry("c5: 1024 x f32[4096], t=a*b; u=t+c; y=sqrt(abs(u))*0.3, 3072 launches recorded once, then replayed",
+               nbuf * m, 16, plain["us_per_replay"] * 1e-3, cpu_s, nbuf * m,
+               note="GB/s on the minimal 16 B/element; the recorded 3-kernel form moves 32 B/element")
+    e["us_per_replay"] = plain["us_per_replay"]
+    e["replayed_as"] = plain["replayed_as"]
+    e["replays"] = plain["replays"]
     e["graph_kernel_nodes"] = graph.kernel_nodes
     e["recorded_launches"] = 3 * nbuf
     e["graph_build_ms"] = round(build_s * 1e3, 2)
-    e["kernels"] = [dev.kernel_name(q, nbuf * m) + "_batched" for q in (kmul, kadd, kun)]
+    e["kernels"] = [dev.kernel_name(q) + "_batched" for q in (kmul, kadd, kun)]
     graph.destroy()
+    # the same recording instantiated as a hipGraph and replayed with one hipGraphLaunch
+    dev.set_graph_direct_replay(0)
+    graph, _ = record_c5()
+    e["as_hipgraph"] = timed_c5(graph, "one hipGraphLaunch of the instantiated 3-node graph")
+    graph.destroy()
+    dev.set_graph_direct_replay(default_direct)
 
-    # the same work after element-wise fusing (what `Lazy::elementwise_fusing` of the host stack
-    # records): one three-operand kernel per buffer, 16 B/element, merged into one kernel node
-    kf = dev.compile(capi.KIND_APPLY, "f32", "(sqrt(abs(((a * b) + c))) * 0.3)", ("a", "b", "c"))
-    Y.clear()
-    dev.capture_begin()
-    for i in range(nbuf):
-        o = i * m * 4
-        ptrs = (C.c_uint64 * 3)(A.ptr + o, B.ptr + o, Cc.ptr + o)
-        capi.check(lib.custos_hip_apply_fn_n(h, kf, ptrs, 3, Y.ptr + o, m), h)
-    fgraph = dev.capture_end()
-    fms, fwall = time_steps(dev, fgraph.launch, replays, 3, settle_ms=50)
-    assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), "c5 fused replay differs from the CPU port"
-    e["fused"] = {
-        "us_per_replay": round(fms / replays * 1e3, 2),
-        "wall_us_per_replay": round(fwall / replays * 1e3, 2),
-        "GBps": round(16 * nbuf * m / (fms / replays * 1e-3) / 1e9, 2),
-        "graph_kernel_nodes": fgraph.kernel_nodes,
-        "expression": "(sqrt(abs(((a * b) + c))) * 0.3)",
-        "kernel": dev.kernel_name(kf, nbuf * m) + "_batched",
-    }
+    # the same work after element-wise fusing (the text `Lazy::elementwise_fusing` of the host stack
+    # emits for these operations): one three-operand kernel per buffer, 16 B/element, one node
+    kfused = dev.compile(capi.KIND_APPLY, "f32", "(sqrt(abs(((a * b) + c))) * 0.3)", ("a", "b", "c"))
+    graph, _ = record_c5(kfused)
+    e["fused"] = timed_c5(graph, "1 plain launch on the compute stream")
+    e["fused"]["expression"] = "(sqrt(abs(((a * b) + c))) * 0.3)"
+    e["fused"]["kernel"] = dev.kernel_name(kfused) + "_batched"
+    e["fused"]["GBps"] = e["fused"]["GBps_on_16B"]
+    graph.destroy()
+    e["module_stack"] = stack_c5
     out["c5"] = e
-    fgraph.destroy()
     return out
 
 
@@ -402,10 +544,26 @@ def main():
                     help="1: tiles first to last; 2: every launch the other way round; 0: library default")
     ap.add_argument("--no-others", dest="others", action="store_false",
                     help="skip the other BASELINE configurations (c1, c3, c4, c5)")
+    ap.add_argument("--no-module-stack", dest="module_stack", action="store_false",
+                    help="skip the child processes that time the C++ module stack")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU; the element-wise path needs no second one "
                          "(--gpus must be 1)")
+    if args.steps < 1 or args.warmup < 0:
+        raise SystemExit("bench.py: --steps must be positive, --warmup not negative")
+
+    # The module stack runs in child processes, one after the other, before this process
+    # touches the GPU.
+    stack, stack_c5 = {"skipped": True}, {"skipped": True}
+    if args.module_stack:
+        with tempfile.TemporaryDirectory() as tmp:
+            dump = os.path.join(tmp, "c2_first.f32")
+            stack = module_stack("c2", args.steps, args.warmup, log2n=args.log2n, dump=(1 << 20, dump))
+            if "error" not in stack and os.path.exists(dump):
+                stack["dump"] = np.fromfile(dump, dtype=np.float32)
+        if args.others:
+            stack_c5 = {"as_recorded": module_stack("c5", 500, 20), "after_elementwise_fusing": module_stack("c5", 500, 20, fuse=True)}
 
     import custos_amd
 
@@ -415,9 +573,9 @@ def main():
     if args.block or args.unroll or args.blocks_per_cu or args.nontemporal or args.direction:
         dev.set_tuning(args.block, args.unroll, args.blocks_per_cu, args.nontemporal, args.direction)
     info = dev.info()
-    res = {"c2": bench_c2}[args.workload](dev, args)
+    res = {"c2": bench_c2}[args.workload](dev, args, stack)
     if args.others:
-        res["other_configs"] = bench_others(dev, args)
+        res["other_configs"] = bench_others(dev, args, stack_c5)
     res.update({
         "n_gpus": 1,
         "steps": args.steps,

@@ -153,6 +153,8 @@ PROTOTYPES = {
     "custos_hip_graph_destroy": (C.c_int32, [_P, _P]),
     "custos_hip_timer_begin": (C.c_int32, [_P]),
     "custos_hip_timer_end": (C.c_int32, [_P, C.POINTER(C.c_double)]),
+    "custos_hip_timer_mark": (C.c_int32, [_P, C.c_uint32]),
+    "custos_hip_timer_between": (C.c_int32, [_P, C.c_uint32, C.c_uint32, C.POINTER(C.c_double)]),
 }
 
 _lib = None

@@ -418,6 +418,8 @@ int32_t custos_hip_device_destroy(custos_hip_device* dev) {
             if (k->module) (void)hipModuleUnload(k->module);
     (void)hipEventDestroy(dev->t0);
     (void)hipEventDestroy(dev->t1);
+    for (hipEvent_t mark : dev->marks)
+        if (mark) (void)hipEventDestroy(mark);
     (void)hipStreamDestroy(dev->stream);
     (void)hipStreamDestroy(dev->transfer);
     if (dev->done_flag) (void)hipHostFree(dev->done_flag);
@@ -767,6 +769,29 @@ int32_t custos_hip_timer_end(custos_hip_device* dev, double* ms) {
     HIP_TRY(dev, hipEventSynchronize(dev->t1));
     float f = 0.f;
     HIP_TRY(dev, hipEventElapsedTime(&f, dev->t0, dev->t1));
+    *ms = f;
+    return CUSTOS_HIP_OK;
+}
+
+// Numbered marks for per-step timing: an event per index, created on first use.
+int32_t custos_hip_timer_mark(custos_hip_device* dev, uint32_t index) {
+    REQUIRE_DEV(dev);
+    if (index >= 4096) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "timer marks are numbered 0..4095");
+    if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot time a recording stream");
+    if (dev->marks.size() <= index) dev->marks.resize(index + 1, nullptr);
+    if (!dev->marks[index]) HIP_TRY(dev, hipEventCreate(&dev->marks[index]));
+    HIP_TRY(dev, hipEventRecord(dev->marks[index], dev->stream));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_timer_between(custos_hip_device* dev, uint32_t first, uint32_t second, double* ms) {
+    REQUIRE_DEV(dev);
+    if (!ms) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "ms is null");
+    if (first >= dev->marks.size() || second >= dev->marks.size() || !dev->marks[first] || !dev->marks[second])
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "a timer mark that was never recorded");
+    HIP_TRY(dev, hipEventSynchronize(dev->marks[second]));
+    float f = 0.f;
+    HIP_TRY(dev, hipEventElapsedTime(&f, dev->marks[first], dev->marks[second]));
     *ms = f;
     return CUSTOS_HIP_OK;
 }

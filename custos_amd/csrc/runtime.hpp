@@ -118,6 +118,7 @@ struct custos_hip_device {
     hipStream_t stream = nullptr;    // compute stream: every launch, in call order
     hipStream_t transfer = nullptr;  // copies that must not be recorded while capturing
     hipEvent_t t0 = nullptr, t1 = nullptr;
+    std::vector<hipEvent_t> marks;   // custos_hip_timer_mark: an event per index, created on first use
     hipDeviceProp_t props{};
     std::string arch;
     custos_hip::Tuning tuning;

@@ -376,3 +376,13 @@ class HIP:
         ms = C.c_double(0)
         self._check(self.lib.custos_hip_timer_end(self.handle, C.byref(ms)))
         return ms.value
+
+    def timer_mark(self, index: int) -> None:
+        """Records mark `index` (0..4095) on the compute stream behind the work issued so far."""
+        self._check(self.lib.custos_hip_timer_mark(self.handle, index))
+
+    def timer_between(self, first: int, second: int) -> float:
+        """Milliseconds from mark `first` to mark `second` (waits for the second)."""
+        ms = C.c_double(0)
+        self._check(self.lib.custos_hip_timer_between(self.handle, first, second, C.byref(ms)))
+        return ms.value

@@ -115,4 +115,6 @@ extern "C" {
     pub fn custos_hip_graph_destroy(dev: *mut HipDeviceHandle, graph: *mut HipGraph) -> i32;
     pub fn custos_hip_timer_begin(dev: *mut HipDeviceHandle) -> i32;
     pub fn custos_hip_timer_end(dev: *mut HipDeviceHandle, ms: *mut f64) -> i32;
+    pub fn custos_hip_timer_mark(dev: *mut HipDeviceHandle, index: u32) -> i32;
+    pub fn custos_hip_timer_between(dev: *mut HipDeviceHandle, first: u32, second: u32, ms: *mut f64) -> i32;
 }

@@ -49,8 +49,14 @@ struct Timing {
     double mean_us, median_us, min_us;
 };
 
+// `settle_ms`: after the first run (which records, compiles and builds the graph) runs are
+// repeated untimed until that much time has passed; after an idle period the device needs some
+// tens of milliseconds of work to return to its steady clocks.
 template <class F>
-static Timing time_runs(F run, int warmup, int steps) {
+static Timing time_runs(F run, int warmup, int steps, int settle_ms) {
+    run();
+    const auto settled = std::chrono::steady_clock::now() + std::chrono::milliseconds(settle_ms);
+    while (std::chrono::steady_clock::now() < settled) run();
     for (int i = 0; i < warmup; i++) run();
     std::vector<double> us(static_cast<size_t>(steps));
     for (int i = 0; i < steps; i++) {
@@ -77,7 +83,7 @@ static void dump(Dev& device, uint64_t ptr, size_t count, const char* path) {
 
 int main(int argc, char** argv) {
     std::string config = "c2", dump_path;
-    int log2n = 28, steps = 100, warmup = 20;
+    int log2n = 28, steps = 100, warmup = 20, settle_ms = 150;
     size_t dump_count = 0;
     bool fuse = false;
     for (int i = 1; i < argc; i++) {
@@ -93,6 +99,7 @@ int main(int argc, char** argv) {
         else if (a == "--log2n") log2n = std::atoi(value());
         else if (a == "--steps") steps = std::atoi(value());
         else if (a == "--warmup") warmup = std::atoi(value());
+        else if (a == "--settle-ms") settle_ms = std::atoi(value());
         else if (a == "--fuse") fuse = true;
         else if (a == "--dump") {
             dump_count = static_cast<size_t>(std::atoll(value()));
@@ -102,7 +109,7 @@ int main(int argc, char** argv) {
             return 2;
         }
     }
-    if (steps < 1 || warmup < 0 || log2n < 4 || log2n > 32) return 2;
+    if (steps < 1 || warmup < 0 || settle_ms < 0 || log2n < 4 || log2n > 32) return 2;
 
     try {
         if (config == "c2") {
@@ -117,7 +124,7 @@ int main(int argc, char** argv) {
             auto out = device.apply_fn(r, [](auto x) { return x.sub(0.5f); });
             device.optimize_mem_graph();
             device.unary_fusing();
-            const Timing t = time_runs([&] { device.run(); }, warmup, steps);
+            const Timing t = time_runs([&] { device.run(); }, warmup, steps, settle_ms);
             if (dump_count) dump(device, out.replace().ptr(), std::min(dump_count, n), dump_path.c_str());
             const double gbs = 8.0 * static_cast<double>(n) / (t.mean_us * 1e-6) / 1e9;
             std::printf("{\"config\": \"c2\", \"stack\": \"HIP<Graph<Lazy<Base>>>\", \"calls\": \"5 x apply_fn, optimize_mem_graph, "
@@ -142,7 +149,7 @@ int main(int argc, char** argv) {
                 ys.push_back(device.apply_fn(u, [](auto x) { return x.abs().sqrt().mul(0.3f); }));
             }
             if (fuse) device.elementwise_fusing();
-            const Timing t = time_runs([&] { device.run(); }, warmup, steps);
+            const Timing t = time_runs([&] { device.run(); }, warmup, steps, settle_ms);
             if (dump_count) dump(device, ys[0].replace().ptr(), std::min(dump_count, m), dump_path.c_str());
             const double gbs = 16.0 * static_cast<double>(nbuf * m) / (t.mean_us * 1e-6) / 1e9;
             std::printf("{\"config\": \"c5\", \"stack\": \"HIP<Graph<Lazy<Base>>>\", \"calls\": \"1024 x (apply_fn2, apply_fn2, apply_fn)%s, "

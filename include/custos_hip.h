@@ -437,6 +437,13 @@ int32_t custos_hip_timer_begin(custos_hip_device *dev);
 /* Records the end event, waits for it, returns milliseconds since timer_begin. */
 int32_t custos_hip_timer_end(custos_hip_device *dev, double *ms);
 
+/* Per-step timing: records mark number `index` (0..4095) on the compute stream, behind the work
+ * issued so far; `timer_between` waits for mark `second` and returns the milliseconds from mark
+ * `first` to it.  A mark between every two steps of a loop gives every step's own duration
+ * (median, minimum) without a wait inside the loop. */
+int32_t custos_hip_timer_mark(custos_hip_device *dev, uint32_t index);
+int32_t custos_hip_timer_between(custos_hip_device *dev, uint32_t first, uint32_t second, double *ms);
+
 #ifdef __cplusplus
 }
 #endif
