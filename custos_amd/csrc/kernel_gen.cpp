@@ -163,7 +163,16 @@ static __device__ __forceinline__ double custos_sqrt(double a) { return sqrt(a);
         // tanh / log keep the full-precision routines: their results pass through
         // zero, where only a relative bound in f32 keeps the 16-bit result within
         // one ulp.
-        if (dtype == DType::F16 || dtype == DType::BF16 || dtype_rounds_per_node(dtype))
+        // bf16 has f32's exponent range, and the hardware exp2 gives 0 where the result is an
+        // f32 denormal (inputs below -87.3, which the reference's expf turns into bf16
+        // denormals): there the exponent is raised by 64 and the result scaled back, a
+        // multiplication that rounds into the denormal range correctly.
+        if (dtype == DType::BF16 || dtype == DType::BF16_PERNODE)
+            s += "static __device__ __forceinline__ float custos_exp(float a) {\n"
+                 "    const float t = a * 0x1.715476p+0f;\n"
+                 "    const bool tiny = t < -126.0f;\n"
+                 "    return __builtin_amdgcn_exp2f(tiny ? t + 64.0f : t) * (tiny ? 0x1p-64f : 1.0f);\n}\n";
+        else if (dtype == DType::F16 || dtype == DType::F16_PERNODE)
             s += "static __device__ __forceinline__ float custos_exp(float a) {\n"
                  "    return __builtin_amdgcn_exp2f(a * 0x1.715476p+0f);\n}\n";
         else
@@ -481,7 +490,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds the vectors per thread as requested: 0 = chosen per launch)
     int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, 13 /* template version */};
+                       k.tuning.blocks_per_cu, 14 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
