@@ -411,8 +411,8 @@ int32_t custos_hip_device_destroy(custos_hip_device* dev) {
     (void)hipStreamSynchronize(dev->stream);
     (void)hipStreamSynchronize(dev->transfer);
     for (custos_hip_graph* g : dev->graphs) destroy_graph(g);
-    for (auto& kv : dev->pool)
-        for (void* p : kv.second) (void)hipFree(p);
+    // every block of this handle goes back to the driver, pooled or still held by the caller
+    for (auto& kv : dev->block_bytes) (void)hipFree(reinterpret_cast<void*>(kv.first));
     for (auto& bucket : dev->cache)
         for (auto& k : bucket.second)
             if (k->module) (void)hipModuleUnload(k->module);
@@ -507,6 +507,7 @@ int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, ui
         pooled->second.pop_back();
         dev->pooled_bytes -= rounded;
         dev->pool_reused++;
+        dev->block_bytes[reinterpret_cast<uint64_t>(p)].pooled = false;
     } else {
         hipError_t e = hipMalloc(&p, rounded);
         if (e != hipSuccess && dev->pooled_bytes > 0) {
@@ -515,7 +516,7 @@ int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, ui
             e = hipMalloc(&p, rounded);
         }
         if (e != hipSuccess) return hip_fail(dev, e, "hipMalloc");
-        dev->block_bytes[reinterpret_cast<uint64_t>(p)] = rounded;
+        dev->block_bytes[reinterpret_cast<uint64_t>(p)] = {rounded, false};
         dev->pool_allocated++;
     }
     uint64_t addr = reinterpret_cast<uint64_t>(p);
@@ -541,15 +542,20 @@ int32_t custos_hip_free(custos_hip_device* dev, uint64_t dptr) {
     REQUIRE_DEV(dev);
     if (dptr == 0) return CUSTOS_HIP_OK;
     auto known = dev->block_bytes.find(dptr);
-    if (known != dev->block_bytes.end() && dev->pooled_bytes + known->second <= dev->pool_limit) {
+    if (known == dev->block_bytes.end())
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "not the address of a block this device handle allocated");
+    if (known->second.pooled)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "the block was freed already");
+    if (dev->pooled_bytes + known->second.bytes <= dev->pool_limit) {
         // Reuse is ordered on the compute stream behind whatever still uses the block.
         // (A recorded graph that names the address must not be replayed after this,
         // exactly as after a real free.)
-        dev->pool[known->second].push_back(reinterpret_cast<void*>(dptr));
-        dev->pooled_bytes += known->second;
+        known->second.pooled = true;
+        dev->pool[known->second.bytes].push_back(reinterpret_cast<void*>(dptr));
+        dev->pooled_bytes += known->second.bytes;
         return CUSTOS_HIP_OK;
     }
-    if (known != dev->block_bytes.end()) dev->block_bytes.erase(known);
+    dev->block_bytes.erase(known);
     // work that still uses the range must finish first
     if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
     HIP_TRY(dev, hipFree(reinterpret_cast<void*>(dptr)));

@@ -132,9 +132,14 @@ struct custos_hip_device {
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     bool graph_verify = false;       // built graphs are checked by brute force against the recorded conflicts
     int32_t graph_edges = CUSTOS_HIP_GRAPH_EDGES_CHAIN;  // how built graphs order their nodes
-    // allocation pool: freed blocks by rounded size; every block this handle allocated, by address
+    // allocation pool: freed blocks by rounded size; every block this handle allocated and has not
+    // returned to the driver, by address
     std::unordered_map<size_t, std::vector<void*>> pool;
-    std::unordered_map<uint64_t, size_t> block_bytes;
+    struct Block {
+        size_t bytes = 0;     // rounded size
+        bool pooled = false;  // in `pool` (freed by the caller), else handed out
+    };
+    std::unordered_map<uint64_t, Block> block_bytes;
     size_t pooled_bytes = 0, pool_limit = 0;
     uint64_t pool_reused = 0, pool_allocated = 0;
     custos_hip_kernel* identity_u32 = nullptr;  // copies run through these

@@ -21,6 +21,17 @@ def _np_dtype(dtype: str):
     return np.dtype(capi.DTYPES[dtype][1])
 
 
+def _same_shape(first, *others):
+    """Operands of one launch have one length and one element type: a shorter one would be read
+    or written beyond its end on the device (`None` entries, an output still to allocate, pass)."""
+    for other in others:
+        if other is None:
+            continue
+        if other.len != first.len or other.dtype != first.dtype:
+            raise ValueError(f"operands differ in length or element type: {first.len} x {first.dtype} "
+                             f"and {other.len} x {other.dtype}")
+
+
 class Buffer:
     """A device allocation of `len` elements (`Buffer<T, HIP>` with `CUDAPtr`-like
     base: address, length, ownership flag -- src/devices/cuda/cuda_ptr.rs:7-15)."""
@@ -222,6 +233,7 @@ class HIP:
 
     def apply_fn(self, buf: Buffer, f, out: Buffer | None = None) -> Buffer:
         """`device.apply_fn(&buf, |x| ...)`: out[i] = f(buf[i]) in a new buffer."""
+        _same_shape(buf, out)
         src = _wrap(f(Resolve("x"))).to_cl_source(buf.dtype)
         kernel = self.compile(capi.KIND_APPLY, buf.dtype, src, ("x",))
         if out is None:
@@ -231,8 +243,7 @@ class HIP:
 
     def apply_fn2(self, lhs: Buffer, rhs: Buffer, f, out: Buffer | None = None) -> Buffer:
         """Two-operand expression: out[i] = f(lhs[i], rhs[i])."""
-        if lhs.len != rhs.len or lhs.dtype != rhs.dtype:
-            raise ValueError("operands differ in length or element type")
+        _same_shape(lhs, rhs, out)
         src = _wrap(f(Resolve("x", 0), Resolve("y", 1))).to_cl_source(lhs.dtype)
         kernel = self.compile(capi.KIND_APPLY, lhs.dtype, src, ("x", "y"))
         if out is None:
@@ -242,6 +253,7 @@ class HIP:
 
     def apply_fn_n(self, ins, f, out: Buffer | None = None) -> Buffer:
         """k-operand expression (k <= 4) over markers a, b, c, d."""
+        _same_shape(*ins, out)
         names = ("a", "b", "c", "d")[: len(ins)]
         src = _wrap(f(*[Resolve(n, i) for i, n in enumerate(names)])).to_cl_source(ins[0].dtype)
         kernel = self.compile(capi.KIND_APPLY, ins[0].dtype, src, names)
@@ -268,6 +280,7 @@ class HIP:
 
     def fused_apply_fn(self, buf: Buffer, ops, out: Buffer | None = None) -> Buffer:
         """The op `unary_fuse_op` returns: all `ops` applied in sequence in one kernel."""
+        _same_shape(buf, out)
         src = fused_source(ops, buf.dtype)
         kernel = self.compile(capi.KIND_APPLY, buf.dtype, src, ("x",))
         if out is None:
@@ -277,6 +290,7 @@ class HIP:
 
     def add_unary_grad(self, lhs: Buffer, lhs_grad: Buffer, out_grad: Buffer, lhs_grad_fn) -> None:
         """`device.add_unary_grad(&lhs, &mut lhs_grad, &out_grad, |x| ...)`."""
+        _same_shape(lhs, lhs_grad, out_grad)
         src = _wrap(lhs_grad_fn(Resolve("x"))).to_cl_source(lhs.dtype)
         kernel = self.compile(capi.KIND_UNARY_GRAD, lhs.dtype, src, ("x",))
         self._check(self.lib.custos_hip_add_unary_grad(self.handle, kernel, lhs.ptr, lhs_grad.ptr, out_grad.ptr, lhs.len))

@@ -8,3 +8,4 @@
 #include "hip.hpp"
 #include "modules.hpp"
 #include "opt_graph.hpp"
+#include "serde.hpp"

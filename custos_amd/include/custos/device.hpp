@@ -207,6 +207,8 @@ class Device {
     // expression written in the `Combiner` vocabulary: out[i] = f(lhs[i], rhs[i]).
     template <class T, class F>
     Buffer<T, Derived> apply_fn2(const Buffer<T, Derived>& lhs, const Buffer<T, Derived>& rhs, F f) {
+        // (a shorter operand would be read beyond its end on the device)
+        if (rhs.len() != lhs.len()) throw Error(DeviceError::ShapeLengthMismatch);
         Buffer<T, Derived> out = retrieve_output<T>(lhs.len(), lhs, rhs);
         add_op(std::tie(lhs, rhs, out),
                [f](const Buffer<T, Derived>& l, const Buffer<T, Derived>& r, Buffer<T, Derived>& o, Derived& dev) {
@@ -220,6 +222,7 @@ class Device {
     template <class T, class F>
     void add_unary_grad(const Buffer<T, Derived>& lhs, Buffer<T, Derived>& lhs_grad,
                         const Buffer<T, Derived>& out_grad, F lhs_grad_fn) {
+        if (lhs_grad.len() != lhs.len() || out_grad.len() != lhs.len()) throw Error(DeviceError::ShapeLengthMismatch);
         add_op(std::tie(lhs, lhs_grad, out_grad),
                [lhs_grad_fn](const Buffer<T, Derived>& l, Buffer<T, Derived>& g, const Buffer<T, Derived>& o, Derived& dev) {
                    dev.add_unary_grad_impl(l, g, o, lhs_grad_fn);

@@ -45,22 +45,3 @@ impl<Mods> crate::LazySetup for HIP<Mods> {
         Ok(())
     }
 }
-
-#[cfg(test)]
-mod tests {
-    use crate::{AddOperation, ApplyFunction, Base, Buffer, Combiner, HIP, Lazy, Run};
-
-    // the shape of src/devices/cuda/lazy.rs:96-196: nothing runs before `run`, and ten runs of
-    // the same program give the result of one (each run starts from the same inputs)
-    #[test]
-    fn test_lazy_apply_fn_runs_once_per_run() {
-        let device = HIP::<Lazy<Base>>::new(0).unwrap();
-        let x = Buffer::from((&device, [1., 2., 3., 4., 5., 6.]));
-        let out = device.apply_fn(&x, |x| x.mul(2.));
-        assert_eq!(device.ops_count(), 1);
-        for _ in 0..10 {
-            device.run().unwrap();
-            assert_eq!(out.replace().read(), [2., 4., 6., 8., 10., 12.]);
-        }
-    }
-}

@@ -10,6 +10,7 @@
 
 #include "check.hpp"
 #include "custos/device.hpp"
+#include "custos/serde.hpp"
 
 namespace module_tests {
 
@@ -1126,6 +1127,83 @@ void cached_errors() {
     }
 }
 
+// operands of one operation have one length: a shorter one would be read or written beyond its
+// end on the device (`DeviceError::ShapeLengthMismatch`, src/error.rs)
+template <template <class> class DEV>
+void operand_lengths_must_match() {
+    DEV<Base> dev;
+    auto six = dev.template buffer<float>({1.f, 2.f, 3.f, 4.f, 5.f, 6.f});
+    auto five = dev.template buffer<float>({1.f, 2.f, 3.f, 4.f, 5.f});
+    auto grad = dev.template buffer<float>({0.f, 0.f, 0.f, 0.f, 0.f, 0.f});
+    CHECK_THROWS_KIND(dev.apply_fn2(six, five, [](auto x, auto y) { return x.add(y); }), DeviceError::ShapeLengthMismatch);
+    CHECK_THROWS_KIND(dev.add_unary_grad(six, five, six, [](auto x) { return x.mul(2.f); }), DeviceError::ShapeLengthMismatch);
+    CHECK_THROWS_KIND(dev.add_unary_grad(six, grad, five, [](auto x) { return x.mul(2.f); }), DeviceError::ShapeLengthMismatch);
+    dev.add_unary_grad(six, grad, six, [](auto x) { return x.mul(2.f); });
+    CHECK_VEC_EQ(grad.read(), (std::vector<float>{2.f, 8.f, 18.f, 32.f, 50.f, 72.f}));  // 0 + x * 2x
+}
+
+// Buffers as sequences of elements: the token stream the reference pins for a pointer of ten
+// i32 (src/devices/cuda/cuda_ptr.rs:163-189, src/devices/cpu/cpu_ptr.rs:402-424), and the round
+// trip device -> sequence -> new device buffer for every element type, as tokens and as JSON.
+template <class T, class D>
+void serde_round_trip(D& dev, const std::vector<T>& values) {
+    auto buf = dev.template buffer<T>(values);
+    const std::vector<serde::Token> tokens = serde::to_tokens(buf);
+    CHECK_EQ(tokens.size(), values.size() + 2);
+    CHECK(tokens.front() == serde::Token::seq(values.size()) && tokens.back() == serde::Token::seq_end());
+    auto back = serde::from_tokens<T>(dev, tokens);
+    CHECK(back.ptr() != buf.ptr());
+    const std::vector<T> a = buf.read(), b = back.read(), c = serde::from_json<T>(dev, serde::to_json(buf)).read();
+    CHECK_EQ(b.size(), values.size());
+    CHECK(std::memcmp(a.data(), b.data(), a.size() * sizeof(T)) == 0);
+    CHECK_EQ(c.size(), values.size());
+    CHECK(std::memcmp(a.data(), c.data(), a.size() * sizeof(T)) == 0);
+}
+
+template <template <class> class DEV>
+void serde_of_buffers() {
+    using D = DEV<Base>;
+    D dev;
+    auto ten = dev.template buffer<int32_t>({1, 2, 3, 4, 5, 6, 7, 8, 9, 10});
+    std::vector<serde::Token> want = {serde::Token::seq(10)};
+    for (int32_t v = 1; v <= 10; v++) want.push_back({serde::TokenKind::I32, static_cast<uint64_t>(v)});
+    want.push_back(serde::Token::seq_end());
+    CHECK(serde::to_tokens(ten) == want);
+    CHECK_EQ(serde::to_json(ten), std::string("[1,2,3,4,5,6,7,8,9,10]"));
+    CHECK_VEC_EQ(serde::from_tokens<int32_t>(dev, want).read(), (std::vector<int32_t>{1, 2, 3, 4, 5, 6, 7, 8, 9, 10}));
+    CHECK_EQ(serde::to_json(dev.template buffer<float>({1.5f, -0.25f, 3.f, 0.1f})), std::string("[1.5,-0.25,3.0,0.1]"));
+    CHECK_VEC_EQ(serde::from_json<float>(dev, " [ 1.5 , -0.25,3.0 ,1e-3 ] ").read(), (std::vector<float>{1.5f, -0.25f, 3.f, 1e-3f}));
+
+    serde_round_trip<int8_t>(dev, {-128, -1, 0, 1, 127});
+    serde_round_trip<uint8_t>(dev, {0, 1, 200, 255});
+    serde_round_trip<int16_t>(dev, {-32768, -2, 0, 32767});
+    serde_round_trip<uint16_t>(dev, {0, 1, 65535});
+    serde_round_trip<int32_t>(dev, {INT32_MIN, -7, 0, 9, INT32_MAX});
+    serde_round_trip<uint32_t>(dev, {0u, 3u, 4000000000u, UINT32_MAX});
+    serde_round_trip<int64_t>(dev, {INT64_MIN, -5, 0, 5, INT64_MAX});
+    serde_round_trip<uint64_t>(dev, {0ull, 1ull, 1ull << 63, UINT64_MAX});
+    serde_round_trip<float>(dev, {0.f, -0.f, 1.f, 0.1f, -3.4028235e38f, 1.17549435e-38f, 1e-45f, 16777217.f});
+    serde_round_trip<double>(dev, {0., -0., 0.1, 1. / 3., -1.7976931348623157e308, 4.9e-324, 2.2250738585072014e-308});
+    serde_round_trip<f16>(dev, {f16(1.f), f16(-0.333f), f16::from_bits(0x0001), f16::from_bits(0x7bff), f16::from_bits(0xfc00)});
+    serde_round_trip<bf16>(dev, {bf16(1.f), bf16(-3.14f), bf16::from_bits(0x0001), bf16::from_bits(0x7f7f)});
+    serde_round_trip<f16_pernode>(dev, {f16_pernode(0.5f), f16_pernode(-65504.f)});
+    serde_round_trip<bf16_pernode>(dev, {bf16_pernode(0.5f), bf16_pernode(1e30f)});
+
+    // what is not a sequence of this element type is an error, not a buffer
+    std::vector<serde::Token> wrong_kind = want;
+    wrong_kind[3].kind = serde::TokenKind::F32;
+    CHECK_THROWS_KIND(serde::from_tokens<int32_t>(dev, wrong_kind), DeviceError::TypeMismatch);
+    CHECK_THROWS_KIND(serde::from_tokens<float>(dev, want), DeviceError::TypeMismatch);
+    std::vector<serde::Token> short_one = want;
+    short_one.erase(short_one.begin() + 4);
+    CHECK_THROWS_KIND(serde::from_tokens<int32_t>(dev, short_one), DeviceError::ShapeLengthMismatch);
+    CHECK_THROWS_KIND(serde::from_tokens<int32_t>(dev, {serde::Token::seq(0), serde::Token::seq_end()}), DeviceError::ZeroLengthBuffer);
+    CHECK_THROWS_KIND(serde::from_json<int32_t>(dev, "[1,2.5]"), DeviceError::TypeMismatch);
+    CHECK_THROWS_KIND(serde::from_json<uint8_t>(dev, "[1,256]"), DeviceError::TypeMismatch);
+    CHECK_THROWS_KIND(serde::from_json<int32_t>(dev, "[1,2"), DeviceError::ShapeLengthMismatch);
+    CHECK_THROWS_KIND(serde::from_json<int32_t>(dev, "[]"), DeviceError::ZeroLengthBuffer);
+}
+
 }  // namespace module_tests
 
 // Registers every generic case for one device template.
@@ -1180,4 +1258,6 @@ void cached_errors() {
     TEST_CASE(cached_multi_level_retrieve) { module_tests::cached_multi_level_retrieve<DEV>(); }  \
     TEST_CASE(cached_apply_fn_and_unary_ew) { module_tests::cached_apply_fn_and_unary_ew<DEV>(); } \
     TEST_CASE(cached_graph_optimize_aliases) { module_tests::cached_graph_optimize_aliases<DEV>(); } \
-    TEST_CASE(cached_errors) { module_tests::cached_errors<DEV>(); }
+    TEST_CASE(cached_errors) { module_tests::cached_errors<DEV>(); }                              \
+    TEST_CASE(serde_of_buffers) { module_tests::serde_of_buffers<DEV>(); }                        \
+    TEST_CASE(operand_lengths_must_match) { module_tests::operand_lengths_must_match<DEV>(); }

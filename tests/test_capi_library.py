@@ -138,3 +138,20 @@ def test_launch_shape_by_bytes_touched():
     assert shape(2048 * MiB, 2) == (2, 1, True)            # config 2
     with pytest.raises(capi.CustosHipError):
         shape(1, 0)
+
+
+def test_operands_of_different_lengths_are_rejected_on_the_host():
+    """A shorter operand would be read or written beyond its end on the device: the binding checks
+    lengths and element types before anything reaches the library (no device needed to see it)."""
+    from custos_amd.device import HIP, Buffer
+    dev = object.__new__(HIP)          # no library call is made before the checks
+    dev.lib, dev.handle = None, None
+    a, b = Buffer(dev, 256, 8, "f32", owned=False), Buffer(dev, 512, 7, "f32", owned=False)
+    h = Buffer(dev, 1024, 8, "f16", owned=False)
+    ident = lambda *v: v[0]
+    for call in (lambda: dev.apply_fn(a, ident, out=b), lambda: dev.apply_fn2(a, b, ident), lambda: dev.apply_fn2(a, a, ident, out=b),
+                 lambda: dev.apply_fn_n([a, a, b], ident), lambda: dev.apply_fn_n([a, a], ident, out=b),
+                 lambda: dev.fused_apply_fn(a, [ident], out=b), lambda: dev.add_unary_grad(a, b, a, ident),
+                 lambda: dev.add_unary_grad(a, a, b, ident), lambda: dev.apply_fn2(a, h, ident)):
+        with pytest.raises(ValueError):
+            call()

@@ -50,7 +50,12 @@ def test_fused_chain_c2_small(hip, oracle):
     # sin within 4 ulp; the following exact ops scale that error by at most 2 in absolute terms
     sin_ulp = np.spacing(np.float32(1.0))
     assert np.max(np.abs(got - want)) <= 4 * 2 * sin_ulp
-    assert_bits_equal(got, oracle.c2_chain_fused(x).astype(np.float32) * 0 + got)  # shape/dtype sanity
+    # the oracle's compiled loop for this chain and its expression interpreter are two pieces of
+    # code: on these inputs they agree bit for bit, and the kernel is as close to either
+    loop = oracle.c2_chain_fused(x)
+    assert_bits_equal(loop, want)
+    assert got.dtype == loop.dtype and got.shape == loop.shape
+    assert np.max(np.abs(got - loop)) <= 4 * 2 * sin_ulp
 
 
 def test_add_unary_grad_exact(hip, oracle):

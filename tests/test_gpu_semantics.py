@@ -194,6 +194,40 @@ def test_f64(hip, oracle):
                              -0.6320633326681093, 2.978716493246764], rtol=0, atol=1e-14)
 
 
+def test_f64_transcendentals(hip, oracle):
+    """f64 routine nodes against the oracle (glibc, under 1 ulp) on random inputs.  BASELINE states no
+    f64 tolerance; the bound here is 4 units in the last place of the f64 result, measured on the bit
+    patterns (the device's routines are documented to 1-2 ulp)."""
+    n = 20001
+    rng = np.random.default_rng(11)
+    x = rng.uniform(-3, 3, n)
+    pos = rng.uniform(1e-3, 50, n)
+    y = rng.uniform(-3, 3, n)
+
+    def ulps(got, want):
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        ok = ~np.isnan(want)
+        return np.abs(got[ok].view(np.int64) - want[ok].view(np.int64)).max()
+
+    for name, f, arg in (("exp", lambda v: v.exp(), x), ("cos", lambda v: v.cos(), x), ("sin", lambda v: v.sin(), x),
+                         ("tan", lambda v: v.tan(), x), ("tanh", lambda v: v.tanh(), x), ("ln", lambda v: v.ln(), pos)):
+        got = hip.apply_fn(hip.buffer(arg, "f64"), f).read()
+        want = oracle.apply_fn(f, arg, dtype="f64")
+        assert ulps(got, want) <= 4, f"f64 {name}: {ulps(got, want)} ulp"
+    power = lambda a, b: a.pow(b)
+    got = hip.apply_fn2(hip.buffer(pos, "f64"), hip.buffer(y, "f64"), power).read()
+    assert ulps(got, oracle.apply_fn(power, pos, y, dtype="f64")) <= 4
+    # special values: the same infinities, zeros and NaNs
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 709.9, -745.2, 5e-324, 1e308])
+    for name, f in (("exp", lambda v: v.exp()), ("tanh", lambda v: v.tanh()), ("ln", lambda v: v.ln()), ("cos", lambda v: v.cos())):
+        got = hip.apply_fn(hip.buffer(special, "f64"), f).read()
+        want = oracle.apply_fn(f, special, dtype="f64")
+        assert np.array_equal(np.isnan(got), np.isnan(want)), name
+        assert np.array_equal(np.isinf(got), np.isinf(want)) and np.array_equal(np.signbit(got[~np.isnan(want)]), np.signbit(want[~np.isnan(want)])), name
+        fin = np.isfinite(want)
+        assert np.abs(got[fin].view(np.int64) - want[fin].view(np.int64)).max() <= 4, name
+
+
 def test_bf16(hip, oracle):
     n = 40003
     x32 = synth.uniform_f32(71, n, -4, 4)
@@ -678,14 +712,16 @@ def test_caller_written_kernels_in_a_graph_are_fences(hip, oracle):
         assert_bits_equal(o.read(), (x * np.float32(4)).astype(np.float32))
 
 
-def test_disk_cache_of_code_objects(tmp_path, monkeypatch):
-    """CUSTOS_HIP_KERNEL_CACHE_DIR: a second device loads the code object instead of compiling."""
+def test_disk_cache_of_code_objects(tmp_path, monkeypatch, oracle):
+    """CUSTOS_HIP_KERNEL_CACHE_DIR: a second device loads the code object instead of compiling, and
+    what the loaded code computes is what the CPU oracle computes."""
     import custos_amd
     monkeypatch.setenv("CUSTOS_HIP_KERNEL_CACHE_DIR", str(tmp_path / "kcache"))
     x = synth.uniform_f32(5, 1000, -1, 1)
     f = lambda v: v.mul(0.37).add(11.5)
+    want = oracle.apply_fn(f, x)
     first = custos_amd.HIP(0)
-    want = first.apply_fn(first.buffer(x), f).read()
+    assert_bits_equal(first.apply_fn(first.buffer(x), f).read(), want)
     assert first.cache_stats()[0] == 1 and first.disk_cache_hits() == 0
     files = list((tmp_path / "kcache").iterdir())
     assert len(files) == 1 and files[0].suffix == ".co" and "gfx950" in files[0].name
@@ -1046,7 +1082,7 @@ def test_allocation_pool():
         again.free()
         smaller = dev.alloc(n - 100)                 # rounds to the same class
         assert smaller.ptr == addr
-        dirty = dev.apply_fn(a, lambda v: v.mul(2.0), out=smaller.slice(0, n - 100))
+        dev.apply_fn(a.slice(0, n - 100), lambda v: v.mul(2.0), out=smaller)
         assert_bits_equal(smaller.read(), want[: n - 100])
         smaller.free()
         dev.pool_trim()
@@ -1091,3 +1127,26 @@ def test_device_to_device_copies(hip):
             head = dst.slice(0, do + min(n, 64)).read()
             assert not head[:do].any()
             assert_bits_equal(head[do:], pattern[(np.arange(so, so + min(n, 64))) % period])
+
+
+def test_a_block_is_freed_once(hip):
+    """A second free of the same address is an error, as is the free of an address the device handle
+    never handed out; neither puts a block into the pool twice."""
+    ptr = C.c_uint64(0)
+    lib, h = hip.lib, hip.handle
+    capi.check(lib.custos_hip_alloc(h, 4096, capi.ALLOC_ZEROED, C.byref(ptr)), h)
+    assert lib.custos_hip_free(h, ptr.value) == 0
+    assert lib.custos_hip_free(h, ptr.value) == capi.ERR_INVALID_ARGUMENT
+    assert "freed already" in capi.last_error(h)
+    assert lib.custos_hip_free(h, ptr.value + 16) == capi.ERR_INVALID_ARGUMENT
+    assert lib.custos_hip_free(h, 0) == 0
+    # the pool holds the block once: two allocations of that size get two different addresses
+    a, b = hip.alloc(1024), hip.alloc(1024)
+    assert a.ptr != b.ptr
+    # blocks still held when the handle is destroyed go back to the driver with it
+    import custos_amd
+    other = custos_amd.HIP(0)
+    held = [other.alloc(1 << 20) for _ in range(4)]
+    other.close()
+    for buf in held:
+        buf.ptr = 0
