@@ -12,8 +12,9 @@ resident in HBM.  What is timed, and where:
                         launch walks the array against the direction of the launch before it and
                         so starts on the 256 MiB the memory-side cache still holds.
   per_step              the same replays with an event between every two (>= 50): median and min.
-  roofline              the same kernel pinned to plain HBM streaming (every launch first tile to
-                        last, non-temporal accesses): no help from the memory-side cache.
+  roofline              the same expression pinned to plain HBM streaming (every launch first tile to
+                        last, non-temporal accesses, one-wavefront workgroups): no help from the
+                        memory-side cache.
   module_stack          a child process started before this one touches the GPU: the C++ module
                         stack HIP<Graph<Lazy<Base>>>, five apply_fn calls, optimize_mem_graph,
                         unary_fusing, then run() with the reference's wait after every run.
@@ -244,10 +245,11 @@ def bench_c2(dev, args, stack):
 
     # The fused step pinned to plain HBM streaming: every launch walks the array from the first tile
     # to the last, non-temporal loads and stores, so nothing of the previous launch is found in the
-    # memory-side cache.  This is the figure the roofline fraction is quoted on.
+    # memory-side cache (one-wavefront workgroups with one vector per thread stream best that way).
+    # This is the figure the roofline fraction is quoted on.
     streaming = None
     if not tuned:
-        dev.set_tuning(0, 2, 0, 3, 1)
+        dev.set_tuning(64, 1, 0, 3 | 64, 1)
         skernel = dev.compile(capi.KIND_APPLY, "f32", src, ("x",))
         dev.capture_begin()
         capi.check(lib.custos_hip_apply_fn(dev.handle, skernel, xb.ptr, out.ptr, n), dev.handle)
@@ -258,7 +260,8 @@ def bench_c2(dev, args, stack):
         streaming = {"ms_per_step": round(sms, 5), "GBps": round(gbs_of(sms), 2),
                      "per_step": per_step_stats(dev, sgraph.launch, args.steps),
                      "kernel": dev.kernel_name(skernel),
-                     "shape": "tiles first to last, non-temporal loads and stores, 2 vectors per thread"}
+                     "shape": "tiles first to last, non-temporal loads, non-temporal stores written through at once, "
+                              "one-wavefront workgroups, 1 vector per thread"}
         check_chain(out.slice(0, 1 << 20).read(), cpu_oracle_chain(x[: 1 << 20]), "the streaming-pinned fused chain")
         sgraph.destroy()
 

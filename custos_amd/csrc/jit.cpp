@@ -286,7 +286,7 @@ ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kerne
     r.alternate = direction == 2 || (direction == 0 && shape.alternate);
     r.unroll = k->spec.auto_unroll ? shape.unroll : k->spec.tuning.unroll;
     r.nontemporal = dev->tuning.nontemporal >= 0
-                        ? dev->tuning.nontemporal & 3
+                        ? dev->tuning.nontemporal & (3 | kStoresWriteThrough)
                         : shape.nontemporal | ((shape.nontemporal & 1) ? (keep_loads & 15) << 2 : 0);
     return r;
 }

@@ -15,7 +15,7 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
     }
     if (unroll > 0) t.unroll = std::min(16, unroll);
     t.blocks_per_cu = blocks_per_cu > 0 ? std::min(64, blocks_per_cu) : 0;
-    if (nontemporal != 0) t.nontemporal = nontemporal < 0 ? 0 : (nontemporal & 3);
+    if (nontemporal != 0) t.nontemporal = nontemporal < 0 ? 0 : (nontemporal & (3 | kStoresWriteThrough));
     if (direction == 1 || direction == 2) t.direction = direction;
     return t;
 }
@@ -65,7 +65,8 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // launch.cpp hot_operands).
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint) {
     constexpr unsigned long long MiB = 1ull << 20;
-    constexpr int kLoads = 1, kBoth = 3;  // non-temporal loads only / loads and stores
+    // non-temporal loads with temporal stores that are written through at once / both non-temporal
+    constexpr int kLoads = 1 | kStoresWriteThrough, kBoth = 3;
     if (footprint_bytes < 64 * MiB) return {2, 0, false};
     if (hint == CacheHint::Resident) return {2, 0, false};
     if (hint == CacheHint::Streams) return {2, kLoads, footprint_bytes > 256 * MiB};
@@ -342,7 +343,6 @@ struct KernelText {
             s += "    const bool nt" + id + " = (mode & 2) && !(mode & " + std::to_string(8 << i) + ");\n";
         }
         s += k.kind == Kind::UnaryGrad ? "    const custos_rsrc rso = rs1;\n" : "    const custos_rsrc rso = custos_make_rsrc(vout + first, bound);\n";
-        s += "    const bool nts = mode & 4;\n";
         s += "    const unsigned int lane = threadIdx.x * 16u;\n";
         for (int i = 0; i < n_ops; i++) s += "    vec_t a" + std::to_string(i) + "[" + U + "];\n";
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
@@ -354,7 +354,7 @@ struct KernelText {
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
         s += "        vec_t r;\n#pragma unroll\n        for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
              list("a", "[u][k]") + " CUSTOS_KC_ARG);\n";
-        s += "        custos_st(rso, lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), r, nts);\n    }\n";
+        s += "        custos_st(rso, lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), r, mode);\n    }\n";
         s += "}\n";
         return s;
     }
@@ -490,7 +490,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds the vectors per thread as requested: 0 = chosen per launch)
     int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, 14 /* template version */};
+                       k.tuning.blocks_per_cu, 15 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -532,9 +532,15 @@ static __device__ __forceinline__ vec_t custos_ld(const custos_rsrc rs, const un
     else v = __builtin_amdgcn_raw_buffer_load_b128(rs, offset, 0, 0);
     return __builtin_bit_cast(vec_t, v);
 }
-static __device__ __forceinline__ void custos_st(const custos_rsrc rs, const unsigned int offset, const vec_t v, const bool nt) {
-    if (nt) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(custos_u4, v), rs, offset, 0, 2);
-    else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(custos_u4, v), rs, offset, 0, 0);
+static __device__ __forceinline__ void custos_st(const custos_rsrc rs, const unsigned int offset, const vec_t v, const u64 mode) {
+    const custos_u4 bits = __builtin_bit_cast(custos_u4, v);
+    if (mode & 4) {
+        if (mode & 128) __builtin_amdgcn_raw_buffer_store_b128(bits, rs, offset, 0, 18);
+        else __builtin_amdgcn_raw_buffer_store_b128(bits, rs, offset, 0, 2);
+    } else {
+        if (mode & 128) __builtin_amdgcn_raw_buffer_store_b128(bits, rs, offset, 0, 16);
+        else __builtin_amdgcn_raw_buffer_store_b128(bits, rs, offset, 0, 0);
+    }
 }
 )";
     s += expr_fn(k, body);

@@ -58,10 +58,14 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
 //   bit 0      the tiles are walked from the last to the first
 //   bit 1, 2   non-temporal loads, non-temporal stores
 //   bits 3..6  operand 0..3 is loaded temporally although bit 1 is set
+//   bit 7      stores are written through to device scope at once instead of lingering in an L2
 //   bits 8..11 vectors per thread (only read by kernels whose unroll factor was left open)
+// `nontemporal` as in Tuning: bit 0 loads, bit 1 stores, bits 2..5 the operands kept temporal,
+// kStoresWriteThrough the write-through stores.
+constexpr int kStoresWriteThrough = 64;
 inline uint64_t launch_mode(int unroll, int nontemporal, bool rev) {
     return (rev ? 1u : 0u) | static_cast<uint64_t>(nontemporal & 3) << 1 | static_cast<uint64_t>((nontemporal >> 2) & 15) << 3 |
-           static_cast<uint64_t>(unroll & 15) << 8;
+           static_cast<uint64_t>((nontemporal & kStoresWriteThrough) ? 1 : 0) << 7 | static_cast<uint64_t>(unroll & 15) << 8;
 }
 
 // Fills unset (zero) fields with the defaults and clamps to legal values

@@ -111,14 +111,17 @@ typedef struct custos_hip_device_info {
 } custos_hip_device_info;
 
 /* Launch shape knobs of the generated kernels.  Zero fields keep the default.
- * They are part of the kernel cache key. */
+ * `block_threads`, `unroll` and `blocks_per_cu` are compiled into a kernel (part of its cache
+ * key: they apply to kernels compiled while they are set); `nontemporal` and `direction` are
+ * arguments of every launch and apply to launches issued, and graphs built, while they are set. */
 typedef struct custos_hip_tuning {
     int32_t block_threads;   /* threads per workgroup (multiple of 64), default 128 */
-    int32_t unroll;          /* 16-byte vectors per thread per tile; 0 (default): 2 for kernels
-                                with one input operand, 1 for kernels that read several */
+    int32_t unroll;          /* 16-byte vectors per thread per tile; 0 (default): the kernel holds the
+                                code for 2 and for 1, chosen per launch from the bytes it touches */
     int32_t blocks_per_cu;   /* > 0: persistent grid of CUs*blocks_per_cu workgroups that
                                 stride over the tiles; <= 0 (default): one tile per workgroup */
-    int32_t nontemporal;     /* bit 0: non-temporal loads, bit 1: non-temporal stores; -1 = off;
+    int32_t nontemporal;     /* bit 0: non-temporal loads, bit 1: non-temporal stores, 64: stores are
+                                written through to device scope at once; -1 = all off;
                                 0 (default): chosen per launch from the bytes it touches */
     int32_t direction;       /* 1: tiles from the first to the last; 2: every launch walks them the
                                 other way round than the launch before, so that it starts on what
@@ -230,10 +233,10 @@ const char *custos_hip_kernel_source(const custos_hip_kernel *kernel);
 const char *custos_hip_kernel_name(const custos_hip_kernel *kernel);
 uint64_t custos_hip_kernel_hash(const custos_hip_kernel *kernel);
 int32_t custos_hip_kernel_arity(const custos_hip_kernel *kernel);
-/* The kernel a launch of `kernel` over `n` elements really runs: `kernel` itself, or the
- * variant of the same expression whose launch shape (vectors per thread, cache policy)
- * suits the bytes such a launch touches, compiled on first use.  Its name is what a
- * profiler shows.  Only knobs that custos_hip_set_tuning left at 0 vary. */
+/* The kernel a launch of `kernel` over `n` elements runs: always `kernel` itself.  (One kernel
+ * per expression serves every launch size: vectors per thread, cache policy and direction are
+ * arguments of the launch, so nothing is compiled after custos_hip_expr_compile has returned --
+ * the reference compiles once per text too, src/devices/cuda/kernel_cache.rs:39-61.) */
 int32_t custos_hip_kernel_launched_as(custos_hip_device *dev, custos_hip_kernel *kernel, size_t n,
                                       custos_hip_kernel **variant);
 /* How literal values reach a kernel (see custos_hip_expr_compile). */

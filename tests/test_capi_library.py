@@ -132,10 +132,11 @@ def test_launch_shape_by_bytes_touched():
     assert shape(128 * MiB, 2) == (2, 0, False) and shape(256 * MiB, 2) == (2, 0, False)
     assert shape(257 * MiB, 2) == (2, 3, True)
     assert shape(512 * MiB, 2) == (2, 3, True)             # config 3 forward
-    assert shape(768 * MiB, 3) == (1, 1, True)             # config 3 backward
-    assert shape(512 * MiB, 3) == (1, 1, True) and shape(511 * MiB, 3) == (2, 3, True)
-    assert shape(1024 * MiB, 2) == (2, 1, True)            # config 4
-    assert shape(2048 * MiB, 2) == (2, 1, True)            # config 2
+    loads = 1 | 64                                         # non-temporal loads, stores written through at once
+    assert shape(768 * MiB, 3) == (1, loads, True)         # config 3 backward
+    assert shape(512 * MiB, 3) == (1, loads, True) and shape(511 * MiB, 3) == (2, 3, True)
+    assert shape(1024 * MiB, 2) == (2, loads, True)        # config 4
+    assert shape(2048 * MiB, 2) == (2, loads, True)        # config 2
     with pytest.raises(capi.CustosHipError):
         shape(1, 0)
 
