@@ -303,6 +303,7 @@ def bench_c2(dev, args, stack):
             "elements": n,
             "algorithmic_bytes_per_element": 8,
         },
+        "kernel": dev.kernel_name(kernel),
         "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "elements_per_s": round(n / (per_launch_ms * 1e-3), 1),
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
@@ -403,14 +404,15 @@ def bench_others(dev, args, stack_c5):
     out["c1"]["kernel"] = dev.kernel_name(k)
     # the same launch recorded 64 times into one graph (every launch writes the same output, so
     # the graph is a chain of 64 nodes): the device's time per launch, without the host's
-    dev.capture_begin()
-    for i in range(64):
-        capi.check(lib.custos_hip_apply_fn(h, k, xb.ptr, ob.ptr, n), h)
-    g = dev.capture_end()
-    gms, _ = time_floor(dev, g.launch, launches_per_step=g.kernel_nodes)
-    out["c1"]["in_a_graph"] = {"us_per_launch": round(gms / g.kernel_nodes * 1e3, 3), "kernel_nodes": g.kernel_nodes,
-                               "what": "64 such launches into the same output recorded as one hipGraph (a chain of 64 nodes)"}
-    g.destroy()
+    if args.hipgraph:
+        dev.capture_begin()
+        for i in range(64):
+            capi.check(lib.custos_hip_apply_fn(h, k, xb.ptr, ob.ptr, n), h)
+        g = dev.capture_end()
+        gms, _ = time_floor(dev, g.launch, launches_per_step=g.kernel_nodes)
+        out["c1"]["in_a_graph"] = {"us_per_launch": round(gms / g.kernel_nodes * 1e3, 3), "kernel_nodes": g.kernel_nodes,
+                                   "what": "64 such launches into the same output recorded as one hipGraph (a chain of 64 nodes)"}
+        g.destroy()
 
     # c3: unary_ew tanh forward + backward, f32 N = 2^26
     n = 1 << 26
@@ -508,11 +510,12 @@ def bench_others(dev, args, stack_c5):
     e["kernels"] = [dev.kernel_name(q) + "_batched" for q in (kmul, kadd, kun)]
     graph.destroy()
     # the same recording instantiated as a hipGraph and replayed with one hipGraphLaunch
-    dev.set_graph_direct_replay(0)
-    graph, _ = record_c5()
-    e["as_hipgraph"] = timed_c5(graph, "one hipGraphLaunch of the instantiated 3-node graph")
-    graph.destroy()
-    dev.set_graph_direct_replay(default_direct)
+    if args.hipgraph:
+        dev.set_graph_direct_replay(0)
+        graph, _ = record_c5()
+        e["as_hipgraph"] = timed_c5(graph, "one hipGraphLaunch of the instantiated 3-node graph")
+        graph.destroy()
+        dev.set_graph_direct_replay(default_direct)
 
     # the same work after element-wise fusing (the text `Lazy::elementwise_fusing` of the host stack
     # emits for these operations): one three-operand kernel per buffer, 16 B/element, one node
@@ -547,6 +550,9 @@ def main():
                     help="1: tiles first to last; 2: every launch the other way round; 0: library default")
     ap.add_argument("--no-others", dest="others", action="store_false",
                     help="skip the other BASELINE configurations (c1, c3, c4, c5)")
+    ap.add_argument("--no-hipgraph", dest="hipgraph", action="store_false",
+                    help="skip the two comparisons that launch an instantiated hipGraph (c1 in a 64-node graph, c5 as a "
+                         "3-node graph): for runs under rocprofv3, whose kernel tracing ended the process in hipGraphLaunch")
     ap.add_argument("--no-module-stack", dest="module_stack", action="store_false",
                     help="skip the child processes that time the C++ module stack")
     args = ap.parse_args()

@@ -722,3 +722,53 @@ def test_unmerged_graph_nodes_take_literals_by_value(hip):
     finally:
         hip.set_graph_batching(True)
         hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
+
+
+def test_waits_follow_the_work(hip):
+    """`custos_hip_sync` after a graph launch polls, and for work it has seen take milliseconds
+    sleeps up to shortly before the predicted end: a launch + wait of a 5 ms graph must not cost
+    more wall time than the graph takes on the device (plus slack), run after run, and a short
+    graph right after it must not inherit the long graph's prediction."""
+    import time
+    n = 1 << 26
+    x = hip.alloc(n)
+    hip.write(x.slice(0, 1 << 12), synth.uniform_f32(3, 1 << 12, -1, 1))
+    bufs = [hip.alloc(n) for _ in range(2)]
+    k = hip.compile(capi.KIND_APPLY, "f32", "((x * 1.0001) + 0.25)", ("x",))
+    hip.set_graph_direct_replay(0)
+    try:
+        hip.capture_begin()
+        src = x
+        for i in range(48):                       # a chain: each launch reads what the one before wrote
+            dst = bufs[i % 2]
+            capi.check(hip.lib.custos_hip_apply_fn(hip.handle, k, src.ptr, dst.ptr, n), hip.handle)
+            src = dst
+        long_graph = hip.capture_end()
+        hip.capture_begin()
+        capi.check(hip.lib.custos_hip_apply_fn(hip.handle, k, x.ptr, bufs[0].ptr, 1 << 12), hip.handle)
+        short_graph = hip.capture_end()
+    finally:
+        hip.set_graph_direct_replay(4)
+    long_graph.launch()
+    hip.sync()
+    hip.timer_begin()
+    long_graph.launch()
+    device_ms = hip.timer_end()
+    assert device_ms > 2.0                    # long enough for the wait to sleep through most of it
+    walls = []
+    for _ in range(6):
+        t0 = time.perf_counter()
+        long_graph.launch()
+        hip.sync()
+        walls.append((time.perf_counter() - t0) * 1e3)
+    assert max(walls[1:]) < 1.5 * device_ms + 0.3, (walls, device_ms)
+    t0 = time.perf_counter()
+    short_graph.launch()
+    hip.sync()
+    assert (time.perf_counter() - t0) * 1e3 < 0.5 * device_ms + 0.3    # not slept on the long graph's account
+    want = x.slice(0, 1 << 12).read()
+    for _ in range(1):
+        want = want * np.float32(1.0001) + np.float32(0.25)
+    assert_bits_equal(bufs[0].slice(0, 1 << 12).read(), want)
+    long_graph.destroy()
+    short_graph.destroy()
