@@ -271,17 +271,12 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
             unsigned long long footprint = 0;
             for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
             CacheHint hint = CacheHint::Unknown;
-            int keep_loads = 0;
             if (footprint >= kHintFromBytes) {
                 hint = hint_for(nodes, p, *history, later_reads);
                 dev->hinted[static_cast<int>(hint)]++;
-                std::vector<const std::vector<Access>*> member_accesses;
-                for (size_t i : p.members) member_accesses.push_back(&nodes[i].acc);
-                keep_loads = hot_operands(*history, member_accesses, hint);
-                dev->kept_loads += keep_loads != 0;
             }
             p.kern = first.k;
-            p.shape = resolve_shape(dev, first.k, footprint, hint, keep_loads);
+            p.shape = resolve_shape(dev, first.k, footprint, hint);
         }
         if (p.members.size() > 1) append_tables(nodes, &p, host_table);
     }

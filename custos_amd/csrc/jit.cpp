@@ -278,7 +278,7 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 }
 
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
-                            CacheHint hint, int keep_loads) {
+                            CacheHint hint) {
     const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;
     const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint);
     ResolvedShape r;
@@ -287,7 +287,7 @@ ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kerne
     r.unroll = k->spec.auto_unroll ? shape.unroll : k->spec.tuning.unroll;
     r.nontemporal = dev->tuning.nontemporal >= 0
                         ? dev->tuning.nontemporal & (3 | kStoresWriteThrough)
-                        : shape.nontemporal | ((shape.nontemporal & 1) ? (keep_loads & 15) << 2 : 0);
+                        : shape.nontemporal;
     return r;
 }
 

@@ -60,9 +60,6 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // 6507, u2L 6271, u2N 5802); beyond, L with two vectors per thread, whatever the
 // direction (192 MiB: u2L 6956, u2T 6229, u2N 6153; 256 MiB: 7081 / 5653 / 6340;
 // 512 MiB: 7142 / 5993 / 6467; 768 MiB: 6970 / 6075 / 6475).
-// An operand that every kernel of a streaming chain reads again (and nobody
-// writes) keeps temporal loads while the rest streams (bits 2.. of the policy,
-// launch.cpp hot_operands).
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint) {
     constexpr unsigned long long MiB = 1ull << 20;
     // non-temporal loads with temporal stores that are written through at once / both non-temporal
@@ -70,11 +67,9 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
     if (footprint_bytes < 64 * MiB) return {2, 0, false};
     if (hint == CacheHint::Resident) return {2, 0, false};
     if (hint == CacheHint::Streams) return {2, kLoads, footprint_bytes > 256 * MiB};
-    if (footprint_bytes < 128 * MiB) return {2, kBoth, false};
-    if (footprint_bytes <= 256 * MiB) return {2, hint == CacheHint::Crowded ? kBoth : 0, false};
-    const bool one_vector = footprint_bytes >= 768 * MiB || (n_operands >= 3 && footprint_bytes >= 512 * MiB);
-    if (one_vector) return {n_operands < 3 ? 2 : 1, kLoads, true};
-    return {2, kBoth, true};
+    if (footprint_bytes <= 256 * MiB) return {2, kLoads, false};
+    if (n_operands < 3 && footprint_bytes < 768 * MiB) return {2, kBoth, true};
+    return {2, kLoads, true};
 }
 
 std::vector<std::string> hiprtc_options(const std::string& arch) {
@@ -336,11 +331,9 @@ struct KernelText {
             const std::string id = std::to_string(i);
             if (k.kind == Kind::UnaryGrad && i == 1) {
                 s += "    const custos_rsrc rs1 = custos_make_rsrc(vout + first, bound);\n";
-                s += "    const bool nt1 = (mode & 2) && !(mode & 16);\n";
                 continue;
             }
             s += "    const custos_rsrc rs" + id + " = custos_make_rsrc(vin" + id + " + first, bound);\n";
-            s += "    const bool nt" + id + " = (mode & 2) && !(mode & " + std::to_string(8 << i) + ");\n";
         }
         s += k.kind == Kind::UnaryGrad ? "    const custos_rsrc rso = rs1;\n" : "    const custos_rsrc rso = custos_make_rsrc(vout + first, bound);\n";
         s += "    const unsigned int lane = threadIdx.x * 16u;\n";
@@ -348,7 +341,7 @@ struct KernelText {
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
         for (int i = 0; i < n_ops; i++) {
             const std::string id = std::to_string(i);
-            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), nt" + id + ");\n";
+            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), mode & 2);\n";
         }
         s += "    }\n";
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
@@ -490,7 +483,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds the vectors per thread as requested: 0 = chosen per launch)
     int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, 15 /* template version */};
+                       k.tuning.blocks_per_cu, 16 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {

@@ -27,9 +27,8 @@ struct Tuning {
     int block_threads = 128;
     int unroll = 0;         // 16-byte vectors per thread and tile; 0: chosen per launch (2 or 1)
     int blocks_per_cu = 0;  // <= 0: one tile per workgroup
-    int nontemporal = -1;   // bit 0 loads, bit 1 stores; -1: chosen per launch.  Bits 2..5 (set by the
-                            // library only): operand 0..3 is loaded temporally although bit 0 is set.
-                            // Read from the device's tuning when a launch is issued or a graph built.
+    int nontemporal = -1;   // bit 0 loads, bit 1 stores, 64 stores written through at once; -1: chosen per
+                            // launch.  Read from the device's tuning when a launch is issued or a graph built.
     int direction = 0;      // 1: tiles first to last; 2: every launch the other way round; 0: chosen per launch
 };
 
@@ -57,14 +56,12 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
 // of it is compiled in, so one kernel per expression serves every launch size.
 //   bit 0      the tiles are walked from the last to the first
 //   bit 1, 2   non-temporal loads, non-temporal stores
-//   bits 3..6  operand 0..3 is loaded temporally although bit 1 is set
 //   bit 7      stores are written through to device scope at once instead of lingering in an L2
 //   bits 8..11 vectors per thread (only read by kernels whose unroll factor was left open)
-// `nontemporal` as in Tuning: bit 0 loads, bit 1 stores, bits 2..5 the operands kept temporal,
-// kStoresWriteThrough the write-through stores.
+// `nontemporal` as in Tuning: bit 0 loads, bit 1 stores, kStoresWriteThrough the write-through stores.
 constexpr int kStoresWriteThrough = 64;
 inline uint64_t launch_mode(int unroll, int nontemporal, bool rev) {
-    return (rev ? 1u : 0u) | static_cast<uint64_t>(nontemporal & 3) << 1 | static_cast<uint64_t>((nontemporal >> 2) & 15) << 3 |
+    return (rev ? 1u : 0u) | static_cast<uint64_t>(nontemporal & 3) << 1 |
            static_cast<uint64_t>((nontemporal & kStoresWriteThrough) ? 1 : 0) << 7 | static_cast<uint64_t>(unroll & 15) << 8;
 }
 

@@ -58,20 +58,6 @@ custos_hip::CacheHint RecentTraffic::classify(const std::vector<Access>& reads, 
     return fits ? custos_hip::CacheHint::Resident : custos_hip::CacheHint::Streams;
 }
 
-bool RecentTraffic::read_only_by(const Access& range, int times) const {
-    int readers = 0;
-    for (const std::vector<Access>& launch : launches_) {
-        bool reads = false;
-        for (const Access& a : launch) {
-            if (!(a.begin < range.end && range.begin < a.end)) continue;
-            if (a.write) return false;
-            reads = true;
-        }
-        readers += reads;
-    }
-    return readers >= times;
-}
-
 void RecentTraffic::record(const std::vector<Access>& all) {
     if (launches_.size() == kTrafficDepth) launches_.erase(launches_.begin());
     // written and read ranges are merged separately, so that the writer flag stays exact
@@ -135,32 +121,6 @@ unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* 
     return static_cast<unsigned int>(std::min(g, 1ull << 22));
 }
 
-// Operands (bit i = i-th pointer parameter) that a streaming launch should still load
-// temporally: the launches before it only read them, at least two of them did, and together
-// they take no more than three quarters of the cache (192 MiB kept: 6.73 TB/s against 6.46;
-// nothing is gained beyond).  `members`: the access lists (in parameter order)
-// of the launches merged into this one; an operand qualifies if it does for every member.
-int hot_operands(const RecentTraffic& recent, const std::vector<const std::vector<Access>*>& members, CacheHint hint) {
-    if ((hint != CacheHint::Streams && hint != CacheHint::Crowded) || members.empty()) return 0;
-    int mask = 0;
-    unsigned long long bytes = 0;
-    for (size_t i = 0; i < members[0]->size() && i < 4; i++) {
-        bool hot = true;
-        unsigned long long operand_bytes = 0;
-        for (const std::vector<Access>* all : members) {
-            if (!hot || i >= all->size() || (*all)[i].write || !recent.read_only_by((*all)[i], 2)) {
-                hot = false;
-                break;
-            }
-            operand_bytes += (*all)[i].end - (*all)[i].begin;
-        }
-        if (!hot) continue;
-        mask |= 1 << static_cast<int>(i);
-        bytes += operand_bytes;
-    }
-    return bytes <= kCacheWorkingSet * 3 / 4 ? mask : 0;
-}
-
 // Launches the kernel over one set of operands, or records the launch while
 // the device is recording.  `ops` are the operand addresses in the order of the
 // kernel's pointer parameters.
@@ -190,7 +150,6 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
     const unsigned long long footprint = static_cast<unsigned long long>(ops.size()) * bytes;
     CacheHint hint = CacheHint::Unknown;
-    int keep_loads = 0;
     if (footprint >= kTrafficFromBytes) {
         std::vector<Access> all, reads;
         for (const Range& r : ops) {
@@ -201,12 +160,10 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
         if (footprint >= kHintFromBytes) {
             hint = dev->recent.classify(reads, all);
             dev->hinted[static_cast<int>(hint)]++;
-            keep_loads = hot_operands(dev->recent, {&all}, hint);
-            dev->kept_loads += keep_loads != 0;
         }
         dev->recent.record(all);
     }
-    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, keep_loads);
+    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint);
     const unsigned int grid = launch_grid(dev, k, n, n_vec, shape.unroll);
     unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, shape.alternate && (dev->launch_parity ^= 1));
     uint64_t ptrs[8];
@@ -251,13 +208,11 @@ int32_t custos_hip_apply_fn_n(custos_hip_device* dev, custos_hip_kernel* kernel,
     return launch_or_record(dev, kernel, ops, n);
 }
 
-int32_t custos_hip_launch_hint_stats(custos_hip_device* dev, uint64_t* unrelated, uint64_t* resident, uint64_t* streaming,
-                                     uint64_t* kept_operand) {
+int32_t custos_hip_launch_hint_stats(custos_hip_device* dev, uint64_t* unrelated, uint64_t* resident, uint64_t* streaming) {
     REQUIRE_DEV(dev);
     if (unrelated) *unrelated = dev->hinted[static_cast<int>(CacheHint::Unknown)] + dev->hinted[static_cast<int>(CacheHint::Crowded)];
     if (resident) *resident = dev->hinted[static_cast<int>(CacheHint::Resident)];
     if (streaming) *streaming = dev->hinted[static_cast<int>(CacheHint::Streams)];
-    if (kept_operand) *kept_operand = dev->kept_loads;
     return CUSTOS_HIP_OK;
 }
 

@@ -106,8 +106,6 @@ class RecentTraffic {
     // that a launch soon after it reads what it writes.
     custos_hip::CacheHint classify(const std::vector<Access>& reads, const std::vector<Access>& all,
                                    bool feeds_later = false) const;
-    // Whether the recorded launches only ever read `range`, and at least `times` of them do.
-    bool read_only_by(const Access& range, int times) const;
 
    private:
     std::vector<std::vector<Access>> launches_;  // oldest first, at most 8, each merged and sorted
@@ -127,8 +125,7 @@ struct custos_hip_device {
     // per shared-form key: how many distinct texts of that structure were compiled or looked up
     std::unordered_map<uint64_t, uint32_t> value_sets_seen;
     RecentTraffic recent;            // of the launches issued directly (not recorded)
-    uint64_t hinted[4] = {0, 0, 0, 0};
-    uint64_t kept_loads = 0;         // of those, launches that keep an operand's loads temporal while streaming  // launches and graph nodes of at least kHintFromBytes by CacheHint
+    uint64_t hinted[4] = {0, 0, 0, 0};  // launches and graph nodes of at least kHintFromBytes by CacheHint
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     bool graph_verify = false;       // built graphs are checked by brute force against the recorded conflicts
     int32_t graph_edges = CUSTOS_HIP_GRAPH_EDGES_CHAIN;  // how built graphs order their nodes
@@ -224,25 +221,20 @@ int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k);
 // The kernel of the expression `x` over `dtype` elements (compiled once per device).
 int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel** out);
 // How a launch of `k` that touches `footprint_bytes` runs: vectors per thread and cache policy
-// from the bytes touched and from what is known about the launches around it (`hint`,
-// `keep_loads`: bit i = operand i is read by those launches again and again, and is still
-// loaded temporally where the launch streams), unless the caller pinned them (the vectors per
-// thread when the kernel was compiled, cache policy and direction in the device's tuning now).
-// `alternate`: the launch walks its tiles against the direction of the previous such launch.
+// from the bytes touched and from what is known about the launches around it (`hint`), unless
+// the caller pinned them (the vectors per thread when the kernel was compiled, cache policy and
+// direction in the device's tuning now).  `alternate`: the launch walks its tiles against the
+// direction of the previous such launch.
 struct ResolvedShape {
     int unroll = 2;
     int nontemporal = 0;
     bool alternate = false;
 };
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
-                            CacheHint hint = CacheHint::Unknown, int keep_loads = 0);
+                            CacheHint hint = CacheHint::Unknown);
 
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
-// The operands (bit i = i-th pointer parameter) that a streaming launch should keep loading
-// temporally, given what the launches before did with them; `members`: the access lists of the
-// launches merged into this one, each in parameter order.
-int hot_operands(const RecentTraffic& recent, const std::vector<const std::vector<Access>*>& members, CacheHint hint);
 // Workgroups of a single launch of `k` over n_vec vectors and n elements with `unroll` vectors per thread.
 unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
                          unsigned long long n_vec, int unroll);

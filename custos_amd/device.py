@@ -356,11 +356,11 @@ class HIP:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 
     def launch_hint_stats(self):
-        """(not part of a chain, chain that stays in the memory-side cache, chain that streams, streaming
-        with one operand kept cached) counts of the launches and graph nodes of 64 MiB and more so far."""
-        a, b, c, d = C.c_uint64(0), C.c_uint64(0), C.c_uint64(0), C.c_uint64(0)
-        self._check(self.lib.custos_hip_launch_hint_stats(self.handle, C.byref(a), C.byref(b), C.byref(c), C.byref(d)))
-        return a.value, b.value, c.value, d.value
+        """(not part of a chain, chain that stays in the memory-side cache, chain that streams) counts of
+        the launches and graph nodes of 64 MiB and more so far."""
+        a, b, c = C.c_uint64(0), C.c_uint64(0), C.c_uint64(0)
+        self._check(self.lib.custos_hip_launch_hint_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
 
     def set_literal_policy(self, policy: int) -> None:
         """How literal values reach kernels: capi.LITERALS_ADAPTIVE (default), _IN_CODE, _AS_PARAMETERS."""

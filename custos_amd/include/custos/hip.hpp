@@ -251,10 +251,10 @@ class HIP : public Device<HIP<Mods>, Mods> {
         return {compiles, hits};
     }
     // Launches and graph nodes of 64 MiB and more so far: {not part of a chain, chain that stays in the
-    // memory-side cache, chain that streams, streaming with one operand kept cached}.
-    std::array<uint64_t, 4> launch_hint_stats() const {
-        std::array<uint64_t, 4> s{};
-        custos_hip_launch_hint_stats(dev_, &s[0], &s[1], &s[2], &s[3]);
+    // memory-side cache, chain that streams}.
+    std::array<uint64_t, 3> launch_hint_stats() const {
+        std::array<uint64_t, 3> s{};
+        custos_hip_launch_hint_stats(dev_, &s[0], &s[1], &s[2]);
         return s;
     }
     // Longest recorded chain that is replayed as plain launches instead of a graph launch.

@@ -64,7 +64,7 @@ extern "C" {
                                          variant: *mut *mut HipKernel) -> i32;
     pub fn custos_hip_set_literal_policy(dev: *mut HipDeviceHandle, policy: i32) -> i32;
     pub fn custos_hip_launch_hint_stats(dev: *mut HipDeviceHandle, unrelated: *mut u64, resident: *mut u64,
-                                        streaming: *mut u64, kept_operand: *mut u64) -> i32;
+                                        streaming: *mut u64) -> i32;
     pub fn custos_hip_cache_stats(dev: *mut HipDeviceHandle, compiles: *mut u64, hits: *mut u64) -> i32;
     pub fn custos_hip_cache_disk_hits(dev: *mut HipDeviceHandle, disk_hits: *mut u64) -> i32;
     pub fn custos_hip_source_compile(dev: *mut HipDeviceHandle, src: *const c_char, fn_name: *const c_char,

@@ -295,13 +295,10 @@ int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const cha
  * then follows the bytes the launch touches, custos_hip_preferred_shape); part of a chain
  * -- it reads what one of the last eight launches wrote, or in a graph one of the next
  * levels reads what it writes -- whose working set stays in the 256 MiB memory-side cache
- * (temporal accesses, two vectors per thread); part of a chain whose working set does not
- * (non-temporal accesses, one vector per thread).  `*kept_operand`: how many of the streaming
- * ones still load one of their operands temporally, because the launches before them read
- * that operand again and again and never wrote it (a weight that every kernel of a chain
- * multiplies by stays cached while the activations stream). */
+ * (temporal accesses); part of a chain whose working set does not (loads past the caches,
+ * stores written through). */
 int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated, uint64_t *resident,
-                                     uint64_t *streaming, uint64_t *kept_operand);
+                                     uint64_t *streaming);
 /* Host-only: the launch shape the library picks for a launch that touches `footprint_bytes`
  * (all operands together) through `n_operands` pointers, for the knobs left at 0 in
  * custos_hip_tuning: vectors per thread, the `nontemporal` bits, and whether the launch

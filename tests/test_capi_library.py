@@ -120,21 +120,21 @@ def test_product_never_imports_the_oracle():
 
 
 def test_launch_shape_by_bytes_touched():
-    """The shape for the knobs a caller leaves open: temporal accesses for what fits the caches,
-    non-temporal streaming beyond; the largest launches load non-temporally, store temporally and
-    alternate their direction (what they wrote last is what the next launch starts on)."""
+    """The shape for the knobs a caller leaves open: temporal accesses below the L2 capacity; above,
+    loads past the caches and temporal stores written through at once (what a launch wrote last is what
+    the next launch over the same buffers starts on: the largest launches alternate their direction);
+    a two-pointer launch of 256 to 768 MiB streams both ways."""
     MiB = 1 << 20
     shape = capi.preferred_shape
+    loads = 1 | 64                                         # non-temporal loads, stores written through at once
     assert shape(8 * MiB, 2) == (2, 0, False)              # config 1: 2^20 f32 in, out
     assert shape(48 * MiB, 3) == (2, 0, False)             # config 5, one recorded level merged
-    assert shape(64 * MiB, 4) == (2, 3, False)             # config 5 after element-wise fusing
-    assert shape(96 * MiB, 3) == (2, 3, False)             # just above the L2 capacity
-    assert shape(128 * MiB, 2) == (2, 0, False) and shape(256 * MiB, 2) == (2, 0, False)
+    assert shape(64 * MiB, 4) == (2, loads, False)         # config 5 after element-wise fusing
+    assert shape(128 * MiB, 2) == (2, loads, False) and shape(256 * MiB, 2) == (2, loads, False)
     assert shape(257 * MiB, 2) == (2, 3, True)
     assert shape(512 * MiB, 2) == (2, 3, True)             # config 3 forward
-    loads = 1 | 64                                         # non-temporal loads, stores written through at once
-    assert shape(768 * MiB, 3) == (1, loads, True)         # config 3 backward
-    assert shape(512 * MiB, 3) == (1, loads, True) and shape(511 * MiB, 3) == (2, 3, True)
+    assert shape(768 * MiB, 3) == (2, loads, True)         # config 3 backward
+    assert shape(384 * MiB, 3) == (2, loads, True) and shape(767 * MiB, 2) == (2, 3, True)
     assert shape(1024 * MiB, 2) == (2, loads, True)        # config 4
     assert shape(2048 * MiB, 2) == (2, loads, True)        # config 2
     with pytest.raises(capi.CustosHipError):

@@ -36,6 +36,23 @@ def test_reference_strings():
     assert to_val(2.0).to_cl_source("f64") == "2.0"
 
 
+def test_operand_order_of_every_binary_node(oracle):
+    """`lhs.op(rhs)` prints the receiver first, as every `ToCLSource` of the reference does
+    (src/two_way_ops/ops.rs:28-310: "({} * {})", "({} + {})", "({} - {})", "({} / {})", "pow({}, {})",
+    "min({}, {})", "max({}, {})"; ops/cmps.rs:17-130: "({} >= {})", "({} <= {})", "({} == {})"), and the
+    oracle's postfix program takes its operands in that order too: the receiver is the left operand
+    of the scalar evaluation (asymmetric inputs tell the two orders apart)."""
+    a, b = to_marker("a", "b")
+    formats = {"mul": "(a * b)", "add": "(a + b)", "sub": "(a - b)", "div": "(a / b)", "pow": "pow(a, b)", "min": "min(a, b)",
+               "max": "max(a, b)", "geq": "(a >= b)", "leq": "(a <= b)", "eq": "(a == b)"}
+    for op, text in formats.items():
+        assert getattr(a, op)(b).to_cl_source() == text, op
+        assert capi.expr_canonical(text, ["a", "b"]) == text
+    scalar = {"sub": 7.0 - 2.0, "div": 7.0 / 2.0, "pow": 49.0, "geq": 1.0, "leq": 0.0, "min": 2.0, "max": 7.0}
+    for op, want in scalar.items():
+        assert oracle.eval_scalar(lambda x, y, op=op: getattr(x, op)(y), 7.0, 2.0) == want, op
+
+
 def test_fused_source():
     # src/devices/fusing.rs:104-120
     ops = [lambda x: x.sin(), lambda x: x.neg(), lambda x: x.cos()]

@@ -980,7 +980,7 @@ def test_random_expression_trees_are_bit_exact(hip, oracle, dtype):
 def test_launch_shape_follows_the_launches_around_it(oracle):
     """A launch of 64 MiB and more that reads what one of the last launches wrote is part of a
     chain: temporal accesses while the chain's working set stays in the 256 MiB memory-side cache,
-    streaming with one vector per thread beyond that.  Results are the same either way."""
+    loads past the caches and stores written through beyond that.  Results are the same either way."""
     import custos_amd
     dev = custos_amd.HIP(0)
     try:
@@ -994,7 +994,7 @@ def test_launch_shape_follows_the_launches_around_it(oracle):
         dev.apply_fn(b, g, out=c)                     # consumer after producer, 96 MiB in all
         dev.apply_fn(c, f, out=b)
         s1 = dev.launch_hint_stats()
-        assert (s1[0] - base[0], s1[1] - base[1], s1[2] - base[2], s1[3] - base[3]) == (1, 2, 0, 0)
+        assert (s1[0] - base[0], s1[1] - base[1], s1[2] - base[2]) == (1, 2, 0)
         want = (np.abs(x * np.float32(1.5) - np.float32(0.25)) + np.float32(1.0)) * np.float32(1.5) - np.float32(0.25)
         assert_bits_equal(b.read(), want)
         # the same chain over arrays that do not fit: 3 x 128 MiB
@@ -1008,14 +1008,14 @@ def test_launch_shape_follows_the_launches_around_it(oracle):
         assert (s2[0] - s1[0], s2[1] - s1[1], s2[2] - s1[2]) == (1, 0, 2)
         wantb = (np.abs(xb * np.float32(1.5) - np.float32(0.25)) + np.float32(1.0)) * np.float32(1.5) - np.float32(0.25)
         assert_bits_equal(q.read(), wantb)
-        # a streaming chain whose kernels all read one more array: that operand stays cached
+        # a streaming chain whose kernels all read one more array
         w = dev.buffer(synth.uniform_f32(5, big, 0.5, 1.5))
         mul = lambda u, v: u.mul(v)
         for _ in range(2):
             dev.apply_fn2(q, w, mul, out=r)
             dev.apply_fn2(r, w, mul, out=q)
         s2b = dev.launch_hint_stats()
-        assert s2b[2] - s2[2] == 4 and s2b[3] - s2[3] == 2            # from the third launch on, w has been read twice
+        assert s2b[2] - s2[2] == 4
         wb = synth.uniform_f32(5, big, 0.5, 1.5)
         assert_bits_equal(q.read(), ((((wantb * wb) * wb) * wb) * wb))
         s2 = s2b
