@@ -22,53 +22,45 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 
 // Launch shape by the bytes a launch touches, measured on MI355X (8 x 4 MiB L2,
 // 256 MiB memory-side cache, HBM3E) over buffers of random data (buffers of
-// zeros run 5-10 % faster and hide differences).  Abbreviations: vectors per
-// thread (u1 / u2); cache policy T (all temporal), L (non-temporal loads,
-// temporal stores), S (temporal loads, non-temporal stores), N (both
-// non-temporal); tiles always first to last (f) or every launch the other way
-// round (a).  GB/s on the algorithmic bytes.
+// zeros run 5-10 % faster and hide differences).  Abbreviations: cache policy T
+// (all temporal), N (loads and stores non-temporal), W (non-temporal loads,
+// temporal stores written through to device scope at once); tiles always first
+// to last (f) or every launch the other way round (a).  Two vectors per thread
+// throughout (one was never more than 1 % ahead with W).  GB/s on the
+// algorithmic bytes.
 //
-// What fits the memory-side cache (up to 256 MiB touched): temporal accesses,
-// two vectors per thread; a chain whose working set fits runs 4 % faster with
-// them (a non-temporal store pushes what the next kernel reads out to HBM).  The
-// exception is the range just above the L2 capacity, 64 to 128 MiB, where N is
-// ahead for a launch that does not read what a launch just before it wrote
-// (1R+1W at 64 MiB: u2N 7074, u2T 6454; 3R+1W at 64 MiB: u2N 6874, u2T 6588).
+// Below 64 MiB touched: T.  (Between 32 and 64 MiB the scenarios disagree by 2-4 %
+// either way: an eager forward/backward sequence over 16 MiB arrays runs 4 %
+// faster with T, a cycle over three 16 MiB arrays 2 % faster with W.)
 //
-// What does not fit streams, and the policy that streams best is L, not N: loads
-// pass the caches by, while the stores stay in the memory-side cache, so that the
-// 256 MiB written last are still there when the next launch over the same
-// buffers starts at that end (direction a), and a consumer finds them.  The same
-// launch repeated, u2La / u1La / u2Nf / u1Nf / u2Tf:
-//   1R+1W   768 MiB 7115 / 6583 / 6580 / 6514 / 6112   1 GiB 7333 / 7045 / 6536 / 6476 / 6124
-//           2 GiB   6896 / 6737 / 6418 / 6518 / 6169
-//   2R+1W   768 MiB 6998 / 6763 / 6576 / 6708 / 5792   1 GiB 6810 / 6710 / 6521 / 6684 / 5917
-//   3R+1W (gradient kernel, in place)
-//           768 MiB 7135 / 7091 / 6257 / 6824 / 5492   1 GiB 6874 / 7086 / 6389 / 6792 / 5668
-// Launches through three or more pointers keep one vector per thread from 512 MiB
-// on (3R+1W at 1 GiB above, and in sequence: tanh forward 1R+1W over 512 MiB with
-// u2N followed by backward 3R+1W over 768 MiB with u1L sustains 6830 on 24 bytes per
-// element, more than any single shape for both: u1N 6636, u2L 5895, u2T 5712).
-// Between 256 and 768 MiB a launch through two pointers keeps N (in that very
-// sequence L for the forward kernel alone is faster, 7147 against 6451, and the
-// sequence slower, 5918 against 6742: its stores push out what the backward kernel
-// could have kept).
+// Above: W.  Loads pass the caches by; the stores stay in the memory-side cache,
+// so the 256 MiB written last are still there when the next launch over the same
+// buffers starts at that end (direction a, above 256 MiB) and a consumer finds
+// them; writing them through at once instead of leaving them dirty in an L2
+// smooths the write traffic (worth 2-5 % by itself).  The same launch repeated,
+// W / N / T:
+//   1R+1W   128 MiB 7382 / 6589 / 6803   512 MiB 7395 / 6510 / 6009   1 GiB 7513 / 6536 / 6124
+//           2 GiB   6987 / 6418 / 6169
+//   2R+1W   512 MiB 7345 / 6583 / 5840   1 GiB 7085 / 6521 / 5917
+//   3R+1W (gradient kernel, in place)    768 MiB 7616 / 6257 / 5492   2 GiB 6756 / 6355 / 5725
+// Chains (a launch reads what the launch before it wrote; eager cycle over three
+// arrays, by the bytes one launch touches): 128 MiB W 6948, T 6779; 256 MiB 7241 /
+// 5653; 512 MiB 7279 / 5993.  A rule that kept T for chains whose working set fits
+// the memory-side cache lost 1-3 % to W wherever it applied and is gone, as is one
+// that kept single operands temporal.
 //
-// Chains (a launch reads what the launch before it wrote; 1R+1W kernels, eager
-// cycle over three arrays, by the bytes one launch touches): while everything the
-// chain touches fits the memory-side cache, temporal accesses win (64 MiB: u2T
-// 6507, u2L 6271, u2N 5802); beyond, L with two vectors per thread, whatever the
-// direction (192 MiB: u2L 6956, u2T 6229, u2N 6153; 256 MiB: 7081 / 5653 / 6340;
-// 512 MiB: 7142 / 5993 / 6467; 768 MiB: 6970 / 6075 / 6475).
+// Exception: a launch through two pointers of 256-768 MiB that is not part of a
+// chain takes N.  Alone it is slower that way (512 MiB: 6510 against 7395), but as
+// the forward kernel of tanh forward + backward over 2^26 elements its temporal
+// stores push out what the backward kernel keeps: 7090 on 24 bytes per element
+// with N for the forward kernel, 6200 with W.
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint) {
     constexpr unsigned long long MiB = 1ull << 20;
     // non-temporal loads with temporal stores that are written through at once / both non-temporal
     constexpr int kLoads = 1 | kStoresWriteThrough, kBoth = 3;
     if (footprint_bytes < 64 * MiB) return {2, 0, false};
-    if (hint == CacheHint::Resident) return {2, 0, false};
-    if (hint == CacheHint::Streams) return {2, kLoads, footprint_bytes > 256 * MiB};
     if (footprint_bytes <= 256 * MiB) return {2, kLoads, false};
-    if (n_operands < 3 && footprint_bytes < 768 * MiB) return {2, kBoth, true};
+    if (n_operands < 3 && footprint_bytes < 768 * MiB && hint != CacheHint::Streams) return {2, kBoth, true};
     return {2, kLoads, true};
 }
 

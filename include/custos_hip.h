@@ -291,12 +291,11 @@ int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const cha
                                           const char *const *markers, int32_t n_markers,
                                           const custos_hip_tuning *tuning, size_t *code_size);
 /* Launches of 64 MiB and more (issued directly, or nodes of built graphs) so far, by what the
- * address ranges of the launches around them told: not part of a chain (the launch shape
- * then follows the bytes the launch touches, custos_hip_preferred_shape); part of a chain
- * -- it reads what one of the last eight launches wrote, or in a graph one of the next
- * levels reads what it writes -- whose working set stays in the 256 MiB memory-side cache
- * (temporal accesses); part of a chain whose working set does not (loads past the caches,
- * stores written through). */
+ * address ranges of the launches around them told: not part of a chain; part of a chain -- it
+ * reads what one of the last eight launches wrote, or in a graph one of the next levels reads
+ * what it writes -- whose working set stays in the 256 MiB memory-side cache; part of a chain
+ * whose working set does not.  (Only the last kind changes a launch shape: a two-pointer launch
+ * of 256 to 768 MiB keeps its stores temporal when it is part of a streaming chain.) */
 int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated, uint64_t *resident,
                                      uint64_t *streaming);
 /* Host-only: the launch shape the library picks for a launch that touches `footprint_bytes`
