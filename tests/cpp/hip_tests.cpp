@@ -400,4 +400,37 @@ TEST_CASE(hip_graph_orders_reuse_and_fill) {
     CHECK_EQ(custos_hip_set_graph_verify(dev, 0), 0);
 }
 
+// The merged launch whose operand table sits in a static device array (no allocation on the
+// way): the same values as one launch per operand set, on two calls in a row, the second smaller;
+// sizes beyond the table and operand sets that overlap are refused.
+TEST_CASE(hip_apply_fn_many_noalloc) {
+    HIP<Base> device;
+    custos_hip_device* dev = device.handle();
+    custos_hip_kernel* k = device.compile(CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, "((a * b) + 0.5)", {"a", "b"});
+    for (const auto& shape : {std::pair<size_t, size_t>{19, 3001}, std::pair<size_t, size_t>{4, 130}}) {
+        const size_t sets = shape.first, n = shape.second;
+        std::vector<Buffer<float, HIP<Base>>> as, bs, outs, singles;
+        std::vector<uint64_t> rows;
+        for (size_t s = 0; s < sets; s++) {
+            std::vector<float> av(n), bv(n);
+            for (size_t i = 0; i < n; i++) av[i] = 0.5f + static_cast<float>((i * 7 + s) % 13), bv[i] = 1.25f - static_cast<float>((i + 3 * s) % 5);
+            as.push_back(device.buffer(av));
+            bs.push_back(device.buffer(bv));
+            outs.push_back(device.new_buffer<float>(n));
+            singles.push_back(device.new_buffer<float>(n));
+            rows.insert(rows.end(), {as[s].ptr(), bs[s].ptr(), outs[s].ptr()});
+            CHECK_EQ(custos_hip_apply_fn2(dev, k, as[s].ptr(), bs[s].ptr(), singles[s].ptr(), n), 0);
+        }
+        CHECK_EQ(custos_hip_apply_fn_many_noalloc(dev, k, rows.data(), 3, sets, n), 0);
+        for (size_t s = 0; s < sets; s++) CHECK_VEC_EQ(outs[s].read(), singles[s].read());
+        // a set that writes what another set reads
+        std::vector<uint64_t> clash = rows;
+        clash[5] = as[0].ptr();
+        CHECK_EQ(custos_hip_apply_fn_many_noalloc(dev, k, clash.data(), 3, sets, n), static_cast<int32_t>(CUSTOS_HIP_ERR_BAD_OVERLAP));
+    }
+    std::vector<uint64_t> too_many(3 * 3000, 256);
+    CHECK_EQ(custos_hip_apply_fn_many_noalloc(dev, k, too_many.data(), 3, 3000, 16), static_cast<int32_t>(CUSTOS_HIP_ERR_TOO_LARGE));
+    CHECK_EQ(custos_hip_apply_fn_many_noalloc(dev, k, too_many.data(), 2, 10, 16), static_cast<int32_t>(CUSTOS_HIP_ERR_ARITY_MISMATCH));
+}
+
 int main(int argc, char** argv) { return check::run(argc, argv); }
