@@ -111,6 +111,7 @@ PROTOTYPES = {
     "custos_hip_kernel_name": (C.c_char_p, [_P]),
     "custos_hip_kernel_hash": (C.c_uint64, [_P]),
     "custos_hip_preferred_shape": (C.c_int32, [C.c_uint64, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "custos_hip_last_launch_shape": (C.c_int32, [_P, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "custos_hip_kernel_launched_as": (C.c_int32, [_P, _P, C.c_size_t, C.POINTER(C.c_void_p)]),
     "custos_hip_kernel_arity": (C.c_int32, [_P]),
     "custos_hip_cache_stats": (C.c_int32, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),

@@ -157,7 +157,7 @@ void record_level(const std::vector<RecNode>& nodes, const std::vector<size_t>& 
         if (nodes[i].type != RecNode::Source) all.insert(all.end(), nodes[i].acc.begin(), nodes[i].acc.end());
     unsigned long long bytes = 0;
     for (const Access& a : all) bytes += a.end - a.begin;
-    if (bytes >= kTrafficFromBytes) history->record(all);
+    if (bytes > kTrafficBeyondBytes) history->record(all);
 }
 
 // The nodes of one dependency level: launches of one kernel (or of one code with different
@@ -271,12 +271,18 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
             unsigned long long footprint = 0;
             for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
             CacheHint hint = CacheHint::Unknown;
+            unsigned long long working_set = 0;
             if (footprint >= kHintFromBytes) {
                 hint = hint_for(nodes, p, *history, later_reads);
                 dev->hinted[static_cast<int>(hint)]++;
+            } else if (footprint > kTrafficBeyondBytes && footprint <= kL2WorkingSet) {
+                std::vector<Access> all;
+                for (size_t i : p.members) all.insert(all.end(), nodes[i].acc.begin(), nodes[i].acc.end());
+                working_set = history->working_set_with(all);
             }
             p.kern = first.k;
-            p.shape = resolve_shape(dev, first.k, footprint, hint);
+            p.shape = resolve_shape(dev, first.k, footprint, hint, working_set);
+            dev->last_shape[0] = p.shape.unroll, dev->last_shape[1] = p.shape.nontemporal, dev->last_shape[2] = p.shape.alternate;
         }
         if (p.members.size() > 1) append_tables(nodes, &p, host_table);
     }

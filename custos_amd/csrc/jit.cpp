@@ -278,9 +278,9 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 }
 
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
-                            CacheHint hint) {
+                            CacheHint hint, unsigned long long working_set_bytes) {
     const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;
-    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint);
+    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint, working_set_bytes);
     ResolvedShape r;
     const int direction = dev->tuning.direction;
     r.alternate = direction == 2 || (direction == 0 && shape.alternate);

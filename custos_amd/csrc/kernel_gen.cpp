@@ -29,11 +29,19 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // throughout (one was never more than 1 % ahead with W).  GB/s on the
 // algorithmic bytes.
 //
-// Below 64 MiB touched: T.  (Between 32 and 64 MiB the scenarios disagree by 2-4 %
-// either way: an eager forward/backward sequence over 16 MiB arrays runs 4 %
-// faster with T, a cycle over three 16 MiB arrays 2 % faster with W.)
+// While the launch and the launches just before it touch no more than 32 MiB
+// together (what the eight L2s hold): T.  The in-place gradient kernel repeated
+// over 28 MiB: T 9144, W 7569.  A launch that would fit the L2s after launches
+// that do not leave them to it streams like a large one (tanh forward, 20 MiB,
+// + backward, 30 MiB, over 40 MiB of arrays: W 6073, T 5227; three merged
+// launches of 48, 48 and 32 MiB in a replayed graph: 23.6 us with W or T
+// throughout, 25.1 us with W, W, T).
 //
-// Above: W.  Loads pass the caches by; the stores stay in the memory-side cache,
+// Above: W.  Already just above the L2s, where the working set still fits the
+// memory-side cache, T loses to it (1R+1W repeated over 48 MiB: T 6012, W 8951;
+// 2R+1W 7146 / 6307; gradient kernel 7201 / 6406; tanh forward + backward over
+// 40 MiB 6073 / 5227): temporal accesses thrash the L2s and leave dirty lines to
+// be evicted later, W is served by the memory-side cache.  Loads pass the caches by; the stores stay in the memory-side cache,
 // so the 256 MiB written last are still there when the next launch over the same
 // buffers starts at that end (direction a, above 256 MiB) and a consumer finds
 // them; writing them through at once instead of leaving them dirty in an L2
@@ -54,11 +62,12 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // the forward kernel of tanh forward + backward over 2^26 elements its temporal
 // stores push out what the backward kernel keeps: 7090 on 24 bytes per element
 // with N for the forward kernel, 6200 with W.
-LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint) {
+LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint,
+                            unsigned long long working_set_bytes) {
     constexpr unsigned long long MiB = 1ull << 20;
     // non-temporal loads with temporal stores that are written through at once / both non-temporal
     constexpr int kLoads = 1 | kStoresWriteThrough, kBoth = 3;
-    if (footprint_bytes < 64 * MiB) return {2, 0, false};
+    if (std::max(footprint_bytes, working_set_bytes) <= kL2WorkingSet) return {2, 0, false};
     if (footprint_bytes <= 256 * MiB) return {2, kLoads, false};
     if (n_operands < 3 && footprint_bytes < 768 * MiB && hint != CacheHint::Streams) return {2, kBoth, true};
     return {2, kLoads, true};

@@ -50,7 +50,11 @@ enum class CacheHint {
     Streams,   // it does not: stream past the cache
 };
 constexpr unsigned long long kCacheWorkingSet = 256ull << 20;
-LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint = CacheHint::Unknown);
+// `working_set_bytes`: distinct bytes touched by the launch and the last few launches before it
+// together (0 = not known: the launch's own bytes count).
+constexpr unsigned long long kL2WorkingSet = 32ull << 20;  // what the eight L2s hold together
+LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint = CacheHint::Unknown,
+                            unsigned long long working_set_bytes = 0);
 
 // The last argument of every generated entry point: how this launch runs the kernel.  Nothing
 // of it is compiled in, so one kernel per expression serves every launch size.

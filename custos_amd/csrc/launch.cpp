@@ -150,7 +150,8 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
     const unsigned long long footprint = static_cast<unsigned long long>(ops.size()) * bytes;
     CacheHint hint = CacheHint::Unknown;
-    if (footprint >= kTrafficFromBytes) {
+    unsigned long long working_set = 0;
+    if (footprint > kTrafficBeyondBytes) {
         std::vector<Access> all, reads;
         for (const Range& r : ops) {
             all.push_back({r.ptr, r.ptr + bytes, r.written});
@@ -160,10 +161,14 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
         if (footprint >= kHintFromBytes) {
             hint = dev->recent.classify(reads, all);
             dev->hinted[static_cast<int>(hint)]++;
+        } else if (footprint <= kL2WorkingSet) {
+            // a launch that fits the L2s by itself: do the launches before it leave them to it?
+            working_set = dev->recent.working_set_with(all);
         }
         dev->recent.record(all);
     }
-    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint);
+    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set);
+    dev->last_shape[0] = shape.unroll, dev->last_shape[1] = shape.nontemporal, dev->last_shape[2] = shape.alternate;
     const unsigned int grid = launch_grid(dev, k, n, n_vec, shape.unroll);
     unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, shape.alternate && (dev->launch_parity ^= 1));
     uint64_t ptrs[8];
@@ -206,6 +211,14 @@ int32_t custos_hip_apply_fn_n(custos_hip_device* dev, custos_hip_kernel* kernel,
     for (int i = 0; i < n_ins; i++) ops.push_back({ins[i], false});
     ops.push_back({out, true});
     return launch_or_record(dev, kernel, ops, n);
+}
+
+int32_t custos_hip_last_launch_shape(custos_hip_device* dev, int32_t* unroll, int32_t* nontemporal, int32_t* alternate) {
+    REQUIRE_DEV(dev);
+    if (unroll) *unroll = dev->last_shape[0];
+    if (nontemporal) *nontemporal = dev->last_shape[1];
+    if (alternate) *alternate = dev->last_shape[2];
+    return CUSTOS_HIP_OK;
 }
 
 int32_t custos_hip_launch_hint_stats(custos_hip_device* dev, uint64_t* unrelated, uint64_t* resident, uint64_t* streaming) {

@@ -91,10 +91,11 @@ struct RecNode {
 
 // The address ranges of the last few launches, from which a launch learns whether it reads
 // what one of them wrote and how much was touched since (see CacheHint).
-// Launches below kHintFromBytes take the small-launch shape whatever the cache holds; launches
-// below kTrafficFromBytes are not worth tracking (their kernels are shorter than a launch call).
+// Launches up to kTrafficBeyondBytes are not tracked (their kernels are shorter than a launch
+// call, and they keep the small-launch shape whatever came before); whether a launch is part of
+// a chain is asked from kHintFromBytes on, the smallest launch whose shape could follow from it.
 constexpr unsigned long long kHintFromBytes = 64ull << 20;
-constexpr unsigned long long kTrafficFromBytes = 32ull << 20;
+constexpr unsigned long long kTrafficBeyondBytes = 8ull << 20;
 class RecentTraffic {
    public:
     // Whether one of the recorded launches wrote something in `reads`.
@@ -126,6 +127,8 @@ struct custos_hip_device {
     std::unordered_map<uint64_t, uint32_t> value_sets_seen;
     RecentTraffic recent;            // of the launches issued directly (not recorded)
     uint64_t hinted[4] = {0, 0, 0, 0};  // launches and graph nodes of at least kHintFromBytes by CacheHint
+    int32_t last_shape[3] = {0, 0, 0};  // vectors per thread, cache policy, alternating: of the generated kernel
+                                        // launched or planned into a graph last (custos_hip_last_launch_shape)
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     bool graph_verify = false;       // built graphs are checked by brute force against the recorded conflicts
     int32_t graph_edges = CUSTOS_HIP_GRAPH_EDGES_CHAIN;  // how built graphs order their nodes
@@ -231,7 +234,7 @@ struct ResolvedShape {
     bool alternate = false;
 };
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
-                            CacheHint hint = CacheHint::Unknown);
+                            CacheHint hint = CacheHint::Unknown, unsigned long long working_set_bytes = 0);
 
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);

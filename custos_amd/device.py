@@ -362,6 +362,13 @@ class HIP:
         self._check(self.lib.custos_hip_launch_hint_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
         return a.value, b.value, c.value
 
+    def last_launch_shape(self):
+        """(vectors per thread, cache-policy bits, alternating) of the generated kernel launched, or
+        planned into a graph, last."""
+        u, nt, alt = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+        self._check(self.lib.custos_hip_last_launch_shape(self.handle, C.byref(u), C.byref(nt), C.byref(alt)))
+        return u.value, nt.value, bool(alt.value)
+
     def set_literal_policy(self, policy: int) -> None:
         """How literal values reach kernels: capi.LITERALS_ADAPTIVE (default), _IN_CODE, _AS_PARAMETERS."""
         self._check(self.lib.custos_hip_set_literal_policy(self.handle, policy))

@@ -85,6 +85,8 @@ extern "C" {
                                              tuning: *const HipTuning, code_size: *mut usize) -> i32;
     pub fn custos_hip_preferred_shape(footprint_bytes: u64, n_operands: i32, unroll: *mut i32,
                                       nontemporal: *mut i32, alternate: *mut i32) -> i32;
+    pub fn custos_hip_last_launch_shape(dev: *mut HipDeviceHandle, unroll: *mut i32, nontemporal: *mut i32,
+                                        alternate: *mut i32) -> i32;
     pub fn custos_hip_expr_canonical(src: *const c_char, markers: *const *const c_char, n_markers: i32,
                                      buf: *mut c_char, cap: usize, needed: *mut usize) -> i32;
     pub fn custos_hip_expr_constants(dtype: i32, src: *const c_char, markers: *const *const c_char, n_markers: i32,

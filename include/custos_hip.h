@@ -302,9 +302,17 @@ int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated
  * (all operands together) through `n_operands` pointers, for the knobs left at 0 in
  * custos_hip_tuning: vectors per thread, the `nontemporal` bits, and whether the launch
  * walks its tiles against the direction of the previous one -- for a launch that is not part
- * of a chain (see custos_hip_launch_hint_stats). */
+ * of a chain (see custos_hip_launch_hint_stats) and comes after nothing: a launch of more than
+ * 8 and up to 32 MiB (what the eight L2s hold together) keeps temporal accesses only if it and
+ * the up to eight tracked launches (or graph levels) before it touch no more than those 32 MiB
+ * together; otherwise it streams like a larger one. */
 int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t *unroll,
                                    int32_t *nontemporal, int32_t *alternate);
+/* The shape of the generated kernel that was launched directly, or planned into a graph by
+ * custos_hip_capture_end, last on this device (same three values; all 0 before the first).
+ * No counterpart in the reference, whose launches have one shape. */
+int32_t custos_hip_last_launch_shape(custos_hip_device *dev, int32_t *unroll, int32_t *nontemporal,
+                                     int32_t *alternate);
 /* Canonical re-print of an expression in the reference's ToCLSource format. */
 int32_t custos_hip_expr_canonical(const char *src, const char *const *markers, int32_t n_markers,
                                   char *buf, size_t cap, size_t *needed);

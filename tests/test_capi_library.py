@@ -120,7 +120,7 @@ def test_product_never_imports_the_oracle():
 
 
 def test_launch_shape_by_bytes_touched():
-    """The shape for the knobs a caller leaves open: temporal accesses below the L2 capacity; above,
+    """The shape for the knobs a caller leaves open: temporal accesses up to the L2 capacity; above,
     loads past the caches and temporal stores written through at once (what a launch wrote last is what
     the next launch over the same buffers starts on: the largest launches alternate their direction);
     a two-pointer launch of 256 to 768 MiB streams both ways."""
@@ -128,7 +128,9 @@ def test_launch_shape_by_bytes_touched():
     shape = capi.preferred_shape
     loads = 1 | 64                                         # non-temporal loads, stores written through at once
     assert shape(8 * MiB, 2) == (2, 0, False)              # config 1: 2^20 f32 in, out
-    assert shape(48 * MiB, 3) == (2, 0, False)             # config 5, one recorded level merged
+    assert shape(32 * MiB, 2) == (2, 0, False)             # what the eight L2s hold together
+    assert shape(32 * MiB + 1, 2) == (2, loads, False)
+    assert shape(48 * MiB, 3) == (2, loads, False)         # config 5, one recorded level merged
     assert shape(64 * MiB, 4) == (2, loads, False)         # config 5 after element-wise fusing
     assert shape(128 * MiB, 2) == (2, loads, False) and shape(256 * MiB, 2) == (2, loads, False)
     assert shape(257 * MiB, 2) == (2, 3, True)

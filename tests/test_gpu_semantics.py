@@ -1034,6 +1034,58 @@ def test_launch_shape_follows_the_launches_around_it(oracle):
         dev.close()
 
 
+def test_temporal_accesses_while_the_working_set_fits_the_l2s(oracle):
+    """A launch of up to 32 MiB keeps temporal accesses only while it and the launches before it touch no
+    more than 32 MiB together (the eight L2s); after launches that do not leave the L2s to it, it streams
+    like a larger one.  Directly issued launches and the nodes of a graph."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        loads = 1 | 64
+        n = 3 << 20                                   # 12 MiB per array
+        x = synth.uniform_f32(11, n, -2, 2)
+        f = lambda v: v.mul(1.5).sub(0.25)
+        a, b, c, d = dev.buffer(x), dev.alloc(n), dev.alloc(n), dev.alloc(n)
+        dev.apply_fn(a, f, out=b)                     # 24 MiB, nothing before it
+        assert dev.last_launch_shape() == (2, 0, False)
+        dev.apply_fn(a, f, out=b)                     # the same 24 MiB again
+        assert dev.last_launch_shape() == (2, 0, False)
+        dev.apply_fn(b, f, out=c)                     # 36 MiB with the launches before
+        assert dev.last_launch_shape() == (2, loads, False)
+        dev.apply_fn(c, f, out=d)
+        assert dev.last_launch_shape() == (2, loads, False)
+        want = x
+        for _ in range(3):
+            want = want * np.float32(1.5) - np.float32(0.25)
+        assert_bits_equal(d.read(), want)
+        small = dev.buffer(x[: 1 << 20])              # 8 MiB and less: not tracked, temporal
+        dev.apply_fn(small, f)
+        assert dev.last_launch_shape() == (2, 0, False)
+        # the window is eight launches: after eight over the same 24 MiB the ninth has the L2s to itself
+        for _ in range(9):
+            dev.apply_fn(a, f, out=b)
+        assert dev.last_launch_shape() == (2, 0, False)
+        # in a graph: the levels before a node count, the last ones before the first (a graph is replayed)
+        dev.capture_begin()
+        dev.apply_fn(a, f, out=b)
+        dev.apply_fn(b, f, out=c)
+        dev.apply_fn(c, f, out=d)
+        graph = dev.capture_end()
+        assert dev.last_launch_shape() == (2, loads, False)
+        for _ in range(3):
+            graph.launch()
+        assert_bits_equal(d.read(), want)
+        graph.destroy()
+        dev.capture_begin()
+        dev.apply_fn(a, f, out=b)
+        graph = dev.capture_end()                     # one 24 MiB node alone
+        assert dev.last_launch_shape() == (2, 0, False)
+        graph.launch()
+        graph.destroy()
+    finally:
+        dev.close()
+
+
 def test_more_than_two_to_the_32_elements(hip):
     """Indices are 64-bit throughout: 2^32 + 5 one-byte elements (4 GiB in, 4 GiB out), launched
     directly and from a replayed graph; windows around 2^31, 2^32 and the scalar tail."""
