@@ -402,6 +402,13 @@ def bench_others(dev, args, stack_c5):
                             "and the host's time per launch")
     out["c1"]["launches"] = launches
     out["c1"]["kernel"] = dev.kernel_name(k)
+    # the same through the C++ device, eager: `HIP<Base>::apply_fn` call after call, child process
+    stack_c1 = dict(stack_c5.pop("c1", {"skipped": True}))
+    if "dump" in stack_c1:
+        first = stack_c1.pop("dump")
+        assert np.max(np.abs(first.view(np.int32).astype(np.int64) - want[: first.size].view(np.int32).astype(np.int64))) <= 4
+        stack_c1["max_ulp_vs_cpu_oracle"] = int(np.max(np.abs(first.view(np.int32).astype(np.int64) - want[: first.size].view(np.int32).astype(np.int64))))
+    out["c1"]["module_stack"] = stack_c1
     # the same launch recorded 64 times into one graph (every launch writes the same output, so
     # the graph is a chain of 64 nodes): the device's time per launch, without the host's
     if args.hipgraph:
@@ -571,8 +578,12 @@ def main():
             stack = module_stack("c2", args.steps, args.warmup, log2n=args.log2n, dump=(1 << 20, dump))
             if "error" not in stack and os.path.exists(dump):
                 stack["dump"] = np.fromfile(dump, dtype=np.float32)
-        if args.others:
-            stack_c5 = {"as_recorded": module_stack("c5", 500, 20), "after_elementwise_fusing": module_stack("c5", 500, 20, fuse=True)}
+            if args.others:
+                stack_c5 = {"as_recorded": module_stack("c5", 500, 20), "after_elementwise_fusing": module_stack("c5", 500, 20, fuse=True)}
+                dump1 = os.path.join(tmp, "c1_first.f32")
+                stack_c5["c1"] = module_stack("c1", 200, 20, dump=(1 << 20, dump1))
+                if "error" not in stack_c5["c1"] and os.path.exists(dump1):
+                    stack_c5["c1"]["dump"] = np.fromfile(dump1, dtype=np.float32)
 
     import custos_amd
 

@@ -2,6 +2,10 @@
 // stack `HIP<Graph<Lazy<Base>>>`, with the reference's run semantics (every `run()` launches
 // the recorded graph and waits for it: src/devices/cuda/lazy.rs:31-49).
 //
+//   c1  eager `apply_fn(|x| x.exp())` on `HIP<Base>` over 2^20 f32, again and again: every call prints
+//       the expression, looks the kernel up, retrieves a new output buffer and launches; nothing
+//       waits between the calls (the reference's eager launches do not wait either), one wait at
+//       the end of each timed batch of 64 calls
 //   c2  five `apply_fn` calls (sin, *2, +1, max 0, -0.5) on a lazily recorded f32 buffer,
 //       `optimize_mem_graph`, `unary_fusing`, then `run()` again and again
 //       (the shape of src/op_hint.rs:121-140 and examples/lazy_and_fusing.rs)
@@ -83,7 +87,7 @@ static void dump(Dev& device, uint64_t ptr, size_t count, const char* path) {
 
 int main(int argc, char** argv) {
     std::string config = "c2", dump_path;
-    int log2n = 28, steps = 100, warmup = 20, settle_ms = 150;
+    int log2n = 0, steps = 100, warmup = 20, settle_ms = 150;
     size_t dump_count = 0;
     bool fuse = false;
     for (int i = 1; i < argc; i++) {
@@ -109,11 +113,35 @@ int main(int argc, char** argv) {
             return 2;
         }
     }
-    if (steps < 1 || warmup < 0 || settle_ms < 0 || log2n < 4 || log2n > 32) return 2;
+    if (steps < 1 || warmup < 0 || settle_ms < 0 || (log2n != 0 && (log2n < 4 || log2n > 32))) return 2;
 
     try {
-        if (config == "c2") {
-            const size_t n = size_t(1) << log2n;
+        if (config == "c1") {
+            const size_t n = size_t(1) << (log2n ? log2n : 20);
+            HIP<Base> device(0);
+            auto buf = device.buffer(uniform_f32(0, n, -4.f, 8.f));
+            const int batch = 64;
+            auto out = device.apply_fn(buf, [](auto x) { return x.exp(); });
+            const Timing t = time_runs(
+                [&] {
+                    for (int i = 0; i < batch; i++) out = device.apply_fn(buf, [](auto x) { return x.exp(); });
+                    device.sync();
+                },
+                warmup, steps, settle_ms);
+            if (dump_count) {
+                std::vector<float> first(std::min(dump_count, n));
+                device.read_raw(first.data(), out.ptr(), first.size() * sizeof(float));
+                FILE* f = std::fopen(dump_path.c_str(), "wb");
+                if (!f || std::fwrite(first.data(), sizeof(float), first.size(), f) != first.size()) return 2;
+                std::fclose(f);
+            }
+            std::printf("{\"config\": \"c1\", \"stack\": \"HIP<Base>\", \"calls\": \"apply_fn(exp) x %d, sync()\", \"waits\": false, "
+                        "\"elements\": %zu, \"steps\": %d, \"warmup\": %d, \"us_per_call\": %.3f, \"median_us\": %.3f, "
+                        "\"min_us\": %.3f, \"GBps\": %.2f}\n",
+                        batch, n, steps, warmup, t.mean_us / batch, t.median_us / batch, t.min_us / batch,
+                        8.0 * static_cast<double>(n) / (t.mean_us / batch * 1e-6) / 1e9);
+        } else if (config == "c2") {
+            const size_t n = size_t(1) << (log2n ? log2n : 28);
             Dev device(0);
             const float pi = 3.14159265358979323846f;
             auto buf = device.buffer(uniform_f32(0, n, -pi, static_cast<float>(3.14159265358979323846 - -3.14159265358979323846)));
