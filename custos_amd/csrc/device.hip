@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <thread>
 
 #include "runtime.hpp"
@@ -38,11 +39,13 @@ constexpr size_t kScratchWords = 8192;
 static __device__ __align__(256) unsigned long long scratch[kScratchWords];
 constexpr int kMaxDevices = 64;
 static unsigned long long* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;  // handles are created from several threads
 static_assert(kScratchWords * sizeof(unsigned long long) <= kStagedReadMax, "the table travels through one staging slot");
 
 // With device `idx` current: the address of that device's copy of `scratch`.
 static hipError_t scratch_address(int idx, unsigned long long** out) {
     if (idx < 0 || idx >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (!g_scratch_ptr[idx]) {
         void* p = nullptr;
         hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
