@@ -275,7 +275,8 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
             if (footprint >= kHintFromBytes) {
                 hint = hint_for(nodes, p, *history, later_reads);
                 dev->hinted[static_cast<int>(hint)]++;
-            } else if (footprint > kTrafficBeyondBytes && footprint <= kL2WorkingSet) {
+            }
+            if (footprint > kTrafficBeyondBytes) {
                 std::vector<Access> all;
                 for (size_t i : p.members) all.insert(all.end(), nodes[i].acc.begin(), nodes[i].acc.end());
                 working_set = history->working_set_with(all);

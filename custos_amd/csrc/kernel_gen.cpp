@@ -58,18 +58,22 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // that kept single operands temporal.
 //
 // Exception: a launch through two pointers of 256-768 MiB that is not part of a
-// chain takes N.  Alone it is slower that way (512 MiB: 6510 against 7395), but as
-// the forward kernel of tanh forward + backward over 2^26 elements its temporal
-// stores push out what the backward kernel keeps: 7090 on 24 bytes per element
-// with N for the forward kernel, 6200 with W.
+// chain takes N when the launches before it touched other memory as well (its
+// working set is larger than the launch).  Repeated alone it is slower that way
+// (512 MiB: 6510 against 7395) and keeps W; but as the forward kernel of tanh
+// forward + backward over 2^26 elements its temporal stores push out what the
+// backward kernel keeps: 7090 on 24 bytes per element with N for the forward
+// kernel, 6200 with W.
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint,
                             unsigned long long working_set_bytes) {
     constexpr unsigned long long MiB = 1ull << 20;
     // non-temporal loads with temporal stores that are written through at once / both non-temporal
     constexpr int kLoads = 1 | kStoresWriteThrough, kBoth = 3;
-    if (std::max(footprint_bytes, working_set_bytes) <= kL2WorkingSet) return {2, 0, false};
+    const unsigned long long working_set = std::max(footprint_bytes, working_set_bytes);
+    if (working_set <= kL2WorkingSet) return {2, 0, false};
     if (footprint_bytes <= 256 * MiB) return {2, kLoads, false};
-    if (n_operands < 3 && footprint_bytes < 768 * MiB && hint != CacheHint::Streams) return {2, kBoth, true};
+    if (n_operands < 3 && footprint_bytes < 768 * MiB && hint != CacheHint::Streams && working_set > footprint_bytes)
+        return {2, kBoth, true};
     return {2, kLoads, true};
 }
 

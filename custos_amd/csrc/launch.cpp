@@ -161,10 +161,10 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
         if (footprint >= kHintFromBytes) {
             hint = dev->recent.classify(reads, all);
             dev->hinted[static_cast<int>(hint)]++;
-        } else if (footprint <= kL2WorkingSet) {
-            // a launch that fits the L2s by itself: do the launches before it leave them to it?
-            working_set = dev->recent.working_set_with(all);
         }
+        // what the launches before it leave to this one: the L2s to a small launch, the
+        // memory-side cache to a large one
+        working_set = dev->recent.working_set_with(all);
         dev->recent.record(all);
     }
     const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set);

@@ -305,7 +305,9 @@ int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated
  * of a chain (see custos_hip_launch_hint_stats) and comes after nothing: a launch of more than
  * 8 and up to 32 MiB (what the eight L2s hold together) keeps temporal accesses only if it and
  * the up to eight tracked launches (or graph levels) before it touch no more than those 32 MiB
- * together; otherwise it streams like a larger one. */
+ * together; otherwise it streams like a larger one.  And a launch of 256 to 768 MiB through two
+ * pointers streams its stores past the memory-side cache as well when those launches touched
+ * other memory too. */
 int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t *unroll,
                                    int32_t *nontemporal, int32_t *alternate);
 /* The shape of the generated kernel that was launched directly, or planned into a graph by

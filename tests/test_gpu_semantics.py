@@ -1110,6 +1110,31 @@ def test_temporal_accesses_while_the_working_set_fits_the_l2s(oracle):
         dev.close()
 
 
+def test_mid_sized_launches_leave_the_cache_to_their_neighbours(oracle):
+    """A two-pointer launch of 256 to 768 MiB keeps its stores in the memory-side cache while it has the
+    cache to itself (the same launch again and again), and streams them past it once the launches before it
+    touched other memory as well (tanh forward between gradient launches over other arrays)."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        loads, both = 1 | 64, 3
+        n = 1 << 26                                   # 256 MiB per array
+        x, y = dev.alloc(n), dev.alloc(n)
+        fwd = lambda v: v.tanh()
+        dev.apply_fn(x, fwd, out=y)
+        assert dev.last_launch_shape() == (2, loads, True)
+        dev.apply_fn(x, fwd, out=y)                   # nothing else in between
+        assert dev.last_launch_shape() == (2, loads, True)
+        g, o = dev.alloc(n), dev.alloc(n)
+        dev.add_unary_grad(x, g, o, lambda v: v.mul(2.0))
+        assert dev.last_launch_shape() == (2, loads, True)      # three pointers: always loads only
+        dev.apply_fn(x, fwd, out=y)                   # g and o were touched since
+        assert dev.last_launch_shape() == (2, both, True)
+        assert np.all(y.slice(n - 4096, n).read() == 0)
+    finally:
+        dev.close()
+
+
 def test_more_than_two_to_the_32_elements(hip):
     """Indices are 64-bit throughout: 2^32 + 5 one-byte elements (4 GiB in, 4 GiB out), launched
     directly and from a replayed graph; windows around 2^31, 2^32 and the scalar tail."""
