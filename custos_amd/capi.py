@@ -111,6 +111,11 @@ PROTOTYPES = {
     "custos_hip_kernel_name": (C.c_char_p, [_P]),
     "custos_hip_kernel_hash": (C.c_uint64, [_P]),
     "custos_hip_preferred_shape": (C.c_int32, [C.c_uint64, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "custos_hip_set_graph_fusing": (C.c_int32, [_P, C.c_int32]),
+    "custos_hip_graph_fused_launches": (C.c_int32, [_P, C.POINTER(C.c_size_t)]),
+    "custos_hip_chain_emit": (C.c_int32, [C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.c_int32, C.POINTER(C.c_int32),
+                                          C.POINTER(C.c_int32), C.c_int32, C.c_int32, C.c_char_p, C.c_size_t,
+                                          C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "custos_hip_last_launch_shape": (C.c_int32, [_P, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "custos_hip_kernel_launched_as": (C.c_int32, [_P, _P, C.c_size_t, C.POINTER(C.c_void_p)]),
     "custos_hip_kernel_arity": (C.c_int32, [_P]),
@@ -219,6 +224,23 @@ def expr_emit(kind: int, dtype: str, src: str, markers, tuning: Tuning | None = 
     buf = C.create_string_buffer(needed.value)
     check(emit(kind, DTYPES[dtype][0], src.encode(), arr, n, t, buf, needed.value, None, None))
     return buf.value.decode(), h.value
+
+
+def chain_emit(dtype: str, stages, n_inputs: int, n_outputs: int, compile_it: bool = False):
+    """Host-only: source (and, with `compile_it`, the gfx950 code size) of the kernel that joins several
+    expressions.  `stages`: (source text over v0.., [where each variable comes from], output index or -1)."""
+    lib = load_library()
+    srcs = (C.c_char_p * len(stages))(*[s[0].encode() for s in stages])
+    n_vars = (C.c_int32 * len(stages))(*[len(s[1]) for s in stages])
+    flat = [v for s in stages for v in s[1]]
+    sources = (C.c_int32 * len(flat))(*flat)
+    outs = (C.c_int32 * len(stages))(*[s[2] for s in stages])
+    needed, size = C.c_size_t(0), C.c_size_t(0)
+    args = (DTYPES[dtype][0], srcs, n_vars, len(stages), sources, outs, n_inputs, n_outputs)
+    check(lib.custos_hip_chain_emit(*args, None, 0, C.byref(needed), C.byref(size) if compile_it else None))
+    buf = C.create_string_buffer(needed.value)
+    check(lib.custos_hip_chain_emit(*args, buf, needed.value, None, None))
+    return buf.value.decode(), size.value
 
 
 def expr_build_code_object(kind: int, dtype: str, src: str, markers, tuning: Tuning | None = None) -> int:

@@ -120,6 +120,234 @@ void assign_levels(std::vector<RecNode>& nodes, bool edges) {
     }
 }
 
+// ---- joining producers with their consumers ----
+//
+// A recorded apply launch whose output a later apply launch reads element for element (the
+// same address and length) is joined with that launch: ONE kernel evaluates both expressions
+// per element, stores both results where the two launches stored them, and hands the first
+// result to the second expression in a register instead of through memory.  `t = a * b;
+// u = t + c; y = f(u)` becomes one launch that reads a, b, c and writes t, u, y: 24 instead of
+// 32 bytes per f32 element, one launch instead of three.  Every buffer still receives exactly
+// the value the separate launches gave it (the value handed on is the stored one, rounded to
+// the storage type), so nothing a caller can observe changes.
+//
+// What may be joined.  Both are apply launches of generated kernels with the same element
+// type, length and alignment phase.  The consumer reads at least one output of the producer.
+// Every address range of the one that the other also touches, one of them writing, is the
+// SAME range (same address): the fused kernel handles element i of every operand in one
+// lane, all loads before all stores, so equal ranges behave as in the separate launches and
+// disjoint ones do not matter, but a range shifted against another would be read or written
+// by another lane at another time.  And nothing recorded between the two conflicts with the
+// producer (reads what it writes, writes what it reads or writes): the joined launch takes the
+// consumer's place in the recording.  Joined launches are producers and consumers in turn.
+
+struct ChainBuild {
+    std::vector<ChainStage> stages;
+    std::vector<uint64_t> ext;        // input pointers of the kernel to be
+    std::vector<uint64_t> stage_ptr;  // per stage: where its launch stored its result
+};
+
+// The last stage that writes `ptr`, or -1.
+int writer_of(const ChainBuild& c, uint64_t ptr) {
+    for (size_t s = c.stage_ptr.size(); s-- > 0;)
+        if (c.stage_ptr[s] == ptr) return static_cast<int>(s);
+    return -1;
+}
+
+int input_index(ChainBuild* c, uint64_t ptr) {
+    for (size_t i = 0; i < c->ext.size(); i++)
+        if (c->ext[i] == ptr) return static_cast<int>(i);
+    c->ext.push_back(ptr);
+    return static_cast<int>(c->ext.size()) - 1;
+}
+
+size_t distinct_outputs(const ChainBuild& c) {
+    size_t n = 0;
+    for (size_t s = 0; s < c.stage_ptr.size(); s++) n += writer_of(c, c.stage_ptr[s]) == static_cast<int>(s);
+    return n;
+}
+
+bool fusable_kernel(const RecNode& n) {
+    if (n.type != RecNode::Kernel || n.k->spec.kind != Kind::Apply || !n.k->spec.auto_unroll) return false;
+    return n.k->spec.tuning.blocks_per_cu <= 0;
+}
+
+ChainBuild chain_of(const RecNode& n) {
+    ChainBuild c;
+    ChainStage stage;
+    stage.expr = n.k->spec.expr;
+    for (int v = 0; v < stage.expr.n_vars; v++) stage.source.push_back(input_index(&c, n.ptrs[static_cast<size_t>(v)]));
+    c.stages.push_back(std::move(stage));
+    c.stage_ptr.push_back(n.ptrs.back());
+    return c;
+}
+
+// `producer` followed by `consumer` as one chain, or false if they may not be joined.
+bool join_chains(const ChainBuild& producer, const ChainBuild& consumer, uint64_t bytes, ChainBuild* joined) {
+    // every range of the one against every range of the other, one of them written: equal or disjoint
+    auto clash = [&](uint64_t p, uint64_t q) { return p != q && p < q + bytes && q < p + bytes; };
+    for (uint64_t w : producer.stage_ptr) {
+        for (uint64_t q : consumer.ext)
+            if (clash(w, q)) return false;
+        for (uint64_t q : consumer.stage_ptr)
+            if (clash(w, q)) return false;
+    }
+    for (uint64_t w : consumer.stage_ptr)
+        for (uint64_t p : producer.ext)
+            if (clash(w, p)) return false;
+    bool reads_producer = false;
+    for (uint64_t q : consumer.ext) reads_producer = reads_producer || writer_of(producer, q) >= 0;
+    if (!reads_producer) return false;
+    ChainBuild c = producer;
+    const int shift = static_cast<int>(producer.stages.size());
+    // what an input pointer of the consumer becomes: the stored value of the producer's stage
+    // that wrote that memory last, or an input pointer of the joined kernel
+    std::vector<int> mapped;
+    for (uint64_t q : consumer.ext) {
+        const int w = writer_of(producer, q);
+        mapped.push_back(w >= 0 ? -(1 + w) : input_index(&c, q));
+    }
+    for (size_t s = 0; s < consumer.stages.size(); s++) {
+        ChainStage stage = consumer.stages[s];
+        for (int& from : stage.source) from = from >= 0 ? mapped[static_cast<size_t>(from)] : from - shift;
+        c.stages.push_back(std::move(stage));
+        c.stage_ptr.push_back(consumer.stage_ptr[s]);
+    }
+    if (c.stages.size() > static_cast<size_t>(kMaxChainStages) || c.ext.size() > static_cast<size_t>(kMaxChainInputs) ||
+        distinct_outputs(c) > static_cast<size_t>(kMaxChainOutputs))
+        return false;
+    *joined = std::move(c);
+    return true;
+}
+
+// The recording with producers joined into their consumers (see above); kernels for the new
+// chains are compiled here, at most kMaxNewChainKernels of them per graph -- a recording that
+// would need more stays as it is, as does one for which a compilation fails.
+constexpr size_t kMaxNewChainKernels = 16;
+int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, size_t* fused_away) {
+    const std::vector<RecNode>& nodes = *recorded;
+    struct Candidate {
+        size_t at;  // index into `out`
+        ChainBuild chain;
+        std::vector<Access> acc;
+        bool open;
+    };
+    std::vector<RecNode> out;
+    std::vector<char> dead;
+    std::vector<ChainBuild> chain_at;  // per entry of `out`: its chain if it has more than one stage
+    std::vector<Candidate> cands;
+    std::unordered_map<uint64_t, std::vector<uint32_t>> buckets;
+    size_t closed_below = 0;  // every candidate with a lower id is closed (a kernel with unknown memory use came by)
+    size_t joined_launches = 0;
+    std::vector<uint32_t> hits;
+    for (const RecNode& node : nodes) {
+        if (node.type == RecNode::Source) {
+            closed_below = cands.size();
+            out.push_back(node);
+            dead.push_back(0);
+            chain_at.emplace_back();
+            continue;
+        }
+        // open candidates this node conflicts with
+        hits.clear();
+        for (const Access& a : node.acc) {
+            if (a.end <= a.begin) continue;
+            for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) {
+                auto it = buckets.find(c);
+                if (it == buckets.end()) continue;
+                std::vector<uint32_t>& ids = it->second;
+                size_t kept = 0;
+                for (uint32_t id : ids) {
+                    if (id < closed_below || !cands[id].open) continue;  // dropped from the list
+                    ids[kept++] = id;
+                    for (const Access& b : cands[id].acc)
+                        if ((a.write || b.write) && a.begin < b.end && b.begin < a.end) {
+                            hits.push_back(id);
+                            break;
+                        }
+                }
+                ids.resize(kept);
+            }
+        }
+        std::sort(hits.begin(), hits.end());
+        hits.erase(std::unique(hits.begin(), hits.end()), hits.end());
+        const bool fusable = fusable_kernel(node);
+        ChainBuild chain;
+        if (fusable) chain = chain_of(node);
+        const uint64_t bytes = node.n * (fusable ? dtype_size(node.k->spec.dtype) : 1);
+        for (uint32_t id : hits) {
+            Candidate& p = cands[id];
+            p.open = false;  // joined or not, nothing later may be joined with it
+            if (!fusable) continue;
+            const RecNode& pn = out[p.at];
+            if (pn.k->spec.dtype != node.k->spec.dtype || pn.n != node.n || pn.head != node.head || pn.n_vec != node.n_vec ||
+                pn.k->spec.tuning.block_threads != node.k->spec.tuning.block_threads)
+                continue;
+            ChainBuild joined;
+            if (!join_chains(p.chain, chain, bytes, &joined)) continue;
+            chain = std::move(joined);
+            dead[p.at] = 1;
+            joined_launches++;
+        }
+        out.push_back(node);
+        dead.push_back(0);
+        chain_at.emplace_back();
+        if (!fusable) continue;
+        Candidate c;
+        c.at = out.size() - 1;
+        c.open = true;
+        for (uint64_t p : chain.ext) c.acc.push_back({p, p + bytes, false});
+        for (size_t s = 0; s < chain.stage_ptr.size(); s++)
+            if (writer_of(chain, chain.stage_ptr[s]) == static_cast<int>(s))
+                c.acc.push_back({chain.stage_ptr[s], chain.stage_ptr[s] + bytes, true});
+        for (const Access& a : c.acc)
+            for (uint64_t ch = a.begin >> kChunkShift; ch <= (a.end - 1) >> kChunkShift; ch++)
+                buckets[ch].push_back(static_cast<uint32_t>(cands.size()));
+        if (chain.stages.size() > 1) chain_at.back() = chain;
+        c.chain = std::move(chain);
+        cands.push_back(std::move(c));
+    }
+    if (joined_launches == 0) return CUSTOS_HIP_OK;
+    // kernels of the chains; the nodes take their final form
+    std::vector<RecNode> fused;
+    size_t compiled_here = 0;
+    for (size_t i = 0; i < out.size(); i++) {
+        if (dead[i]) continue;
+        RecNode node = out[i];
+        const ChainBuild& chain = chain_at[i];
+        if (chain.stages.size() > 1) {
+            std::vector<ChainStage> stages = chain.stages;
+            std::vector<uint64_t> outs;
+            for (size_t s = 0; s < stages.size(); s++) {
+                stages[s].out = -1;
+                if (writer_of(chain, chain.stage_ptr[s]) != static_cast<int>(s)) continue;
+                stages[s].out = static_cast<int>(outs.size());
+                outs.push_back(chain.stage_ptr[s]);
+            }
+            custos_hip_kernel* k = nullptr;
+            bool compiled = false;
+            Tuning tuning = node.k->spec.tuning;
+            tuning.unroll = 0;  // (only kernels whose vectors per thread were left open are joined)
+            const int32_t rc = chain_kernel(dev, node.k->spec.dtype, std::move(stages), static_cast<int>(chain.ext.size()),
+                                            static_cast<int>(outs.size()), tuning, &k, &compiled);
+            if (rc != CUSTOS_HIP_OK) return rc;
+            compiled_here += compiled;
+            if (compiled_here > kMaxNewChainKernels) return CUSTOS_HIP_ERR_TOO_LARGE;
+            const uint64_t bytes = node.n * dtype_size(node.k->spec.dtype);
+            node.k = k;
+            node.ptrs = chain.ext;
+            node.ptrs.insert(node.ptrs.end(), outs.begin(), outs.end());
+            node.acc.clear();
+            for (uint64_t p : chain.ext) node.acc.push_back({p, p + bytes, false});
+            for (uint64_t p : outs) node.acc.push_back({p, p + bytes, true});
+        }
+        fused.push_back(std::move(node));
+    }
+    *fused_away = nodes.size() - fused.size();
+    *recorded = std::move(fused);
+    return CUSTOS_HIP_OK;
+}
+
 bool batchable(const RecNode& n) {
     if (n.type != RecNode::Kernel || n.head != 0 || !n.k->fn_batched) return false;
     for (uint64_t p : n.ptrs)
@@ -574,6 +802,17 @@ int32_t instantiate(custos_hip_device* dev, custos_hip_graph* g, std::vector<std
 
 int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     std::vector<RecNode>& nodes = dev->recorded;
+    g->recorded = nodes.size();
+    g->signature = signature(nodes);
+    if (dev->fusing) {
+        // (a recording that cannot be joined -- too many new kernels, a kernel that does not
+        // compile -- is built as it was recorded)
+        const std::string error_before = dev->last_error;
+        if (fuse_producers(dev, &nodes, &g->fused_away) != CUSTOS_HIP_OK) {
+            g->fused_away = 0;
+            dev->last_error = error_before;
+        }
+    }
     const bool serial = dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN || dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN_BY_LEVEL;
     // The order of a chain only matters where a launch is large enough for the caches to matter;
     // a recording of small launches keeps the level order and the cheaper analysis.
@@ -587,10 +826,9 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     assign_levels(nodes, dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_PER_NODE || follow_recording);
     int max_level = -1;
     for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
-    g->recorded = nodes.size();
     g->levels = static_cast<size_t>(max_level + 1);
-    g->signature = signature(nodes);
-    g->built_with = {dev->batching ? 1u : 0u, static_cast<uint64_t>(dev->graph_edges), dev->direct_replay_max};
+    g->built_with = {dev->batching ? 1u : 0u, static_cast<uint64_t>(dev->graph_edges), dev->direct_replay_max,
+                     dev->fusing ? 1u : 0u};
 
     std::vector<std::vector<Planned>> plan;
     std::vector<uint64_t> host_table;
@@ -745,8 +983,8 @@ int32_t custos_hip_capture_end_reuse(custos_hip_device* dev, custos_hip_graph* p
     if (!dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the device is not recording");
     if (previous && std::find(dev->graphs.begin(), dev->graphs.end(), previous) == dev->graphs.end())
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "the previous graph does not belong to this device");
-    const std::array<uint64_t, 3> settings = {dev->batching ? 1u : 0u, static_cast<uint64_t>(dev->graph_edges),
-                                              dev->direct_replay_max};
+    const std::array<uint64_t, 4> settings = {dev->batching ? 1u : 0u, static_cast<uint64_t>(dev->graph_edges),
+                                              dev->direct_replay_max, dev->fusing ? 1u : 0u};
     if (previous && previous->built_with == settings && previous->signature == signature(dev->recorded)) {
         dev->capturing = false;
         dev->recorded.clear();
@@ -759,6 +997,12 @@ int32_t custos_hip_capture_end_reuse(custos_hip_device* dev, custos_hip_graph* p
 int32_t custos_hip_set_graph_batching(custos_hip_device* dev, int32_t enabled) {
     REQUIRE_DEV(dev);
     dev->batching = enabled != 0;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_graph_fusing(custos_hip_device* dev, int32_t enabled) {
+    REQUIRE_DEV(dev);
+    dev->fusing = enabled != 0;
     return CUSTOS_HIP_OK;
 }
 
@@ -806,6 +1050,12 @@ int32_t custos_hip_graph_launch(custos_hip_device* dev, custos_hip_graph* graph)
 int32_t custos_hip_graph_node_count(custos_hip_graph* graph, size_t* kernel_nodes) {
     if (!graph || !kernel_nodes) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
     *kernel_nodes = graph->kernel_nodes;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_fused_launches(custos_hip_graph* graph, size_t* launches) {
+    if (!graph || !launches) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    *launches = graph->fused_away;
     return CUSTOS_HIP_OK;
 }
 

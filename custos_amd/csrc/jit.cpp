@@ -208,6 +208,18 @@ static custos_hip_kernel* handle_for_values(custos_hip_kernel* owner, std::uniqu
     return sibling->second.get();
 }
 
+// Entry points of a freshly built module for many launches in one grid.
+static void find_merged_entries(custos_hip_kernel* k) {
+    if (hipModuleGetFunction(&k->fn_batched, k->module, (k->spec.name + "_batched").c_str()) != hipSuccess) {
+        (void)hipGetLastError();
+        k->fn_batched = nullptr;
+    }
+    if (hipModuleGetFunction(&k->fn_ragged, k->module, (k->spec.name + "_ragged").c_str()) != hipSuccess) {
+        (void)hipGetLastError();
+        k->fn_ragged = nullptr;
+    }
+}
+
 // Parses, looks the key up in the cache, compiles on a miss.
 //
 // Literal values: the first set of values an expression is seen with is compiled into the
@@ -250,18 +262,35 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
     rc = build_module(dev, k.get());
     if (rc != CUSTOS_HIP_OK) return rc;
     // further entry points of the module: many launches in one grid
-    if (hipModuleGetFunction(&k->fn_batched, k->module, (k->spec.name + "_batched").c_str()) != hipSuccess) {
-        (void)hipGetLastError();
-        k->fn_batched = nullptr;
-    }
-    if (hipModuleGetFunction(&k->fn_ragged, k->module, (k->spec.name + "_ragged").c_str()) != hipSuccess) {
-        (void)hipGetLastError();
-        k->fn_ragged = nullptr;
-    }
+    find_merged_entries(k.get());
     k->expr_src = src;
     for (int i = 0; i < n_markers; i++) k->markers.push_back(markers[i]);
     k->code = k.get();
     *out = k.get();
+    dev->cache[k->spec.hash].push_back(std::move(k));
+    return CUSTOS_HIP_OK;
+}
+
+int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs,
+                     const Tuning& tuning, custos_hip_kernel** out, bool* compiled) {
+    std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
+    ParseError err;
+    if (compiled) *compiled = false;
+    if (!build_chain_spec(dtype, std::move(stages), n_ext, n_outs, tuning, &k->spec, &err, /*with_source=*/false))
+        return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+    if (custos_hip_kernel* known = find_code(dev, k->spec)) {
+        dev->hits++;
+        *out = known;
+        return CUSTOS_HIP_OK;
+    }
+    if (!emit_kernel_source(&k->spec, &err)) return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+    int32_t rc = build_module(dev, k.get());
+    if (rc != CUSTOS_HIP_OK) return rc;
+    find_merged_entries(k.get());
+    k->expr_src = k->spec.chain_text;
+    k->code = k.get();
+    *out = k.get();
+    if (compiled) *compiled = true;
     dev->cache[k->spec.hash].push_back(std::move(k));
     return CUSTOS_HIP_OK;
 }
@@ -279,7 +308,7 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
                             CacheHint hint, unsigned long long working_set_bytes) {
-    const int n_operands = k->spec.kind == Kind::UnaryGrad ? 3 : k->spec.expr.n_vars + 1;
+    const int n_operands = kernel_pointers(k->spec);
     const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint, working_set_bytes);
     ResolvedShape r;
     const int direction = dev->tuning.direction;
@@ -433,6 +462,43 @@ int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const cha
     if (rc != CUSTOS_HIP_OK) return rc;
     if (code_size) *code_size = code.size();
     return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_chain_emit(int32_t dtype, const char* const* stage_srcs, const int32_t* stage_vars, int32_t n_stages,
+                              const int32_t* sources, const int32_t* stage_outs, int32_t n_inputs, int32_t n_outputs,
+                              char* buf, size_t cap, size_t* needed, size_t* code_size) {
+    if (!dtype_valid(dtype)) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown element type");
+    if (!stage_srcs || !stage_vars || !sources || !stage_outs || n_stages < 1 || n_stages > kMaxChainStages)
+        return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 8 stages are required");
+    std::vector<ChainStage> stages;
+    const int32_t* from = sources;
+    for (int32_t s = 0; s < n_stages; s++) {
+        if (!stage_srcs[s] || stage_vars[s] < 1 || stage_vars[s] > 4)
+            return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "a stage takes 1 to 4 variables");
+        std::vector<std::string> names;
+        for (int32_t v = 0; v < stage_vars[s]; v++) names.push_back("v" + std::to_string(v));
+        ChainStage stage;
+        ParseError err;
+        if (!parse_expr(stage_srcs[s], names, &stage.expr, &err))
+            return set_error(nullptr, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+        // (an expression need not use every variable: the stage still takes stage_vars[s] of them)
+        stage.expr.n_vars = stage_vars[s];
+        stage.source.assign(from, from + stage_vars[s]);
+        from += stage_vars[s];
+        stage.out = stage_outs[s];
+        stages.push_back(std::move(stage));
+    }
+    KernelSpec spec;
+    ParseError err;
+    if (!build_chain_spec(static_cast<DType>(dtype), std::move(stages), n_inputs, n_outputs, Tuning{}, &spec, &err))
+        return set_error(nullptr, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+    if (code_size) {
+        std::vector<char> code;
+        const int32_t rc = compile_to_code_object(nullptr, spec, "gfx950", &code);
+        if (rc != CUSTOS_HIP_OK) return rc;
+        *code_size = code.size();
+    }
+    return copy_out_string(spec.source, buf, cap, needed);
 }
 
 int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t* unroll,

@@ -225,15 +225,30 @@ struct KernelText {
     const int const_words;  // 8-byte words of a table row that hold the literal parameters
     std::string params;     // pointer parameters of the single-launch entry point
     std::string vec_ptrs;   // declarations of the vector views of the operands
-    std::string tile_args;  // the views custos_tile takes
+    std::string tile_args;  // the input views custos_tile takes
+    std::string out_views;  // the output views custos_tile takes
 
     explicit KernelText(const KernelSpec& spec)
         : k(spec),
-          n_in(spec.expr.n_vars),
-          n_ops(spec.kind == Kind::Apply ? spec.expr.n_vars : 3),
-          n_ptrs(spec.kind == Kind::Apply ? spec.expr.n_vars + 1 : 3),
-          const_words(static_cast<int>((spec.consts.bytes.size() + 7) / 8)) {
-        if (k.kind == Kind::Apply) {
+          n_in(spec.kind == Kind::Chain ? spec.n_ext : spec.expr.n_vars),
+          n_ops(spec.kind == Kind::Apply ? spec.expr.n_vars : spec.kind == Kind::Chain ? spec.n_ext : 3),
+          n_ptrs(kernel_pointers(spec)),
+          const_words(static_cast<int>((spec.consts.bytes.size() + 7) / 8)),
+          out_views("vout, ") {
+        if (k.kind == Kind::Chain) {
+            out_views.clear();
+            for (int i = 0; i < n_in; i++) {
+                const std::string id = std::to_string(i);
+                params += "const S* in" + id + ", ";
+                vec_ptrs += "    const vec_t* vin" + id + " = (const vec_t*)(in" + id + " + head);\n";
+            }
+            for (int j = 0; j < k.n_outs; j++) {
+                const std::string id = std::to_string(j);
+                params += std::string(j ? ", " : "") + "S* out" + id;
+                vec_ptrs += "    vec_t* vout" + id + " = (vec_t*)(out" + id + " + head);\n";
+                out_views += "vout" + id + ", ";
+            }
+        } else if (k.kind == Kind::Apply) {
             for (int i = 0; i < n_in; i++) {
                 const std::string id = std::to_string(i);
                 params += "const S* in" + id + ", ";
@@ -265,6 +280,7 @@ struct KernelText {
     // Per-element function on storage values: `custos_elem(in0.., [g])`.
     std::string elem_fn() const {
         std::string s;
+        if (k.kind == Kind::Chain) return chain_fn();
         if (k.kind == Kind::Apply) {
             s += "static __device__ __forceinline__ S custos_elem(";
             for (int i = 0; i < n_in; i++) s += std::string(i ? ", " : "") + "const S s" + std::to_string(i);
@@ -276,6 +292,85 @@ struct KernelText {
             s += "static __device__ __forceinline__ S custos_elem(const S s0, const S s1, const S s2 CUSTOS_KC_PARAM) {\n"
                  "    return custos_store(custos_grad(custos_load(s1), custos_load(s2), custos_expr(custos_load(s0) CUSTOS_KC_ARG)));\n}\n";
         }
+        return s;
+    }
+
+    // One element outside the vector body: `out[idx] = custos_elem(in0[idx], ..)`; a chain
+    // stores every output.
+    std::string scalar_stmt(const std::string& idx) const {
+        if (k.kind != Kind::Chain) return "out[" + idx + "] = custos_elem(" + list("in", "[" + idx + "]") + " CUSTOS_KC_ARG);";
+        std::string s = "{ S o[" + std::to_string(k.n_outs) + "]; custos_chain(" + list("in", "[" + idx + "]") + ", o);";
+        for (int j = 0; j < k.n_outs; j++) s += " out" + std::to_string(j) + "[" + idx + "] = o[" + std::to_string(j) + "];";
+        return s + " }";
+    }
+
+    // Chain: one function per stage, and `custos_chain(s0.., o)`, which evaluates the stages in
+    // order on storage values and leaves the value of every output pointer in `o`.  A stage that
+    // reads an earlier one takes its result as it was stored (rounded to the storage type).
+    std::string chain_fn() const {
+        std::string s;
+        for (size_t st = 0; st < k.stages.size(); st++) {
+            const ChainStage& stage = k.stages[st];
+            ConstPlan plan;
+            ParseError err;
+            std::string body;
+            // (checked when the spec was built)
+            (void)plan_constants(stage.expr, k.dtype, /*all_in_code=*/true, &plan, &err);
+            (void)emit_expr_body(stage.expr, k.dtype, plan, &body, &err);
+            s += "static __device__ __forceinline__ C custos_expr_s" + std::to_string(st) + "(";
+            for (int v = 0; v < stage.expr.n_vars; v++) s += std::string(v ? ", " : "") + "const C v" + std::to_string(v);
+            s += ") {\n" + body + "}\n";
+        }
+        s += "static __device__ __forceinline__ void custos_chain(";
+        for (int i = 0; i < n_in; i++) s += "const S s" + std::to_string(i) + ", ";
+        s += "S* o) {\n";
+        for (int i = 0; i < n_in; i++) s += "    const C e" + std::to_string(i) + " = custos_load(s" + std::to_string(i) + ");\n";
+        for (size_t st = 0; st < k.stages.size(); st++) {
+            const ChainStage& stage = k.stages[st];
+            const std::string id = std::to_string(st);
+            s += "    const S t" + id + " = custos_store(custos_expr_s" + id + "(";
+            for (size_t v = 0; v < stage.source.size(); v++) {
+                const int from = stage.source[v];
+                s += std::string(v ? ", " : "") + (from >= 0 ? "e" + std::to_string(from) : "r" + std::to_string(-from - 1));
+            }
+            s += "));\n    const C r" + id + " = custos_load(t" + id + ");\n    (void)r" + id + ";\n";
+            if (stage.out >= 0) s += "    o[" + std::to_string(stage.out) + "] = t" + id + ";\n";
+        }
+        s += "}\n";
+        return s;
+    }
+
+    // Chain: one tile, all loads before the first store, one store per output.
+    std::string chain_tile_fn(int unroll) const {
+        const std::string U = std::to_string(unroll);
+        std::string s = "static __device__ __forceinline__ void custos_tile" + U + "(";
+        for (int i = 0; i < n_in; i++) s += "const vec_t* vin" + std::to_string(i) + ", ";
+        for (int j = 0; j < k.n_outs; j++) s += "vec_t* vout" + std::to_string(j) + ", ";
+        s += "const u64 first, const u64 n_vec, const u64 mode) {\n";
+        s += "    const u64 left = (n_vec - first) * 16;\n";
+        s += "    const int bound = left > 0x7ffffff0ull ? 0x7ffffff0 : (int)left;\n";
+        for (int i = 0; i < n_in; i++)
+            s += "    const custos_rsrc rs" + std::to_string(i) + " = custos_make_rsrc(vin" + std::to_string(i) + " + first, bound);\n";
+        for (int j = 0; j < k.n_outs; j++)
+            s += "    const custos_rsrc rso" + std::to_string(j) + " = custos_make_rsrc(vout" + std::to_string(j) + " + first, bound);\n";
+        s += "    const unsigned int lane = threadIdx.x * 16u;\n";
+        for (int i = 0; i < n_in; i++) s += "    vec_t a" + std::to_string(i) + "[" + U + "];\n";
+        s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
+        for (int i = 0; i < n_in; i++) {
+            const std::string id = std::to_string(i);
+            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), mode & 2);\n";
+        }
+        s += "    }\n";
+        s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
+        for (int j = 0; j < k.n_outs; j++) s += "        vec_t r" + std::to_string(j) + ";\n";
+        s += "#pragma unroll\n        for (int k = 0; k < CUSTOS_VEC; k++) {\n";
+        s += "            S o[" + std::to_string(k.n_outs) + "];\n";
+        s += "            custos_chain(" + list("a", "[u][k]") + ", o);\n";
+        for (int j = 0; j < k.n_outs; j++) s += "            r" + std::to_string(j) + "[k] = o[" + std::to_string(j) + "];\n";
+        s += "        }\n";
+        for (int j = 0; j < k.n_outs; j++)
+            s += "        custos_st(rso" + std::to_string(j) + ", lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), r" + std::to_string(j) + ", mode);\n";
+        s += "    }\n}\n";
         return s;
     }
 
@@ -321,6 +416,7 @@ struct KernelText {
     // may be exactly one of the inputs: every lane has loaded all its vectors before its first
     // store.
     std::string tile_fn(int unroll) const {
+        if (k.kind == Kind::Chain) return chain_tile_fn(unroll);
         const std::string U = std::to_string(unroll);
         std::string ptr_params;
         for (int i = 0; i < n_ops; i++) {
@@ -370,15 +466,14 @@ struct KernelText {
         s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * U;\n";
         s += "    const u64 n_tiles = " + n_tiles_expr() + ";\n";
         s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {\n";
-        s += tile_call("        ", tile_args + "vout, (rev ? n_tiles - 1 - tile : tile) * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
+        s += tile_call("        ", tile_args + out_views + "(rev ? n_tiles - 1 - tile : tile) * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
         s += "    }\n";
         // Elements outside the 16-byte aligned body: `head` leading ones and the
         // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
         s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
         s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BLOCK;\n";
-        s += "    if (gid < head) out[gid] = custos_elem(" + list("in", "[gid]") + " CUSTOS_KC_ARG);\n";
-        s += "    for (u64 i = head + n_vec * CUSTOS_VEC + gid; i < n; i += n_threads) out[i] = custos_elem(" +
-             list("in", "[i]") + " CUSTOS_KC_ARG);\n";
+        s += "    if (gid < head) " + scalar_stmt("gid") + "\n";
+        s += "    for (u64 i = head + n_vec * CUSTOS_VEC + gid; i < n; i += n_threads) " + scalar_stmt("i") + "\n";
         s += "}\n";
         return s;
     }
@@ -394,7 +489,12 @@ struct KernelText {
     // operand pointers of a merged launch, read from the table row `ptrs`
     std::string table_operands() const {
         std::string s;
-        if (k.kind == Kind::Apply) {
+        if (k.kind == Kind::Chain) {
+            for (int i = 0; i < n_in; i++)
+                s += "    const S* in" + std::to_string(i) + " = (const S*)ptrs[" + std::to_string(i) + "];\n";
+            for (int j = 0; j < k.n_outs; j++)
+                s += "    S* out" + std::to_string(j) + " = (S*)ptrs[" + std::to_string(n_in + j) + "];\n";
+        } else if (k.kind == Kind::Apply) {
             for (int i = 0; i < n_in; i++)
                 s += "    const S* in" + std::to_string(i) + " = (const S*)ptrs[" + std::to_string(i) + "];\n";
             s += "    S* out = (S*)ptrs[" + std::to_string(n_in) + "];\n";
@@ -422,10 +522,9 @@ struct KernelText {
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
-        s += tile_call("    ", tile_args + "vout, tile * (u64)CUSTOS_BLOCK * U, n_vec, mode CUSTOS_KC_ARG");
+        s += tile_call("    ", tile_args + out_views + "tile * (u64)CUSTOS_BLOCK * U, n_vec, mode CUSTOS_KC_ARG");
         s += "    if (tile == tiles_per_seg - 1)\n";
-        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
-             list("in", "[i]") + " CUSTOS_KC_ARG);\n";
+        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) " + scalar_stmt("i") + "\n";
         s += "    (void)head;\n}\n";
         return s;
     }
@@ -450,10 +549,9 @@ struct KernelText {
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
-        s += tile_call("    ", tile_args + "vout, tile * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
+        s += tile_call("    ", tile_args + out_views + "tile * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
         s += "    if (tile == n_tiles - 1)\n";
-        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) out[i] = custos_elem(" +
-             list("in", "[i]") + " CUSTOS_KC_ARG);\n";
+        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) " + scalar_stmt("i") + "\n";
         s += "    (void)head;\n}\n";
         return s;
     }
@@ -509,10 +607,20 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
 bool emit_kernel_source(KernelSpec* spec, ParseError* err) {
     KernelSpec& k = *spec;
     std::string body;
-    if (!emit_expr_body(k.expr, k.dtype, k.consts, &body, err)) return false;
+    if (k.kind == Kind::Chain) {
+        // (the stage functions are emitted by KernelText; here only what cannot be compiled is found)
+        for (const ChainStage& stage : k.stages) {
+            ConstPlan plan;
+            std::string unused;
+            if (!plan_constants(stage.expr, k.dtype, /*all_in_code=*/true, &plan, err)) return false;
+            if (!emit_expr_body(stage.expr, k.dtype, plan, &unused, err)) return false;
+        }
+    } else if (!emit_expr_body(k.expr, k.dtype, k.consts, &body, err)) {
+        return false;
+    }
 
     std::string s;
-    s += "// generated by custos-hip: " + to_cl_source(k.expr, k.markers, &k.consts) + "\n";
+    s += "// generated by custos-hip: " + (k.kind == Kind::Chain ? k.chain_text : to_cl_source(k.expr, k.markers, &k.consts)) + "\n";
     s += "#define CUSTOS_BLOCK " + std::to_string(k.tuning.block_threads) + "\n";
     s += "#define CUSTOS_VEC " + std::to_string(k.vec_elems) + "\n";
     s += prelude(k.dtype, k.vec_elems, k.consts.n_params);
@@ -541,7 +649,7 @@ static __device__ __forceinline__ void custos_st(const custos_rsrc rs, const uns
     }
 }
 )";
-    s += expr_fn(k, body);
+    if (k.kind != Kind::Chain) s += expr_fn(k, body);
 
     const KernelText text(k);
     s += text.elem_fn();
@@ -554,11 +662,85 @@ static __device__ __forceinline__ void custos_st(const custos_rsrc rs, const uns
     return true;
 }
 
+int kernel_pointers(const KernelSpec& k) {
+    if (k.kind == Kind::Chain) return k.n_ext + k.n_outs;
+    return k.kind == Kind::UnaryGrad ? 3 : k.expr.n_vars + 1;
+}
+
+bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs, const Tuning& tuning,
+                      KernelSpec* out, ParseError* err, bool with_source) {
+    KernelSpec k;
+    k.kind = Kind::Chain;
+    k.dtype = dtype;
+    k.tuning = tuning;
+    k.auto_unroll = tuning.unroll <= 0;
+    if (k.auto_unroll) k.tuning.unroll = 2;
+    k.tuning.nontemporal = -1;
+    k.tuning.direction = 0;
+    k.n_ext = n_ext;
+    k.n_outs = n_outs;
+    if (stages.empty() || stages.size() > static_cast<size_t>(kMaxChainStages) || n_ext < 1 || n_ext > kMaxChainInputs ||
+        n_outs < 1 || n_outs > kMaxChainOutputs) {
+        err->code = CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+        err->message = "a chain kernel takes 1 to 8 stages, 1 to 8 inputs and 1 to 6 outputs";
+        return false;
+    }
+    // key and text: every stage's expression (literal values included), where its variables come
+    // from and where its value goes
+    uint64_t h = fnv1a64("custos-chain", 12);
+    for (size_t st = 0; st < stages.size(); st++) {
+        const ChainStage& stage = stages[st];
+        if (static_cast<int>(stage.source.size()) != stage.expr.n_vars || stage.out >= n_outs) {
+            err->code = CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+            err->message = "malformed chain stage";
+            return false;
+        }
+        ConstPlan plan;
+        if (!plan_constants(stage.expr, dtype, /*all_in_code=*/true, &plan, err)) return false;
+        uint64_t hs;
+        std::vector<uint64_t> literals;
+        if (!hash_expr(stage.expr, dtype, plan, &hs, err, &literals)) return false;
+        h = fnv1a64(&hs, sizeof hs, h);
+        std::vector<std::string> names;
+        for (int from : stage.source) {
+            if (from >= n_ext || -from - 1 >= static_cast<int>(st)) {
+                err->code = CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+                err->message = "a chain stage reads an input or a stage that does not exist";
+                return false;
+            }
+            h = fnv1a64(&from, sizeof from, h);
+            names.push_back(from >= 0 ? "x" + std::to_string(from) : "s" + std::to_string(-from - 1));
+        }
+        h = fnv1a64(&stage.out, sizeof stage.out, h);
+        for (const Node& n : stage.expr.nodes) k.n_literals += n.op == Op::Const;
+        k.code_literals.insert(k.code_literals.end(), literals.begin(), literals.end());
+        k.chain_text += "s" + std::to_string(st) + " = " + to_cl_source(stage.expr, names) +
+                        (stage.out >= 0 ? " -> out" + std::to_string(stage.out) : std::string()) + "; ";
+    }
+    int32_t tail[7] = {static_cast<int32_t>(Kind::Chain), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
+                       k.tuning.blocks_per_cu, n_ext, n_outs, 16 /* template version */};
+    k.hash = fnv1a64(tail, sizeof tail, h);
+    k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
+    k.stages = std::move(stages);
+    {
+        static const char* const dtype_names[] = {"f32", "f64", "i32", "i64", "f16", "bf16", "u8", "i8", "i16", "u16", "u32", "u64",
+                                                  "f16n", "bf16n"};
+        char hex[17];
+        std::snprintf(hex, sizeof hex, "%016llx", static_cast<unsigned long long>(k.hash));
+        k.name = std::string("custos_chain_") + dtype_names[static_cast<int>(dtype)] + "_" + hex;
+    }
+    if (with_source && !emit_kernel_source(&k, err)) return false;
+    *out = std::move(k);
+    return true;
+}
+
 bool same_code(const KernelSpec& a, const KernelSpec& b) {
     if (a.kind != b.kind || a.dtype != b.dtype || a.hash != b.hash) return false;
     if (a.tuning.block_threads != b.tuning.block_threads || a.tuning.unroll != b.tuning.unroll ||
         a.tuning.blocks_per_cu != b.tuning.blocks_per_cu || a.auto_unroll != b.auto_unroll)
         return false;
+    // (a chain's text spells its stages, their wiring and every literal)
+    if (a.kind == Kind::Chain) return a.n_ext == b.n_ext && a.n_outs == b.n_outs && a.chain_text == b.chain_text;
     if (a.expr.n_vars != b.expr.n_vars || a.expr.root != b.expr.root || a.expr.nodes.size() != b.expr.nodes.size()) return false;
     for (size_t i = 0; i < a.expr.nodes.size(); i++) {
         const Node& x = a.expr.nodes[i];

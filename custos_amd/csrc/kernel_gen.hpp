@@ -15,7 +15,12 @@
 
 namespace custos_hip {
 
-enum class Kind : int32_t { Apply = 0, UnaryGrad = 1, Source = 2 /* caller-written kernel source */ };
+enum class Kind : int32_t {
+    Apply = 0,
+    UnaryGrad = 1,
+    Source = 2,  // caller-written kernel source
+    Chain = 3,   // several apply expressions in one kernel, every one with its own output (made when a graph is built)
+};
 
 struct Tuning {
     // Launch shape of the generated kernels.  Workgroups of 64 or 128 threads
@@ -73,10 +78,26 @@ inline uint64_t launch_mode(int unroll, int nontemporal, bool rev) {
 // (`nontemporal` and `direction` as in custos_hip_tuning).
 Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int nontemporal, int direction);
 
+// One expression of a chain kernel.  A chain stands for apply launches that were recorded one
+// after the other, the later ones reading what the earlier ones wrote: every stage computes its
+// expression, stores the result where its launch stored it, and a later stage that read that
+// memory takes the value as it was stored (rounded to the storage type) from a register.
+struct ChainStage {
+    Expr expr;
+    std::vector<int> source;  // per variable of `expr`: index of an input pointer of the kernel, or
+                              // -(1 + s) for the stored value of stage s
+    int out = -1;             // which output pointer of the kernel receives the value; -1: none, a
+                              // later stage writes the same memory
+};
+constexpr int kMaxChainStages = 8, kMaxChainInputs = 8, kMaxChainOutputs = 6;
+
 struct KernelSpec {
     Kind kind = Kind::Apply;
     DType dtype = DType::F32;
-    Expr expr;
+    Expr expr;                       // Apply, UnaryGrad
+    std::vector<ChainStage> stages;  // Chain
+    int n_ext = 0, n_outs = 0;       // Chain: input and output pointers (inputs first)
+    std::string chain_text;          // Chain: the stages spelt out, literal values included
     Tuning tuning;             // as compiled: workgroup size, grid kind, most vectors per thread
     bool auto_unroll = false;  // the caller left the vectors per thread open: the kernel holds the
                                // tile functions for 2 and for 1, and every launch picks one
@@ -99,6 +120,12 @@ struct KernelSpec {
 bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
                        const std::vector<std::string>& markers, const Tuning& tuning,
                        bool literals_in_code, KernelSpec* out, ParseError* err, bool with_source = true);
+// The same for a chain kernel (all literals in the code).
+bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs, const Tuning& tuning,
+                      KernelSpec* out, ParseError* err, bool with_source = true);
+// Pointer parameters of a generated kernel's single-launch entry point (= the width of a table
+// row of a merged launch, before the literal parameters).
+int kernel_pointers(const KernelSpec& k);
 // Generates `k->source` (which also finds node / element type combinations that cannot be
 // compiled, such as a transcendental node over integers).
 bool emit_kernel_source(KernelSpec* k, ParseError* err);

@@ -64,7 +64,8 @@ struct custos_hip_graph {
     // what the graph was built from: the recording, word by word, and the device's graph settings
     // (merging, edge mode, direct replay limit) -- see custos_hip_capture_end_reuse
     std::vector<uint64_t> signature;
-    std::array<uint64_t, 3> built_with{};
+    std::array<uint64_t, 4> built_with{};
+    size_t fused_away = 0;    // recorded launches that became stages of a later launch's kernel
     // how long the last wait took that waited for one launch of this graph and nothing else
     uint64_t last_wait_ns = 0;
 };
@@ -163,6 +164,7 @@ struct custos_hip_device {
     std::array<bool, 16> write_slot_used{};
     unsigned long long launch_parity = 0;  // direction of the last launch that alternates
     bool batching = true;            // merge equal independent launches of a level into one grid
+    bool fusing = true;              // a recorded apply launch is joined with the apply launches that read what it wrote
     std::vector<RecNode> recorded;
     uint64_t compiles = 0, hits = 0, disk_hits = 0;
     std::string last_error;
@@ -236,6 +238,9 @@ struct ResolvedShape {
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
                             CacheHint hint = CacheHint::Unknown, unsigned long long working_set_bytes = 0);
 
+// jit.cpp: the kernel for a chain of apply expressions (compiled on first use, then cached).
+int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs,
+                     const Tuning& tuning, custos_hip_kernel** out, bool* compiled);
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
 // Workgroups of a single launch of `k` over n_vec vectors and n elements with `unroll` vectors per thread.

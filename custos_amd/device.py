@@ -104,6 +104,13 @@ class Graph:
         self.device._check(self.device.lib.custos_hip_graph_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
         return a.value, b.value, c.value
 
+    @property
+    def fused_launches(self) -> int:
+        """Recorded launches that became part of a later launch's kernel."""
+        n = C.c_size_t(0)
+        self.device._check(self.device.lib.custos_hip_graph_fused_launches(self.handle, C.byref(n)))
+        return n.value
+
     def edge_count(self) -> int:
         """Dependency edges of the instantiated graph, joins included (0 for a directly replayed chain)."""
         e = C.c_size_t(0)
@@ -354,6 +361,10 @@ class HIP:
 
     def set_graph_batching(self, enabled: bool) -> None:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
+
+    def set_graph_fusing(self, enabled: bool) -> None:
+        """Whether a graph build joins recorded apply launches with the apply launches that read their output."""
+        self._check(self.lib.custos_hip_set_graph_fusing(self.handle, 1 if enabled else 0))
 
     def launch_hint_stats(self):
         """(not part of a chain, chain that stays in the memory-side cache, chain that streams) counts of

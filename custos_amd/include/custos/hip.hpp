@@ -261,6 +261,9 @@ class HIP : public Device<HIP<Mods>, Mods> {
     void set_graph_direct_replay(int32_t max_nodes) { check(custos_hip_set_graph_direct_replay(dev_, max_nodes)); }
     // How built graphs order their nodes: CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS, _PER_NODE or _CHAIN.
     void set_graph_edges(int32_t mode) { check(custos_hip_set_graph_edges(dev_, mode)); }
+    // Whether a lazy run joins recorded apply launches with the apply launches that read their
+    // output into one kernel (default: yes; every buffer still receives the same values).
+    void set_graph_fusing(bool enabled) { check(custos_hip_set_graph_fusing(dev_, enabled ? 1 : 0)); }
 
     custos_hip_kernel* compile(int32_t kind, int32_t dtype, const std::string& src,
                                std::initializer_list<const char*> markers) {

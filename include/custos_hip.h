@@ -390,6 +390,33 @@ int32_t custos_hip_capture_end_reuse(custos_hip_device *dev, custos_hip_graph *p
 /* Switches the merging of equal independent launches off (0) or on (default):
  * with it off every recorded launch becomes its own kernel node. */
 int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
+/* Switches the joining of producers with their consumers off (0) or on (default).  With it on, a
+ * recorded apply launch whose output a later recorded apply launch reads element for element
+ * (same address, length and element type) becomes one kernel with that launch: both expressions
+ * are evaluated per element, both results are stored where the two launches stored them, and
+ * the second expression takes the first result -- as it was stored, rounded to the storage type
+ * -- from a register.  `t = a * b; u = t + c; y = f(u)` replays as one launch that reads a, b, c
+ * and writes t, u, y.  Every buffer receives exactly what the separate launches gave it.  Only
+ * launches whose address ranges are pairwise equal or disjoint are joined, and only if nothing
+ * recorded between them touches what the earlier one reads or writes; a joined launch is
+ * producer and consumer in turn (up to 8 expressions, 8 inputs and 6 outputs per kernel).  The
+ * kernels are compiled when the graph is built (at most 16 new ones per graph; a recording that
+ * would need more is built as recorded).  No counterpart in the reference, whose captured
+ * graphs replay launch by launch (src/devices/cuda/lazy.rs:31-49). */
+int32_t custos_hip_set_graph_fusing(custos_hip_device *dev, int32_t enabled);
+/* Recorded launches of a built graph that became part of a later launch's kernel. */
+int32_t custos_hip_graph_fused_launches(custos_hip_graph *graph, size_t *launches);
+/* Host-only: the source of the kernel that joins `n_stages` expressions (for tests and
+ * inspection; nothing is launched).  `stage_srcs[s]` is an expression over the variables v0 ..
+ * v{stage_vars[s]-1}; `sources` lists, stage after stage, where each variable comes from: the
+ * index of an input pointer (0 .. n_inputs-1), or -(1 + t) for the stored value of stage t < s;
+ * `stage_outs[s]` is the output pointer (0 .. n_outputs-1) that receives the stage's value, or -1
+ * if a later stage writes the same memory.  With `code_size` the source is also compiled for
+ * gfx950 and the size of the code object returned. */
+int32_t custos_hip_chain_emit(int32_t dtype, const char *const *stage_srcs, const int32_t *stage_vars,
+                              int32_t n_stages, const int32_t *sources, const int32_t *stage_outs,
+                              int32_t n_inputs, int32_t n_outputs, char *buf, size_t cap,
+                              size_t *needed, size_t *code_size);
 /* A recording that comes out as a plain chain (every dependency level one node, or any
  * recording under CUSTOS_HIP_GRAPH_EDGES_CHAIN) of at most `max_nodes` nodes is replayed by
  * issuing its nodes on the compute stream instead of launching an instantiated graph: for a

@@ -36,14 +36,26 @@ TEST_CASE(hip_lazy_run_replays_one_graph) {
         CHECK_VEC_EQ(lhs.read(), (std::vector<int32_t>{6, 24, 54, 96, 150, 216}));
     }
     CHECK_EQ(device.graph_builds(), uint64_t(1));      // recorded once, replayed ten times
-    CHECK_EQ(device.graph_kernel_nodes(), size_t(3));  // and every op ran once per run, not twice
+    // every op ran once per run, not twice; the three launches, each reading what the one before
+    // wrote, are joined into one kernel
+    CHECK_EQ(device.graph_kernel_nodes(), size_t(1));
     // a new operation invalidates the graph: the next run records again
     auto extra = device.apply_fn(out, [](auto x) { return x.add(1); });
     lhs.write({1, 2, 3, 4, 5, 6});
     rhs.write({1, 2, 3, 4, 5, 6});
     device.run();
     CHECK_EQ(device.graph_builds(), uint64_t(2));
-    CHECK_EQ(device.graph_kernel_nodes(), size_t(4));
+    CHECK_EQ(device.graph_kernel_nodes(), size_t(1));
+    // as recorded: one node per operation
+    device.set_graph_fusing(false);
+    auto more = device.apply_fn(out, [](auto x) { return x.add(2); });
+    lhs.write({1, 2, 3, 4, 5, 6});
+    rhs.write({1, 2, 3, 4, 5, 6});
+    device.run();
+    CHECK_EQ(device.graph_builds(), uint64_t(3));
+    CHECK_EQ(device.graph_kernel_nodes(), size_t(5));
+    CHECK_VEC_EQ(more.replace().read(), (std::vector<int32_t>{4, 6, 8, 10, 12, 14}));
+    CHECK_VEC_EQ(lhs.read(), (std::vector<int32_t>{6, 24, 54, 96, 150, 216}));
     CHECK_VEC_EQ(extra.replace().read(), (std::vector<int32_t>{3, 5, 7, 9, 11, 13}));
 }
 
@@ -342,6 +354,7 @@ TEST_CASE(hip_graph_orders_reuse_and_fill) {
     CHECK_EQ(custos_hip_source_compile(dev, halve, "halve", &scale), 0);
     CHECK_EQ(custos_hip_set_graph_verify(dev, 1), 0);
     CHECK_EQ(custos_hip_set_graph_direct_replay(dev, 0), 0);
+    CHECK_EQ(custos_hip_set_graph_fusing(dev, 0), 0);  // the nodes as recorded (joined, a's and b's launches would be three kernels)
     std::vector<std::vector<float>> results;
     const size_t want_edges[3] = {11, 8, 8};
     for (int32_t mode : {CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS, CUSTOS_HIP_GRAPH_EDGES_PER_NODE, CUSTOS_HIP_GRAPH_EDGES_CHAIN}) {

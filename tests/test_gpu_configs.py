@@ -112,16 +112,20 @@ def test_c5_graph_replay(hip, oracle):
             hip.fused_apply_fn(u[i], unary, out=y[i])
         return hip.capture_end()
 
-    for batching in (True, False):
+    for batching, fusing in ((True, True), (True, False), (False, True), (False, False)):
         hip.set_graph_batching(batching)
+        hip.set_graph_fusing(fusing)
         try:
             graph = record()
         finally:
             hip.set_graph_batching(True)
+            hip.set_graph_fusing(True)
         recorded, kernel_nodes, levels = graph.stats()
-        assert (recorded, levels) == (3 * nbuf, 3)
+        # the three launches of a buffer become one kernel that reads a, b, c and writes t, u, y
+        assert (recorded, levels, graph.fused_launches) == ((3 * nbuf, 1, 2 * nbuf) if fusing else (3 * nbuf, 3, 0))
         # the 64 independent chains run side by side; with batching every level is ONE launch
-        assert kernel_nodes == (3 if batching else 3 * nbuf)
+        per_buffer = 1 if fusing else 3
+        assert kernel_nodes == (per_buffer if batching else per_buffer * nbuf)
         # nothing ran while recording: outputs are still the zeros of alloc / of the last clear
         assert not y[0].read().any()
         for replay in range(3):
@@ -129,10 +133,13 @@ def test_c5_graph_replay(hip, oracle):
             hip.sync()
             for i in (0, 1, nbuf // 2, nbuf - 1):
                 tt, uu, yy = oracle.c5_graph(a[i], b[i], c[i])
-                assert_bits_equal(t[i].read(), tt)
-                assert_bits_equal(u[i].read(), uu)
-                assert_bits_equal(y[i].read(), yy, f"batching={batching} replay {replay} buffer {i}")
+                what = f"batching={batching} fusing={fusing} replay {replay} buffer {i}"
+                assert_bits_equal(t[i].read(), tt, what)
+                assert_bits_equal(u[i].read(), uu, what)
+                assert_bits_equal(y[i].read(), yy, what)
             for i in range(nbuf):
+                t[i].clear()
+                u[i].clear()
                 y[i].clear()
             hip.sync()
         graph.destroy()
@@ -234,8 +241,9 @@ def test_c4_full_size_properties(hip, oracle):
 
 
 def test_c5_full_size_graph(hip, oracle):
-    """configs[4] at its full shape, 1024 buffers of 4096 f32: three kernel nodes for 3072
-    recorded launches, 100 replays, bit-exact against the oracle after the first and the last."""
+    """configs[4] at its full shape, 1024 buffers of 4096 f32: ONE kernel node for 3072 recorded
+    launches (the three launches of a buffer joined, the 1024 joined launches merged), 100 replays,
+    every buffer bit-exact against the oracle after the first and the last."""
     nbuf, m = 1024, 4096
     a = synth.uniform_f32(1, nbuf * m, 0, 1)
     b = synth.uniform_f32(2, nbuf * m, 0, 1)
@@ -249,13 +257,16 @@ def test_c5_full_size_graph(hip, oracle):
         hip.apply_fn2(T.slice(s.start, s.stop), Cc.slice(s.start, s.stop), lambda p, q: p.add(q), out=U.slice(s.start, s.stop))
         hip.fused_apply_fn(U.slice(s.start, s.stop), [lambda v: v.abs().sqrt(), lambda v: v.mul(0.3)], out=Y.slice(s.start, s.stop))
     g = hip.capture_end()
-    assert g.stats() == (3 * nbuf, 3, 3)
-    _, _, want = oracle.c5_graph(a, b, c)
+    assert g.stats() == (3 * nbuf, 1, 1) and g.fused_launches == 2 * nbuf
+    want_t, want_u, want = oracle.c5_graph(a, b, c)
     for replay in range(100):
         if replay in (0, 99):
-            Y.clear()
+            for buf in (T, U, Y):
+                buf.clear()
         g.launch()
         if replay in (0, 99):
             hip.sync()
+            assert_bits_equal(T.read(), want_t, f"t, replay {replay}")
+            assert_bits_equal(U.read(), want_u, f"u, replay {replay}")
             assert_bits_equal(Y.read(), want, f"replay {replay}")
     g.destroy()

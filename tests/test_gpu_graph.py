@@ -32,7 +32,9 @@ def test_lazy_run_reference_vectors(hip):
     assert rhs.read().tolist() == [1, 2, 3, 4, 5, 6]
     graph = hip.capture_end()
     assert not hip.is_capturing()
-    assert graph.kernel_nodes == 3
+    # every launch reads what the one before wrote, and writes an operand of an earlier one in
+    # place: the three are joined into one kernel (each lane loads before it stores)
+    assert graph.kernel_nodes == 1 and graph.fused_launches == 2
     graph.launch()
     hip.sync()
     assert out.read().tolist() == [2, 4, 6, 8, 10, 12]
@@ -50,7 +52,7 @@ def test_lazy_run_multiple_times(hip):
     out.clear()              # a clear is recorded as a kernel node, too
     _add_add_mul(hip, lhs, rhs, out)
     graph = hip.capture_end()
-    assert graph.kernel_nodes == 4
+    assert graph.kernel_nodes == 2      # the clear, and the three launches joined
     for _ in range(10):
         lhs.write([1, 2, 3, 4, 5, 6])
         rhs.write([1, 2, 3, 4, 5, 6])
@@ -216,6 +218,7 @@ def checked_graphs(hip):
     yield hip
     hip.set_graph_verify(False)
     hip.set_graph_edges(capi.GRAPH_EDGES_CHAIN)
+    hip.set_graph_fusing(True)
 
 
 EDGE_MODES = {"level joins": capi.GRAPH_EDGES_LEVEL_JOINS, "per node": capi.GRAPH_EDGES_PER_NODE, "chain": capi.GRAPH_EDGES_CHAIN,
@@ -236,6 +239,7 @@ def test_recorded_dependencies_random(checked_graphs, oracle, edges):
     n = 2048
     fns1 = [lambda v: v.mul(1.25).add(0.5), lambda v: v.neg().max(-3.0), lambda v: v.abs().sqrt(), lambda v: v.mul(v).min(9.0)]
     fns2 = [lambda p, q: p.add(q), lambda p, q: p.mul(q).sub(0.125), lambda p, q: p.max(q)]
+    fused_launches = 0
     for trial in range(int(os.environ.get("CUSTOS_RANDOM_PROGRAMS", "6"))):   # more for a longer run
         nbuf = 6
         init = [synth.uniform_f32(trial * 10 + i, n, -2, 2) for i in range(nbuf)]
@@ -279,22 +283,33 @@ def test_recorded_dependencies_random(checked_graphs, oracle, edges):
         run(eager)
         hip.sync()
         want = [b.read() for b in eager]
-        lazy = [hip.buffer(x) for x in init]
-        hip.capture_begin()
-        run(lazy)
-        g = hip.capture_end()
-        for b, x in zip(lazy, init):
-            assert_bits_equal(b.read(), x, "nothing may run while recording")
-        g.launch()
+        run(eager)          # a second replay continues from the first one's results, like a second eager run
         hip.sync()
-        for i, b in enumerate(lazy):
-            assert_bits_equal(b.read(), want[i], f"trial {trial} buffer {i} (levels {g.stats()})")
-        g.launch()          # a second replay continues from the first one's results, like a second eager run
-        run(eager)
-        hip.sync()
-        for i, b in enumerate(lazy):
-            assert_bits_equal(b.read(), eager[i].read(), f"trial {trial} second replay, buffer {i}")
-        g.destroy()
+        want_twice = [b.read() for b in eager]
+        # once with producers joined into their consumers (the default), once as recorded
+        for fusing in (True, False):
+            lazy = [hip.buffer(x) for x in init]
+            hip.set_graph_fusing(fusing)
+            try:
+                hip.capture_begin()
+                run(lazy)
+                g = hip.capture_end()
+            finally:
+                hip.set_graph_fusing(True)
+            fused_launches += g.fused_launches
+            assert fusing or g.fused_launches == 0
+            for b, x in zip(lazy, init):
+                assert_bits_equal(b.read(), x, "nothing may run while recording")
+            g.launch()
+            hip.sync()
+            for i, b in enumerate(lazy):
+                assert_bits_equal(b.read(), want[i], f"trial {trial} fusing {fusing} buffer {i} (levels {g.stats()})")
+            g.launch()
+            hip.sync()
+            for i, b in enumerate(lazy):
+                assert_bits_equal(b.read(), want_twice[i], f"trial {trial} fusing {fusing} second replay, buffer {i}")
+            g.destroy()
+    assert fused_launches > 0, "no trial joined a producer with its consumer"
 
 
 def test_per_node_edges_let_independent_chains_run_apart(checked_graphs, oracle):
@@ -304,6 +319,7 @@ def test_per_node_edges_let_independent_chains_run_apart(checked_graphs, oracle)
     than level joins need); as one chain the nodes follow each other in level order.  The same
     bits in every mode, replay after replay."""
     hip = checked_graphs
+    hip.set_graph_fusing(False)         # this test is about the nodes as recorded (joined, each chain would be one kernel)
     n = 30011
     x, y = synth.uniform_f32(31, n, -2, 2), synth.uniform_f32(32, n, -2, 2)
     f = lambda v: v.mul(1.5).sub(0.25)
@@ -423,17 +439,19 @@ def test_ordering_check_accepts_merged_and_fenced_graphs(checked_graphs):
     n, count = 4096, 64
     xs = [hip.buffer(synth.uniform_f32(100 + i, n, 0, 1)) for i in range(count)]
     ts = [hip.alloc(n) for _ in range(count)]
-    for mode in EDGE_MODES.values():
-        hip.set_graph_edges(mode)
-        hip.capture_begin()
-        for x, t in zip(xs, ts):
-            hip.apply_fn(x, lambda v: v.mul(2.0), out=t)
-            hip.apply_fn(t, lambda v: v.add(1.0), out=x)
-        g = hip.capture_end()
-        assert g.stats() == (2 * count, 2, 2)
-        g.launch()
-        hip.sync()
-        g.destroy()
+    for fusing in (False, True):
+        hip.set_graph_fusing(fusing)
+        for mode in EDGE_MODES.values():
+            hip.set_graph_edges(mode)
+            hip.capture_begin()
+            for x, t in zip(xs, ts):
+                hip.apply_fn(x, lambda v: v.mul(2.0), out=t)
+                hip.apply_fn(t, lambda v: v.add(1.0), out=x)
+            g = hip.capture_end()
+            assert g.stats() == ((2 * count, 1, 1) if fusing else (2 * count, 2, 2))
+            g.launch()
+            hip.sync()
+            g.destroy()
 
 
 def test_a_repeated_recording_reuses_its_graph(hip, oracle):
@@ -736,6 +754,7 @@ def test_waits_follow_the_work(hip):
     bufs = [hip.alloc(n) for _ in range(2)]
     k = hip.compile(capi.KIND_APPLY, "f32", "((x * 1.0001) + 0.25)", ("x",))
     hip.set_graph_direct_replay(0)
+    hip.set_graph_fusing(False)                   # 48 launches that take their time (joined they would be six)
     try:
         hip.capture_begin()
         src = x
@@ -749,6 +768,7 @@ def test_waits_follow_the_work(hip):
         short_graph = hip.capture_end()
     finally:
         hip.set_graph_direct_replay(4)
+        hip.set_graph_fusing(True)
     long_graph.launch()
     hip.sync()
     hip.timer_begin()

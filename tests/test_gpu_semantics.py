@@ -1044,6 +1044,7 @@ def test_launch_shape_follows_the_launches_around_it(oracle):
         assert_bits_equal(q.read(), ((((wantb * wb) * wb) * wb) * wb))
         s2 = s2b
         # in a recorded graph the first kernel counts as part of the chain too: a later level reads its output
+        dev.set_graph_fusing(False)          # (joined, the two launches would be one node)
         dev.capture_begin()
         dev.apply_fn(a, f, out=b)
         dev.apply_fn(b, g, out=c)
