@@ -508,22 +508,31 @@ def bench_others(dev, args, stack_c5):
                      else "one hipGraphLaunch")
     e = _entry("c5: 1024 x f32[4096], t=a*b; u=t+c; y=sqrt(abs(u))*0.3, 3072 launches recorded once, then replayed",
                nbuf * m, 16, plain["us_per_replay"] * 1e-3, cpu_s, nbuf * m,
-               note="GB/s on the minimal 16 B/element; the recorded 3-kernel form moves 32 B/element")
+               note="GB/s on the minimal 16 B/element; the graph build joins the three launches of a buffer into one "
+                    "kernel that still writes t, u and y (24 B/element) and merges the 1024 joined launches into one "
+                    "grid; launch by launch the recording moves 32 B/element")
     e["us_per_replay"] = plain["us_per_replay"]
     e["replayed_as"] = plain["replayed_as"]
     e["replays"] = plain["replays"]
     e["graph_kernel_nodes"] = graph.kernel_nodes
     e["recorded_launches"] = 3 * nbuf
     e["graph_build_ms"] = round(build_s * 1e3, 2)
-    e["kernels"] = [dev.kernel_name(q) + "_batched" for q in (kmul, kadd, kun)]
+    e["launches_joined_into_later_ones"] = graph.fused_launches
     graph.destroy()
     # the same recording instantiated as a hipGraph and replayed with one hipGraphLaunch
     if args.hipgraph:
         dev.set_graph_direct_replay(0)
         graph, _ = record_c5()
-        e["as_hipgraph"] = timed_c5(graph, "one hipGraphLaunch of the instantiated 3-node graph")
+        e["as_hipgraph"] = timed_c5(graph, f"one hipGraphLaunch of the instantiated {graph.kernel_nodes}-node graph")
         graph.destroy()
         dev.set_graph_direct_replay(default_direct)
+    # without joining producers and consumers: one merged launch per recorded level
+    dev.set_graph_fusing(False)
+    graph, _ = record_c5()
+    e["launch_by_launch"] = timed_c5(graph, f"{graph.kernel_nodes} plain launches, one per recorded level (custos_hip_set_graph_fusing off)")
+    e["launch_by_launch"]["kernels"] = [dev.kernel_name(q) + "_batched" for q in (kmul, kadd, kun)]
+    graph.destroy()
+    dev.set_graph_fusing(True)
 
     # the same work after element-wise fusing (the text `Lazy::elementwise_fusing` of the host stack
     # emits for these operations): one three-operand kernel per buffer, 16 B/element, one node

@@ -142,9 +142,13 @@ void assign_levels(std::vector<RecNode>& nodes, bool edges) {
 // consumer's place in the recording.  Joined launches are producers and consumers in turn.
 
 struct ChainBuild {
-    std::vector<ChainStage> stages;
-    std::vector<uint64_t> ext;        // input pointers of the kernel to be
-    std::vector<uint64_t> stage_ptr;  // per stage: where its launch stored its result
+    // per stage: the kernel of its launch (whose expression it evaluates), where each variable of
+    // that expression comes from (ChainStage::source), and where the launch stored its result
+    std::vector<const custos_hip_kernel*> stage_kernel;
+    std::vector<std::vector<int>> source;
+    std::vector<uint64_t> stage_ptr;
+    std::vector<uint64_t> ext;  // input pointers of the kernel to be
+    size_t size() const { return stage_kernel.size(); }
 };
 
 // The last stage that writes `ptr`, or -1.
@@ -174,11 +178,11 @@ bool fusable_kernel(const RecNode& n) {
 
 ChainBuild chain_of(const RecNode& n) {
     ChainBuild c;
-    ChainStage stage;
-    stage.expr = n.k->spec.expr;
-    for (int v = 0; v < stage.expr.n_vars; v++) stage.source.push_back(input_index(&c, n.ptrs[static_cast<size_t>(v)]));
-    c.stages.push_back(std::move(stage));
+    std::vector<int> source;
+    for (int v = 0; v < n.k->spec.expr.n_vars; v++) source.push_back(input_index(&c, n.ptrs[static_cast<size_t>(v)]));
+    c.source.push_back(std::move(source));
     c.stage_ptr.push_back(n.ptrs.back());
+    c.stage_kernel.push_back(n.k);
     return c;
 }
 
@@ -199,7 +203,7 @@ bool join_chains(const ChainBuild& producer, const ChainBuild& consumer, uint64_
     for (uint64_t q : consumer.ext) reads_producer = reads_producer || writer_of(producer, q) >= 0;
     if (!reads_producer) return false;
     ChainBuild c = producer;
-    const int shift = static_cast<int>(producer.stages.size());
+    const int shift = static_cast<int>(producer.size());
     // what an input pointer of the consumer becomes: the stored value of the producer's stage
     // that wrote that memory last, or an input pointer of the joined kernel
     std::vector<int> mapped;
@@ -207,13 +211,14 @@ bool join_chains(const ChainBuild& producer, const ChainBuild& consumer, uint64_
         const int w = writer_of(producer, q);
         mapped.push_back(w >= 0 ? -(1 + w) : input_index(&c, q));
     }
-    for (size_t s = 0; s < consumer.stages.size(); s++) {
-        ChainStage stage = consumer.stages[s];
-        for (int& from : stage.source) from = from >= 0 ? mapped[static_cast<size_t>(from)] : from - shift;
-        c.stages.push_back(std::move(stage));
+    for (size_t s = 0; s < consumer.size(); s++) {
+        std::vector<int> source = consumer.source[s];
+        for (int& from : source) from = from >= 0 ? mapped[static_cast<size_t>(from)] : from - shift;
+        c.source.push_back(std::move(source));
         c.stage_ptr.push_back(consumer.stage_ptr[s]);
+        c.stage_kernel.push_back(consumer.stage_kernel[s]);
     }
-    if (c.stages.size() > static_cast<size_t>(kMaxChainStages) || c.ext.size() > static_cast<size_t>(kMaxChainInputs) ||
+    if (c.size() > static_cast<size_t>(kMaxChainStages) || c.ext.size() > static_cast<size_t>(kMaxChainInputs) ||
         distinct_outputs(c) > static_cast<size_t>(kMaxChainOutputs))
         return false;
     *joined = std::move(c);
@@ -303,7 +308,7 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
         for (const Access& a : c.acc)
             for (uint64_t ch = a.begin >> kChunkShift; ch <= (a.end - 1) >> kChunkShift; ch++)
                 buckets[ch].push_back(static_cast<uint32_t>(cands.size()));
-        if (chain.stages.size() > 1) chain_at.back() = chain;
+        if (chain.size() > 1) chain_at.back() = chain;
         c.chain = std::move(chain);
         cands.push_back(std::move(c));
     }
@@ -311,28 +316,43 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
     // kernels of the chains; the nodes take their final form
     std::vector<RecNode> fused;
     size_t compiled_here = 0;
+    // chains of the same launches wired the same way share a kernel: looked up once per shape
+    std::map<std::vector<uint64_t>, custos_hip_kernel*> kernel_of_shape;
     for (size_t i = 0; i < out.size(); i++) {
         if (dead[i]) continue;
         RecNode node = out[i];
         const ChainBuild& chain = chain_at[i];
-        if (chain.stages.size() > 1) {
-            std::vector<ChainStage> stages = chain.stages;
+        if (chain.size() > 1) {
+            std::vector<int> out_of(chain.size(), -1);
             std::vector<uint64_t> outs;
-            for (size_t s = 0; s < stages.size(); s++) {
-                stages[s].out = -1;
+            for (size_t s = 0; s < chain.size(); s++) {
                 if (writer_of(chain, chain.stage_ptr[s]) != static_cast<int>(s)) continue;
-                stages[s].out = static_cast<int>(outs.size());
+                out_of[s] = static_cast<int>(outs.size());
                 outs.push_back(chain.stage_ptr[s]);
             }
-            custos_hip_kernel* k = nullptr;
-            bool compiled = false;
-            Tuning tuning = node.k->spec.tuning;
-            tuning.unroll = 0;  // (only kernels whose vectors per thread were left open are joined)
-            const int32_t rc = chain_kernel(dev, node.k->spec.dtype, std::move(stages), static_cast<int>(chain.ext.size()),
-                                            static_cast<int>(outs.size()), tuning, &k, &compiled);
-            if (rc != CUSTOS_HIP_OK) return rc;
-            compiled_here += compiled;
-            if (compiled_here > kMaxNewChainKernels) return CUSTOS_HIP_ERR_TOO_LARGE;
+            std::vector<uint64_t> shape = {chain.ext.size(), outs.size()};
+            for (size_t s = 0; s < chain.size(); s++) {
+                shape.push_back(reinterpret_cast<uint64_t>(chain.stage_kernel[s]));
+                shape.push_back(static_cast<uint64_t>(static_cast<int64_t>(out_of[s])));
+                for (int from : chain.source[s]) shape.push_back(static_cast<uint64_t>(static_cast<int64_t>(from)));
+            }
+            custos_hip_kernel*& k = kernel_of_shape[shape];
+            if (!k) {
+                std::vector<ChainStage> stages(chain.size());
+                for (size_t s = 0; s < chain.size(); s++) {
+                    stages[s].expr = chain.stage_kernel[s]->spec.expr;
+                    stages[s].source = chain.source[s];
+                    stages[s].out = out_of[s];
+                }
+                bool compiled = false;
+                Tuning tuning = node.k->spec.tuning;
+                tuning.unroll = 0;  // (only kernels whose vectors per thread were left open are joined)
+                const int32_t rc = chain_kernel(dev, node.k->spec.dtype, std::move(stages), static_cast<int>(chain.ext.size()),
+                                                static_cast<int>(outs.size()), tuning, &k, &compiled);
+                if (rc != CUSTOS_HIP_OK) return rc;
+                compiled_here += compiled;
+                if (compiled_here > kMaxNewChainKernels) return CUSTOS_HIP_ERR_TOO_LARGE;
+            }
             const uint64_t bytes = node.n * dtype_size(node.k->spec.dtype);
             node.k = k;
             node.ptrs = chain.ext;

@@ -157,3 +157,42 @@ def test_operands_of_different_lengths_are_rejected_on_the_host():
                  lambda: dev.add_unary_grad(a, a, b, ident), lambda: dev.apply_fn2(a, h, ident)):
         with pytest.raises(ValueError):
             call()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "f16", "bf16", "i32", "i64", "u8", "i8", "i16", "u16", "u32", "u64",
+                                   "f16_pernode", "bf16_pernode"])
+def test_chain_kernels_compile_for_every_dtype(dtype):
+    """The kernel a graph build makes of a producer and its consumers: several expressions, several outputs."""
+    last = "max(v0, v1)" if dtype[0] in "iu" else "(sqrt(abs(v0)) * 0.3)"
+    stages = [("(v0 * v1)", [0, 1], 0), ("(v0 + v1)", [-1, 2], 1), (last, [-2, -1] if dtype[0] in "iu" else [-2], 2)]
+    text, size = capi.chain_emit(dtype, stages, 3, 3, compile_it=True)
+    assert size > 1000
+    entry = re.search(r"custos_chain_\w+", text).group(0)
+    for suffix in ("(", "_batched(", "_ragged("):
+        assert entry + suffix in text
+    # three inputs, three outputs; a stage takes an earlier stage's value as it was stored
+    assert "const S* in2, S* out0, S* out1, S* out2" in text
+    assert "const S t1 = custos_store(custos_expr_s1(r0, e2));" in text
+
+
+def test_chain_kernel_stores_what_is_overwritten_only_once():
+    """x = f(x); x = g(x) in place: the first store is dropped, the second stage reads the first value from a register."""
+    text, _ = capi.chain_emit("f32", [("(v0 * 2.0)", [0], -1), ("(v0 + 1.0)", [-1], 0)], 1, 1)
+    assert "o[0] = t1;" in text and "o[0] = t0;" not in text and "S* out1" not in text
+
+
+def test_chain_emit_rejects_malformed_stages():
+    ok = [("(v0 * v1)", [0, 1], 0)]
+    bad = [
+        ([("(v0 * v1)", [0, 2], 0)], 2, 1),            # reads an input that does not exist
+        ([("(v0 * v1)", [0, -1], 0)], 2, 1),           # reads itself
+        ([("(v0 * v1)", [0, 1], 1)], 2, 1),            # writes an output that does not exist
+        ([("(v0 * ", [0], 0)], 1, 1),                  # not an expression
+        (ok * 9, 2, 1),                                # too many stages
+        (ok, 0, 1), (ok, 2, 0), (ok, 9, 1), (ok, 2, 7),
+    ]
+    for stages, n_in, n_out in bad:
+        with pytest.raises(capi.CustosHipError):
+            capi.chain_emit("f32", stages, n_in, n_out)
+    with pytest.raises(capi.CustosHipError):
+        capi.chain_emit("i32", [("sin(v0)", [0], 0)], 1, 1)    # no such node over integers

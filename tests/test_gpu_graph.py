@@ -792,3 +792,160 @@ def test_waits_follow_the_work(hip):
     assert_bits_equal(bufs[0].slice(0, 1 << 12).read(), want)
     long_graph.destroy()
     short_graph.destroy()
+
+
+def _both_ways(hip, inputs, program, dtype="f32"):
+    """Runs `program(bufs)` eagerly and as a replayed graph (twice) over copies of `inputs`; the graph's
+    buffers must equal the eager ones bit for bit after every replay.  Returns the graph's
+    (kernel nodes, launches joined into later ones)."""
+    eager = [hip.buffer(x, dtype) for x in inputs]
+    lazy = [hip.buffer(x, dtype) for x in inputs]
+    hip.capture_begin()
+    program(lazy)
+    g = hip.capture_end()
+    shape = (g.kernel_nodes, g.fused_launches)
+    for replay in range(2):
+        program(eager)
+        g.launch()
+        hip.sync()
+        for i, (a, b) in enumerate(zip(lazy, eager)):
+            assert_bits_equal(a.read(), b.read(), f"replay {replay}, buffer {i}")
+    g.destroy()
+    return shape
+
+
+def test_producers_join_their_consumers(hip):
+    """Recorded apply launches that read, element for element, what an earlier one wrote become one
+    kernel with it; every buffer still gets what the separate launches gave it."""
+    n = 5003
+    xs = [synth.uniform_f32(200 + i, n, -2, 2) for i in range(6)]
+    f = lambda v: v.mul(1.5).sub(0.25)
+    g = lambda v: v.abs().sqrt()
+    h = lambda v: v.neg().max(-1.0)
+    add = lambda p, q: p.add(q)
+    mul = lambda p, q: p.mul(q)
+
+    def fan_out(b):                 # two consumers of one result
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.apply_fn(b[1], g, out=b[2])
+        hip.apply_fn(b[1], h, out=b[3])
+    assert _both_ways(hip, xs, fan_out) == (1, 2)
+
+    def diamond(b):                 # two producers of one consumer
+        hip.apply_fn(b[0], f, out=b[2])
+        hip.apply_fn(b[1], g, out=b[3])
+        hip.apply_fn2(b[2], b[3], add, out=b[4])
+        hip.apply_fn2(b[4], b[2], mul, out=b[5])
+    assert _both_ways(hip, xs, diamond) == (1, 3)
+
+    def in_place(b):                # the same buffer read and written by every launch: one output
+        for fn in (f, g, h):
+            hip.apply_fn(b[0], fn, out=b[0])
+    assert _both_ways(hip, xs, in_place) == (1, 2)
+
+    def writes_an_input_of_its_producer(b):
+        hip.apply_fn2(b[0], b[1], add, out=b[2])
+        hip.apply_fn2(b[2], b[1], mul, out=b[0])      # b[0] was read by the first launch
+        hip.apply_fn(b[0], f, out=b[1])               # and b[1] by both
+    assert _both_ways(hip, xs, writes_an_input_of_its_producer) == (1, 2)
+
+    def same_operand_twice(b):
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.apply_fn2(b[1], b[1], mul, out=b[2])
+    assert _both_ways(hip, xs, same_operand_twice) == (1, 1)
+
+    def another_length(b):          # the consumer reads a part only: another launch geometry
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.apply_fn(b[1].slice(0, 4000), g, out=b[2].slice(0, 4000))
+    assert _both_ways(hip, xs, another_length) == (2, 0)
+
+    def shifted(b):                 # the same length, but element i of the consumer is element i + 16 of the producer
+        hip.apply_fn(b[0].slice(0, 4000), f, out=b[1].slice(0, 4000))
+        hip.apply_fn(b[1].slice(16, 4016), g, out=b[2].slice(0, 4000))
+    assert _both_ways(hip, xs, shifted) == (2, 0)
+
+    def shifted_output(b):          # the consumer writes over a shifted part of what the producer read
+        hip.apply_fn(b[0].slice(0, 4000), f, out=b[1].slice(0, 4000))
+        hip.apply_fn(b[1].slice(0, 4000), g, out=b[0].slice(8, 4008))
+    assert _both_ways(hip, xs, shifted_output) == (2, 0)
+
+    def input_rewritten_in_between(b):
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.apply_fn(b[0], h, out=b[0])               # writes what the first launch read
+        hip.apply_fn(b[1], g, out=b[2])               # may not take the first launch along past that
+    assert _both_ways(hip, xs, input_rewritten_in_between) == (3, 0)
+
+    def result_read_in_between(b):
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.add_unary_grad(b[1], b[3], b[4], g)       # another kind of launch reads the result
+        hip.apply_fn(b[1], g, out=b[2])
+    assert _both_ways(hip, xs, result_read_in_between) == (3, 0)
+
+    def cleared_in_between(b):
+        hip.apply_fn(b[0], f, out=b[1])
+        b[0].clear()
+        hip.apply_fn(b[1], g, out=b[2])
+    assert _both_ways(hip, xs, cleared_in_between) == (3, 0)
+
+    def untouched_in_between(b):    # launches on other buffers in between do not matter
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.apply_fn(b[3], h, out=b[4])
+        b[5].clear()
+        hip.apply_fn(b[1], g, out=b[2])
+    assert _both_ways(hip, xs, untouched_in_between) == (3, 1)
+
+    def long_chain(b):              # at most eight expressions per kernel
+        for i in range(20):
+            hip.apply_fn(b[i % 2], f if i % 3 else h, out=b[(i + 1) % 2])
+    assert _both_ways(hip, xs, long_chain) == (3, 17)
+
+    def unaligned(b):               # views that start 3 elements into their buffers: scalar head and tail
+        v = [q.slice(3, 3 + 1001) for q in b]
+        hip.apply_fn2(v[0], v[1], mul, out=v[2])
+        hip.apply_fn2(v[2], v[3], add, out=v[4])
+        hip.apply_fn(v[4], g, out=v[5])
+    assert _both_ways(hip, xs, unaligned) == (1, 2)
+
+    def other_phase(b):             # producer and consumer views start at different offsets within 16 bytes
+        hip.apply_fn(b[0].slice(1, 1001), f, out=b[1].slice(1, 1001))
+        hip.apply_fn(b[1].slice(1, 1001), g, out=b[2].slice(2, 1002))
+    assert _both_ways(hip, xs, other_phase)[1] in (0, 1)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "f16", "bf16", "f16_pernode", "bf16_pernode", "i32", "u8", "i64"])
+def test_joined_launches_in_every_element_type(hip, dtype):
+    """t = a * b; u = t + c; y = max(u, t) as one kernel: what a later stage takes from an earlier one is
+    the STORED value (rounded to the storage type), so every buffer equals the launch-by-launch result."""
+    n = 4099
+    npdt = np.dtype(capi.DTYPES[dtype][1])
+    rng = np.random.default_rng(5)
+    if dtype[0] in "iu":
+        info = np.iinfo(npdt)
+        xs = [rng.integers(info.min, info.max, size=n, dtype=npdt, endpoint=True) for _ in range(3)]
+    elif npdt == np.uint16:           # 16-bit floats travel as bits
+        from oracle import cpu_oracle
+        conv = cpu_oracle.f32_to_f16_bits if dtype.startswith("f16") else (lambda a: (a.view(np.uint32) >> 16).astype(np.uint16))
+        xs = [conv(synth.uniform_f32(300 + i, n, -3, 3)) for i in range(3)]
+    else:
+        xs = [synth.uniform_f32(300 + i, n, -3, 3).astype(npdt) for i in range(3)]
+    xs += [np.zeros(n, dtype=npdt) for _ in range(3)]
+
+    def program(b):
+        hip.apply_fn2(b[0], b[1], lambda p, q: p.mul(q), out=b[3])
+        hip.apply_fn2(b[3], b[2], lambda p, q: p.add(q), out=b[4])
+        hip.apply_fn2(b[4], b[3], lambda p, q: p.max(q), out=b[5])
+    assert _both_ways(hip, xs, program, dtype) == (1, 2)
+
+
+def test_joined_launches_of_many_buffers_merge(hip):
+    """Chains over many buffers of different lengths: each chain one kernel, all of them one grid."""
+    lengths = [256 * (1 + i % 7) + 4 * (i % 3) for i in range(40)]
+    xs = [synth.uniform_f32(400 + i, ln, -2, 2) for i, ln in enumerate(lengths)]
+    zeros = [np.zeros(ln, dtype=np.float32) for ln in lengths]
+
+    def program(b):
+        k = len(lengths)
+        for i in range(k):
+            hip.apply_fn(b[i], lambda v: v.mul(0.5).add(1.0), out=b[k + i])
+            hip.apply_fn2(b[k + i], b[i], lambda p, q: p.mul(q), out=b[2 * k + i])
+    assert _both_ways(hip, xs + zeros + zeros, program) == (1, 40)
