@@ -229,9 +229,10 @@ EDGE_MODES = {"level joins": capi.GRAPH_EDGES_LEVEL_JOINS, "per node": capi.GRAP
 def test_recorded_dependencies_random(checked_graphs, oracle, edges):
     """Random programs over a small pool of buffers, with in-place updates, views and clears:
     replaying the built graph (ordered by level joins, per-node edges or as one chain; merged launches)
-    must equal running the same calls eagerly, bit for bit.  Even trials use aligned half-buffer
-    views, odd trials views of any offset and length (partial overlaps between operations,
-    scalar launches).  The library also checks each graph's ordering by brute force."""
+    must equal running the same calls eagerly, bit for bit.  One trial in three uses aligned half-buffer
+    views, one views of any offset and length (partial overlaps between operations, scalar launches),
+    one whole buffers (chains of launches that join).  The library also checks each graph's ordering by
+    brute force."""
     import os
     hip = checked_graphs
     hip.set_graph_edges(EDGE_MODES[edges])
@@ -246,11 +247,13 @@ def test_recorded_dependencies_random(checked_graphs, oracle, edges):
         program = []
         for _ in range(40):
             kind = rng.integers(0, 5)
-            if trial % 2:
+            if trial % 3 == 1:
                 lo = int(rng.integers(0, 1500))
                 ln = int(rng.integers(1, n - lo + 1))
-            else:
+            elif trial % 3 == 0:
                 lo, ln = int(rng.integers(0, 3)) * 512, 1024     # [lo, lo + 1024) keeps 16-byte phases equal
+            else:
+                lo, ln = 0, n                                     # whole buffers: most launches join their producers
             if kind == 0:
                 program.append(("u", int(rng.integers(len(fns1))), int(rng.integers(nbuf)), int(rng.integers(nbuf)), lo, ln))
             elif kind in (1, 2):
