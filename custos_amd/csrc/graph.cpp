@@ -131,8 +131,9 @@ void assign_levels(std::vector<RecNode>& nodes, bool edges) {
 // the value the separate launches gave it (the value handed on is the stored one, rounded to
 // the storage type), so nothing a caller can observe changes.
 //
-// What may be joined.  Both are apply launches of generated kernels with the same element
-// type, length and alignment phase.  The consumer reads at least one output of the producer.
+// What may be joined.  Both are apply or unary-gradient launches of generated kernels (a
+// gradient launch is the expression `g + (o * f'(x))` stored to g) with the same element type,
+// length and alignment phase.  The consumer reads at least one output of the producer.
 // Every address range of the one that the other also touches, one of them writing, is the
 // SAME range (same address): the fused kernel handles element i of every operand in one
 // lane, all loads before all stores, so equal ranges behave as in the separate launches and
@@ -172,16 +173,47 @@ size_t distinct_outputs(const ChainBuild& c) {
 }
 
 bool fusable_kernel(const RecNode& n) {
-    if (n.type != RecNode::Kernel || n.k->spec.kind != Kind::Apply || !n.k->spec.auto_unroll) return false;
+    if (n.type != RecNode::Kernel || !n.k->spec.auto_unroll) return false;
+    if (n.k->spec.kind != Kind::Apply && n.k->spec.kind != Kind::UnaryGrad) return false;
     return n.k->spec.tuning.blocks_per_cu <= 0;
+}
+
+// What a recorded launch evaluates per element, as an expression over its pointers: an apply
+// launch its own expression over its inputs; a unary-gradient launch `g + (o * f'(x))` over
+// (x, g, o) = (lhs, lhs_grad, out_grad), the product rounded before the sum like in its own kernel
+// (src/devices/cpu_stack_ops.rs:27-29), stored to g.
+Expr stage_expr(const custos_hip_kernel* k) {
+    Expr e = k->spec.expr;
+    if (k->spec.kind != Kind::UnaryGrad) return e;
+    Node g, o, prod, sum;
+    g.op = o.op = Op::Var;
+    g.var = 1;
+    o.var = 2;
+    const int derivative = e.root, first = static_cast<int>(e.nodes.size());
+    prod.op = Op::Mul;
+    prod.a = first + 1;  // o
+    prod.b = derivative;
+    sum.op = Op::Add;
+    sum.a = first;       // g
+    sum.b = first + 2;   // o * f'(x)
+    e.nodes.insert(e.nodes.end(), {g, o, prod, sum});
+    e.root = first + 3;
+    e.n_vars = 3;
+    return e;
 }
 
 ChainBuild chain_of(const RecNode& n) {
     ChainBuild c;
     std::vector<int> source;
-    for (int v = 0; v < n.k->spec.expr.n_vars; v++) source.push_back(input_index(&c, n.ptrs[static_cast<size_t>(v)]));
+    if (n.k->spec.kind == Kind::UnaryGrad) {
+        // (x, g, o) in the order of the launch's pointers; g is read and written
+        for (size_t v = 0; v < 3; v++) source.push_back(input_index(&c, n.ptrs[v]));
+        c.stage_ptr.push_back(n.ptrs[1]);
+    } else {
+        for (int v = 0; v < n.k->spec.expr.n_vars; v++) source.push_back(input_index(&c, n.ptrs[static_cast<size_t>(v)]));
+        c.stage_ptr.push_back(n.ptrs.back());
+    }
     c.source.push_back(std::move(source));
-    c.stage_ptr.push_back(n.ptrs.back());
     c.stage_kernel.push_back(n.k);
     return c;
 }
@@ -340,7 +372,7 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
             if (!k) {
                 std::vector<ChainStage> stages(chain.size());
                 for (size_t s = 0; s < chain.size(); s++) {
-                    stages[s].expr = chain.stage_kernel[s]->spec.expr;
+                    stages[s].expr = stage_expr(chain.stage_kernel[s]);
                     stages[s].source = chain.source[s];
                     stages[s].out = out_of[s];
                 }

@@ -391,8 +391,10 @@ int32_t custos_hip_capture_end_reuse(custos_hip_device *dev, custos_hip_graph *p
  * with it off every recorded launch becomes its own kernel node. */
 int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
 /* Switches the joining of producers with their consumers off (0) or on (default).  With it on, a
- * recorded apply launch whose output a later recorded apply launch reads element for element
- * (same address, length and element type) becomes one kernel with that launch: both expressions
+ * recorded apply or unary-gradient launch whose output a later recorded apply or unary-gradient
+ * launch reads element for element (same address, length and element type; a gradient launch
+ * counts as the expression `lhs_grad + (out_grad * f'(lhs))` stored to lhs_grad) becomes one
+ * kernel with that launch: both expressions
  * are evaluated per element, both results are stored where the two launches stored them, and
  * the second expression takes the first result -- as it was stored, rounded to the storage type
  * -- from a register.  `t = a * b; u = t + c; y = f(u)` replays as one launch that reads a, b, c

@@ -878,11 +878,19 @@ def test_producers_join_their_consumers(hip):
         hip.apply_fn(b[1], g, out=b[2])               # may not take the first launch along past that
     assert _both_ways(hip, xs, input_rewritten_in_between) == (3, 0)
 
-    def result_read_in_between(b):
+    def result_copied_in_between(b):
         hip.apply_fn(b[0], f, out=b[1])
-        hip.add_unary_grad(b[1], b[3], b[4], g)       # another kind of launch reads the result
+        hip.copy(b[3], b[1])                          # a copy reads the result: it has to be in memory by then
         hip.apply_fn(b[1], g, out=b[2])
-    assert _both_ways(hip, xs, result_read_in_between) == (3, 0)
+    assert _both_ways(hip, xs, result_copied_in_between) == (3, 0)
+
+    def gradient_launches_join_too(b):                # x_grad += out_grad * f'(x) is the expression g + (o * f'(x)) stored to g
+        hip.apply_fn(b[0], f, out=b[1])               # y1 = f(x)
+        hip.apply_fn(b[1], g, out=b[2])               # y2 = g(y1)
+        hip.add_unary_grad(b[1], b[4], b[3], lambda v: v.mul(0.5).abs())   # g1 += g2 * g'(y1)
+        hip.add_unary_grad(b[0], b[5], b[4], lambda v: v.mul(2.0))         # gx += g1 * f'(x)
+        hip.add_unary_grad(b[0], b[5], b[3], lambda v: v.neg())            # and once more into the same gradient
+    assert _both_ways(hip, xs, gradient_launches_join_too) == (1, 4)
 
     def cleared_in_between(b):
         hip.apply_fn(b[0], f, out=b[1])
@@ -937,7 +945,8 @@ def test_joined_launches_in_every_element_type(hip, dtype):
         hip.apply_fn2(b[0], b[1], lambda p, q: p.mul(q), out=b[3])
         hip.apply_fn2(b[3], b[2], lambda p, q: p.add(q), out=b[4])
         hip.apply_fn2(b[4], b[3], lambda p, q: p.max(q), out=b[5])
-    assert _both_ways(hip, xs, program, dtype) == (1, 2)
+        hip.add_unary_grad(b[3], b[5], b[4], lambda v: v.mul(3).add(1))    # b5 += b4 * (3 * b3 + 1)
+    assert _both_ways(hip, xs, program, dtype) == (1, 3)
 
 
 def test_joined_launches_of_many_buffers_merge(hip):
