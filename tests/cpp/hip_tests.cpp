@@ -446,4 +446,84 @@ TEST_CASE(hip_apply_fn_many_noalloc) {
     CHECK_EQ(custos_hip_apply_fn_many_noalloc(dev, k, too_many.data(), 2, 10, 16), static_cast<int32_t>(CUSTOS_HIP_ERR_ARITY_MISMATCH));
 }
 
+// Random programs of apply and gradient launches over whole buffers and half views, through the C
+// ABI: the replayed graph (producers joined into their consumers, equal launches merged) leaves every
+// buffer exactly as the same calls issued one by one do, replay after replay; with joining switched
+// off as well.
+TEST_CASE(hip_joined_launches_random_programs) {
+    HIP<Base> device;
+    custos_hip_device* dev = device.handle();
+    const size_t n = 3000, nbuf = 6;
+    const char* m1[] = {"x"};
+    const char* m2[] = {"x", "y"};
+    std::vector<custos_hip_kernel*> unary, binary, grads;
+    for (const char* src : {"((x * 1.25) + 0.5)", "max(-(x), -3.0)", "sqrt(abs(x))", "min((x * x), 9.0)"}) {
+        custos_hip_kernel* k = nullptr;
+        CHECK_EQ(custos_hip_expr_compile(dev, CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, src, m1, 1, &k), 0);
+        unary.push_back(k);
+        CHECK_EQ(custos_hip_expr_compile(dev, CUSTOS_HIP_KIND_UNARY_GRAD, CUSTOS_HIP_F32, src, m1, 1, &k), 0);
+        grads.push_back(k);
+    }
+    for (const char* src : {"(x + y)", "((x * y) - 0.125)", "max(x, y)"}) {
+        custos_hip_kernel* k = nullptr;
+        CHECK_EQ(custos_hip_expr_compile(dev, CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, src, m2, 2, &k), 0);
+        binary.push_back(k);
+    }
+    struct Op {
+        int kind, fn, a, b, c;
+        size_t lo, len;
+    };
+    uint64_t state = 12345;
+    auto next = [&](uint64_t below) {
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        return (state >> 33) % below;
+    };
+    size_t joined = 0;
+    for (int trial = 0; trial < 6; trial++) {
+        std::vector<Op> program;
+        for (int i = 0; i < 30; i++) {
+            Op op{static_cast<int>(next(4)), 0, static_cast<int>(next(nbuf)), static_cast<int>(next(nbuf)), static_cast<int>(next(nbuf)), 0, n};
+            if (next(4) == 0) op.lo = next(2) * 1500, op.len = 1500;   // a half view now and then
+            op.fn = static_cast<int>(next(op.kind == 0 ? unary.size() : op.kind == 3 ? grads.size() : binary.size()));
+            if (op.kind == 3 && (op.a == op.b || op.b == op.c || op.a == op.c)) op.kind = 0;   // gradient operands are distinct buffers
+            program.push_back(op);
+        }
+        std::vector<std::vector<float>> init(nbuf, std::vector<float>(n));
+        for (size_t b = 0; b < nbuf; b++)
+            for (size_t i = 0; i < n; i++) init[b][i] = static_cast<float>(static_cast<int>(next(4001)) - 2000) * 0.001f;
+        auto run = [&](std::vector<Buffer<float, HIP<Base>>>& bufs) {
+            for (const Op& op : program) {
+                const uint64_t a = bufs[op.a].ptr() + op.lo * 4, b = bufs[op.b].ptr() + op.lo * 4, c = bufs[op.c].ptr() + op.lo * 4;
+                if (op.kind == 0) CHECK_EQ(custos_hip_apply_fn(dev, unary[op.fn], a, b, op.len), 0);
+                else if (op.kind == 3) CHECK_EQ(custos_hip_add_unary_grad(dev, grads[op.fn], a, b, c, op.len), 0);
+                else CHECK_EQ(custos_hip_apply_fn2(dev, binary[op.fn], a, b, c, op.len), 0);
+            }
+        };
+        for (int fusing = 1; fusing >= 0; fusing--) {
+            std::vector<Buffer<float, HIP<Base>>> eager, lazy;
+            for (size_t b = 0; b < nbuf; b++) eager.push_back(device.buffer(init[b])), lazy.push_back(device.buffer(init[b]));
+            CHECK_EQ(custos_hip_set_graph_fusing(dev, fusing), 0);
+            CHECK_EQ(custos_hip_capture_begin(dev), 0);
+            run(lazy);
+            custos_hip_graph* graph = nullptr;
+            CHECK_EQ(custos_hip_capture_end(dev, &graph), 0);
+            size_t fused = 0;
+            CHECK_EQ(custos_hip_graph_fused_launches(graph, &fused), 0);
+            CHECK(fusing || fused == 0);
+            joined += fused;
+            for (int replay = 0; replay < 2; replay++) {
+                run(eager);
+                CHECK_EQ(custos_hip_graph_launch(dev, graph), 0);
+                for (size_t b = 0; b < nbuf; b++) {
+                    const std::vector<float> got = lazy[b].read(), want = eager[b].read();
+                    CHECK(std::memcmp(got.data(), want.data(), n * sizeof(float)) == 0);
+                }
+            }
+            CHECK_EQ(custos_hip_graph_destroy(dev, graph), 0);
+        }
+    }
+    CHECK_EQ(custos_hip_set_graph_fusing(dev, 1), 0);
+    CHECK(joined > 20);
+}
+
 int main(int argc, char** argv) { return check::run(argc, argv); }
