@@ -237,6 +237,14 @@ def bench_c2(dev, args, stack):
             one()
 
     unfused_ms, unfused_n = time_floor(dev, unfused_step, launches_per_step=5)
+    # the same five launches recorded and replayed: the graph build joins them into one kernel that
+    # still writes both intermediates (1 read + 3 writes per element instead of 5 + 5)
+    dev.capture_begin()
+    unfused_step()
+    recorded_unfused = dev.capture_end()
+    recorded_ms, recorded_n = time_floor(dev, recorded_unfused.launch)
+    recorded_nodes, recorded_joined = recorded_unfused.kernel_nodes, recorded_unfused.fused_launches
+    recorded_unfused.destroy()
 
     # plain copy (identity expression) over the same buffers: the achievable 1R+1W rate on
     # this box, and the known-size dispatch the profiler counters are scaled by
@@ -317,6 +325,13 @@ def bench_c2(dev, args, stack):
             "effective_GBps_on_8B_basis": round(gbs_of(unfused_ms), 2),
             "moved_GBps_on_40B_basis": round(5 * gbs_of(unfused_ms), 2),
             "speedup_fused": round(unfused_ms / per_launch_ms, 3),
+            "recorded_and_replayed": {
+                "ms_per_replay": round(recorded_ms, 5), "replays": recorded_n, "kernel_nodes": recorded_nodes,
+                "launches_joined_into_later_ones": recorded_joined,
+                "effective_GBps_on_8B_basis": round(gbs_of(recorded_ms), 2),
+                "what": "the five launches recorded without unary fusing; the graph build joins them into one kernel "
+                        "that still writes the two intermediate buffers (16 B/element)",
+            },
         },
         "copy_kernel": {
             "name": dev.kernel_name(copy_kernel),
