@@ -114,7 +114,7 @@ PROTOTYPES = {
     "custos_hip_set_graph_fusing": (C.c_int32, [_P, C.c_int32]),
     "custos_hip_graph_fused_launches": (C.c_int32, [_P, C.POINTER(C.c_size_t)]),
     "custos_hip_chain_emit": (C.c_int32, [C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.c_int32, C.POINTER(C.c_int32),
-                                          C.POINTER(C.c_int32), C.c_int32, C.c_int32, C.c_char_p, C.c_size_t,
+                                          C.POINTER(C.c_int32), C.c_int32, C.c_int32, C.c_int32, C.c_char_p, C.c_size_t,
                                           C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "custos_hip_last_launch_shape": (C.c_int32, [_P, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "custos_hip_kernel_launched_as": (C.c_int32, [_P, _P, C.c_size_t, C.POINTER(C.c_void_p)]),
@@ -226,7 +226,7 @@ def expr_emit(kind: int, dtype: str, src: str, markers, tuning: Tuning | None = 
     return buf.value.decode(), h.value
 
 
-def chain_emit(dtype: str, stages, n_inputs: int, n_outputs: int, compile_it: bool = False):
+def chain_emit(dtype: str, stages, n_inputs: int, n_outputs: int, compile_it: bool = False, literals_as_parameters: bool = False):
     """Host-only: source (and, with `compile_it`, the gfx950 code size) of the kernel that joins several
     expressions.  `stages`: (source text over v0.., [where each variable comes from], output index or -1)."""
     lib = load_library()
@@ -236,7 +236,7 @@ def chain_emit(dtype: str, stages, n_inputs: int, n_outputs: int, compile_it: bo
     sources = (C.c_int32 * len(flat))(*flat)
     outs = (C.c_int32 * len(stages))(*[s[2] for s in stages])
     needed, size = C.c_size_t(0), C.c_size_t(0)
-    args = (DTYPES[dtype][0], srcs, n_vars, len(stages), sources, outs, n_inputs, n_outputs)
+    args = (DTYPES[dtype][0], srcs, n_vars, len(stages), sources, outs, n_inputs, n_outputs, 1 if literals_as_parameters else 0)
     check(lib.custos_hip_chain_emit(*args, None, 0, C.byref(needed), C.byref(size) if compile_it else None))
     buf = C.create_string_buffer(needed.value)
     check(lib.custos_hip_chain_emit(*args, buf, needed.value, None, None))

@@ -364,7 +364,8 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
             }
             std::vector<uint64_t> shape = {chain.ext.size(), outs.size()};
             for (size_t s = 0; s < chain.size(); s++) {
-                shape.push_back(reinterpret_cast<uint64_t>(chain.stage_kernel[s]));
+                // (handles of one code differ in the values of their literal parameters only)
+                shape.push_back(reinterpret_cast<uint64_t>(chain.stage_kernel[s]->code ? chain.stage_kernel[s]->code : chain.stage_kernel[s]));
                 shape.push_back(static_cast<uint64_t>(static_cast<int64_t>(out_of[s])));
                 for (int from : chain.source[s]) shape.push_back(static_cast<uint64_t>(static_cast<int64_t>(from)));
             }
@@ -372,9 +373,18 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
             if (!k) {
                 std::vector<ChainStage> stages(chain.size());
                 for (size_t s = 0; s < chain.size(); s++) {
-                    stages[s].expr = stage_expr(chain.stage_kernel[s]);
+                    const custos_hip_kernel* sk = chain.stage_kernel[s];
+                    stages[s].expr = stage_expr(sk);
                     stages[s].source = chain.source[s];
                     stages[s].out = out_of[s];
+                    // a literal is in the chain's code, or one of its launch parameters, as it is for
+                    // the launch's own kernel (the nodes a gradient stage adds hold no literals)
+                    if (sk->spec.consts.n_params > 0) {
+                        stages[s].slot = sk->spec.consts.slot;
+                        stages[s].slot.resize(stages[s].expr.nodes.size(), -1);
+                        stages[s].n_params = sk->spec.consts.n_params;
+                        stages[s].param_bytes = sk->spec.consts.bytes.size();
+                    }
                 }
                 bool compiled = false;
                 Tuning tuning = node.k->spec.tuning;
@@ -386,6 +396,9 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
                 if (compiled_here > kMaxNewChainKernels) return CUSTOS_HIP_ERR_TOO_LARGE;
             }
             const uint64_t bytes = node.n * dtype_size(node.k->spec.dtype);
+            node.const_bytes.clear();
+            for (const custos_hip_kernel* sk : chain.stage_kernel)
+                node.const_bytes.insert(node.const_bytes.end(), sk->spec.consts.bytes.begin(), sk->spec.consts.bytes.end());
             node.k = k;
             node.ptrs = chain.ext;
             node.ptrs.insert(node.ptrs.end(), outs.begin(), outs.end());
@@ -521,7 +534,7 @@ void append_tables(const std::vector<RecNode>& nodes, Planned* p, std::vector<ui
     for (size_t member : p->members) {
         for (uint64_t ptr : nodes[member].ptrs) host_table->push_back(ptr);
         if (p->ragged) host_table->push_back(nodes[member].n);
-        const std::vector<unsigned char>& values = nodes[member].k->spec.consts.bytes;
+        const std::vector<unsigned char>& values = literal_values(nodes[member]);
         for (size_t at = 0; at < values.size(); at += 8) {
             uint64_t word = 0;
             std::memcpy(&word, values.data() + at, std::min<size_t>(8, values.size() - at));
@@ -634,8 +647,7 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
         // a generated entry point ends with the block of literal parameters (if the
         // expression has any) and the direction
         // (a merged launch reads them from its table rows instead)
-        const ConstPlan& consts = first.k->spec.consts;
-        if (consts.n_params > 0 && p.members.size() == 1) ln.args.push_back(consts.bytes);
+        if (first.k->spec.consts.n_params > 0 && p.members.size() == 1) ln.args.push_back(literal_values(first));
         const unsigned long long mode = launch_mode(p.shape.unroll, p.shape.nontemporal, rev != 0);
         ln.args.push_back(value(&mode, 8));
         if (p.shape.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;

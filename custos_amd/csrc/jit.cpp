@@ -466,7 +466,7 @@ int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const cha
 
 int32_t custos_hip_chain_emit(int32_t dtype, const char* const* stage_srcs, const int32_t* stage_vars, int32_t n_stages,
                               const int32_t* sources, const int32_t* stage_outs, int32_t n_inputs, int32_t n_outputs,
-                              char* buf, size_t cap, size_t* needed, size_t* code_size) {
+                              int32_t literals_as_parameters, char* buf, size_t cap, size_t* needed, size_t* code_size) {
     if (!dtype_valid(dtype)) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown element type");
     if (!stage_srcs || !stage_vars || !sources || !stage_outs || n_stages < 1 || n_stages > kMaxChainStages)
         return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "1 to 8 stages are required");
@@ -486,6 +486,16 @@ int32_t custos_hip_chain_emit(int32_t dtype, const char* const* stage_srcs, cons
         stage.source.assign(from, from + stage_vars[s]);
         from += stage_vars[s];
         stage.out = stage_outs[s];
+        if (literals_as_parameters) {
+            ConstPlan plan;
+            if (!plan_constants(stage.expr, static_cast<DType>(dtype), /*all_in_code=*/false, &plan, &err))
+                return set_error(nullptr, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+            if (plan.n_params > 0) {
+                stage.slot = plan.slot;
+                stage.n_params = plan.n_params;
+                stage.param_bytes = plan.bytes.size();
+            }
+        }
         stages.push_back(std::move(stage));
     }
     KernelSpec spec;

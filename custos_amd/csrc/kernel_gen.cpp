@@ -214,6 +214,23 @@ std::string grad_fn(DType dtype) {
            "    return (C)((" + U + ")g + (" + U + ")prod);\n}\n";
 }
 
+// The constant plan of one stage of a chain: its own slots, moved behind the parameters of the
+// stages before it (`base`).
+bool stage_plan(const ChainStage& stage, DType dtype, int base, ConstPlan* plan, ParseError* err) {
+    if (stage.slot.empty()) return plan_constants(stage.expr, dtype, /*all_in_code=*/true, plan, err);
+    if (stage.slot.size() != stage.expr.nodes.size()) {
+        err->code = CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+        err->message = "malformed chain stage";
+        return false;
+    }
+    plan->slot = stage.slot;
+    for (int& s : plan->slot)
+        if (s >= 0) s += base;
+    plan->n_params = stage.n_params;
+    plan->bytes.clear();
+    return true;
+}
+
 // Text of the per-element function, the tile function and the three entry points of one
 // kernel.  Operand naming inside a kernel: in0.. are the inputs, `out` the output; for a unary
 // gradient 0 = lhs, 1 = lhs_grad (also the output), 2 = out_grad.
@@ -299,7 +316,7 @@ struct KernelText {
     // stores every output.
     std::string scalar_stmt(const std::string& idx) const {
         if (k.kind != Kind::Chain) return "out[" + idx + "] = custos_elem(" + list("in", "[" + idx + "]") + " CUSTOS_KC_ARG);";
-        std::string s = "{ S o[" + std::to_string(k.n_outs) + "]; custos_chain(" + list("in", "[" + idx + "]") + ", o);";
+        std::string s = "{ S o[" + std::to_string(k.n_outs) + "]; custos_chain(" + list("in", "[" + idx + "]") + ", o CUSTOS_KC_ARG);";
         for (int j = 0; j < k.n_outs; j++) s += " out" + std::to_string(j) + "[" + idx + "] = o[" + std::to_string(j) + "];";
         return s + " }";
     }
@@ -309,21 +326,23 @@ struct KernelText {
     // reads an earlier one takes its result as it was stored (rounded to the storage type).
     std::string chain_fn() const {
         std::string s;
+        int base = 0;
         for (size_t st = 0; st < k.stages.size(); st++) {
             const ChainStage& stage = k.stages[st];
             ConstPlan plan;
             ParseError err;
             std::string body;
             // (checked when the spec was built)
-            (void)plan_constants(stage.expr, k.dtype, /*all_in_code=*/true, &plan, &err);
+            (void)stage_plan(stage, k.dtype, base, &plan, &err);
             (void)emit_expr_body(stage.expr, k.dtype, plan, &body, &err);
+            base += stage.n_params;
             s += "static __device__ __forceinline__ C custos_expr_s" + std::to_string(st) + "(";
             for (int v = 0; v < stage.expr.n_vars; v++) s += std::string(v ? ", " : "") + "const C v" + std::to_string(v);
-            s += ") {\n" + body + "}\n";
+            s += " CUSTOS_KC_PARAM) {\n" + body + "}\n";
         }
         s += "static __device__ __forceinline__ void custos_chain(";
         for (int i = 0; i < n_in; i++) s += "const S s" + std::to_string(i) + ", ";
-        s += "S* o) {\n";
+        s += "S* o CUSTOS_KC_PARAM) {\n";
         for (int i = 0; i < n_in; i++) s += "    const C e" + std::to_string(i) + " = custos_load(s" + std::to_string(i) + ");\n";
         for (size_t st = 0; st < k.stages.size(); st++) {
             const ChainStage& stage = k.stages[st];
@@ -333,7 +352,7 @@ struct KernelText {
                 const int from = stage.source[v];
                 s += std::string(v ? ", " : "") + (from >= 0 ? "e" + std::to_string(from) : "r" + std::to_string(-from - 1));
             }
-            s += "));\n    const C r" + id + " = custos_load(t" + id + ");\n    (void)r" + id + ";\n";
+            s += " CUSTOS_KC_ARG));\n    const C r" + id + " = custos_load(t" + id + ");\n    (void)r" + id + ";\n";
             if (stage.out >= 0) s += "    o[" + std::to_string(stage.out) + "] = t" + id + ";\n";
         }
         s += "}\n";
@@ -346,7 +365,7 @@ struct KernelText {
         std::string s = "static __device__ __forceinline__ void custos_tile" + U + "(";
         for (int i = 0; i < n_in; i++) s += "const vec_t* vin" + std::to_string(i) + ", ";
         for (int j = 0; j < k.n_outs; j++) s += "vec_t* vout" + std::to_string(j) + ", ";
-        s += "const u64 first, const u64 n_vec, const u64 mode) {\n";
+        s += "const u64 first, const u64 n_vec, const u64 mode CUSTOS_KC_PARAM) {\n";
         s += "    const u64 left = (n_vec - first) * 16;\n";
         s += "    const int bound = left > 0x7ffffff0ull ? 0x7ffffff0 : (int)left;\n";
         for (int i = 0; i < n_in; i++)
@@ -365,7 +384,7 @@ struct KernelText {
         for (int j = 0; j < k.n_outs; j++) s += "        vec_t r" + std::to_string(j) + ";\n";
         s += "#pragma unroll\n        for (int k = 0; k < CUSTOS_VEC; k++) {\n";
         s += "            S o[" + std::to_string(k.n_outs) + "];\n";
-        s += "            custos_chain(" + list("a", "[u][k]") + ", o);\n";
+        s += "            custos_chain(" + list("a", "[u][k]") + ", o CUSTOS_KC_ARG);\n";
         for (int j = 0; j < k.n_outs; j++) s += "            r" + std::to_string(j) + "[k] = o[" + std::to_string(j) + "];\n";
         s += "        }\n";
         for (int j = 0; j < k.n_outs; j++)
@@ -612,7 +631,7 @@ bool emit_kernel_source(KernelSpec* spec, ParseError* err) {
         for (const ChainStage& stage : k.stages) {
             ConstPlan plan;
             std::string unused;
-            if (!plan_constants(stage.expr, k.dtype, /*all_in_code=*/true, &plan, err)) return false;
+            if (!stage_plan(stage, k.dtype, 0, &plan, err)) return false;
             if (!emit_expr_body(stage.expr, k.dtype, plan, &unused, err)) return false;
         }
     } else if (!emit_expr_body(k.expr, k.dtype, k.consts, &body, err)) {
@@ -696,7 +715,8 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
             return false;
         }
         ConstPlan plan;
-        if (!plan_constants(stage.expr, dtype, /*all_in_code=*/true, &plan, err)) return false;
+        if (!stage_plan(stage, dtype, k.consts.n_params, &plan, err)) return false;
+        k.consts.n_params += stage.n_params;
         uint64_t hs;
         std::vector<uint64_t> literals;
         if (!hash_expr(stage.expr, dtype, plan, &hs, err, &literals)) return false;
@@ -714,7 +734,7 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
         h = fnv1a64(&stage.out, sizeof stage.out, h);
         for (const Node& n : stage.expr.nodes) k.n_literals += n.op == Op::Const;
         k.code_literals.insert(k.code_literals.end(), literals.begin(), literals.end());
-        k.chain_text += "s" + std::to_string(st) + " = " + to_cl_source(stage.expr, names) +
+        k.chain_text += "s" + std::to_string(st) + " = " + to_cl_source(stage.expr, names, &plan) +
                         (stage.out >= 0 ? " -> out" + std::to_string(stage.out) : std::string()) + "; ";
     }
     int32_t tail[7] = {static_cast<int32_t>(Kind::Chain), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
@@ -722,6 +742,10 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     k.stages = std::move(stages);
+    // (the values travel with every launch of the kernel; here only their size counts)
+    size_t param_bytes = 0;
+    for (const ChainStage& stage : k.stages) param_bytes += stage.param_bytes;
+    k.consts.bytes.assign(param_bytes, 0);
     {
         static const char* const dtype_names[] = {"f32", "f64", "i32", "i64", "f16", "bf16", "u8", "i8", "i16", "u16", "u32", "u64",
                                                   "f16n", "bf16n"};

@@ -88,6 +88,11 @@ struct ChainStage {
                               // -(1 + s) for the stored value of stage s
     int out = -1;             // which output pointer of the kernel receives the value; -1: none, a
                               // later stage writes the same memory
+    std::vector<int> slot;    // per node of `expr`: the literal is launch parameter `slot` of this stage, or
+                              // -1 (ConstPlan::slot of the launch's own kernel); empty: every literal in the code
+    int n_params = 0;         // launch parameters of this stage; in the kernel's block they follow those of the
+                              // stages before it
+    size_t param_bytes = 0;   // their size (n_params values of the compute type)
 };
 constexpr int kMaxChainStages = 8, kMaxChainInputs = 8, kMaxChainOutputs = 6;
 
@@ -120,7 +125,8 @@ struct KernelSpec {
 bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
                        const std::vector<std::string>& markers, const Tuning& tuning,
                        bool literals_in_code, KernelSpec* out, ParseError* err, bool with_source = true);
-// The same for a chain kernel (all literals in the code).
+// The same for a chain kernel; a stage's literals are in the code or launch parameters as they are
+// for the kernel of the stage's own launch.
 bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs, const Tuning& tuning,
                       KernelSpec* out, ParseError* err, bool with_source = true);
 // Pointer parameters of a generated kernel's single-launch entry point (= the width of a table

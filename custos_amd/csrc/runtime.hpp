@@ -81,6 +81,8 @@ struct RecNode {
     std::vector<uint64_t> ptrs;  // kernel: operand addresses in parameter order; fill: {ptr}; copy: {dst, src}
     unsigned long long n = 0, head = 0, n_vec = 0, bytes = 0;
     std::vector<uint32_t> pattern;  // fill: the 16 bytes that repeat; empty = zeros
+    std::vector<unsigned char> const_bytes;  // chain kernel: this launch's values of the literal parameters
+                                             // (every other generated kernel carries them in its handle)
     std::vector<Access> acc;
     int level = 0;
     std::vector<uint32_t> deps;  // recorded nodes this one has to follow (filled when a graph is built with per-node edges)
@@ -241,6 +243,10 @@ ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kerne
 // jit.cpp: the kernel for a chain of apply expressions (compiled on first use, then cached).
 int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs,
                      const Tuning& tuning, custos_hip_kernel** out, bool* compiled);
+// The values of a recorded launch's literal parameters.
+inline const std::vector<unsigned char>& literal_values(const RecNode& n) {
+    return n.k->spec.kind == custos_hip::Kind::Chain ? n.const_bytes : n.k->spec.consts.bytes;
+}
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
 // Workgroups of a single launch of `k` over n_vec vectors and n elements with `unroll` vectors per thread.

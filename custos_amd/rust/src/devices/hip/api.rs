@@ -89,7 +89,7 @@ extern "C" {
     pub fn custos_hip_graph_fused_launches(graph: *mut HipGraph, launches: *mut usize) -> i32;
     pub fn custos_hip_chain_emit(dtype: i32, stage_srcs: *const *const c_char, stage_vars: *const i32, n_stages: i32,
                                  sources: *const i32, stage_outs: *const i32, n_inputs: i32, n_outputs: i32,
-                                 buf: *mut c_char, cap: usize, needed: *mut usize, code_size: *mut usize) -> i32;
+                                 literals_as_parameters: i32, buf: *mut c_char, cap: usize, needed: *mut usize, code_size: *mut usize) -> i32;
     pub fn custos_hip_last_launch_shape(dev: *mut HipDeviceHandle, unroll: *mut i32, nontemporal: *mut i32,
                                         alternate: *mut i32) -> i32;
     pub fn custos_hip_expr_canonical(src: *const c_char, markers: *const *const c_char, n_markers: i32,

@@ -401,7 +401,10 @@ int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
  * and writes t, u, y.  Every buffer receives exactly what the separate launches gave it.  Only
  * launches whose address ranges are pairwise equal or disjoint are joined, and only if nothing
  * recorded between them touches what the earlier one reads or writes; a joined launch is
- * producer and consumer in turn (up to 8 expressions, 8 inputs and 6 outputs per kernel).  The
+ * producer and consumer in turn (up to 8 expressions, 8 inputs and 6 outputs per kernel).  A
+ * literal is part of the joined kernel's code or one of its launch parameters as it is for the
+ * launch's own kernel, so expressions that keep arriving with new values share their joined
+ * kernels as they share their own.  The
  * kernels are compiled when the graph is built (at most 16 new ones per graph; a recording that
  * would need more is built as recorded).  No counterpart in the reference, whose captured
  * graphs replay launch by launch (src/devices/cuda/lazy.rs:31-49). */
@@ -413,12 +416,14 @@ int32_t custos_hip_graph_fused_launches(custos_hip_graph *graph, size_t *launche
  * v{stage_vars[s]-1}; `sources` lists, stage after stage, where each variable comes from: the
  * index of an input pointer (0 .. n_inputs-1), or -(1 + t) for the stored value of stage t < s;
  * `stage_outs[s]` is the output pointer (0 .. n_outputs-1) that receives the stage's value, or -1
- * if a later stage writes the same memory.  With `code_size` the source is also compiled for
- * gfx950 and the size of the code object returned. */
+ * if a later stage writes the same memory.  `literals_as_parameters`: the literals are launch
+ * parameters of the kernel (what a stage gets whose own kernel takes them that way, see
+ * custos_hip_expr_compile) instead of part of its code.  With `code_size` the source is also
+ * compiled for gfx950 and the size of the code object returned. */
 int32_t custos_hip_chain_emit(int32_t dtype, const char *const *stage_srcs, const int32_t *stage_vars,
                               int32_t n_stages, const int32_t *sources, const int32_t *stage_outs,
-                              int32_t n_inputs, int32_t n_outputs, char *buf, size_t cap,
-                              size_t *needed, size_t *code_size);
+                              int32_t n_inputs, int32_t n_outputs, int32_t literals_as_parameters,
+                              char *buf, size_t cap, size_t *needed, size_t *code_size);
 /* A recording that comes out as a plain chain (every dependency level one node, or any
  * recording under CUSTOS_HIP_GRAPH_EDGES_CHAIN) of at most `max_nodes` nodes is replayed by
  * issuing its nodes on the compute stream instead of launching an instantiated graph: for a

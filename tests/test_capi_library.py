@@ -172,7 +172,23 @@ def test_chain_kernels_compile_for_every_dtype(dtype):
         assert entry + suffix in text
     # three inputs, three outputs; a stage takes an earlier stage's value as it was stored
     assert "const S* in2, S* out0, S* out1, S* out2" in text
-    assert "const S t1 = custos_store(custos_expr_s1(r0, e2));" in text
+    assert "const S t1 = custos_store(custos_expr_s1(r0, e2 CUSTOS_KC_ARG));" in text
+
+
+def test_chain_kernels_take_literals_as_parameters():
+    """Stages whose own kernels take their literals as launch parameters keep doing so in the joined
+    kernel: one block of scalars, every stage's slots behind those of the stages before it."""
+    stages = [("((v0 * 0.5) + 0.75)", [0], 0), ("(v0 / 3.0)", [-1], 1), ("max(v0, 0.25)", [-2], 2)]
+    for dtype in ("f32", "f64", "f16", "bf16_pernode", "i32", "u8"):
+        st = stages if dtype[0] not in "iu" else [("((v0 * 5) + 7)", [0], 0), ("(v0 / 3)", [-1], 1), ("max(v0, 2)", [-2], 2)]
+        text, size = capi.chain_emit(dtype, st, 1, 3, compile_it=True, literals_as_parameters=True)
+        assert size > 1000
+        # integer divisors stay in the code (a division by a known value is a multiplication)
+        n_params = 3 if dtype[0] in "iu" else 4
+        assert f"struct CustosConsts {{ C c[{n_params}]; }};" in text
+        assert "kc.c[2]" in text and f"kc.c[{n_params - 1}]" in text and f"kc.c[{n_params}]" not in text
+    in_code, _ = capi.chain_emit("f32", stages, 1, 3)
+    assert "CustosConsts {" not in in_code and "kc.c[" not in in_code
 
 
 def test_chain_kernel_stores_what_is_overwritten_only_once():

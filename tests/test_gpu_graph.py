@@ -961,3 +961,54 @@ def test_joined_launches_of_many_buffers_merge(hip):
             hip.apply_fn(b[i], lambda v: v.mul(0.5).add(1.0), out=b[k + i])
             hip.apply_fn2(b[k + i], b[i], lambda p, q: p.mul(q), out=b[2 * k + i])
     assert _both_ways(hip, xs + zeros + zeros, program) == (1, 40)
+
+
+def test_changing_literals_do_not_compile_chain_after_chain(hip):
+    """A literal is part of a joined kernel's code, or one of its launch parameters, as it is for the
+    launch's own kernel: an expression that keeps arriving with new values (its literals have become
+    launch parameters by then) still joins, and a graph per value compiles nothing."""
+    n = 4096
+    x = synth.uniform_f32(7, n, -2, 2)
+    a, b, c = hip.buffer(x), hip.alloc(n), hip.alloc(n)
+
+    def record(rate):
+        hip.capture_begin()
+        hip.apply_fn(a, lambda v: v.mul(rate).add(0.75), out=b)
+        hip.apply_fn(b, lambda v: v.abs().sqrt().mul(rate), out=c)
+        return hip.capture_end()
+
+    def check(rate, g):
+        assert (g.kernel_nodes, g.fused_launches) == (1, 1)
+        b.clear()
+        c.clear()
+        g.launch()
+        hip.sync()
+        want_b = x * np.float32(rate) + np.float32(0.75)
+        assert_bits_equal(b.read(), want_b)
+        assert_bits_equal(c.read(), np.sqrt(np.abs(want_b)) * np.float32(rate))
+        g.destroy()
+
+    check(0.5, record(0.5))                           # the first values: compiled into the code
+    check(0.25, record(0.25))                         # the second: the forms that take them as parameters are compiled
+    before = hip.cache_stats()[0]
+    for step in range(3, 9):
+        check(1.0 / step, record(1.0 / step))
+    assert hip.cache_stats()[0] == before             # six more values, nothing compiled
+    # many buffers with a value of their own each: one merged launch, every row its own parameters
+    bufs = [(hip.buffer(x), hip.alloc(n), hip.alloc(n)) for _ in range(12)]
+    hip.capture_begin()
+    for i, (p, q, r) in enumerate(bufs):
+        rate = 0.3 + 0.01 * i
+        hip.apply_fn(p, lambda v: v.mul(rate).add(0.75), out=q)
+        hip.apply_fn(q, lambda v: v.abs().sqrt().mul(rate), out=r)
+    g = hip.capture_end()
+    assert (g.kernel_nodes, g.fused_launches) == (1, 12)
+    g.launch()
+    hip.sync()
+    for i, (p, q, r) in enumerate(bufs):
+        rate = np.float32(0.3 + 0.01 * i)
+        want_q = x * rate + np.float32(0.75)
+        assert_bits_equal(q.read(), want_q, f"buffer {i}")
+        assert_bits_equal(r.read(), np.sqrt(np.abs(want_q)) * rate, f"buffer {i}")
+    g.destroy()
+    assert hip.cache_stats()[0] == before
