@@ -963,10 +963,20 @@ def test_joined_launches_of_many_buffers_merge(hip):
     assert _both_ways(hip, xs + zeros + zeros, program) == (1, 40)
 
 
-def test_changing_literals_do_not_compile_chain_after_chain(hip):
+@pytest.fixture
+def fresh_device():
+    """A device handle of its own: which literal values a kernel has seen decides whether they are in
+    its code, so a test of that starts from nothing."""
+    dev = custos_amd.HIP(0)
+    yield dev
+    dev.close()
+
+
+def test_changing_literals_do_not_compile_chain_after_chain(fresh_device):
     """A literal is part of a joined kernel's code, or one of its launch parameters, as it is for the
     launch's own kernel: an expression that keeps arriving with new values (its literals have become
     launch parameters by then) still joins, and a graph per value compiles nothing."""
+    hip = fresh_device
     n = 4096
     x = synth.uniform_f32(7, n, -2, 2)
     a, b, c = hip.buffer(x), hip.alloc(n), hip.alloc(n)
