@@ -218,8 +218,9 @@ ChainBuild chain_of(const RecNode& n) {
     return c;
 }
 
-// `producer` followed by `consumer` as one chain, or false if they may not be joined.
-bool join_chains(const ChainBuild& producer, const ChainBuild& consumer, uint64_t bytes, ChainBuild* joined) {
+// `producer` followed by `consumer` as one chain (which takes `producer`'s place), or false if
+// they may not be joined (`producer` is left as it was).
+bool join_chains(ChainBuild& producer, const ChainBuild& consumer, uint64_t bytes, ChainBuild* joined) {
     // every range of the one against every range of the other, one of them written: equal or disjoint
     auto clash = [&](uint64_t p, uint64_t q) { return p != q && p < q + bytes && q < p + bytes; };
     for (uint64_t w : producer.stage_ptr) {
@@ -234,13 +235,23 @@ bool join_chains(const ChainBuild& producer, const ChainBuild& consumer, uint64_
     bool reads_producer = false;
     for (uint64_t q : consumer.ext) reads_producer = reads_producer || writer_of(producer, q) >= 0;
     if (!reads_producer) return false;
-    ChainBuild c = producer;
+    // the limits of one kernel, before anything is moved
+    size_t inputs = producer.ext.size(), outputs = 0;
+    for (uint64_t q : consumer.ext)
+        inputs += writer_of(producer, q) < 0 && std::find(producer.ext.begin(), producer.ext.end(), q) == producer.ext.end();
+    for (size_t s = 0; s < producer.size(); s++)
+        outputs += writer_of(producer, producer.stage_ptr[s]) == static_cast<int>(s) && writer_of(consumer, producer.stage_ptr[s]) < 0;
+    outputs += distinct_outputs(consumer);
+    if (producer.size() + consumer.size() > static_cast<size_t>(kMaxChainStages) || inputs > static_cast<size_t>(kMaxChainInputs) ||
+        outputs > static_cast<size_t>(kMaxChainOutputs))
+        return false;
     const int shift = static_cast<int>(producer.size());
+    ChainBuild c = std::move(producer);
     // what an input pointer of the consumer becomes: the stored value of the producer's stage
     // that wrote that memory last, or an input pointer of the joined kernel
     std::vector<int> mapped;
     for (uint64_t q : consumer.ext) {
-        const int w = writer_of(producer, q);
+        const int w = writer_of(c, q);
         mapped.push_back(w >= 0 ? -(1 + w) : input_index(&c, q));
     }
     for (size_t s = 0; s < consumer.size(); s++) {
@@ -250,9 +261,6 @@ bool join_chains(const ChainBuild& producer, const ChainBuild& consumer, uint64_
         c.stage_ptr.push_back(consumer.stage_ptr[s]);
         c.stage_kernel.push_back(consumer.stage_kernel[s]);
     }
-    if (c.size() > static_cast<size_t>(kMaxChainStages) || c.ext.size() > static_cast<size_t>(kMaxChainInputs) ||
-        distinct_outputs(c) > static_cast<size_t>(kMaxChainOutputs))
-        return false;
     *joined = std::move(c);
     return true;
 }
@@ -271,7 +279,7 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
     };
     std::vector<RecNode> out;
     std::vector<char> dead;
-    std::vector<ChainBuild> chain_at;  // per entry of `out`: its chain if it has more than one stage
+    std::vector<int32_t> cand_at;  // per entry of `out`: its candidate (whose chain it stands for), or -1
     std::vector<Candidate> cands;
     std::unordered_map<uint64_t, std::vector<uint32_t>> buckets;
     size_t closed_below = 0;  // every candidate with a lower id is closed (a kernel with unknown memory use came by)
@@ -282,7 +290,7 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
             closed_below = cands.size();
             out.push_back(node);
             dead.push_back(0);
-            chain_at.emplace_back();
+            cand_at.push_back(-1);
             continue;
         }
         // open candidates this node conflicts with
@@ -328,7 +336,7 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
         }
         out.push_back(node);
         dead.push_back(0);
-        chain_at.emplace_back();
+        cand_at.push_back(-1);
         if (!fusable) continue;
         Candidate c;
         c.at = out.size() - 1;
@@ -340,7 +348,7 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
         for (const Access& a : c.acc)
             for (uint64_t ch = a.begin >> kChunkShift; ch <= (a.end - 1) >> kChunkShift; ch++)
                 buckets[ch].push_back(static_cast<uint32_t>(cands.size()));
-        if (chain.size() > 1) chain_at.back() = chain;
+        cand_at.back() = static_cast<int32_t>(cands.size());
         c.chain = std::move(chain);
         cands.push_back(std::move(c));
     }
@@ -352,8 +360,9 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
     std::map<std::vector<uint64_t>, custos_hip_kernel*> kernel_of_shape;
     for (size_t i = 0; i < out.size(); i++) {
         if (dead[i]) continue;
-        RecNode node = out[i];
-        const ChainBuild& chain = chain_at[i];
+        RecNode node = std::move(out[i]);
+        static const ChainBuild single;
+        const ChainBuild& chain = cand_at[i] >= 0 ? cands[static_cast<size_t>(cand_at[i])].chain : single;
         if (chain.size() > 1) {
             std::vector<int> out_of(chain.size(), -1);
             std::vector<uint64_t> outs;
