@@ -463,6 +463,17 @@ def bench_others(dev, args, stack_c5):
     alone = "the same launch repeated by itself (in the sequence above each kernel finds what the other left in the caches)"
     e["forward"] = {"ms": round(ms_f, 5), "GBps": round(8 * n / (ms_f * 1e-3) / 1e9, 2), "kernel": dev.kernel_name(kf), "what": alone}
     e["backward"] = {"ms": round(ms_b, 5), "GBps": round(16 * n / (ms_b * 1e-3) / 1e9, 2), "kernel": dev.kernel_name(kb), "what": alone}
+    # forward + backward recorded once and replayed (a lazy run of the two): the graph build joins them
+    # into one kernel that loads x once (20 instead of 24 B/element) and writes y and x_grad
+    dev.capture_begin()
+    c3_step()
+    g3 = dev.capture_end()
+    ms_g, replays_g = time_floor(dev, g3.launch)
+    e["recorded_and_replayed"] = {"ms": round(ms_g, 5), "replays": replays_g, "kernel_nodes": g3.kernel_nodes,
+                                  "launches_joined_into_later_ones": g3.fused_launches,
+                                  "GBps_on_24B": round(24 * n / (ms_g * 1e-3) / 1e9, 2),
+                                  "moved_GBps_on_20B": round(20 * n / (ms_g * 1e-3) / 1e9, 2)}
+    g3.destroy()
     out["c3"] = e
     del xb, ygb, yb, gb
 

@@ -141,6 +141,10 @@ void assign_levels(std::vector<RecNode>& nodes, bool edges) {
 // by another lane at another time.  And nothing recorded between the two conflicts with the
 // producer (reads what it writes, writes what it reads or writes): the joined launch takes the
 // consumer's place in the recording.  Joined launches are producers and consumers in turn.
+//
+// Two launches that only READ a common input (the forward launch of an operation and its
+// gradient launch both read x) are joined under the same conditions: the earlier one commutes
+// with everything up to the later one, and the joined kernel loads the common input once.
 
 struct ChainBuild {
     // per stage: the kernel of its launch (whose expression it evaluates), where each variable of
@@ -219,8 +223,10 @@ ChainBuild chain_of(const RecNode& n) {
 }
 
 // `producer` followed by `consumer` as one chain (which takes `producer`'s place), or false if
-// they may not be joined (`producer` is left as it was).
-bool join_chains(ChainBuild& producer, const ChainBuild& consumer, uint64_t bytes, ChainBuild* joined) {
+// they may not be joined (`producer` is left as it was).  The consumer reads what the producer
+// wrote -- or, with `sharing`, the two only read a common input, which the joined kernel then
+// loads once.
+bool join_chains(ChainBuild& producer, const ChainBuild& consumer, uint64_t bytes, bool sharing, ChainBuild* joined) {
     // every range of the one against every range of the other, one of them written: equal or disjoint
     auto clash = [&](uint64_t p, uint64_t q) { return p != q && p < q + bytes && q < p + bytes; };
     for (uint64_t w : producer.stage_ptr) {
@@ -232,9 +238,11 @@ bool join_chains(ChainBuild& producer, const ChainBuild& consumer, uint64_t byte
     for (uint64_t w : consumer.stage_ptr)
         for (uint64_t p : producer.ext)
             if (clash(w, p)) return false;
-    bool reads_producer = false;
-    for (uint64_t q : consumer.ext) reads_producer = reads_producer || writer_of(producer, q) >= 0;
-    if (!reads_producer) return false;
+    bool related = false;
+    for (uint64_t q : consumer.ext)
+        related = related || writer_of(producer, q) >= 0 ||
+                  (sharing && std::find(producer.ext.begin(), producer.ext.end(), q) != producer.ext.end());
+    if (!related) return false;
     // the limits of one kernel, before anything is moved
     size_t inputs = producer.ext.size(), outputs = 0;
     for (uint64_t q : consumer.ext)
@@ -269,7 +277,7 @@ bool join_chains(ChainBuild& producer, const ChainBuild& consumer, uint64_t byte
 // chains are compiled here, at most kMaxNewChainKernels of them per graph -- a recording that
 // would need more stays as it is, as does one for which a compilation fails.
 constexpr size_t kMaxNewChainKernels = 16;
-int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, size_t* fused_away) {
+int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, bool share_reads, size_t* fused_away) {
     const std::vector<RecNode>& nodes = *recorded;
     struct Candidate {
         size_t at;  // index into `out`
@@ -284,7 +292,7 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
     std::unordered_map<uint64_t, std::vector<uint32_t>> buckets;
     size_t closed_below = 0;  // every candidate with a lower id is closed (a kernel with unknown memory use came by)
     size_t joined_launches = 0;
-    std::vector<uint32_t> hits;
+    std::vector<uint32_t> hits, sharers;
     for (const RecNode& node : nodes) {
         if (node.type == RecNode::Source) {
             closed_below = cands.size();
@@ -293,8 +301,9 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
             cand_at.push_back(-1);
             continue;
         }
-        // open candidates this node conflicts with
+        // open candidates this node conflicts with, and those that read exactly what it reads
         hits.clear();
+        sharers.clear();
         for (const Access& a : node.acc) {
             if (a.end <= a.begin) continue;
             for (uint64_t c = a.begin >> kChunkShift; c <= (a.end - 1) >> kChunkShift; c++) {
@@ -305,11 +314,13 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
                 for (uint32_t id : ids) {
                     if (id < closed_below || !cands[id].open) continue;  // dropped from the list
                     ids[kept++] = id;
-                    for (const Access& b : cands[id].acc)
-                        if ((a.write || b.write) && a.begin < b.end && b.begin < a.end) {
-                            hits.push_back(id);
-                            break;
-                        }
+                    bool conflict = false, same_read = false;
+                    for (const Access& b : cands[id].acc) {
+                        conflict = conflict || ((a.write || b.write) && a.begin < b.end && b.begin < a.end);
+                        same_read = same_read || (!a.write && !b.write && a.begin == b.begin && a.end == b.end);
+                    }
+                    if (conflict) hits.push_back(id);
+                    else if (same_read && share_reads) sharers.push_back(id);
                 }
                 ids.resize(kept);
             }
@@ -329,8 +340,25 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, s
                 pn.k->spec.tuning.block_threads != node.k->spec.tuning.block_threads)
                 continue;
             ChainBuild joined;
-            if (!join_chains(p.chain, chain, bytes, &joined)) continue;
+            if (!join_chains(p.chain, chain, bytes, /*sharing=*/false, &joined)) continue;
             chain = std::move(joined);
+            dead[p.at] = 1;
+            joined_launches++;
+        }
+        // then the candidates that only share an input with it (they stay open if they cannot be joined)
+        std::sort(sharers.begin(), sharers.end());
+        sharers.erase(std::unique(sharers.begin(), sharers.end()), sharers.end());
+        for (uint32_t id : sharers) {
+            Candidate& p = cands[id];
+            if (!fusable || !p.open || std::binary_search(hits.begin(), hits.end(), id)) continue;
+            const RecNode& pn = out[p.at];
+            if (pn.k->spec.dtype != node.k->spec.dtype || pn.n != node.n || pn.head != node.head || pn.n_vec != node.n_vec ||
+                pn.k->spec.tuning.block_threads != node.k->spec.tuning.block_threads)
+                continue;
+            ChainBuild joined;
+            if (!join_chains(p.chain, chain, bytes, /*sharing=*/true, &joined)) continue;
+            chain = std::move(joined);
+            p.open = false;
             dead[p.at] = 1;
             joined_launches++;
         }
@@ -880,8 +908,11 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     if (dev->fusing) {
         // (a recording that cannot be joined -- too many new kernels, a kernel that does not
         // compile -- is built as it was recorded)
+        // (joining launches that only share an input makes for more kinds of kernels: left out
+        // if that is what takes the recording over the limit)
         const std::string error_before = dev->last_error;
-        if (fuse_producers(dev, &nodes, &g->fused_away) != CUSTOS_HIP_OK) {
+        if (fuse_producers(dev, &nodes, /*share_reads=*/true, &g->fused_away) != CUSTOS_HIP_OK &&
+            fuse_producers(dev, &nodes, /*share_reads=*/false, &g->fused_away) != CUSTOS_HIP_OK) {
             g->fused_away = 0;
             dev->last_error = error_before;
         }

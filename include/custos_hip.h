@@ -394,7 +394,8 @@ int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
  * recorded apply or unary-gradient launch whose output a later recorded apply or unary-gradient
  * launch reads element for element (same address, length and element type; a gradient launch
  * counts as the expression `lhs_grad + (out_grad * f'(lhs))` stored to lhs_grad) becomes one
- * kernel with that launch: both expressions
+ * kernel with that launch (so do two such launches that only read a common input, which is then
+ * loaded once): both expressions
  * are evaluated per element, both results are stored where the two launches stored them, and
  * the second expression takes the first result -- as it was stored, rounded to the storage type
  * -- from a register.  `t = a * b; u = t + c; y = f(u)` replays as one launch that reads a, b, c

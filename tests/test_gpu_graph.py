@@ -176,18 +176,22 @@ def test_merged_launches_of_different_lengths(hip, oracle):
         assert_bits_equal(huge_out.read(), oracle.apply_fn(f, huge.read()))
     g.destroy()
 
-    # equal lengths only: the uniform grid, still one node
-    hip.capture_begin()
-    same = [hip.alloc(lens[0]) for _ in range(8)]
-    for o in same:
-        hip.apply_fn(bufs[0], f, out=o)
-    g = hip.capture_end()
-    assert g.stats() == (8, 1, 1)
-    g.launch()
-    hip.sync()
-    for o in same:
-        assert_bits_equal(o.read(), oracle.apply_fn(f, xs[0]))
-    g.destroy()
+    # equal lengths only: the uniform grid, still one node.  (As recorded: eight launches that read
+    # the same input are otherwise joined into kernels that load it once, six outputs at most each.)
+    for fusing, want_stats in ((False, (8, 1, 1)), (True, (8, 2, 1))):
+        hip.set_graph_fusing(fusing)
+        hip.capture_begin()
+        same = [hip.alloc(lens[0]) for _ in range(8)]
+        for o in same:
+            hip.apply_fn(bufs[0], f, out=o)
+        g = hip.capture_end()
+        hip.set_graph_fusing(True)
+        assert g.stats() == want_stats
+        g.launch()
+        hip.sync()
+        for o in same:
+            assert_bits_equal(o.read(), oracle.apply_fn(f, xs[0]))
+        g.destroy()
 
     # unary gradient, f16 storage, lengths with tails
     d = lambda v: v.mul(2.0)
@@ -904,6 +908,22 @@ def test_producers_join_their_consumers(hip):
         b[5].clear()
         hip.apply_fn(b[1], g, out=b[2])
     assert _both_ways(hip, xs, untouched_in_between) == (3, 1)
+
+    def forward_and_gradient_share_their_input(b):    # y = f(x); g += o * f'(x): x is loaded once
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.add_unary_grad(b[0], b[2], b[3], lambda v: v.mul(0.5).abs())
+    assert _both_ways(hip, xs, forward_and_gradient_share_their_input) == (1, 1)
+
+    def readers_of_one_input(b):    # five launches that read b[0] and nothing of each other
+        for i, fn in enumerate((f, g, h, f, g)):
+            hip.apply_fn(b[0], fn, out=b[1 + i])
+    assert _both_ways(hip, xs, readers_of_one_input) == (1, 4)
+
+    def reader_after_a_writer(b):   # the second reader comes after the input was rewritten: not the same value
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.apply_fn(b[2], h, out=b[0])
+        hip.apply_fn(b[0], g, out=b[3])
+    assert _both_ways(hip, xs, reader_after_a_writer) == (2, 1)
 
     def long_chain(b):              # at most eight expressions per kernel
         for i in range(20):
