@@ -345,12 +345,18 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, b
             dead[p.at] = 1;
             joined_launches++;
         }
-        // then the candidates that only share an input with it (they stay open if they cannot be joined)
+        // then the candidate that only shares an input with it (it stays open if it cannot be
+        // joined).  Only if there is exactly one: an input that several open launches read is a
+        // common operand (a bias, a mask), not a sign that those launches belong together.
         std::sort(sharers.begin(), sharers.end());
         sharers.erase(std::unique(sharers.begin(), sharers.end()), sharers.end());
+        sharers.erase(std::remove_if(sharers.begin(), sharers.end(),
+                                     [&](uint32_t id) { return !cands[id].open || std::binary_search(hits.begin(), hits.end(), id); }),
+                      sharers.end());
+        if (sharers.size() != 1) sharers.clear();
         for (uint32_t id : sharers) {
             Candidate& p = cands[id];
-            if (!fusable || !p.open || std::binary_search(hits.begin(), hits.end(), id)) continue;
+            if (!fusable) continue;
             const RecNode& pn = out[p.at];
             if (pn.k->spec.dtype != node.k->spec.dtype || pn.n != node.n || pn.head != node.head || pn.n_vec != node.n_vec ||
                 pn.k->spec.tuning.block_threads != node.k->spec.tuning.block_threads)

@@ -919,6 +919,23 @@ def test_producers_join_their_consumers(hip):
             hip.apply_fn(b[0], fn, out=b[1 + i])
     assert _both_ways(hip, xs, readers_of_one_input) == (1, 4)
 
+    def common_operand_of_separate_chains(b):         # b[5] is read by three chains that have nothing else in common
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.apply_fn2(b[1], b[5], add, out=b[1])
+        hip.apply_fn(b[2], g, out=b[3])
+        hip.apply_fn2(b[3], b[5], add, out=b[3])      # the one open reader of b[5] so far comes along
+        hip.apply_fn(b[4], h, out=b[4])
+        hip.apply_fn2(b[4], b[5], mul, out=b[4])      # and so does the joined launch
+    assert _both_ways(hip, xs, common_operand_of_separate_chains) == (1, 5)
+
+    def common_operand_of_many_chains(b):             # a kernel holds eight expressions: the fourth chain starts anew,
+        for _ in range(5):                            # and with two open readers of b[5] the fifth joins neither
+            hip.apply_fn(b[0], f, out=b[1])
+            hip.apply_fn2(b[1], b[5], add, out=b[2])
+            b = b[2:4] + b[0:2] + b[4:]               # the next chain over the other buffers (b[5] stays)
+    five = _both_ways(hip, xs, common_operand_of_many_chains)
+    assert five[0] >= 2 and five[0] + five[1] >= 8
+
     def reader_after_a_writer(b):   # the second reader comes after the input was rewritten: not the same value
         hip.apply_fn(b[0], f, out=b[1])
         hip.apply_fn(b[2], h, out=b[0])
