@@ -468,6 +468,17 @@ def bench_others(dev, args, stack_c5):
     dev.capture_begin()
     c3_step()
     g3 = dev.capture_end()
+    # (one replay over a fresh gradient, checked against the CPU port on the first 2^20 elements)
+    m3 = 1 << 20
+    gb.slice(0, m3).write(np.full(m3, 0.1, dtype=np.float32))
+    yb.slice(0, m3).clear()
+    g3.launch()
+    dev.sync()
+    want_y = cpu_oracle.c3_tanh_fwd(x[:m3])
+    want_g = cpu_oracle.c3_tanh_bwd(x[:m3], np.full(m3, 0.1, dtype=np.float32), yg[:m3])
+    got_y, got_g = yb.slice(0, m3).read(), gb.slice(0, m3).read()
+    assert np.max(np.abs(got_y.view(np.int32).astype(np.int64) - want_y.view(np.int32).astype(np.int64))) <= 4, "c3 replay: y"
+    assert np.max(np.abs(got_g - want_g)) <= 2e-6, "c3 replay: x_grad"
     ms_g, replays_g = time_floor(dev, g3.launch)
     e["recorded_and_replayed"] = {"ms": round(ms_g, 5), "replays": replays_g, "kernel_nodes": g3.kernel_nodes,
                                   "launches_joined_into_later_ones": g3.fused_launches,
