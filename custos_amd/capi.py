@@ -112,6 +112,7 @@ PROTOTYPES = {
     "custos_hip_kernel_hash": (C.c_uint64, [_P]),
     "custos_hip_preferred_shape": (C.c_int32, [C.c_uint64, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "custos_hip_set_graph_fusing": (C.c_int32, [_P, C.c_int32]),
+    "custos_hip_graph_node_kernel": (C.c_int32, [_P, C.c_size_t, C.POINTER(C.c_char_p)]),
     "custos_hip_graph_fused_launches": (C.c_int32, [_P, C.POINTER(C.c_size_t)]),
     "custos_hip_chain_emit": (C.c_int32, [C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.c_int32, C.POINTER(C.c_int32),
                                           C.POINTER(C.c_int32), C.c_int32, C.c_int32, C.c_int32, C.c_char_p, C.c_size_t,

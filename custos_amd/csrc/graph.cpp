@@ -979,7 +979,13 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
             LoweredNode ln;
             int32_t rc = lower_node(dev, nodes, p, reinterpret_cast<uint64_t>(g->table), rev, &ln);
             if (rc != CUSTOS_HIP_OK) return rc;
-            if (!ln.is_copy) g->kernel_nodes++;
+            if (!ln.is_copy) {
+                g->kernel_nodes++;
+                const RecNode& first = nodes[p.members[0]];
+                if (first.type == RecNode::Fill) g->node_names.push_back(first.pattern.empty() ? "custos_fill_zero" : "custos_fill_pattern");
+                else if (first.type == RecNode::Source) g->node_names.push_back(first.k->spec.name);
+                else g->node_names.push_back(p.kern->spec.name + (p.members.size() == 1 ? "" : p.ragged ? "_ragged" : "_batched"));
+            }
             lowered[level].push_back(std::move(ln));
             total++;
         }
@@ -1160,6 +1166,13 @@ int32_t custos_hip_graph_launch(custos_hip_device* dev, custos_hip_graph* graph)
 int32_t custos_hip_graph_node_count(custos_hip_graph* graph, size_t* kernel_nodes) {
     if (!graph || !kernel_nodes) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
     *kernel_nodes = graph->kernel_nodes;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_node_kernel(custos_hip_graph* graph, size_t node, const char** name) {
+    if (!graph || !name) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    if (node >= graph->node_names.size()) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "no such kernel node");
+    *name = graph->node_names[node].c_str();
     return CUSTOS_HIP_OK;
 }
 

@@ -66,6 +66,7 @@ struct custos_hip_graph {
     std::vector<uint64_t> signature;
     std::array<uint64_t, 4> built_with{};
     size_t fused_away = 0;    // recorded launches that became stages of a later launch's kernel
+    std::vector<std::string> node_names;  // entry point of every kernel node, in the order of the chain / the levels
     // how long the last wait took that waited for one launch of this graph and nothing else
     uint64_t last_wait_ns = 0;
 };

@@ -104,6 +104,15 @@ class Graph:
         self.device._check(self.device.lib.custos_hip_graph_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
         return a.value, b.value, c.value
 
+    def kernel_names(self):
+        """Entry points of the graph's kernel nodes in replay order, as a profiler lists them."""
+        names = []
+        for i in range(self.kernel_nodes):
+            name = C.c_char_p()
+            self.device._check(self.device.lib.custos_hip_graph_node_kernel(self.handle, i, C.byref(name)))
+            names.append(name.value.decode())
+        return names
+
     @property
     def fused_launches(self) -> int:
         """Recorded launches that became part of a later launch's kernel."""

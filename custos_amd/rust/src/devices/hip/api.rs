@@ -86,6 +86,7 @@ extern "C" {
     pub fn custos_hip_preferred_shape(footprint_bytes: u64, n_operands: i32, unroll: *mut i32,
                                       nontemporal: *mut i32, alternate: *mut i32) -> i32;
     pub fn custos_hip_set_graph_fusing(dev: *mut HipDeviceHandle, enabled: i32) -> i32;
+    pub fn custos_hip_graph_node_kernel(graph: *mut HipGraph, node: usize, name: *mut *const c_char) -> i32;
     pub fn custos_hip_graph_fused_launches(graph: *mut HipGraph, launches: *mut usize) -> i32;
     pub fn custos_hip_chain_emit(dtype: i32, stage_srcs: *const *const c_char, stage_vars: *const i32, n_stages: i32,
                                  sources: *const i32, stage_outs: *const i32, n_inputs: i32, n_outputs: i32,

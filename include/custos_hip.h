@@ -410,6 +410,10 @@ int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
  * would need more is built as recorded).  No counterpart in the reference, whose captured
  * graphs replay launch by launch (src/devices/cuda/lazy.rs:31-49). */
 int32_t custos_hip_set_graph_fusing(custos_hip_device *dev, int32_t enabled);
+/* The entry point kernel node `node` (0 .. kernel_nodes-1, in replay order) of a built graph
+ * launches, as a profiler lists it; the string lives as long as the graph.  No counterpart in
+ * the reference. */
+int32_t custos_hip_graph_node_kernel(custos_hip_graph *graph, size_t node, const char **name);
 /* Recorded launches of a built graph that became part of a later launch's kernel. */
 int32_t custos_hip_graph_fused_launches(custos_hip_graph *graph, size_t *launches);
 /* Host-only: the source of the kernel that joins `n_stages` expressions (for tests and

@@ -1059,3 +1059,21 @@ def test_changing_literals_do_not_compile_chain_after_chain(fresh_device):
         assert_bits_equal(r.read(), np.sqrt(np.abs(want_q)) * rate, f"buffer {i}")
     g.destroy()
     assert hip.cache_stats()[0] == before
+
+
+def test_graph_names_its_kernels(hip):
+    """The entry points a built graph launches, as a profiler lists them."""
+    n = 2048
+    a, b, c = hip.buffer(synth.uniform_f32(1, n, -1, 1)), hip.alloc(n), hip.alloc(n)
+    hip.capture_begin()
+    hip.apply_fn(a, lambda v: v.mul(2.0), out=b)
+    hip.apply_fn(b, lambda v: v.add(1.0), out=c)
+    c.slice(0, 16).clear()
+    g = hip.capture_end()
+    names = g.kernel_names()
+    assert len(names) == g.kernel_nodes == 2
+    assert names[0].startswith("custos_chain_f32_") and names[1] == "custos_fill_zero"
+    import ctypes as C
+    name = C.c_char_p()
+    assert hip.lib.custos_hip_graph_node_kernel(g.handle, 2, C.byref(name)) == capi.ERR_INVALID_ARGUMENT
+    g.destroy()
