@@ -374,10 +374,12 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device *dev, custos_hip_kern
 int32_t custos_hip_capture_begin(custos_hip_device *dev);
 /* Ends recording and instantiates an executable graph (LazyCudaGraph::new).
  * The graph is built from the recorded work, not replayed launch by launch:
- * the work is sorted into dependency levels (work of one level touches no common
- * memory), and launches of one level that use the same kernel are merged into one
- * grid, whatever their lengths (1024 buffers x 3 operations replay as 3 kernel
- * nodes). How the nodes are ordered: custos_hip_set_graph_edges. */
+ * launches that read what an earlier launch wrote are joined with it into one
+ * kernel (custos_hip_set_graph_fusing), the work is sorted into dependency levels
+ * (work of one level touches no common memory), and launches of one level that use
+ * the same kernel are merged into one grid, whatever their lengths (1024 buffers x 3
+ * operations replay as ONE kernel node; 3 with the joining switched off). How the
+ * nodes are ordered: custos_hip_set_graph_edges. */
 int32_t custos_hip_capture_end(custos_hip_device *dev, custos_hip_graph **graph);
 /* capture_end for a caller that records the same program before every run (the reference's
  * Lazy::run calls every recorded operation again before each launch of its graph,
