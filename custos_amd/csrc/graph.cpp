@@ -274,9 +274,9 @@ bool join_chains(ChainBuild& producer, const ChainBuild& consumer, uint64_t byte
 }
 
 // The recording with producers joined into their consumers (see above); kernels for the new
-// chains are compiled here, at most kMaxNewChainKernels of them per graph -- a recording that
-// would need more stays as it is, as does one for which a compilation fails.
-constexpr size_t kMaxNewChainKernels = 16;
+// chains are compiled here, at most `dev->fusing_new_kernels` of them per graph: a chain whose
+// kernel is neither cached nor compiled within that limit (or does not compile) stays the
+// launches it was recorded as.
 int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, bool share_reads, size_t* fused_away) {
     const std::vector<RecNode>& nodes = *recorded;
     struct Candidate {
@@ -412,8 +412,9 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, b
                 shape.push_back(static_cast<uint64_t>(static_cast<int64_t>(out_of[s])));
                 for (int from : chain.source[s]) shape.push_back(static_cast<uint64_t>(static_cast<int64_t>(from)));
             }
-            custos_hip_kernel*& k = kernel_of_shape[shape];
-            if (!k) {
+            auto known = kernel_of_shape.find(shape);
+            if (known == kernel_of_shape.end()) {
+                custos_hip_kernel* k = nullptr;
                 std::vector<ChainStage> stages(chain.size());
                 for (size_t s = 0; s < chain.size(); s++) {
                     const custos_hip_kernel* sk = chain.stage_kernel[s];
@@ -432,11 +433,40 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, b
                 bool compiled = false;
                 Tuning tuning = node.k->spec.tuning;
                 tuning.unroll = 0;  // (only kernels whose vectors per thread were left open are joined)
-                const int32_t rc = chain_kernel(dev, node.k->spec.dtype, std::move(stages), static_cast<int>(chain.ext.size()),
-                                                static_cast<int>(outs.size()), tuning, &k, &compiled);
-                if (rc != CUSTOS_HIP_OK) return rc;
+                // a kernel that is not there yet is compiled while the limit lasts; a shape without a
+                // kernel (the limit, a compilation that failed) stays the launches it was recorded as
+                if (compiled_here >= dev->fusing_new_kernels) {
+                    KernelSpec probe;
+                    ParseError err;
+                    const int n_ext = static_cast<int>(chain.ext.size()), n_outs = static_cast<int>(outs.size());
+                    if (build_chain_spec(node.k->spec.dtype, stages, n_ext, n_outs, tuning, &probe, &err, /*with_source=*/false))
+                        k = cached_chain_kernel(dev, probe);
+                } else if (chain_kernel(dev, node.k->spec.dtype, std::move(stages), static_cast<int>(chain.ext.size()),
+                                        static_cast<int>(outs.size()), tuning, &k, &compiled) != CUSTOS_HIP_OK) {
+                    k = nullptr;
+                }
                 compiled_here += compiled;
-                if (compiled_here > kMaxNewChainKernels) return CUSTOS_HIP_ERR_TOO_LARGE;
+                known = kernel_of_shape.emplace(std::move(shape), k).first;
+            }
+            custos_hip_kernel* const k = known->second;
+            if (!k) {
+                // the chain's launches again, in the order of its stages
+                const uint64_t bytes = node.n * dtype_size(node.k->spec.dtype);
+                for (size_t s = 0; s < chain.size(); s++) {
+                    RecNode single = node;
+                    single.k = const_cast<custos_hip_kernel*>(chain.stage_kernel[s]);
+                    single.ptrs.clear();
+                    single.acc.clear();
+                    single.const_bytes.clear();
+                    for (int from : chain.source[s]) single.ptrs.push_back(from >= 0 ? chain.ext[static_cast<size_t>(from)] : chain.stage_ptr[static_cast<size_t>(-from - 1)]);
+                    if (single.k->spec.kind != Kind::UnaryGrad) single.ptrs.push_back(chain.stage_ptr[s]);
+                    for (size_t p = 0; p < single.ptrs.size(); p++) {
+                        const bool written = single.k->spec.kind == Kind::UnaryGrad ? p == 1 : p + 1 == single.ptrs.size();
+                        single.acc.push_back({single.ptrs[p], single.ptrs[p] + bytes, written});
+                    }
+                    fused.push_back(std::move(single));
+                }
+                continue;
             }
             const uint64_t bytes = node.n * dtype_size(node.k->spec.dtype);
             node.const_bytes.clear();
@@ -914,14 +944,9 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
     if (dev->fusing) {
         // (a recording that cannot be joined -- too many new kernels, a kernel that does not
         // compile -- is built as it was recorded)
-        // (joining launches that only share an input makes for more kinds of kernels: left out
-        // if that is what takes the recording over the limit)
         const std::string error_before = dev->last_error;
-        if (fuse_producers(dev, &nodes, /*share_reads=*/true, &g->fused_away) != CUSTOS_HIP_OK &&
-            fuse_producers(dev, &nodes, /*share_reads=*/false, &g->fused_away) != CUSTOS_HIP_OK) {
-            g->fused_away = 0;
-            dev->last_error = error_before;
-        }
+        if (fuse_producers(dev, &nodes, /*share_reads=*/true, &g->fused_away) != CUSTOS_HIP_OK) g->fused_away = 0;
+        dev->last_error = error_before;
     }
     const bool serial = dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN || dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN_BY_LEVEL;
     // The order of a chain only matters where a launch is large enough for the caches to matter;
@@ -1118,7 +1143,9 @@ int32_t custos_hip_set_graph_batching(custos_hip_device* dev, int32_t enabled) {
 
 int32_t custos_hip_set_graph_fusing(custos_hip_device* dev, int32_t enabled) {
     REQUIRE_DEV(dev);
+    if (enabled < 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "negative value");
     dev->fusing = enabled != 0;
+    dev->fusing_new_kernels = enabled > 1 ? static_cast<size_t>(enabled) : 16;
     return CUSTOS_HIP_OK;
 }
 

@@ -168,6 +168,7 @@ struct custos_hip_device {
     unsigned long long launch_parity = 0;  // direction of the last launch that alternates
     bool batching = true;            // merge equal independent launches of a level into one grid
     bool fusing = true;              // a recorded apply launch is joined with the apply launches that read what it wrote
+    size_t fusing_new_kernels = 16;  // kernels of joined launches a graph build may compile
     std::vector<RecNode> recorded;
     uint64_t compiles = 0, hits = 0, disk_hits = 0;
     std::string last_error;
@@ -248,6 +249,8 @@ int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage
 inline const std::vector<unsigned char>& literal_values(const RecNode& n) {
     return n.k->spec.kind == custos_hip::Kind::Chain ? n.const_bytes : n.k->spec.consts.bytes;
 }
+// The cached kernel of a chain spec (built without its text), or null.
+custos_hip_kernel* cached_chain_kernel(custos_hip_device* dev, const KernelSpec& spec);
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
 // Workgroups of a single launch of `k` over n_vec vectors and n elements with `unroll` vectors per thread.

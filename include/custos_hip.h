@@ -408,8 +408,9 @@ int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
  * literal is part of the joined kernel's code or one of its launch parameters as it is for the
  * launch's own kernel, so expressions that keep arriving with new values share their joined
  * kernels as they share their own.  The
- * kernels are compiled when the graph is built (at most 16 new ones per graph; a recording that
- * would need more is built as recorded).  No counterpart in the reference, whose captured
+ * kernels are compiled when the graph is built, at most 16 new ones per graph (or `enabled` of them,
+ * if that is more than 1); launches whose joined kernel is neither cached nor within that limit
+ * replay as they were recorded.  No counterpart in the reference, whose captured
  * graphs replay launch by launch (src/devices/cuda/lazy.rs:31-49). */
 int32_t custos_hip_set_graph_fusing(custos_hip_device *dev, int32_t enabled);
 /* The entry point kernel node `node` (0 .. kernel_nodes-1, in replay order) of a built graph

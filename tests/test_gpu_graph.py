@@ -1077,3 +1077,30 @@ def test_graph_names_its_kernels(hip):
     name = C.c_char_p()
     assert hip.lib.custos_hip_graph_node_kernel(g.handle, 2, C.byref(name)) == capi.ERR_INVALID_ARGUMENT
     g.destroy()
+
+
+def test_a_graph_build_compiles_a_limited_number_of_joined_kernels(fresh_device):
+    """Four chains of four different shapes with a limit of two new kernels per graph: two are joined, the
+    other two replay as the launches they were recorded as; the next build finds the two kernels cached and
+    compiles the others."""
+    hip = fresh_device
+    n = 3000
+    xs = [synth.uniform_f32(500 + i, n, -2, 2) for i in range(4)]
+    fns = [lambda v: v.mul(1.5), lambda v: v.abs().sqrt(), lambda v: v.neg().max(-1.0), lambda v: v.add(0.25).min(1.0)]
+
+    def program(b):
+        for i in range(4):                            # chain i: fns[i] twice, then fns[(i + 1) % 4]
+            hip.apply_fn(b[i], fns[i], out=b[4 + i])
+            hip.apply_fn(b[4 + i], fns[i], out=b[8 + i])
+            hip.apply_fn(b[8 + i], fns[(i + 1) % 4], out=b[4 + i])
+
+    zeros = [np.zeros(n, dtype=np.float32) for _ in range(8)]
+    for f in fns:                                     # the launches' own kernels exist before anything is counted
+        hip.apply_fn(hip.buffer(xs[0]), f)
+    hip.lib.custos_hip_set_graph_fusing(hip.handle, 2)
+    before = hip.cache_stats()[0]
+    assert _both_ways(hip, xs + zeros, program) == (2 + 6, 4)
+    assert hip.cache_stats()[0] - before == 2
+    assert _both_ways(hip, xs + zeros, program) == (4, 8)
+    assert hip.cache_stats()[0] - before == 4
+    hip.set_graph_fusing(True)
