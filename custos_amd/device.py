@@ -371,9 +371,10 @@ class HIP:
     def set_graph_batching(self, enabled: bool) -> None:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 
-    def set_graph_fusing(self, enabled: bool) -> None:
-        """Whether a graph build joins recorded apply launches with the apply launches that read their output."""
-        self._check(self.lib.custos_hip_set_graph_fusing(self.handle, 1 if enabled else 0))
+    def set_graph_fusing(self, enabled) -> None:
+        """Whether a graph build joins recorded launches with the launches that read their output; a number
+        above 1 also sets how many kernels of joined launches a graph build may compile (default 16)."""
+        self._check(self.lib.custos_hip_set_graph_fusing(self.handle, int(enabled)))
 
     def launch_hint_stats(self):
         """(not part of a chain, chain that stays in the memory-side cache, chain that streams) counts of

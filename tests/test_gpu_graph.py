@@ -1097,7 +1097,7 @@ def test_a_graph_build_compiles_a_limited_number_of_joined_kernels(fresh_device)
     zeros = [np.zeros(n, dtype=np.float32) for _ in range(8)]
     for f in fns:                                     # the launches' own kernels exist before anything is counted
         hip.apply_fn(hip.buffer(xs[0]), f)
-    hip.lib.custos_hip_set_graph_fusing(hip.handle, 2)
+    hip.set_graph_fusing(2)
     before = hip.cache_stats()[0]
     assert _both_ways(hip, xs + zeros, program) == (2 + 6, 4)
     assert hip.cache_stats()[0] - before == 2
