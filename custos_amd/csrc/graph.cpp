@@ -721,7 +721,9 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
         // expression has any) and the direction
         // (a merged launch reads them from its table rows instead)
         if (first.k->spec.consts.n_params > 0 && p.members.size() == 1) ln.args.push_back(literal_values(first));
-        const unsigned long long mode = launch_mode(p.shape.unroll, p.shape.nontemporal, rev != 0);
+        const unsigned long long mode = p.members.size() == 1
+                                            ? single_launch_mode(p.kern, first.n, first.head, first.n_vec, p.shape, rev != 0)
+                                            : launch_mode(p.shape.unroll, p.shape.nontemporal, rev != 0);
         ln.args.push_back(value(&mode, 8));
         if (p.shape.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
     }

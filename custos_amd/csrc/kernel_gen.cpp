@@ -483,12 +483,14 @@ struct KernelText {
         s += "    const u64 rev = mode & 1;\n";
         s += unroll_of_mode();
         s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * U;\n";
-        s += "    const u64 n_tiles = " + n_tiles_expr() + ";\n";
+        s += "    const u64 n_tiles = mode >> 16;\n";
         s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {\n";
         s += tile_call("        ", tile_args + out_views + "(rev ? n_tiles - 1 - tile : tile) * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
         s += "    }\n";
         // Elements outside the 16-byte aligned body: `head` leading ones and the
-        // tail. Lanes beyond the count are masked off by the wavefront's EXEC.
+        // tail. Lanes beyond the count are masked off by the wavefront's EXEC.  Most launches
+        // have none (bit 12 of the mode word): one scalar test instead of per-lane arithmetic.
+        s += "    if (!(mode & 4096)) return;\n";
         s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
         s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BLOCK;\n";
         s += "    if (gid < head) " + scalar_stmt("gid") + "\n";
@@ -605,7 +607,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds the vectors per thread as requested: 0 = chosen per launch)
     int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, 16 /* template version */};
+                       k.tuning.blocks_per_cu, 17 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -738,7 +740,7 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
                         (stage.out >= 0 ? " -> out" + std::to_string(stage.out) : std::string()) + "; ";
     }
     int32_t tail[7] = {static_cast<int32_t>(Kind::Chain), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, n_ext, n_outs, 16 /* template version */};
+                       k.tuning.blocks_per_cu, n_ext, n_outs, 17 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     k.stages = std::move(stages);

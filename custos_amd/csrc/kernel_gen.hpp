@@ -67,11 +67,17 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
 //   bit 1, 2   non-temporal loads, non-temporal stores
 //   bit 7      stores are written through to device scope at once instead of lingering in an L2
 //   bits 8..11 vectors per thread (only read by kernels whose unroll factor was left open)
+//   bit 12     (single-launch entry point) the range has scalar elements: a head before the first
+//              16-byte boundary or a tail after the last whole vector
+//   bits 16..  (single-launch entry point) the number of tiles of the vector range
+// The last two spare every workgroup of a launch the arithmetic that finds them out again: the
+// host knows them.
 // `nontemporal` as in Tuning: bit 0 loads, bit 1 stores, kStoresWriteThrough the write-through stores.
 constexpr int kStoresWriteThrough = 64;
-inline uint64_t launch_mode(int unroll, int nontemporal, bool rev) {
+inline uint64_t launch_mode(int unroll, int nontemporal, bool rev, uint64_t n_tiles = 0, bool scalar_edges = true) {
     return (rev ? 1u : 0u) | static_cast<uint64_t>(nontemporal & 3) << 1 |
-           static_cast<uint64_t>((nontemporal & kStoresWriteThrough) ? 1 : 0) << 7 | static_cast<uint64_t>(unroll & 15) << 8;
+           static_cast<uint64_t>((nontemporal & kStoresWriteThrough) ? 1 : 0) << 7 | static_cast<uint64_t>(unroll & 15) << 8 |
+           (scalar_edges ? 1u << 12 : 0u) | n_tiles << 16;
 }
 
 // Fills unset (zero) fields with the defaults and clamps to legal values

@@ -170,7 +170,7 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set);
     dev->last_shape[0] = shape.unroll, dev->last_shape[1] = shape.nontemporal, dev->last_shape[2] = shape.alternate;
     const unsigned int grid = launch_grid(dev, k, n, n_vec, shape.unroll);
-    unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, shape.alternate && (dev->launch_parity ^= 1));
+    unsigned long long mode = single_launch_mode(k, n, head, n_vec, shape, shape.alternate && (dev->launch_parity ^= 1));
     uint64_t ptrs[8];
     std::vector<void*> args;
     for (size_t i = 0; i < ops.size(); i++) {

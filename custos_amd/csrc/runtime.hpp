@@ -245,6 +245,14 @@ ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kerne
 // jit.cpp: the kernel for a chain of apply expressions (compiled on first use, then cached).
 int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs,
                      const Tuning& tuning, custos_hip_kernel** out, bool* compiled);
+// The mode word of a single launch of `k` over n elements (n_vec vectors after `head` scalar
+// elements) in the given shape.
+inline uint64_t single_launch_mode(const custos_hip_kernel* k, unsigned long long n, unsigned long long head,
+                                   unsigned long long n_vec, const ResolvedShape& shape, bool rev) {
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(k->spec.tuning.block_threads) * shape.unroll;
+    const bool edges = head > 0 || head + n_vec * static_cast<unsigned long long>(k->spec.vec_elems) < n;
+    return custos_hip::launch_mode(shape.unroll, shape.nontemporal, rev, (n_vec + tile_vecs - 1) / tile_vecs, edges);
+}
 // The values of a recorded launch's literal parameters.
 inline const std::vector<unsigned char>& literal_values(const RecNode& n) {
     return n.k->spec.kind == custos_hip::Kind::Chain ? n.const_bytes : n.k->spec.consts.bytes;
