@@ -535,9 +535,11 @@ struct KernelText {
         s += "extern \"C\" __global__ void __launch_bounds__(CUSTOS_BLOCK)\n";
         s += k.name + "_batched(const u64* __restrict__ table, const u64 n, const u64 n_vec, const u64 tiles_per_seg, const u64 mode) {\n";
         s += unroll_of_mode();
-        s += "    const u64 blk = (mode & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
-        s += "    const u64 seg = blk / tiles_per_seg;\n";
-        s += "    const u64 tile = blk - seg * tiles_per_seg;\n";
+        // (a grid has fewer than 2^31 workgroups: a 32-bit division, a third of the 64-bit one)
+        s += "    const unsigned int blk = (mode & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x;\n";
+        s += "    const unsigned int per_seg = (unsigned int)tiles_per_seg;\n";
+        s += "    const u64 seg = blk / per_seg;\n";
+        s += "    const u64 tile = blk - (unsigned int)seg * per_seg;\n";
         s += "    const u64* ptrs = table + seg * " + std::to_string(n_ptrs + const_words) + ";\n";
         s += row_consts(n_ptrs);
         s += "    const u64 head = 0;\n";
@@ -607,7 +609,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds the vectors per thread as requested: 0 = chosen per launch)
     int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, 17 /* template version */};
+                       k.tuning.blocks_per_cu, 18 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -740,7 +742,7 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
                         (stage.out >= 0 ? " -> out" + std::to_string(stage.out) : std::string()) + "; ";
     }
     int32_t tail[7] = {static_cast<int32_t>(Kind::Chain), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, n_ext, n_outs, 17 /* template version */};
+                       k.tuning.blocks_per_cu, n_ext, n_outs, 18 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     k.stages = std::move(stages);
