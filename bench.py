@@ -6,18 +6,21 @@ operations fused into ONE kernel, over f32 N = 2^28, x uniform in [-pi, pi) from
 resident in HBM.  What is timed, and where:
 
   value / ms_per_step   this process, through the C ABI: one step = one replay of the one-node
-                        recording that holds the fused kernel (what a lazy run holds from its
-                        second run on); exactly --steps replays between two events on the
-                        library's compute stream, no wait between steps.  By default such a
-                        launch walks the array against the direction of the launch before it and
-                        so starts on the 256 MiB the memory-side cache still holds.
-  per_step              the same replays with an event between every two (>= 50): median and min.
-  roofline              the same expression pinned to plain HBM streaming (every launch first tile to
-                        last, non-temporal accesses, one-wavefront workgroups): no help from the
-                        memory-side cache.
-  module_stack          a child process started before this one touches the GPU: the C++ module
-                        stack HIP<Graph<Lazy<Base>>>, five apply_fn calls, optimize_mem_graph,
-                        unary_fusing, then run() with the reference's wait after every run.
+                        recording that holds the fused kernel, pinned to plain HBM streaming (every
+                        launch walks the array from the first tile to the last with non-temporal
+                        accesses, so nothing of the previous launch is found in the memory-side
+                        cache); exactly --steps replays between two events on the library's compute
+                        stream, no wait between steps.
+  sustained / roofline  the same replay back to back for at least two seconds with an event between
+                        every two launches: mean (what `roofline.achieved` is quoted on), median, the
+                        rate 99 % of the launches reach, and the slowest launch.
+  default_replay        the same recording with the library's own launch shape: launches alternate
+                        their direction and so start on the 256 MiB the memory-side cache still holds.
+  module_stack          child processes started before this one touches the GPU: the C++ module
+                        stacks on the HIP device (c2: HIP<Graph<Lazy<Base>>>, five apply_fn calls,
+                        optimize_mem_graph, unary_fusing, run(); the other configurations likewise).
+  first_use             child processes with an empty compiler cache, then a warm one: what the first
+                        call of a new expression costs (compilation included).
   cpu_baseline          the oracle's compiled loop for the same chain, one thread.
 
 `other_configs` carries the other four BASELINE configurations (c1 exp, c3 tanh forward +
@@ -143,25 +146,123 @@ def per_step_stats(dev, step, steps):
             "min_ms": round(float(ms.min()), 5), "max_ms": round(float(ms.max()), 5)}
 
 
-def module_stack(config, steps, warmup, log2n=None, fuse=False, dump=None):
+def sustained_stats(dev, step, bytes_per_step, seconds=2.0, chunk=2048):
+    """`step` back to back for at least `seconds` of device time, an event between every two steps.
+    The events of a chunk are read while the next chunk is already queued, so the device does not idle
+    in between; the first event of a chunk is recorded right behind the last one of the chunk before."""
+    dev.sync()
+    durations = []
+    total_ms = 0.0
+    while total_ms < seconds * 1e3 and len(durations) < 200000:
+        dev.timer_mark(0)
+        for i in range(chunk):
+            step()
+            dev.timer_mark(i + 1)
+        ms = np.array([dev.timer_between(i, i + 1) for i in range(chunk)])
+        durations.append(ms)
+        total_ms += float(ms.sum())
+    ms = np.concatenate(durations)
+    gbs = bytes_per_step / (ms * 1e-3) / 1e9
+    return {
+        "launches": int(ms.size), "device_seconds": round(total_ms * 1e-3, 3),
+        "mean_ms": round(float(ms.mean()), 5), "median_ms": round(float(np.median(ms)), 5),
+        "p99_ms": round(float(np.percentile(ms, 99)), 5), "max_ms": round(float(ms.max()), 5),
+        "mean_GBps": round(bytes_per_step / (float(ms.mean()) * 1e-3) / 1e9, 2),
+        "median_GBps": round(float(np.median(gbs)), 2),
+        "p99_GBps": round(float(np.percentile(gbs, 1)), 2),
+        "min_GBps": round(float(gbs.min()), 2),
+        "what": "p99_GBps: 99 % of the launches are at least this fast; min_GBps: the slowest launch",
+    }
+
+
+def module_stack(config, steps, warmup, log2n=None, fuse=False, dump=None, stack=None, inputs=(), settle_ms=None, env=None):
     """Runs examples/bench_module_stack as a child process and returns its JSON line."""
     exe = os.path.join(ROOT, "examples", "bench_module_stack")
     if not os.path.exists(exe):
         return {"error": f"{exe} is not built (make -C examples)"}
-    cmd = [exe, "--config", config, "--steps", str(max(steps, MIN_LAUNCHES)), "--warmup", str(warmup)]
+    cmd = [exe, "--config", config, "--steps", str(steps), "--warmup", str(warmup)]
     if log2n is not None:
         cmd += ["--log2n", str(log2n)]
     if fuse:
         cmd += ["--fuse"]
+    if stack:
+        cmd += ["--stack", stack]
+    if settle_ms is not None:
+        cmd += ["--settle-ms", str(settle_ms)]
+    for flag, path in zip(("--input", "--input2"), inputs):
+        cmd += [flag, path]
     if dump:
         cmd += ["--dump", str(dump[0]), dump[1]]
     try:
-        proc = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
+        proc = subprocess.run(cmd, capture_output=True, text=True, timeout=240, env=env)
     except subprocess.TimeoutExpired:
         return {"error": "timed out"}
     if proc.returncode != 0:
         return {"error": (proc.stderr or proc.stdout)[-400:]}
     return json.loads(proc.stdout.strip().splitlines()[-1])
+
+
+def cold_cache_env(tmp):
+    """An environment in which the ROCm compiler library finds none of its cached results: its cache
+    sits under the home directory (or where AMD_COMGR_CACHE_DIR / XDG_CACHE_HOME point)."""
+    env = dict(os.environ)
+    env.update({"HOME": tmp, "XDG_CACHE_HOME": os.path.join(tmp, ".cache"), "AMD_COMGR_CACHE_DIR": os.path.join(tmp, "comgr")})
+    env.pop("CUSTOS_HIP_KERNEL_CACHE_DIR", None)
+    return env
+
+
+FIRST_CALL_EXPRESSIONS = {
+    "c1": (lambda: "exp(x)", 1 << 20),
+    "c2": (lambda: __import__("custos_amd.expr", fromlist=["fused_source"]).fused_source(C2_OPS, "f32"), 1 << 20),
+}
+
+
+def first_call_child(which):
+    """(child process) One first call of an expression: compile, launch over a small buffer, wait."""
+    import custos_amd
+    from custos_amd import capi
+
+    make_src, n = FIRST_CALL_EXPRESSIONS[which]
+    dev = custos_amd.HIP(0)
+    x, out = dev.alloc(n), dev.alloc(n)
+    dev.sync()
+    t0 = time.perf_counter()
+    kernel = dev.compile(capi.KIND_APPLY, "f32", make_src(), ("x",))
+    t1 = time.perf_counter()
+    capi.check(dev.lib.custos_hip_apply_fn(dev.handle, kernel, x.ptr, out.ptr, n), dev.handle)
+    dev.sync()
+    t2 = time.perf_counter()
+    units, hiprtc_ms = dev.compile_stats()
+    print(json.dumps({"first_call_ms": round((t2 - t0) * 1e3, 2), "compile_ms": round((t1 - t0) * 1e3, 2),
+                      "translation_units": units, "hiprtc_ms": round(hiprtc_ms, 2)}))
+
+
+def first_use(tmp, with_c5):
+    """First-call cost of c1 and c2 (this process's interpreter, C ABI) and first run() of c5 through the
+    module stack, each in a fresh process with an empty compiler cache and again with the cache the
+    first process left."""
+    env = cold_cache_env(tmp)
+    out = {"what": "a fresh process each; cold = the ROCm compiler library's cache is empty (temporary HOME), warm = the "
+                   "same again on the cache the cold process left; first_call_ms = custos_hip_expr_compile + the first "
+                   "launch + a wait"}
+    for which in ("c1", "c2"):
+        entry = {}
+        for state in ("cold", "warm"):
+            try:
+                proc = subprocess.run([sys.executable, os.path.abspath(__file__), "--first-call", which], capture_output=True,
+                                      text=True, timeout=120, env=env)
+                entry[state] = json.loads(proc.stdout.strip().splitlines()[-1]) if proc.returncode == 0 else {"error": proc.stderr[-300:]}
+            except (subprocess.TimeoutExpired, ValueError, IndexError) as e:
+                entry[state] = {"error": str(e)[-300:]}
+        out[which] = entry
+    if with_c5:
+        for fuse in (False, True):
+            entry = {}
+            for state in ("cold", "warm"):
+                r = module_stack("c5", 1, 0, fuse=fuse, settle_ms=0, env=env)
+                entry[state] = {"first_run_ms": r.get("first_run_ms"), "kernel_nodes": r.get("kernel_nodes")} if "error" not in r else r
+            out["c5_module_stack" + ("_after_elementwise_fusing" if fuse else "")] = entry
+    return out
 
 
 def measured_traffic(kernel_label):
@@ -252,53 +353,57 @@ def bench_c2(dev, args, stack):
     copy_kernel = dev.compile(capi.KIND_APPLY, "f32", "x", ("x",))
     copy_ms, copy_n = time_floor(dev, launcher(dev, lib.custos_hip_apply_fn, copy_kernel, xb.ptr, tmp_a.ptr, n))
 
-    # The fused step pinned to plain HBM streaming: every launch walks the array from the first tile
-    # to the last, non-temporal loads and stores, so nothing of the previous launch is found in the
-    # memory-side cache (one-wavefront workgroups with one vector per thread stream best that way).
-    # This is the figure the roofline fraction is quoted on.
-    streaming = None
-    if not tuned:
-        dev.set_tuning(64, 1, 0, 3 | 64, 1)
-        skernel = dev.compile(capi.KIND_APPLY, "f32", src, ("x",))
-        dev.capture_begin()
-        capi.check(lib.custos_hip_apply_fn(dev.handle, skernel, xb.ptr, out.ptr, n), dev.handle)
-        sgraph = dev.capture_end()
-        dev.set_tuning(0, 0, 0, 0, 0)
-        sms, _ = time_exactly(dev, sgraph.launch, max(args.steps, MIN_LAUNCHES), args.warmup)
-        sms /= max(args.steps, MIN_LAUNCHES)
-        streaming = {"ms_per_step": round(sms, 5), "GBps": round(gbs_of(sms), 2),
-                     "per_step": per_step_stats(dev, sgraph.launch, args.steps),
-                     "kernel": dev.kernel_name(skernel),
-                     "shape": "tiles first to last, non-temporal loads, non-temporal stores written through at once, "
-                              "one-wavefront workgroups, 1 vector per thread"}
-        check_chain(out.slice(0, 1 << 20).read(), cpu_oracle_chain(x[: 1 << 20]), "the streaming-pinned fused chain")
-        sgraph.destroy()
-
     direct_ms, direct_n = time_floor(dev, fused_step)   # the fused kernel launched directly, not replayed
 
-    # Headline.  One step = what a lazy run does from its second run on: replay the recording that
-    # holds the fused kernel.  (The first run records and builds it; that is outside the timed region.)
+    # The library's own launch shape: launches alternate their direction and start on the 256 MiB the
+    # memory-side cache still holds.  One step = what a lazy run does from its second run on: replay the
+    # recording that holds the fused kernel.
     dev.capture_begin()
     fused_step()
     graph = dev.capture_end()
     assert graph.kernel_nodes == 1
+    dms, _ = time_exactly(dev, graph.launch, max(args.steps, MIN_LAUNCHES), args.warmup)
+    dms /= max(args.steps, MIN_LAUNCHES)
+    default_replay = {"ms_per_step": round(dms, 5), "GBps": round(gbs_of(dms), 2), "frac_of_peak": round(gbs_of(dms) / HBM_PEAK_GBS, 4),
+                      "per_step": per_step_stats(dev, graph.launch, args.steps), "kernel": dev.kernel_name(kernel),
+                      "what": "the library's own launch shape: launches alternate their direction and start on the 256 MiB "
+                              "the memory-side cache still holds, so part of this rate is not HBM bandwidth"}
+    graph.destroy()
+
+    # Headline.  The same step pinned to plain HBM streaming: every launch walks the array from the first
+    # tile to the last, non-temporal loads and stores, so nothing of the previous launch is found in the
+    # memory-side cache (one-wavefront workgroups with one vector per thread stream best that way).
+    # (With a launch shape given on the command line, that shape is what is timed.)
+    if not tuned:
+        dev.set_tuning(64, 1, 0, 3 | 64, 1)
+    skernel = dev.compile(capi.KIND_APPLY, "f32", src, ("x",))
+    dev.capture_begin()
+    capi.check(lib.custos_hip_apply_fn(dev.handle, skernel, xb.ptr, out.ptr, n), dev.handle)
+    graph = dev.capture_end()
+    if not tuned:
+        dev.set_tuning(0, 0, 0, 0, 0)
+    assert graph.kernel_nodes == 1
     ms, wall_ms = time_exactly(dev, graph.launch, args.steps, args.warmup)
     per_launch_ms = ms / args.steps
-    per_step = per_step_stats(dev, graph.launch, args.steps)
-    graph.destroy()
     gbs = gbs_of(per_launch_ms)
+    per_step = per_step_stats(dev, graph.launch, args.steps)
+    sustained = sustained_stats(dev, graph.launch, algo_bytes, seconds=args.sustain_seconds)
+    shape = ("the launch shape given on the command line" if tuned else
+             "tiles first to last, non-temporal loads, non-temporal stores written through at once, one-wavefront "
+             "workgroups, 1 vector per thread")
 
     # parity of the very buffer that was timed, on the CPU sample
-    fused_step()
+    graph.launch()
     got = out.read()
+    graph.destroy()
     base, want = cpu_baseline_c2(x, min(n, 1 << args.cpu_log2n))
     diff = check_chain(got, want, "the fused chain")
     if stack.get("dump") is not None:
         stack["max_abs_diff_vs_cpu_oracle"] = check_chain(stack.pop("dump"), want, "the module stack's fused chain")
 
-    roof_ms = streaming["ms_per_step"] if streaming else per_launch_ms
-    roof_kernel = streaming["kernel"] if streaming else dev.kernel_name(kernel)
-    traffic, traffic_source = measured_traffic("c2 streaming") if (streaming and args.log2n == 28) else (None, None)
+    roof_ms = sustained["mean_ms"]
+    roof_kernel = dev.kernel_name(skernel)
+    traffic, traffic_source = measured_traffic("c2 streaming") if (not tuned and args.log2n == 28) else (None, None)
     return {
         "metric": "fused unary-chain GB/s and % of HBM peak, f32 N=2^28, 1xMI355X",
         "value": round(gbs, 2),
@@ -307,19 +412,22 @@ def bench_c2(dev, args, stack):
         "config": {
             "workload": f"c2: y = relu(sin(x)*2+1)-0.5 as ONE fused kernel (the text that unary fusing of the five recorded "
                         f"apply_fn operations emits), f32, N=2^{args.log2n}, x~U[-pi,pi) seed 0; one step = one replay of the "
-                        "one-node recording through custos_hip_graph_launch (C ABI), launches alternate their direction, no "
-                        "wait between steps; the same workload through the C++ module stack with a wait per run: module_stack",
+                        "one-node recording through custos_hip_graph_launch (C ABI) in the HBM-only launch shape (" + shape +
+                        "), no wait between steps; the library's own launch shape: default_replay; the same workload through "
+                        "the C++ module stack: module_stack",
             "elements": n,
             "algorithmic_bytes_per_element": 8,
         },
-        "kernel": dev.kernel_name(kernel),
+        "kernel": roof_kernel,
         "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "elements_per_s": round(n / (per_launch_ms * 1e-3), 1),
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
         "per_step": per_step,
+        "sustained": sustained,
+        "default_replay": default_replay,
         "module_stack": stack,
-        "direct_launch": {"ms_per_step": round(direct_ms, 5), "GBps": round(gbs_of(direct_ms), 2), "launches": direct_n},
-        "hbm_streaming_only": streaming,
+        "direct_launch": {"ms_per_step": round(direct_ms, 5), "GBps": round(gbs_of(direct_ms), 2), "launches": direct_n,
+                          "what": "the fused kernel launched directly (custos_hip_apply_fn), the library's own launch shape"},
         "unfused": {
             "ms_per_step": round(unfused_ms, 5),
             "steps": unfused_n,
@@ -330,8 +438,9 @@ def bench_c2(dev, args, stack):
                 "ms_per_replay": round(recorded_ms, 5), "replays": recorded_n, "kernel_nodes": recorded_nodes,
                 "launches_joined_into_later_ones": recorded_joined, "kernels": recorded_kernels,
                 "effective_GBps_on_8B_basis": round(gbs_of(recorded_ms), 2),
+                "moved_GBps_on_16B_basis": round(2 * gbs_of(recorded_ms), 2),
                 "what": "the five launches recorded without unary fusing; the graph build joins them into one kernel "
-                        "that still writes the two intermediate buffers (16 B/element)",
+                        "that still writes the two intermediate buffers (1 read + 3 writes: 16 B/element)",
             },
         },
         "copy_kernel": {
@@ -348,16 +457,16 @@ def bench_c2(dev, args, stack):
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs_of(roof_ms) / HBM_PEAK_GBS, 4),
+            "frac_median": round(sustained["median_GBps"] / HBM_PEAK_GBS, 4),
+            "frac_p99": round(sustained["p99_GBps"] / HBM_PEAK_GBS, 4),
             "traffic": traffic,
             "traffic_source": traffic_source,
             "kernel": roof_kernel,
             "algorithmic_bytes_per_launch": algo_bytes,
             "avg_launch_ms": round(roof_ms, 5),
-            "what": ("the fused kernel pinned to first-to-last streaming (hbm_streaming_only): HBM only" if streaming
-                     else "the fused kernel with the launch shape given on the command line"),
-            "with_memory_side_cache": {"achieved": round(gbs, 2), "frac": round(gbs / HBM_PEAK_GBS, 4),
-                                       "what": "the headline replay: launches alternate their direction and start on "
-                                               "the 256 MiB the memory-side cache still holds"},
+            "launches": sustained["launches"],
+            "what": "the headline's kernel and launch shape (HBM only) over the `sustained` region: algorithmic bytes / mean launch "
+                    "duration from events on the library's compute stream",
         },
         "cpu_baseline": base,
     }
@@ -486,6 +595,19 @@ def bench_others(dev, args, stack_c5):
                                   "GBps_on_24B": round(24 * n / (ms_g * 1e-3) / 1e9, 2),
                                   "moved_GBps_on_20B": round(20 * n / (ms_g * 1e-3) / 1e9, 2)}
     g3.destroy()
+    # the same through the C++ module stacks (child processes that ran before this one touched the GPU)
+    stacks3 = stack_c5.pop("c3", {"skipped": True})
+    for name, r in (stacks3.items() if "skipped" not in stacks3 else ()):
+        if "dump" not in r:
+            continue
+        both = r.pop("dump")
+        k3 = both.size // 2
+        dy = np.abs(both[:k3].view(np.int32).astype(np.int64) - cpu_oracle.c3_tanh_fwd(x[:k3]).view(np.int32).astype(np.int64))
+        dg = np.abs(both[k3:] - cpu_oracle.c3_tanh_bwd(x[:k3], np.full(k3, 0.1, dtype=np.float32), yg[:k3]))
+        if dy.max() > 4 or dg.max() > 2e-6:
+            raise SystemExit(f"bench: c3 through the module stack ({name}) differs from the CPU oracle: {dy.max()} ulp, {dg.max()}")
+        r["max_ulp_y_vs_cpu_oracle"], r["max_abs_diff_x_grad_vs_cpu_oracle"] = int(dy.max()), float(dg.max())
+    e["module_stack"] = stacks3
     out["c3"] = e
     del xb, ygb, yb, gb
 
@@ -504,6 +626,14 @@ def bench_others(dev, args, stack_c5):
     out["c4"] = _entry(f"c4: f16 chain exp(x*0.5)*x + x^2, f32 compute, N=2^{args.log2n}", n, 4, ms, cpu_s, cn)
     out["c4"]["launches"] = c4_steps
     out["c4"]["kernel"] = dev.kernel_name(k)
+    stack4 = stack_c5.pop("c4", {"skipped": True})
+    if "dump" in stack4:
+        first = stack4.pop("dump")
+        d4 = np.abs(first.view(np.int16).astype(np.int32) - want[: first.size].view(np.int16).astype(np.int32))
+        if d4.max() > 1:
+            raise SystemExit("bench: c4 through the module stack differs from the CPU port by more than 1 f16 ulp")
+        stack4["max_f16_ulp_vs_cpu_oracle"] = int(d4.max())
+    out["c4"]["module_stack"] = stack4
     del xb, ob
 
     # c5: 1024 buffers x 4096 f32: t=a*b; u=t+c; y=sqrt(abs(u))*0.3, recorded once, replayed
@@ -582,6 +712,19 @@ def bench_others(dev, args, stack_c5):
     e["fused"]["kernel"] = dev.kernel_name(kfused) + "_batched"
     e["fused"]["GBps"] = e["fused"]["GBps_on_16B"]
     graph.destroy()
+    # the same fused expression over the same 1024 operand sets through the entry point that allocates
+    # nothing (its table sits in a static device array; every call checks the operand sets on the host
+    # and sends the rows through a pinned staging slot)
+    dev.prepare_merged(kfused)
+    rows = (C.c_uint64 * (4 * nbuf))(*[p for i in range(nbuf) for p in (A.ptr + i * m * 4, B.ptr + i * m * 4, Cc.ptr + i * m * 4, Y.ptr + i * m * 4)])
+    Y.clear()
+    na_step = launcher(dev, lib.custos_hip_apply_fn_many_noalloc, kfused, rows, 4, nbuf, m)
+    na_ms, na_calls = time_floor(dev, na_step)
+    assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), "c5 through the allocation-free entry point differs"
+    e["fused"]["allocation_free_entry_point"] = {
+        "us_per_call": round(na_ms * 1e3, 2), "calls": na_calls, "GBps_on_16B": round(16 * nbuf * m / (na_ms * 1e-3) / 1e9, 2),
+        "what": "custos_hip_apply_fn_many_noalloc over the same 1024 operand sets, back to back from Python: operand checks on "
+                "the host, 32 KiB of table rows through a staging slot and the copy kernel, then the same grid"}
     e["module_stack"] = stack_c5
     out["c5"] = e
     return out
@@ -611,28 +754,56 @@ def main():
                          "3-node graph): for runs under rocprofv3, whose kernel tracing ended the process in hipGraphLaunch")
     ap.add_argument("--no-module-stack", dest="module_stack", action="store_false",
                     help="skip the child processes that time the C++ module stack")
+    ap.add_argument("--no-first-use", dest="first_use", action="store_false",
+                    help="skip the child processes that measure first calls with an empty compiler cache")
+    ap.add_argument("--sustain-seconds", dest="sustain_seconds", type=float, default=2.0,
+                    help="device time of the back-to-back region behind `sustained` and `roofline`")
+    ap.add_argument("--first-call", dest="first_call", choices=sorted(FIRST_CALL_EXPRESSIONS), default=None, help=argparse.SUPPRESS)
     args = ap.parse_args()
+    if args.first_call:
+        first_call_child(args.first_call)
+        return
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU; the element-wise path needs no second one "
                          "(--gpus must be 1)")
     if args.steps < 1 or args.warmup < 0:
         raise SystemExit("bench.py: --steps must be positive, --warmup not negative")
 
-    # The module stack runs in child processes, one after the other, before this process
-    # touches the GPU.
-    stack, stack_c5 = {"skipped": True}, {"skipped": True}
-    if args.module_stack:
-        with tempfile.TemporaryDirectory() as tmp:
+    # The module stack and the first-use measurements run in child processes, one after the other,
+    # before this process touches the GPU.
+    stack, stack_c5, first = {"skipped": True}, {"skipped": True}, {"skipped": True}
+    with tempfile.TemporaryDirectory() as tmp:
+        if args.first_use:
+            first = first_use(os.path.join(tmp, "home"), with_c5=args.others and args.module_stack)
+        if args.module_stack:
             dump = os.path.join(tmp, "c2_first.f32")
-            stack = module_stack("c2", args.steps, args.warmup, log2n=args.log2n, dump=(1 << 20, dump))
+            stack = module_stack("c2", max(args.steps, MIN_LAUNCHES), args.warmup, log2n=args.log2n, dump=(1 << 20, dump))
             if "error" not in stack and os.path.exists(dump):
                 stack["dump"] = np.fromfile(dump, dtype=np.float32)
-            if args.others:
-                stack_c5 = {"as_recorded": module_stack("c5", 500, 20), "after_elementwise_fusing": module_stack("c5", 500, 20, fuse=True)}
-                dump1 = os.path.join(tmp, "c1_first.f32")
-                stack_c5["c1"] = module_stack("c1", 200, 20, dump=(1 << 20, dump1))
-                if "error" not in stack_c5["c1"] and os.path.exists(dump1):
-                    stack_c5["c1"]["dump"] = np.fromfile(dump1, dtype=np.float32)
+        if args.module_stack and args.others:
+            from custos_amd import synth
+            stack_c5 = {"as_recorded": module_stack("c5", 500, 20), "after_elementwise_fusing": module_stack("c5", 500, 20, fuse=True)}
+            dump1 = os.path.join(tmp, "c1_first.f32")
+            stack_c5["c1"] = module_stack("c1", 200, 20, dump=(1 << 20, dump1))
+            if "error" not in stack_c5["c1"] and os.path.exists(dump1):
+                stack_c5["c1"]["dump"] = np.fromfile(dump1, dtype=np.float32)
+            # c3 and c4 read their inputs from files (the same synthetic arrays this process generates later)
+            n3, n4 = 1 << 26, 1 << args.log2n
+            x3, yg3, x4 = (os.path.join(tmp, f) for f in ("c3_x.f32", "c3_yg.f32", "c4_x.f16"))
+            gen_chunked(lambda q, off: synth.normal_f32(0, q, off), n3).tofile(x3)
+            gen_chunked(lambda q, off: synth.uniform_f32(1, q, -1, 1, off), n3).tofile(yg3)
+            gen_chunked(lambda q, off: synth.uniform_f16_bits(0, q, -2, 2, off), n4).tofile(x4)
+            stack_c5["c3"] = {}
+            for which in ("eager", "lazy", "joined"):
+                dump3 = os.path.join(tmp, f"c3_{which}.f32")
+                r = module_stack("c3", MIN_LAUNCHES, 10, stack=which, inputs=(x3, yg3), dump=(1 << 20, dump3))
+                if "error" not in r and os.path.exists(dump3):
+                    r["dump"] = np.fromfile(dump3, dtype=np.float32)
+                stack_c5["c3"][which] = r
+            dump4 = os.path.join(tmp, "c4_first.f16")
+            stack_c5["c4"] = module_stack("c4", MIN_LAUNCHES, 10, log2n=args.log2n, inputs=(x4,), dump=(1 << 20, dump4))
+            if "error" not in stack_c5["c4"] and os.path.exists(dump4):
+                stack_c5["c4"]["dump"] = np.fromfile(dump4, dtype=np.uint16)
 
     import custos_amd
 
@@ -643,6 +814,7 @@ def main():
         dev.set_tuning(args.block, args.unroll, args.blocks_per_cu, args.nontemporal, args.direction)
     info = dev.info()
     res = {"c2": bench_c2}[args.workload](dev, args, stack)
+    res["first_use"] = first
     if args.others:
         res["other_configs"] = bench_others(dev, args, stack_c5)
     res.update({

@@ -38,6 +38,7 @@ ERR_EXPR_UNSUPPORTED = 10012
 ERR_COMPILE = 10020
 ERR_KIND_MISMATCH = 10030
 ERR_ARITY_MISMATCH = 10031
+ERR_NOT_PREPARED = 10032
 ERR_CAPTURE_STATE = 10040
 ERR_GRAPH_ORDER = 10041
 ERR_BAD_OVERLAP = 10050
@@ -142,6 +143,10 @@ PROTOTYPES = {
     "custos_hip_apply_fn2": (C.c_int32, [_P, _P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_apply_fn_n": (C.c_int32, [_P, _P, C.POINTER(C.c_uint64), C.c_int32, C.c_uint64, C.c_size_t]),
     "custos_hip_apply_fn_many_noalloc": (C.c_int32, [_P, _P, C.POINTER(C.c_uint64), C.c_int32, C.c_size_t, C.c_size_t]),
+    "custos_hip_kernel_prepare_merged": (C.c_int32, [_P, _P]),
+    "custos_hip_set_graph_fusing_budget": (C.c_int32, [_P, C.c_uint32]),
+    "custos_hip_graph_unjoined": (C.c_int32, [_P, C.POINTER(C.c_size_t), C.POINTER(C.c_char_p)]),
+    "custos_hip_compile_stats": (C.c_int32, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_double)]),
     "custos_hip_fill": (C.c_int32, [_P, C.c_uint64, C.c_size_t, C.c_void_p, C.c_size_t]),
     "custos_hip_add_unary_grad": (C.c_int32, [_P, _P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_capture_begin": (C.c_int32, [_P]),

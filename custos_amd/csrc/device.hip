@@ -39,10 +39,18 @@ constexpr size_t kScratchWords = 8192;
 static __device__ __align__(256) unsigned long long scratch[kScratchWords];
 constexpr int kMaxDevices = 64;
 static unsigned long long* g_scratch_ptr[kMaxDevices];
-static std::mutex g_scratch_mutex;  // handles are created from several threads
+// All handles on a GPU share that GPU's table, each launching on a stream of its own.  The
+// table's last user and an event recorded behind its launch let the next call through ANOTHER
+// handle order its rewrite of the table behind that launch (calls through one handle are
+// ordered by its stream).  The mutex covers the look-up, and in the entry point everything
+// from the wait to the event record, so that calls from several threads take turns.
+static hipEvent_t g_scratch_event[kMaxDevices];
+static const custos_hip_device* g_scratch_last_user[kMaxDevices];
+static std::mutex g_scratch_mutex;
 static_assert(kScratchWords * sizeof(unsigned long long) <= kStagedReadMax, "the table travels through one staging slot");
 
-// With device `idx` current: the address of that device's copy of `scratch`.
+// With device `idx` current: the address of that device's copy of `scratch` (and, made with
+// it, the event that orders the table's users).
 static hipError_t scratch_address(int idx, unsigned long long** out) {
     if (idx < 0 || idx >= kMaxDevices) return hipErrorInvalidDevice;
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
@@ -50,6 +58,10 @@ static hipError_t scratch_address(int idx, unsigned long long** out) {
         void* p = nullptr;
         hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return e;
+        hipEvent_t event = nullptr;
+        e = hipEventCreateWithFlags(&event, hipEventDisableTiming);
+        if (e != hipSuccess) return e;
+        g_scratch_event[idx] = event;
         g_scratch_ptr[idx] = static_cast<unsigned long long*>(p);
     }
     *out = g_scratch_ptr[idx];
@@ -122,6 +134,20 @@ hipError_t wait_compute_stream(custos_hip_device* dev) {
     const uint64_t mine = ++dev->waits_begun;
     hipError_t e = wait_compute_stream_now(dev);
     if (e == hipSuccess) dev->waits_done = mine;
+    return e;
+}
+
+// Recording begins without a wait (custos_hip_capture_begin), so that a caller who records
+// right after launching a graph does not drain the stream between two runs.  What still runs
+// at once while the device records -- allocation with its zero fill, reads, writes, a free
+// that goes back to the driver -- uses the transfer stream or the driver, outside the compute
+// stream's order: the first of them takes the wait for the work that was in flight when the
+// recording began (nothing is launched on the compute stream while recording, so one wait is
+// enough).
+hipError_t drain_before_immediate_work(custos_hip_device* dev) {
+    if (!dev->undrained_at_capture) return hipSuccess;
+    hipError_t e = wait_compute_stream(dev);
+    if (e == hipSuccess) dev->undrained_at_capture = false;
     return e;
 }
 
@@ -226,20 +252,37 @@ static int32_t launch_stage_copy(custos_hip_device* dev, uint64_t dst, uint64_t 
 // order and without a wait; a slot is reused once a wait that began after its launch has
 // finished, and a seventeenth write in a row without one waits first.
 // Needs the staging memory, at most kStagedReadMax bytes, and a device that is not recording.
-static int32_t staged_write(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes) {
+// The next staging slot, free to be filled: host address and device address of its byte 0 at
+// the 16-byte phase of `dst`.
+static int32_t staging_slot(custos_hip_device* dev, uint64_t dst, unsigned char** host, uint64_t* device) {
     const size_t slot = dev->write_slot;
     static_assert(kWriteSlots == std::tuple_size<decltype(dev->write_slot_issued)>::value, "one entry per slot");
     if (dev->write_slot_used[slot] && dev->waits_done <= dev->write_slot_issued[slot])
         HIP_TRY(dev, wait_compute_stream(dev));
-    const uint64_t phase = dst & 15;
-    const size_t offset = (kStagedReadMax + 16) * (1 + slot) + phase;
-    std::memcpy(dev->read_stage + offset, src, bytes);
-    int32_t rc = launch_stage_copy(dev, dst, dev->read_stage_dev + offset, bytes);
+    const size_t offset = (kStagedReadMax + 16) * (1 + slot) + (dst & 15);
+    *host = dev->read_stage + offset;
+    *device = dev->read_stage_dev + offset;
+    return CUSTOS_HIP_OK;
+}
+
+// Launches the copy of `bytes` bytes from the slot staging_slot handed out to `dst`.
+static int32_t staging_slot_send(custos_hip_device* dev, uint64_t dst, uint64_t slot_device, size_t bytes) {
+    int32_t rc = launch_stage_copy(dev, dst, slot_device, bytes);
     if (rc != CUSTOS_HIP_OK) return rc;
+    const size_t slot = dev->write_slot;
     dev->write_slot_issued[slot] = dev->waits_begun;
     dev->write_slot_used[slot] = true;
     dev->write_slot = (slot + 1) % kWriteSlots;
     return CUSTOS_HIP_OK;
+}
+
+static int32_t staged_write(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes) {
+    unsigned char* host = nullptr;
+    uint64_t device = 0;
+    int32_t rc = staging_slot(dev, dst, &host, &device);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    std::memcpy(host, src, bytes);
+    return staging_slot_send(dev, dst, device, bytes);
 }
 
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec) {
@@ -374,7 +417,12 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
     HIP_TRY(nullptr, hipEventCreate(&dev->t0));
     HIP_TRY(nullptr, hipEventCreate(&dev->t1));
     dev->pool_limit = dev->props.totalGlobalMem / 4;
-    HIP_TRY(nullptr, scratch_address(idx, &dev->scratch_table));
+    // (optional: without it only the allocation-free merged launch is unavailable)
+    if (scratch_address(idx, &dev->scratch_table) != hipSuccess) {
+        (void)hipGetLastError();
+        dev->scratch_table = nullptr;
+    }
+    dev->noalloc_spans.reserve(kScratchWords);  // so that the entry point that may not allocate finds its room
     // completion word for short waits (pinned, mapped host memory); optional
     void* flag = nullptr;
     if (hipHostMalloc(&flag, 64, hipHostMallocMapped) == hipSuccess) {
@@ -413,12 +461,18 @@ int32_t custos_hip_device_destroy(custos_hip_device* dev) {
     (void)hipSetDevice(dev->idx);
     (void)hipStreamSynchronize(dev->stream);
     (void)hipStreamSynchronize(dev->transfer);
+    if (dev->idx >= 0 && dev->idx < kMaxDevices) {
+        // (its launches have finished: the next user of the table need not wait for this handle)
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (g_scratch_last_user[dev->idx] == dev) g_scratch_last_user[dev->idx] = nullptr;
+    }
     for (custos_hip_graph* g : dev->graphs) destroy_graph(g);
     // every block of this handle goes back to the driver, pooled or still held by the caller
     for (auto& kv : dev->block_bytes) (void)hipFree(reinterpret_cast<void*>(kv.first));
     for (auto& bucket : dev->cache)
         for (auto& k : bucket.second)
-            if (k->module) (void)hipModuleUnload(k->module);
+            for (hipModule_t module : k->modules)
+                if (module) (void)hipModuleUnload(module);
     (void)hipEventDestroy(dev->t0);
     (void)hipEventDestroy(dev->t1);
     for (hipEvent_t mark : dev->marks)
@@ -453,8 +507,12 @@ const char* custos_hip_last_error(custos_hip_device* dev) {
 
 int32_t custos_hip_sync(custos_hip_device* dev) {
     REQUIRE_DEV(dev);
-    if (dev->capturing)
-        return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "cannot wait for a stream that is recording");
+    // While the device records nothing new reaches the compute stream: the wait is for the
+    // work that was in flight when the recording began.
+    if (dev->capturing) {
+        HIP_TRY(dev, drain_before_immediate_work(dev));
+        return CUSTOS_HIP_OK;
+    }
     HIP_TRY(dev, wait_compute_stream(dev));
     return CUSTOS_HIP_OK;
 }
@@ -504,6 +562,7 @@ int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, ui
     if (bytes == 0) return set_error(dev, CUSTOS_HIP_ERR_ZERO_LENGTH_BUFFER, "zero length buffers are not supported");
     const size_t rounded = pool_size_class(bytes);
     void* p = nullptr;
+    if (dev->capturing && flags != CUSTOS_HIP_ALLOC_UNINIT) HIP_TRY(dev, drain_before_immediate_work(dev));
     auto pooled = dev->pool.find(rounded);
     if (pooled != dev->pool.end() && !pooled->second.empty()) {
         p = pooled->second.back();
@@ -561,6 +620,7 @@ int32_t custos_hip_free(custos_hip_device* dev, uint64_t dptr) {
     dev->block_bytes.erase(known);
     // work that still uses the range must finish first
     if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    else HIP_TRY(dev, drain_before_immediate_work(dev));
     HIP_TRY(dev, hipFree(reinterpret_cast<void*>(dptr)));
     return CUSTOS_HIP_OK;
 }
@@ -591,6 +651,7 @@ int32_t custos_hip_write(custos_hip_device* dev, uint64_t dst, const void* src, 
     if (bytes == 0) return CUSTOS_HIP_OK;
     if (!dst || !src) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null pointer");
     if (dev->capturing) {
+        HIP_TRY(dev, drain_before_immediate_work(dev));
         HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(dst), src, bytes, hipMemcpyHostToDevice, dev->transfer));
         HIP_TRY(dev, hipStreamSynchronize(dev->transfer));
         return CUSTOS_HIP_OK;
@@ -622,6 +683,7 @@ int32_t custos_hip_read(custos_hip_device* dev, void* dst, uint64_t src, size_t 
         return CUSTOS_HIP_OK;
     }
     hipStream_t s = dev->capturing ? dev->transfer : dev->stream;
+    if (dev->capturing) HIP_TRY(dev, drain_before_immediate_work(dev));
     HIP_TRY(dev, hipMemcpyAsync(dst, reinterpret_cast<const void*>(src), bytes, hipMemcpyDeviceToHost, s));
     HIP_TRY(dev, hipStreamSynchronize(s));
     return CUSTOS_HIP_OK;
@@ -663,8 +725,15 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
                                          int32_t operands_per_set, size_t n_sets, size_t n) {
     REQUIRE_DEV(dev);
     if (!kernel || !operands) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel or operand table");
-    if (kernel->spec.kind == Kind::Source || !kernel->fn_batched)
-        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "kernel has no entry point for merged launches");
+    if (kernel->spec.kind == Kind::Source)
+        return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "a caller-written kernel has no entry point for merged launches");
+    // (loading code allocates: the entry point must be there already)
+    const custos_hip_kernel* owner = kernel->code ? kernel->code : kernel;
+    const hipFunction_t fn = owner->fns[static_cast<int>(EntrySet::Batched)];
+    if (!fn)
+        return set_error(dev, CUSTOS_HIP_ERR_NOT_PREPARED,
+                         "the kernel's entry point for merged launches is not loaded: call custos_hip_kernel_prepare_merged "
+                         "where allocation is allowed");
     if (dev->capturing)
         return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the allocation-free merged launch cannot be recorded");
     const int n_ptrs = kernel->spec.kind == Kind::UnaryGrad ? 3 : kernel->spec.expr.n_vars + 1;
@@ -684,15 +753,12 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
                              std::to_string(kScratchWords * 8) + " bytes), got " + std::to_string(n_sets));
     // Operand checks on the host, before anything is launched: aligned, no partial overlap
     // inside a set (`out == in` exactly is fine), and no set writes what another set touches.
+    // The spans live in a buffer the handle reserved when it was created.
     const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(kernel->spec.dtype);
     const int written = kernel->spec.kind == Kind::UnaryGrad ? 1 : n_ptrs - 1;
-    struct Span {
-        uint64_t begin;
-        uint32_t set;
-        bool write;
-    };
-    std::vector<Span> spans;
-    spans.reserve(n_sets * static_cast<size_t>(n_ptrs));
+    using Span = custos_hip_device::OperandSpan;
+    std::vector<Span>& spans = dev->noalloc_spans;
+    spans.clear();
     for (size_t s = 0; s < n_sets; s++) {
         const uint64_t* row = operands + s * static_cast<size_t>(n_ptrs);
         for (int i = 0; i < n_ptrs; i++) {
@@ -704,7 +770,9 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
             spans.push_back({row[i], static_cast<uint32_t>(s), i == written});
         }
     }
-    std::sort(spans.begin(), spans.end(), [](const Span& a, const Span& b) { return a.begin < b.begin; });
+    // (sorted already when the caller lists its sets by address, as a pool of equal buffers does)
+    const auto by_begin = [](const Span& a, const Span& b) { return a.begin < b.begin; };
+    if (!std::is_sorted(spans.begin(), spans.end(), by_begin)) std::sort(spans.begin(), spans.end(), by_begin);
     // sweep by start address: the furthest-reaching earlier span of any kind and the furthest
     // written one, each with a runner-up from another set
     struct Reach {
@@ -735,10 +803,24 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
     unsigned long long tiles_per_seg = std::max(1ull, (n_vec + tile_vecs - 1) / tile_vecs);
     if (tiles_per_seg * n_sets > (1ull << 31) - 1)
         return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
-    // table rows as the `_batched` entry point reads them: addresses, then the literal parameters
-    std::vector<uint64_t> table(n_sets * row_words);
+
+    // From here to the event record one caller at a time per process: the table has one copy per GPU.
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    // The launch of another handle may still be reading the table: this stream's work from here
+    // on waits for it.  (The launches of this handle are ordered by its stream.)
+    if (g_scratch_last_user[dev->idx] && g_scratch_last_user[dev->idx] != dev)
+        HIP_TRY(dev, hipStreamWaitEvent(dev->stream, g_scratch_event[dev->idx], 0));
+    // Table rows as the `_batched` entry point reads them (addresses, then the literal
+    // parameters), written straight into a pinned staging slot; the library's copy kernel moves
+    // them into the table on the compute stream, behind the previous call's launch.
+    const uint64_t table_dev = reinterpret_cast<uint64_t>(dev->scratch_table);
+    unsigned char* slot_host = nullptr;
+    uint64_t slot_dev = 0;
+    int32_t rc = staging_slot(dev, table_dev, &slot_host, &slot_dev);
+    if (rc != CUSTOS_HIP_OK) return rc;
+    uint64_t* table = reinterpret_cast<uint64_t*>(slot_host);  // (the table is 256-byte aligned: phase 0)
     for (size_t s = 0; s < n_sets; s++) {
-        uint64_t* row = table.data() + s * row_words;
+        uint64_t* row = table + s * row_words;
         std::memcpy(row, operands + s * static_cast<size_t>(n_ptrs), static_cast<size_t>(n_ptrs) * 8);
         for (size_t w = 0; w < const_words; w++) {
             uint64_t word = 0;
@@ -746,19 +828,25 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
             row[n_ptrs + w] = word;
         }
     }
-    // The table goes through a pinned staging slot and a copy kernel on the compute stream: it
-    // lands behind the previous call's launch, which still reads the table.
-    const uint64_t table_dev = reinterpret_cast<uint64_t>(dev->scratch_table);
-    int32_t rc = staged_write(dev, table_dev, table.data(), table.size() * 8);
+    rc = staging_slot_send(dev, table_dev, slot_dev, n_sets * row_words * 8);
     if (rc != CUSTOS_HIP_OK) return rc;
     unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, false);
     uint64_t table_arg = table_dev;
     unsigned long long count_arg = count, n_vec_arg = n_vec;
     void* args[] = {&table_arg, &count_arg, &n_vec_arg, &tiles_per_seg, &mode};
     dev->launches_since_wait = true;
-    HIP_TRY(dev, hipModuleLaunchKernel(kernel->fn_batched, static_cast<unsigned int>(tiles_per_seg * n_sets), 1, 1,
+    HIP_TRY(dev, hipModuleLaunchKernel(fn, static_cast<unsigned int>(tiles_per_seg * n_sets), 1, 1,
                                        static_cast<unsigned int>(t.block_threads), 1, 1, 0, dev->stream, args, nullptr));
+    HIP_TRY(dev, hipEventRecord(g_scratch_event[dev->idx], dev->stream));
+    g_scratch_last_user[dev->idx] = dev;
     return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_kernel_prepare_merged(custos_hip_device* dev, custos_hip_kernel* kernel) {
+    REQUIRE_DEV(dev);
+    if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null kernel");
+    hipFunction_t fn = nullptr;
+    return entry_point(dev, kernel, EntrySet::Batched, &fn);
 }
 
 // ---- timing ----

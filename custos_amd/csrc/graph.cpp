@@ -5,6 +5,7 @@
 #include <array>
 #include <cstring>
 #include <queue>
+#include <set>
 
 #include "runtime.hpp"
 
@@ -273,12 +274,17 @@ bool join_chains(ChainBuild& producer, const ChainBuild& consumer, uint64_t byte
     return true;
 }
 
-// The recording with producers joined into their consumers (see above); kernels for the new
-// chains are compiled here, at most `dev->fusing_new_kernels` of them per graph: a chain whose
-// kernel is neither cached nor compiled within that limit (or does not compile) stays the
-// launches it was recorded as.
-int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, bool share_reads, size_t* fused_away) {
-    const std::vector<RecNode>& nodes = *recorded;
+// The recording `nodes` with producers joined into their consumers (see above), in `fused`.
+// The kernels of the joined launches are only named here (handles from the cache, or new ones);
+// the graph build compiles the entry point it replays each of them through, and hands back in
+// `refused` those it could not get (time budget spent, compilation failed): their chains stay
+// the launches they were recorded as (`left_unjoined` counts those launches).
+int32_t fuse_producers(custos_hip_device* dev, const std::vector<RecNode>& nodes, bool share_reads,
+                       const std::set<const custos_hip_kernel*>& refused, std::vector<RecNode>* fused_out, size_t* fused_away,
+                       size_t* left_unjoined) {
+    *fused_away = 0;
+    *left_unjoined = 0;
+    fused_out->clear();
     struct Candidate {
         size_t at;  // index into `out`
         ChainBuild chain;
@@ -389,7 +395,6 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, b
     if (joined_launches == 0) return CUSTOS_HIP_OK;
     // kernels of the chains; the nodes take their final form
     std::vector<RecNode> fused;
-    size_t compiled_here = 0;
     // chains of the same launches wired the same way share a kernel: looked up once per shape
     std::map<std::vector<uint64_t>, custos_hip_kernel*> kernel_of_shape;
     for (size_t i = 0; i < out.size(); i++) {
@@ -430,27 +435,20 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, b
                         stages[s].param_bytes = sk->spec.consts.bytes.size();
                     }
                 }
-                bool compiled = false;
                 Tuning tuning = node.k->spec.tuning;
                 tuning.unroll = 0;  // (only kernels whose vectors per thread were left open are joined)
-                // a kernel that is not there yet is compiled while the limit lasts; a shape without a
-                // kernel (the limit, a compilation that failed) stays the launches it was recorded as
-                if (compiled_here >= dev->fusing_new_kernels) {
-                    KernelSpec probe;
-                    ParseError err;
-                    const int n_ext = static_cast<int>(chain.ext.size()), n_outs = static_cast<int>(outs.size());
-                    if (build_chain_spec(node.k->spec.dtype, stages, n_ext, n_outs, tuning, &probe, &err, /*with_source=*/false))
-                        k = cached_chain_kernel(dev, probe);
-                } else if (chain_kernel(dev, node.k->spec.dtype, std::move(stages), static_cast<int>(chain.ext.size()),
-                                        static_cast<int>(outs.size()), tuning, &k, &compiled) != CUSTOS_HIP_OK) {
+                // a shape without a kernel (one that cannot be generated, one the build refused) stays
+                // the launches it was recorded as
+                if (chain_kernel(dev, node.k->spec.dtype, std::move(stages), static_cast<int>(chain.ext.size()),
+                                 static_cast<int>(outs.size()), tuning, &k) != CUSTOS_HIP_OK ||
+                    refused.count(k))
                     k = nullptr;
-                }
-                compiled_here += compiled;
                 known = kernel_of_shape.emplace(std::move(shape), k).first;
             }
             custos_hip_kernel* const k = known->second;
             if (!k) {
                 // the chain's launches again, in the order of its stages
+                *left_unjoined += chain.size();
                 const uint64_t bytes = node.n * dtype_size(node.k->spec.dtype);
                 for (size_t s = 0; s < chain.size(); s++) {
                     RecNode single = node;
@@ -482,12 +480,12 @@ int32_t fuse_producers(custos_hip_device* dev, std::vector<RecNode>* recorded, b
         fused.push_back(std::move(node));
     }
     *fused_away = nodes.size() - fused.size();
-    *recorded = std::move(fused);
+    *fused_out = std::move(fused);
     return CUSTOS_HIP_OK;
 }
 
 bool batchable(const RecNode& n) {
-    if (n.type != RecNode::Kernel || n.head != 0 || !n.k->fn_batched) return false;
+    if (n.type != RecNode::Kernel || n.head != 0 || n.k->spec.kind == Kind::Source) return false;
     for (uint64_t p : n.ptrs)
         if (p & 15) return false;
     return true;
@@ -504,6 +502,11 @@ struct Planned {
     ResolvedShape shape;                // kernels: vectors per thread and cache policy that suit the bytes the
                                         // node touches; whether it walks its tiles against the previous such node
 };
+
+// The entry point a planned kernel node is replayed through.
+EntrySet entry_of(const Planned& p) {
+    return p.members.size() == 1 ? EntrySet::Single : p.ragged ? EntrySet::Ragged : EntrySet::Batched;
+}
 
 unsigned long long tiles_of(const custos_hip_kernel* k, const RecNode& n, int unroll) {
     const unsigned long long tile_vecs = static_cast<unsigned long long>(k->spec.tuning.block_threads) * unroll;
@@ -550,9 +553,8 @@ std::vector<Planned> group_level(const custos_hip_device* dev, const std::vector
     for (auto& g : groups) {
         bool uniform = true;
         for (size_t i : g.second) uniform = uniform && nodes[i].n == nodes[g.second[0]].n;
-        if (uniform || !g.first->fn_ragged) {
-            // equal lengths: one grid, segment = block / tiles per segment.  (Without the
-            // ragged entry point, different lengths fall back to one batch per length.)
+        if (uniform) {
+            // equal lengths: one grid, segment = block / tiles per segment
             std::vector<std::pair<unsigned long long, Planned>> by_n;
             for (size_t i : g.second) {
                 auto it = std::find_if(by_n.begin(), by_n.end(), [&](const auto& kv) { return kv.first == nodes[i].n; });
@@ -675,7 +677,7 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
         ln.bytes = first.bytes;
     } else if (first.type == RecNode::Source) {
         ln.args = first.arg_values;
-        ln.func = reinterpret_cast<void*>(first.k->fn);
+        ln.func = reinterpret_cast<void*>(first.k->fns[0]);
         ln.grid = dim3(first.grid3[0], first.grid3[1], first.grid3[2]);
         ln.block = dim3(first.block3[0], first.block3[1], first.block3[2]);
         ln.shared_mem = first.shared_mem;
@@ -690,13 +692,17 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
     } else {
         const Tuning& t = p.kern->spec.tuning;
         ln.block = dim3(static_cast<unsigned int>(t.block_threads));
+        // (compiled by now: build_graph asked for the entry point of every planned node)
+        hipFunction_t fn = nullptr;
+        int32_t rc = entry_point(dev, p.kern, entry_of(p), &fn);
+        if (rc != CUSTOS_HIP_OK) return rc;
+        ln.func = reinterpret_cast<void*>(fn);
         if (p.members.size() == 1) {
             for (uint64_t ptr : first.ptrs) ln.args.push_back(value(&ptr, 8));
             const unsigned long long a0 = first.n, a1 = first.head, a2 = first.n_vec;
             ln.args.push_back(value(&a0, 8));
             ln.args.push_back(value(&a1, 8));
             ln.args.push_back(value(&a2, 8));
-            ln.func = reinterpret_cast<void*>(p.kern->fn);
             ln.grid = dim3(launch_grid(dev, p.kern, first.n, first.n_vec, p.shape.unroll));
         } else if (p.ragged) {
             if (p.blocks > (1ull << 31) - 1)
@@ -704,7 +710,6 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
             const uint64_t rows = table + p.table_offset * sizeof(uint64_t);
             const uint64_t map = table + p.map_offset * sizeof(uint64_t);
             ln.args = {value(&rows, 8), value(&map, 8)};
-            ln.func = reinterpret_cast<void*>(p.kern->fn_ragged);
             ln.grid = dim3(static_cast<unsigned int>(p.blocks));
         } else {
             const unsigned long long tiles_per_seg = tiles_of(p.kern, first, p.shape.unroll);
@@ -714,7 +719,6 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
             const uint64_t rows = table + p.table_offset * sizeof(uint64_t);
             const unsigned long long a0 = first.n, a1 = first.n_vec;
             ln.args = {value(&rows, 8), value(&a0, 8), value(&a1, 8), value(&tiles_per_seg, 8)};
-            ln.func = reinterpret_cast<void*>(p.kern->fn_batched);
             ln.grid = dim3(static_cast<unsigned int>(blocks));
         }
         // a generated entry point ends with the block of literal parameters (if the
@@ -940,56 +944,113 @@ int32_t instantiate(custos_hip_device* dev, custos_hip_graph* g, std::vector<std
 }  // namespace
 
 int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
-    std::vector<RecNode>& nodes = dev->recorded;
-    g->recorded = nodes.size();
-    g->signature = signature(nodes);
-    if (dev->fusing) {
-        // (a recording that cannot be joined -- too many new kernels, a kernel that does not
-        // compile -- is built as it was recorded)
-        const std::string error_before = dev->last_error;
-        if (fuse_producers(dev, &nodes, /*share_reads=*/true, &g->fused_away) != CUSTOS_HIP_OK) g->fused_away = 0;
-        dev->last_error = error_before;
-    }
-    const bool serial = dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN || dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN_BY_LEVEL;
-    // The order of a chain only matters where a launch is large enough for the caches to matter;
-    // a recording of small launches keeps the level order and the cheaper analysis.
-    bool follow_recording = false;
-    if (dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN)
-        for (const RecNode& n : nodes) {
-            unsigned long long touched = 0;
-            for (const Access& a : n.acc) touched += a.end - a.begin;
-            follow_recording = follow_recording || touched >= kFollowRecordingFromBytes;
-        }
-    assign_levels(nodes, dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_PER_NODE || follow_recording);
-    int max_level = -1;
-    for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
-    g->levels = static_cast<size_t>(max_level + 1);
+    g->recorded = dev->recorded.size();
+    g->signature = signature(dev->recorded);
     g->built_with = {dev->batching ? 1u : 0u, static_cast<uint64_t>(dev->graph_edges), dev->direct_replay_max,
                      dev->fusing ? 1u : 0u};
+    const bool serial = dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN || dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN_BY_LEVEL;
 
+    // Plan, then get the entry point every planned kernel node is replayed through.  The kernels
+    // of joined launches are new code that nothing but this graph asked for: they are compiled
+    // while the build has spent less than its budget on them, and a chain whose kernel the build
+    // does not get (budget, a compilation that fails) goes back to the launches it was recorded
+    // as -- the recording is then joined and planned again without it (once or twice: what was
+    // compiled on the way is cached).
+    std::vector<RecNode> joined;
+    std::set<const custos_hip_kernel*> refused;
+    uint64_t spent_on_joined_ns = 0;
     std::vector<std::vector<Planned>> plan;
     std::vector<uint64_t> host_table;
-    std::vector<std::vector<size_t>> by_level(static_cast<size_t>(max_level + 1));
-    for (size_t i = 0; i < nodes.size(); i++) by_level[static_cast<size_t>(nodes[i].level)].push_back(i);
-    // One chain: from here on a "level" is one node, in the order the chain will have.
-    if (follow_recording) by_level = stages_in_recording_order(dev, nodes, by_level);
-    // A graph is built to be replayed: its first levels follow its last ones, so the traffic
-    // history starts with one pass over the whole graph.
-    RecentTraffic history;
-    for (const auto& of_level : by_level) record_level(nodes, of_level, &history);
-    // what every level reads, for the producers in the levels before it (the levels after the
-    // last one are the first ones of the next replay)
-    std::vector<std::vector<Access>> level_reads(by_level.size());
-    for (size_t level = 0; level < by_level.size(); level++)
-        for (size_t i : by_level[level])
-            for (const Access& a : nodes[i].acc)
-                if (nodes[i].type != RecNode::Source && reads_operand(nodes[i], a)) level_reads[level].push_back(a);
-    for (size_t level = 0; level < by_level.size(); level++) {
-        std::vector<const std::vector<Access>*> later_reads;
-        for (size_t ahead = 1; ahead <= kLookAheadLevels && ahead <= by_level.size(); ahead++)
-            later_reads.push_back(&level_reads[(level + ahead) % by_level.size()]);
-        plan.push_back(plan_level(dev, nodes, by_level[level], &history, later_reads, &host_table));
+    const std::vector<RecNode>* planned_from = nullptr;
+    for (;;) {
+        std::vector<RecNode>* use = &dev->recorded;
+        g->fused_away = g->unjoined = 0;
+        if (dev->fusing) {
+            const std::string error_before = dev->last_error;
+            if (fuse_producers(dev, dev->recorded, /*share_reads=*/true, refused, &joined, &g->fused_away, &g->unjoined) == CUSTOS_HIP_OK &&
+                g->fused_away > 0)
+                use = &joined;
+            else
+                g->fused_away = 0;
+            dev->last_error = error_before;
+        }
+        std::vector<RecNode>& nodes = *use;
+        // The order of a chain only matters where a launch is large enough for the caches to matter;
+        // a recording of small launches keeps the level order and the cheaper analysis.
+        bool follow_recording = false;
+        if (dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_CHAIN)
+            for (const RecNode& n : nodes) {
+                unsigned long long touched = 0;
+                for (const Access& a : n.acc) touched += a.end - a.begin;
+                follow_recording = follow_recording || touched >= kFollowRecordingFromBytes;
+            }
+        assign_levels(nodes, dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_PER_NODE || follow_recording);
+        int max_level = -1;
+        for (const RecNode& n : nodes) max_level = std::max(max_level, n.level);
+        g->levels = static_cast<size_t>(max_level + 1);
+
+        plan.clear();
+        host_table.clear();
+        std::vector<std::vector<size_t>> by_level(static_cast<size_t>(max_level + 1));
+        for (size_t i = 0; i < nodes.size(); i++) by_level[static_cast<size_t>(nodes[i].level)].push_back(i);
+        // One chain: from here on a "level" is one node, in the order the chain will have.
+        if (follow_recording) by_level = stages_in_recording_order(dev, nodes, by_level);
+        // A graph is built to be replayed: its first levels follow its last ones, so the traffic
+        // history starts with one pass over the whole graph.
+        RecentTraffic history;
+        for (const auto& of_level : by_level) record_level(nodes, of_level, &history);
+        // what every level reads, for the producers in the levels before it (the levels after the
+        // last one are the first ones of the next replay)
+        std::vector<std::vector<Access>> level_reads(by_level.size());
+        for (size_t level = 0; level < by_level.size(); level++)
+            for (size_t i : by_level[level])
+                for (const Access& a : nodes[i].acc)
+                    if (nodes[i].type != RecNode::Source && reads_operand(nodes[i], a)) level_reads[level].push_back(a);
+        for (size_t level = 0; level < by_level.size(); level++) {
+            std::vector<const std::vector<Access>*> later_reads;
+            for (size_t ahead = 1; ahead <= kLookAheadLevels && ahead <= by_level.size(); ahead++)
+                later_reads.push_back(&level_reads[(level + ahead) % by_level.size()]);
+            plan.push_back(plan_level(dev, nodes, by_level[level], &history, later_reads, &host_table));
+        }
+        planned_from = use;
+
+        bool plan_again = false;
+        for (const auto& level : plan)
+            for (const Planned& p : level) {
+                if (!p.kern) continue;
+                custos_hip_kernel* owner = p.kern->code ? p.kern->code : p.kern;
+                const EntrySet which = entry_of(p);
+                if (owner->fns[static_cast<int>(which)] || refused.count(owner)) continue;
+                hipFunction_t fn = nullptr;
+                if (owner->spec.kind != Kind::Chain) {
+                    // (a kernel made while the device was recording, or its first merged launch)
+                    int32_t rc = entry_point(dev, owner, which, &fn);
+                    if (rc != CUSTOS_HIP_OK) return rc;
+                    continue;
+                }
+                if (spent_on_joined_ns >= dev->fusing_budget_ms * 1000000ull) {
+                    refused.insert(owner);
+                    if (g->unjoined_reason.empty())
+                        g->unjoined_reason = "the build's time budget for compiling kernels of joined launches (" +
+                                             std::to_string(dev->fusing_budget_ms) + " ms) was spent";
+                    plan_again = true;
+                    continue;
+                }
+                const uint64_t before = dev->compile_ns;
+                const std::string error_before = dev->last_error;
+                const int32_t rc = entry_point(dev, owner, which, &fn);
+                spent_on_joined_ns += dev->compile_ns - before;
+                if (rc != CUSTOS_HIP_OK) {
+                    refused.insert(owner);
+                    g->unjoined_reason = dev->last_error;
+                    dev->last_error = error_before;
+                    plan_again = true;
+                }
+            }
+        if (!plan_again) break;
     }
+    std::vector<RecNode>& nodes = *const_cast<std::vector<RecNode>*>(planned_from);
+
     if (!host_table.empty()) {
         HIP_TRY(dev, hipMalloc(&g->table, host_table.size() * sizeof(uint64_t)));
         HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
@@ -1092,12 +1153,14 @@ extern "C" {
 int32_t custos_hip_capture_begin(custos_hip_device* dev) {
     REQUIRE_DEV(dev);
     if (dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the device is already recording");
-    // Earlier eager work must be complete before anything recorded can run, and
-    // the recorded list starts empty.  Allocation, reads and writes stay legal
-    // while recording: they execute at once and are not part of the graph.
-    HIP_TRY(dev, hipStreamSynchronize(dev->stream));
+    // The recorded list starts empty.  Allocation, reads and writes stay legal while
+    // recording: they execute at once, outside the compute stream's order, and are not part
+    // of the graph; the first of them waits for the work that is in flight now
+    // (drain_before_immediate_work).  Recording itself launches nothing, and a replay of
+    // the graph is ordered on the compute stream behind that work, so beginning takes no wait.
     dev->recorded.clear();
     dev->capturing = true;
+    dev->undrained_at_capture = true;
     return CUSTOS_HIP_OK;
 }
 
@@ -1147,7 +1210,19 @@ int32_t custos_hip_set_graph_fusing(custos_hip_device* dev, int32_t enabled) {
     REQUIRE_DEV(dev);
     if (enabled < 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "negative value");
     dev->fusing = enabled != 0;
-    dev->fusing_new_kernels = enabled > 1 ? static_cast<size_t>(enabled) : 16;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_set_graph_fusing_budget(custos_hip_device* dev, uint32_t milliseconds) {
+    REQUIRE_DEV(dev);
+    dev->fusing_budget_ms = milliseconds;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t custos_hip_graph_unjoined(custos_hip_graph* graph, size_t* launches, const char** reason) {
+    if (!graph || !launches) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    *launches = graph->unjoined;
+    if (reason) *reason = graph->unjoined_reason.c_str();
     return CUSTOS_HIP_OK;
 }
 

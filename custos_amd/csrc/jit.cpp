@@ -4,6 +4,7 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -18,11 +19,11 @@ namespace {
 // ---- code objects on disk ----
 //
 // With CUSTOS_HIP_KERNEL_CACHE_DIR set, every compiled code object is stored as
-// <dir>/<key>-<arch>-<hiprtc version>.co together with the source it was built
+// <dir>/<key>[_batched|_ragged]-<arch>-<hiprtc version>.co together with the source it was built
 // from; a later process loads it instead of compiling when the stored source is
 // identical (the 64-bit key alone is not trusted).
 
-std::string cache_file(const KernelSpec& spec, const std::string& arch) {
+std::string cache_file(const KernelSpec& spec, const std::string& arch, EntrySet which) {
     const char* dir = std::getenv("CUSTOS_HIP_KERNEL_CACHE_DIR");
     if (!dir || !*dir) return "";
     int major = 0, minor = 0;
@@ -32,18 +33,19 @@ std::string cache_file(const KernelSpec& spec, const std::string& arch) {
         if (c == ':' || c == '/' || c == '+') c = '_';
     char key[17];
     std::snprintf(key, sizeof key, "%016llx", static_cast<unsigned long long>(spec.hash));
-    return std::string(dir) + "/" + key + "-" + a + "-" + std::to_string(major) + "." + std::to_string(minor) + ".co";
+    return std::string(dir) + "/" + key + entry_suffix(which) + "-" + a + "-" + std::to_string(major) + "." + std::to_string(minor) + ".co";
 }
 
 // the text hiprtc compiles: generated kernels start with a comment line that
 // spells the expression as the caller wrote it; it is not part of the identity
-std::string source_identity(const KernelSpec& spec) {
-    if (spec.kind == Kind::Source) return spec.name + "\n" + spec.source;
-    return spec.source.substr(spec.source.find('\n') + 1);
+std::string source_identity(const KernelSpec& spec, EntrySet which) {
+    const std::string& text = spec.source[static_cast<int>(which)];
+    if (spec.kind == Kind::Source) return spec.name + "\n" + text;
+    return text.substr(text.find('\n') + 1);
 }
 
-bool load_cached_code(const KernelSpec& spec, const std::string& arch, std::vector<char>* code) {
-    const std::string path = cache_file(spec, arch);
+bool load_cached_code(const KernelSpec& spec, const std::string& arch, EntrySet which, std::vector<char>* code) {
+    const std::string path = cache_file(spec, arch, which);
     if (path.empty()) return false;
     std::ifstream f(path, std::ios::binary);
     if (!f) return false;
@@ -55,21 +57,21 @@ bool load_cached_code(const KernelSpec& spec, const std::string& arch, std::vect
     std::string src(src_len, '\0');
     f.read(&src[0], static_cast<std::streamsize>(src_len));
     f.read(reinterpret_cast<char*>(&code_len), 8);
-    if (!f || src != source_identity(spec) || code_len == 0 || code_len > (1u << 28)) return false;
+    if (!f || src != source_identity(spec, which) || code_len == 0 || code_len > (1u << 28)) return false;
     code->resize(code_len);
     f.read(code->data(), static_cast<std::streamsize>(code_len));
     return static_cast<bool>(f);
 }
 
-void store_cached_code(const KernelSpec& spec, const std::string& arch, const std::vector<char>& code) {
-    const std::string path = cache_file(spec, arch);
+void store_cached_code(const KernelSpec& spec, const std::string& arch, EntrySet which, const std::vector<char>& code) {
+    const std::string path = cache_file(spec, arch, which);
     if (path.empty()) return;
     (void)mkdir(std::getenv("CUSTOS_HIP_KERNEL_CACHE_DIR"), 0777);
     const std::string tmp = path + ".tmp" + std::to_string(static_cast<long>(getpid()));
     {
         std::ofstream f(tmp, std::ios::binary | std::ios::trunc);
         if (!f) return;
-        const std::string src = source_identity(spec);
+        const std::string src = source_identity(spec, which);
         const uint64_t src_len = src.size(), code_len = code.size();
         f.write("CUSTOSC1", 8);
         f.write(reinterpret_cast<const char*>(&src_len), 8);
@@ -110,6 +112,19 @@ int32_t spec_from_c(custos_hip_device* dev, int32_t kind, int32_t dtype, const c
     return CUSTOS_HIP_OK;
 }
 
+// The three translation units of a generated kernel, one after the other (generated on the way).
+std::string all_units(KernelSpec* spec) {
+    std::string text;
+    for (int w = 0; w < kEntrySets; w++) {
+        ParseError err;
+        if (spec->source[w].empty()) (void)emit_kernel_source(spec, &err, static_cast<EntrySet>(w));
+        // (every unit starts with a line that spells the expression: once is enough here)
+        if (w) text += "\n// ---- translation unit of the entry point " + spec->name + entry_suffix(static_cast<EntrySet>(w)) + " ----\n";
+        text += w ? spec->source[w].substr(spec->source[w].find('\n') + 1) : spec->source[w];
+    }
+    return text;
+}
+
 int32_t copy_out_string(const std::string& s, char* buf, size_t cap, size_t* needed) {
     if (needed) *needed = s.size() + 1;
     if (buf && cap) {
@@ -125,9 +140,15 @@ int32_t copy_out_string(const std::string& s, char* buf, size_t cap, size_t* nee
 // ---- hiprtc ----
 
 int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec,
-                               const std::string& arch, std::vector<char>* code) {
+                               const std::string& arch, std::vector<char>* code, EntrySet which) {
+    const std::string& text = spec.source[static_cast<int>(which)];
+    // A switch for tests of the error paths: kernels whose entry name contains the value fail to
+    // compile (what a compiler defect or an exhausted machine would do, neither of which a test can call up).
+    if (const char* fail = std::getenv("CUSTOS_HIP_FAIL_COMPILE_OF"))
+        if (*fail && spec.name.find(fail) != std::string::npos)
+            return set_error(dev, CUSTOS_HIP_ERR_COMPILE, "hiprtcCompileProgram: refused, CUSTOS_HIP_FAIL_COMPILE_OF names " + spec.name);
     hiprtcProgram prog = nullptr;
-    hiprtcResult r = hiprtcCreateProgram(&prog, spec.source.c_str(), "custos_kernel.hip", 0, nullptr, nullptr);
+    hiprtcResult r = hiprtcCreateProgram(&prog, text.c_str(), "custos_kernel.hip", 0, nullptr, nullptr);
     if (r != HIPRTC_SUCCESS)
         return set_error(dev, CUSTOS_HIP_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
     std::vector<std::string> opts = hiprtc_options(arch);
@@ -142,7 +163,7 @@ int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec,
         hiprtcDestroyProgram(&prog);
         return set_error(dev, CUSTOS_HIP_ERR_COMPILE,
                          std::string("hiprtcCompileProgram: ") + hiprtcGetErrorString(r) + "\n" + log +
-                             "\n--- source ---\n" + spec.source);
+                             "\n--- source ---\n" + text);
     }
     size_t size = 0;
     hiprtcGetCodeSize(prog, &size);
@@ -152,30 +173,59 @@ int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec,
     return CUSTOS_HIP_OK;
 }
 
-// Code object from the disk cache or from hiprtc, loaded as a module; entry point looked up.
-int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k) {
+// The translation unit `which` of `k`: code object from the disk cache or from hiprtc, loaded as
+// a module, entry point looked up.  `k` owns its code.
+static int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k, EntrySet which) {
+    const int w = static_cast<int>(which);
+    if (k->spec.source[w].empty()) {
+        ParseError err;
+        if (k->spec.kind == Kind::Source || !emit_kernel_source(&k->spec, &err, which))
+            return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+    }
     std::vector<char> code;
-    bool from_disk = load_cached_code(k->spec, dev->arch, &code);
-    if (from_disk && hipModuleLoadData(&k->module, code.data()) != hipSuccess) {
+    hipModule_t module = nullptr;
+    bool from_disk = load_cached_code(k->spec, dev->arch, which, &code);
+    if (from_disk && hipModuleLoadData(&module, code.data()) != hipSuccess) {
         (void)hipGetLastError();  // a stale or damaged file: compile instead
-        k->module = nullptr;
+        module = nullptr;
         from_disk = false;
     }
     if (!from_disk) {
-        int32_t rc = compile_to_code_object(dev, k->spec, dev->arch, &code);
+        const auto t0 = std::chrono::steady_clock::now();
+        int32_t rc = compile_to_code_object(dev, k->spec, dev->arch, &code, which);
+        dev->compile_ns += static_cast<uint64_t>(
+            std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count());
         if (rc != CUSTOS_HIP_OK) return rc;
-        HIP_TRY(dev, hipModuleLoadData(&k->module, code.data()));
-        store_cached_code(k->spec, dev->arch, code);
+        HIP_TRY(dev, hipModuleLoadData(&module, code.data()));
+        store_cached_code(k->spec, dev->arch, which, code);
         dev->compiles++;
     } else {
         dev->disk_hits++;
     }
-    hipError_t e = hipModuleGetFunction(&k->fn, k->module, k->spec.name.c_str());
+    hipFunction_t fn = nullptr;
+    hipError_t e = hipModuleGetFunction(&fn, module, (k->spec.name + entry_suffix(which)).c_str());
     if (e != hipSuccess) {
-        (void)hipModuleUnload(k->module);
-        k->module = nullptr;
+        (void)hipModuleUnload(module);
         return hip_fail(dev, e, "hipModuleGetFunction");
     }
+    k->modules[w] = module;
+    k->fns[w] = fn;
+    return CUSTOS_HIP_OK;
+}
+
+int32_t entry_point(custos_hip_device* dev, custos_hip_kernel* k, EntrySet which, hipFunction_t* fn) {
+    const int w = static_cast<int>(which);
+    if (!k->fns[w]) {
+        custos_hip_kernel* owner = k->code ? k->code : k;
+        if (!owner->fns[w]) {
+            if (owner->spec.kind == Kind::Source && which != EntrySet::Single)
+                return set_error(dev, CUSTOS_HIP_ERR_KIND_MISMATCH, "a caller-written kernel has no entry point for merged launches");
+            int32_t rc = build_module(dev, owner, which);
+            if (rc != CUSTOS_HIP_OK) return rc;
+        }
+        k->fns[w] = owner->fns[w];
+    }
+    *fn = k->fns[w];
     return CUSTOS_HIP_OK;
 }
 
@@ -197,27 +247,12 @@ static custos_hip_kernel* handle_for_values(custos_hip_kernel* owner, std::uniqu
     const std::string values(k->spec.consts.bytes.begin(), k->spec.consts.bytes.end());
     auto sibling = owner->siblings.find(values);
     if (sibling == owner->siblings.end()) {
-        k->code = owner;  // (which also holds the text)
-        k->fn = owner->fn;
-        k->fn_batched = owner->fn_batched;
-        k->fn_ragged = owner->fn_ragged;
+        k->code = owner;  // (which also holds the text, the modules and the entry points)
         k->expr_src = src;
         for (int i = 0; i < n_markers; i++) k->markers.push_back(markers[i]);
         sibling = owner->siblings.emplace(values, std::move(k)).first;
     }
     return sibling->second.get();
-}
-
-// Entry points of a freshly built module for many launches in one grid.
-static void find_merged_entries(custos_hip_kernel* k) {
-    if (hipModuleGetFunction(&k->fn_batched, k->module, (k->spec.name + "_batched").c_str()) != hipSuccess) {
-        (void)hipGetLastError();
-        k->fn_batched = nullptr;
-    }
-    if (hipModuleGetFunction(&k->fn_ragged, k->module, (k->spec.name + "_ragged").c_str()) != hipSuccess) {
-        (void)hipGetLastError();
-        k->fn_ragged = nullptr;
-    }
 }
 
 // Parses, looks the key up in the cache, compiles on a miss.
@@ -257,15 +292,21 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
             }
         }
     }
+    // The text also finds what cannot be compiled (a transcendental node over integers, say).
     ParseError err;
     if (!emit_kernel_source(&k->spec, &err)) return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
-    rc = build_module(dev, k.get());
-    if (rc != CUSTOS_HIP_OK) return rc;
-    // further entry points of the module: many launches in one grid
-    find_merged_entries(k.get());
+    k->code = k.get();
+    // The entry point for single launches is compiled now, so that no launch compiles anything --
+    // unless the device is recording: nothing is launched then, and the graph build compiles the
+    // entry point each kernel is replayed through (for launches that are joined or merged that
+    // is not this one).
+    if (!dev->capturing) {
+        hipFunction_t unused = nullptr;
+        rc = entry_point(dev, k.get(), EntrySet::Single, &unused);
+        if (rc != CUSTOS_HIP_OK) return rc;
+    }
     k->expr_src = src;
     for (int i = 0; i < n_markers; i++) k->markers.push_back(markers[i]);
-    k->code = k.get();
     *out = k.get();
     dev->cache[k->spec.hash].push_back(std::move(k));
     return CUSTOS_HIP_OK;
@@ -274,10 +315,9 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
 custos_hip_kernel* cached_chain_kernel(custos_hip_device* dev, const KernelSpec& spec) { return find_code(dev, spec); }
 
 int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs,
-                     const Tuning& tuning, custos_hip_kernel** out, bool* compiled) {
+                     const Tuning& tuning, custos_hip_kernel** out) {
     std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
     ParseError err;
-    if (compiled) *compiled = false;
     if (!build_chain_spec(dtype, std::move(stages), n_ext, n_outs, tuning, &k->spec, &err, /*with_source=*/false))
         return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
     if (custos_hip_kernel* known = find_code(dev, k->spec)) {
@@ -285,14 +325,11 @@ int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage
         *out = known;
         return CUSTOS_HIP_OK;
     }
+    // (nothing is compiled here: the graph build asks for the entry point it replays the chain through)
     if (!emit_kernel_source(&k->spec, &err)) return set_error(dev, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
-    int32_t rc = build_module(dev, k.get());
-    if (rc != CUSTOS_HIP_OK) return rc;
-    find_merged_entries(k.get());
     k->expr_src = k->spec.chain_text;
     k->code = k.get();
     *out = k.get();
-    if (compiled) *compiled = true;
     dev->cache[k->spec.hash].push_back(std::move(k));
     return CUSTOS_HIP_OK;
 }
@@ -369,17 +406,17 @@ int32_t custos_hip_source_compile(custos_hip_device* dev, const char* src, const
     std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);
     k->spec.kind = Kind::Source;
     k->spec.name = fn_name;
-    k->spec.source = src;
+    k->spec.source[0] = src;
     k->spec.hash = fnv1a64(fn_name, std::strlen(fn_name), fnv1a64(src, std::strlen(src), fnv1a64("custos-source-v1", 16)));
     auto& bucket = dev->cache[k->spec.hash];
     for (auto& cached : bucket) {
-        if (cached->spec.kind == Kind::Source && cached->spec.name == k->spec.name && cached->spec.source == k->spec.source) {
+        if (cached->spec.kind == Kind::Source && cached->spec.name == k->spec.name && cached->spec.source[0] == k->spec.source[0]) {
             dev->hits++;
             *kernel = cached.get();
             return CUSTOS_HIP_OK;
         }
     }
-    int32_t rc = build_module(dev, k.get());
+    int32_t rc = build_module(dev, k.get(), EntrySet::Single);
     if (rc != CUSTOS_HIP_OK) return rc;
     *kernel = k.get();
     bucket.push_back(std::move(k));
@@ -388,7 +425,7 @@ int32_t custos_hip_source_compile(custos_hip_device* dev, const char* src, const
 
 const char* custos_hip_kernel_source(const custos_hip_kernel* kernel) {
     if (!kernel) return "";
-    return (kernel->code ? kernel->code : kernel)->spec.source.c_str();
+    return (kernel->code ? kernel->code : kernel)->spec.source[0].c_str();
 }
 
 const char* custos_hip_kernel_name(const custos_hip_kernel* kernel) {
@@ -417,6 +454,13 @@ int32_t custos_hip_cache_stats(custos_hip_device* dev, uint64_t* compiles, uint6
     return CUSTOS_HIP_OK;
 }
 
+int32_t custos_hip_compile_stats(custos_hip_device* dev, uint64_t* units, double* milliseconds) {
+    REQUIRE_DEV(dev);
+    if (units) *units = dev->compiles;
+    if (milliseconds) *milliseconds = static_cast<double>(dev->compile_ns) * 1e-6;
+    return CUSTOS_HIP_OK;
+}
+
 int32_t custos_hip_cache_disk_hits(custos_hip_device* dev, uint64_t* disk_hits) {
     REQUIRE_DEV(dev);
     if (disk_hits) *disk_hits = dev->disk_hits;
@@ -430,7 +474,7 @@ int32_t custos_hip_expr_emit(int32_t kind, int32_t dtype, const char* src, const
     int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), true, &spec);
     if (rc != CUSTOS_HIP_OK) return rc;
     if (hash) *hash = spec.hash;
-    return copy_out_string(spec.source, buf, cap, needed);
+    return copy_out_string(all_units(&spec), buf, cap, needed);
 }
 
 int32_t custos_hip_expr_emit_shared(int32_t kind, int32_t dtype, const char* src, const char* const* markers,
@@ -440,7 +484,7 @@ int32_t custos_hip_expr_emit_shared(int32_t kind, int32_t dtype, const char* src
     int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), false, &spec);
     if (rc != CUSTOS_HIP_OK) return rc;
     if (hash) *hash = spec.hash;
-    return copy_out_string(spec.source, buf, cap, needed);
+    return copy_out_string(all_units(&spec), buf, cap, needed);
 }
 
 int32_t custos_hip_set_literal_policy(custos_hip_device* dev, int32_t policy) {
@@ -459,10 +503,15 @@ int32_t custos_hip_expr_build_code_object(int32_t kind, int32_t dtype, const cha
     KernelSpec spec;
     int32_t rc = spec_from_c(nullptr, kind, dtype, src, markers, n_markers, tuning_from_c(tuning), true, &spec);
     if (rc != CUSTOS_HIP_OK) return rc;
-    std::vector<char> code;
-    rc = compile_to_code_object(nullptr, spec, "gfx950", &code);
-    if (rc != CUSTOS_HIP_OK) return rc;
-    if (code_size) *code_size = code.size();
+    (void)all_units(&spec);
+    size_t total = 0;
+    for (int w = 0; w < kEntrySets; w++) {
+        std::vector<char> code;
+        rc = compile_to_code_object(nullptr, spec, "gfx950", &code, static_cast<EntrySet>(w));
+        if (rc != CUSTOS_HIP_OK) return rc;
+        total += code.size();
+    }
+    if (code_size) *code_size = total;
     return CUSTOS_HIP_OK;
 }
 
@@ -504,13 +553,17 @@ int32_t custos_hip_chain_emit(int32_t dtype, const char* const* stage_srcs, cons
     ParseError err;
     if (!build_chain_spec(static_cast<DType>(dtype), std::move(stages), n_inputs, n_outputs, Tuning{}, &spec, &err))
         return set_error(nullptr, err.code ? err.code : CUSTOS_HIP_ERR_EXPR_SYNTAX, err.message);
+    const std::string text = all_units(&spec);
     if (code_size) {
-        std::vector<char> code;
-        const int32_t rc = compile_to_code_object(nullptr, spec, "gfx950", &code);
-        if (rc != CUSTOS_HIP_OK) return rc;
-        *code_size = code.size();
+        *code_size = 0;
+        for (int w = 0; w < kEntrySets; w++) {
+            std::vector<char> code;
+            const int32_t rc = compile_to_code_object(nullptr, spec, "gfx950", &code, static_cast<EntrySet>(w));
+            if (rc != CUSTOS_HIP_OK) return rc;
+            *code_size += code.size();
+        }
     }
-    return copy_out_string(spec.source, buf, cap, needed);
+    return copy_out_string(text, buf, cap, needed);
 }
 
 int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t* unroll,

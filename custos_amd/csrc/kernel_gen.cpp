@@ -231,8 +231,8 @@ bool stage_plan(const ChainStage& stage, DType dtype, int base, ConstPlan* plan,
     return true;
 }
 
-// Text of the per-element function, the tile function and the three entry points of one
-// kernel.  Operand naming inside a kernel: in0.. are the inputs, `out` the output; for a unary
+// Text of the per-element function, the tile function and the entry points of one kernel
+// (every translation unit holds the functions and ONE entry point: emit_kernel_source).  Operand naming inside a kernel: in0.. are the inputs, `out` the output; for a unary
 // gradient 0 = lhs, 1 = lhs_grad (also the output), 2 = out_grad.
 struct KernelText {
     const KernelSpec& k;
@@ -393,37 +393,20 @@ struct KernelText {
         return s;
     }
 
-    // The numbers of vectors per thread this kernel has a tile function for: the caller's
-    // choice, or both shapes the library picks from per launch.
-    std::vector<int> unrolls() const {
-        if (k.auto_unroll) return {2, 1};
-        return {k.tuning.unroll};
-    }
-
-    // `custos_tile<U>(args)` for the launch's number of vectors per thread `U`.
+    // `custos_tile<U>(args)`: the kernel's one tile function (U vectors per thread: the caller's
+    // choice, or 2 -- what every automatic launch shape takes).
     std::string tile_call(const std::string& indent, const std::string& args) const {
-        const std::vector<int> us = unrolls();
-        if (us.size() == 1) return indent + "custos_tile" + std::to_string(us[0]) + "(" + args + ");\n";
-        return indent + "if (U == 2) custos_tile2(" + args + ");\n" + indent + "else custos_tile1(" + args + ");\n";
+        return indent + "custos_tile" + std::to_string(k.tuning.unroll) + "(" + args + ");\n";
     }
 
-    // Tiles of a range of `n_vec` vectors, as an expression over constant divisors (a division by
-    // the launch's own `U` would cost every wavefront a 64-bit division routine).
+    // Tiles of a range of `n_vec` vectors (a constant divisor: no division routine).
     std::string n_tiles_expr() const {
-        auto tiles = [](int unroll) {
-            const std::string tv = "((u64)CUSTOS_BLOCK * " + std::to_string(unroll) + ")";
-            return "(n_vec + " + tv + " - 1) / " + tv;
-        };
-        const std::vector<int> us = unrolls();
-        if (us.size() == 1) return tiles(us[0]);
-        return "(U == 2 ? " + tiles(2) + " : " + tiles(1) + ")";
+        const std::string tv = "((u64)CUSTOS_BLOCK * " + std::to_string(k.tuning.unroll) + ")";
+        return "(n_vec + " + tv + " - 1) / " + tv;
     }
 
-    // `const u64 U = ...;`: vectors per thread of this launch, from the mode word
-    std::string unroll_of_mode() const {
-        if (!k.auto_unroll) return "    const u64 U = " + std::to_string(k.tuning.unroll) + ";\n";
-        return "    const u64 U = (mode >> 8) & 15;\n";
-    }
+    // `const u64 U = ...;`: vectors per thread
+    std::string unroll_of_mode() const { return "    const u64 U = " + std::to_string(k.tuning.unroll) + ";\n"; }
 
     // One tile of `unroll` vectors per thread, starting at vector `first` of the operands (the
     // same for the whole workgroup): every lane loads all its vectors, then computes and stores.
@@ -490,11 +473,15 @@ struct KernelText {
         // Elements outside the 16-byte aligned body: `head` leading ones and the
         // tail. Lanes beyond the count are masked off by the wavefront's EXEC.  Most launches
         // have none (bit 12 of the mode word): one scalar test instead of per-lane arithmetic.
+        // (One loop over both, so that the expression is expanded once for them.)
         s += "    if (!(mode & 4096)) return;\n";
         s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
         s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BLOCK;\n";
-        s += "    if (gid < head) " + scalar_stmt("gid") + "\n";
-        s += "    for (u64 i = head + n_vec * CUSTOS_VEC + gid; i < n; i += n_threads) " + scalar_stmt("i") + "\n";
+        s += "    const u64 body_end = head + n_vec * CUSTOS_VEC;\n";
+        s += "    const u64 n_edge = head + (n - body_end);\n";
+        s += "    for (u64 e = gid; e < n_edge; e += n_threads) {\n";
+        s += "        const u64 i = e < head ? e : e - head + body_end;\n";
+        s += "        " + scalar_stmt("i") + "\n    }\n";
         s += "}\n";
         return s;
     }
@@ -609,7 +596,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds the vectors per thread as requested: 0 = chosen per launch)
     int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, 18 /* template version */};
+                       k.tuning.blocks_per_cu, 19 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -627,7 +614,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     return true;
 }
 
-bool emit_kernel_source(KernelSpec* spec, ParseError* err) {
+bool emit_kernel_source(KernelSpec* spec, ParseError* err, EntrySet which) {
     KernelSpec& k = *spec;
     std::string body;
     if (k.kind == Kind::Chain) {
@@ -676,12 +663,10 @@ static __device__ __forceinline__ void custos_st(const custos_rsrc rs, const uns
 
     const KernelText text(k);
     s += text.elem_fn();
-    for (int unroll : text.unrolls()) s += text.tile_fn(unroll);
-    s += text.single_entry();
-    s += text.batched_entry();
-    s += text.ragged_entry();
+    s += text.tile_fn(k.tuning.unroll);
+    s += which == EntrySet::Single ? text.single_entry() : which == EntrySet::Batched ? text.batched_entry() : text.ragged_entry();
 
-    k.source = std::move(s);
+    k.source[static_cast<int>(which)] = std::move(s);
     return true;
 }
 
@@ -742,7 +727,7 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
                         (stage.out >= 0 ? " -> out" + std::to_string(stage.out) : std::string()) + "; ";
     }
     int32_t tail[7] = {static_cast<int32_t>(Kind::Chain), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, n_ext, n_outs, 18 /* template version */};
+                       k.tuning.blocks_per_cu, n_ext, n_outs, 19 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     k.stages = std::move(stages);

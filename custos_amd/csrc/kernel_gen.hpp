@@ -30,7 +30,7 @@ struct Tuning {
     // knobs are chosen per launch from the bytes it touches (preferred_shape)
     // unless the caller fixes them.
     int block_threads = 128;
-    int unroll = 0;         // 16-byte vectors per thread and tile; 0: chosen per launch (2 or 1)
+    int unroll = 0;         // 16-byte vectors per thread and tile; 0: the library's choice (2)
     int blocks_per_cu = 0;  // <= 0: one tile per workgroup
     int nontemporal = -1;   // bit 0 loads, bit 1 stores, 64 stores written through at once; -1: chosen per
                             // launch.  Read from the device's tuning when a launch is issued or a graph built.
@@ -66,7 +66,7 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
 //   bit 0      the tiles are walked from the last to the first
 //   bit 1, 2   non-temporal loads, non-temporal stores
 //   bit 7      stores are written through to device scope at once instead of lingering in an L2
-//   bits 8..11 vectors per thread (only read by kernels whose unroll factor was left open)
+//   bits 8..11 vectors per thread (for the record: the kernel's one tile function has them compiled in)
 //   bit 12     (single-launch entry point) the range has scalar elements: a head before the first
 //              16-byte boundary or a tail after the last whole vector
 //   bits 16..  (single-launch entry point) the number of tiles of the vector range
@@ -102,6 +102,20 @@ struct ChainStage {
 };
 constexpr int kMaxChainStages = 8, kMaxChainInputs = 8, kMaxChainOutputs = 6;
 
+// A generated kernel has three entry points, each in a translation unit of its own (the
+// per-element function and the tile function repeat in all three) that is compiled when it is
+// first needed: a transcendental expression is expanded eight or nine times per entry point,
+// and most kernels are only ever launched through one of them.
+enum class EntrySet : int {
+    Single = 0,   // `<name>`: one launch over one set of operands
+    Batched = 1,  // `<name>_batched`: many operand sets of equal length in one grid
+    Ragged = 2,   // `<name>_ragged`: many operand sets of different lengths in one grid
+};
+constexpr int kEntrySets = 3;
+inline const char* entry_suffix(EntrySet which) {
+    return which == EntrySet::Single ? "" : which == EntrySet::Batched ? "_batched" : "_ragged";
+}
+
 struct KernelSpec {
     Kind kind = Kind::Apply;
     DType dtype = DType::F32;
@@ -110,8 +124,7 @@ struct KernelSpec {
     int n_ext = 0, n_outs = 0;       // Chain: input and output pointers (inputs first)
     std::string chain_text;          // Chain: the stages spelt out, literal values included
     Tuning tuning;             // as compiled: workgroup size, grid kind, most vectors per thread
-    bool auto_unroll = false;  // the caller left the vectors per thread open: the kernel holds the
-                               // tile functions for 2 and for 1, and every launch picks one
+    bool auto_unroll = false;  // the caller left the vectors per thread open (the kernel takes 2)
     ConstPlan consts;          // literals that are launch parameters, and this text's values for them
     int n_literals = 0;        // literals in the expression, parameters or not
     std::vector<uint64_t> code_literals;  // values of the literals that stay in the code, in node order
@@ -119,7 +132,7 @@ struct KernelSpec {
     uint64_t hash = 0;   // cache key: expression without the parameter values, dtype, kind, tuning
     std::string name;    // entry point: custos_<kind>_<dtype>_<hash>, unique per kernel so
                          // that profiler output tells the kernels apart
-    std::string source;  // complete translation unit (empty until emit_kernel_source)
+    std::string source[3];  // the kernel's translation units by EntrySet (each empty until emit_kernel_source)
     int vec_elems = 4;   // elements per 16-byte vector
 };
 
@@ -138,9 +151,9 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
 // Pointer parameters of a generated kernel's single-launch entry point (= the width of a table
 // row of a merged launch, before the literal parameters).
 int kernel_pointers(const KernelSpec& k);
-// Generates `k->source` (which also finds node / element type combinations that cannot be
+// Generates `k->source[which]` (which also finds node / element type combinations that cannot be
 // compiled, such as a transcendental node over integers).
-bool emit_kernel_source(KernelSpec* k, ParseError* err);
+bool emit_kernel_source(KernelSpec* k, ParseError* err, EntrySet which = EntrySet::Single);
 // Whether two specs describe the same translation unit, without looking at the text: kind,
 // element type, launch shape, expression structure and the literals that stay in the code.
 bool same_code(const KernelSpec& a, const KernelSpec& b);

@@ -145,6 +145,10 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
         dev->recorded.push_back(std::move(node));
         return CUSTOS_HIP_OK;
     }
+    // (compiled when custos_hip_expr_compile returned, unless the device was recording then)
+    hipFunction_t fn = nullptr;
+    rc = entry_point(dev, k, EntrySet::Single, &fn);
+    if (rc != CUSTOS_HIP_OK) return rc;
     // the launch shape that suits the bytes this launch touches and what the launches just
     // before it left in the memory-side cache
     const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
@@ -184,7 +188,7 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     if (k->spec.consts.n_params > 0) args.push_back(k->spec.consts.bytes.data());
     args.push_back(&mode);
     dev->launches_since_wait = true;
-    HIP_TRY(dev, hipModuleLaunchKernel(k->fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
+    HIP_TRY(dev, hipModuleLaunchKernel(fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
                                        1, 1, 0, dev->stream, args.data(), nullptr));
     return CUSTOS_HIP_OK;
 }
@@ -277,7 +281,7 @@ int32_t custos_hip_source_launch(custos_hip_device* dev, custos_hip_kernel* kern
     }
     std::vector<void*> args(params, params + n_params);
     dev->launches_since_wait = true;
-    HIP_TRY(dev, hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+    HIP_TRY(dev, hipModuleLaunchKernel(kernel->fns[0], grid[0], grid[1], grid[2], block[0], block[1], block[2],
                                        shared_mem_bytes, dev->stream, args.data(), nullptr));
     return CUSTOS_HIP_OK;
 }
@@ -291,7 +295,7 @@ int32_t custos_hip_source_launch1d(custos_hip_device* dev, custos_hip_kernel* ke
     if (len == 0) return CUSTOS_HIP_OK;
     // block size from the occupancy calculator, grid = ceil(len / block) (kernel_launch.rs:141-151)
     int min_grid = 0, block_size = 0;
-    HIP_TRY(dev, hipModuleOccupancyMaxPotentialBlockSize(&min_grid, &block_size, kernel->fn, 0, 0));
+    HIP_TRY(dev, hipModuleOccupancyMaxPotentialBlockSize(&min_grid, &block_size, kernel->fns[0], 0, 0));
     if (block_size <= 0) block_size = 256;
     const uint64_t blocks = (len + static_cast<size_t>(block_size) - 1) / static_cast<size_t>(block_size);
     if (blocks > 0x7fffffffull) return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "more workgroups than a one-dimensional grid holds");

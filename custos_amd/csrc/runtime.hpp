@@ -20,14 +20,16 @@
 
 struct custos_hip_kernel {
     custos_hip::KernelSpec spec;
-    hipModule_t module = nullptr;
-    hipFunction_t fn = nullptr;
-    hipFunction_t fn_batched = nullptr;  // equal launches in one grid
-    hipFunction_t fn_ragged = nullptr;   // launches of different lengths in one grid
+    // One module and entry point per EntrySet (single launch; equal launches in one grid;
+    // launches of different lengths in one grid), each compiled and loaded when it is first
+    // needed (custos_hip::entry_point).  Only the kernel that owns the code loads modules; a
+    // caller-written kernel has the first one only.
+    hipModule_t modules[custos_hip::kEntrySets] = {nullptr, nullptr, nullptr};
+    hipFunction_t fns[custos_hip::kEntrySets] = {nullptr, nullptr, nullptr};
     std::string expr_src;  // the expression as the caller spelt it
     std::vector<std::string> markers;
     // Handles for the same code with other values of the literal parameters, by those
-    // values: they share this kernel's module (their own `module` stays null) and differ
+    // values: they share this kernel's modules (their own stay null) and differ
     // in `spec.consts.bytes`, `spec.expr` and `expr_src`.  `code` points at the kernel that
     // owns the module (itself for the owner).
     std::map<std::string, std::unique_ptr<custos_hip_kernel>> siblings;
@@ -66,6 +68,8 @@ struct custos_hip_graph {
     std::vector<uint64_t> signature;
     std::array<uint64_t, 4> built_with{};
     size_t fused_away = 0;    // recorded launches that became stages of a later launch's kernel
+    size_t unjoined = 0;      // recorded launches that would have been joined, had the build got their kernel
+    std::string unjoined_reason;  // why not: the time budget, or the compiler's message
     std::vector<std::string> node_names;  // entry point of every kernel node, in the order of the chain / the levels
     // how long the last wait took that waited for one launch of this graph and nothing else
     uint64_t last_wait_ns = 0;
@@ -126,6 +130,8 @@ struct custos_hip_device {
     std::string arch;
     custos_hip::Tuning tuning;
     bool capturing = false;          // recording: launches, clears and copies go to `recorded`
+    bool undrained_at_capture = false;  // work was (possibly) in flight on the compute stream when the recording
+                                        // began and nothing has waited for it since (drain_before_immediate_work)
     int32_t literal_policy = 0;      // CUSTOS_HIP_LITERALS_*
     // per shared-form key: how many distinct texts of that structure were compiled or looked up
     std::unordered_map<uint64_t, uint32_t> value_sets_seen;
@@ -159,6 +165,14 @@ struct custos_hip_device {
     uint32_t graphs_since_wait = 0;
     bool launches_since_wait = false;
     unsigned long long* scratch_table = nullptr;  // this device's copy of the library's static operand table
+    // operand ranges of a call of custos_hip_apply_fn_many_noalloc, for its overlap checks (room
+    // reserved when the handle is created: that call may not allocate, on the host either)
+    struct OperandSpan {
+        uint64_t begin;
+        uint32_t set;
+        bool write;
+    };
+    std::vector<OperandSpan> noalloc_spans;
     unsigned char* read_stage = nullptr;  // pinned host memory short reads (first slot) and writes are staged in
     uint64_t read_stage_dev = 0;          // its device address
     uint64_t waits_begun = 0, waits_done = 0;  // waits for the compute stream, numbered
@@ -168,9 +182,11 @@ struct custos_hip_device {
     unsigned long long launch_parity = 0;  // direction of the last launch that alternates
     bool batching = true;            // merge equal independent launches of a level into one grid
     bool fusing = true;              // a recorded apply launch is joined with the apply launches that read what it wrote
-    size_t fusing_new_kernels = 16;  // kernels of joined launches a graph build may compile
+    uint64_t fusing_budget_ms = 1000;  // a graph build starts compiling kernels of joined launches while it has spent
+                                       // less than this on them
     std::vector<RecNode> recorded;
-    uint64_t compiles = 0, hits = 0, disk_hits = 0;
+    uint64_t compiles = 0, hits = 0, disk_hits = 0;  // translation units compiled; cache hits; units loaded from disk
+    uint64_t compile_ns = 0;                          // time spent in hiprtc so far
     std::string last_error;
     std::unordered_map<uint64_t, std::vector<std::unique_ptr<custos_hip_kernel>>> cache;
     // expression exactly as the caller spelt it (with kind, type, markers, tuning) -> kernel:
@@ -215,6 +231,7 @@ inline Tuning tuning_from_c(const custos_hip_tuning* t) {
 
 // device.hip
 hipError_t wait_compute_stream(custos_hip_device* dev);
+hipError_t drain_before_immediate_work(custos_hip_device* dev);
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec);
 unsigned int fill_block();
 // device-to-device copy, launched or recorded: the identity kernel, or the runtime's copy
@@ -225,8 +242,11 @@ void* fill_zero_kernel();  // host handle of the zero-fill kernel, for graph ker
 
 // jit.cpp
 int32_t compile_to_code_object(custos_hip_device* dev, const KernelSpec& spec, const std::string& arch,
-                               std::vector<char>* code);
-int32_t build_module(custos_hip_device* dev, custos_hip_kernel* k);
+                               std::vector<char>* code, EntrySet which = EntrySet::Single);
+// The entry point `which` of `k`, compiled (or loaded from the disk cache) and looked up on first
+// use.  Kernels made while the device records are not compiled until a graph build or a launch
+// asks for the entry point it uses.
+int32_t entry_point(custos_hip_device* dev, custos_hip_kernel* k, EntrySet which, hipFunction_t* fn);
 // The kernel of the expression `x` over `dtype` elements (compiled once per device).
 int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel** out);
 // How a launch of `k` that touches `footprint_bytes` runs: vectors per thread and cache policy
@@ -242,9 +262,9 @@ struct ResolvedShape {
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
                             CacheHint hint = CacheHint::Unknown, unsigned long long working_set_bytes = 0);
 
-// jit.cpp: the kernel for a chain of apply expressions (compiled on first use, then cached).
+// jit.cpp: the kernel handle for a chain of apply expressions (cached; compiled when an entry point is asked for).
 int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs,
-                     const Tuning& tuning, custos_hip_kernel** out, bool* compiled);
+                     const Tuning& tuning, custos_hip_kernel** out);
 // The mode word of a single launch of `k` over n elements (n_vec vectors after `head` scalar
 // elements) in the given shape.
 inline uint64_t single_launch_mode(const custos_hip_kernel* k, unsigned long long n, unsigned long long head,

@@ -120,6 +120,13 @@ class Graph:
         self.device._check(self.device.lib.custos_hip_graph_fused_launches(self.handle, C.byref(n)))
         return n.value
 
+    def unjoined(self):
+        """(recorded launches the build would have joined but left as recorded, reason): the time budget of
+        the build, or the compiler's message."""
+        n, why = C.c_size_t(0), C.c_char_p()
+        self.device._check(self.device.lib.custos_hip_graph_unjoined(self.handle, C.byref(n), C.byref(why)))
+        return n.value, (why.value or b"").decode()
+
     def edge_count(self) -> int:
         """Dependency edges of the instantiated graph, joins included (0 for a directly replayed chain)."""
         e = C.c_size_t(0)
@@ -372,9 +379,23 @@ class HIP:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 
     def set_graph_fusing(self, enabled) -> None:
-        """Whether a graph build joins recorded launches with the launches that read their output; a number
-        above 1 also sets how many kernels of joined launches a graph build may compile (default 16)."""
-        self._check(self.lib.custos_hip_set_graph_fusing(self.handle, int(enabled)))
+        """Whether a graph build joins recorded launches with the launches that read their output."""
+        self._check(self.lib.custos_hip_set_graph_fusing(self.handle, int(bool(enabled))))
+
+    def set_graph_fusing_budget(self, milliseconds: int) -> None:
+        """How long a graph build may spend compiling kernels of joined launches (default 1000 ms; 0: only
+        kernels from the caches)."""
+        self._check(self.lib.custos_hip_set_graph_fusing_budget(self.handle, int(milliseconds)))
+
+    def prepare_merged(self, kernel) -> None:
+        """Compiles and loads the kernel's entry point for many launches of equal length in one grid."""
+        self._check(self.lib.custos_hip_kernel_prepare_merged(self.handle, kernel))
+
+    def compile_stats(self):
+        """(translation units compiled by hiprtc so far, milliseconds spent in them)."""
+        units, ms = C.c_uint64(0), C.c_double(0)
+        self._check(self.lib.custos_hip_compile_stats(self.handle, C.byref(units), C.byref(ms)))
+        return units.value, ms.value
 
     def launch_hint_stats(self):
         """(not part of a chain, chain that stays in the memory-side cache, chain that streams) counts of

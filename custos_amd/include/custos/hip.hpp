@@ -196,8 +196,10 @@ class HIP : public Device<HIP<Mods>, Mods> {
 
     // `LazyRun::run` (src/devices/cuda/lazy.rs:31-49): the first run of a given
     // operation list records it into a graph and instantiates it; every run
-    // launches the graph once and waits.  `version` changes whenever the
-    // recorded operations change; then the graph is rebuilt.
+    // launches the graph once.  `version` changes whenever the recorded
+    // operations change; then the graph is rebuilt.  The wait that ends the
+    // reference's run is deferred to whatever next looks at the results (see
+    // `set_run_waits`).
     template <class Replay>
     void lazy_run(uint64_t version, Replay replay) {
         if (!graph_ || graph_version_ != version) {
@@ -223,10 +225,21 @@ class HIP : public Device<HIP<Mods>, Mods> {
     }
 
     // The reference's run returns after the stream has drained
-    // (src/devices/cuda/lazy.rs:42-43).  A caller that runs the same graph many times
-    // and reads results only at the end can switch the wait off: runs then queue behind
-    // each other on the stream, and `read`, `sync` and every copy to the host still wait
-    // for them.
+    // (src/devices/cuda/lazy.rs:42-43).  Here a run returns once its graph is queued on
+    // the device's one compute stream, and the wait is taken by whatever looks at the
+    // results next: `read` (and everything built on it: `read_to_vec`, serialisation,
+    // `Display`), `sync`, dropping the device; a `write` into a buffer of the program is a
+    // copy on the same stream behind the run (it waits only for its own host range);
+    // dropping a buffer returns its block to a pool whose reuse is ordered on that stream
+    // too, or waits before the block goes back to the driver; re-recording a changed
+    // program waits before its first allocation or transfer.  Device memory cannot be
+    // reached from the host except through these calls, so a program sees the same values
+    // whether the wait sits in `run` or there; what moves is the time `run` itself takes
+    // and the call that reports a failure of the device (an error of the launch itself --
+    // a dropped buffer, a rejected graph -- is still thrown by `run`).  Runs that follow
+    // each other without looking at results queue back to back: a small program then costs
+    // its kernels, not kernels + completion signal + wake-up + launch latency per run.
+    // `set_run_waits(true)` restores the wait inside every run.
     void set_run_waits(bool waits) { run_waits_ = waits; }
     bool run_waits() const { return run_waits_; }
 
@@ -308,7 +321,7 @@ class HIP : public Device<HIP<Mods>, Mods> {
     custos_hip_graph* graph_ = nullptr;
     uint64_t graph_version_ = 0;
     uint64_t graph_builds_ = 0;
-    bool run_waits_ = true;
+    bool run_waits_ = false;
 };
 
 }  // namespace custos

@@ -104,6 +104,10 @@ extern "C" {
                                  out: u64, n: usize) -> i32;
     pub fn custos_hip_apply_fn_many_noalloc(dev: *mut HipDeviceHandle, kernel: *mut HipKernel, operands: *const u64,
                                             operands_per_set: i32, n_sets: usize, n: usize) -> i32;
+    pub fn custos_hip_kernel_prepare_merged(dev: *mut HipDeviceHandle, kernel: *mut HipKernel) -> i32;
+    pub fn custos_hip_set_graph_fusing_budget(dev: *mut HipDeviceHandle, milliseconds: u32) -> i32;
+    pub fn custos_hip_graph_unjoined(graph: *mut HipGraph, launches: *mut usize, reason: *mut *const c_char) -> i32;
+    pub fn custos_hip_compile_stats(dev: *mut HipDeviceHandle, units: *mut u64, milliseconds: *mut f64) -> i32;
     pub fn custos_hip_add_unary_grad(dev: *mut HipDeviceHandle, kernel: *mut HipKernel, lhs: u64, lhs_grad: u64,
                                      out_grad: u64, n: usize) -> i32;
     pub fn custos_hip_capture_begin(dev: *mut HipDeviceHandle) -> i32;

@@ -71,6 +71,9 @@ pub struct HipDevice {
     #[cfg(feature = "lazy")]
     pub graph: Cell<*mut HipGraph>,
     /// Whether `LazyRun::run` waits for the stream (the reference does, `cuda/lazy.rs:42-43`).
+    /// Off by default: a run returns once its graph is queued, and `read`, `write`, `sync`,
+    /// dropping a buffer or the device, and an allocation during the next recording are
+    /// ordered behind it or wait for it, so a program sees the same values either way.
     pub run_waits: Cell<bool>,
 }
 
@@ -84,7 +87,7 @@ impl HipDevice {
             handle,
             #[cfg(feature = "lazy")]
             graph: Cell::new(core::ptr::null_mut()),
-            run_waits: Cell::new(true),
+            run_waits: Cell::new(false),
         })
     }
 

@@ -9,7 +9,9 @@ use super::api::{custos_hip_capture_begin, custos_hip_capture_end_reuse, custos_
 /// first recording; later runs record the same program, get the same graph back without
 /// any build, and launch it once -- the CUDA device runs every operation eagerly and then
 /// the graph again from the second run on (`src/devices/cuda/lazy.rs:31-49`).  A changed
-/// program (a new operation, another buffer) builds a new graph by itself.
+/// program (a new operation, another buffer) builds a new graph by itself.  The reference's
+/// wait after the launch is deferred (`HipDevice::run_waits`): beginning the next recording
+/// takes no wait either, and the first read, write, allocation or `sync` while it is open does.
 impl<Mods> crate::LazyRun for HIP<Mods> {
     fn run(&self) -> crate::Result<()> {
         let previous = self.graph.get();

@@ -1,24 +1,40 @@
 // Times the benchmark configurations the way user code runs them: through the module
-// stack `HIP<Graph<Lazy<Base>>>`, with the reference's run semantics (every `run()` launches
-// the recorded graph and waits for it: src/devices/cuda/lazy.rs:31-49).
+// stacks of the C++ mirror on the `HIP` device.
 //
 //   c1  eager `apply_fn(|x| x.exp())` on `HIP<Base>` over 2^20 f32, again and again: every call prints
 //       the expression, looks the kernel up, retrieves a new output buffer and launches; nothing
 //       waits between the calls (the reference's eager launches do not wait either), one wait at
 //       the end of each timed batch of 64 calls
-//   c2  five `apply_fn` calls (sin, *2, +1, max 0, -0.5) on a lazily recorded f32 buffer,
-//       `optimize_mem_graph`, `unary_fusing`, then `run()` again and again
+//   c2  five `apply_fn` calls (sin, *2, +1, max 0, -0.5) on a lazily recorded f32 buffer of
+//       `HIP<Graph<Lazy<Base>>>`, `optimize_mem_graph`, `unary_fusing`, then `run()` again and again
 //       (the shape of src/op_hint.rs:121-140 and examples/lazy_and_fusing.rs)
+//   c3  `unary_ew` tanh with its gradient function (src/unary.rs:97-132) over 2^26 f32, three ways:
+//       `--stack eager`  `HIP<Autograd<Base>>`: every step calls `unary_ew` (a new output buffer, the
+//                        forward launch, a gradient function on the tape) and `backward` (the tape
+//                        runs the gradient launch);
+//       `--stack lazy`   `HIP<Autograd<Lazy<Base>>>`: `unary_ew` recorded once, every step is `run()`
+//                        (the forward graph) and `backward` (the gradient launch, eagerly), the loop
+//                        of src/unary.rs:284-341;
+//       `--stack joined` `HIP<Lazy<Base>>`: `apply_fn` and `add_unary_grad` both recorded, every step is
+//                        `run()`: the graph build joins the two launches into one kernel that loads x once.
+//       The seed of the backward pass is y_grad itself: it is written into y's gradient buffer once,
+//       on the device, before the timed steps (what src/unary.rs:383 does with `grad_mut_unbound`), and
+//       `backward_from` starts the tape from it.
+//   c4  eager `apply_fn(|x| exp(x*0.5)*x + x*x)` on `HIP<Base>` over 2^28 f16
 //   c5  1024 buffers of 4096 f32: t = a*b; u = t+c; y = sqrt(abs(u))*0.3, recorded once, run
 //       again and again; `--fuse` also calls `elementwise_fusing` first
 //
-// Every run is timed on the host clock around `device.run()`, wait included, and the program
-// prints one JSON line (mean, median and minimum per run).  `bench.py` starts it as a child
-// process; with `--dump K FILE` the first K outputs are written to FILE so that the caller can
-// compare them with its own reference.
+// Two figures per configuration, both on the host clock.  `us_per_run`: `steps` steps in a row and one
+// wait for the device at the end, divided by `steps`: what a loop of runs costs when nothing looks at
+// the results in between (a run returns once its work is queued; `read`, `sync` and the like take the
+// wait).  `run_and_wait`: every step followed by `sync()`, timed one by one: what a run costs when
+// its result is looked at straight away (the reference's run always waits: src/devices/cuda/lazy.rs:31-49).
+// The program prints one JSON line; `bench.py` starts it as a child process.  With `--dump K FILE` the
+// first K outputs of a last, separate step are written to FILE so that the caller can compare them with
+// its own reference; c3 and c4 read their inputs from files the caller wrote (`--input`, `--input2`).
 //
-// Inputs are the synthetic ones of the benchmark: SplitMix64 over a counter, 24 bits mapped to
-// lo + u * (hi - lo) in f32 arithmetic.
+// Inputs of c1, c2, c5 are the synthetic ones of the benchmark: SplitMix64 over a counter, 24 bits
+// mapped to lo + u * (hi - lo) in f32 arithmetic.
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
@@ -31,6 +47,7 @@
 
 using namespace custos;
 using Dev = HIP<Graph<Lazy<Base>>>;
+using Clock = std::chrono::steady_clock;
 
 static uint64_t splitmix64(uint64_t seed, uint64_t index) {
     uint64_t z = seed + (index + 1) * 0x9E3779B97F4A7C15ull;
@@ -49,44 +66,94 @@ static std::vector<float> uniform_f32(uint64_t seed, size_t n, float lo, float s
     return v;
 }
 
-struct Timing {
-    double mean_us, median_us, min_us;
-};
-
-// `settle_ms`: after the first run (which records, compiles and builds the graph) runs are
-// repeated untimed until that much time has passed; after an idle period the device needs some
-// tens of milliseconds of work to return to its steady clocks.
-template <class F>
-static Timing time_runs(F run, int warmup, int steps, int settle_ms) {
-    run();
-    const auto settled = std::chrono::steady_clock::now() + std::chrono::milliseconds(settle_ms);
-    while (std::chrono::steady_clock::now() < settled) run();
-    for (int i = 0; i < warmup; i++) run();
-    std::vector<double> us(static_cast<size_t>(steps));
-    for (int i = 0; i < steps; i++) {
-        const auto t0 = std::chrono::steady_clock::now();
-        run();
-        us[static_cast<size_t>(i)] = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+template <class T>
+static std::vector<T> read_file(const std::string& path, size_t count) {
+    static_assert(std::is_trivially_copyable_v<T>, "raw element type");
+    std::vector<T> v(count);
+    FILE* f = std::fopen(path.c_str(), "rb");
+    if (!f || std::fread(static_cast<void*>(v.data()), sizeof(T), count, f) != count) {
+        std::fprintf(stderr, "cannot read %zu elements from %s\n", count, path.c_str());
+        std::exit(2);
     }
-    double sum = 0;
-    for (double v : us) sum += v;
-    std::sort(us.begin(), us.end());
-    return {sum / steps, us[us.size() / 2], us.front()};
+    std::fclose(f);
+    return v;
 }
 
-static void dump(Dev& device, uint64_t ptr, size_t count, const char* path) {
-    std::vector<float> first(count);
-    device.read_raw(first.data(), ptr, count * sizeof(float));
-    FILE* f = std::fopen(path, "wb");
-    if (!f || std::fwrite(first.data(), sizeof(float), count, f) != count) {
-        std::fprintf(stderr, "cannot write %s\n", path);
+static void write_file(const std::string& path, const void* data, size_t bytes, bool append = false) {
+    FILE* f = std::fopen(path.c_str(), append ? "ab" : "wb");
+    if (!f || std::fwrite(data, 1, bytes, f) != bytes) {
+        std::fprintf(stderr, "cannot write %s\n", path.c_str());
         std::exit(2);
     }
     std::fclose(f);
 }
 
+static double us_since(Clock::time_point t0) { return std::chrono::duration<double, std::micro>(Clock::now() - t0).count(); }
+
+struct Timing {
+    double queued_us;                      // per step: `steps` steps and one wait
+    double wait_mean_us, wait_median_us, wait_min_us;  // per step: every step followed by a wait
+    int steps;
+};
+
+// `settle_ms`: after the first step (which records, compiles and builds the graph) steps are
+// repeated untimed until that much time has passed; after an idle period the device needs some
+// tens of milliseconds of work to return to its steady clocks.
+template <class F, class W>
+static Timing time_runs(F step, W wait, int warmup, int steps, int settle_ms) {
+    step();
+    wait();
+    const auto settled = Clock::now() + std::chrono::milliseconds(settle_ms);
+    while (Clock::now() < settled) {
+        for (int i = 0; i < 8; i++) step();
+        wait();
+    }
+    for (int i = 0; i < warmup; i++) step();
+    wait();
+    Timing t{};
+    t.steps = steps;
+    const auto t0 = Clock::now();
+    for (int i = 0; i < steps; i++) step();
+    wait();
+    t.queued_us = us_since(t0) / steps;
+    std::vector<double> us(static_cast<size_t>(steps));
+    for (int i = 0; i < steps; i++) {
+        const auto t1 = Clock::now();
+        step();
+        wait();
+        us[static_cast<size_t>(i)] = us_since(t1);
+    }
+    double sum = 0;
+    for (double v : us) sum += v;
+    std::sort(us.begin(), us.end());
+    t.wait_mean_us = sum / steps;
+    t.wait_median_us = us[us.size() / 2];
+    t.wait_min_us = us.front();
+    return t;
+}
+
+static std::string timing_json(const Timing& t, double bytes_per_step) {
+    char buf[512];
+    std::snprintf(buf, sizeof buf,
+                  "\"steps\": %d, \"us_per_run\": %.3f, \"GBps\": %.2f, \"run_and_wait\": {\"mean_us\": %.3f, \"median_us\": %.3f, "
+                  "\"min_us\": %.3f, \"GBps_median\": %.2f}",
+                  t.steps, t.queued_us, bytes_per_step / (t.queued_us * 1e-6) / 1e9, t.wait_mean_us, t.wait_median_us, t.wait_min_us,
+                  bytes_per_step / (t.wait_median_us * 1e-6) / 1e9);
+    return buf;
+}
+
+template <class D>
+static void dump_f32(D& device, uint64_t ptr, size_t count, const std::string& path, bool append = false) {
+    std::vector<float> first(count);
+    device.read_raw(first.data(), ptr, count * sizeof(float));
+    write_file(path, first.data(), count * sizeof(float), append);
+}
+
+static auto tanh_forward = [](auto x) { return x.tanh(); };
+static auto tanh_gradient = [](auto x) { return Scalar<float>(1.f).sub(x.tanh().mul(x.tanh())); };
+
 int main(int argc, char** argv) {
-    std::string config = "c2", dump_path;
+    std::string config = "c2", dump_path, input, input2, stack = "eager";
     int log2n = 0, steps = 100, warmup = 20, settle_ms = 150;
     size_t dump_count = 0;
     bool fuse = false;
@@ -100,10 +167,13 @@ int main(int argc, char** argv) {
             return argv[++i];
         };
         if (a == "--config") config = value();
+        else if (a == "--stack") stack = value();
         else if (a == "--log2n") log2n = std::atoi(value());
         else if (a == "--steps") steps = std::atoi(value());
         else if (a == "--warmup") warmup = std::atoi(value());
         else if (a == "--settle-ms") settle_ms = std::atoi(value());
+        else if (a == "--input") input = value();
+        else if (a == "--input2") input2 = value();
         else if (a == "--fuse") fuse = true;
         else if (a == "--dump") {
             dump_count = static_cast<size_t>(std::atoll(value()));
@@ -125,21 +195,14 @@ int main(int argc, char** argv) {
             const Timing t = time_runs(
                 [&] {
                     for (int i = 0; i < batch; i++) out = device.apply_fn(buf, [](auto x) { return x.exp(); });
-                    device.sync();
                 },
-                warmup, steps, settle_ms);
-            if (dump_count) {
-                std::vector<float> first(std::min(dump_count, n));
-                device.read_raw(first.data(), out.ptr(), first.size() * sizeof(float));
-                FILE* f = std::fopen(dump_path.c_str(), "wb");
-                if (!f || std::fwrite(first.data(), sizeof(float), first.size(), f) != first.size()) return 2;
-                std::fclose(f);
-            }
-            std::printf("{\"config\": \"c1\", \"stack\": \"HIP<Base>\", \"calls\": \"apply_fn(exp) x %d, sync()\", \"waits\": false, "
+                [&] { device.sync(); }, warmup, steps, settle_ms);
+            if (dump_count) dump_f32(device, out.ptr(), std::min(dump_count, n), dump_path);
+            std::printf("{\"config\": \"c1\", \"stack\": \"HIP<Base>\", \"calls\": \"apply_fn(exp) x %d, sync()\", "
                         "\"elements\": %zu, \"steps\": %d, \"warmup\": %d, \"us_per_call\": %.3f, \"median_us\": %.3f, "
                         "\"min_us\": %.3f, \"GBps\": %.2f}\n",
-                        batch, n, steps, warmup, t.mean_us / batch, t.median_us / batch, t.min_us / batch,
-                        8.0 * static_cast<double>(n) / (t.mean_us / batch * 1e-6) / 1e9);
+                        batch, n, steps, warmup, t.wait_mean_us / batch, t.wait_median_us / batch, t.wait_min_us / batch,
+                        8.0 * static_cast<double>(n) / (t.wait_mean_us / batch * 1e-6) / 1e9);
         } else if (config == "c2") {
             const size_t n = size_t(1) << (log2n ? log2n : 28);
             Dev device(0);
@@ -152,16 +215,130 @@ int main(int argc, char** argv) {
             auto out = device.apply_fn(r, [](auto x) { return x.sub(0.5f); });
             device.optimize_mem_graph();
             device.unary_fusing();
-            const Timing t = time_runs([&] { device.run(); }, warmup, steps, settle_ms);
-            if (dump_count) dump(device, out.replace().ptr(), std::min(dump_count, n), dump_path.c_str());
-            const double gbs = 8.0 * static_cast<double>(n) / (t.mean_us * 1e-6) / 1e9;
+            const auto first = Clock::now();
+            device.run();
+            device.sync();
+            const double first_run_ms = us_since(first) * 1e-3;
+            const Timing t = time_runs([&] { device.run(); }, [&] { device.sync(); }, warmup, steps, settle_ms);
+            if (dump_count) dump_f32(device, out.replace().ptr(), std::min(dump_count, n), dump_path);
             std::printf("{\"config\": \"c2\", \"stack\": \"HIP<Graph<Lazy<Base>>>\", \"calls\": \"5 x apply_fn, optimize_mem_graph, "
-                        "unary_fusing, run()\", \"waits\": true, \"elements\": %zu, \"steps\": %d, \"warmup\": %d, "
-                        "\"us_per_run\": %.3f, \"median_us\": %.3f, \"min_us\": %.3f, \"GBps\": %.2f, \"GBps_median\": %.2f, "
+                        "unary_fusing, run()\", \"elements\": %zu, \"warmup\": %d, %s, \"first_run_ms\": %.2f, "
                         "\"kernel_nodes\": %zu, \"graph_builds\": %llu}\n",
-                        n, steps, warmup, t.mean_us, t.median_us, t.min_us, gbs,
-                        8.0 * static_cast<double>(n) / (t.median_us * 1e-6) / 1e9, device.graph_kernel_nodes(),
+                        n, warmup, timing_json(t, 8.0 * static_cast<double>(n)).c_str(), first_run_ms, device.graph_kernel_nodes(),
                         static_cast<unsigned long long>(device.graph_builds()));
+        } else if (config == "c3") {
+            const size_t n = size_t(1) << (log2n ? log2n : 26);
+            if (input.empty() || input2.empty()) {
+                std::fprintf(stderr, "c3 needs --input (x) and --input2 (y_grad)\n");
+                return 2;
+            }
+            const std::vector<float> xs = read_file<float>(input, n), ygs = read_file<float>(input2, n);
+            const std::vector<float> tenth(n, 0.1f);
+            const double bytes = 24.0 * static_cast<double>(n);
+            const size_t k = std::min(dump_count, n);
+            if (stack == "eager") {
+                using D = HIP<Autograd<Base>>;
+                D device(0);
+                auto x = device.buffer(xs).require_grad();
+                auto x_grad = x.grad(device);
+                uint64_t y_ptr = 0;
+                bool moved = false;
+                auto step = [&] {
+                    auto y = device.unary_ew(x, tanh_forward, tanh_gradient);
+                    if (y_ptr == 0) {
+                        // the first output: its gradient buffer is made and takes y_grad, once
+                        y_ptr = y.ptr();
+                        auto y_grad = y.grad(device);
+                        y_grad.write(ygs);
+                    }
+                    moved = moved || y.ptr() != y_ptr;  // (the pool hands every step's output the same block)
+                    device.backward_from(y, [](auto&) {});
+                };
+                const Timing t = time_runs(step, [&] { device.sync(); }, warmup, steps, settle_ms);
+                if (moved) {
+                    std::fprintf(stderr, "c3: the output buffer moved between steps, so its gradient was not y_grad\n");
+                    return 1;
+                }
+                if (k) {
+                    x_grad.write(tenth);
+                    auto y = device.unary_ew(x, tanh_forward, tanh_gradient);
+                    device.backward_from(y, [](auto&) {});
+                    dump_f32(device, y.ptr(), k, dump_path);
+                    dump_f32(device, x_grad.ptr(), k, dump_path, true);
+                }
+                std::printf("{\"config\": \"c3\", \"stack\": \"HIP<Autograd<Base>>\", \"calls\": \"per step: unary_ew(tanh, 1 - tanh^2), "
+                            "backward from y_grad in y's gradient buffer\", \"elements\": %zu, \"warmup\": %d, %s}\n",
+                            n, warmup, timing_json(t, bytes).c_str());
+            } else if (stack == "lazy") {
+                using D = HIP<Autograd<Lazy<Base>>>;
+                D device(0);
+                auto x = device.buffer(xs).require_grad();
+                auto x_grad = x.grad(device);
+                auto y = device.unary_ew(x, tanh_forward, tanh_gradient);
+                device.run();
+                {
+                    auto y_grad = y.replace().grad(device);
+                    y_grad.write(ygs);
+                }
+                auto step = [&] {
+                    device.run();
+                    device.backward_from(y.replace(), [](auto&) {});
+                };
+                const Timing t = time_runs(step, [&] { device.sync(); }, warmup, steps, settle_ms);
+                if (k) {
+                    x_grad.write(tenth);
+                    step();
+                    dump_f32(device, y.replace().ptr(), k, dump_path);
+                    dump_f32(device, x_grad.ptr(), k, dump_path, true);
+                }
+                std::printf("{\"config\": \"c3\", \"stack\": \"HIP<Autograd<Lazy<Base>>>\", \"calls\": \"unary_ew recorded once; per step: "
+                            "run(), backward from y_grad in y's gradient buffer\", \"elements\": %zu, \"warmup\": %d, %s, "
+                            "\"kernel_nodes\": %zu, \"graph_builds\": %llu}\n",
+                            n, warmup, timing_json(t, bytes).c_str(), device.graph_kernel_nodes(),
+                            static_cast<unsigned long long>(device.graph_builds()));
+            } else if (stack == "joined") {
+                using D = HIP<Lazy<Base>>;
+                D device(0);
+                auto x = device.buffer(xs);
+                auto x_grad = device.buffer(tenth);
+                auto y_grad = device.buffer(ygs);
+                auto y = device.apply_fn(x, tanh_forward);
+                device.add_unary_grad(x, x_grad, y_grad, tanh_gradient);
+                const Timing t = time_runs([&] { device.run(); }, [&] { device.sync(); }, warmup, steps, settle_ms);
+                if (k) {
+                    x_grad.write(tenth);
+                    device.run();
+                    dump_f32(device, y.replace().ptr(), k, dump_path);
+                    dump_f32(device, x_grad.ptr(), k, dump_path, true);
+                }
+                std::printf("{\"config\": \"c3\", \"stack\": \"HIP<Lazy<Base>>\", \"calls\": \"apply_fn(tanh) and add_unary_grad recorded once; "
+                            "per step: run() (one kernel: x is loaded once, 20 B/element moved)\", \"elements\": %zu, \"warmup\": %d, %s, "
+                            "\"kernel_nodes\": %zu, \"graph_builds\": %llu}\n",
+                            n, warmup, timing_json(t, bytes).c_str(), device.graph_kernel_nodes(),
+                            static_cast<unsigned long long>(device.graph_builds()));
+            } else {
+                std::fprintf(stderr, "unknown stack %s\n", stack.c_str());
+                return 2;
+            }
+        } else if (config == "c4") {
+            const size_t n = size_t(1) << (log2n ? log2n : 28);
+            if (input.empty()) {
+                std::fprintf(stderr, "c4 needs --input (x as f16 bits)\n");
+                return 2;
+            }
+            HIP<Base> device(0);
+            auto x = device.buffer(read_file<f16>(input, n));
+            auto chain = [](auto v) { return v.mul(0.5f).exp().mul(v).add(v.mul(v)); };
+            auto out = device.apply_fn(x, chain);
+            const Timing t = time_runs([&] { out = device.apply_fn(x, chain); }, [&] { device.sync(); }, warmup, steps, settle_ms);
+            if (dump_count) {
+                std::vector<f16> first(std::min(dump_count, n));
+                device.read_raw(first.data(), out.ptr(), first.size() * sizeof(f16));
+                write_file(dump_path, first.data(), first.size() * sizeof(f16));
+            }
+            std::printf("{\"config\": \"c4\", \"stack\": \"HIP<Base>\", \"calls\": \"per step: apply_fn(exp(x*0.5)*x + x*x), f16\", "
+                        "\"elements\": %zu, \"warmup\": %d, %s}\n",
+                        n, warmup, timing_json(t, 4.0 * static_cast<double>(n)).c_str());
         } else if (config == "c5") {
             const size_t nbuf = 1024, m = 4096;
             Dev device(0);
@@ -177,14 +354,17 @@ int main(int argc, char** argv) {
                 ys.push_back(device.apply_fn(u, [](auto x) { return x.abs().sqrt().mul(0.3f); }));
             }
             if (fuse) device.elementwise_fusing();
-            const Timing t = time_runs([&] { device.run(); }, warmup, steps, settle_ms);
-            if (dump_count) dump(device, ys[0].replace().ptr(), std::min(dump_count, m), dump_path.c_str());
-            const double gbs = 16.0 * static_cast<double>(nbuf * m) / (t.mean_us * 1e-6) / 1e9;
+            const auto first = Clock::now();
+            device.run();
+            device.sync();
+            const double first_run_ms = us_since(first) * 1e-3;
+            const Timing t = time_runs([&] { device.run(); }, [&] { device.sync(); }, warmup, steps, settle_ms);
+            if (dump_count) dump_f32(device, ys[0].replace().ptr(), std::min(dump_count, m), dump_path);
             std::printf("{\"config\": \"c5\", \"stack\": \"HIP<Graph<Lazy<Base>>>\", \"calls\": \"1024 x (apply_fn2, apply_fn2, apply_fn)%s, "
-                        "run()\", \"waits\": true, \"elements\": %zu, \"steps\": %d, \"warmup\": %d, \"us_per_run\": %.3f, "
-                        "\"median_us\": %.3f, \"min_us\": %.3f, \"GBps_on_16B\": %.2f, \"kernel_nodes\": %zu, \"graph_builds\": %llu}\n",
-                        fuse ? ", elementwise_fusing" : "", nbuf * m, steps, warmup, t.mean_us, t.median_us, t.min_us, gbs,
-                        device.graph_kernel_nodes(), static_cast<unsigned long long>(device.graph_builds()));
+                        "run()\", \"elements\": %zu, \"warmup\": %d, %s, \"first_run_ms\": %.2f, \"kernel_nodes\": %zu, "
+                        "\"graph_builds\": %llu}\n",
+                        fuse ? ", elementwise_fusing" : "", nbuf * m, warmup, timing_json(t, 16.0 * static_cast<double>(nbuf * m)).c_str(),
+                        first_run_ms, device.graph_kernel_nodes(), static_cast<unsigned long long>(device.graph_builds()));
         } else {
             std::fprintf(stderr, "unknown config %s\n", config.c_str());
             return 2;

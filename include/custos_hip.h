@@ -49,6 +49,7 @@ enum custos_hip_status {
     CUSTOS_HIP_ERR_COMPILE = 10020,          /* hiprtc rejected the generated kernel */
     CUSTOS_HIP_ERR_KIND_MISMATCH = 10030,    /* kernel launched through the wrong entry point */
     CUSTOS_HIP_ERR_ARITY_MISMATCH = 10031,
+    CUSTOS_HIP_ERR_NOT_PREPARED = 10032,     /* an entry point that may not load code was called before the code was loaded */
     CUSTOS_HIP_ERR_CAPTURE_STATE = 10040,    /* begin while capturing / end while not / op illegal in capture */
     CUSTOS_HIP_ERR_GRAPH_ORDER = 10041,      /* the ordering check of a built graph failed (custos_hip_set_graph_verify) */
     CUSTOS_HIP_ERR_BAD_OVERLAP = 10050,      /* output partially overlaps an input */
@@ -142,7 +143,9 @@ int32_t custos_hip_get_device_info(custos_hip_device *dev, custos_hip_device_inf
 /* Message of the last failed call on `dev`; with dev == NULL, of the last
  * failed call of this thread that had no device (create, emit). */
 const char *custos_hip_last_error(custos_hip_device *dev);
-/* Blocks until the compute stream is idle (Stream::sync, src/devices/cuda/api/cuda.rs). */
+/* Blocks until the compute stream is idle (Stream::sync, src/devices/cuda/api/cuda.rs).
+ * While the device records, nothing new reaches the stream: the wait is then for the work
+ * that was in flight when the recording began. */
 int32_t custos_hip_sync(custos_hip_device *dev);
 int32_t custos_hip_set_tuning(custos_hip_device *dev, const custos_hip_tuning *tuning);
 int32_t custos_hip_get_tuning(custos_hip_device *dev, custos_hip_tuning *tuning);
@@ -343,14 +346,18 @@ int32_t custos_hip_apply_fn_n(custos_hip_device *dev, custos_hip_kernel *kernel,
 int32_t custos_hip_add_unary_grad(custos_hip_device *dev, custos_hip_kernel *kernel, uint64_t lhs,
                                   uint64_t lhs_grad, uint64_t out_grad, size_t n);
 
-/* No counterpart in the reference.  For callers that cannot allocate device memory where they
- * launch: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+/* No counterpart in the reference.  For callers that cannot allocate where they launch: tight
+ * serving loops, harnesses that forbid hipMalloc, code that runs between the begin and the end
+ * of a stream capture on ANOTHER stream (this call launches on the library's own stream, cannot
+ * be recorded itself, and may wait for a staging slot).
  * What it does is what a recording of `n_sets` independent launches of `kernel` does when it is
  * built and replayed (custos_hip_capture_end merges them into one grid whose operand addresses
  * sit in a device table that the graph allocates): ONE grid over `n_sets` operand sets of `n`
  * elements each, but with the table in a static device array of the library (64 KiB per GPU,
- * held until the process ends) instead of an allocation.  This call never calls hipMalloc,
- * hipFree, or compiles or loads code: `kernel` runs exactly as custos_hip_expr_compile built it.
+ * held until the process ends) instead of an allocation.  This call never calls hipMalloc or
+ * hipFree, compiles or loads no code and allocates nothing on the host heap: the kernel's entry
+ * point for merged launches must have been loaded before, where allocation is allowed, with
+ * custos_hip_kernel_prepare_merged (else CUSTOS_HIP_ERR_NOT_PREPARED).
  * `operands`: `n_sets` rows of `operands_per_set` device addresses in the order of the
  * kernel's pointer parameters (apply kernel: the inputs, then the output; unary-gradient kernel:
  * lhs, lhs_grad, out_grad), every address 16-byte aligned.  A row may name its output as one of
@@ -361,16 +368,28 @@ int32_t custos_hip_add_unary_grad(custos_hip_device *dev, custos_hip_kernel *ker
  * while the device records (CUSTOS_HIP_ERR_CAPTURE_STATE).
  * All calls on one GPU share that GPU's table, which keeps the rows of the last call (nothing in
  * it has to start at zero: every row a launch reads is rewritten by its call).  Calls through one
- * device handle are ordered by its compute stream; calls through two handles on the same GPU that
- * overlap in time race on the table. */
+ * device handle are ordered by its compute stream; a call through another handle on the same GPU
+ * makes its stream wait for the launch of the table's last user before it rewrites the table
+ * (one event per GPU, made when the first handle on that GPU is created), and calls from several
+ * threads take turns. */
 int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device *dev, custos_hip_kernel *kernel,
                                          const uint64_t *operands, int32_t operands_per_set,
                                          size_t n_sets, size_t n);
+/* Compiles (or takes from the caches) and loads the entry point of `kernel` for merged launches
+ * of equal length.  A generated kernel has three entry points -- one launch; many launches of
+ * equal length in one grid; many launches of different lengths in one grid -- each a translation
+ * unit of its own that is built when it is first needed: custos_hip_expr_compile builds the
+ * first (the reference compiles one function per text too, src/devices/cuda/kernel_cache.rs:39-61),
+ * a graph build the ones its nodes use, this call the second.  No counterpart in the reference. */
+int32_t custos_hip_kernel_prepare_merged(custos_hip_device *dev, custos_hip_kernel *kernel);
 
 /* ---- lazy run: capture once, replay (src/devices/cuda/lazy.rs:10-72) ---- */
 
 /* LazySetup::lazy_setup: from here on launches/clears/copies are recorded, not run.
- * Allocation, reads and writes stay legal while recording and execute at once. */
+ * Allocation, reads and writes stay legal while recording and execute at once.
+ * Takes no wait: work launched before (a graph of the run before, say) may still be in
+ * flight; the first allocation, read, write or custos_hip_sync during the recording waits
+ * for it, and a replay of the recorded graph is ordered behind it on the compute stream. */
 int32_t custos_hip_capture_begin(custos_hip_device *dev);
 /* Ends recording and instantiates an executable graph (LazyCudaGraph::new).
  * The graph is built from the recorded work, not replayed launch by launch:
@@ -408,11 +427,25 @@ int32_t custos_hip_set_graph_batching(custos_hip_device *dev, int32_t enabled);
  * literal is part of the joined kernel's code or one of its launch parameters as it is for the
  * launch's own kernel, so expressions that keep arriving with new values share their joined
  * kernels as they share their own.  The
- * kernels are compiled when the graph is built, at most 16 new ones per graph (or `enabled` of them,
- * if that is more than 1); launches whose joined kernel is neither cached nor within that limit
- * replay as they were recorded.  No counterpart in the reference, whose captured
+ * kernels are compiled when the graph is built, within a time budget
+ * (custos_hip_set_graph_fusing_budget); launches whose joined kernel is neither cached nor
+ * compiled within it, or does not compile, replay as they were recorded
+ * (custos_hip_graph_unjoined).  No counterpart in the reference, whose captured
  * graphs replay launch by launch (src/devices/cuda/lazy.rs:31-49). */
 int32_t custos_hip_set_graph_fusing(custos_hip_device *dev, int32_t enabled);
+/* How long a graph build may spend compiling kernels of joined launches (default 1000 ms): a
+ * compilation starts only while less than that has been spent on them in this build, so 0 means
+ * that only kernels from the caches are used.  A compilation takes 0.2-0.5 s the first time a
+ * machine sees the kernel and about 0.03 s afterwards (the compiler library's own cache). */
+int32_t custos_hip_set_graph_fusing_budget(custos_hip_device *dev, uint32_t milliseconds);
+/* Recorded launches of `graph` that the build would have joined with others but left as they were
+ * recorded, because their joined kernel was not compiled within the budget or did not compile;
+ * `reason` (may be null) receives a text that lives as long as the graph: empty, the budget, or
+ * the compiler's message. */
+int32_t custos_hip_graph_unjoined(custos_hip_graph *graph, size_t *launches, const char **reason);
+/* hiprtc compilations so far (translation units: a kernel has up to three, see
+ * custos_hip_kernel_prepare_merged) and the time spent in them.  No counterpart in the reference. */
+int32_t custos_hip_compile_stats(custos_hip_device *dev, uint64_t *units, double *milliseconds);
 /* The entry point kernel node `node` (0 .. kernel_nodes-1, in replay order) of a built graph
  * launches, as a profiler lists it; the string lives as long as the graph.  No counterpart in
  * the reference. */
@@ -474,7 +507,11 @@ int32_t custos_hip_set_graph_verify(custos_hip_device *dev, int32_t enabled);
  * No counterpart in the reference. */
 int32_t custos_hip_graph_edge_count(custos_hip_graph *graph, size_t *edges);
 int32_t custos_hip_is_capturing(custos_hip_device *dev, int32_t *capturing);
-/* LazyCudaGraph::launch on the compute stream (no wait; call custos_hip_sync). */
+/* LazyCudaGraph::launch on the compute stream.  No wait: launches queue behind each other in
+ * call order, and custos_hip_read, custos_hip_write, custos_hip_sync, a free that returns memory
+ * to the driver, custos_hip_graph_destroy and custos_hip_device_destroy are ordered behind them or
+ * wait for them.  The reference waits after every launch (src/devices/cuda/lazy.rs:42-43); a
+ * caller who wants that calls custos_hip_sync. */
 int32_t custos_hip_graph_launch(custos_hip_device *dev, custos_hip_graph *graph);
 int32_t custos_hip_graph_node_count(custos_hip_graph *graph, size_t *kernel_nodes);
 /* Recorded pieces of work, kernel nodes in the instantiated graph, dependency levels. */

@@ -59,24 +59,137 @@ TEST_CASE(hip_lazy_run_replays_one_graph) {
     CHECK_VEC_EQ(extra.replace().read(), (std::vector<int32_t>{3, 5, 7, 9, 11, 13}));
 }
 
-// Runs that do not wait queue behind each other on the stream; a read still sees all of
-// them (the reference's run always waits: src/devices/cuda/lazy.rs:42-43)
-TEST_CASE(hip_runs_without_wait_queue_in_order) {
-    using D = HIP<Lazy<Base, int32_t>>;
-    D device;
-    const size_t n = (size_t(1) << 20) + 3;
-    auto acc = device.buffer(std::vector<int32_t>(n, 0));
-    auto one = device.buffer(std::vector<int32_t>(n, 1));
+// ---- a run returns once its graph is queued; whatever looks at the results next waits ----
+//
+// The reference's run waits for the stream (src/devices/cuda/lazy.rs:42-43).  The cases below
+// go through every way a program can look at device memory, or take it away, after a run, with
+// launches long enough (2^22 and more elements, several runs queued) that they are still in
+// flight when the next call is made; each is run with the deferred wait (the default) and with
+// the wait inside every run, and must see the same values.
+
+namespace {
+using LazyI32 = HIP<Lazy<Base, int32_t>>;
+constexpr size_t kInFlightLen = (size_t(1) << 22) + 3;
+
+// acc += step, recorded once
+void record_accumulate(LazyI32& device, Buffer<int32_t, LazyI32>& acc, Buffer<int32_t, LazyI32>& step) {
     auto add = [](auto a, auto b) { return a.add(b); };
-    device.add_op(std::tie(acc, one), [add](Buffer<int32_t, D>& a, Buffer<int32_t, D>& o, D& d) { d.apply_fn2_impl(a, o, a, add); });
-    CHECK(device.run_waits());
-    device.set_run_waits(false);
-    for (int i = 0; i < 25; i++) device.run();
-    CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(n, 25)));
-    device.set_run_waits(true);
-    device.run();
-    CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(n, 26)));
-    CHECK_EQ(device.graph_builds(), uint64_t(1));
+    device.add_op(std::tie(acc, step),
+                  [add](Buffer<int32_t, LazyI32>& a, Buffer<int32_t, LazyI32>& o, LazyI32& d) { d.apply_fn2_impl(a, o, a, add); });
+}
+}  // namespace
+
+TEST_CASE(hip_run_defers_its_wait_and_read_takes_it) {
+    for (bool waits : {false, true}) {
+        LazyI32 device;
+        CHECK(!device.run_waits());  // deferred by default
+        device.set_run_waits(waits);
+        auto acc = device.buffer(std::vector<int32_t>(kInFlightLen, 0));
+        auto one = device.buffer(std::vector<int32_t>(kInFlightLen, 1));
+        record_accumulate(device, acc, one);
+        for (int i = 0; i < 25; i++) device.run();
+        CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(kInFlightLen, 25)));
+        device.run();
+        device.sync();
+        CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(kInFlightLen, 26)));
+        CHECK_EQ(device.graph_builds(), uint64_t(1));
+    }
+}
+
+// A write into an operand lands behind the run that is still reading it: short writes go
+// through a staging slot and a copy kernel, long ones through the runtime's copy; both on the
+// compute stream.
+TEST_CASE(hip_write_after_a_run_lands_behind_it) {
+    for (bool waits : {false, true})
+        for (size_t n : {size_t(1000), kInFlightLen}) {
+            LazyI32 device;
+            device.set_run_waits(waits);
+            // a long launch in front, so that the short program is still queued when the write comes
+            auto big = device.buffer(std::vector<int32_t>(kInFlightLen, 0));
+            auto big_step = device.buffer(std::vector<int32_t>(kInFlightLen, 1));
+            auto acc = device.buffer(std::vector<int32_t>(n, 0));
+            auto step = device.buffer(std::vector<int32_t>(n, 3));
+            record_accumulate(device, big, big_step);
+            record_accumulate(device, acc, step);
+            for (int i = 0; i < 4; i++) device.run();
+            step.write(std::vector<int32_t>(n, 100));  // the four runs before must have added 3 each
+            for (int i = 0; i < 2; i++) device.run();
+            CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(n, 4 * 3 + 2 * 100)));
+            CHECK_VEC_EQ(big.read(), (std::vector<int32_t>(kInFlightLen, 6)));
+        }
+}
+
+// A buffer dropped while runs that use it are queued: its block goes to the pool, the next
+// buffer of that size gets the block, and everything that touches it is ordered behind the runs.
+TEST_CASE(hip_buffer_dropped_while_runs_are_queued) {
+    for (bool waits : {false, true}) {
+        LazyI32 device;
+        device.set_run_waits(waits);
+        auto acc = device.buffer(std::vector<int32_t>(kInFlightLen, 0));
+        uint64_t dropped_ptr = 0;
+        {
+            auto step = device.buffer(std::vector<int32_t>(kInFlightLen, 7));
+            dropped_ptr = step.ptr();
+            record_accumulate(device, acc, step);
+            for (int i = 0; i < 6; i++) device.run();
+        }
+        // the recorded operation names a buffer that is gone: the error is the run's own, thrown at
+        // once, and the runs queued before it are not disturbed
+        CHECK_THROWS_KIND(device.run(), DeviceError::InvalidLazyBuf);
+        auto fresh = device.buffer(std::vector<int32_t>(kInFlightLen, -1));  // takes the dropped block
+        CHECK_EQ(fresh.ptr(), dropped_ptr);
+        CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(kInFlightLen, 42)));
+        CHECK_VEC_EQ(fresh.read(), (std::vector<int32_t>(kInFlightLen, -1)));
+    }
+}
+
+// With a pool that keeps nothing, a dropped buffer goes back to the driver, which waits first.
+TEST_CASE(hip_buffer_freed_to_the_driver_while_runs_are_queued) {
+    LazyI32 device;
+    CHECK_EQ(custos_hip_set_pool_limit(device.handle(), 0), CUSTOS_HIP_OK);
+    auto acc = device.buffer(std::vector<int32_t>(kInFlightLen, 0));
+    {
+        auto step = device.buffer(std::vector<int32_t>(kInFlightLen, 5));
+        record_accumulate(device, acc, step);
+        for (int i = 0; i < 6; i++) device.run();
+    }
+    CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(kInFlightLen, 30)));
+}
+
+// The device dropped with runs in flight: its destructor waits before memory, graph and
+// streams go.
+TEST_CASE(hip_device_dropped_while_runs_are_queued) {
+    for (int round = 0; round < 3; round++) {
+        LazyI32 device;
+        auto acc = device.buffer(std::vector<int32_t>(kInFlightLen, 0));
+        auto one = device.buffer(std::vector<int32_t>(kInFlightLen, 1));
+        record_accumulate(device, acc, one);
+        for (int i = 0; i < 8; i++) device.run();
+    }
+    CHECK(true);
+}
+
+// A changed program is recorded again while the runs of the old one are queued: the new
+// recording allocates and the old graph is destroyed, both behind those runs; `exec_now`
+// launches directly on the same stream.
+TEST_CASE(hip_program_changed_while_runs_are_queued) {
+    for (bool waits : {false, true}) {
+        LazyI32 device;
+        device.set_run_waits(waits);
+        auto acc = device.buffer(std::vector<int32_t>(kInFlightLen, 0));
+        auto one = device.buffer(std::vector<int32_t>(kInFlightLen, 1));
+        record_accumulate(device, acc, one);
+        for (int i = 0; i < 5; i++) device.run();
+        auto twice = device.apply_fn(acc, [](auto x) { return x.mul(2); });  // lazily allocated output
+        device.run();  // records acc += 1; twice = acc * 2
+        CHECK_EQ(device.graph_builds(), uint64_t(2));
+        CHECK_VEC_EQ(twice.replace().read(), (std::vector<int32_t>(kInFlightLen, 12)));
+        for (int i = 0; i < 3; i++) device.run();
+        device.exec_now(0);  // drains the two operations: one more pass, eagerly
+        CHECK_EQ(device.ops_count(), size_t(0));
+        CHECK_VEC_EQ(acc.read(), (std::vector<int32_t>(kInFlightLen, 10)));
+        CHECK_VEC_EQ(twice.replace().read(), (std::vector<int32_t>(kInFlightLen, 20)));
+    }
 }
 
 // One device per thread (tests/threading/threads.rs:5-25; the reference's devices are not
@@ -420,6 +533,13 @@ TEST_CASE(hip_apply_fn_many_noalloc) {
     HIP<Base> device;
     custos_hip_device* dev = device.handle();
     custos_hip_kernel* k = device.compile(CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, "((a * b) + 0.5)", {"a", "b"});
+    {
+        // the entry point for merged launches is loaded where allocation is allowed, not by the call
+        auto a = device.new_buffer<float>(16), b = device.new_buffer<float>(16), o = device.new_buffer<float>(16);
+        const uint64_t row[3] = {a.ptr(), b.ptr(), o.ptr()};
+        CHECK_EQ(custos_hip_apply_fn_many_noalloc(dev, k, row, 3, 1, 16), static_cast<int32_t>(CUSTOS_HIP_ERR_NOT_PREPARED));
+        CHECK_EQ(custos_hip_kernel_prepare_merged(dev, k), 0);
+    }
     for (const auto& shape : {std::pair<size_t, size_t>{19, 3001}, std::pair<size_t, size_t>{4, 130}}) {
         const size_t sets = shape.first, n = shape.second;
         std::vector<Buffer<float, HIP<Base>>> as, bs, outs, singles;

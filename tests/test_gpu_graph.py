@@ -111,9 +111,7 @@ def test_capture_state_errors(hip):
     with pytest.raises(capi.CustosHipError) as e:
         hip.capture_begin()
     assert e.value.code == capi.ERR_CAPTURE_STATE
-    with pytest.raises(capi.CustosHipError) as e:
-        hip.sync()
-    assert e.value.code == capi.ERR_CAPTURE_STATE
+    hip.sync()                               # legal: waits for what was in flight when the recording began
     g = hip.capture_end()
     assert g.kernel_nodes == 0
     g.launch()                               # an empty graph replays fine
@@ -558,6 +556,51 @@ def test_lazy_run_sequence_of_an_unmodified_lazy_module(hip, oracle):
     finally:
         hip.capture_end().destroy()
     graph.destroy()
+
+
+def test_recording_begins_without_a_wait_and_immediate_work_takes_it(hip):
+    """The same sequence with the run's wait deferred: the graph is launched, the next recording begins
+    while it is still running, and what executes at once during a recording (a read, a write, an
+    allocation with its zero fill, a wait) is ordered behind it."""
+    n = (1 << 24) + 5
+    ones = np.ones(n, dtype=np.int32)
+    hip.capture_begin()
+    try:
+        step, acc = hip.buffer(ones, "i32"), hip.buffer(np.zeros(n, dtype=np.int32), "i32")
+        graph, runs = None, 0
+        def run(times):
+            nonlocal graph, runs
+            for _ in range(times):
+                hip.apply_fn2(acc, step, lambda p, q: p.add(q), out=acc)
+                new = hip.capture_end_reuse(graph)
+                assert graph is None or new is graph
+                graph = new
+                graph.launch()                       # no wait
+                hip.capture_begin()
+                runs += 1
+        run(6)
+        got = acc.read()                             # a read while recording waits for the six launches
+        assert (got == runs).all(), (got.min(), got.max(), runs)
+        run(6)
+        step.write(ones * 10)                        # so does a write: the launches before it added 1 each
+        run(2)
+        hip.sync()                                   # and a wait
+        got = acc.read()
+        assert (got == 12 + 20).all(), (got.min(), got.max())
+        # an allocation while recording: the block of a buffer freed with launches still reading it
+        # comes back from the pool and is zero-filled outside the compute stream's order
+        step.write(ones)
+        run(6)
+        freed = acc.ptr
+        acc.free()
+        again = hip.alloc(n, dtype="i32")
+        assert again.ptr == freed
+        got = again.read()
+        assert not got.any(), "the zero fill ran while a launch was still writing the block"
+    finally:
+        hip.capture_end().destroy()
+    if graph is not None:
+        graph.destroy()
 
 
 @pytest.mark.parametrize("n", [5000, 5001])
@@ -1058,7 +1101,8 @@ def test_changing_literals_do_not_compile_chain_after_chain(fresh_device):
         assert_bits_equal(q.read(), want_q, f"buffer {i}")
         assert_bits_equal(r.read(), np.sqrt(np.abs(want_q)) * rate, f"buffer {i}")
     g.destroy()
-    assert hip.cache_stats()[0] == before
+    # one unit: the joined kernel's entry point for merged launches, which nothing had asked for before
+    assert hip.cache_stats()[0] == before + 1
 
 
 def test_graph_names_its_kernels(hip):
@@ -1079,10 +1123,11 @@ def test_graph_names_its_kernels(hip):
     g.destroy()
 
 
-def test_a_graph_build_compiles_a_limited_number_of_joined_kernels(fresh_device):
-    """Four chains of four different shapes with a limit of two new kernels per graph: two are joined, the
-    other two replay as the launches they were recorded as; the next build finds the two kernels cached and
-    compiles the others."""
+def test_a_graph_build_compiles_joined_kernels_within_a_time_budget(fresh_device):
+    """Four chains of four different shapes.  With no time for new kernels nothing is joined and the graph
+    says so; with a budget that the first compilation uses up, one chain is joined and the others replay as
+    the launches they were recorded as; with time enough, the next build finds that kernel cached and
+    compiles the other three.  Results are the eager ones every time."""
     hip = fresh_device
     n = 3000
     xs = [synth.uniform_f32(500 + i, n, -2, 2) for i in range(4)]
@@ -1094,13 +1139,64 @@ def test_a_graph_build_compiles_a_limited_number_of_joined_kernels(fresh_device)
             hip.apply_fn(b[4 + i], fns[i], out=b[8 + i])
             hip.apply_fn(b[8 + i], fns[(i + 1) % 4], out=b[4 + i])
 
+    def build(bufs):
+        hip.capture_begin()
+        program(bufs)
+        return hip.capture_end()
+
     zeros = [np.zeros(n, dtype=np.float32) for _ in range(8)]
     for f in fns:                                     # the launches' own kernels exist before anything is counted
         hip.apply_fn(hip.buffer(xs[0]), f)
-    hip.set_graph_fusing(2)
-    before = hip.cache_stats()[0]
-    assert _both_ways(hip, xs + zeros, program) == (2 + 6, 4)
-    assert hip.cache_stats()[0] - before == 2
-    assert _both_ways(hip, xs + zeros, program) == (4, 8)
-    assert hip.cache_stats()[0] - before == 4
-    hip.set_graph_fusing(True)
+    before = hip.compile_stats()[0]
+    try:
+        hip.set_graph_fusing_budget(0)
+        assert _both_ways(hip, xs + zeros, program) == (12, 0)
+        g = build([hip.buffer(x) for x in xs + zeros])
+        launches, reason = g.unjoined()
+        assert launches == 12 and "budget" in reason and "0 ms" in reason
+        g.destroy()
+        assert hip.compile_stats()[0] == before
+        hip.set_graph_fusing_budget(1)                # the first compilation starts, and spends more than that
+        assert _both_ways(hip, xs + zeros, program) == (1 + 9, 2)
+        assert hip.compile_stats()[0] - before == 1
+        hip.set_graph_fusing_budget(0)                # a cached kernel needs no budget
+        g = build([hip.buffer(x) for x in xs + zeros])
+        assert g.unjoined()[0] == 9 and (g.kernel_nodes, g.fused_launches) == (1 + 9, 2)
+        g.destroy()
+        assert hip.compile_stats()[0] - before == 1
+        hip.set_graph_fusing_budget(60000)
+        assert _both_ways(hip, xs + zeros, program) == (4, 8)
+        assert hip.compile_stats()[0] - before == 4
+        g = build([hip.buffer(x) for x in xs + zeros])
+        assert g.unjoined() == (0, "")
+        g.destroy()
+    finally:
+        hip.set_graph_fusing_budget(1000)
+
+
+def test_a_joined_kernel_that_does_not_compile_is_reported(fresh_device, monkeypatch):
+    """A chain whose kernel the compiler rejects replays as the launches it was recorded as, and the graph
+    carries the compiler's message instead of losing it."""
+    hip = fresh_device
+    n = 2000
+    x = synth.uniform_f32(77, n, -2, 2)
+    f, g_ = (lambda v: v.mul(1.25)), (lambda v: v.add(0.5))
+    for fn in (f, g_):
+        hip.apply_fn(hip.buffer(x), fn)
+
+    def program(b):
+        hip.apply_fn(b[0], f, out=b[1])
+        hip.apply_fn(b[1], g_, out=b[2])
+
+    monkeypatch.setenv("CUSTOS_HIP_FAIL_COMPILE_OF", "custos_chain_")   # compilations of such kernels fail
+    try:
+        assert _both_ways(hip, [x, np.zeros(n, np.float32), np.zeros(n, np.float32)], program) == (2, 0)
+        hip.capture_begin()
+        program([hip.buffer(x), hip.alloc(n), hip.alloc(n)])
+        graph = hip.capture_end()
+        launches, reason = graph.unjoined()
+        assert launches == 2 and "hiprtc" in reason
+        graph.destroy()
+    finally:
+        monkeypatch.delenv("CUSTOS_HIP_FAIL_COMPILE_OF")
+    assert _both_ways(hip, [x, np.zeros(n, np.float32), np.zeros(n, np.float32)], program) == (1, 1)

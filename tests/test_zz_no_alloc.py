@@ -35,10 +35,15 @@ def _case(hip, oracle, n_sets, n, seed):
     expr = lambda a, b, c: a.mul(b).add(c.mul(0.5))
     src = expr(Resolve("a", 0), Resolve("b", 1), Resolve("c", 2)).to_cl_source("f32")
     kernel = hip.compile(capi.KIND_APPLY, "f32", src, ("a", "b", "c"))
+    hip.prepare_merged(kernel)                    # compiles and loads: where allocation is allowed
     host = [[synth.uniform_f32(seed + 3 * s + k, n, -2, 2) for k in range(3)] for s in range(n_sets)]
     rows = [[hip.buffer(v) for v in hs] + [hip.alloc(n)] for hs in host]
     rows_graph = [[r[0], r[1], r[2], hip.alloc(n)] for r in rows]
+    hip.sync()
+    pool_before, compiled_before = hip.pool_stats(), hip.compile_stats()[0]
     hip.apply_fn_many_noalloc(kernel, rows, n)
+    # nothing was allocated, taken from the pool or compiled on the way
+    assert hip.pool_stats() == pool_before and hip.compile_stats()[0] == compiled_before
     got = [r[3].read() for r in rows]
     _graph_result(hip, kernel, 3, rows_graph, n)
     for s in range(n_sets):
@@ -58,6 +63,7 @@ def test_unary_grad_and_literal_parameters(hip, oracle):
     n, n_sets = 2048 + 3, 9
     grad = lambda v: v.mul(2.0).add(1.0)
     kernel = hip.compile(capi.KIND_UNARY_GRAD, "f32", grad(Resolve("x")).to_cl_source("f32"), ("x",))
+    hip.prepare_merged(kernel)
     xs = [synth.uniform_f32(10 + s, n, -1, 1) for s in range(n_sets)]
     gs = [synth.uniform_f32(40 + s, n, -1, 1) for s in range(n_sets)]
     os_ = [synth.uniform_f32(70 + s, n, -1, 1) for s in range(n_sets)]
@@ -71,6 +77,7 @@ def test_unary_grad_and_literal_parameters(hip, oracle):
     try:
         f = lambda v: v.mul(1.25).sub(0.75)
         k2 = hip.compile(capi.KIND_APPLY, "f32", f(Resolve("x")).to_cl_source("f32"), ("x",))
+        hip.prepare_merged(k2)
         outs = [hip.alloc(n) for _ in range(n_sets)]
         hip.apply_fn_many_noalloc(k2, [[rows[s][0], outs[s]] for s in range(n_sets)], n)
         for s in range(n_sets):
@@ -80,6 +87,36 @@ def test_unary_grad_and_literal_parameters(hip, oracle):
         hip.set_literal_policy(capi.LITERALS_ADAPTIVE)
 
 
+def test_calls_through_two_handles_take_turns_on_the_table(hip, oracle):
+    """Two device handles on one GPU share the GPU's table but launch on streams of their own: a call
+    makes its stream wait for the launch of the table's last user before it rewrites the rows.  Long
+    grids, so that the other handle's launch is still running when the next call comes."""
+    import custos_amd
+    other = custos_amd.HIP(0)
+    try:
+        n, n_sets = (1 << 18) + 7, 24
+        f = lambda v: v.mul(3.0).sub(1.0)
+        g = lambda v: v.abs().sqrt()
+        handles = [(hip, f), (other, g)]
+        kernels, rows, hosts = [], [], []
+        for i, (dev, fn) in enumerate(handles):
+            k = dev.compile(capi.KIND_APPLY, "f32", fn(Resolve("x")).to_cl_source("f32"), ("x",))
+            dev.prepare_merged(k)
+            xs = [synth.uniform_f32(300 + 50 * i + s, n, -2, 2) for s in range(n_sets)]
+            kernels.append(k)
+            hosts.append(xs)
+            rows.append([[dev.buffer(x), dev.alloc(n)] for x in xs])
+        for round_ in range(6):                       # A, B, A, B ... without a wait in between
+            for i, (dev, _) in enumerate(handles):
+                dev.apply_fn_many_noalloc(kernels[i], rows[i], n)
+        for i, (dev, fn) in enumerate(handles):
+            for s in range(n_sets):
+                want = oracle.apply_fn(fn, hosts[i][s])
+                assert np.array_equal(rows[i][s][1].read().view(np.uint32), want.view(np.uint32)), f"handle {i}, set {s}"
+    finally:
+        other.close()
+
+
 def test_limits_and_operand_checks(hip):
     kernel = hip.compile(capi.KIND_APPLY, "f32", "(x * 2.0)", ("x",))
     a, b = hip.alloc(4096), hip.alloc(4096)
@@ -87,6 +124,12 @@ def test_limits_and_operand_checks(hip):
     def call(rows, per_set, n):
         flat = (C.c_uint64 * len(rows))(*rows)
         return lib.custos_hip_apply_fn_many_noalloc(h, kernel, flat, per_set, len(rows) // per_set, n)
+    # loading code allocates: the entry point for merged launches has to be there before the call
+    fresh = hip.compile(capi.KIND_APPLY, "f32", "(tan(x) - 0.4321)", ("x",))    # (an expression no other test uses)
+    flat = (C.c_uint64 * 2)(a.ptr, b.ptr)
+    assert lib.custos_hip_apply_fn_many_noalloc(h, fresh, flat, 2, 1, 16) == capi.ERR_NOT_PREPARED
+    assert "custos_hip_kernel_prepare_merged" in capi.last_error(h)
+    hip.prepare_merged(kernel)
     # beyond the static table: 8192 words / 2 addresses per set = 4096 sets
     assert call([a.ptr, b.ptr] * 4097, 2, 16) == capi.ERR_TOO_LARGE
     assert "static operand table" in capi.last_error(h)
