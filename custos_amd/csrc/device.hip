@@ -753,53 +753,61 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
                              std::to_string(kScratchWords * 8) + " bytes), got " + std::to_string(n_sets));
     // Operand checks on the host, before anything is launched: aligned, no partial overlap
     // inside a set (`out == in` exactly is fine), and no set writes what another set touches.
-    // The spans live in a buffer the handle reserved when it was created.
+    // The spans live in a buffer the handle reserved when it was created.  A serving loop calls
+    // with the same table again and again: the table that passed last is remembered by a hash
+    // of everything the checks depend on, and passes again without them.
     const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(kernel->spec.dtype);
-    const int written = kernel->spec.kind == Kind::UnaryGrad ? 1 : n_ptrs - 1;
-    using Span = custos_hip_device::OperandSpan;
-    std::vector<Span>& spans = dev->noalloc_spans;
-    spans.clear();
-    for (size_t s = 0; s < n_sets; s++) {
-        const uint64_t* row = operands + s * static_cast<size_t>(n_ptrs);
-        for (int i = 0; i < n_ptrs; i++) {
-            if (row[i] == 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null device pointer");
-            if (row[i] & 15)
-                return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "operands of a merged launch are 16-byte aligned");
-            if (i != written && row[i] != row[written] && row[i] < row[written] + bytes && row[written] < row[i] + bytes)
-                return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP, "the output range partially overlaps an input range");
-            spans.push_back({row[i], static_cast<uint32_t>(s), i == written});
-        }
+    uint64_t table_hash = 0x9e3779b97f4a7c15ull ^ reinterpret_cast<uint64_t>(owner) ^ (static_cast<uint64_t>(n) * 0xbf58476d1ce4e5b9ull) ^
+                          (static_cast<uint64_t>(n_sets) << 40);
+    for (size_t w = 0; w < n_sets * static_cast<size_t>(n_ptrs); w++) {
+        table_hash = (table_hash ^ operands[w]) * 0x94d049bb133111ebull;
+        table_hash ^= table_hash >> 29;
     }
-    // (sorted already when the caller lists its sets by address, as a pool of equal buffers does)
-    const auto by_begin = [](const Span& a, const Span& b) { return a.begin < b.begin; };
-    if (!std::is_sorted(spans.begin(), spans.end(), by_begin)) std::sort(spans.begin(), spans.end(), by_begin);
-    // sweep by start address: the furthest-reaching earlier span of any kind and the furthest
-    // written one, each with a runner-up from another set
-    struct Reach {
-        uint64_t end[2] = {0, 0};
-        uint32_t set[2] = {0xffffffffu, 0xffffffffu};
-        void add(uint64_t e, uint32_t s) {
-            if (s == set[0]) {
-                end[0] = std::max(end[0], e);
-            } else if (e > end[0]) {
-                end[1] = end[0], set[1] = set[0];
-                end[0] = e, set[0] = s;
-            } else if (e > end[1]) {
-                end[1] = e, set[1] = s;
+    if (table_hash != dev->noalloc_checked) {
+        const int written = kernel->spec.kind == Kind::UnaryGrad ? 1 : n_ptrs - 1;
+        using Span = custos_hip_device::OperandSpan;
+        std::vector<Span>& spans = dev->noalloc_spans;
+        spans.clear();
+        for (size_t s = 0; s < n_sets; s++) {
+            const uint64_t* row = operands + s * static_cast<size_t>(n_ptrs);
+            for (int i = 0; i < n_ptrs; i++) {
+                if (row[i] == 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null device pointer");
+                if (row[i] & 15)
+                    return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "operands of a merged launch are 16-byte aligned");
+                if (i != written && row[i] != row[written] && row[i] < row[written] + bytes && row[written] < row[i] + bytes)
+                    return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP, "the output range partially overlaps an input range");
+                spans.push_back({row[i], static_cast<uint32_t>(s), i == written});
             }
         }
-        uint64_t other_than(uint32_t s) const { return set[0] != s ? end[0] : end[1]; }
-    } any, writes;
-    for (const Span& sp : spans) {
-        if ((sp.write && any.other_than(sp.set) > sp.begin) || writes.other_than(sp.set) > sp.begin)
-            return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP, "an operand set writes memory that another operand set uses");
-        any.add(sp.begin + bytes, sp.set);
-        if (sp.write) writes.add(sp.begin + bytes, sp.set);
+        std::sort(spans.begin(), spans.end(), [](const Span& a, const Span& b) { return a.begin < b.begin; });
+        // sweep by start address: the furthest-reaching earlier span of any kind and the furthest
+        // written one, each with a runner-up from another set
+        struct Reach {
+            uint64_t end[2] = {0, 0};
+            uint32_t set[2] = {0xffffffffu, 0xffffffffu};
+            void add(uint64_t e, uint32_t s) {
+                if (s == set[0]) {
+                    end[0] = std::max(end[0], e);
+                } else if (e > end[0]) {
+                    end[1] = end[0], set[1] = set[0];
+                    end[0] = e, set[0] = s;
+                } else if (e > end[1]) {
+                    end[1] = e, set[1] = s;
+                }
+            }
+            uint64_t other_than(uint32_t s) const { return set[0] != s ? end[0] : end[1]; }
+        } any, writes;
+        for (const Span& sp : spans) {
+            if ((sp.write && any.other_than(sp.set) > sp.begin) || writes.other_than(sp.set) > sp.begin)
+                return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP, "an operand set writes memory that another operand set uses");
+            any.add(sp.begin + bytes, sp.set);
+            if (sp.write) writes.add(sp.begin + bytes, sp.set);
+        }
+        dev->noalloc_checked = table_hash;
     }
-    const Tuning& t = kernel->spec.tuning;
     const ResolvedShape shape = resolve_shape(dev, kernel, static_cast<unsigned long long>(n_sets) * n_ptrs * bytes);
     const unsigned long long count = n, n_vec = n / static_cast<unsigned long long>(kernel->spec.vec_elems);
-    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * shape.unroll;
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(shape.block) * shape.unroll;
     unsigned long long tiles_per_seg = std::max(1ull, (n_vec + tile_vecs - 1) / tile_vecs);
     if (tiles_per_seg * n_sets > (1ull << 31) - 1)
         return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
@@ -830,13 +838,13 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
     }
     rc = staging_slot_send(dev, table_dev, slot_dev, n_sets * row_words * 8);
     if (rc != CUSTOS_HIP_OK) return rc;
-    unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, false);
+    unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, false, shape.block);
     uint64_t table_arg = table_dev;
     unsigned long long count_arg = count, n_vec_arg = n_vec;
     void* args[] = {&table_arg, &count_arg, &n_vec_arg, &tiles_per_seg, &mode};
     dev->launches_since_wait = true;
     HIP_TRY(dev, hipModuleLaunchKernel(fn, static_cast<unsigned int>(tiles_per_seg * n_sets), 1, 1,
-                                       static_cast<unsigned int>(t.block_threads), 1, 1, 0, dev->stream, args, nullptr));
+                                       static_cast<unsigned int>(shape.block), 1, 1, 0, dev->stream, args, nullptr));
     HIP_TRY(dev, hipEventRecord(g_scratch_event[dev->idx], dev->stream));
     g_scratch_last_user[dev->idx] = dev;
     return CUSTOS_HIP_OK;

@@ -501,6 +501,7 @@ struct Planned {
     custos_hip_kernel* kern = nullptr;  // kernels: the kernel of the (first) member
     ResolvedShape shape;                // kernels: vectors per thread and cache policy that suit the bytes the
                                         // node touches; whether it walks its tiles against the previous such node
+    bool feeds_later = false;           // single launches: one of the next levels reads what it writes
 };
 
 // The entry point a planned kernel node is replayed through.
@@ -508,6 +509,7 @@ EntrySet entry_of(const Planned& p) {
     return p.members.size() == 1 ? EntrySet::Single : p.ragged ? EntrySet::Ragged : EntrySet::Batched;
 }
 
+// Tiles of one segment of a merged launch (merged launches keep the workgroup size the kernel was compiled for).
 unsigned long long tiles_of(const custos_hip_kernel* k, const RecNode& n, int unroll) {
     const unsigned long long tile_vecs = static_cast<unsigned long long>(k->spec.tuning.block_threads) * unroll;
     return std::max(1ull, (n.n_vec + tile_vecs - 1) / tile_vecs);
@@ -636,22 +638,35 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
         const RecNode& first = nodes[p.members[0]];
         if (first.type == RecNode::Kernel) {
             // the launch shape follows the bytes the (merged) launch touches and the launches around it
-            unsigned long long footprint = 0;
-            for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
-            CacheHint hint = CacheHint::Unknown;
-            unsigned long long working_set = 0;
-            if (footprint >= kHintFromBytes) {
-                hint = hint_for(nodes, p, *history, later_reads);
-                dev->hinted[static_cast<int>(hint)]++;
-            }
-            if (footprint > kTrafficBeyondBytes) {
-                std::vector<Access> all;
-                for (size_t i : p.members) all.insert(all.end(), nodes[i].acc.begin(), nodes[i].acc.end());
-                working_set = history->working_set_with(all);
-            }
             p.kern = first.k;
-            p.shape = resolve_shape(dev, first.k, footprint, hint, working_set);
-            dev->last_shape[0] = p.shape.unroll, dev->last_shape[1] = p.shape.nontemporal, dev->last_shape[2] = p.shape.alternate;
+            if (p.members.size() == 1) {
+                // one launch: decided as for a launch issued directly, with what the graph knows on top
+                // (whether one of the next levels reads what it writes)
+                bool feeds_later = false;
+                for (const Access& a : first.acc)
+                    for (const std::vector<Access>* level : later_reads)
+                        for (const Access& r : *level) feeds_later = feeds_later || (a.write && r.begin < a.end && a.begin < r.end);
+                p.feeds_later = feeds_later;
+                RecentTraffic before = *history;  // (the level's traffic joins the history below, once)
+                p.shape = shape_of_launch(dev, first.k, first.acc, &before, feeds_later);
+            } else {
+                unsigned long long footprint = 0;
+                for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);
+                CacheHint hint = CacheHint::Unknown;
+                unsigned long long working_set = 0;
+                if (footprint >= kHintFromBytes) {
+                    hint = hint_for(nodes, p, *history, later_reads);
+                    dev->hinted[static_cast<int>(hint)]++;
+                }
+                if (footprint > kTrafficBeyondBytes) {
+                    std::vector<Access> all;
+                    for (size_t i : p.members) all.insert(all.end(), nodes[i].acc.begin(), nodes[i].acc.end());
+                    working_set = history->working_set_with(all);
+                }
+                p.shape = resolve_shape(dev, first.k, footprint, hint, working_set);
+                dev->last_shape[0] = p.shape.unroll, dev->last_shape[1] = p.shape.nontemporal, dev->last_shape[2] = p.shape.alternate;
+                dev->last_shape[3] = p.shape.block;
+            }
         }
         if (p.members.size() > 1) append_tables(nodes, &p, host_table);
     }
@@ -690,8 +705,7 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
         ln.grid = dim3(fill_grid(dev, first.n_vec));
         ln.block = dim3(fill_block());
     } else {
-        const Tuning& t = p.kern->spec.tuning;
-        ln.block = dim3(static_cast<unsigned int>(t.block_threads));
+        ln.block = dim3(static_cast<unsigned int>(p.shape.block));
         // (compiled by now: build_graph asked for the entry point of every planned node)
         hipFunction_t fn = nullptr;
         int32_t rc = entry_point(dev, p.kern, entry_of(p), &fn);
@@ -703,7 +717,16 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
             ln.args.push_back(value(&a0, 8));
             ln.args.push_back(value(&a1, 8));
             ln.args.push_back(value(&a2, 8));
-            ln.grid = dim3(launch_grid(dev, p.kern, first.n, first.n_vec, p.shape.unroll));
+            ln.grid = dim3(launch_grid(dev, p.kern, first.n, first.n_vec, p.shape));
+            // what a replay as plain launches needs to choose the shape again (replay_graph)
+            unsigned long long touched = 0;
+            for (const Access& a : first.acc) touched += a.end - a.begin;
+            if (touched > kTrafficBeyondBytes && p.kern->spec.auto_unroll) {
+                ln.kern = p.kern;
+                ln.n = first.n, ln.head = first.head, ln.n_vec = first.n_vec;
+                ln.acc = first.acc;
+                ln.feeds_later = p.feeds_later;
+            }
         } else if (p.ragged) {
             if (p.blocks > (1ull << 31) - 1)
                 return set_error(dev, CUSTOS_HIP_ERR_TOO_LARGE, "a merged launch would need more than 2^31 workgroups");
@@ -727,9 +750,10 @@ int32_t lower_node(custos_hip_device* dev, const std::vector<RecNode>& nodes, co
         if (first.k->spec.consts.n_params > 0 && p.members.size() == 1) ln.args.push_back(literal_values(first));
         const unsigned long long mode = p.members.size() == 1
                                             ? single_launch_mode(p.kern, first.n, first.head, first.n_vec, p.shape, rev != 0)
-                                            : launch_mode(p.shape.unroll, p.shape.nontemporal, rev != 0);
+                                            : launch_mode(p.shape.unroll, p.shape.nontemporal, rev != 0, p.shape.block);
         ln.args.push_back(value(&mode, 8));
-        if (p.shape.alternate) ln.rev_arg = static_cast<int>(ln.args.size()) - 1;
+        ln.mode_arg = static_cast<int>(ln.args.size()) - 1;
+        if (p.shape.alternate) ln.rev_arg = ln.mode_arg;
     }
     *out = std::move(ln);
     return CUSTOS_HIP_OK;
@@ -1122,7 +1146,19 @@ int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
                                         hipMemcpyDeviceToDevice, dev->stream));
             continue;
         }
-        if (ln.rev_arg >= 0 && g->flip_each_replay) ln.args[ln.rev_arg][0] ^= 1;
+        if (ln.kern) {
+            // A large launch of a short recording is a plain launch like any other: its shape follows
+            // what ran before it on this device (the rest of the recording, the replay before, whatever
+            // the caller launched in between), as for a launch issued directly.
+            const ResolvedShape shape = shape_of_launch(dev, ln.kern, ln.acc, &dev->recent, ln.feeds_later);
+            const unsigned long long mode =
+                single_launch_mode(ln.kern, ln.n, ln.head, ln.n_vec, shape, shape.alternate && (dev->launch_parity ^= 1));
+            std::memcpy(ln.args[static_cast<size_t>(ln.mode_arg)].data(), &mode, 8);
+            ln.grid = dim3(launch_grid(dev, ln.kern, ln.n, ln.n_vec, shape));
+            ln.block = dim3(static_cast<unsigned int>(shape.block));
+        } else if (ln.rev_arg >= 0 && g->flip_each_replay) {
+            ln.args[ln.rev_arg][0] ^= 1;
+        }
         std::vector<void*> argv(ln.args.size());
         for (size_t i = 0; i < ln.args.size(); i++) argv[i] = ln.args[i].data();
         void** args = argv.data();

@@ -346,13 +346,16 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 }
 
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
-                            CacheHint hint, unsigned long long working_set_bytes) {
+                            CacheHint hint, unsigned long long working_set_bytes, bool revisits) {
     const int n_operands = kernel_pointers(k->spec);
-    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint, working_set_bytes);
+    const int n_written = k->spec.kind == Kind::Chain ? k->spec.n_outs : 1;
+    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint, working_set_bytes, revisits, n_written);
     ResolvedShape r;
     const int direction = dev->tuning.direction;
     r.alternate = direction == 2 || (direction == 0 && shape.alternate);
+    // a kernel whose shape the caller left open runs as the launch says; a pinned one as it was compiled
     r.unroll = k->spec.auto_unroll ? shape.unroll : k->spec.tuning.unroll;
+    r.block = k->spec.auto_unroll && shape.block > 0 ? std::min(shape.block, k->spec.tuning.block_threads) : k->spec.tuning.block_threads;
     r.nontemporal = dev->tuning.nontemporal >= 0
                         ? dev->tuning.nontemporal & (3 | kStoresWriteThrough)
                         : shape.nontemporal;

@@ -64,17 +64,41 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // forward + backward over 2^26 elements its temporal stores push out what the
 // backward kernel keeps: 7090 on 24 bytes per element with N for the forward
 // kernel, 6200 with W.
+//
+// Two refinements, both about launches whose traffic the memory-side cache cannot help:
+//
+// A launch that touches nothing the launch before it wrote (an eager chain's first launch over
+// a fresh input, a loop whose every call gets another output block, anything that streams through
+// more memory than the caches hold) runs as one-wavefront workgroups with one vector per thread
+// once it touches more than 32 MiB.  Distinct (x, out) pairs over 2 GiB in turn, 1R+1W, GB/s with
+// 128 x 2 / 64 x 1: 32 MiB launches 4629 / 4795, 64 MiB 5407 / 5720, 128 MiB 5977 / 6283, 256 MiB
+// 6350 / 6625, 1 GiB 6449 / 6759; every kernel tried (copy, sin, tanh, exp, the f16 chain) goes
+// from 6350-6420 to 6740-6800 that way.  The same launch repeated over the same buffers, which
+// starts on what the cache still holds, loses 2-13 % with that shape and keeps 128 x 2.
+//
+// A launch that writes through at least two pointers more than it reads through (a joined chain
+// that still stores its intermediates) takes temporal loads and non-temporal stores written
+// through at once: what the cache keeps for the launch that comes back is then the input, which
+// that launch reads, instead of outputs, which it only overwrites.  1R+3W over 2^28 f32: 5634 ->
+// 6161-6310; 1R+5W 5436 -> 5885; over 2^26: 6749 -> 7230, 6141 -> 7196.  (With two inputs it is
+// the other way round: 2R+2W over 2^26 7150 / 6362; and below 128 MiB touched the usual policy is
+// ahead: 1R+3W over 64 MiB 8204 / 7779, 1R+5W over 96 MiB 7868 / 6714.)
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint,
-                            unsigned long long working_set_bytes) {
+                            unsigned long long working_set_bytes, bool revisits, int n_written) {
     constexpr unsigned long long MiB = 1ull << 20;
-    // non-temporal loads with temporal stores that are written through at once / both non-temporal
-    constexpr int kLoads = 1 | kStoresWriteThrough, kBoth = 3;
+    // non-temporal loads with temporal stores that are written through at once / both non-temporal /
+    // temporal loads with non-temporal stores that are written through at once
+    constexpr int kLoads = 1 | kStoresWriteThrough, kBoth = 3, kStores = 2 | kStoresWriteThrough;
     const unsigned long long working_set = std::max(footprint_bytes, working_set_bytes);
-    if (working_set <= kL2WorkingSet) return {2, 0, false};
-    if (footprint_bytes <= 256 * MiB) return {2, kLoads, false};
-    if (n_operands < 3 && footprint_bytes < 768 * MiB && hint != CacheHint::Streams && working_set > footprint_bytes)
-        return {2, kBoth, true};
-    return {2, kLoads, true};
+    if (working_set <= kL2WorkingSet) return {2, 0, false, 0};
+    LaunchShape shape{2, kLoads, footprint_bytes > 256 * MiB, 0};
+    if (n_written >= n_operands - n_written + 2 && footprint_bytes >= 128 * MiB)
+        shape.nontemporal = kStores;
+    else if (footprint_bytes > 256 * MiB && n_operands < 3 && footprint_bytes < 768 * MiB && hint != CacheHint::Streams &&
+             working_set > footprint_bytes)
+        shape.nontemporal = kBoth;
+    if (!revisits && footprint_bytes > kL2WorkingSet) shape.unroll = 1, shape.block = 64;
+    return shape;
 }
 
 std::vector<std::string> hiprtc_options(const std::string& arch) {
@@ -377,7 +401,7 @@ struct KernelText {
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
         for (int i = 0; i < n_in; i++) {
             const std::string id = std::to_string(i);
-            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), mode & 2);\n";
+            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BT * 16u), mode & 2);\n";
         }
         s += "    }\n";
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
@@ -388,25 +412,41 @@ struct KernelText {
         for (int j = 0; j < k.n_outs; j++) s += "            r" + std::to_string(j) + "[k] = o[" + std::to_string(j) + "];\n";
         s += "        }\n";
         for (int j = 0; j < k.n_outs; j++)
-            s += "        custos_st(rso" + std::to_string(j) + ", lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), r" + std::to_string(j) + ", mode);\n";
+            s += "        custos_st(rso" + std::to_string(j) + ", lane + (unsigned int)u * (CUSTOS_BT * 16u), r" + std::to_string(j) + ", mode);\n";
         s += "    }\n}\n";
         return s;
     }
 
-    // `custos_tile<U>(args)`: the kernel's one tile function (U vectors per thread: the caller's
-    // choice, or 2 -- what every automatic launch shape takes).
-    std::string tile_call(const std::string& indent, const std::string& args) const {
-        return indent + "custos_tile" + std::to_string(k.tuning.unroll) + "(" + args + ");\n";
+    // The numbers of vectors per thread this kernel has a tile function for: the caller's
+    // choice, or the two shapes the library picks from per launch (2 with workgroups of
+    // CUSTOS_BLOCK threads; 1 with one-wavefront workgroups, for launches that stream from and
+    // to memory without finding anything in the caches).
+    std::vector<int> unrolls() const {
+        if (k.auto_unroll) return {2, 1};
+        return {k.tuning.unroll};
     }
 
-    // Tiles of a range of `n_vec` vectors (a constant divisor: no division routine).
+    // `custos_tile<U>(args)` for the launch's number of vectors per thread `U`.
+    std::string tile_call(const std::string& indent, const std::string& args) const {
+        const std::vector<int> us = unrolls();
+        if (us.size() == 1) return indent + "custos_tile" + std::to_string(us[0]) + "(" + args + ");\n";
+        return indent + "if (U == 2) custos_tile2(" + args + ");\n" + indent + "else custos_tile1(" + args + ");\n";
+    }
+
+    // Tiles of a range of `n_vec` vectors, without a division by a run-time value (which would
+    // cost every wavefront a 64-bit division routine): a constant divisor, or, where the launch
+    // names its shape, a shift (64 << b threads times 1 or 2 vectors).
     std::string n_tiles_expr() const {
+        if (k.auto_unroll) return "((n_vec + tile_vecs - 1) >> (6 + ((mode >> 13) & 3) + (U >> 1)))";
         const std::string tv = "((u64)CUSTOS_BLOCK * " + std::to_string(k.tuning.unroll) + ")";
         return "(n_vec + " + tv + " - 1) / " + tv;
     }
 
-    // `const u64 U = ...;`: vectors per thread
-    std::string unroll_of_mode() const { return "    const u64 U = " + std::to_string(k.tuning.unroll) + ";\n"; }
+    // `const u64 U = ...;`: vectors per thread of this launch, from the mode word
+    std::string unroll_of_mode() const {
+        if (!k.auto_unroll) return "    const u64 U = " + std::to_string(k.tuning.unroll) + ";\n";
+        return "    const u64 U = (mode >> 8) & 15;\n";
+    }
 
     // One tile of `unroll` vectors per thread, starting at vector `first` of the operands (the
     // same for the whole workgroup): every lane loads all its vectors, then computes and stores.
@@ -444,13 +484,13 @@ struct KernelText {
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
         for (int i = 0; i < n_ops; i++) {
             const std::string id = std::to_string(i);
-            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), mode & 2);\n";
+            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BT * 16u), mode & 2);\n";
         }
         s += "    }\n";
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
         s += "        vec_t r;\n#pragma unroll\n        for (int k = 0; k < CUSTOS_VEC; k++) r[k] = custos_elem(" +
              list("a", "[u][k]") + " CUSTOS_KC_ARG);\n";
-        s += "        custos_st(rso, lane + (unsigned int)u * (CUSTOS_BLOCK * 16u), r, mode);\n    }\n";
+        s += "        custos_st(rso, lane + (unsigned int)u * (CUSTOS_BT * 16u), r, mode);\n    }\n";
         s += "}\n";
         return s;
     }
@@ -465,7 +505,7 @@ struct KernelText {
         s += vec_ptrs;
         s += "    const u64 rev = mode & 1;\n";
         s += unroll_of_mode();
-        s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * U;\n";
+        s += "    const u64 tile_vecs = (u64)CUSTOS_BT * U;\n";
         s += "    const u64 n_tiles = mode >> 16;\n";
         s += "    for (u64 tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {\n";
         s += tile_call("        ", tile_args + out_views + "(rev ? n_tiles - 1 - tile : tile) * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
@@ -475,8 +515,8 @@ struct KernelText {
         // have none (bit 12 of the mode word): one scalar test instead of per-lane arithmetic.
         // (One loop over both, so that the expression is expanded once for them.)
         s += "    if (!(mode & 4096)) return;\n";
-        s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BLOCK + threadIdx.x;\n";
-        s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BLOCK;\n";
+        s += "    const u64 gid = (u64)blockIdx.x * CUSTOS_BT + threadIdx.x;\n";
+        s += "    const u64 n_threads = (u64)gridDim.x * CUSTOS_BT;\n";
         s += "    const u64 body_end = head + n_vec * CUSTOS_VEC;\n";
         s += "    const u64 n_edge = head + (n - body_end);\n";
         s += "    for (u64 e = gid; e < n_edge; e += n_threads) {\n";
@@ -532,9 +572,9 @@ struct KernelText {
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
-        s += tile_call("    ", tile_args + out_views + "tile * (u64)CUSTOS_BLOCK * U, n_vec, mode CUSTOS_KC_ARG");
+        s += tile_call("    ", tile_args + out_views + "tile * (u64)CUSTOS_BT * U, n_vec, mode CUSTOS_KC_ARG");
         s += "    if (tile == tiles_per_seg - 1)\n";
-        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) " + scalar_stmt("i") + "\n";
+        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BT) " + scalar_stmt("i") + "\n";
         s += "    (void)head;\n}\n";
         return s;
     }
@@ -554,14 +594,14 @@ struct KernelText {
         s += "    const u64 n = ptrs[" + std::to_string(n_ptrs) + "];\n";
         s += row_consts(n_ptrs + 1);
         s += "    const u64 n_vec = n / CUSTOS_VEC;\n";
-        s += "    const u64 tile_vecs = (u64)CUSTOS_BLOCK * U;\n";
+        s += "    const u64 tile_vecs = (u64)CUSTOS_BT * U;\n";
         s += "    const u64 n_tiles = n_vec == 0 ? 1 : " + n_tiles_expr() + ";\n";
         s += "    const u64 head = 0;\n";
         s += table_operands();
         s += vec_ptrs;
         s += tile_call("    ", tile_args + out_views + "tile * tile_vecs, n_vec, mode CUSTOS_KC_ARG");
         s += "    if (tile == n_tiles - 1)\n";
-        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BLOCK) " + scalar_stmt("i") + "\n";
+        s += "        for (u64 i = n_vec * CUSTOS_VEC + threadIdx.x; i < n; i += CUSTOS_BT) " + scalar_stmt("i") + "\n";
         s += "    (void)head;\n}\n";
         return s;
     }
@@ -596,7 +636,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds the vectors per thread as requested: 0 = chosen per launch)
     int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, 19 /* template version */};
+                       k.tuning.blocks_per_cu, 20 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -631,7 +671,11 @@ bool emit_kernel_source(KernelSpec* spec, ParseError* err, EntrySet which) {
 
     std::string s;
     s += "// generated by custos-hip: " + (k.kind == Kind::Chain ? k.chain_text : to_cl_source(k.expr, k.markers, &k.consts)) + "\n";
+    // CUSTOS_BLOCK: the most threads a workgroup of this kernel has.  CUSTOS_BT: the threads of the
+    // launch at hand -- a kernel whose shape the caller left open reads them from bits 13-14 of its
+    // mode word (64 << bits), like the vectors per thread from bits 8-11.
     s += "#define CUSTOS_BLOCK " + std::to_string(k.tuning.block_threads) + "\n";
+    s += k.auto_unroll ? "#define CUSTOS_BT (64u << ((mode >> 13) & 3))\n" : "#define CUSTOS_BT CUSTOS_BLOCK\n";
     s += "#define CUSTOS_VEC " + std::to_string(k.vec_elems) + "\n";
     s += prelude(k.dtype, k.vec_elems, k.consts.n_params);
     // Loads and stores of one 16-byte vector through a buffer descriptor, with the cache policy
@@ -663,7 +707,7 @@ static __device__ __forceinline__ void custos_st(const custos_rsrc rs, const uns
 
     const KernelText text(k);
     s += text.elem_fn();
-    s += text.tile_fn(k.tuning.unroll);
+    for (int unroll : text.unrolls()) s += text.tile_fn(unroll);
     s += which == EntrySet::Single ? text.single_entry() : which == EntrySet::Batched ? text.batched_entry() : text.ragged_entry();
 
     k.source[static_cast<int>(which)] = std::move(s);
@@ -727,7 +771,7 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
                         (stage.out >= 0 ? " -> out" + std::to_string(stage.out) : std::string()) + "; ";
     }
     int32_t tail[7] = {static_cast<int32_t>(Kind::Chain), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, n_ext, n_outs, 19 /* template version */};
+                       k.tuning.blocks_per_cu, n_ext, n_outs, 20 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     k.stages = std::move(stages);

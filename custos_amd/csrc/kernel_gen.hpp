@@ -30,7 +30,7 @@ struct Tuning {
     // knobs are chosen per launch from the bytes it touches (preferred_shape)
     // unless the caller fixes them.
     int block_threads = 128;
-    int unroll = 0;         // 16-byte vectors per thread and tile; 0: the library's choice (2)
+    int unroll = 0;         // 16-byte vectors per thread and tile; 0: chosen per launch (2, or 1 with one-wavefront workgroups)
     int blocks_per_cu = 0;  // <= 0: one tile per workgroup
     int nontemporal = -1;   // bit 0 loads, bit 1 stores, 64 stores written through at once; -1: chosen per
                             // launch.  Read from the device's tuning when a launch is issued or a graph built.
@@ -43,6 +43,7 @@ struct LaunchShape {
     int unroll;
     int nontemporal;
     bool alternate;  // walk the tiles in the direction opposite to the previous launch
+    int block = 0;   // threads per workgroup; 0: the most the kernel was compiled for
 };
 // What is known about a launch from the address ranges of the launches around it.  A launch
 // that reads what one of the last few launches wrote (or whose output one of the next few
@@ -58,15 +59,18 @@ constexpr unsigned long long kCacheWorkingSet = 256ull << 20;
 // `working_set_bytes`: distinct bytes touched by the launch and the last few launches before it
 // together (0 = not known: the launch's own bytes count).
 constexpr unsigned long long kL2WorkingSet = 32ull << 20;  // what the eight L2s hold together
+// `revisits`: the launch touches memory that the launch before it wrote (the same launch repeated,
+// a consumer of the last launch); `n_written`: how many of its operands it writes.
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint = CacheHint::Unknown,
-                            unsigned long long working_set_bytes = 0);
+                            unsigned long long working_set_bytes = 0, bool revisits = true, int n_written = 1);
 
 // The last argument of every generated entry point: how this launch runs the kernel.  Nothing
 // of it is compiled in, so one kernel per expression serves every launch size.
 //   bit 0      the tiles are walked from the last to the first
 //   bit 1, 2   non-temporal loads, non-temporal stores
 //   bit 7      stores are written through to device scope at once instead of lingering in an L2
-//   bits 8..11 vectors per thread (for the record: the kernel's one tile function has them compiled in)
+//   bits 8..11 vectors per thread (only read by kernels whose launch shape was left open)
+//   bits 13,14 threads per workgroup as 64 << bits (likewise)
 //   bit 12     (single-launch entry point) the range has scalar elements: a head before the first
 //              16-byte boundary or a tail after the last whole vector
 //   bits 16..  (single-launch entry point) the number of tiles of the vector range
@@ -74,10 +78,12 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
 // host knows them.
 // `nontemporal` as in Tuning: bit 0 loads, bit 1 stores, kStoresWriteThrough the write-through stores.
 constexpr int kStoresWriteThrough = 64;
-inline uint64_t launch_mode(int unroll, int nontemporal, bool rev, uint64_t n_tiles = 0, bool scalar_edges = true) {
+inline uint64_t launch_mode(int unroll, int nontemporal, bool rev, int block_threads, uint64_t n_tiles = 0,
+                            bool scalar_edges = true) {
+    const uint64_t log2_waves = block_threads >= 512 ? 3 : block_threads >= 256 ? 2 : block_threads >= 128 ? 1 : 0;
     return (rev ? 1u : 0u) | static_cast<uint64_t>(nontemporal & 3) << 1 |
            static_cast<uint64_t>((nontemporal & kStoresWriteThrough) ? 1 : 0) << 7 | static_cast<uint64_t>(unroll & 15) << 8 |
-           (scalar_edges ? 1u << 12 : 0u) | n_tiles << 16;
+           (scalar_edges ? 1u << 12 : 0u) | log2_waves << 13 | n_tiles << 16;
 }
 
 // Fills unset (zero) fields with the defaults and clamps to legal values
@@ -124,7 +130,9 @@ struct KernelSpec {
     int n_ext = 0, n_outs = 0;       // Chain: input and output pointers (inputs first)
     std::string chain_text;          // Chain: the stages spelt out, literal values included
     Tuning tuning;             // as compiled: workgroup size, grid kind, most vectors per thread
-    bool auto_unroll = false;  // the caller left the vectors per thread open (the kernel takes 2)
+    bool auto_unroll = false;  // the caller left the launch shape open: the kernel holds the tile functions for
+                               // 2 and for 1 vectors per thread, and every launch names its vectors per thread
+                               // and its workgroup size (64 threads, or `tuning.block_threads`) in its mode word
     ConstPlan consts;          // literals that are launch parameters, and this text's values for them
     int n_literals = 0;        // literals in the expression, parameters or not
     std::vector<uint64_t> code_literals;  // values of the literals that stay in the code, in node order

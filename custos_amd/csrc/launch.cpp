@@ -45,6 +45,16 @@ bool RecentTraffic::wrote_any_of(const std::vector<Access>& reads) const {
     return false;
 }
 
+bool RecentTraffic::last_wrote_any_of(const std::vector<Access>& ranges) const {
+    if (launches_.empty()) return false;
+    for (const Access& w : launches_.back()) {
+        if (!w.write) continue;
+        for (const Access& r : ranges)
+            if (r.begin < w.end && w.begin < r.end) return true;
+    }
+    return false;
+}
+
 unsigned long long RecentTraffic::working_set_with(const std::vector<Access>& all) const {
     std::vector<Access> touched = all;
     for (const std::vector<Access>& launch : launches_) touched.insert(touched.end(), launch.begin(), launch.end());
@@ -109,13 +119,14 @@ int32_t plan_launch(custos_hip_device* dev, const custos_hip_kernel* k, const st
 }  // namespace
 
 unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
-                         unsigned long long n_vec, int unroll) {
+                         unsigned long long n_vec, const ResolvedShape& shape) {
     const Tuning& t = k->spec.tuning;
-    const unsigned long long tile_vecs = static_cast<unsigned long long>(t.block_threads) * unroll;
+    const unsigned long long block = static_cast<unsigned long long>(shape.block);
+    const unsigned long long tile_vecs = block * shape.unroll;
     unsigned long long tiles = (n_vec + tile_vecs - 1) / tile_vecs;
     const unsigned long long scalar = n - n_vec * k->spec.vec_elems;
     const unsigned long long cus = static_cast<unsigned long long>(dev->props.multiProcessorCount);
-    const unsigned long long scalar_blocks = std::min((scalar + t.block_threads - 1) / t.block_threads, cus * 32);
+    const unsigned long long scalar_blocks = std::min((scalar + block - 1) / block, cus * 32);
     if (t.blocks_per_cu > 0) tiles = std::min(tiles, cus * t.blocks_per_cu);
     unsigned long long g = std::max(1ull, std::max(tiles, scalar_blocks));
     return static_cast<unsigned int>(std::min(g, 1ull << 22));
@@ -150,30 +161,12 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     rc = entry_point(dev, k, EntrySet::Single, &fn);
     if (rc != CUSTOS_HIP_OK) return rc;
     // the launch shape that suits the bytes this launch touches and what the launches just
-    // before it left in the memory-side cache
+    // before it left in the caches
     const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(k->spec.dtype);
-    const unsigned long long footprint = static_cast<unsigned long long>(ops.size()) * bytes;
-    CacheHint hint = CacheHint::Unknown;
-    unsigned long long working_set = 0;
-    if (footprint > kTrafficBeyondBytes) {
-        std::vector<Access> all, reads;
-        for (const Range& r : ops) {
-            all.push_back({r.ptr, r.ptr + bytes, r.written});
-            // (the gradient operand of a unary-gradient kernel is read and written)
-            if (!r.written || k->spec.kind == Kind::UnaryGrad) reads.push_back(all.back());
-        }
-        if (footprint >= kHintFromBytes) {
-            hint = dev->recent.classify(reads, all);
-            dev->hinted[static_cast<int>(hint)]++;
-        }
-        // what the launches before it leave to this one: the L2s to a small launch, the
-        // memory-side cache to a large one
-        working_set = dev->recent.working_set_with(all);
-        dev->recent.record(all);
-    }
-    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set);
-    dev->last_shape[0] = shape.unroll, dev->last_shape[1] = shape.nontemporal, dev->last_shape[2] = shape.alternate;
-    const unsigned int grid = launch_grid(dev, k, n, n_vec, shape.unroll);
+    std::vector<Access> acc;
+    for (const Range& r : ops) acc.push_back({r.ptr, r.ptr + bytes, r.written});
+    const ResolvedShape shape = shape_of_launch(dev, k, acc, &dev->recent, /*feeds_later=*/false);
+    const unsigned int grid = launch_grid(dev, k, n, n_vec, shape);
     unsigned long long mode = single_launch_mode(k, n, head, n_vec, shape, shape.alternate && (dev->launch_parity ^= 1));
     uint64_t ptrs[8];
     std::vector<void*> args;
@@ -188,9 +181,37 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
     if (k->spec.consts.n_params > 0) args.push_back(k->spec.consts.bytes.data());
     args.push_back(&mode);
     dev->launches_since_wait = true;
-    HIP_TRY(dev, hipModuleLaunchKernel(fn, grid, 1, 1, static_cast<unsigned int>(k->spec.tuning.block_threads),
-                                       1, 1, 0, dev->stream, args.data(), nullptr));
+    HIP_TRY(dev, hipModuleLaunchKernel(fn, grid, 1, 1, static_cast<unsigned int>(shape.block), 1, 1, 0, dev->stream, args.data(),
+                                       nullptr));
     return CUSTOS_HIP_OK;
+}
+
+ResolvedShape shape_of_launch(custos_hip_device* dev, const custos_hip_kernel* k, const std::vector<Access>& acc,
+                              RecentTraffic* history, bool feeds_later) {
+    unsigned long long footprint = 0;
+    for (const Access& a : acc) footprint += a.end - a.begin;
+    CacheHint hint = CacheHint::Unknown;
+    unsigned long long working_set = 0;
+    bool revisits = true;
+    if (footprint > kTrafficBeyondBytes) {
+        if (footprint >= kHintFromBytes) {
+            std::vector<Access> reads;
+            // (the gradient operand of a unary-gradient kernel is read and written)
+            for (const Access& a : acc)
+                if (!a.write || k->spec.kind == Kind::UnaryGrad) reads.push_back(a);
+            hint = history->classify(reads, acc, feeds_later);
+            dev->hinted[static_cast<int>(hint)]++;
+        }
+        // what the launches before it leave to this one: the L2s to a small launch, the
+        // memory-side cache to a large one
+        working_set = history->working_set_with(acc);
+        revisits = history->last_wrote_any_of(acc);
+        history->record(acc);
+    }
+    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set, revisits);
+    dev->last_shape[0] = shape.unroll, dev->last_shape[1] = shape.nontemporal, dev->last_shape[2] = shape.alternate;
+    dev->last_shape[3] = shape.block;
+    return shape;
 }
 
 }  // namespace custos_hip

@@ -36,6 +36,12 @@ struct custos_hip_kernel {
     custos_hip_kernel* code = nullptr;
 };
 
+// An address range an operand of a launch covers, and whether the launch writes it.
+struct Access {
+    uint64_t begin, end;
+    bool write;
+};
+
 // A graph node in launchable form: function, shape and a copy of the argument values.
 struct LoweredNode {
     bool is_copy = false;
@@ -47,6 +53,13 @@ struct LoweredNode {
     unsigned int shared_mem = 0;
     std::vector<std::vector<unsigned char>> args;
     int rev_arg = -1;  // index of the mode word (bit 0 = direction) of a node that alternates, else -1
+    int mode_arg = -1;  // index of the mode word of a generated kernel
+    // A single launch of more than kTrafficBeyondBytes, for a replay as plain launches, which chooses
+    // the launch shape like a launch issued directly (`kern` is null for every other node):
+    custos_hip_kernel* kern = nullptr;
+    unsigned long long n = 0, head = 0, n_vec = 0;
+    std::vector<Access> acc;
+    bool feeds_later = false;
 };
 
 struct custos_hip_graph {
@@ -76,10 +89,6 @@ struct custos_hip_graph {
 };
 
 // One recorded piece of work (while the device is recording, nothing is launched).
-struct Access {
-    uint64_t begin, end;
-    bool write;
-};
 struct RecNode {
     enum Type { Kernel, Fill, Copy, Source } type = Kernel;
     custos_hip_kernel* k = nullptr;
@@ -108,6 +117,8 @@ class RecentTraffic {
    public:
     // Whether one of the recorded launches wrote something in `reads`.
     bool wrote_any_of(const std::vector<Access>& reads) const;
+    // Whether the launch recorded last wrote something in `ranges`.
+    bool last_wrote_any_of(const std::vector<Access>& ranges) const;
     // Distinct bytes touched by the recorded launches and by `all` together.
     unsigned long long working_set_with(const std::vector<Access>& all) const;
     void record(const std::vector<Access>& all);
@@ -137,7 +148,7 @@ struct custos_hip_device {
     std::unordered_map<uint64_t, uint32_t> value_sets_seen;
     RecentTraffic recent;            // of the launches issued directly (not recorded)
     uint64_t hinted[4] = {0, 0, 0, 0};  // launches and graph nodes of at least kHintFromBytes by CacheHint
-    int32_t last_shape[3] = {0, 0, 0};  // vectors per thread, cache policy, alternating: of the generated kernel
+    int32_t last_shape[4] = {0, 0, 0, 0};  // vectors per thread, cache policy, alternating, workgroup size: of the generated kernel
                                         // launched or planned into a graph last (custos_hip_last_launch_shape)
     size_t direct_replay_max = 4;    // longest chain replayed as plain launches instead of a hipGraph
     bool graph_verify = false;       // built graphs are checked by brute force against the recorded conflicts
@@ -173,6 +184,7 @@ struct custos_hip_device {
         bool write;
     };
     std::vector<OperandSpan> noalloc_spans;
+    uint64_t noalloc_checked = 0;  // hash of the kernel, length and operand table that passed those checks last
     unsigned char* read_stage = nullptr;  // pinned host memory short reads (first slot) and writes are staged in
     uint64_t read_stage_dev = 0;          // its device address
     uint64_t waits_begun = 0, waits_done = 0;  // waits for the compute stream, numbered
@@ -258,9 +270,18 @@ struct ResolvedShape {
     int unroll = 2;
     int nontemporal = 0;
     bool alternate = false;
+    int block = 128;  // threads per workgroup of this launch
 };
+// `revisits`: the launch touches memory the launch before it wrote (see preferred_shape).
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
-                            CacheHint hint = CacheHint::Unknown, unsigned long long working_set_bytes = 0);
+                            CacheHint hint = CacheHint::Unknown, unsigned long long working_set_bytes = 0, bool revisits = true);
+// The shape of ONE launch of `k` over the operand ranges `acc`, from the launches before it
+// (`history`, which the launch then joins) and from whether a launch soon after it reads what it
+// writes (`feeds_later`); counts the hint in the device's statistics.  The same decision for a
+// launch issued directly, a node of a graph being built, and a node of a short recording that is
+// replayed as plain launches.
+ResolvedShape shape_of_launch(custos_hip_device* dev, const custos_hip_kernel* k, const std::vector<Access>& acc,
+                              RecentTraffic* history, bool feeds_later);
 
 // jit.cpp: the kernel handle for a chain of apply expressions (cached; compiled when an entry point is asked for).
 int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs,
@@ -269,9 +290,9 @@ int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage
 // elements) in the given shape.
 inline uint64_t single_launch_mode(const custos_hip_kernel* k, unsigned long long n, unsigned long long head,
                                    unsigned long long n_vec, const ResolvedShape& shape, bool rev) {
-    const unsigned long long tile_vecs = static_cast<unsigned long long>(k->spec.tuning.block_threads) * shape.unroll;
+    const unsigned long long tile_vecs = static_cast<unsigned long long>(shape.block) * shape.unroll;
     const bool edges = head > 0 || head + n_vec * static_cast<unsigned long long>(k->spec.vec_elems) < n;
-    return custos_hip::launch_mode(shape.unroll, shape.nontemporal, rev, (n_vec + tile_vecs - 1) / tile_vecs, edges);
+    return custos_hip::launch_mode(shape.unroll, shape.nontemporal, rev, shape.block, (n_vec + tile_vecs - 1) / tile_vecs, edges);
 }
 // The values of a recorded launch's literal parameters.
 inline const std::vector<unsigned char>& literal_values(const RecNode& n) {
@@ -281,9 +302,9 @@ inline const std::vector<unsigned char>& literal_values(const RecNode& n) {
 custos_hip_kernel* cached_chain_kernel(custos_hip_device* dev, const KernelSpec& spec);
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
-// Workgroups of a single launch of `k` over n_vec vectors and n elements with `unroll` vectors per thread.
+// Workgroups of a single launch of `k` over n_vec vectors and n elements in the given shape.
 unsigned int launch_grid(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long n,
-                         unsigned long long n_vec, int unroll);
+                         unsigned long long n_vec, const ResolvedShape& shape);
 
 // graph.cpp
 int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g);

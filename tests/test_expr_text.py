@@ -219,10 +219,12 @@ def test_tuning_is_part_of_the_key_and_source():
     t = capi.Tuning(256, 4, 0, -1)
     src, h1 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], t)
     assert "#define CUSTOS_BLOCK 256" in src and "custos_tile4(" in src and "custos_tile2(" not in src
-    # vectors per thread left open: the kernel takes two, what every automatic launch shape uses
+    # launch shape left open: the kernel holds the tile functions for two vectors per thread and for one,
+    # and every launch names its vectors per thread and its workgroup size in its mode word
     src2, h2 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"])
-    assert "#define CUSTOS_BLOCK 128" in src2 and "custos_tile2(" in src2 and "custos_tile1(" not in src2
-    assert "const u64 U = 2;" in src2
+    assert "#define CUSTOS_BLOCK 128" in src2 and "custos_tile2(" in src2 and "custos_tile1(" in src2
+    assert "const u64 U = (mode >> 8) & 15;" in src2 and "#define CUSTOS_BT (64u << ((mode >> 13) & 3))" in src2
+    assert "#define CUSTOS_BT CUSTOS_BLOCK" in src
     # the cache policy is never compiled in: it is an operand of the launch, so one kernel per
     # expression serves every launch size
     src4, h4 = capi.expr_emit(capi.KIND_APPLY, "f32", "x", ["x"], capi.Tuning(0, 0, 0, 3))
@@ -238,8 +240,9 @@ def test_one_entry_point_per_translation_unit():
     """What `custos_hip_expr_compile` compiles is ONE function, as the reference's cache does per text
     (src/devices/cuda/kernel_cache.rs:39-61): the entry points for merged launches are translation
     units of their own, compiled when a graph build or `custos_hip_kernel_prepare_merged` asks for
-    them.  An expression is expanded once per element of the tile (2 vectors x 4 elements) and once
-    for the scalar elements at the edges of a view -- nine times in the unit of the single launch."""
+    them.  An expression is expanded once per element of a tile (2 vectors x 4 elements, and 1 x 4 for
+    the one-wavefront shape) and once for the scalar elements at the edges of a view -- thirteen times
+    in the unit of the single launch, where the one unit of all three entry points held 41."""
     chain = fused_source([lambda v: v.sin(), lambda v: v.mul(2.0), lambda v: v.add(1.0), lambda v: v.max(0.0),
                           lambda v: v.sub(0.5)], "f32")
     text, _ = capi.expr_emit(capi.KIND_APPLY, "f32", chain, ["x"])
@@ -251,7 +254,7 @@ def test_one_entry_point_per_translation_unit():
         assert entries == [name + suffix]
         # the per-element function is called from the tile's element loop and from ONE loop over
         # the scalar elements (head and tail of a view together)
-        assert len(re.findall(r"custos_elem\(", unit)) == 3        # definition + tile + edges
+        assert len(re.findall(r"custos_elem\(", unit)) == 4        # definition + two tile functions + edges
         assert len(re.findall(r"custos_sin\(", unit)) == 2         # wrapper definition + the one use in the expression
     assert "for (u64 e = gid; e < n_edge; e += n_threads)" in units[0]
 

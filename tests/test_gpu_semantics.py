@@ -1114,7 +1114,9 @@ def test_temporal_accesses_while_the_working_set_fits_the_l2s(oracle):
 def test_mid_sized_launches_leave_the_cache_to_their_neighbours(oracle):
     """A two-pointer launch of 256 to 768 MiB keeps its stores in the memory-side cache while it has the
     cache to itself (the same launch again and again), and streams them past it once the launches before it
-    touched other memory as well (tanh forward between gradient launches over other arrays)."""
+    touched other memory as well (tanh forward between gradient launches over other arrays).  And a launch of
+    more than 32 MiB that touches nothing the launch before it wrote runs as one-wavefront workgroups with one
+    vector per thread; one that comes back to what was just written keeps two vectors per thread."""
     import custos_amd
     dev = custos_amd.HIP(0)
     try:
@@ -1122,15 +1124,17 @@ def test_mid_sized_launches_leave_the_cache_to_their_neighbours(oracle):
         n = 1 << 26                                   # 256 MiB per array
         x, y = dev.alloc(n), dev.alloc(n)
         fwd = lambda v: v.tanh()
-        dev.apply_fn(x, fwd, out=y)
-        assert dev.last_launch_shape() == (2, loads, True)
-        dev.apply_fn(x, fwd, out=y)                   # nothing else in between
+        dev.apply_fn(x, fwd, out=y)                   # nothing before it
+        assert dev.last_launch_shape() == (1, loads, True)
+        dev.apply_fn(x, fwd, out=y)                   # nothing else in between: it overwrites what was just written
         assert dev.last_launch_shape() == (2, loads, True)
         g, o = dev.alloc(n), dev.alloc(n)
         dev.add_unary_grad(x, g, o, lambda v: v.mul(2.0))
-        assert dev.last_launch_shape() == (2, loads, True)      # three pointers: always loads only
-        dev.apply_fn(x, fwd, out=y)                   # g and o were touched since
-        assert dev.last_launch_shape() == (2, both, True)
+        assert dev.last_launch_shape() == (1, loads, True)      # three pointers: always loads only; y is not among them
+        dev.apply_fn(x, fwd, out=y)                   # g and o were touched since, and g is what was written last
+        assert dev.last_launch_shape() == (1, both, True)
+        dev.apply_fn(y, fwd, out=x)                   # reads what the launch before it wrote
+        assert dev.last_launch_shape()[0] == 2
         assert np.all(y.slice(n - 4096, n).read() == 0)
     finally:
         dev.close()
