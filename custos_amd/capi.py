@@ -29,6 +29,7 @@ DTYPES = {
     "bf16_pernode": (13, "uint16"),
 }
 
+EQ_EXACT, EQ_AS_CPU_EVAL = 0, 1
 ERR_INVALID_ARGUMENT = 10001
 ERR_ZERO_LENGTH_BUFFER = 10002
 ERR_INVALID_DEVICE_INDEX = 10003
@@ -132,6 +133,7 @@ PROTOTYPES = {
     "custos_hip_expr_emit_shared": (C.c_int32, [C.c_int32, C.c_int32, C.c_char_p, _STRS, C.c_int32, C.POINTER(Tuning),
                                                 C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint64)]),
     "custos_hip_set_literal_policy": (C.c_int32, [_P, C.c_int32]),
+    "custos_hip_set_eq_policy": (C.c_int32, [_P, C.c_int32]),
     "custos_hip_launch_hint_stats": (C.c_int32, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "custos_hip_expr_build_code_object": (C.c_int32, [C.c_int32, C.c_int32, C.c_char_p, _STRS, C.c_int32,
                                                       C.POINTER(Tuning), C.POINTER(C.c_size_t)]),

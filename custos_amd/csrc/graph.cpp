@@ -915,6 +915,57 @@ std::vector<std::vector<uint32_t>> level_waits(const std::vector<std::vector<Pla
     return waits;
 }
 
+// Issues one lowered node on `stream` (a replay as plain launches; the recording pass of
+// instantiate_chain).
+hipError_t issue_node(LoweredNode& ln, hipStream_t stream) {
+    if (ln.is_copy)
+        return hipMemcpyAsync(reinterpret_cast<void*>(ln.dst), reinterpret_cast<const void*>(ln.src), ln.bytes,
+                              hipMemcpyDeviceToDevice, stream);
+    void* argv[24];
+    std::vector<void*> more;
+    void** args = argv;
+    if (ln.args.size() > 24) {
+        more.resize(ln.args.size());
+        args = more.data();
+    }
+    for (size_t i = 0; i < ln.args.size(); i++) args[i] = ln.args[i].data();
+    if (ln.module_fn)
+        return hipModuleLaunchKernel(static_cast<hipFunction_t>(ln.func), ln.grid.x, ln.grid.y, ln.grid.z, ln.block.x, ln.block.y,
+                                     ln.block.z, ln.shared_mem, stream, args, nullptr);
+    return hipLaunchKernel(ln.func, ln.grid, ln.block, args, ln.shared_mem, stream);
+}
+
+// One chain as an instantiated hipGraph: the nodes are launched, in the chain's order, on a
+// stream of their own that is in capture mode, which is how the runtime takes kernels of
+// run-time compiled modules into a graph (hipModuleLaunchKernel with their hipFunction_t; the
+// `func` of hipGraphAddKernelNode's parameters is documented as a host function, and handing it
+// a hipFunction_t, which the runtime happens to accept, ended a traced run inside
+// hipGraphLaunch).  Relaxed mode: other threads with devices of their own keep allocating.
+int32_t instantiate_chain(custos_hip_device* dev, custos_hip_graph* g, std::vector<std::vector<LoweredNode>>& lowered) {
+    hipStream_t recording = nullptr;
+    HIP_TRY(dev, hipStreamCreateWithFlags(&recording, hipStreamNonBlocking));
+    hipError_t e = hipStreamBeginCapture(recording, hipStreamCaptureModeRelaxed);
+    size_t issued = 0;
+    for (auto& level : lowered)
+        for (LoweredNode& ln : level) {
+            if (e != hipSuccess) break;
+            e = issue_node(ln, recording);
+            issued++;
+        }
+    hipGraph_t captured = nullptr;
+    const hipError_t ended = hipStreamEndCapture(recording, &captured);  // (also after a failure: it closes the capture)
+    (void)hipStreamDestroy(recording);
+    if (e == hipSuccess) e = ended;
+    if (e != hipSuccess) {
+        if (captured) (void)hipGraphDestroy(captured);
+        return hip_fail(dev, e, "recording a chain of launches into a hipGraph");
+    }
+    g->graph = captured;
+    g->edges = issued ? issued - 1 : 0;
+    HIP_TRY(dev, hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
+    return CUSTOS_HIP_OK;
+}
+
 // The plan as an instantiated hipGraph.  With level joins the nodes of a level sit side by side
 // behind one empty node that waits for the level before (instead of |previous| x |level|
 // edges); with per-node edges (`waits`) every node follows exactly what it conflicts with.
@@ -1130,6 +1181,7 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
         if (!ordering_holds(nodes, plan, waits))
             return set_error(dev, CUSTOS_HIP_ERR_GRAPH_ORDER, "built graph does not order two conflicting pieces of recorded work");
     }
+    if (serial) return instantiate_chain(dev, g, lowered);
     return instantiate(dev, g, lowered, dev->graph_edges == CUSTOS_HIP_GRAPH_EDGES_LEVEL_JOINS ? nullptr : &waits);
 }
 
@@ -1141,11 +1193,6 @@ int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
         return CUSTOS_HIP_OK;
     }
     for (LoweredNode& ln : g->direct) {
-        if (ln.is_copy) {
-            HIP_TRY(dev, hipMemcpyAsync(reinterpret_cast<void*>(ln.dst), reinterpret_cast<const void*>(ln.src), ln.bytes,
-                                        hipMemcpyDeviceToDevice, dev->stream));
-            continue;
-        }
         if (ln.kern) {
             // A large launch of a short recording is a plain launch like any other: its shape follows
             // what ran before it on this device (the rest of the recording, the replay before, whatever
@@ -1159,14 +1206,7 @@ int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
         } else if (ln.rev_arg >= 0 && g->flip_each_replay) {
             ln.args[ln.rev_arg][0] ^= 1;
         }
-        std::vector<void*> argv(ln.args.size());
-        for (size_t i = 0; i < ln.args.size(); i++) argv[i] = ln.args[i].data();
-        void** args = argv.data();
-        if (ln.module_fn)
-            HIP_TRY(dev, hipModuleLaunchKernel(static_cast<hipFunction_t>(ln.func), ln.grid.x, ln.grid.y, ln.grid.z,
-                                               ln.block.x, ln.block.y, ln.block.z, ln.shared_mem, dev->stream, args, nullptr));
-        else
-            HIP_TRY(dev, hipLaunchKernel(ln.func, ln.grid, ln.block, args, ln.shared_mem, dev->stream));
+        HIP_TRY(dev, issue_node(ln, dev->stream));
     }
     return CUSTOS_HIP_OK;
 }

@@ -380,7 +380,8 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
     if (src && markers && n_markers >= 1 && n_markers <= 4) {
         const Tuning& t = dev->tuning;
         text_key = std::to_string(kind) + "," + std::to_string(dtype) + "," + std::to_string(t.block_threads) + "," +
-                   std::to_string(t.unroll) + "," + std::to_string(t.blocks_per_cu) + "," + std::to_string(t.nontemporal);
+                   std::to_string(t.unroll) + "," + std::to_string(t.blocks_per_cu) + "," + std::to_string(t.nontemporal) +
+                   (dev->eq_as_cpu_eval ? ",le" : "");
         for (int i = 0; i < n_markers; i++) text_key.append(1, '\x1f').append(markers[i] ? markers[i] : "");
         text_key.append(1, '\x1e').append(src);
         auto known = dev->by_text.find(text_key);
@@ -391,7 +392,9 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
         }
     }
     custos_hip_kernel* k = nullptr;
-    int32_t rc = compile_expr(dev, kind, dtype, src, markers, n_markers, dev->tuning, &k);
+    Tuning tuning = dev->tuning;
+    tuning.eq_as_leq = dev->eq_as_cpu_eval;
+    int32_t rc = compile_expr(dev, kind, dtype, src, markers, n_markers, tuning, &k);
     if (rc != CUSTOS_HIP_OK) return rc;
     *kernel = k;
     dev->by_text.emplace(std::move(text_key), k);
@@ -488,6 +491,14 @@ int32_t custos_hip_expr_emit_shared(int32_t kind, int32_t dtype, const char* src
     if (rc != CUSTOS_HIP_OK) return rc;
     if (hash) *hash = spec.hash;
     return copy_out_string(all_units(&spec), buf, cap, needed);
+}
+
+int32_t custos_hip_set_eq_policy(custos_hip_device* dev, int32_t policy) {
+    REQUIRE_DEV(dev);
+    if (policy != CUSTOS_HIP_EQ_EXACT && policy != CUSTOS_HIP_EQ_AS_CPU_EVAL)
+        return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown eq policy");
+    dev->eq_as_cpu_eval = policy == CUSTOS_HIP_EQ_AS_CPU_EVAL;
+    return CUSTOS_HIP_OK;
 }
 
 int32_t custos_hip_set_literal_policy(custos_hip_device* dev, int32_t policy) {

@@ -617,6 +617,9 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.dtype = dtype;
     k.tuning = tuning;
     if (!parse_expr(src, markers, &k.expr, err)) return false;
+    if (tuning.eq_as_leq)
+        for (Node& n : k.expr.nodes)
+            if (n.op == Op::Eq) n.op = Op::LEq;
     if (kind == Kind::UnaryGrad && k.expr.n_vars != 1) {
         err->code = CUSTOS_HIP_ERR_ARITY_MISMATCH;
         err->message = "a unary gradient expression takes exactly one marker";

@@ -35,6 +35,10 @@ struct Tuning {
     int nontemporal = -1;   // bit 0 loads, bit 1 stores, 64 stores written through at once; -1: chosen per
                             // launch.  Read from the device's tuning when a launch is issued or a graph built.
     int direction = 0;      // 1: tiles first to last; 2: every launch the other way round; 0: chosen per launch
+    // Not a shape, but it travels the same way: `eq` nodes are compiled as `<=`, which is what the
+    // reference's CPU device evaluates for them (src/two_way_ops/ops/cmps.rs:135), instead of `==`,
+    // which is what the reference's GPU kernels compute.
+    bool eq_as_leq = false;
 };
 
 // What suits a launch that touches `footprint_bytes` (all operands together)

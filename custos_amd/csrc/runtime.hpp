@@ -144,6 +144,7 @@ struct custos_hip_device {
     bool undrained_at_capture = false;  // work was (possibly) in flight on the compute stream when the recording
                                         // began and nothing has waited for it since (drain_before_immediate_work)
     int32_t literal_policy = 0;      // CUSTOS_HIP_LITERALS_*
+    bool eq_as_cpu_eval = false;     // custos_hip_set_eq_policy: `eq` compiled as `<=`
     // per shared-form key: how many distinct texts of that structure were compiled or looked up
     std::unordered_map<uint64_t, uint32_t> value_sets_seen;
     RecentTraffic recent;            // of the launches issued directly (not recorded)

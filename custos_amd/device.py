@@ -378,6 +378,11 @@ class HIP:
     def set_graph_batching(self, enabled: bool) -> None:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 
+    def set_eq_policy(self, policy: int) -> None:
+        """What `eq` nodes compiled from now on compute: capi.EQ_EXACT (`==`, the reference's GPU kernels) or
+        capi.EQ_AS_CPU_EVAL (`<=`, what the reference's CPU device evaluates)."""
+        self._check(self.lib.custos_hip_set_eq_policy(self.handle, int(policy)))
+
     def set_graph_fusing(self, enabled) -> None:
         """Whether a graph build joins recorded launches with the launches that read their output."""
         self._check(self.lib.custos_hip_set_graph_fusing(self.handle, int(bool(enabled))))

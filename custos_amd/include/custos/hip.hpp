@@ -257,6 +257,9 @@ class HIP : public Device<HIP<Mods>, Mods> {
     // How literal values reach kernels (CUSTOS_HIP_LITERALS_*): by default the first set of values of an
     // expression is compiled in, later sets are launch parameters of one shared kernel.
     void set_literal_policy(int32_t policy) { check(custos_hip_set_literal_policy(dev_, policy)); }
+    // What `eq` computes in kernels compiled from now on: `==` (CUSTOS_HIP_EQ_EXACT, the default, like the
+    // reference's GPU kernels) or `<=` (CUSTOS_HIP_EQ_AS_CPU_EVAL, what the reference's CPU device evaluates).
+    void set_eq_policy(int32_t policy) { check(custos_hip_set_eq_policy(dev_, policy)); }
     // (hiprtc compilations, cache hits) so far
     std::pair<uint64_t, uint64_t> cache_stats() const {
         uint64_t compiles = 0, hits = 0;

@@ -104,6 +104,7 @@ extern "C" {
                                  out: u64, n: usize) -> i32;
     pub fn custos_hip_apply_fn_many_noalloc(dev: *mut HipDeviceHandle, kernel: *mut HipKernel, operands: *const u64,
                                             operands_per_set: i32, n_sets: usize, n: usize) -> i32;
+    pub fn custos_hip_set_eq_policy(dev: *mut HipDeviceHandle, policy: i32) -> i32;
     pub fn custos_hip_kernel_prepare_merged(dev: *mut HipDeviceHandle, kernel: *mut HipKernel) -> i32;
     pub fn custos_hip_set_graph_fusing_budget(dev: *mut HipDeviceHandle, milliseconds: u32) -> i32;
     pub fn custos_hip_graph_unjoined(graph: *mut HipGraph, launches: *mut usize, reason: *mut *const c_char) -> i32;

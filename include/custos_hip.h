@@ -247,6 +247,13 @@ int32_t custos_hip_kernel_launched_as(custos_hip_device *dev, custos_hip_kernel 
 #define CUSTOS_HIP_LITERALS_IN_CODE 1       /* every distinct set of values is compiled (the reference's way) */
 #define CUSTOS_HIP_LITERALS_AS_PARAMETERS 2 /* always the shared form */
 int32_t custos_hip_set_literal_policy(custos_hip_device *dev, int32_t policy);
+/* What an `eq` node of expressions compiled from now on computes.  The reference disagrees with
+ * itself: its GPU kernels are the text "(a == b)" (src/two_way_ops/ops/cmps.rs:117-130), its CPU
+ * device evaluates `a <= b` (cmps.rs:135).  Default: `==`, like every GPU backend of the
+ * reference; AS_CPU_EVAL compiles `<=`, so that results equal CPU<Base>'s for `eq` as well. */
+#define CUSTOS_HIP_EQ_EXACT 0
+#define CUSTOS_HIP_EQ_AS_CPU_EVAL 1
+int32_t custos_hip_set_eq_policy(custos_hip_device *dev, int32_t policy);
 /* Number of hiprtc compilations / cache hits since the device was created. */
 int32_t custos_hip_cache_stats(custos_hip_device *dev, uint64_t *compiles, uint64_t *hits);
 

@@ -36,6 +36,36 @@ def test_binary_nodes_on_special_values(hip, oracle, name):
     assert_bits_equal(got, oracle.apply_fn(f, a, b), name)
 
 
+def test_eq_as_the_cpu_device_evaluates_it(oracle):
+    """The reference's CPU `Eval` of `eq` is `<=` (src/two_way_ops/ops/cmps.rs:135) while its GPU kernels are
+    the text `(a == b)`.  Kernels compute `==` by default; with CUSTOS_HIP_EQ_AS_CPU_EVAL they compute what
+    CPU<Base> computes, bit for bit against the oracle's restatement of that `Eval`, NaNs and zeros included;
+    the two forms are different kernels, and switching back brings `==` back."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        a, b = pairs()
+        ints_a = np.array([1, 2, 3, 4, 5, -7, 0], dtype=np.int32)
+        ints_b = np.array([1, 3, 2, 4, -5, -7, 1], dtype=np.int32)
+        eq = lambda p, q: p.eq(q)
+        clip_eq = lambda p, q: p.eq(q).mul(p).add(q)          # an eq node inside a larger expression
+        exact = dev.apply_fn2(dev.buffer(a), dev.buffer(b), eq).read()
+        assert_bits_equal(exact, oracle.apply_fn(eq, a, b), "== by default")
+        dev.set_eq_policy(capi.EQ_AS_CPU_EVAL)
+        for f in (eq, clip_eq):
+            got = dev.apply_fn2(dev.buffer(a), dev.buffer(b), f).read()
+            assert_bits_equal(got, oracle.apply_fn(f, a, b, eq_mode="eq_cpuref"), "eq as CPU<Base> evaluates it")
+        got = dev.apply_fn2(dev.buffer(ints_a, "i32"), dev.buffer(ints_b, "i32"), eq).read()
+        assert got.tolist() == [1, 1, 0, 1, 0, 1, 1]           # a <= b; eq(3, 3) = 1 is the value src/two_way_ops/mod.rs:108-111 holds
+        assert not np.array_equal(exact, dev.apply_fn2(dev.buffer(a), dev.buffer(b), eq).read())
+        dev.set_eq_policy(capi.EQ_EXACT)
+        assert_bits_equal(dev.apply_fn2(dev.buffer(a), dev.buffer(b), eq).read(), exact, "== again")
+        with pytest.raises(capi.CustosHipError):
+            dev.set_eq_policy(7)
+    finally:
+        dev.close()
+
+
 @pytest.mark.parametrize("name,f", [("neg", lambda v: v.neg()), ("abs", lambda v: v.abs()), ("identity", lambda v: v.identity()),
                                     ("sqrt", lambda v: v.sqrt()), ("relu_geq", lambda v: v.geq(0.).mul(v)),
                                     ("relu_max", lambda v: v.max(0.)), ("clip", lambda v: v.max(3.).min(5.))])
