@@ -280,6 +280,23 @@ class HIP : public Device<HIP<Mods>, Mods> {
     // Whether a lazy run joins recorded apply launches with the apply launches that read their
     // output into one kernel (default: yes; every buffer still receives the same values).
     void set_graph_fusing(bool enabled) { check(custos_hip_set_graph_fusing(dev_, enabled ? 1 : 0)); }
+    // How long the first run of a program may spend compiling kernels of joined launches (default 1000 ms);
+    // what it does not get within that replays as the launches that were recorded.
+    void set_graph_fusing_budget(uint32_t milliseconds) { check(custos_hip_set_graph_fusing_budget(dev_, milliseconds)); }
+    // Recorded launches of the current graph that would have been joined, had the build got their kernel, and why not.
+    std::pair<size_t, std::string> graph_unjoined() const {
+        size_t launches = 0;
+        const char* reason = "";
+        if (graph_) custos_hip_graph_unjoined(graph_, &launches, &reason);
+        return {launches, reason ? reason : ""};
+    }
+    // (hiprtc translation units compiled so far, milliseconds spent in them)
+    std::pair<uint64_t, double> compile_stats() const {
+        uint64_t units = 0;
+        double ms = 0;
+        custos_hip_compile_stats(dev_, &units, &ms);
+        return {units, ms};
+    }
 
     custos_hip_kernel* compile(int32_t kind, int32_t dtype, const std::string& src,
                                std::initializer_list<const char*> markers) {

@@ -318,6 +318,57 @@ def test_unaligned_views(hip, oracle, off_in, off_out, n):
     assert_bits_equal(got, want)
 
 
+def test_every_launch_shape_the_library_picks_gives_the_same_bits(oracle):
+    """Large launches over views with a scalar head and tail, in every shape the library picks by itself:
+    one-wavefront workgroups with one vector per thread (nothing of the launch before is revisited), 128
+    threads x 2 vectors (the same launch again), alternating directions, directly and as a replayed
+    recording; and a recorded chain that mostly writes (temporal loads, stores past the cache)."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        n = (12 << 20) + 7                           # 48 MiB per array and a ragged end
+        x = synth.uniform_f32(83, n + 16, -2, 2)
+        f = lambda v: v.mul(3.0).sub(1.0)
+        xb, ob = dev.buffer(x), dev.alloc(n + 16)
+        seen = set()
+        for off in (0, 1, 3):                        # aligned; equal phase with a head; (same phase in and out)
+            want = oracle.apply_fn(f, x[off:off + n])
+            for repeat in range(3):
+                ob.clear()
+                dev.apply_fn(xb.slice(off, off + n), f, out=ob.slice(off, off + n))
+                seen.add(dev.last_launch_shape()[0])
+                assert_bits_equal(ob.slice(off, off + n).read(), want, f"offset {off}, launch {repeat}")
+            dev.capture_begin()
+            dev.apply_fn(xb.slice(off, off + n), f, out=ob.slice(off, off + n))
+            g = dev.capture_end()
+            for replay in range(3):
+                ob.clear()                            # (a fill in between: the replay revisits nothing it wrote)
+                g.launch()
+                assert_bits_equal(ob.slice(off, off + n).read(), want, f"offset {off}, replay {replay}")
+            g.destroy()
+        assert seen == {1, 2}
+        # 1 read + 3 writes, 192 MiB: the joined kernel of three recorded launches
+        a, b, c = dev.alloc(n), dev.alloc(n), dev.alloc(n)
+        g1, g2 = (lambda v: v.abs().sqrt()), (lambda v: v.neg().max(-1.0))
+        dev.capture_begin()
+        dev.apply_fn(xb.slice(0, n), f, out=a)
+        dev.apply_fn(a, g1, out=b)
+        dev.apply_fn(b, g2, out=c)
+        g = dev.capture_end()
+        assert (g.kernel_nodes, g.fused_launches) == (1, 2)
+        assert dev.last_launch_shape()[1] == (2 | 64)           # stores non-temporal and written through, loads temporal
+        for replay in range(2):
+            g.launch()
+            wa = oracle.apply_fn(f, x[:n])
+            wb = oracle.apply_fn(g1, wa)
+            assert_bits_equal(a.read(), wa)
+            assert_bits_equal(b.read(), wb)
+            assert_bits_equal(c.read(), oracle.apply_fn(g2, wb))
+        g.destroy()
+    finally:
+        dev.close()
+
+
 def test_f16_unaligned_views(hip, oracle):
     total = 5000
     xb = synth.uniform_f16_bits(5, total, -2, 2)
