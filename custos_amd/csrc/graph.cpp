@@ -639,16 +639,18 @@ std::vector<Planned> plan_level(custos_hip_device* dev, const std::vector<RecNod
         if (first.type == RecNode::Kernel) {
             // the launch shape follows the bytes the (merged) launch touches and the launches around it
             p.kern = first.k;
-            if (p.members.size() == 1) {
-                // one launch: decided as for a launch issued directly, with what the graph knows on top
-                // (whether one of the next levels reads what it writes)
-                bool feeds_later = false;
-                for (const Access& a : first.acc)
-                    for (const std::vector<Access>* level : later_reads)
-                        for (const Access& r : *level) feeds_later = feeds_later || (a.write && r.begin < a.end && a.begin < r.end);
-                p.feeds_later = feeds_later;
+            unsigned long long touched = 0;
+            for (const Access& a : first.acc) touched += a.end - a.begin;
+            if (p.members.size() == 1 && touched > kTrafficBeyondBytes) {
+                // one large launch: decided as for a launch issued directly, with what the graph knows on
+                // top (whether one of the next levels reads what it writes)
+                if (touched >= kHintFromBytes)
+                    for (const Access& a : first.acc)
+                        for (const std::vector<Access>* level : later_reads)
+                            for (const Access& r : *level)
+                                p.feeds_later = p.feeds_later || (a.write && r.begin < a.end && a.begin < r.end);
                 RecentTraffic before = *history;  // (the level's traffic joins the history below, once)
-                p.shape = shape_of_launch(dev, first.k, first.acc, &before, feeds_later);
+                p.shape = shape_of_launch(dev, first.k, first.acc, &before, p.feeds_later);
             } else {
                 unsigned long long footprint = 0;
                 for (size_t i : p.members) footprint += nodes[i].ptrs.size() * nodes[i].n * dtype_size(nodes[i].k->spec.dtype);

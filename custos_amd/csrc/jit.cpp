@@ -312,8 +312,6 @@ static int32_t compile_expr(custos_hip_device* dev, int32_t kind, int32_t dtype,
     return CUSTOS_HIP_OK;
 }
 
-custos_hip_kernel* cached_chain_kernel(custos_hip_device* dev, const KernelSpec& spec) { return find_code(dev, spec); }
-
 int32_t chain_kernel(custos_hip_device* dev, DType dtype, std::vector<ChainStage> stages, int n_ext, int n_outs,
                      const Tuning& tuning, custos_hip_kernel** out) {
     std::unique_ptr<custos_hip_kernel> k(new custos_hip_kernel);

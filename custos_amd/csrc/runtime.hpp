@@ -299,8 +299,6 @@ inline uint64_t single_launch_mode(const custos_hip_kernel* k, unsigned long lon
 inline const std::vector<unsigned char>& literal_values(const RecNode& n) {
     return n.k->spec.kind == custos_hip::Kind::Chain ? n.const_bytes : n.k->spec.consts.bytes;
 }
-// The cached kernel of a chain spec (built without its text), or null.
-custos_hip_kernel* cached_chain_kernel(custos_hip_device* dev, const KernelSpec& spec);
 // launch.cpp
 int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std::vector<Range>& ops, size_t n);
 // Workgroups of a single launch of `k` over n_vec vectors and n elements in the given shape.
