@@ -113,6 +113,8 @@ PROTOTYPES = {
     "custos_hip_kernel_name": (C.c_char_p, [_P]),
     "custos_hip_kernel_hash": (C.c_uint64, [_P]),
     "custos_hip_preferred_shape": (C.c_int32, [C.c_uint64, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "custos_hip_preferred_shape_of": (C.c_int32, [C.c_uint64, C.c_int32, C.c_int32, C.c_uint64, C.c_int32, C.POINTER(C.c_int32),
+                                                  C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "custos_hip_set_graph_fusing": (C.c_int32, [_P, C.c_int32]),
     "custos_hip_graph_node_kernel": (C.c_int32, [_P, C.c_size_t, C.POINTER(C.c_char_p)]),
     "custos_hip_graph_fused_launches": (C.c_int32, [_P, C.POINTER(C.c_size_t)]),
@@ -214,6 +216,15 @@ def preferred_shape(footprint_bytes: int, n_operands: int):
     u, nt, alt = C.c_int32(0), C.c_int32(0), C.c_int32(0)
     check(load_library().custos_hip_preferred_shape(footprint_bytes, n_operands, C.byref(u), C.byref(nt), C.byref(alt)))
     return u.value, nt.value, bool(alt.value)
+
+
+def preferred_shape_of(footprint_bytes: int, n_operands: int, n_written: int = 1, working_set_bytes: int = 0, revisits: bool = True):
+    """(vectors per thread, nontemporal bits, alternates direction, threads per workgroup or 0) with everything
+    the choice depends on."""
+    u, nt, alt, block = C.c_int32(0), C.c_int32(0), C.c_int32(0), C.c_int32(0)
+    check(load_library().custos_hip_preferred_shape_of(footprint_bytes, n_operands, n_written, working_set_bytes, int(revisits),
+                                                       C.byref(u), C.byref(nt), C.byref(alt), C.byref(block)))
+    return u.value, nt.value, bool(alt.value), block.value
 
 
 LITERALS_ADAPTIVE, LITERALS_IN_CODE, LITERALS_AS_PARAMETERS = 0, 1, 2

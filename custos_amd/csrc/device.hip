@@ -28,6 +28,7 @@ int32_t hip_fail(custos_hip_device* dev, hipError_t e, const char* what) {
 const std::string& thread_last_error() { return g_last_error; }
 
 constexpr size_t kStagedReadMax = 64u << 10;  // reads and writes up to this size go through pinned staging memory
+constexpr size_t kSignalledReadMax = 4u << 10;  // reads up to this size: the copy kernel also writes the wait's completion word
 constexpr size_t kWriteSlots = 16;            // staging slots of short writes (the first slot of the block is the read's)
 
 // Operand table of custos_hip_apply_fn_many_noalloc: device memory that belongs to the
@@ -86,14 +87,8 @@ static inline void cpu_pause() {
 #endif
 }
 
-static hipError_t wait_compute_stream_now(custos_hip_device* dev) {
-    if (!dev->done_flag) return hipStreamSynchronize(dev->stream);
-    const uint32_t seq = ++dev->done_seq;
-    hipError_t e = hipStreamWriteValue32(dev->stream, dev->done_flag_dev, seq, 0);
-    if (e != hipSuccess) {
-        (void)hipGetLastError();
-        return hipStreamSynchronize(dev->stream);
-    }
+// Polls the completion word until it holds `seq` (see above for how long).
+static hipError_t poll_completion_word(custos_hip_device* dev, uint32_t seq) {
     using clock = std::chrono::steady_clock;
     using std::chrono::nanoseconds;
     custos_hip_graph* const graph = dev->graphs_since_wait == 1 && !dev->launches_since_wait ? dev->graph_since_wait : nullptr;
@@ -126,6 +121,17 @@ static hipError_t wait_compute_stream_now(custos_hip_device* dev) {
     dev->graphs_since_wait = 0;
     dev->launches_since_wait = false;
     return result;
+}
+
+static hipError_t wait_compute_stream_now(custos_hip_device* dev) {
+    if (!dev->done_flag) return hipStreamSynchronize(dev->stream);
+    const uint32_t seq = ++dev->done_seq;
+    hipError_t e = hipStreamWriteValue32(dev->stream, dev->done_flag_dev, seq, 0);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return hipStreamSynchronize(dev->stream);
+    }
+    return poll_completion_word(dev, seq);
 }
 
 // `waits_begun` / `waits_done` number the waits: work issued while `waits_begun` was w has
@@ -230,6 +236,25 @@ __global__ void __launch_bounds__(kFillBlock) custos_stage_copy(unsigned char* d
     for (unsigned long long i = gid; i < n_vec; i += n_threads) d[i] = s[i];
     if (gid < head) dst[gid] = src[gid];
     for (unsigned long long i = head + n_vec * 16 + gid; i < bytes; i += n_threads) dst[i] = src[i];
+}
+
+// The same copy by ONE workgroup that writes the completion word of the wait itself when it is
+// done (a few KiB at most: what a caller reads back between launches is a loss value, a
+// handful of parameters).  The word is written behind the data: all copies of the workgroup,
+// a fence to system scope, then the store, which travels the same way to host memory as the data.
+__global__ void __launch_bounds__(kFillBlock) custos_stage_copy_and_signal(unsigned char* dst, const unsigned char* src,
+                                                                           unsigned long long bytes, unsigned long long head,
+                                                                           unsigned long long n_vec, unsigned int* word,
+                                                                           unsigned int seq) {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    u4* d = reinterpret_cast<u4*>(dst + head);
+    const u4* s = reinterpret_cast<const u4*>(src + head);
+    for (unsigned long long i = threadIdx.x; i < n_vec; i += kFillBlock) d[i] = s[i];
+    if (threadIdx.x < head) dst[threadIdx.x] = src[threadIdx.x];
+    for (unsigned long long i = head + n_vec * 16 + threadIdx.x; i < bytes; i += kFillBlock) dst[i] = src[i];
+    __threadfence_system();
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_store(word, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // `dst` and `src` at the same 16-byte phase; runs on the compute stream, never recorded.
@@ -676,6 +701,22 @@ int32_t custos_hip_read(custos_hip_device* dev, void* dst, uint64_t src, size_t 
     // about 8 us.
     if (!dev->capturing && dev->read_stage && bytes <= kStagedReadMax) {
         const uint64_t phase = src & 15;
+        if (bytes <= kSignalledReadMax) {
+            // one dispatch instead of two: the copy's one workgroup ends with the completion word
+            unsigned long long head = (16 - phase) & 15;
+            if (head > bytes) head = bytes;
+            const unsigned long long n_vec = (bytes - head) / 16;
+            const uint64_t mine = ++dev->waits_begun;
+            const uint32_t seq = ++dev->done_seq;
+            hipLaunchKernelGGL(custos_stage_copy_and_signal, dim3(1), dim3(kFillBlock), 0, dev->stream,
+                               reinterpret_cast<unsigned char*>(dev->read_stage_dev + phase), reinterpret_cast<const unsigned char*>(src),
+                               static_cast<unsigned long long>(bytes), head, n_vec, static_cast<unsigned int*>(dev->done_flag_dev), seq);
+            HIP_TRY(dev, hipGetLastError());
+            HIP_TRY(dev, poll_completion_word(dev, seq));
+            dev->waits_done = mine;
+            std::memcpy(dst, dev->read_stage + phase, bytes);
+            return CUSTOS_HIP_OK;
+        }
         int32_t rc = launch_stage_copy(dev, dev->read_stage_dev + phase, src, bytes);
         if (rc != CUSTOS_HIP_OK) return rc;
         HIP_TRY(dev, wait_compute_stream(dev));

@@ -588,6 +588,19 @@ int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands,
     return CUSTOS_HIP_OK;
 }
 
+int32_t custos_hip_preferred_shape_of(uint64_t footprint_bytes, int32_t n_operands, int32_t n_written,
+                                      uint64_t working_set_bytes, int32_t revisits, int32_t* unroll, int32_t* nontemporal,
+                                      int32_t* alternate, int32_t* block_threads) {
+    if (n_operands < 1 || n_written < 0 || n_written > n_operands)
+        return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "n_operands must be positive and n_written within it");
+    const LaunchShape s = preferred_shape(footprint_bytes, n_operands, CacheHint::Unknown, working_set_bytes, revisits != 0, n_written);
+    if (unroll) *unroll = s.unroll;
+    if (nontemporal) *nontemporal = s.nontemporal;
+    if (alternate) *alternate = s.alternate ? 1 : 0;
+    if (block_threads) *block_threads = s.block;
+    return CUSTOS_HIP_OK;
+}
+
 int32_t custos_hip_expr_canonical(const char* src, const char* const* markers, int32_t n_markers,
                                   char* buf, size_t cap, size_t* needed) {
     if (!src) return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "expression source is null");

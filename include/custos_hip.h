@@ -318,6 +318,17 @@ int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated
  * together; otherwise it streams like a larger one.  And a launch of 256 to 768 MiB through two
  * pointers streams its stores past the memory-side cache as well when those launches touched
  * other memory too. */
+/* The same with everything else the choice depends on: how many of the operands the launch
+ * writes (`n_written`: a kernel that writes through at least two pointers more than it reads
+ * through, and touches 128 MiB or more, takes temporal loads and non-temporal stores written
+ * through at once, so that the cache keeps its input and not its outputs), the distinct bytes the
+ * launch and the launches before it touch together (`working_set_bytes`, 0 = unknown), and
+ * whether it touches memory that the launch before it wrote (`revisits`: a launch of more than
+ * 32 MiB that does not runs as one-wavefront workgroups with one vector per thread;
+ * `block_threads` receives 64 then, else 0 for the workgroup size the kernel was compiled for). */
+int32_t custos_hip_preferred_shape_of(uint64_t footprint_bytes, int32_t n_operands, int32_t n_written,
+                                      uint64_t working_set_bytes, int32_t revisits, int32_t *unroll,
+                                      int32_t *nontemporal, int32_t *alternate, int32_t *block_threads);
 int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands, int32_t *unroll,
                                    int32_t *nontemporal, int32_t *alternate);
 /* The shape of the generated kernel that was launched directly, or planned into a graph by

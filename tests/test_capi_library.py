@@ -142,6 +142,41 @@ def test_launch_shape_by_bytes_touched():
         shape(1, 0)
 
 
+def test_launch_shape_by_what_a_launch_revisits_and_writes():
+    """The two refinements of the choice: a launch of more than 32 MiB that touches nothing the launch before
+    it wrote streams as one-wavefront workgroups with one vector per thread; a kernel that writes through at
+    least two pointers more than it reads through keeps its input in the cache instead of its outputs, from
+    128 MiB touched on.  The rest of the choice does not move with either."""
+    MiB = 1 << 20
+    shape = capi.preferred_shape_of
+    loads, both, stores = 1 | 64, 3, 2 | 64
+    for footprint, n_ops in ((8 * MiB, 2), (32 * MiB, 2), (64 * MiB, 4), (512 * MiB, 2), (2048 * MiB, 2)):
+        assert shape(footprint, n_ops)[:3] == capi.preferred_shape(footprint, n_ops)        # revisiting, one output: as before
+        assert shape(footprint, n_ops)[3] == 0
+    # revisits nothing
+    assert shape(32 * MiB, 2, revisits=False) == (2, 0, False, 0)                            # the L2s still hold it
+    assert shape(32 * MiB + 1, 2, revisits=False) == (1, loads, False, 64)
+    assert shape(48 * MiB, 3, revisits=False) == (1, loads, False, 64)
+    assert shape(512 * MiB, 2, revisits=False) == (1, loads, True, 64)                       # config 3 forward after backward
+    assert shape(512 * MiB, 2, working_set_bytes=1280 * MiB, revisits=False) == (1, both, True, 64)
+    assert shape(768 * MiB, 3, revisits=False) == (1, loads, True, 64)                       # config 3 backward after forward
+    assert shape(2048 * MiB, 2, revisits=False) == (1, loads, True, 64)                      # the first launch of an unfused chain
+    assert shape(20 * MiB, 2, working_set_bytes=60 * MiB, revisits=False) == (2, loads, False, 0)   # small launches keep 128 x 2
+    # mostly writes
+    assert shape(4096 * MiB, 4, n_written=3) == (2, stores, True, 0)                         # config 2 recorded unfused: 1R + 3W
+    assert shape(256 * MiB, 4, n_written=3) == (2, stores, False, 0)
+    assert shape(128 * MiB, 4, n_written=3) == (2, stores, False, 0)
+    assert shape(127 * MiB, 4, n_written=3) == (2, loads, False, 0)                          # below: the usual policy is ahead
+    assert shape(96 * MiB, 6, n_written=3) == (2, loads, False, 0)                           # config 5 as recorded: 3R + 3W
+    assert shape(1024 * MiB, 4, n_written=2) == (2, loads, True, 0)                          # 2R + 2W
+    assert shape(1024 * MiB, 3, n_written=2) == (2, loads, True, 0)                          # 1R + 2W: one more, not two
+    assert shape(1280 * MiB, 5, n_written=2) == (2, loads, True, 0)                          # config 3 joined: 3R + 2W
+    assert shape(1536 * MiB, 6, n_written=5) == (2, stores, True, 0)                         # 1R + 5W
+    assert shape(1536 * MiB, 6, n_written=5, revisits=False) == (1, stores, True, 64)
+    with pytest.raises(capi.CustosHipError):
+        shape(1 * MiB, 2, n_written=3)
+
+
 def test_operands_of_different_lengths_are_rejected_on_the_host():
     """A shorter operand would be read or written beyond its end on the device: the binding checks
     lengths and element types before anything reaches the library (no device needed to see it)."""
