@@ -734,18 +734,42 @@ def bench_others(dev, args, stack_c5):
     e["fused"]["GBps"] = e["fused"]["GBps_on_16B"]
     graph.destroy()
     # the same fused expression over the same 1024 operand sets through the entry point that allocates
-    # nothing (its table sits in a static device array; every call checks the operand sets on the host
-    # and sends the rows through a pinned staging slot)
+    # nothing (its table sits in a static device array).  A call identical to the last one finds its
+    # rows in the table; a call with other rows is checked on the host and sends its rows through a
+    # pinned staging slot: timed here with the sets in two orders, alternating.
     dev.prepare_merged(kfused)
-    rows = (C.c_uint64 * (4 * nbuf))(*[p for i in range(nbuf) for p in (A.ptr + i * m * 4, B.ptr + i * m * 4, Cc.ptr + i * m * 4, Y.ptr + i * m * 4)])
+    sets = [(A.ptr + i * m * 4, B.ptr + i * m * 4, Cc.ptr + i * m * 4, Y.ptr + i * m * 4) for i in range(nbuf)]
+    rows = (C.c_uint64 * (4 * nbuf))(*[p for row in sets for p in row])
+    rows_backwards = (C.c_uint64 * (4 * nbuf))(*[p for row in reversed(sets) for p in row])
     Y.clear()
     na_step = launcher(dev, lib.custos_hip_apply_fn_many_noalloc, kfused, rows, 4, nbuf, m)
     na_ms, na_calls = time_floor(dev, na_step)
     assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), "c5 through the allocation-free entry point differs"
+    Y.clear()
+    na_other = launcher(dev, lib.custos_hip_apply_fn_many_noalloc, kfused, rows_backwards, 4, nbuf, m)
+    def na_alternating():
+        na_step()
+        na_other()
+    alt_ms, alt_calls = time_floor(dev, na_alternating)
+    assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), "c5 through the allocation-free entry point differs"
+    # sixteen orders in turn: more than the entry point remembers, so every call is checked in full
+    Y.clear()
+    rotated = [launcher(dev, lib.custos_hip_apply_fn_many_noalloc, kfused,
+                        (C.c_uint64 * (4 * nbuf))(*[p for row in sets[k * 61:] + sets[:k * 61] for p in row]), 4, nbuf, m) for k in range(16)]
+    def na_new_every_time():
+        for call in rotated:
+            call()
+    new_ms, new_calls = time_floor(dev, na_new_every_time)
+    assert np.array_equal(Y.read().view(np.uint32), want.view(np.uint32)), "c5 through the allocation-free entry point differs"
     e["fused"]["allocation_free_entry_point"] = {
         "us_per_call": round(na_ms * 1e3, 2), "calls": na_calls, "GBps_on_16B": round(16 * nbuf * m / (na_ms * 1e-3) / 1e9, 2),
-        "what": "custos_hip_apply_fn_many_noalloc over the same 1024 operand sets, back to back from Python: operand checks on "
-                "the host, 32 KiB of table rows through a staging slot and the copy kernel, then the same grid"}
+        "us_per_call_alternating_two_tables": round(alt_ms * 1e3 / 2, 2), "calls_alternating": 2 * alt_calls,
+        "us_per_call_with_rows_never_seen": round(new_ms * 1e3 / 16, 2), "calls_never_seen": 16 * new_calls,
+        "what": "custos_hip_apply_fn_many_noalloc over the same 1024 operand sets, back to back from Python; us_per_call: the same "
+                "call again and again (its rows are still in the table: one launch); alternating two tables: both have passed the "
+                "operand checks before, 32 KiB of table rows go through a staging slot and the copy kernel before each launch; "
+                "rows never seen: sixteen orders of the sets in turn, each call checked in full on the host (4096 address ranges, "
+                "in time linear in their number) before its rows are sent"}
     e["module_stack"] = stack_c5
     out["c5"] = e
     return out

@@ -47,6 +47,10 @@ static unsigned long long* g_scratch_ptr[kMaxDevices];
 // from the wait to the event record, so that calls from several threads take turns.
 static hipEvent_t g_scratch_event[kMaxDevices];
 static const custos_hip_device* g_scratch_last_user[kMaxDevices];
+// Handles alive per GPU.  While a GPU has one handle its stream alone orders the table's users and
+// no event is recorded; when a second handle appears, the event is recorded once behind whatever
+// the last user has launched so far, and from then on behind every launch.
+static int g_scratch_handles[kMaxDevices];
 static std::mutex g_scratch_mutex;
 static_assert(kScratchWords * sizeof(unsigned long long) <= kStagedReadMax, "the table travels through one staging slot");
 
@@ -66,6 +70,13 @@ static hipError_t scratch_address(int idx, unsigned long long** out) {
         g_scratch_ptr[idx] = static_cast<unsigned long long*>(p);
     }
     *out = g_scratch_ptr[idx];
+    if (++g_scratch_handles[idx] == 2 && g_scratch_last_user[idx]) {
+        hipError_t e = hipEventRecord(g_scratch_event[idx], g_scratch_last_user[idx]->stream);
+        if (e != hipSuccess) {
+            g_scratch_handles[idx]--;
+            return e;
+        }
+    }
     return hipSuccess;
 }
 
@@ -447,7 +458,8 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
         (void)hipGetLastError();
         dev->scratch_table = nullptr;
     }
-    dev->noalloc_spans.reserve(kScratchWords);  // so that the entry point that may not allocate finds its room
+    dev->noalloc_checker.reserve(kScratchWords / 2);  // so that the entry point that may not allocate finds its room
+    for (auto& call : dev->noalloc_checked) call.operands.reserve(kScratchWords);
     // completion word for short waits (pinned, mapped host memory); optional
     void* flag = nullptr;
     if (hipHostMalloc(&flag, 64, hipHostMallocMapped) == hipSuccess) {
@@ -490,6 +502,7 @@ int32_t custos_hip_device_destroy(custos_hip_device* dev) {
         // (its launches have finished: the next user of the table need not wait for this handle)
         std::lock_guard<std::mutex> lock(g_scratch_mutex);
         if (g_scratch_last_user[dev->idx] == dev) g_scratch_last_user[dev->idx] = nullptr;
+        if (dev->scratch_table) g_scratch_handles[dev->idx]--;
     }
     for (custos_hip_graph* g : dev->graphs) destroy_graph(g);
     // every block of this handle goes back to the driver, pooled or still held by the caller
@@ -762,6 +775,99 @@ int32_t custos_hip_fill(custos_hip_device* dev, uint64_t dptr, size_t bytes, con
 
 // ---- many launches of one kernel in one grid, without any allocation ----
 
+}  // extern "C"
+
+namespace custos_hip {
+
+void OperandSetChecker::reserve(size_t max_sets) {
+    size_t size = 16;
+    while (size < 2 * max_sets) size *= 2;
+    if (slots.size() < size) {
+        slots.assign(size, Slot{0, 0, 0, 0});
+        stamp = 0;
+    }
+}
+
+int32_t OperandSetChecker::check(const uint64_t* operands, int n_ptrs, size_t n_sets, int written, uint64_t bytes, const char** why) {
+    if (slots.size() < 2 * n_sets || bytes == 0 || written < 0 || written >= n_ptrs) {
+        *why = "operand check called outside its limits";
+        return CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+    }
+    if (++stamp == 0) {  // (after 2^32 checks: every slot looks empty again)
+        for (Slot& slot : slots) slot.stamp = 0;
+        stamp = 1;
+    }
+    const size_t mask = slots.size() - 1;
+    int shift = 64;
+    for (size_t size = slots.size(); size > 1; size /= 2) shift--;
+    auto home = [&](uint64_t piece) { return static_cast<size_t>((piece * 0x9e3779b97f4a7c15ull) >> shift); };
+    // the rows one by one, and the written operand of each into the table
+    for (size_t s = 0; s < n_sets; s++) {
+        const uint64_t* row = operands + s * static_cast<size_t>(n_ptrs);
+        const uint64_t out = row[written];
+        for (int i = 0; i < n_ptrs; i++) {
+            if (row[i] == 0) {
+                *why = "null device pointer";
+                return CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+            }
+            if (row[i] & 15) {
+                *why = "operands of a merged launch are 16-byte aligned";
+                return CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+            }
+            if (row[i] > UINT64_MAX - bytes) {
+                *why = "an operand range wraps around the address space";
+                return CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+            }
+        }
+        for (int i = 0; i < n_ptrs; i++)
+            if (i != written && row[i] != out && row[i] < out + bytes && out < row[i] + bytes) {
+                *why = "the output range partially overlaps an input range";
+                return CUSTOS_HIP_ERR_BAD_OVERLAP;
+            }
+        const uint64_t piece = out / bytes;
+        size_t at = home(piece);
+        for (; slots[at].stamp == stamp; at = (at + 1) & mask)
+            if (slots[at].piece == piece) {  // two written operands less than their length apart
+                *why = "an operand set writes memory that another operand set uses";
+                return CUSTOS_HIP_ERR_BAD_OVERLAP;
+            }
+        slots[at] = Slot{piece, out, static_cast<uint32_t>(s), stamp};
+    }
+    // every operand against the written operands of the other rows around it
+    for (size_t s = 0; s < n_sets; s++) {
+        const uint64_t* row = operands + s * static_cast<size_t>(n_ptrs);
+        for (int i = 0; i < n_ptrs; i++) {
+            const uint64_t a = row[i], piece = a / bytes;
+            for (uint64_t p = piece == 0 ? 0 : piece - 1; p <= piece + 1; p++)
+                for (size_t at = home(p); slots[at].stamp == stamp; at = (at + 1) & mask) {
+                    if (slots[at].piece != p) continue;
+                    const uint64_t w = slots[at].begin;
+                    if (slots[at].set != s && w < a + bytes && a < w + bytes) {
+                        *why = "an operand set writes memory that another operand set uses";
+                        return CUSTOS_HIP_ERR_BAD_OVERLAP;
+                    }
+                    break;  // (one written operand per piece)
+                }
+        }
+    }
+    return CUSTOS_HIP_OK;
+}
+
+}  // namespace custos_hip
+
+extern "C" {
+
+int32_t custos_hip_check_operand_sets(const uint64_t* operands, int32_t operands_per_set, size_t n_sets, int32_t written,
+                                      uint64_t bytes) {
+    if (!operands || operands_per_set < 1 || written < 0 || written >= operands_per_set || bytes == 0)
+        return CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+    if (n_sets == 0) return CUSTOS_HIP_OK;
+    OperandSetChecker checker;
+    checker.reserve(n_sets);
+    const char* why = "";
+    return checker.check(operands, operands_per_set, n_sets, written, bytes, &why);
+}
+
 int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kernel* kernel, const uint64_t* operands,
                                          int32_t operands_per_set, size_t n_sets, size_t n) {
     REQUIRE_DEV(dev);
@@ -794,57 +900,30 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
                              std::to_string(kScratchWords * 8) + " bytes), got " + std::to_string(n_sets));
     // Operand checks on the host, before anything is launched: aligned, no partial overlap
     // inside a set (`out == in` exactly is fine), and no set writes what another set touches.
-    // The spans live in a buffer the handle reserved when it was created.  A serving loop calls
-    // with the same table again and again: the table that passed last is remembered by a hash
-    // of everything the checks depend on, and passes again without them.
+    // Their work area was made when the handle was created.  A serving loop calls
+    // with the same few tables again and again: the calls that passed last are kept, and a call
+    // identical to one of them passes again without the checks.
     const uint64_t bytes = static_cast<uint64_t>(n) * dtype_size(kernel->spec.dtype);
-    uint64_t table_hash = 0x9e3779b97f4a7c15ull ^ reinterpret_cast<uint64_t>(owner) ^ (static_cast<uint64_t>(n) * 0xbf58476d1ce4e5b9ull) ^
-                          (static_cast<uint64_t>(n_sets) << 40);
-    for (size_t w = 0; w < n_sets * static_cast<size_t>(n_ptrs); w++) {
-        table_hash = (table_hash ^ operands[w]) * 0x94d049bb133111ebull;
-        table_hash ^= table_hash >> 29;
+    const size_t n_words = n_sets * static_cast<size_t>(n_ptrs);
+    int known = -1;
+    for (size_t c = 0; c < dev->noalloc_checked.size() && known < 0; c++) {
+        const auto& call = dev->noalloc_checked[c];
+        if (call.kernel == kernel && call.n == n && call.operands.size() == n_words &&
+            std::memcmp(call.operands.data(), operands, n_words * 8) == 0)
+            known = static_cast<int>(c);
     }
-    if (table_hash != dev->noalloc_checked) {
+    if (known < 0) {
         const int written = kernel->spec.kind == Kind::UnaryGrad ? 1 : n_ptrs - 1;
-        using Span = custos_hip_device::OperandSpan;
-        std::vector<Span>& spans = dev->noalloc_spans;
-        spans.clear();
-        for (size_t s = 0; s < n_sets; s++) {
-            const uint64_t* row = operands + s * static_cast<size_t>(n_ptrs);
-            for (int i = 0; i < n_ptrs; i++) {
-                if (row[i] == 0) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "null device pointer");
-                if (row[i] & 15)
-                    return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "operands of a merged launch are 16-byte aligned");
-                if (i != written && row[i] != row[written] && row[i] < row[written] + bytes && row[written] < row[i] + bytes)
-                    return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP, "the output range partially overlaps an input range");
-                spans.push_back({row[i], static_cast<uint32_t>(s), i == written});
-            }
-        }
-        std::sort(spans.begin(), spans.end(), [](const Span& a, const Span& b) { return a.begin < b.begin; });
-        // sweep by start address: the furthest-reaching earlier span of any kind and the furthest
-        // written one, each with a runner-up from another set
-        struct Reach {
-            uint64_t end[2] = {0, 0};
-            uint32_t set[2] = {0xffffffffu, 0xffffffffu};
-            void add(uint64_t e, uint32_t s) {
-                if (s == set[0]) {
-                    end[0] = std::max(end[0], e);
-                } else if (e > end[0]) {
-                    end[1] = end[0], set[1] = set[0];
-                    end[0] = e, set[0] = s;
-                } else if (e > end[1]) {
-                    end[1] = e, set[1] = s;
-                }
-            }
-            uint64_t other_than(uint32_t s) const { return set[0] != s ? end[0] : end[1]; }
-        } any, writes;
-        for (const Span& sp : spans) {
-            if ((sp.write && any.other_than(sp.set) > sp.begin) || writes.other_than(sp.set) > sp.begin)
-                return set_error(dev, CUSTOS_HIP_ERR_BAD_OVERLAP, "an operand set writes memory that another operand set uses");
-            any.add(sp.begin + bytes, sp.set);
-            if (sp.write) writes.add(sp.begin + bytes, sp.set);
-        }
-        dev->noalloc_checked = table_hash;
+        const char* why = "";
+        const int32_t verdict = dev->noalloc_checker.check(operands, n_ptrs, n_sets, written, bytes, &why);
+        if (verdict != CUSTOS_HIP_OK) return set_error(dev, verdict, why);
+        known = static_cast<int>(dev->noalloc_next);
+        dev->noalloc_next = (dev->noalloc_next + 1) % dev->noalloc_checked.size();
+        if (dev->noalloc_in_table == known) dev->noalloc_in_table = -1;
+        auto& call = dev->noalloc_checked[static_cast<size_t>(known)];
+        call.operands.assign(operands, operands + n_words);  // (within the reserved room: nothing is allocated)
+        call.kernel = kernel;
+        call.n = n;
     }
     const ResolvedShape shape = resolve_shape(dev, kernel, static_cast<unsigned long long>(n_sets) * n_ptrs * bytes);
     const unsigned long long count = n, n_vec = n / static_cast<unsigned long long>(kernel->spec.vec_elems);
@@ -861,24 +940,28 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
         HIP_TRY(dev, hipStreamWaitEvent(dev->stream, g_scratch_event[dev->idx], 0));
     // Table rows as the `_batched` entry point reads them (addresses, then the literal
     // parameters), written straight into a pinned staging slot; the library's copy kernel moves
-    // them into the table on the compute stream, behind the previous call's launch.
+    // them into the table on the compute stream, behind the previous call's launch.  Not needed
+    // when the table still holds the rows of an identical call of this handle.
     const uint64_t table_dev = reinterpret_cast<uint64_t>(dev->scratch_table);
-    unsigned char* slot_host = nullptr;
-    uint64_t slot_dev = 0;
-    int32_t rc = staging_slot(dev, table_dev, &slot_host, &slot_dev);
-    if (rc != CUSTOS_HIP_OK) return rc;
-    uint64_t* table = reinterpret_cast<uint64_t*>(slot_host);  // (the table is 256-byte aligned: phase 0)
-    for (size_t s = 0; s < n_sets; s++) {
-        uint64_t* row = table + s * row_words;
-        std::memcpy(row, operands + s * static_cast<size_t>(n_ptrs), static_cast<size_t>(n_ptrs) * 8);
-        for (size_t w = 0; w < const_words; w++) {
-            uint64_t word = 0;
-            std::memcpy(&word, values.data() + w * 8, std::min<size_t>(8, values.size() - w * 8));
-            row[n_ptrs + w] = word;
+    if (!(dev->noalloc_in_table == known && g_scratch_last_user[dev->idx] == dev)) {
+        dev->noalloc_in_table = -1;
+        unsigned char* slot_host = nullptr;
+        uint64_t slot_dev = 0;
+        int32_t rc = staging_slot(dev, table_dev, &slot_host, &slot_dev);
+        if (rc != CUSTOS_HIP_OK) return rc;
+        uint64_t* table = reinterpret_cast<uint64_t*>(slot_host);  // (the table is 256-byte aligned: phase 0)
+        for (size_t s = 0; s < n_sets; s++) {
+            uint64_t* row = table + s * row_words;
+            std::memcpy(row, operands + s * static_cast<size_t>(n_ptrs), static_cast<size_t>(n_ptrs) * 8);
+            for (size_t w = 0; w < const_words; w++) {
+                uint64_t word = 0;
+                std::memcpy(&word, values.data() + w * 8, std::min<size_t>(8, values.size() - w * 8));
+                row[n_ptrs + w] = word;
+            }
         }
+        rc = staging_slot_send(dev, table_dev, slot_dev, n_sets * row_words * 8);
+        if (rc != CUSTOS_HIP_OK) return rc;
     }
-    rc = staging_slot_send(dev, table_dev, slot_dev, n_sets * row_words * 8);
-    if (rc != CUSTOS_HIP_OK) return rc;
     unsigned long long mode = launch_mode(shape.unroll, shape.nontemporal, false, shape.block);
     uint64_t table_arg = table_dev;
     unsigned long long count_arg = count, n_vec_arg = n_vec;
@@ -886,8 +969,9 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
     dev->launches_since_wait = true;
     HIP_TRY(dev, hipModuleLaunchKernel(fn, static_cast<unsigned int>(tiles_per_seg * n_sets), 1, 1,
                                        static_cast<unsigned int>(shape.block), 1, 1, 0, dev->stream, args, nullptr));
-    HIP_TRY(dev, hipEventRecord(g_scratch_event[dev->idx], dev->stream));
+    if (g_scratch_handles[dev->idx] > 1) HIP_TRY(dev, hipEventRecord(g_scratch_event[dev->idx], dev->stream));
     g_scratch_last_user[dev->idx] = dev;
+    dev->noalloc_in_table = known;
     return CUSTOS_HIP_OK;
 }
 

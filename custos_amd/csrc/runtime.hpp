@@ -131,6 +131,30 @@ class RecentTraffic {
     std::vector<std::vector<Access>> launches_;  // oldest first, at most 8, each merged and sorted
 };
 
+// The operand checks of a merged launch over `n_sets` rows of `n_ptrs` device addresses, every
+// operand `bytes` long, operand number `written` of a row being the one the launch writes:
+// addresses non-null and 16-byte aligned, no partial overlap between a row's output and its inputs
+// (the same address is fine), and no row writes memory that another row reads or writes.
+// Linear in the number of operands: all operands have one length L, so two of them overlap exactly
+// when their addresses are less than L apart.  With memory cut into pieces of L bytes, at most one
+// written operand may start in a piece (two would overlap), and whatever overlaps a written operand
+// starts in its piece or a neighbouring one: the written operands go into a hash table by piece,
+// and every operand looks into three pieces.  The table is sized once (`reserve`) and reused by a
+// stamp per check, so a check allocates nothing.
+namespace custos_hip {
+struct OperandSetChecker {
+    struct Slot {
+        uint64_t piece, begin;
+        uint32_t set, stamp;
+    };
+    std::vector<Slot> slots;  // a power of two, at least twice the rows of a check
+    uint32_t stamp = 0;
+    void reserve(size_t max_sets);
+    // 0, or CUSTOS_HIP_ERR_INVALID_ARGUMENT / CUSTOS_HIP_ERR_BAD_OVERLAP with `*why` set
+    int32_t check(const uint64_t* operands, int n_ptrs, size_t n_sets, int written, uint64_t bytes, const char** why);
+};
+}  // namespace custos_hip
+
 struct custos_hip_device {
     int idx = 0;
     hipStream_t stream = nullptr;    // compute stream: every launch, in call order
@@ -177,15 +201,22 @@ struct custos_hip_device {
     uint32_t graphs_since_wait = 0;
     bool launches_since_wait = false;
     unsigned long long* scratch_table = nullptr;  // this device's copy of the library's static operand table
-    // operand ranges of a call of custos_hip_apply_fn_many_noalloc, for its overlap checks (room
-    // reserved when the handle is created: that call may not allocate, on the host either)
-    struct OperandSpan {
-        uint64_t begin;
-        uint32_t set;
-        bool write;
+    // work area of the operand checks of custos_hip_apply_fn_many_noalloc (made when the handle
+    // is created: that call may not allocate, on the host either)
+    custos_hip::OperandSetChecker noalloc_checker;
+    // The calls that passed those checks last (their addresses, kept in room reserved at creation,
+    // replaced in turn): a serving loop calls with the same few tables again and again, and a call
+    // identical to one of them passes without the checks.  `noalloc_in_table`: the entry whose
+    // rows the GPU's table still holds (nobody rewrote it since), or -1; a call identical to that
+    // one launches without sending its rows again.
+    struct CheckedCall {
+        const custos_hip_kernel* kernel = nullptr;
+        size_t n = 0;
+        std::vector<uint64_t> operands;
     };
-    std::vector<OperandSpan> noalloc_spans;
-    uint64_t noalloc_checked = 0;  // hash of the kernel, length and operand table that passed those checks last
+    std::array<CheckedCall, 4> noalloc_checked;
+    size_t noalloc_next = 0;
+    int noalloc_in_table = -1;
     unsigned char* read_stage = nullptr;  // pinned host memory short reads (first slot) and writes are staged in
     uint64_t read_stage_dev = 0;          // its device address
     uint64_t waits_begun = 0, waits_done = 0;  // waits for the compute stream, numbered

@@ -385,7 +385,10 @@ int32_t custos_hip_add_unary_grad(custos_hip_device *dev, custos_hip_kernel *ker
  * table words, else CUSTOS_HIP_ERR_TOO_LARGE (2048 sets of a three-operand kernel).  Not legal
  * while the device records (CUSTOS_HIP_ERR_CAPTURE_STATE).
  * All calls on one GPU share that GPU's table, which keeps the rows of the last call (nothing in
- * it has to start at zero: every row a launch reads is rewritten by its call).  Calls through one
+ * it has to start at zero: every row a launch reads is rewritten by its call -- except that a
+ * call identical to the handle's last one, kernel, length and addresses, finds its rows still in
+ * the table when no other handle used it in between, and launches without sending them again or
+ * repeating the operand checks).  Calls through one
  * device handle are ordered by its compute stream; a call through another handle on the same GPU
  * makes its stream wait for the launch of the table's last user before it rewrites the table
  * (one event per GPU, made when the first handle on that GPU is created), and calls from several
@@ -393,6 +396,12 @@ int32_t custos_hip_add_unary_grad(custos_hip_device *dev, custos_hip_kernel *ker
 int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device *dev, custos_hip_kernel *kernel,
                                          const uint64_t *operands, int32_t operands_per_set,
                                          size_t n_sets, size_t n);
+/* The operand checks of custos_hip_apply_fn_many_noalloc by themselves, on the host (no device is
+ * touched): `n_sets` rows of `operands_per_set` addresses, every operand `bytes` long, operand
+ * number `written` of a row the one a launch writes.  0, CUSTOS_HIP_ERR_INVALID_ARGUMENT (a null
+ * or unaligned address) or CUSTOS_HIP_ERR_BAD_OVERLAP.  No counterpart in the reference. */
+int32_t custos_hip_check_operand_sets(const uint64_t *operands, int32_t operands_per_set, size_t n_sets,
+                                      int32_t written, uint64_t bytes);
 /* Compiles (or takes from the caches) and loads the entry point of `kernel` for merged launches
  * of equal length.  A generated kernel has three entry points -- one launch; many launches of
  * equal length in one grid; many launches of different lengths in one grid -- each a translation

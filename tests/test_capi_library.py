@@ -247,3 +247,73 @@ def test_chain_emit_rejects_malformed_stages():
             capi.chain_emit("f32", stages, n_in, n_out)
     with pytest.raises(capi.CustosHipError):
         capi.chain_emit("i32", [("sin(v0)", [0], 0)], 1, 1)    # no such node over integers
+
+
+def _operand_sets_verdict(rows, written, length):
+    """What the checks of a merged launch must say, pair by pair."""
+    for row in rows:
+        if any(a == 0 or a % 16 for a in row):
+            return capi.ERR_INVALID_ARGUMENT
+    for row in rows:
+        out = row[written]
+        if any(i != written and a != out and a < out + length and out < a + length for i, a in enumerate(row)):
+            return capi.ERR_BAD_OVERLAP
+    for s, row in enumerate(rows):
+        out = row[written]
+        for t, other in enumerate(rows):
+            if t != s and any(a < out + length and out < a + length for a in other):
+                return capi.ERR_BAD_OVERLAP
+    return 0
+
+
+def test_operand_checks_of_merged_launches_against_all_pairs():
+    """The linear-time operand checks (host only) against the comparison of every pair of operands, on
+    random tables dense enough that about half of them hold a conflict, and on the edge cases: operands
+    exactly one length apart, an output equal to an input, inputs shared between rows, rows that meet
+    at the boundary of the pieces the check cuts memory into."""
+    import ctypes as C
+    import random
+    lib = capi.load_library()
+
+    def verdict(rows, written, length):
+        flat = (C.c_uint64 * (len(rows) * len(rows[0])))(*[a for row in rows for a in row])
+        return lib.custos_hip_check_operand_sets(flat, len(rows[0]), len(rows), written, length)
+
+    base = 0x7F0000000000
+    assert verdict([[base, base + 4096], [base + 64, base + 4096 + 64]], 1, 64) == 0                       # exactly one length apart
+    assert verdict([[base, base + 4096], [base + 48, base + 4096 + 64]], 1, 64) == 0                       # inputs may overlap
+    assert verdict([[base, base + 4096], [base + 64, base + 4096 + 48]], 1, 64) == capi.ERR_BAD_OVERLAP    # outputs may not
+    assert verdict([[base, base], [base + 64, base + 64]], 1, 64) == 0                                     # out == in
+    assert verdict([[base, base + 16]], 1, 64) == capi.ERR_BAD_OVERLAP                                     # partial, inside a row
+    assert verdict([[base, base + 4096], [base + 4096 + 16, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # reads another row's output
+    assert verdict([[base, base + 4096], [base + 4096 - 48, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # ... from the piece before
+    assert verdict([[base, base + 4096 + 16], [base + 4096 + 64, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # ... from the piece after
+    assert verdict([[base + 8, base + 4096]], 1, 64) == capi.ERR_INVALID_ARGUMENT
+    assert verdict([[0, base + 4096]], 1, 64) == capi.ERR_INVALID_ARGUMENT
+    assert verdict([[16, 4096]], 1, 48) == 0                                                               # the first piece of memory
+    rng = random.Random(5)
+    seen = {0: 0, capi.ERR_BAD_OVERLAP: 0}
+    for case in range(600):
+        n_ptrs = rng.choice([2, 3, 4])
+        written = rng.choice([n_ptrs - 1, 1]) if n_ptrs == 3 else n_ptrs - 1
+        n_sets = rng.randint(1, 40)
+        length = 16 * rng.randint(1, 12)
+        room = length * n_sets * n_ptrs * rng.choice([1, 2, 4, 40]) // 16
+        rows = []
+        for s in range(n_sets):
+            row = [base + 16 * rng.randrange(room) for _ in range(n_ptrs)]
+            if rng.random() < 0.2:
+                row[0] = row[written]                          # in place
+            rows.append(row)
+        if rng.random() < 0.5:
+            # tables made valid on purpose: outputs spaced out behind the room of the inputs
+            at = base + 16 * room + 4096
+            for s, row in enumerate(rows):
+                row[written] = at
+                at += length + 16 * rng.randrange(3)
+                if rng.random() < 0.2:
+                    row[0] = row[written]
+        want = _operand_sets_verdict(rows, written, length)
+        assert verdict(rows, written, length) == want, (case, rows, written, length)
+        seen[want] += 1
+    assert seen[0] > 100 and seen[capi.ERR_BAD_OVERLAP] > 100, seen

@@ -117,6 +117,40 @@ def test_calls_through_two_handles_take_turns_on_the_table(hip, oracle):
         other.close()
 
 
+def test_an_identical_call_finds_its_rows_in_the_table(hip, oracle):
+    """A serving loop calls with the same kernel, length and addresses again and again: the rows stay
+    in the table and only the launch is issued.  New data in the same buffers is picked up; a call
+    with other rows in between, through this handle or another, makes the next one send its rows again."""
+    import custos_amd
+    n, n_sets = 3000, 17
+    f = lambda a, b: a.mul(b).add(0.25)
+    kernel = hip.compile(capi.KIND_APPLY, "f32", f(Resolve("a", 0), Resolve("b", 1)).to_cl_source("f32"), ("a", "b"))
+    hip.prepare_merged(kernel)
+    ins = [[hip.alloc(n), hip.alloc(n)] for _ in range(n_sets)]
+    rows = [[a, b, hip.alloc(n)] for a, b in ins]
+    other = custos_amd.HIP(0)
+    try:
+        k_other = other.compile(capi.KIND_APPLY, "f32", "(x * 2.0)", ("x",))
+        other.prepare_merged(k_other)
+        rows_other = [[other.alloc(64), other.alloc(64)] for _ in range(40)]       # more rows than `rows`: all of them overwritten
+        for step in range(6):
+            host = [[synth.uniform_f32(7000 + 100 * step + 2 * s + k, n, -2, 2) for k in range(2)] for s in range(n_sets)]
+            for s in range(n_sets):
+                hip.write(ins[s][0], host[s][0])
+                hip.write(ins[s][1], host[s][1])
+            if step == 2:
+                hip.apply_fn_many_noalloc(kernel, rows[:5], n)                      # other rows through this handle
+            if step == 4:
+                other.apply_fn_many_noalloc(k_other, rows_other, 64)                # other rows through another handle
+                other.sync()
+            hip.apply_fn_many_noalloc(kernel, rows, n)
+            for s in range(n_sets):
+                want = oracle.apply_fn(f, *host[s])
+                assert np.array_equal(rows[s][2].read().view(np.uint32), want.view(np.uint32)), f"step {step}, set {s}"
+    finally:
+        other.close()
+
+
 def test_limits_and_operand_checks(hip):
     kernel = hip.compile(capi.KIND_APPLY, "f32", "(x * 2.0)", ("x",))
     a, b = hip.alloc(4096), hip.alloc(4096)
