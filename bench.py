@@ -262,15 +262,19 @@ def first_use(tmp, with_c5):
     module stack, each in a fresh process with an empty compiler cache and again with the cache the
     first process left."""
     env = cold_cache_env(tmp)
+    own = dict(env, CUSTOS_HIP_KERNEL_CACHE_DIR=os.path.join(tmp, "custos_code_objects"))
     out = {"what": "a fresh process each; cold = the ROCm compiler library's cache is empty (temporary HOME), warm = the "
-                   "same again on the cache the cold process left; first_call_ms = custos_hip_expr_compile + the first "
-                   "launch + a wait"}
+                   "same again on the cache the cold process left, code_objects_on_disk = the same again with the library's "
+                   "own cache of code objects (CUSTOS_HIP_KERNEL_CACHE_DIR, off by default) filled by a process before; "
+                   "first_call_ms = custos_hip_expr_compile + the first launch + a wait"}
     for which in ("c1", "c2"):
         entry = {}
-        for state in ("cold", "warm"):
+        for state in ("cold", "warm", "fill", "code_objects_on_disk"):
             try:
                 proc = subprocess.run([sys.executable, os.path.abspath(__file__), "--first-call", which], capture_output=True,
-                                      text=True, timeout=120, env=env)
+                                      text=True, timeout=120, env=own if state in ("fill", "code_objects_on_disk") else env)
+                if state == "fill":
+                    continue
                 entry[state] = json.loads(proc.stdout.strip().splitlines()[-1]) if proc.returncode == 0 else {"error": proc.stderr[-300:]}
             except (subprocess.TimeoutExpired, ValueError, IndexError) as e:
                 entry[state] = {"error": str(e)[-300:]}
@@ -278,8 +282,10 @@ def first_use(tmp, with_c5):
     if with_c5:
         for fuse in (False, True):
             entry = {}
-            for state in ("cold", "warm"):
-                r = module_stack("c5", 1, 0, fuse=fuse, settle_ms=0, env=env)
+            for state in ("cold", "warm", "fill", "code_objects_on_disk"):
+                r = module_stack("c5", 1, 0, fuse=fuse, settle_ms=0, env=own if state in ("fill", "code_objects_on_disk") else env)
+                if state == "fill":
+                    continue
                 entry[state] = {"first_run_ms": r.get("first_run_ms"), "kernel_nodes": r.get("kernel_nodes")} if "error" not in r else r
             out["c5_module_stack" + ("_after_elementwise_fusing" if fuse else "")] = entry
     return out

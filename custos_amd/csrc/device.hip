@@ -312,13 +312,30 @@ static int32_t staging_slot_send(custos_hip_device* dev, uint64_t dst, uint64_t 
     return CUSTOS_HIP_OK;
 }
 
-static int32_t staged_write(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes) {
+int32_t staged_write(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes) {
     unsigned char* host = nullptr;
     uint64_t device = 0;
     int32_t rc = staging_slot(dev, dst, &host, &device);
     if (rc != CUSTOS_HIP_OK) return rc;
     std::memcpy(host, src, bytes);
     return staging_slot_send(dev, dst, device, bytes);
+}
+
+// Host data the library itself sends (the operand table of a graph): in stream order through the
+// staging slots when the device has them and the data is small -- the runtime's synchronous copy
+// costs 9 ms the first time a process uses it, more than the rest of a small graph's build --
+// else with that copy.  `src` may be reused when this returns.
+int32_t send_to_device(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes) {
+    constexpr size_t kThroughSlotsMax = 1u << 20;
+    if (!dev->read_stage || bytes > kThroughSlotsMax) {
+        HIP_TRY(dev, hipMemcpy(reinterpret_cast<void*>(dst), src, bytes, hipMemcpyHostToDevice));
+        return CUSTOS_HIP_OK;
+    }
+    for (size_t done = 0; done < bytes; done += kStagedReadMax) {
+        int32_t rc = staged_write(dev, dst + done, static_cast<const unsigned char*>(src) + done, std::min(kStagedReadMax, bytes - done));
+        if (rc != CUSTOS_HIP_OK) return rc;
+    }
+    return CUSTOS_HIP_OK;
 }
 
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec) {

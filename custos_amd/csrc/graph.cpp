@@ -1130,7 +1130,9 @@ int32_t build_graph(custos_hip_device* dev, custos_hip_graph* g) {
 
     if (!host_table.empty()) {
         HIP_TRY(dev, hipMalloc(&g->table, host_table.size() * sizeof(uint64_t)));
-        HIP_TRY(dev, hipMemcpy(g->table, host_table.data(), host_table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
+        // (in stream order on the compute stream, where every launch of the graph follows)
+        int32_t rc = send_to_device(dev, reinterpret_cast<uint64_t>(g->table), host_table.data(), host_table.size() * sizeof(uint64_t));
+        if (rc != CUSTOS_HIP_OK) return rc;
     }
 
     std::vector<std::vector<LoweredNode>> lowered(plan.size());

@@ -275,6 +275,7 @@ inline Tuning tuning_from_c(const custos_hip_tuning* t) {
 
 // device.hip
 hipError_t wait_compute_stream(custos_hip_device* dev);
+int32_t send_to_device(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes);
 hipError_t drain_before_immediate_work(custos_hip_device* dev);
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec);
 unsigned int fill_block();
