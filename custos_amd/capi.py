@@ -106,6 +106,7 @@ PROTOTYPES = {
     "custos_hip_free": (C.c_int32, [_P, C.c_uint64]),
     "custos_hip_write": (C.c_int32, [_P, C.c_uint64, C.c_void_p, C.c_size_t]),
     "custos_hip_read": (C.c_int32, [_P, C.c_void_p, C.c_uint64, C.c_size_t]),
+    "custos_hip_capture_stats": (C.c_int32, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "custos_hip_check_operand_sets": (C.c_int32, [C.POINTER(C.c_uint64), C.c_int32, C.c_size_t, C.c_int32, C.c_uint64]),
     "custos_hip_copy": (C.c_int32, [_P, C.c_uint64, C.c_uint64, C.c_size_t]),
     "custos_hip_clear": (C.c_int32, [_P, C.c_uint64, C.c_size_t]),

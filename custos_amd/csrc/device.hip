@@ -357,6 +357,7 @@ int32_t launch_copy(custos_hip_device* dev, uint64_t dst, uint64_t src, size_t b
     const bool words = ((dst | src | bytes) & 3) == 0;
     if (!words && ((dst ^ src) & 15) != 0) {
         if (dev->capturing) {
+            stop_matching(dev);
             RecNode node;
             node.type = RecNode::Copy;
             node.ptrs = {dst, src};
@@ -382,6 +383,15 @@ int32_t launch_fill(custos_hip_device* dev, uint64_t dptr, size_t bytes, hipStre
     if (head > bytes) head = bytes;
     unsigned long long n_vec = (bytes - head) / 16;
     if (dev->capturing && stream == dev->stream) {
+        if (dev->matching && dev->matched < dev->previous_recorded.size()) {
+            const RecNode& was = dev->previous_recorded[dev->matched];
+            const bool same_pattern = pattern ? was.pattern.size() == 4 && std::memcmp(was.pattern.data(), pattern, 16) == 0 : was.pattern.empty();
+            if (was.type == RecNode::Fill && was.ptrs[0] == dptr && was.bytes == bytes && same_pattern) {
+                dev->matched++;
+                return CUSTOS_HIP_OK;
+            }
+        }
+        stop_matching(dev);
         RecNode node;
         node.type = RecNode::Fill;
         node.ptrs = {dptr};

@@ -1215,6 +1215,26 @@ int32_t replay_graph(custos_hip_device* dev, custos_hip_graph* g) {
     return CUSTOS_HIP_OK;
 }
 
+void stop_matching(custos_hip_device* dev) {
+    if (!dev->matching) return;
+    dev->matching = false;
+    dev->recorded.assign(dev->previous_recorded.begin(), dev->previous_recorded.begin() + static_cast<std::ptrdiff_t>(dev->matched));
+}
+
+// After a graph was built from `recorded`, or found to be the graph of the same recording:
+// the recording is kept for the comparison with the next one (unless it is very long).
+static void keep_recording_of(custos_hip_device* dev, custos_hip_graph* g) {
+    constexpr size_t kKeepUpTo = 1u << 16;
+    if (dev->recorded.size() <= kKeepUpTo) {
+        dev->previous_recorded = std::move(dev->recorded);
+        dev->previous_graph = g;
+    } else {
+        dev->previous_recorded.clear();
+        dev->previous_graph = nullptr;
+    }
+    dev->recorded.clear();
+}
+
 void destroy_graph(custos_hip_graph* g) {
     if (g->exec) (void)hipGraphExecDestroy(g->exec);
     if (g->graph) (void)hipGraphDestroy(g->graph);
@@ -1241,6 +1261,8 @@ int32_t custos_hip_capture_begin(custos_hip_device* dev) {
     dev->recorded.clear();
     dev->capturing = true;
     dev->undrained_at_capture = true;
+    dev->matching = dev->previous_graph != nullptr && !dev->previous_recorded.empty();
+    dev->matched = 0;
     return CUSTOS_HIP_OK;
 }
 
@@ -1250,13 +1272,16 @@ int32_t custos_hip_capture_end(custos_hip_device* dev, custos_hip_graph** graph)
     *graph = nullptr;
     if (!dev->capturing) return set_error(dev, CUSTOS_HIP_ERR_CAPTURE_STATE, "the device is not recording");
     dev->capturing = false;
+    stop_matching(dev);
     custos_hip_graph* g = new custos_hip_graph;
     int32_t rc = build_graph(dev, g);
-    dev->recorded.clear();
     if (rc != CUSTOS_HIP_OK) {
+        dev->recorded.clear();
         destroy_graph(g);
         return rc;
     }
+    keep_recording_of(dev, g);
+    dev->graphs_built++;
     dev->graphs.push_back(g);
     *graph = g;
     return CUSTOS_HIP_OK;
@@ -1271,13 +1296,33 @@ int32_t custos_hip_capture_end_reuse(custos_hip_device* dev, custos_hip_graph* p
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "the previous graph does not belong to this device");
     const std::array<uint64_t, 4> settings = {dev->batching ? 1u : 0u, static_cast<uint64_t>(dev->graph_edges),
                                               dev->direct_replay_max, dev->fusing ? 1u : 0u};
+    // the whole recording repeated, launch for launch, the one `previous` stands for
+    if (previous && dev->matching && dev->previous_graph == previous && dev->matched == dev->previous_recorded.size() &&
+        previous->built_with == settings) {
+        dev->capturing = false;
+        dev->matching = false;
+        dev->reused_while_recording++;
+        *graph = previous;
+        return CUSTOS_HIP_OK;
+    }
+    stop_matching(dev);
     if (previous && previous->built_with == settings && previous->signature == signature(dev->recorded)) {
         dev->capturing = false;
-        dev->recorded.clear();
+        keep_recording_of(dev, previous);
+        dev->reused_by_comparison++;
         *graph = previous;
         return CUSTOS_HIP_OK;
     }
     return custos_hip_capture_end(dev, graph);
+}
+
+int32_t custos_hip_capture_stats(custos_hip_device* dev, uint64_t* reused_while_recording, uint64_t* reused_by_comparison,
+                                 uint64_t* built) {
+    REQUIRE_DEV(dev);
+    if (reused_while_recording) *reused_while_recording = dev->reused_while_recording;
+    if (reused_by_comparison) *reused_by_comparison = dev->reused_by_comparison;
+    if (built) *built = dev->graphs_built;
+    return CUSTOS_HIP_OK;
 }
 
 int32_t custos_hip_set_graph_batching(custos_hip_device* dev, int32_t enabled) {
@@ -1380,6 +1425,10 @@ int32_t custos_hip_graph_destroy(custos_hip_device* dev, custos_hip_graph* graph
     auto it = std::find(dev->graphs.begin(), dev->graphs.end(), graph);
     if (it == dev->graphs.end()) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "graph does not belong to this device");
     dev->graphs.erase(it);
+    if (dev->previous_graph == graph) {
+        dev->previous_graph = nullptr;
+        dev->previous_recorded.clear();
+    }
     if (dev->graph_since_wait == graph) {
         dev->graph_since_wait = nullptr;
         dev->launches_since_wait = true;  // the pending work is no longer that of one known graph

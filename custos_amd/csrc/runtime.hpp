@@ -165,6 +165,17 @@ struct custos_hip_device {
     std::string arch;
     custos_hip::Tuning tuning;
     bool capturing = false;          // recording: launches, clears and copies go to `recorded`
+    // A caller that records the same program before every run (the reference's Lazy module does,
+    // src/modules/lazy.rs:190-197): the recording `previous_graph` was built from is kept, and while
+    // a new recording repeats it launch for launch (`matching`, `matched` launches so far) nothing
+    // is stored; the first launch that differs copies the part that matched into `recorded` and
+    // recording goes on as usual.  custos_hip_capture_end_reuse then hands `previous_graph` back
+    // without comparing anything when the whole recording matched.
+    std::vector<RecNode> previous_recorded;
+    custos_hip_graph* previous_graph = nullptr;
+    bool matching = false;
+    size_t matched = 0;
+    uint64_t reused_while_recording = 0, reused_by_comparison = 0, graphs_built = 0;  // how recordings ended (custos_hip_capture_stats)
     bool undrained_at_capture = false;  // work was (possibly) in flight on the compute stream when the recording
                                         // began and nothing has waited for it since (drain_before_immediate_work)
     int32_t literal_policy = 0;      // CUSTOS_HIP_LITERALS_*
@@ -275,6 +286,23 @@ inline Tuning tuning_from_c(const custos_hip_tuning* t) {
 
 // device.hip
 hipError_t wait_compute_stream(custos_hip_device* dev);
+// Ends the comparison with the previous recording (see custos_hip_device::matching): what matched
+// so far becomes the beginning of `recorded`.  Called before anything is appended to `recorded`.
+void stop_matching(custos_hip_device* dev);
+// While the device compares: whether this launch is the next one of the previous recording (then
+// it is counted and nothing else has to be done for it).
+inline bool repeats_previous_launch(custos_hip_device* dev, const custos_hip_kernel* k, const uint64_t* ins, int n_ins, uint64_t out,
+                                    size_t n) {
+    if (dev->matched >= dev->previous_recorded.size()) return false;
+    const RecNode& was = dev->previous_recorded[dev->matched];
+    if (was.type != RecNode::Kernel || was.k != k || was.n != n || was.ptrs.size() != static_cast<size_t>(n_ins) + 1 ||
+        was.ptrs[static_cast<size_t>(n_ins)] != out)
+        return false;
+    for (int i = 0; i < n_ins; i++)
+        if (was.ptrs[static_cast<size_t>(i)] != ins[i]) return false;
+    dev->matched++;
+    return true;
+}
 int32_t send_to_device(custos_hip_device* dev, uint64_t dst, const void* src, size_t bytes);
 hipError_t drain_before_immediate_work(custos_hip_device* dev);
 unsigned int fill_grid(custos_hip_device* dev, unsigned long long n_vec);

@@ -375,6 +375,13 @@ class HIP:
             return previous
         return Graph(self, g)
 
+    def capture_stats(self):
+        """(recordings that repeated the one before and were recognised while recording, recordings
+        recognised by comparison afterwards, graphs built)."""
+        a, b, c = C.c_uint64(), C.c_uint64(), C.c_uint64()
+        self._check(self.lib.custos_hip_capture_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
     def set_graph_batching(self, enabled: bool) -> None:
         self._check(self.lib.custos_hip_set_graph_batching(self.handle, 1 if enabled else 0))
 

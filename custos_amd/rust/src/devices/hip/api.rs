@@ -88,6 +88,8 @@ extern "C" {
     pub fn custos_hip_preferred_shape_of(footprint_bytes: u64, n_operands: i32, n_written: i32, working_set_bytes: u64,
                                          revisits: i32, unroll: *mut i32, nontemporal: *mut i32, alternate: *mut i32,
                                          block_threads: *mut i32) -> i32;
+    pub fn custos_hip_capture_stats(dev: *mut HipDeviceHandle, reused_while_recording: *mut u64, reused_by_comparison: *mut u64,
+                                    built: *mut u64) -> i32;
     pub fn custos_hip_check_operand_sets(operands: *const u64, operands_per_set: i32, n_sets: usize, written: i32, bytes: u64) -> i32;
     pub fn custos_hip_set_graph_fusing(dev: *mut HipDeviceHandle, enabled: i32) -> i32;
     pub fn custos_hip_graph_node_kernel(graph: *mut HipGraph, node: usize, name: *mut *const c_char) -> i32;

@@ -23,6 +23,11 @@
 //   c4  eager `apply_fn(|x| exp(x*0.5)*x + x*x)` on `HIP<Base>` over 2^28 f16
 //   c5  1024 buffers of 4096 f32: t = a*b; u = t+c; y = sqrt(abs(u))*0.3, recorded once, run
 //       again and again; `--fuse` also calls `elementwise_fusing` first
+//       `--rerecord`: the call sequence of the reference's unmodified `Lazy` module on this device
+//       (src/modules/lazy.rs:190-197 calls every recorded operation again before each run, and the
+//       device's `LazyRun::run` follows: custos_hip_capture_end_reuse, custos_hip_graph_launch,
+//       custos_hip_capture_begin), straight through the C ABI: 3072 recorded launches per run, the
+//       graph of the run before handed back because the recording is the same
 //
 // Two figures per configuration, both on the host clock.  `us_per_run`: `steps` steps in a row and one
 // wait for the device at the end, divided by `steps`: what a loop of runs costs when nothing looks at
@@ -40,6 +45,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <stdexcept>
 #include <string>
 #include <vector>
 
@@ -156,7 +162,7 @@ int main(int argc, char** argv) {
     std::string config = "c2", dump_path, input, input2, stack = "eager";
     int log2n = 0, steps = 100, warmup = 20, settle_ms = 150;
     size_t dump_count = 0;
-    bool fuse = false;
+    bool fuse = false, rerecord = false;
     for (int i = 1; i < argc; i++) {
         const std::string a = argv[i];
         auto value = [&]() -> const char* {
@@ -175,6 +181,7 @@ int main(int argc, char** argv) {
         else if (a == "--input") input = value();
         else if (a == "--input2") input2 = value();
         else if (a == "--fuse") fuse = true;
+        else if (a == "--rerecord") rerecord = true;
         else if (a == "--dump") {
             dump_count = static_cast<size_t>(std::atoll(value()));
             dump_path = value();
@@ -339,6 +346,67 @@ int main(int argc, char** argv) {
             std::printf("{\"config\": \"c4\", \"stack\": \"HIP<Base>\", \"calls\": \"per step: apply_fn(exp(x*0.5)*x + x*x), f16\", "
                         "\"elements\": %zu, \"warmup\": %d, %s}\n",
                         n, warmup, timing_json(t, 4.0 * static_cast<double>(n)).c_str());
+        } else if (config == "c5" && rerecord) {
+            const size_t nbuf = 1024, m = 4096;
+            custos_hip_device* dev = nullptr;
+            auto check = [&](int32_t rc) {
+                if (rc != 0) throw std::runtime_error(custos_hip_last_error(dev));
+            };
+            check(custos_hip_device_create(0, &dev));
+            auto compile = [&](const char* src, std::vector<const char*> markers) {
+                custos_hip_kernel* k = nullptr;
+                check(custos_hip_expr_compile(dev, CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, src, markers.data(),
+                                              static_cast<int32_t>(markers.size()), &k));
+                return k;
+            };
+            custos_hip_kernel* kmul = compile("(x * y)", {"x", "y"});
+            custos_hip_kernel* kadd = compile("(x + y)", {"x", "y"});
+            custos_hip_kernel* kun = compile("(sqrt(abs(x)) * 0.3)", {"x"});
+            std::vector<uint64_t> a(nbuf), b(nbuf), c(nbuf), t(nbuf), u(nbuf), y(nbuf);
+            for (size_t i = 0; i < nbuf; i++) {
+                for (auto* v : {&a, &b, &c, &t, &u, &y}) check(custos_hip_alloc(dev, m * sizeof(float), CUSTOS_HIP_ALLOC_ZEROED, &(*v)[i]));
+                const auto ha = uniform_f32(1, m, 0.f, 1.f, i * m), hb = uniform_f32(2, m, 0.f, 1.f, i * m), hc = uniform_f32(3, m, 0.f, 1.f, i * m);
+                check(custos_hip_write(dev, a[i], ha.data(), m * sizeof(float)));
+                check(custos_hip_write(dev, b[i], hb.data(), m * sizeof(float)));
+                check(custos_hip_write(dev, c[i], hc.data(), m * sizeof(float)));
+            }
+            custos_hip_graph* graph = nullptr;
+            uint64_t builds = 0;
+            check(custos_hip_capture_begin(dev));  // LazySetup::lazy_setup
+            auto run = [&] {
+                for (size_t i = 0; i < nbuf; i++) {  // Lazy::run calls every recorded operation
+                    check(custos_hip_apply_fn2(dev, kmul, a[i], b[i], t[i], m));
+                    check(custos_hip_apply_fn2(dev, kadd, t[i], c[i], u[i], m));
+                    check(custos_hip_apply_fn(dev, kun, u[i], y[i], m));
+                }
+                custos_hip_graph* now = nullptr;  // LazyRun::run of the device
+                check(custos_hip_capture_end_reuse(dev, graph, &now));
+                if (now != graph) {
+                    if (graph) check(custos_hip_graph_destroy(dev, graph));
+                    graph = now;
+                    builds++;
+                }
+                check(custos_hip_graph_launch(dev, graph));
+                check(custos_hip_capture_begin(dev));
+            };
+            const auto first = Clock::now();
+            run();
+            check(custos_hip_sync(dev));
+            const double first_run_ms = us_since(first) * 1e-3;
+            const Timing tm = time_runs(run, [&] { check(custos_hip_sync(dev)); }, warmup, steps, settle_ms);
+            if (dump_count) {
+                std::vector<float> firsts(std::min(dump_count, m));
+                check(custos_hip_read(dev, firsts.data(), y[0], firsts.size() * sizeof(float)));
+                write_file(dump_path, firsts.data(), firsts.size() * sizeof(float));
+            }
+            size_t kernel_nodes = 0;
+            check(custos_hip_graph_node_count(graph, &kernel_nodes));
+            std::printf("{\"config\": \"c5\", \"stack\": \"C ABI in the order of the reference's Lazy module\", \"calls\": \"per run: 1024 x "
+                        "(apply_fn2, apply_fn2, apply_fn) recorded again, capture_end_reuse, graph_launch, capture_begin\", \"elements\": %zu, "
+                        "\"warmup\": %d, %s, \"first_run_ms\": %.2f, \"kernel_nodes\": %zu, \"graph_builds\": %llu}\n",
+                        nbuf * m, warmup, timing_json(tm, 16.0 * static_cast<double>(nbuf * m)).c_str(), first_run_ms, kernel_nodes,
+                        static_cast<unsigned long long>(builds));
+            check(custos_hip_device_destroy(dev));
         } else if (config == "c5") {
             const size_t nbuf = 1024, m = 4096;
             Dev device(0);

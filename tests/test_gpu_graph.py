@@ -558,6 +558,108 @@ def test_lazy_run_sequence_of_an_unmodified_lazy_module(hip, oracle):
     graph.destroy()
 
 
+def test_a_recording_that_repeats_the_one_before_and_then_does_not(hip, oracle):
+    """A recording that repeats the previous one launch for launch is compared while it is made and
+    stores nothing; where it stops repeating -- another operand in the middle, fewer launches, more
+    launches, a clear or a copy between them, the graph of the previous run destroyed -- it becomes an
+    ordinary recording with the part that matched in front.  Every variation against the CPU oracle."""
+    n, k = 3000, 12
+    f = lambda p, q: p.mul(q).add(0.5)
+    g = lambda v: v.abs().sqrt()
+    xs = [synth.uniform_f32(600 + i, n, -2, 2) for i in range(k + 1)]
+    a = [hip.buffer(x) for x in xs]
+    t = [hip.alloc(n) for _ in range(k)]
+    y = [hip.alloc(n) for _ in range(k)]
+
+    def record(pairs, extra=None):
+        """t[i] = f(a[i], a[j]); y[i] = g(t[i]) for (i, j) in pairs; `extra(i)` may record something in between."""
+        for i, j in pairs:
+            hip.apply_fn2(a[i], a[j], f, out=t[i])
+            if extra:
+                extra(i)
+            hip.apply_fn(t[i], g, out=y[i])
+
+    def check(pairs, cleared=(), filled={}):
+        hip.sync()
+        for i, j in pairs:
+            want_t = oracle.apply_fn(f, xs[i], xs[j])
+            assert_bits_equal(t[i].read(), want_t, f"t[{i}]")
+            want_y = np.zeros(n, dtype=np.float32) if i in cleared else oracle.apply_fn(g, want_t)
+            if i in filled:
+                want_y = np.broadcast_to(np.asarray(filled[i], dtype=np.float32), (n,))
+            assert_bits_equal(y[i].read(), want_y, f"y[{i}]")
+
+    zeros = np.zeros(n, dtype=np.float32)
+
+    def reset():
+        for b in t + y:
+            b.write(zeros)                              # (a write executes at once; a clear would be recorded)
+
+    same = [(i, i + 1) for i in range(k)]
+    hip.capture_begin()
+    try:
+        record(same)
+        graph = hip.capture_end_reuse(None)
+        graph.launch()
+        hip.capture_begin()
+        check(same)
+        builds = 1
+        def run(pairs, expect_same, extra=None, cleared=(), filled={}):
+            nonlocal graph, builds
+            reset()
+            before = hip.capture_stats()
+            record(pairs, extra)
+            new = hip.capture_end_reuse(graph)
+            assert (new is graph) == expect_same, (pairs, expect_same)
+            after = hip.capture_stats()
+            # a repeated recording is recognised while it is made, a new one builds a graph
+            assert (after[0] - before[0], after[1] - before[1], after[2] - before[2]) == ((1, 0, 0) if expect_same else (0, 0, 1))
+            if new is not graph:
+                graph.destroy()
+                graph = new
+                builds += 1
+            graph.launch()
+            hip.capture_begin()
+            check(pairs, cleared, filled)
+        run(same, True)
+        run(same, True)
+        middle = [(i, (i + 2) % (k + 1)) if i == 5 else (i, i + 1) for i in range(k)]
+        run(middle, False)                              # another operand in launch 10 of 24
+        run(middle, True)
+        run(same, False)
+        run(same[:7], False)                            # stops early
+        run(same[:7], True)
+        run(same, False)                                # goes on after the previous one ended
+        run(same, True)
+        # a recorded clear of y[2] between the two launches of buffer 3: it follows the launch that wrote y[2]
+        run(same, False, extra=lambda i: y[2].clear() if i == 3 else None, cleared=(2,))
+        run(same, True, extra=lambda i: y[2].clear() if i == 3 else None, cleared=(2,))
+        run(same, False, extra=lambda i: y[1].clear() if i == 3 else None, cleared=(1,))     # another buffer cleared
+        run(same, False, extra=lambda i: hip.fill(y[1], 2.5) if i == 3 else None, filled={1: 2.5})   # another value
+        run(same, True, extra=lambda i: hip.fill(y[1], 2.5) if i == 3 else None, filled={1: 2.5})
+        # a recorded copy is compared like a launch (it is one, of the identity kernel)
+        run(same, False, extra=lambda i: hip.copy(y[0], a[4]) if i == 3 else None, filled={0: xs[4]})
+        run(same, True, extra=lambda i: hip.copy(y[0], a[4]) if i == 3 else None, filled={0: xs[4]})
+        run(same, False)
+        # the first launch already differs
+        other = [(0, 2)] + same[1:]
+        run(other, False)
+        # the graph of the run before is gone: the next recording is compared with nothing
+        graph.destroy()
+        graph = None
+        reset()
+        record(same)
+        graph = hip.capture_end_reuse(None)
+        graph.launch()
+        hip.capture_begin()
+        check(same)
+        run(same, True)
+    finally:
+        hip.capture_end().destroy()
+    if graph is not None:
+        graph.destroy()
+
+
 def test_recording_begins_without_a_wait_and_immediate_work_takes_it(hip):
     """The same sequence with the run's wait deferred: the graph is launched, the next recording begins
     while it is still running, and what executes at once during a recording (a read, a write, an
