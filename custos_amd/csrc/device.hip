@@ -585,6 +585,7 @@ int32_t custos_hip_sync(custos_hip_device* dev) {
 int32_t custos_hip_set_tuning(custos_hip_device* dev, const custos_hip_tuning* tuning) {
     REQUIRE_DEV(dev);
     dev->tuning = tuning_from_c(tuning);
+    dev->compile_epoch++;
     return CUSTOS_HIP_OK;
 }
 

@@ -371,6 +371,23 @@ extern "C" {
 int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dtype, const char* src,
                                 const char* const* markers, int32_t n_markers,
                                 custos_hip_kernel** kernel) {
+    // A recording that repeats the one before (custos_hip_device::matching) asks for the kernel of its
+    // next launch again, under the same settings: the handle that launch was recorded with answers,
+    // by a comparison of the text alone.
+    if (dev && kernel && src && markers && dev->capturing && dev->matching && dev->matched < dev->previous_recorded.size()) {
+        custos_hip_kernel* expected = dev->previous_recorded[dev->matched].k;
+        if (expected && expected->request_epoch == dev->compile_epoch && expected->request_kind == kind &&
+            expected->request_dtype == dtype && expected->markers.size() == static_cast<size_t>(n_markers) &&
+            std::strcmp(expected->expr_src.c_str(), src) == 0) {
+            bool same = true;
+            for (int i = 0; same && i < n_markers; i++) same = markers[i] && expected->markers[static_cast<size_t>(i)] == markers[i];
+            if (same) {
+                dev->hits++;
+                *kernel = expected;
+                return CUSTOS_HIP_OK;
+            }
+        }
+    }
     REQUIRE_DEV(dev);
     if (!kernel) return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "kernel out pointer is null");
     *kernel = nullptr;
@@ -386,6 +403,7 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
         if (known != dev->by_text.end()) {
             dev->hits++;
             *kernel = known->second;
+            known->second->request_kind = kind, known->second->request_dtype = dtype, known->second->request_epoch = dev->compile_epoch;
             return CUSTOS_HIP_OK;
         }
     }
@@ -395,6 +413,7 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
     int32_t rc = compile_expr(dev, kind, dtype, src, markers, n_markers, tuning, &k);
     if (rc != CUSTOS_HIP_OK) return rc;
     *kernel = k;
+    k->request_kind = kind, k->request_dtype = dtype, k->request_epoch = dev->compile_epoch;
     dev->by_text.emplace(std::move(text_key), k);
     return CUSTOS_HIP_OK;
 }
@@ -496,6 +515,7 @@ int32_t custos_hip_set_eq_policy(custos_hip_device* dev, int32_t policy) {
     if (policy != CUSTOS_HIP_EQ_EXACT && policy != CUSTOS_HIP_EQ_AS_CPU_EVAL)
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown eq policy");
     dev->eq_as_cpu_eval = policy == CUSTOS_HIP_EQ_AS_CPU_EVAL;
+    dev->compile_epoch++;
     return CUSTOS_HIP_OK;
 }
 
@@ -506,6 +526,7 @@ int32_t custos_hip_set_literal_policy(custos_hip_device* dev, int32_t policy) {
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "unknown literal policy");
     dev->literal_policy = policy;
     dev->by_text.clear();  // the same text may now map to another kernel
+    dev->compile_epoch++;
     return CUSTOS_HIP_OK;
 }
 

@@ -27,6 +27,10 @@ struct custos_hip_kernel {
     hipModule_t modules[custos_hip::kEntrySets] = {nullptr, nullptr, nullptr};
     hipFunction_t fns[custos_hip::kEntrySets] = {nullptr, nullptr, nullptr};
     std::string expr_src;  // the expression as the caller spelt it
+    // the request custos_hip_expr_compile answered with this handle last (kind, dtype, and the device's
+    // compile settings then, by their epoch): a recording that repeats the one before asks again
+    int32_t request_kind = -1, request_dtype = -1;
+    uint64_t request_epoch = ~0ull;
     std::vector<std::string> markers;
     // Handles for the same code with other values of the literal parameters, by those
     // values: they share this kernel's modules (their own stay null) and differ
@@ -248,6 +252,7 @@ struct custos_hip_device {
     // a repeated call is answered without parsing (what the (source, name) map of
     // src/devices/cuda/kernel_cache.rs:45-49 does for the reference)
     std::unordered_map<std::string, custos_hip_kernel*> by_text;
+    uint64_t compile_epoch = 0;  // advanced by every setting that changes what a text compiles to (tuning, eq and literal policy)
     std::vector<custos_hip_graph*> graphs;
 };
 

@@ -353,15 +353,12 @@ int main(int argc, char** argv) {
                 if (rc != 0) throw std::runtime_error(custos_hip_last_error(dev));
             };
             check(custos_hip_device_create(0, &dev));
-            auto compile = [&](const char* src, std::vector<const char*> markers) {
+            static const char* const kXY[] = {"x", "y"};
+            auto compile = [&](const char* src, int32_t n_markers) {
                 custos_hip_kernel* k = nullptr;
-                check(custos_hip_expr_compile(dev, CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, src, markers.data(),
-                                              static_cast<int32_t>(markers.size()), &k));
+                check(custos_hip_expr_compile(dev, CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, src, kXY, n_markers, &k));
                 return k;
             };
-            custos_hip_kernel* kmul = compile("(x * y)", {"x", "y"});
-            custos_hip_kernel* kadd = compile("(x + y)", {"x", "y"});
-            custos_hip_kernel* kun = compile("(sqrt(abs(x)) * 0.3)", {"x"});
             std::vector<uint64_t> a(nbuf), b(nbuf), c(nbuf), t(nbuf), u(nbuf), y(nbuf);
             for (size_t i = 0; i < nbuf; i++) {
                 for (auto* v : {&a, &b, &c, &t, &u, &y}) check(custos_hip_alloc(dev, m * sizeof(float), CUSTOS_HIP_ALLOC_ZEROED, &(*v)[i]));
@@ -374,10 +371,12 @@ int main(int argc, char** argv) {
             uint64_t builds = 0;
             check(custos_hip_capture_begin(dev));  // LazySetup::lazy_setup
             auto run = [&] {
-                for (size_t i = 0; i < nbuf; i++) {  // Lazy::run calls every recorded operation
-                    check(custos_hip_apply_fn2(dev, kmul, a[i], b[i], t[i], m));
-                    check(custos_hip_apply_fn2(dev, kadd, t[i], c[i], u[i], m));
-                    check(custos_hip_apply_fn(dev, kun, u[i], y[i], m));
+                // Lazy::run calls every recorded operation; each asks for its kernel by the text of its
+                // expression and launches it (src/devices/cuda/ops.rs:144-177 formats and looks up per call too)
+                for (size_t i = 0; i < nbuf; i++) {
+                    check(custos_hip_apply_fn2(dev, compile("(x * y)", 2), a[i], b[i], t[i], m));
+                    check(custos_hip_apply_fn2(dev, compile("(x + y)", 2), t[i], c[i], u[i], m));
+                    check(custos_hip_apply_fn(dev, compile("(sqrt(abs(x)) * 0.3)", 1), u[i], y[i], m));
                 }
                 custos_hip_graph* now = nullptr;  // LazyRun::run of the device
                 check(custos_hip_capture_end_reuse(dev, graph, &now));
@@ -402,7 +401,7 @@ int main(int argc, char** argv) {
             size_t kernel_nodes = 0;
             check(custos_hip_graph_node_count(graph, &kernel_nodes));
             std::printf("{\"config\": \"c5\", \"stack\": \"C ABI in the order of the reference's Lazy module\", \"calls\": \"per run: 1024 x "
-                        "(apply_fn2, apply_fn2, apply_fn) recorded again, capture_end_reuse, graph_launch, capture_begin\", \"elements\": %zu, "
+                        "(expr_compile + apply_fn2, expr_compile + apply_fn2, expr_compile + apply_fn) again, capture_end_reuse, graph_launch, capture_begin\", \"elements\": %zu, "
                         "\"warmup\": %d, %s, \"first_run_ms\": %.2f, \"kernel_nodes\": %zu, \"graph_builds\": %llu}\n",
                         nbuf * m, warmup, timing_json(tm, 16.0 * static_cast<double>(nbuf * m)).c_str(), first_run_ms, kernel_nodes,
                         static_cast<unsigned long long>(builds));
