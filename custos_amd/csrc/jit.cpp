@@ -394,9 +394,14 @@ int32_t custos_hip_expr_compile(custos_hip_device* dev, int32_t kind, int32_t dt
     std::string text_key;
     if (src && markers && n_markers >= 1 && n_markers <= 4) {
         const Tuning& t = dev->tuning;
-        text_key = std::to_string(kind) + "," + std::to_string(dtype) + "," + std::to_string(t.block_threads) + "," +
-                   std::to_string(t.unroll) + "," + std::to_string(t.blocks_per_cu) + "," + std::to_string(t.nontemporal) +
-                   (dev->eq_as_cpu_eval ? ",le" : "");
+        // (the settings as raw bytes, then the markers and the text: one allocation)
+        size_t length = 6 * sizeof(int32_t) + 2 + std::strlen(src);
+        for (int i = 0; i < n_markers; i++) length += 1 + (markers[i] ? std::strlen(markers[i]) : 0);
+        text_key.reserve(length);
+        for (int32_t v : {kind, dtype, static_cast<int32_t>(t.block_threads), static_cast<int32_t>(t.unroll),
+                          static_cast<int32_t>(t.blocks_per_cu), static_cast<int32_t>(t.nontemporal)})
+            text_key.append(reinterpret_cast<const char*>(&v), sizeof v);
+        text_key.push_back(dev->eq_as_cpu_eval ? 'l' : 'e');
         for (int i = 0; i < n_markers; i++) text_key.append(1, '\x1f').append(markers[i] ? markers[i] : "");
         text_key.append(1, '\x1e').append(src);
         auto known = dev->by_text.find(text_key);

@@ -566,6 +566,91 @@ TEST_CASE(hip_apply_fn_many_noalloc) {
     CHECK_EQ(custos_hip_apply_fn_many_noalloc(dev, k, too_many.data(), 2, 10, 16), static_cast<int32_t>(CUSTOS_HIP_ERR_ARITY_MISMATCH));
 }
 
+// The call sequence of a device under the reference's own Lazy module (src/modules/lazy.rs:190-197:
+// every recorded operation is called again before each run; each asks for its kernel by text and
+// launches it), through the C ABI: a recording that repeats the one before is recognised as it is
+// made, one that stops repeating (another operand, fewer or more operations, a clear in between)
+// becomes an ordinary recording, and every run leaves what the same calls issued eagerly leave.
+TEST_CASE(hip_program_recorded_again_before_every_run) {
+    HIP<Base> device;
+    custos_hip_device* dev = device.handle();
+    const size_t n = 2000, nbuf = 9;
+    const char* xy[] = {"x", "y"};
+    std::vector<Buffer<float, HIP<Base>>> a, t, y, te, ye;
+    for (size_t i = 0; i <= nbuf; i++) {
+        std::vector<float> v(n);
+        for (size_t e = 0; e < n; e++) v[e] = 0.25f * static_cast<float>((e * 5 + i * 11) % 23) - 2.f;
+        a.push_back(device.buffer(v));
+    }
+    for (size_t i = 0; i < nbuf; i++) {
+        t.push_back(device.new_buffer<float>(n)), y.push_back(device.new_buffer<float>(n));
+        te.push_back(device.new_buffer<float>(n)), ye.push_back(device.new_buffer<float>(n));
+    }
+    struct Step {
+        size_t i, j;
+        int clear_y = -1;  // index of a y buffer cleared between the two launches of the step, or -1
+    };
+    auto issue = [&](const std::vector<Step>& program, std::vector<Buffer<float, HIP<Base>>>& ts, std::vector<Buffer<float, HIP<Base>>>& ys) {
+        for (const Step& s : program) {
+            custos_hip_kernel* k = nullptr;
+            CHECK_EQ(custos_hip_expr_compile(dev, CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, "((x * y) + 0.5)", xy, 2, &k), 0);
+            CHECK_EQ(custos_hip_apply_fn2(dev, k, a[s.i].ptr(), a[s.j].ptr(), ts[s.i].ptr(), n), 0);
+            if (s.clear_y >= 0) CHECK_EQ(custos_hip_clear(dev, ys[static_cast<size_t>(s.clear_y)].ptr(), n * sizeof(float)), 0);
+            CHECK_EQ(custos_hip_expr_compile(dev, CUSTOS_HIP_KIND_APPLY, CUSTOS_HIP_F32, "sqrt(abs(x))", xy, 1, &k), 0);
+            CHECK_EQ(custos_hip_apply_fn(dev, k, ts[s.i].ptr(), ys[s.i].ptr(), n), 0);
+        }
+    };
+    std::vector<Step> same, middle, shorter, cleared;
+    for (size_t i = 0; i < nbuf; i++) same.push_back({i, i + 1});
+    middle = same, middle[4].j = 0;
+    shorter.assign(same.begin(), same.begin() + 5);
+    cleared = same, cleared[6].clear_y = 2;
+    custos_hip_graph* graph = nullptr;
+    const std::vector<float> zeros(n, 0.f);
+    auto run = [&](const std::vector<Step>& program, bool expect_same) {
+        for (size_t i = 0; i < nbuf; i++) {
+            // (writes execute at once while the device records; a clear would be recorded)
+            for (auto* buffers : {&t, &y, &te, &ye}) CHECK_EQ(custos_hip_write(dev, (*buffers)[i].ptr(), zeros.data(), n * sizeof(float)), 0);
+        }
+        uint64_t before[3], after[3];
+        CHECK_EQ(custos_hip_capture_stats(dev, &before[0], &before[1], &before[2]), 0);
+        issue(program, t, y);
+        custos_hip_graph* now = nullptr;
+        CHECK_EQ(custos_hip_capture_end_reuse(dev, graph, &now), 0);
+        CHECK_EQ(now == graph, expect_same);
+        CHECK_EQ(custos_hip_capture_stats(dev, &after[0], &after[1], &after[2]), 0);
+        CHECK_EQ(after[0] - before[0], expect_same ? 1u : 0u);
+        CHECK_EQ(after[2] - before[2], expect_same ? 0u : 1u);
+        if (now != graph) {
+            if (graph) CHECK_EQ(custos_hip_graph_destroy(dev, graph), 0);
+            graph = now;
+        }
+        CHECK_EQ(custos_hip_graph_launch(dev, graph), 0);
+        issue(program, te, ye);  // the same calls, eagerly
+        CHECK_EQ(custos_hip_capture_begin(dev), 0);
+        for (size_t i = 0; i < nbuf; i++) {
+            CHECK_VEC_EQ(t[i].read(), te[i].read());
+            CHECK_VEC_EQ(y[i].read(), ye[i].read());
+        }
+    };
+    CHECK_EQ(custos_hip_capture_begin(dev), 0);
+    run(same, false);
+    run(same, true);
+    run(same, true);
+    run(middle, false);
+    run(middle, true);
+    run(shorter, false);
+    run(shorter, true);
+    run(same, false);
+    run(cleared, false);
+    run(cleared, true);
+    run(same, false);
+    custos_hip_graph* last = nullptr;
+    CHECK_EQ(custos_hip_capture_end(dev, &last), 0);
+    CHECK_EQ(custos_hip_graph_destroy(dev, last), 0);
+    CHECK_EQ(custos_hip_graph_destroy(dev, graph), 0);
+}
+
 // Random programs of apply and gradient launches over whole buffers and half views, through the C
 // ABI: the replayed graph (producers joined into their consumers, equal launches merged) leaves every
 // buffer exactly as the same calls issued one by one do, replay after replay; with joining switched
