@@ -2,6 +2,7 @@
 // into scalar head / 16-byte vectors / scalar tail, and recording while the
 // device records (include/custos_hip.h).
 #include <algorithm>
+#include <cstring>
 
 #include "runtime.hpp"
 
@@ -307,6 +308,20 @@ int32_t custos_hip_source_launch(custos_hip_device* dev, custos_hip_kernel* kern
     if (static_cast<uint64_t>(block[0]) * block[1] * block[2] > 1024)
         return set_error(dev, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "more than 1024 threads per workgroup");
     if (dev->capturing) {
+        if (dev->matching && dev->matched < dev->previous_recorded.size()) {
+            const RecNode& was = dev->previous_recorded[dev->matched];
+            bool same = was.type == RecNode::Source && was.k == kernel && was.shared_mem == shared_mem_bytes &&
+                        was.arg_values.size() == static_cast<size_t>(n_params);
+            for (int i = 0; same && i < 3; i++) same = was.grid3[i] == grid[i] && was.block3[i] == block[i];
+            for (int i = 0; same && i < n_params; i++) {
+                const auto& value = was.arg_values[static_cast<size_t>(i)];
+                same = params[i] && value.size() == param_sizes[i] && std::memcmp(value.data(), params[i], param_sizes[i]) == 0;
+            }
+            if (same) {
+                dev->matched++;
+                return CUSTOS_HIP_OK;
+            }
+        }
         stop_matching(dev);
         RecNode node;
         node.type = RecNode::Source;

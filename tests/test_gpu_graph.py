@@ -640,6 +640,18 @@ def test_a_recording_that_repeats_the_one_before_and_then_does_not(hip, oracle):
         # a recorded copy is compared like a launch (it is one, of the identity kernel)
         run(same, False, extra=lambda i: hip.copy(y[0], a[4]) if i == 3 else None, filled={0: xs[4]})
         run(same, True, extra=lambda i: hip.copy(y[0], a[4]) if i == 3 else None, filled={0: xs[4]})
+        # a launch of caller-written source is compared by its kernel, its shape and its argument values
+        scale = '''extern "C" __global__ void scale(float* p, float by, int n) {
+            int i = blockIdx.x * blockDim.x + threadIdx.x;
+            if (i < n) p[i] *= by;
+        }'''
+        def scaled(i, by):
+            if i == 3:
+                hip.launch_kernel1d(n, scale, "scale", [y[0], by, n])
+        y0 = oracle.apply_fn(g, oracle.apply_fn(f, xs[0], xs[1]))
+        run(same, False, extra=lambda i: scaled(i, 2.0), filled={0: y0 * np.float32(2.0)})
+        run(same, True, extra=lambda i: scaled(i, 2.0), filled={0: y0 * np.float32(2.0)})
+        run(same, False, extra=lambda i: scaled(i, 4.0), filled={0: y0 * np.float32(4.0)})    # another argument value
         run(same, False)
         # the first launch already differs
         other = [(0, 2)] + same[1:]
