@@ -645,6 +645,30 @@ TEST_CASE(hip_program_recorded_again_before_every_run) {
     run(cleared, false);
     run(cleared, true);
     run(same, false);
+    // random walks: each program is the one before with one change at a random place (another
+    // operand, a clear put in or taken out, the end cut off, a step appended), or no change
+    uint64_t state = 12345;
+    auto next = [&](uint64_t below) {
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        return (state >> 33) % below;
+    };
+    std::vector<Step> program = same;
+    for (int round = 0; round < 40; round++) {
+        std::vector<Step> changed = program;
+        switch (next(6)) {
+            case 0: break;
+            case 1: changed[next(changed.size())].j = next(nbuf + 1); break;
+            case 2: changed[next(changed.size())].clear_y = static_cast<int>(next(nbuf)); break;
+            case 3: changed[next(changed.size())].clear_y = -1; break;
+            case 4: if (changed.size() > 1) changed.resize(1 + next(changed.size() - 1)); break;
+            default: if (changed.size() < 2 * nbuf) changed.push_back({next(nbuf), next(nbuf + 1)}); break;
+        }
+        bool equal = changed.size() == program.size();
+        for (size_t k = 0; equal && k < changed.size(); k++)
+            equal = changed[k].i == program[k].i && changed[k].j == program[k].j && changed[k].clear_y == program[k].clear_y;
+        run(changed, equal);
+        program = changed;
+    }
     custos_hip_graph* last = nullptr;
     CHECK_EQ(custos_hip_capture_end(dev, &last), 0);
     CHECK_EQ(custos_hip_graph_destroy(dev, last), 0);
