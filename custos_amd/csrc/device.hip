@@ -8,6 +8,7 @@
 #include <thread>
 
 #include "runtime.hpp"
+#include "scratch_order.hpp"
 
 namespace custos_hip {
 
@@ -40,17 +41,12 @@ constexpr size_t kScratchWords = 8192;
 static __device__ __align__(256) unsigned long long scratch[kScratchWords];
 constexpr int kMaxDevices = 64;
 static unsigned long long* g_scratch_ptr[kMaxDevices];
-// All handles on a GPU share that GPU's table, each launching on a stream of its own.  The
-// table's last user and an event recorded behind its launch let the next call through ANOTHER
-// handle order its rewrite of the table behind that launch (calls through one handle are
-// ordered by its stream).  The mutex covers the look-up, and in the entry point everything
-// from the wait to the event record, so that calls from several threads take turns.
+// All handles on a GPU share that GPU's table, each launching on a stream of its own: an event
+// per GPU orders calls through different handles (who waits and who records: ScratchOrder).  The
+// mutex covers the look-up, and in the entry point everything from the wait to the event record,
+// so that calls from several threads take turns.
 static hipEvent_t g_scratch_event[kMaxDevices];
-static const custos_hip_device* g_scratch_last_user[kMaxDevices];
-// Handles alive per GPU.  While a GPU has one handle its stream alone orders the table's users and
-// no event is recorded; when a second handle appears, the event is recorded once behind whatever
-// the last user has launched so far, and from then on behind every launch.
-static int g_scratch_handles[kMaxDevices];
+static ScratchOrder g_scratch_order[kMaxDevices];
 static std::mutex g_scratch_mutex;
 static_assert(kScratchWords * sizeof(unsigned long long) <= kStagedReadMax, "the table travels through one staging slot");
 
@@ -70,10 +66,11 @@ static hipError_t scratch_address(int idx, unsigned long long** out) {
         g_scratch_ptr[idx] = static_cast<unsigned long long*>(p);
     }
     *out = g_scratch_ptr[idx];
-    if (++g_scratch_handles[idx] == 2 && g_scratch_last_user[idx]) {
-        hipError_t e = hipEventRecord(g_scratch_event[idx], g_scratch_last_user[idx]->stream);
+    if (g_scratch_order[idx].handle_created()) {
+        const auto* last_user = static_cast<const custos_hip_device*>(g_scratch_order[idx].last_user);
+        hipError_t e = hipEventRecord(g_scratch_event[idx], last_user->stream);
         if (e != hipSuccess) {
-            g_scratch_handles[idx]--;
+            g_scratch_order[idx].handle_not_created();
             return e;
         }
     }
@@ -528,8 +525,7 @@ int32_t custos_hip_device_destroy(custos_hip_device* dev) {
     if (dev->idx >= 0 && dev->idx < kMaxDevices) {
         // (its launches have finished: the next user of the table need not wait for this handle)
         std::lock_guard<std::mutex> lock(g_scratch_mutex);
-        if (g_scratch_last_user[dev->idx] == dev) g_scratch_last_user[dev->idx] = nullptr;
-        if (dev->scratch_table) g_scratch_handles[dev->idx]--;
+        if (dev->scratch_table) g_scratch_order[dev->idx].handle_destroyed(dev);
     }
     for (custos_hip_graph* g : dev->graphs) destroy_graph(g);
     // every block of this handle goes back to the driver, pooled or still held by the caller
@@ -964,14 +960,14 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     // The launch of another handle may still be reading the table: this stream's work from here
     // on waits for it.  (The launches of this handle are ordered by its stream.)
-    if (g_scratch_last_user[dev->idx] && g_scratch_last_user[dev->idx] != dev)
-        HIP_TRY(dev, hipStreamWaitEvent(dev->stream, g_scratch_event[dev->idx], 0));
+    ScratchOrder& order = g_scratch_order[dev->idx];
+    if (order.must_wait(dev)) HIP_TRY(dev, hipStreamWaitEvent(dev->stream, g_scratch_event[dev->idx], 0));
     // Table rows as the `_batched` entry point reads them (addresses, then the literal
     // parameters), written straight into a pinned staging slot; the library's copy kernel moves
     // them into the table on the compute stream, behind the previous call's launch.  Not needed
     // when the table still holds the rows of an identical call of this handle.
     const uint64_t table_dev = reinterpret_cast<uint64_t>(dev->scratch_table);
-    if (!(dev->noalloc_in_table == known && g_scratch_last_user[dev->idx] == dev)) {
+    if (!(dev->noalloc_in_table == known && order.still_holds_rows_of(dev))) {
         dev->noalloc_in_table = -1;
         unsigned char* slot_host = nullptr;
         uint64_t slot_dev = 0;
@@ -997,8 +993,7 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
     dev->launches_since_wait = true;
     HIP_TRY(dev, hipModuleLaunchKernel(fn, static_cast<unsigned int>(tiles_per_seg * n_sets), 1, 1,
                                        static_cast<unsigned int>(shape.block), 1, 1, 0, dev->stream, args, nullptr));
-    if (g_scratch_handles[dev->idx] > 1) HIP_TRY(dev, hipEventRecord(g_scratch_event[dev->idx], dev->stream));
-    g_scratch_last_user[dev->idx] = dev;
+    if (order.launched(dev)) HIP_TRY(dev, hipEventRecord(g_scratch_event[dev->idx], dev->stream));
     dev->noalloc_in_table = known;
     return CUSTOS_HIP_OK;
 }

@@ -5,6 +5,7 @@
 #include "custos/opt_graph.hpp"
 #include "module_tests.hpp"
 #include "test_cpu_device.hpp"
+#include "../../custos_amd/csrc/scratch_order.hpp"
 
 using namespace custos;
 
@@ -306,3 +307,77 @@ TEST_CASE(half_conversions_round_to_nearest_even) {
 }
 
 int main(int argc, char** argv) { return check::run(argc, argv); }
+
+// ---- the shared operand table of the allocation-free merged launch: who waits for whom ----
+//
+// A model of what the library does with the decisions of ScratchOrder: every handle has a stream
+// (a count of the launches issued on it), the GPU's event remembers the stream and position it
+// was recorded at, a wait makes a stream depend on that position.  Random creations, calls and
+// destructions of up to four handles; before every rewrite of the table, the grid that read the
+// table last must be ordered before the rewriting stream's next work: it ran on the same stream,
+// or that stream waits for an event recorded on the reader's stream at or behind the reader, or
+// the reader's handle was destroyed (which drains its stream first).
+TEST_CASE(scratch_table_order_against_a_model_of_streams) {
+    using custos_hip::ScratchOrder;
+    struct Handle {
+        bool alive = false;
+        uint64_t issued = 0;       // launches issued on its stream
+        uint64_t waits_for[4] = {0, 0, 0, 0};  // per other stream: position this stream has waited for
+    };
+    uint64_t state = 99;
+    auto next = [&](uint64_t below) {
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        return (state >> 33) % below;
+    };
+    for (int trial = 0; trial < 200; trial++) {
+        ScratchOrder order;
+        Handle handles[4];
+        int event_stream = -1;
+        uint64_t event_position = 0;
+        int reader = -1;              // handle whose grid read the table last and may still run
+        uint64_t reader_position = 0;
+        int reuses = 0;
+        for (int step = 0; step < 60; step++) {
+            const size_t h = next(4);
+            Handle& me = handles[h];
+            if (!me.alive) {
+                me = Handle{};
+                me.alive = true;
+                if (order.handle_created()) {
+                    // recorded on the last user's stream, behind everything it has launched
+                    int last = -1;
+                    for (int k = 0; k < 4; k++)
+                        if (order.last_user == &handles[k]) last = k;
+                    CHECK(last >= 0 && handles[last].alive);
+                    event_stream = last, event_position = handles[last].issued;
+                }
+                continue;
+            }
+            if (next(5) == 0) {
+                // destroyed: its stream drains first, so nothing of it is still running
+                if (reader == static_cast<int>(h)) reader = -1;
+                order.handle_destroyed(&me);
+                me.alive = false;
+                continue;
+            }
+            // a call: wait if told to, (maybe) rewrite the table, launch, record if told to
+            if (order.must_wait(&me)) {
+                CHECK(event_stream >= 0);
+                me.waits_for[event_stream] = std::max(me.waits_for[event_stream], event_position);
+            }
+            if (reader >= 0 && reader != static_cast<int>(h))
+                CHECK(me.waits_for[reader] >= reader_position);   // the last reader is ordered before this rewrite
+            if (order.still_holds_rows_of(&me)) {
+                CHECK(reader == static_cast<int>(h) || reader == -1);  // nobody else used the table in between
+                reuses++;
+            }
+            me.issued++;
+            reader = static_cast<int>(h), reader_position = me.issued;
+            if (order.launched(&me)) event_stream = static_cast<int>(h), event_position = me.issued;
+        }
+        int alive = 0;
+        for (const Handle& handle : handles) alive += handle.alive;
+        CHECK_EQ(order.handles, alive);
+        (void)reuses;
+    }
+}
