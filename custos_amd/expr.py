@@ -43,6 +43,11 @@ class Expr:
     def leq(self, rhs): return Node("leq", self, _wrap(rhs))
     def eq(self, rhs): return Node("eq", self, _wrap(rhs))
 
+    def val(self, value):
+        """The literal `value` as a node (`value.to_val()`, src/two_way_ops/resolve.rs:61-79), for a closure
+        that needs one on the left: `v.val(1.0).sub(v.tanh())`."""
+        return Const(value)
+
     # -- unary --
     def sin(self): return Node("sin", self)
     def cos(self): return Node("cos", self)

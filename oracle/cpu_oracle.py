@@ -3,8 +3,10 @@
 Only tests, `__graft_entry__.smoke()` and the `cpu_baseline` leg of `bench.py`
 may import this module; the shipped package never does.  It loads
 `oracle/libcustos_cpu_oracle.so` (built from custos_cpu_oracle.c by
-`make -C oracle`) and translates expression trees built with
-`custos_amd.expr` into the oracle's postfix programs.
+`make -C oracle`) and turns the closure a test passes (`lambda v: v.mul(2.0).add(1.0)`) into the
+oracle's postfix program with a tracer of its own (`Traced`): nothing of the package under test is
+imported here, so a mistake in the package's expression classes (a swapped operand, a wrong node) is
+not shared by the oracle.
 """
 from __future__ import annotations
 
@@ -61,16 +63,75 @@ def lib():
     return _lib
 
 
-def compile_rpn(expr, dtype: str = "f32", eq_mode: str = "eq"):
-    """Expression tree -> postfix program.
+class Traced:
+    """A value inside a closure that is being traced: the postfix program that computes it, as a
+    tuple of (node name, literal or None).  The methods are the reference's `Combiner` methods
+    (src/two_way_ops/combiner.rs:8-116; `sqrt` is the added node): `lhs.op(rhs)` evaluates lhs, then
+    rhs, then the node (src/two_way_ops/ops.rs:15-314), so its program is lhs's, rhs's, the node.
+    `val` makes a literal (`2.0.to_val()`, src/two_way_ops/resolve.rs:61-79) where a closure needs one
+    on the left: `v.val(1.0).sub(v.tanh())`."""
+
+    __slots__ = ("prog",)
+
+    def __init__(self, prog):
+        self.prog = tuple(prog)
+
+    @staticmethod
+    def _operand(v):
+        if isinstance(v, Traced):
+            return v.prog
+        if isinstance(v, (bool, int, float, str, np.integer, np.floating, np.bool_)):
+            return (("const", v),)
+        raise TypeError(f"the oracle cannot trace an operand of type {type(v).__name__}: closures take their literals as "
+                        "numbers or through `v.val(number)`")
+
+    def _two(self, name, rhs):
+        return Traced(self.prog + Traced._operand(rhs) + ((name, None),))
+
+    def _one(self, name):
+        return Traced(self.prog + ((name, None),))
+
+    def val(self, value):
+        return Traced(Traced._operand(value))
+
+    def add(self, rhs): return self._two("add", rhs)
+    def sub(self, rhs): return self._two("sub", rhs)
+    def mul(self, rhs): return self._two("mul", rhs)
+    def div(self, rhs): return self._two("div", rhs)
+    def pow(self, rhs): return self._two("pow", rhs)
+    def min(self, rhs): return self._two("min", rhs)
+    def max(self, rhs): return self._two("max", rhs)
+    def geq(self, rhs): return self._two("geq", rhs)
+    def leq(self, rhs): return self._two("leq", rhs)
+    def eq(self, rhs): return self._two("eq", rhs)
+    def sin(self): return self._one("sin")
+    def cos(self): return self._one("cos")
+    def tan(self): return self._one("tan")
+    def tanh(self): return self._one("tanh")
+    def exp(self): return self._one("exp")
+    def ln(self): return self._one("ln")
+    def abs(self): return self._one("abs")
+    def neg(self): return self._one("neg")
+    def identity(self): return self._one("identity")
+    def sqrt(self): return self._one("sqrt")
+
+
+def trace(f, n_vars=1):
+    """The closure `f` applied to `n_vars` traced operands."""
+    result = f(*[Traced((("var%d" % i, None),)) for i in range(n_vars)])
+    if not isinstance(result, Traced):
+        result = Traced(Traced._operand(result))
+    return result
+
+
+def compile_rpn(traced, dtype: str = "f32", eq_mode: str = "eq"):
+    """Traced closure -> postfix program of the C oracle.
 
     `eq_mode="eq"` evaluates `eq` as a == b (what the reference's GPU sources
     compute and what the HIP kernels do); `"eq_cpuref"` as a <= b, the
     reference CPU `Eval` (src/two_way_ops/ops/cmps.rs:135).
     Scalars are converted to the element type here, exactly once.
     """
-    prog = []
-
     def const_value(v):
         if isinstance(v, str):
             v = float(v) if dtype in ("f32", "f64", "f16", "bf16", "f16_pernode", "bf16_pernode") else int(float(v))
@@ -80,24 +141,12 @@ def compile_rpn(expr, dtype: str = "f32", eq_mode: str = "eq"):
             return float(v)
         return float(int(v))
 
-    def walk(e):
-        if e.op == "var":
-            prog.append((OPS["var%d" % e.index], 0.0))
-        elif e.op == "const":
-            prog.append((OPS["const"], const_value(e.value)))
-        else:
-            for a in e.args:
-                walk(a)
-            op = e.op
-            if op == "eq":
-                op = eq_mode
-            prog.append((OPS[op], 0.0))
-
-    walk(expr)
-    arr = (Ins * len(prog))()
-    for i, (op, cst) in enumerate(prog):
-        arr[i].op = op
-        arr[i].cst = cst
+    arr = (Ins * len(traced.prog))()
+    for i, (name, literal) in enumerate(traced.prog):
+        if name == "eq":
+            name = eq_mode
+        arr[i].op = OPS[name]
+        arr[i].cst = const_value(literal) if name == "const" else 0.0
     return arr
 
 
@@ -114,17 +163,11 @@ def _rc(rc, what):
         raise RuntimeError(f"oracle {what} failed with {rc}")
 
 
-def _tree(f, n_vars=1, names=("x", "y", "z", "w")):
-    from custos_amd.expr import Resolve, _wrap
-
-    return _wrap(f(*[Resolve(names[i], i) for i in range(n_vars)]))
-
-
 def apply_fn(f, *ins, dtype="f32", eq_mode="eq"):
     """out[i] = f(in0[i], ...) -- src/devices/cpu_stack_ops.rs:7-15."""
     arrs = [_as_storage(a, dtype) for a in ins]
     n = arrs[0].size
-    prog = compile_rpn(_tree(f, len(arrs)), dtype, eq_mode)
+    prog = compile_rpn(trace(f, len(arrs)), dtype, eq_mode)
     out = np.zeros(n, dtype=DTYPES[dtype][1])
     ptrs = (C.c_void_p * len(arrs))(*[a.ctypes.data for a in arrs])
     _rc(lib().oracle_apply_fn(DTYPES[dtype][0], prog, len(prog), ptrs, len(arrs), _ptr(out), C.c_size_t(n)), "apply_fn")
@@ -134,7 +177,7 @@ def apply_fn(f, *ins, dtype="f32", eq_mode="eq"):
 def fused_apply_fn(ops, x, dtype="f32"):
     """Sequential per-element application -- src/devices/cpu/cpu_device.rs:204-232."""
     x = _as_storage(x, dtype)
-    progs = [compile_rpn(_tree(op), dtype) for op in ops]
+    progs = [compile_rpn(trace(op), dtype) for op in ops]
     lens = (C.c_int * len(progs))(*[len(p) for p in progs])
     total = sum(len(p) for p in progs)
     flat = (Ins * max(total, 1))()
@@ -153,7 +196,7 @@ def add_unary_grad(f, lhs, lhs_grad, out_grad, dtype="f32"):
     lhs = _as_storage(lhs, dtype)
     g = _as_storage(lhs_grad, dtype).copy()
     o = _as_storage(out_grad, dtype)
-    prog = compile_rpn(_tree(f), dtype)
+    prog = compile_rpn(trace(f), dtype)
     _rc(lib().oracle_add_unary_grad(DTYPES[dtype][0], prog, len(prog), _ptr(lhs), _ptr(g), _ptr(o), C.c_size_t(lhs.size)), "add_unary_grad")
     return g
 
@@ -165,7 +208,7 @@ def eval_scalar(f, *vals, dtype="f32", eq_mode="eq"):
         "f64": (C.c_double, "oracle_eval_f64"),
         "i32": (C.c_int32, "oracle_eval_i32"),
     }[dtype]
-    prog = compile_rpn(_tree(f, max(len(vals), 1)), dtype, eq_mode)
+    prog = compile_rpn(trace(f, max(len(vals), 1)), dtype, eq_mode)
     vars_ = (ctype * max(len(vals), 1))(*vals)
     res = ctype()
     _rc(getattr(lib(), fn)(prog, len(prog), vars_, len(vals), C.byref(res)), "eval")

@@ -3,13 +3,13 @@ finishes in seconds, and size-independent properties at the full sizes."""
 import numpy as np
 import pytest
 
-from custos_amd import Const, capi, synth
+from custos_amd import capi, synth
 from tests.helpers import assert_bits_equal, ulp_distance_f16, ulp_distance_f32
 
 pytestmark = pytest.mark.gpu
 
 C2_OPS = [lambda v: v.sin(), lambda v: v.mul(2.0), lambda v: v.add(1.0), lambda v: v.max(0.0), lambda v: v.sub(0.5)]
-TANH_GRAD = lambda v: Const(1.0).sub(v.tanh().mul(v.tanh()))
+TANH_GRAD = lambda v: v.val(1.0).sub(v.tanh().mul(v.tanh()))
 C4 = lambda v: v.mul(0.5).exp().mul(v).add(v.mul(v))
 
 

@@ -888,8 +888,8 @@ def test_min_max_of_zeros_return_the_second_operand(hip, oracle, dtype):
     x = hip.buffer(view(xb), dtype)
     cases = (("min(x, 0)", lambda v: v.min(0.0)), ("max(x, 0)", lambda v: v.max(0.0)),
              ("min(x, -0)", lambda v: v.min(-0.0)), ("max(x, -0)", lambda v: v.max(-0.0)),
-             ("min(0, x)", lambda v: Const(0.0).min(v)), ("max(0, x)", lambda v: Const(0.0).max(v)),
-             ("min(-0, x)", lambda v: Const(-0.0).min(v)), ("max(-0, x)", lambda v: Const(-0.0).max(v)),
+             ("min(0, x)", lambda v: v.val(0.0).min(v)), ("max(0, x)", lambda v: v.val(0.0).max(v)),
+             ("min(-0, x)", lambda v: v.val(-0.0).min(v)), ("max(-0, x)", lambda v: v.val(-0.0).max(v)),
              ("min(x, x >= 9)", lambda v: v.min(v.geq(9.0))), ("max(x >= 9, -(x >= 9))", lambda v: v.geq(9.0).max(v.geq(9.0).neg())),
              ("min(-(x >= 9), x >= 9)", lambda v: v.geq(9.0).neg().min(v.geq(9.0))), ("max(x, x * 0)", lambda v: v.max(v.mul(0.0))),
              ("min(|x|, -(|x| * 0))", lambda v: v.abs().min(v.abs().mul(0.0).neg())))
@@ -985,8 +985,8 @@ def _random_tree(rng, leaves, depth, integer, unsigned=False):
     if depth == 0 or rng.random() < 0.15:
         if rng.random() < 0.25:
             if integer:
-                return Const(int(rng.integers(0 if unsigned else -5, 6)))
-            return Const(float(np.float32(rng.uniform(-4, 4))))
+                return leaves[0].val(int(rng.integers(0 if unsigned else -5, 6)))
+            return leaves[0].val(float(np.float32(rng.uniform(-4, 4))))
         return leaves[int(rng.integers(len(leaves)))]
     a = _random_tree(rng, leaves, depth - 1, integer, unsigned)
     # (`abs` needs `Float` in the reference's CPU evaluation, src/two_way_ops/ops/unary.rs:246)

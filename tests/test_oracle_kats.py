@@ -92,8 +92,7 @@ def test_apply_mul2(oracle):
 
 def test_unary_grad_const(oracle):
     # src/unary.rs:40-47: lhs_grad += 1 * 2
-    from custos_amd import to_val
-    out = oracle.add_unary_grad(lambda x: to_val(2.0), [1., 2., 3., 3., 2., 1.], [0.] * 6, [1.] * 6, dtype="f64")
+    out = oracle.add_unary_grad(lambda x: x.val(2.0), [1., 2., 3., 3., 2., 1.], [0.] * 6, [1.] * 6, dtype="f64")
     assert out.tolist() == [2.] * 6
 
 
@@ -179,8 +178,7 @@ def test_monomorphic_loops_equal_interpreter(oracle):
     assert_bits_equal(oracle.c3_tanh_fwd(x), oracle.apply_fn(lambda v: v.tanh(), x))
     g = synth.uniform_f32(1, n, -1, 1)
     o = synth.uniform_f32(2, n, -1, 1)
-    from custos_amd import Const
-    tanh_grad = lambda v: Const(1.0).sub(v.tanh().mul(v.tanh()))
+    tanh_grad = lambda v: v.val(1.0).sub(v.tanh().mul(v.tanh()))
     assert_bits_equal(oracle.c3_tanh_bwd(x, g, o), oracle.add_unary_grad(tanh_grad, x, g, o))
     xb = synth.uniform_f16_bits(0, n, -2, 2)
     c4 = lambda v: v.mul(0.5).exp().mul(v).add(v.mul(v))
@@ -320,3 +318,25 @@ def test_per_node_f16_routines_against_numpy_float16(oracle):
         assert (dist == 0).mean() > 0.99, f"{name}: {(dist == 0).mean():.4f} bit-identical"
         if name == "sqrt":
             assert dist.max() == 0
+
+
+def test_the_oracle_stands_on_its_own():
+    """The oracle traces closures with a tracer of its own: a process that evaluates an expression through it
+    has imported nothing of the package under test (a mistake in the package's expression classes cannot be
+    shared), and the non-commutative nodes keep the order lhs, rhs on known answers."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys\n"
+        "from oracle import cpu_oracle as o\n"
+        "assert o.apply_fn(lambda v: v.val(10.0).sub(v), [1.0, 4.0]).tolist() == [9.0, 6.0]\n"
+        "assert o.apply_fn(lambda a, b: a.div(b), [8.0], [2.0]).tolist() == [4.0]\n"
+        "assert o.apply_fn(lambda a, b: a.pow(b), [2.0], [3.0]).tolist() == [8.0]\n"
+        "assert o.apply_fn(lambda a, b: a.geq(b).sub(a.leq(b)), [3.0, 1.0], [2.0, 2.0]).tolist() == [1.0, -1.0]\n"
+        "assert o.apply_fn(lambda v: v.sub(1.0).mul(2.0), [4.0]).tolist() == [6.0]\n"
+        "assert not [m for m in sys.modules if m.split('.')[0] == 'custos_amd'], 'the oracle imported the package'\n"
+    )
+    proc = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-800:]
