@@ -939,8 +939,8 @@ int32_t custos_hip_apply_fn_many_noalloc(custos_hip_device* dev, custos_hip_kern
     if (known < 0) {
         const int written = kernel->spec.kind == Kind::UnaryGrad ? 1 : n_ptrs - 1;
         const char* why = "";
-        const int32_t verdict = dev->noalloc_checker.check(operands, n_ptrs, n_sets, written, bytes, &why);
-        if (verdict != CUSTOS_HIP_OK) return set_error(dev, verdict, why);
+        const int32_t checked = dev->noalloc_checker.check(operands, n_ptrs, n_sets, written, bytes, &why);
+        if (checked != CUSTOS_HIP_OK) return set_error(dev, checked, why);
         known = static_cast<int>(dev->noalloc_next);
         dev->noalloc_next = (dev->noalloc_next + 1) % dev->noalloc_checked.size();
         if (dev->noalloc_in_table == known) dev->noalloc_in_table = -1;

@@ -249,7 +249,7 @@ def test_chain_emit_rejects_malformed_stages():
         capi.chain_emit("i32", [("sin(v0)", [0], 0)], 1, 1)    # no such node over integers
 
 
-def _operand_sets_verdict(rows, written, length):
+def _operand_sets_answer(rows, written, length):
     """What the checks of a merged launch must say, pair by pair."""
     for row in rows:
         if any(a == 0 or a % 16 for a in row):
@@ -275,22 +275,22 @@ def test_operand_checks_of_merged_launches_against_all_pairs():
     import random
     lib = capi.load_library()
 
-    def verdict(rows, written, length):
+    def answer(rows, written, length):
         flat = (C.c_uint64 * (len(rows) * len(rows[0])))(*[a for row in rows for a in row])
         return lib.custos_hip_check_operand_sets(flat, len(rows[0]), len(rows), written, length)
 
     base = 0x7F0000000000
-    assert verdict([[base, base + 4096], [base + 64, base + 4096 + 64]], 1, 64) == 0                       # exactly one length apart
-    assert verdict([[base, base + 4096], [base + 48, base + 4096 + 64]], 1, 64) == 0                       # inputs may overlap
-    assert verdict([[base, base + 4096], [base + 64, base + 4096 + 48]], 1, 64) == capi.ERR_BAD_OVERLAP    # outputs may not
-    assert verdict([[base, base], [base + 64, base + 64]], 1, 64) == 0                                     # out == in
-    assert verdict([[base, base + 16]], 1, 64) == capi.ERR_BAD_OVERLAP                                     # partial, inside a row
-    assert verdict([[base, base + 4096], [base + 4096 + 16, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # reads another row's output
-    assert verdict([[base, base + 4096], [base + 4096 - 48, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # ... from the piece before
-    assert verdict([[base, base + 4096 + 16], [base + 4096 + 64, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # ... from the piece after
-    assert verdict([[base + 8, base + 4096]], 1, 64) == capi.ERR_INVALID_ARGUMENT
-    assert verdict([[0, base + 4096]], 1, 64) == capi.ERR_INVALID_ARGUMENT
-    assert verdict([[16, 4096]], 1, 48) == 0                                                               # the first piece of memory
+    assert answer([[base, base + 4096], [base + 64, base + 4096 + 64]], 1, 64) == 0                       # exactly one length apart
+    assert answer([[base, base + 4096], [base + 48, base + 4096 + 64]], 1, 64) == 0                       # inputs may overlap
+    assert answer([[base, base + 4096], [base + 64, base + 4096 + 48]], 1, 64) == capi.ERR_BAD_OVERLAP    # outputs may not
+    assert answer([[base, base], [base + 64, base + 64]], 1, 64) == 0                                     # out == in
+    assert answer([[base, base + 16]], 1, 64) == capi.ERR_BAD_OVERLAP                                     # partial, inside a row
+    assert answer([[base, base + 4096], [base + 4096 + 16, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # reads another row's output
+    assert answer([[base, base + 4096], [base + 4096 - 48, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # ... from the piece before
+    assert answer([[base, base + 4096 + 16], [base + 4096 + 64, base + 8192]], 1, 64) == capi.ERR_BAD_OVERLAP  # ... from the piece after
+    assert answer([[base + 8, base + 4096]], 1, 64) == capi.ERR_INVALID_ARGUMENT
+    assert answer([[0, base + 4096]], 1, 64) == capi.ERR_INVALID_ARGUMENT
+    assert answer([[16, 4096]], 1, 48) == 0                                                               # the first piece of memory
     rng = random.Random(5)
     seen = {0: 0, capi.ERR_BAD_OVERLAP: 0}
     for case in range(600):
@@ -313,7 +313,7 @@ def test_operand_checks_of_merged_launches_against_all_pairs():
                 at += length + 16 * rng.randrange(3)
                 if rng.random() < 0.2:
                     row[0] = row[written]
-        want = _operand_sets_verdict(rows, written, length)
-        assert verdict(rows, written, length) == want, (case, rows, written, length)
+        want = _operand_sets_answer(rows, written, length)
+        assert answer(rows, written, length) == want, (case, rows, written, length)
         seen[want] += 1
     assert seen[0] > 100 and seen[capi.ERR_BAD_OVERLAP] > 100, seen
