@@ -529,7 +529,10 @@ int32_t custos_hip_device_destroy(custos_hip_device* dev) {
     }
     for (custos_hip_graph* g : dev->graphs) destroy_graph(g);
     // every block of this handle goes back to the driver, pooled or still held by the caller
-    for (auto& kv : dev->block_bytes) (void)hipFree(reinterpret_cast<void*>(kv.first));
+    for (auto& kv : dev->block_bytes)
+        if (kv.second.slab < 0) (void)hipFree(reinterpret_cast<void*>(kv.first));
+    for (const custos_hip_device::Slab& slab : dev->slabs)
+        if (slab.base) (void)hipFree(reinterpret_cast<void*>(slab.base));
     for (auto& bucket : dev->cache)
         for (auto& k : bucket.second)
             for (hipModule_t module : k->modules)
@@ -606,15 +609,74 @@ static size_t pool_size_class(size_t bytes) {
     return (bytes + step - 1) / step * step;
 }
 
+constexpr size_t kSlabBytes = 4u << 20;        // blocks of up to kSlabBlockMax bytes are cut from allocations of this size
+constexpr size_t kSlabBlockMax = 256u << 10;
+
+// A block whose registry entry was `block` goes back to the driver (the work that used it has
+// finished): an allocation of its own at once, a block of a slab together with the slab's last one.
+static void give_back(custos_hip_device* dev, uint64_t addr, const custos_hip_device::Block& block) {
+    if (block.slab < 0) {
+        (void)hipFree(reinterpret_cast<void*>(addr));
+        return;
+    }
+    custos_hip_device::Slab& slab = dev->slabs[static_cast<size_t>(block.slab)];
+    if (--slab.blocks > 0) return;
+    (void)hipFree(reinterpret_cast<void*>(slab.base));
+    slab = custos_hip_device::Slab{};
+    if (dev->open_slab == block.slab) dev->open_slab = -1;
+}
+
 static void release_pool(custos_hip_device* dev) {
     (void)hipStreamSynchronize(dev->stream);
     for (auto& kv : dev->pool)
         for (void* p : kv.second) {
-            dev->block_bytes.erase(reinterpret_cast<uint64_t>(p));
-            (void)hipFree(p);
+            const uint64_t addr = reinterpret_cast<uint64_t>(p);
+            const custos_hip_device::Block block = dev->block_bytes[addr];
+            dev->block_bytes.erase(addr);
+            give_back(dev, addr, block);
         }
     dev->pool.clear();
     dev->pooled_bytes = 0;
+}
+
+// A new block of `rounded` bytes cut from the open slab, or from a new one (zero-filled as a
+// whole: `*zeroed` tells the caller that the block needs no fill of its own).  0 when no slab
+// could be made; the caller then allocates the block by itself.
+static uint64_t cut_from_slab(custos_hip_device* dev, size_t rounded, bool* zeroed) {
+    *zeroed = false;
+    if (dev->open_slab < 0 || dev->slabs[static_cast<size_t>(dev->open_slab)].used + rounded > kSlabBytes) {
+        void* base = nullptr;
+        if (hipMalloc(&base, kSlabBytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        // (zeros once, in the order every other fill of an allocation has: the compute stream, or,
+        // while the device records, the transfer stream and a wait)
+        hipStream_t s = dev->capturing ? dev->transfer : dev->stream;
+        int32_t rc = launch_fill_zero(dev, reinterpret_cast<uint64_t>(base), kSlabBytes, s);
+        if (rc == CUSTOS_HIP_OK && dev->capturing && hipStreamSynchronize(dev->transfer) != hipSuccess) rc = CUSTOS_HIP_ERR_INVALID_ARGUMENT;
+        if (rc != CUSTOS_HIP_OK) {
+            (void)hipGetLastError();
+            (void)hipFree(base);
+            return 0;
+        }
+        // (the slab that was open keeps its blocks and goes when the last of them does; the entry of
+        // a slab that is gone is used again)
+        custos_hip_device::Slab slab;
+        slab.base = reinterpret_cast<uint64_t>(base);
+        slab.bytes = kSlabBytes;
+        size_t index = 0;
+        while (index < dev->slabs.size() && dev->slabs[index].base != 0) index++;
+        if (index == dev->slabs.size()) dev->slabs.push_back(slab);
+        else dev->slabs[index] = slab;
+        dev->open_slab = static_cast<int32_t>(index);
+    }
+    custos_hip_device::Slab& slab = dev->slabs[static_cast<size_t>(dev->open_slab)];
+    const uint64_t addr = slab.base + slab.used;
+    slab.used += rounded;
+    slab.blocks++;
+    *zeroed = true;
+    return addr;
 }
 
 int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, uint64_t* dptr) {
@@ -624,6 +686,7 @@ int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, ui
     if (bytes == 0) return set_error(dev, CUSTOS_HIP_ERR_ZERO_LENGTH_BUFFER, "zero length buffers are not supported");
     const size_t rounded = pool_size_class(bytes);
     void* p = nullptr;
+    bool already_zero = false;  // a block newly cut from a slab: the slab was zero-filled when it was made
     if (dev->capturing && flags != CUSTOS_HIP_ALLOC_UNINIT) HIP_TRY(dev, drain_before_immediate_work(dev));
     auto pooled = dev->pool.find(rounded);
     if (pooled != dev->pool.end() && !pooled->second.empty()) {
@@ -633,18 +696,26 @@ int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, ui
         dev->pool_reused++;
         dev->block_bytes[reinterpret_cast<uint64_t>(p)].pooled = false;
     } else {
-        hipError_t e = hipMalloc(&p, rounded);
-        if (e != hipSuccess && dev->pooled_bytes > 0) {
-            (void)hipGetLastError();
-            release_pool(dev);  // the pool may hold what this allocation needs
-            e = hipMalloc(&p, rounded);
+        bool zeroed = false;
+        const uint64_t cut = rounded <= kSlabBlockMax ? cut_from_slab(dev, rounded, &zeroed) : 0;
+        if (cut) {
+            p = reinterpret_cast<void*>(cut);
+            dev->block_bytes[cut] = {rounded, false, dev->open_slab};
+            already_zero = zeroed;
+        } else {
+            hipError_t e = hipMalloc(&p, rounded);
+            if (e != hipSuccess && dev->pooled_bytes > 0) {
+                (void)hipGetLastError();
+                release_pool(dev);  // the pool may hold what this allocation needs
+                e = hipMalloc(&p, rounded);
+            }
+            if (e != hipSuccess) return hip_fail(dev, e, "hipMalloc");
+            dev->block_bytes[reinterpret_cast<uint64_t>(p)] = {rounded, false, -1};
         }
-        if (e != hipSuccess) return hip_fail(dev, e, "hipMalloc");
-        dev->block_bytes[reinterpret_cast<uint64_t>(p)] = {rounded, false};
         dev->pool_allocated++;
     }
     uint64_t addr = reinterpret_cast<uint64_t>(p);
-    if (flags != CUSTOS_HIP_ALLOC_UNINIT) {
+    if (flags != CUSTOS_HIP_ALLOC_UNINIT && !already_zero) {
         // While recording, the fill must run now and not become part of the graph.
         hipStream_t s = dev->capturing ? dev->transfer : dev->stream;
         int32_t rc = launch_fill_zero(dev, addr, bytes, s);
@@ -653,8 +724,9 @@ int32_t custos_hip_alloc(custos_hip_device* dev, size_t bytes, int32_t flags, ui
             if (e != hipSuccess) rc = hip_fail(dev, e, "hipStreamSynchronize(transfer)");
         }
         if (rc != CUSTOS_HIP_OK) {
+            const custos_hip_device::Block block = dev->block_bytes[addr];
             dev->block_bytes.erase(addr);
-            (void)hipFree(p);
+            give_back(dev, addr, block);
             return rc;
         }
     }
@@ -679,11 +751,12 @@ int32_t custos_hip_free(custos_hip_device* dev, uint64_t dptr) {
         dev->pooled_bytes += known->second.bytes;
         return CUSTOS_HIP_OK;
     }
+    const custos_hip_device::Block block = known->second;
     dev->block_bytes.erase(known);
     // work that still uses the range must finish first
     if (!dev->capturing) HIP_TRY(dev, hipStreamSynchronize(dev->stream));
     else HIP_TRY(dev, drain_before_immediate_work(dev));
-    HIP_TRY(dev, hipFree(reinterpret_cast<void*>(dptr)));
+    give_back(dev, dptr, block);
     return CUSTOS_HIP_OK;
 }
 

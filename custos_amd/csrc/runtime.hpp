@@ -199,7 +199,19 @@ struct custos_hip_device {
     struct Block {
         size_t bytes = 0;     // rounded size
         bool pooled = false;  // in `pool` (freed by the caller), else handed out
+        int32_t slab = -1;    // index into `slabs` of the allocation the block was cut from, or -1: an allocation of its own
     };
+    // Small blocks are cut from larger allocations ("slabs"), which are zero-filled once when they
+    // are made: a program that allocates thousands of small buffers pays one driver allocation and
+    // one fill launch per slab instead of per buffer.  A slab goes back to the driver when every
+    // block cut from it has (a freed block first waits in the pool like any other).
+    struct Slab {
+        uint64_t base = 0;
+        size_t bytes = 0, used = 0;  // `used`: bytes cut off so far
+        size_t blocks = 0;           // blocks cut from it that have not gone back to the driver
+    };
+    std::vector<Slab> slabs;         // (entries of released slabs stay, with base 0)
+    int32_t open_slab = -1;          // the slab blocks are being cut from
     std::unordered_map<uint64_t, Block> block_bytes;
     size_t pooled_bytes = 0, pool_limit = 0;
     uint64_t pool_reused = 0, pool_allocated = 0;

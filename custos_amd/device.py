@@ -320,15 +320,18 @@ class HIP:
 
     # -- caller-written kernels (`launch_kernel` / `launch_kernel1d`, src/devices/cuda/cuda_device.rs:85-112) --
     def _source_args(self, args):
-        """Buffers pass their device address, ctypes values pass as they are, ints become c_int32,
-        floats c_float (`AsCudaCvoidPtr`, src/devices/cuda/kernel_launch.rs:29-77)."""
+        """Buffers pass their device address, ctypes values and numpy scalars pass with their own
+        width (`np.uint64(n)` for an `unsigned long long` parameter), Python ints become c_int32 and
+        Python floats c_float (`AsCudaCvoidPtr`, src/devices/cuda/kernel_launch.rs:29-77)."""
         vals = []
         for a in args:
             if isinstance(a, Buffer):
                 vals.append(C.c_uint64(a.ptr))
             elif isinstance(a, C._SimpleCData):
                 vals.append(a)
-            elif isinstance(a, (bool, int, np.integer)):
+            elif isinstance(a, np.generic) and not isinstance(a, np.bool_):
+                vals.append(np.ctypeslib.as_ctypes_type(a.dtype)(a.item()))
+            elif isinstance(a, (bool, int, np.bool_)):
                 vals.append(C.c_int32(int(a)))
             else:
                 vals.append(C.c_float(float(a)))

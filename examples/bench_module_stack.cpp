@@ -415,12 +415,15 @@ int main(int argc, char** argv) {
                 bs.push_back(device.buffer(uniform_f32(2, m, 0.f, 1.f, i * m)));
                 cs.push_back(device.buffer(uniform_f32(3, m, 0.f, 1.f, i * m)));
             }
+            device.sync();
+            const auto recording = Clock::now();
             for (size_t i = 0; i < nbuf; i++) {
                 auto t = device.apply_fn2(as[i], bs[i], [](auto x, auto y) { return x.mul(y); });
                 auto u = device.apply_fn2(t, cs[i], [](auto x, auto y) { return x.add(y); });
                 ys.push_back(device.apply_fn(u, [](auto x) { return x.abs().sqrt().mul(0.3f); }));
             }
             if (fuse) device.elementwise_fusing();
+            const double record_ms = us_since(recording) * 1e-3;
             const auto first = Clock::now();
             device.run();
             device.sync();
@@ -428,10 +431,10 @@ int main(int argc, char** argv) {
             const Timing t = time_runs([&] { device.run(); }, [&] { device.sync(); }, warmup, steps, settle_ms);
             if (dump_count) dump_f32(device, ys[0].replace().ptr(), std::min(dump_count, m), dump_path);
             std::printf("{\"config\": \"c5\", \"stack\": \"HIP<Graph<Lazy<Base>>>\", \"calls\": \"1024 x (apply_fn2, apply_fn2, apply_fn)%s, "
-                        "run()\", \"elements\": %zu, \"warmup\": %d, %s, \"first_run_ms\": %.2f, \"kernel_nodes\": %zu, "
+                        "run()\", \"elements\": %zu, \"warmup\": %d, %s, \"record_ms\": %.2f, \"first_run_ms\": %.2f, \"kernel_nodes\": %zu, "
                         "\"graph_builds\": %llu}\n",
                         fuse ? ", elementwise_fusing" : "", nbuf * m, warmup, timing_json(t, 16.0 * static_cast<double>(nbuf * m)).c_str(),
-                        first_run_ms, device.graph_kernel_nodes(), static_cast<unsigned long long>(device.graph_builds()));
+                        record_ms, first_run_ms, device.graph_kernel_nodes(), static_cast<unsigned long long>(device.graph_builds()));
         } else {
             std::fprintf(stderr, "unknown config %s\n", config.c_str());
             return 2;

@@ -1289,6 +1289,57 @@ def test_allocation_pool():
         dev.close()
 
 
+def test_small_blocks_are_cut_from_zeroed_slabs():
+    """Blocks of up to 256 KiB are cut from 4 MiB allocations that are zero-filled once: new blocks are
+    zero, neighbours in a slab do not touch each other (a launch over one leaves the blocks around it
+    alone, up to the last byte of its rounded size), a freed block is reused and zero-filled again, and
+    with the pool switched off a slab goes back to the driver with its last block, after which new
+    blocks are zero again although the memory may be the same."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        n = 4000                                     # 16 000 bytes: rounds to 16 384, 256 blocks per slab
+        blocks = [dev.alloc(n) for _ in range(600)]  # three slabs
+        addrs = sorted(b.ptr for b in blocks)
+        gaps = np.diff(np.array(addrs, dtype=np.uint64))
+        assert (gaps >= 16384).all() and (gaps == 16384).sum() >= 590        # cut one after the other
+        for b in blocks[::37]:
+            assert not b.read().any()
+        x = synth.uniform_f32(3, n, 1, 2)
+        src = dev.buffer(x)
+        for b in blocks[1::2]:
+            dev.apply_fn(src, lambda v: v.mul(3.0), out=b)
+        want = (x * np.float32(3.0)).astype(np.float32)
+        for i in (0, 2, 254, 256, 300, 598):
+            assert not blocks[i].read().any(), i     # even blocks stay zero next to written neighbours
+        for i in (1, 255, 257, 599):
+            assert_bits_equal(blocks[i].read(), want)
+        # a freed block comes back from the pool, zero-filled again
+        addr = blocks[1].ptr
+        blocks[1].free()
+        again = dev.alloc(n)
+        assert again.ptr == addr and not again.read().any()
+        blocks[1] = again
+        # no pool: blocks go back one by one, a slab with its last block; what is allocated afterwards is zero
+        dev.sync()
+        dev.set_pool_limit(0)
+        for b in blocks:
+            b.free()
+        src.free()
+        assert dev.pool_stats()[0] == 0
+        fresh = [dev.alloc(n) for _ in range(300)]
+        for b in fresh[::29]:
+            assert not b.read().any()
+        # larger blocks are allocations of their own
+        big = dev.alloc(100000)
+        assert not big.read().any()
+        for b in fresh:
+            dev.apply_fn(big.slice(0, n), lambda v: v.add(1.5), out=b)
+        assert (fresh[123].read() == np.float32(1.5)).all()
+    finally:
+        dev.close()
+
+
 def test_device_to_device_copies(hip):
     """Aligned ranges go through the library's copy kernel, unaligned ones through the runtime:
     the same bytes either way, small and larger than the memory-side cache."""
