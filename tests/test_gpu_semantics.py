@@ -1340,6 +1340,67 @@ def test_small_blocks_are_cut_from_zeroed_slabs():
         dev.close()
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "i8", "f64"])
+def test_no_launch_writes_outside_its_range(dtype):
+    """Blocks that sit back to back in one slab: every kind of launch over the middle one and over
+    views inside it (odd lengths, offsets that start off a 16-byte boundary: scalar head and tail,
+    partial last tile), eagerly, recorded and joined, merged with equal and with different lengths,
+    filled and copied -- and the guard blocks before and behind it keep their pattern to the byte."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        item = np.dtype(capi.DTYPES[dtype][1]).itemsize
+        per512 = 512 // item
+        guard_n = 8 * per512                      # whole size classes: no slack between the blocks
+        mid_n = 20 * per512
+        pattern = (np.arange(guard_n * item, dtype=np.uint32) * 37 + 11).astype(np.uint8)
+        as_elems = lambda raw: raw.view(capi.DTYPES[dtype][1])
+        before = dev.buffer(as_elems(pattern), dtype)
+        mid = dev.alloc(mid_n, dtype)
+        behind = dev.buffer(as_elems(pattern), dtype)
+        second = dev.alloc(mid_n, dtype)
+        last = dev.buffer(as_elems(pattern), dtype)
+        assert mid.ptr == before.ptr + guard_n * item and behind.ptr == mid.ptr + mid_n * item
+        assert second.ptr == behind.ptr + guard_n * item and last.ptr == second.ptr + mid_n * item
+        src = dev.buffer(np.ones(mid_n, dtype=capi.DTYPES[dtype][1]), dtype)
+        f = lambda v: v.add(1) if dtype == "i8" else v.mul(1.5).add(0.25)
+        g = lambda v: v.add(v)
+        views = [(0, mid_n), (1, mid_n), (0, mid_n - 1), (3, mid_n - 5), (7, 7 + 33), (mid_n - 9, mid_n), (5, 5 + 16 * per512 + 3)]
+        for lo, hi in views:
+            dev.apply_fn(src.slice(lo, hi), f, out=mid.slice(lo, hi))                 # eager
+            dev.apply_fn2(src.slice(lo, hi), mid.slice(lo, hi), lambda p, q: p.add(q), out=second.slice(lo, hi))
+            if dtype in ("f32", "f64"):
+                dev.add_unary_grad(src.slice(lo, hi), mid.slice(lo, hi), second.slice(lo, hi), lambda v: v.mul(2.0))
+            dev.fill(mid.slice(lo, hi), 3)
+            dev.clear(second.slice(lo, hi))
+            dev.copy(mid.slice(lo, hi), src.slice(lo, hi))
+        for merged in (True, False):
+            dev.set_graph_batching(merged)
+            dev.capture_begin()
+            for lo, hi in views:                                                          # recorded: joined, merged (ragged)
+                dev.apply_fn(src.slice(lo, hi), f, out=mid.slice(lo, hi))
+                dev.apply_fn(mid.slice(lo, hi), g, out=second.slice(lo, hi))
+            graph = dev.capture_end()
+            graph.launch()
+            graph.launch()
+            dev.sync()
+            graph.destroy()
+        dev.set_graph_batching(True)
+        dev.capture_begin()
+        for k in range(6):                                                                # equal lengths, aligned: one merged grid
+            lo = k * 3 * per512
+            dev.apply_fn(src.slice(lo, lo + 3 * per512), f, out=mid.slice(lo, lo + 3 * per512))
+        dev.apply_fn(src.slice(18 * per512, mid_n), f, out=mid.slice(18 * per512, mid_n))
+        graph = dev.capture_end()
+        graph.launch()
+        dev.sync()
+        graph.destroy()
+        for name, guard in (("before", before), ("behind", behind), ("last", last)):
+            assert np.array_equal(guard.read().view(np.uint8), pattern), f"{dtype}: the block {name} was written"
+    finally:
+        dev.close()
+
+
 def test_device_to_device_copies(hip):
     """Aligned ranges go through the library's copy kernel, unaligned ones through the runtime:
     the same bytes either way, small and larger than the memory-side cache."""
