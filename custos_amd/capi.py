@@ -220,9 +220,10 @@ def preferred_shape(footprint_bytes: int, n_operands: int):
     return u.value, nt.value, bool(alt.value)
 
 
-def preferred_shape_of(footprint_bytes: int, n_operands: int, n_written: int = 1, working_set_bytes: int = 0, revisits: bool = True):
+def preferred_shape_of(footprint_bytes: int, n_operands: int, n_written: int = 1, working_set_bytes: int = 0, revisits=True):
     """(vectors per thread, nontemporal bits, alternates direction, threads per workgroup or 0) with everything
-    the choice depends on."""
+    the choice depends on.  `revisits`: True / 1 = touches what the launch before wrote, False / 0 = has nothing
+    in common with it, 2 = reads exactly what it read and touches nothing it wrote."""
     u, nt, alt, block = C.c_int32(0), C.c_int32(0), C.c_int32(0), C.c_int32(0)
     check(load_library().custos_hip_preferred_shape_of(footprint_bytes, n_operands, n_written, working_set_bytes, int(revisits),
                                                        C.byref(u), C.byref(nt), C.byref(alt), C.byref(block)))

@@ -66,7 +66,7 @@ constexpr unsigned long long kL2WorkingSet = 32ull << 20;  // what the eight L2s
 // `revisits`: the launch touches memory that the launch before it wrote (the same launch repeated,
 // a consumer of the last launch); `n_written`: how many of its operands it writes.
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint = CacheHint::Unknown,
-                            unsigned long long working_set_bytes = 0, bool revisits = true, int n_written = 1);
+                            unsigned long long working_set_bytes = 0, bool revisits = true, int n_written = 1, bool rereads = false);
 
 // The last argument of every generated entry point: how this launch runs the kernel.  Nothing
 // of it is compiled in, so one kernel per expression serves every launch size.

@@ -2,6 +2,7 @@
 // into scalar head / 16-byte vectors / scalar tail, and recording while the
 // device records (include/custos_hip.h).
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 #include "runtime.hpp"
@@ -44,6 +45,21 @@ bool RecentTraffic::wrote_any_of(const std::vector<Access>& reads) const {
                 if (r.begin < w.end && w.begin < r.end) return true;
         }
     return false;
+}
+
+bool RecentTraffic::last_read_exactly(const std::vector<Access>& all) const {
+    if (launches_.empty()) return false;
+    std::vector<Access> reads;
+    for (const Access& a : all)
+        if (!a.write) reads.push_back(a);
+    reads = merged(std::move(reads));
+    size_t at = 0;
+    for (const Access& was : launches_.back()) {
+        if (was.write) continue;
+        if (at == reads.size() || reads[at].begin != was.begin || reads[at].end != was.end) return false;
+        at++;
+    }
+    return at == reads.size() && at > 0;
 }
 
 bool RecentTraffic::last_wrote_any_of(const std::vector<Access>& ranges) const {
@@ -204,7 +220,7 @@ ResolvedShape shape_of_launch(custos_hip_device* dev, const custos_hip_kernel* k
     for (const Access& a : acc) footprint += a.end - a.begin;
     CacheHint hint = CacheHint::Unknown;
     unsigned long long working_set = 0;
-    bool revisits = true;
+    bool revisits = true, rereads = false;
     if (footprint > kTrafficBeyondBytes) {
         if (footprint >= kHintFromBytes) {
             std::vector<Access> reads;
@@ -218,9 +234,10 @@ ResolvedShape shape_of_launch(custos_hip_device* dev, const custos_hip_kernel* k
         // memory-side cache to a large one
         working_set = history->working_set_with(acc);
         revisits = history->last_wrote_any_of(acc);
+        rereads = !revisits && history->last_read_exactly(acc);
         history->record(acc);
     }
-    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set, revisits);
+    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set, revisits, rereads);
     dev->last_shape[0] = shape.unroll, dev->last_shape[1] = shape.nontemporal, dev->last_shape[2] = shape.alternate;
     dev->last_shape[3] = shape.block;
     return shape;

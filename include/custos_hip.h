@@ -323,9 +323,13 @@ int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated
  * through, and touches 128 MiB or more, takes temporal loads and non-temporal stores written
  * through at once, so that the cache keeps its input and not its outputs), the distinct bytes the
  * launch and the launches before it touch together (`working_set_bytes`, 0 = unknown), and
- * whether it touches memory that the launch before it wrote (`revisits`: a launch of more than
- * 32 MiB that does not runs as one-wavefront workgroups with one vector per thread;
- * `block_threads` receives 64 then, else 0 for the workgroup size the kernel was compiled for). */
+ * what it has in common with the launch before it (`revisits`: 1 = it touches memory that launch
+ * wrote; 0 = nothing of that: a launch of more than 32 MiB then runs as one-wavefront workgroups
+ * with one vector per thread, and `block_threads` receives 64, else 0 for the workgroup size the
+ * kernel was compiled for; 2 = nothing that launch wrote, and it reads exactly what that launch
+ * read (`y = f(x)` into another buffer every time): as for 0, with temporal loads, non-temporal
+ * stores written through at once and the direction alternating, so that the cache keeps the input
+ * both launches read). */
 int32_t custos_hip_preferred_shape_of(uint64_t footprint_bytes, int32_t n_operands, int32_t n_written,
                                       uint64_t working_set_bytes, int32_t revisits, int32_t *unroll,
                                       int32_t *nontemporal, int32_t *alternate, int32_t *block_threads);

@@ -1221,6 +1221,39 @@ def test_mid_sized_launches_leave_the_cache_to_their_neighbours(oracle):
         dev.close()
 
 
+def test_a_launch_that_reads_what_the_one_before_read_keeps_the_input_cached(oracle):
+    """`out = device.apply_fn(&x, f)` in a loop alternates between two output blocks: each launch touches
+    nothing the launch before it wrote and reads exactly what it read, and takes temporal loads, stores
+    past the cache and the alternating direction.  A launch that merely shares an input with the one
+    before (the gradient launch behind the forward launch of the same x) does not.  Same bits either way."""
+    import custos_amd
+    dev = custos_amd.HIP(0)
+    try:
+        loads, stores = 1 | 64, 2 | 64
+        n = (1 << 24) + 3                             # 64 MiB per array
+        xs = synth.uniform_f32(77, n, -2, 2)
+        x = dev.buffer(xs)
+        outs = [dev.alloc(n), dev.alloc(n)]
+        f = lambda v: v.mul(1.5).add(0.25)
+        want = oracle.apply_fn(f, xs)
+        dev.apply_fn(x, f, out=outs[0])
+        assert dev.last_launch_shape() == (1, loads, False)      # nothing before it
+        for step in range(1, 5):
+            dev.apply_fn(x, f, out=outs[step & 1])
+            assert dev.last_launch_shape() == (1, stores, True), step
+        for out in outs:
+            assert_bits_equal(out.read(), want)
+        g, o = dev.alloc(n), dev.buffer(synth.uniform_f32(78, n, -1, 1))
+        dev.add_unary_grad(x, g, o, lambda v: v.mul(2.0))        # reads x too, and two arrays more
+        assert dev.last_launch_shape() == (1, loads, False)
+        dev.apply_fn(x, f, out=outs[0])                          # the launch before it read more than x
+        assert dev.last_launch_shape() == (1, loads, False)
+        dev.apply_fn(x, f, out=outs[0])                          # overwrites what was just written: the usual shape
+        assert dev.last_launch_shape()[0] == 2
+    finally:
+        dev.close()
+
+
 def test_more_than_two_to_the_32_elements(hip):
     """Indices are 64-bit throughout: 2^32 + 5 one-byte elements (4 GiB in, 4 GiB out), launched
     directly and from a replayed graph; windows around 2^31, 2^32 and the scalar tail."""
