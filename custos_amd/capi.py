@@ -223,7 +223,7 @@ def preferred_shape(footprint_bytes: int, n_operands: int):
 def preferred_shape_of(footprint_bytes: int, n_operands: int, n_written: int = 1, working_set_bytes: int = 0, revisits=True):
     """(vectors per thread, nontemporal bits, alternates direction, threads per workgroup or 0) with everything
     the choice depends on.  `revisits`: True / 1 = touches what the launch before wrote, False / 0 = has nothing
-    in common with it, 2 = reads exactly what it read and touches nothing it wrote."""
+    in common with it, 2 = its first input is something that launch read, and it touches nothing that launch wrote."""
     u, nt, alt, block = C.c_int32(0), C.c_int32(0), C.c_int32(0), C.c_int32(0)
     check(load_library().custos_hip_preferred_shape_of(footprint_bytes, n_operands, n_written, working_set_bytes, int(revisits),
                                                        C.byref(u), C.byref(nt), C.byref(alt), C.byref(block)))

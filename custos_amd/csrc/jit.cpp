@@ -344,10 +344,10 @@ int32_t identity_kernel(custos_hip_device* dev, DType dtype, custos_hip_kernel**
 }
 
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
-                            CacheHint hint, unsigned long long working_set_bytes, bool revisits, bool rereads) {
+                            CacheHint hint, unsigned long long working_set_bytes, bool revisits, int keep_inputs) {
     const int n_operands = kernel_pointers(k->spec);
     const int n_written = k->spec.kind == Kind::Chain ? k->spec.n_outs : 1;
-    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint, working_set_bytes, revisits, n_written, rereads);
+    const LaunchShape shape = preferred_shape(footprint_bytes, n_operands, hint, working_set_bytes, revisits, n_written, keep_inputs);
     ResolvedShape r;
     const int direction = dev->tuning.direction;
     r.alternate = direction == 2 || (direction == 0 && shape.alternate);
@@ -620,7 +620,7 @@ int32_t custos_hip_preferred_shape_of(uint64_t footprint_bytes, int32_t n_operan
     if (n_operands < 1 || n_written < 0 || n_written > n_operands)
         return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_ARGUMENT, "n_operands must be positive and n_written within it");
     const LaunchShape s = preferred_shape(footprint_bytes, n_operands, CacheHint::Unknown, working_set_bytes, revisits == 1, n_written,
-                                          revisits == 2);
+                                          revisits == 2 ? 1 : 0);
     if (unroll) *unroll = s.unroll;
     if (nontemporal) *nontemporal = s.nontemporal;
     if (alternate) *alternate = s.alternate ? 1 : 0;

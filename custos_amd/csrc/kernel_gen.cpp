@@ -84,7 +84,7 @@ Tuning normalize_tuning(int block_threads, int unroll, int blocks_per_cu, int no
 // the other way round: 2R+2W over 2^26 7150 / 6362; and below 128 MiB touched the usual policy is
 // ahead: 1R+3W over 64 MiB 8204 / 7779, 1R+5W over 96 MiB 7868 / 6714.)
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint,
-                            unsigned long long working_set_bytes, bool revisits, int n_written, bool rereads) {
+                            unsigned long long working_set_bytes, bool revisits, int n_written, int keep_inputs) {
     constexpr unsigned long long MiB = 1ull << 20;
     // non-temporal loads with temporal stores that are written through at once / both non-temporal /
     // temporal loads with non-temporal stores that are written through at once
@@ -98,15 +98,16 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
              working_set > footprint_bytes)
         shape.nontemporal = kBoth;
     if (!revisits && footprint_bytes > kL2WorkingSet) shape.unroll = 1, shape.block = 64;
-    // It touches nothing the launch before it wrote and reads exactly what that launch read (`y = f(x)`
-    // into another buffer every time, what `out = device.apply_fn(&x, f)` in a loop does): the
-    // memory-side cache is worth more to the input than to outputs nobody is about to read.  Loads
-    // keep their lines, stores go past the cache, and the launch starts where the one before it
-    // ended.  f16 chain over 2^28 elements through the module stack: 6.72 -> 6.99 TB/s; an input of
-    // 256 MiB (zeros): 6.7 -> 8.8; of 1 GiB: no difference.  Not for launches that merely share an
-    // input with the one before (tanh forward and its gradient launch in turn lose 9 % with it: the
-    // cache then holds the gradient buffer for the next gradient launch).
-    if (!revisits && rereads && footprint_bytes > kL2WorkingSet) shape.nontemporal = kStores, shape.alternate = true;
+    // It touches nothing the launch before it wrote but reads, through the inputs `keep_inputs` names,
+    // what that launch read as well (`y = f(x)` into another buffer every time, what
+    // `out = device.apply_fn(&x, f)` in a loop does; the gradient launch behind the forward launch of
+    // the same x, and the next forward launch behind it): the memory-side cache is worth more to
+    // those inputs than to anything else the launch moves.  They are loaded with temporal accesses,
+    // everything else streams past the cache, and the launch starts where the one before it ended.
+    if (!revisits && keep_inputs != 0 && footprint_bytes > kL2WorkingSet) {
+        shape.nontemporal = 3 | kStoresWriteThrough | (keep_inputs & kKeepInputMask) << kKeepInputShift;
+        shape.alternate = true;
+    }
     return shape;
 }
 
@@ -393,6 +394,13 @@ struct KernelText {
     }
 
     // Chain: one tile, all loads before the first store, one store per output.
+    // Whether input `i` is loaded with non-temporal accesses: bit 1 of the mode word, unless the
+    // launch wants this input kept in the cache (bits 3..6, inputs 0..3).
+    static std::string load_policy(int i) {
+        if (i >= 4) return "mode & 2";
+        return "(mode & 2) && !(mode & " + std::to_string(8 << i) + ")";
+    }
+
     std::string chain_tile_fn(int unroll) const {
         const std::string U = std::to_string(unroll);
         std::string s = "static __device__ __forceinline__ void custos_tile" + U + "(";
@@ -410,7 +418,7 @@ struct KernelText {
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
         for (int i = 0; i < n_in; i++) {
             const std::string id = std::to_string(i);
-            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BT * 16u), mode & 2);\n";
+            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BT * 16u), " + load_policy(i) + ");\n";
         }
         s += "    }\n";
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
@@ -493,7 +501,7 @@ struct KernelText {
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
         for (int i = 0; i < n_ops; i++) {
             const std::string id = std::to_string(i);
-            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BT * 16u), mode & 2);\n";
+            s += "        a" + id + "[u] = custos_ld(rs" + id + ", lane + (unsigned int)u * (CUSTOS_BT * 16u), " + load_policy(i) + ");\n";
         }
         s += "    }\n";
         s += "#pragma unroll\n    for (int u = 0; u < " + U + "; u++) {\n";
@@ -648,7 +656,7 @@ bool build_kernel_spec(Kind kind, DType dtype, const std::string& src,
     k.markers = markers;
     // (the key holds the vectors per thread as requested: 0 = chosen per launch)
     int32_t tail[5] = {static_cast<int32_t>(kind), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, 20 /* template version */};
+                       k.tuning.blocks_per_cu, 21 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     {
@@ -783,7 +791,7 @@ bool build_chain_spec(DType dtype, std::vector<ChainStage> stages, int n_ext, in
                         (stage.out >= 0 ? " -> out" + std::to_string(stage.out) : std::string()) + "; ";
     }
     int32_t tail[7] = {static_cast<int32_t>(Kind::Chain), k.tuning.block_threads, k.auto_unroll ? 0 : k.tuning.unroll,
-                       k.tuning.blocks_per_cu, n_ext, n_outs, 20 /* template version */};
+                       k.tuning.blocks_per_cu, n_ext, n_outs, 21 /* template version */};
     k.hash = fnv1a64(tail, sizeof tail, h);
     k.vec_elems = static_cast<int>(16 / dtype_size(dtype));
     k.stages = std::move(stages);

@@ -66,12 +66,14 @@ constexpr unsigned long long kL2WorkingSet = 32ull << 20;  // what the eight L2s
 // `revisits`: the launch touches memory that the launch before it wrote (the same launch repeated,
 // a consumer of the last launch); `n_written`: how many of its operands it writes.
 LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, CacheHint hint = CacheHint::Unknown,
-                            unsigned long long working_set_bytes = 0, bool revisits = true, int n_written = 1, bool rereads = false);
+                            unsigned long long working_set_bytes = 0, bool revisits = true, int n_written = 1, int keep_inputs = 0);
 
 // The last argument of every generated entry point: how this launch runs the kernel.  Nothing
 // of it is compiled in, so one kernel per expression serves every launch size.
 //   bit 0      the tiles are walked from the last to the first
 //   bit 1, 2   non-temporal loads, non-temporal stores
+//   bits 3..6  input 0..3 is loaded with temporal accesses although bit 1 is set: the memory-side cache is
+//              to keep that input (the launch after this one reads it again) and nothing else
 //   bit 7      stores are written through to device scope at once instead of lingering in an L2
 //   bits 8..11 vectors per thread (only read by kernels whose launch shape was left open)
 //   bits 13,14 threads per workgroup as 64 << bits (likewise)
@@ -80,12 +82,15 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
 //   bits 16..  (single-launch entry point) the number of tiles of the vector range
 // The last two spare every workgroup of a launch the arithmetic that finds them out again: the
 // host knows them.
-// `nontemporal` as in Tuning: bit 0 loads, bit 1 stores, kStoresWriteThrough the write-through stores.
+// `nontemporal` as in Tuning: bit 0 loads, bit 1 stores, kStoresWriteThrough the write-through stores;
+// bits kKeepInputShift.. (library's choice only): the inputs that keep temporal loads.
 constexpr int kStoresWriteThrough = 64;
+constexpr int kKeepInputShift = 8, kKeepInputMask = 15;
 inline uint64_t launch_mode(int unroll, int nontemporal, bool rev, int block_threads, uint64_t n_tiles = 0,
                             bool scalar_edges = true) {
     const uint64_t log2_waves = block_threads >= 512 ? 3 : block_threads >= 256 ? 2 : block_threads >= 128 ? 1 : 0;
     return (rev ? 1u : 0u) | static_cast<uint64_t>(nontemporal & 3) << 1 |
+           static_cast<uint64_t>((nontemporal >> kKeepInputShift) & kKeepInputMask) << 3 |
            static_cast<uint64_t>((nontemporal & kStoresWriteThrough) ? 1 : 0) << 7 | static_cast<uint64_t>(unroll & 15) << 8 |
            (scalar_edges ? 1u << 12 : 0u) | log2_waves << 13 | n_tiles << 16;
 }

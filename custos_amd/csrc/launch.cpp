@@ -47,19 +47,11 @@ bool RecentTraffic::wrote_any_of(const std::vector<Access>& reads) const {
     return false;
 }
 
-bool RecentTraffic::last_read_exactly(const std::vector<Access>& all) const {
+bool RecentTraffic::last_read_all_of(const Access& range) const {
     if (launches_.empty()) return false;
-    std::vector<Access> reads;
-    for (const Access& a : all)
-        if (!a.write) reads.push_back(a);
-    reads = merged(std::move(reads));
-    size_t at = 0;
-    for (const Access& was : launches_.back()) {
-        if (was.write) continue;
-        if (at == reads.size() || reads[at].begin != was.begin || reads[at].end != was.end) return false;
-        at++;
-    }
-    return at == reads.size() && at > 0;
+    for (const Access& was : launches_.back())
+        if (!was.write && was.begin <= range.begin && range.end <= was.end) return true;
+    return false;
 }
 
 bool RecentTraffic::last_wrote_any_of(const std::vector<Access>& ranges) const {
@@ -220,7 +212,8 @@ ResolvedShape shape_of_launch(custos_hip_device* dev, const custos_hip_kernel* k
     for (const Access& a : acc) footprint += a.end - a.begin;
     CacheHint hint = CacheHint::Unknown;
     unsigned long long working_set = 0;
-    bool revisits = true, rereads = false;
+    bool revisits = true;
+    int keep_inputs = 0;
     if (footprint > kTrafficBeyondBytes) {
         if (footprint >= kHintFromBytes) {
             std::vector<Access> reads;
@@ -234,10 +227,25 @@ ResolvedShape shape_of_launch(custos_hip_device* dev, const custos_hip_kernel* k
         // memory-side cache to a large one
         working_set = history->working_set_with(acc);
         revisits = history->last_wrote_any_of(acc);
-        rereads = !revisits && history->last_read_exactly(acc);
+        // Inputs (the first four pointers can be named) that this launch only reads and that the
+        // launch before it read as well, while nothing that launch wrote is touched: they are what
+        // the memory-side cache can still hold of that launch, and what the launch after this one
+        // is likely to read again -- if they are no more than twice what that cache holds.
+        if (!revisits) {
+            unsigned long long kept = 0;
+            for (size_t i = 0; i < acc.size() && i < 4; i++) {
+                if (acc[i].write || !history->last_read_all_of(acc[i])) continue;
+                bool also_written = false;
+                for (const Access& w : acc) also_written = also_written || (w.write && w.begin < acc[i].end && acc[i].begin < w.end);
+                if (also_written) continue;
+                keep_inputs |= 1 << i;
+                kept += acc[i].end - acc[i].begin;
+            }
+            if (kept > 2 * kCacheWorkingSet) keep_inputs = 0;
+        }
         history->record(acc);
     }
-    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set, revisits, rereads);
+    const ResolvedShape shape = resolve_shape(dev, k, footprint, hint, working_set, revisits, keep_inputs);
     dev->last_shape[0] = shape.unroll, dev->last_shape[1] = shape.nontemporal, dev->last_shape[2] = shape.alternate;
     dev->last_shape[3] = shape.block;
     return shape;

@@ -123,9 +123,8 @@ class RecentTraffic {
     bool wrote_any_of(const std::vector<Access>& reads) const;
     // Whether the launch recorded last wrote something in `ranges`.
     bool last_wrote_any_of(const std::vector<Access>& ranges) const;
-    // Whether the launch recorded last read exactly the ranges that `all` reads, no more and no less
-    // (ranges that are only read; `all` may hold written ranges too, which are not looked at).
-    bool last_read_exactly(const std::vector<Access>& all) const;
+    // Whether the launch recorded last read (and did not write) all of `range`.
+    bool last_read_all_of(const Access& range) const;
     // Distinct bytes touched by the recorded launches and by `all` together.
     unsigned long long working_set_with(const std::vector<Access>& all) const;
     void record(const std::vector<Access>& all);
@@ -355,7 +354,7 @@ struct ResolvedShape {
 };
 // `revisits`: the launch touches memory the launch before it wrote (see preferred_shape).
 ResolvedShape resolve_shape(const custos_hip_device* dev, const custos_hip_kernel* k, unsigned long long footprint_bytes,
-                            CacheHint hint = CacheHint::Unknown, unsigned long long working_set_bytes = 0, bool revisits = true, bool rereads = false);
+                            CacheHint hint = CacheHint::Unknown, unsigned long long working_set_bytes = 0, bool revisits = true, int keep_inputs = 0);
 // The shape of ONE launch of `k` over the operand ranges `acc`, from the launches before it
 // (`history`, which the launch then joins) and from whether a launch soon after it reads what it
 // writes (`feeds_later`); counts the hint in the device's statistics.  The same decision for a

@@ -326,10 +326,11 @@ int32_t custos_hip_launch_hint_stats(custos_hip_device *dev, uint64_t *unrelated
  * what it has in common with the launch before it (`revisits`: 1 = it touches memory that launch
  * wrote; 0 = nothing of that: a launch of more than 32 MiB then runs as one-wavefront workgroups
  * with one vector per thread, and `block_threads` receives 64, else 0 for the workgroup size the
- * kernel was compiled for; 2 = nothing that launch wrote, and it reads exactly what that launch
- * read (`y = f(x)` into another buffer every time): as for 0, with temporal loads, non-temporal
- * stores written through at once and the direction alternating, so that the cache keeps the input
- * both launches read). */
+ * kernel was compiled for; 2 = nothing that launch wrote, and its first input is something that
+ * launch read as well (`y = f(x)` into another buffer every time; a gradient launch behind the
+ * forward launch of the same x): as for 0, with the direction alternating and everything streaming
+ * past the memory-side cache but that input, which is loaded with temporal accesses -- reported in
+ * `nontemporal` as 256 << i for input i on top of the bits of custos_hip_tuning). */
 int32_t custos_hip_preferred_shape_of(uint64_t footprint_bytes, int32_t n_operands, int32_t n_written,
                                       uint64_t working_set_bytes, int32_t revisits, int32_t *unroll,
                                       int32_t *nontemporal, int32_t *alternate, int32_t *block_threads);

@@ -162,12 +162,13 @@ def test_launch_shape_by_what_a_launch_revisits_and_writes():
     assert shape(768 * MiB, 3, revisits=False) == (1, loads, True, 64)                       # config 3 backward after forward
     assert shape(2048 * MiB, 2, revisits=False) == (1, loads, True, 64)                      # the first launch of an unfused chain
     assert shape(20 * MiB, 2, working_set_bytes=60 * MiB, revisits=False) == (2, loads, False, 0)   # small launches keep 128 x 2
-    # reads exactly what the launch before it read, and touches nothing that launch wrote
+    # its first input is what the launch before it read as well, and it touches nothing that launch wrote
+    keep_first = 3 | 64 | 1 << 8                  # everything streams past the cache but input 0
     assert shape(32 * MiB, 2, revisits=2) == (2, 0, False, 0)
-    assert shape(512 * MiB, 2, revisits=2) == (1, stores, True, 64)                          # y = f(x) into another buffer every time
-    assert shape(768 * MiB, 3, revisits=2) == (1, stores, True, 64)
-    assert shape(48 * MiB, 2, revisits=2) == (1, stores, True, 64)
-    assert shape(2048 * MiB, 2, revisits=2) == (1, stores, True, 64)
+    assert shape(512 * MiB, 2, revisits=2) == (1, keep_first, True, 64)                      # y = f(x) into another buffer every time
+    assert shape(768 * MiB, 3, revisits=2) == (1, keep_first, True, 64)                      # config 3 backward after forward of the same x
+    assert shape(48 * MiB, 2, revisits=2) == (1, keep_first, True, 64)
+    assert shape(2048 * MiB, 2, revisits=2) == (1, keep_first, True, 64)
     assert shape(20 * MiB, 2, working_set_bytes=60 * MiB, revisits=2) == (2, loads, False, 0)
     # mostly writes
     assert shape(4096 * MiB, 4, n_written=3) == (2, stores, True, 0)                         # config 2 recorded unfused: 1R + 3W

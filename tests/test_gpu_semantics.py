@@ -1209,8 +1209,8 @@ def test_mid_sized_launches_leave_the_cache_to_their_neighbours(oracle):
         assert dev.last_launch_shape() == (1, loads, True)
         dev.apply_fn(x, fwd, out=y)                   # nothing else in between: it overwrites what was just written
         assert dev.last_launch_shape() == (2, loads, True)
-        g, o = dev.alloc(n), dev.alloc(n)
-        dev.add_unary_grad(x, g, o, lambda v: v.mul(2.0))
+        g, o, x2 = dev.alloc(n), dev.alloc(n), dev.alloc(n)
+        dev.add_unary_grad(x2, g, o, lambda v: v.mul(2.0))      # (another input: nothing the launch before it read)
         assert dev.last_launch_shape() == (1, loads, True)      # three pointers: always loads only; y is not among them
         dev.apply_fn(x, fwd, out=y)                   # g and o were touched since, and g is what was written last
         assert dev.last_launch_shape() == (1, both, True)
@@ -1223,13 +1223,15 @@ def test_mid_sized_launches_leave_the_cache_to_their_neighbours(oracle):
 
 def test_a_launch_that_reads_what_the_one_before_read_keeps_the_input_cached(oracle):
     """`out = device.apply_fn(&x, f)` in a loop alternates between two output blocks: each launch touches
-    nothing the launch before it wrote and reads exactly what it read, and takes temporal loads, stores
-    past the cache and the alternating direction.  A launch that merely shares an input with the one
-    before (the gradient launch behind the forward launch of the same x) does not.  Same bits either way."""
+    nothing the launch before it wrote and reads what it read, and loads that input with temporal accesses
+    while everything else streams past the cache, in the alternating direction.  The same for the gradient
+    launch behind the forward launch of the same x (x is kept, the other operands stream) and the forward
+    launch behind it.  Same bits as the oracle in every shape."""
     import custos_amd
     dev = custos_amd.HIP(0)
     try:
-        loads, stores = 1 | 64, 2 | 64
+        loads = 1 | 64
+        keep_first = 3 | 64 | 1 << 8
         n = (1 << 24) + 3                             # 64 MiB per array
         xs = synth.uniform_f32(77, n, -2, 2)
         x = dev.buffer(xs)
@@ -1240,16 +1242,26 @@ def test_a_launch_that_reads_what_the_one_before_read_keeps_the_input_cached(ora
         assert dev.last_launch_shape() == (1, loads, False)      # nothing before it
         for step in range(1, 5):
             dev.apply_fn(x, f, out=outs[step & 1])
-            assert dev.last_launch_shape() == (1, stores, True), step
+            assert dev.last_launch_shape() == (1, keep_first, True), step
         for out in outs:
             assert_bits_equal(out.read(), want)
-        g, o = dev.alloc(n), dev.buffer(synth.uniform_f32(78, n, -1, 1))
-        dev.add_unary_grad(x, g, o, lambda v: v.mul(2.0))        # reads x too, and two arrays more
-        assert dev.last_launch_shape() == (1, loads, False)
-        dev.apply_fn(x, f, out=outs[0])                          # the launch before it read more than x
-        assert dev.last_launch_shape() == (1, loads, False)
+        gs, os_ = synth.uniform_f32(79, n, -1, 1), synth.uniform_f32(78, n, -1, 1)
+        g, o = dev.buffer(gs), dev.buffer(os_)
+        grad = lambda v: v.mul(2.0)
+        for step in range(3):
+            dev.add_unary_grad(x, g, o, grad)                    # reads x as the launch before it did, and two arrays more
+            assert dev.last_launch_shape() == (1, keep_first, True)
+            gs = oracle.add_unary_grad(grad, xs, gs, os_)
+            dev.apply_fn(x, f, out=outs[0])                      # x again; nothing the gradient launch wrote
+            assert dev.last_launch_shape() == (1, keep_first, True)
+        assert_bits_equal(g.read(), gs)
+        assert_bits_equal(outs[0].read(), want)
         dev.apply_fn(x, f, out=outs[0])                          # overwrites what was just written: the usual shape
         assert dev.last_launch_shape()[0] == 2
+        y = dev.alloc(n)
+        dev.apply_fn2(o, x, lambda p, q: p.add(q), out=y)        # x is its second input
+        assert dev.last_launch_shape() == (1, 3 | 64 | 2 << 8, True)
+        assert_bits_equal(y.read(), oracle.apply_fn(lambda p, q: p.add(q), os_, xs))
     finally:
         dev.close()
 
