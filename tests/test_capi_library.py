@@ -167,9 +167,16 @@ def test_launch_shape_by_what_a_launch_revisits_and_writes():
     assert shape(32 * MiB, 2, revisits=2) == (2, 0, False, 0)
     assert shape(512 * MiB, 2, revisits=2) == (1, keep_first, True, 64)                      # y = f(x) into another buffer every time
     assert shape(768 * MiB, 3, revisits=2) == (1, keep_first, True, 64)                      # config 3 backward after forward of the same x
-    assert shape(48 * MiB, 2, revisits=2) == (1, keep_first, True, 64)
+    assert shape(48 * MiB, 2, revisits=2) == (1, keep_first, False, 64)                      # (alternating from 256 MiB on, as ever)
+    assert shape(256 * MiB + 1, 2, revisits=2) == (1, keep_first, True, 64)
     assert shape(2048 * MiB, 2, revisits=2) == (1, keep_first, True, 64)
     assert shape(20 * MiB, 2, working_set_bytes=60 * MiB, revisits=2) == (2, loads, False, 0)
+    # two or more inputs and one output over more than 768 MiB: one-wavefront workgroups whatever came before
+    assert shape(1024 * MiB, 3) == (1, loads, True, 64)
+    assert shape(2048 * MiB, 4) == (1, loads, True, 64)
+    assert shape(768 * MiB + 1, 3) == (1, loads, True, 64)
+    assert shape(768 * MiB, 3) == (2, loads, True, 0)                                        # config 3 backward, repeated by itself
+    assert shape(2048 * MiB, 2) == (2, loads, True, 0)                                       # two pointers keep 128 x 2
     # mostly writes
     assert shape(4096 * MiB, 4, n_written=3) == (2, stores, True, 0)                         # config 2 recorded unfused: 1R + 3W
     assert shape(256 * MiB, 4, n_written=3) == (2, stores, False, 0)

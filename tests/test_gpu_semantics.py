@@ -1224,7 +1224,7 @@ def test_mid_sized_launches_leave_the_cache_to_their_neighbours(oracle):
 def test_a_launch_that_reads_what_the_one_before_read_keeps_the_input_cached(oracle):
     """`out = device.apply_fn(&x, f)` in a loop alternates between two output blocks: each launch touches
     nothing the launch before it wrote and reads what it read, and loads that input with temporal accesses
-    while everything else streams past the cache, in the alternating direction.  The same for the gradient
+    while everything else streams past the cache (its direction alternates from 256 MiB touched on, as for other launches).  The same for the gradient
     launch behind the forward launch of the same x (x is kept, the other operands stream) and the forward
     launch behind it.  Same bits as the oracle in every shape."""
     import custos_amd
@@ -1242,7 +1242,7 @@ def test_a_launch_that_reads_what_the_one_before_read_keeps_the_input_cached(ora
         assert dev.last_launch_shape() == (1, loads, False)      # nothing before it
         for step in range(1, 5):
             dev.apply_fn(x, f, out=outs[step & 1])
-            assert dev.last_launch_shape() == (1, keep_first, True), step
+            assert dev.last_launch_shape() == (1, keep_first, False), step
         for out in outs:
             assert_bits_equal(out.read(), want)
         gs, os_ = synth.uniform_f32(79, n, -1, 1), synth.uniform_f32(78, n, -1, 1)
@@ -1250,18 +1250,24 @@ def test_a_launch_that_reads_what_the_one_before_read_keeps_the_input_cached(ora
         grad = lambda v: v.mul(2.0)
         for step in range(3):
             dev.add_unary_grad(x, g, o, grad)                    # reads x as the launch before it did, and two arrays more
-            assert dev.last_launch_shape() == (1, keep_first, True)
+            assert dev.last_launch_shape() == (1, keep_first, False)
             gs = oracle.add_unary_grad(grad, xs, gs, os_)
             dev.apply_fn(x, f, out=outs[0])                      # x again; nothing the gradient launch wrote
-            assert dev.last_launch_shape() == (1, keep_first, True)
+            assert dev.last_launch_shape() == (1, keep_first, False)
         assert_bits_equal(g.read(), gs)
         assert_bits_equal(outs[0].read(), want)
         dev.apply_fn(x, f, out=outs[0])                          # overwrites what was just written: the usual shape
         assert dev.last_launch_shape()[0] == 2
         y = dev.alloc(n)
         dev.apply_fn2(o, x, lambda p, q: p.add(q), out=y)        # x is its second input
-        assert dev.last_launch_shape() == (1, 3 | 64 | 2 << 8, True)
+        assert dev.last_launch_shape() == (1, 3 | 64 | 2 << 8, False)
         assert_bits_equal(y.read(), oracle.apply_fn(lambda p, q: p.add(q), os_, xs))
+        big = 1 << 26                                             # 512 MiB touched per launch: the direction alternates as well
+        bx, bouts = dev.alloc(big), [dev.alloc(big), dev.alloc(big)]
+        for step in range(3):
+            dev.apply_fn(bx, f, out=bouts[step & 1])
+        assert dev.last_launch_shape() == (1, keep_first, True)
+        assert (bouts[0].slice(big - 4096, big).read() == np.float32(0.25)).all()
     finally:
         dev.close()
 
