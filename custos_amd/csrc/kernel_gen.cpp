@@ -98,12 +98,13 @@ LaunchShape preferred_shape(unsigned long long footprint_bytes, int n_operands, 
              working_set > footprint_bytes)
         shape.nontemporal = kBoth;
     if (!revisits && footprint_bytes > kL2WorkingSet) shape.unroll = 1, shape.block = 64;
-    // The same shape for a launch that reads through two or more pointers and writes through one
-    // over more than 768 MiB, whatever came before it (x*a + y over 2^26..2^27 elements per operand:
-    // 7096 -> 7335 and 6921 -> 7322 GB/s; the in-place gradient kernel 7214 -> 7477 and 6724 -> 6958);
-    // a launch through two pointers keeps 128 x 2 there (7500 against 6771), and so do kernels
-    // that write through several.
-    if (n_operands >= 3 && n_written == 1 && footprint_bytes > 768 * MiB) shape.unroll = 1, shape.block = 64;
+    // The same shape for a launch through three or more pointers over more than 768 MiB, whatever
+    // came before it (x*a + y over 2^26..2^27 elements per operand: 7096 -> 7335 and 6921 -> 7322 GB/s;
+    // the in-place gradient kernel 7214 -> 7477 and 6724 -> 6958; joined kernels over 2^28 elements:
+    // 1R+2W 6170 -> 6680, 2R+2W 6260 -> 6750, 1R+3W 6180 -> 6360; tanh forward + gradient joined,
+    // 3R+2W over 2^26: 7783 -> 8516 on 24 bytes per element).  A launch through two pointers keeps
+    // 128 x 2 there (7500 against 6771), and up to 768 MiB the shapes are equal for all of them.
+    if (n_operands >= 3 && footprint_bytes > 768 * MiB) shape.unroll = 1, shape.block = 64;
     // It touches nothing the launch before it wrote but reads, through the inputs `keep_inputs` names,
     // what that launch read as well (`y = f(x)` into another buffer every time, what
     // `out = device.apply_fn(&x, f)` in a loop does; the gradient launch behind the forward launch of

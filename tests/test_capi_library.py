@@ -171,22 +171,24 @@ def test_launch_shape_by_what_a_launch_revisits_and_writes():
     assert shape(256 * MiB + 1, 2, revisits=2) == (1, keep_first, True, 64)
     assert shape(2048 * MiB, 2, revisits=2) == (1, keep_first, True, 64)
     assert shape(20 * MiB, 2, working_set_bytes=60 * MiB, revisits=2) == (2, loads, False, 0)
-    # two or more inputs and one output over more than 768 MiB: one-wavefront workgroups whatever came before
+    # three or more pointers over more than 768 MiB: one-wavefront workgroups whatever came before
     assert shape(1024 * MiB, 3) == (1, loads, True, 64)
     assert shape(2048 * MiB, 4) == (1, loads, True, 64)
     assert shape(768 * MiB + 1, 3) == (1, loads, True, 64)
     assert shape(768 * MiB, 3) == (2, loads, True, 0)                                        # config 3 backward, repeated by itself
     assert shape(2048 * MiB, 2) == (2, loads, True, 0)                                       # two pointers keep 128 x 2
     # mostly writes
-    assert shape(4096 * MiB, 4, n_written=3) == (2, stores, True, 0)                         # config 2 recorded unfused: 1R + 3W
+    assert shape(4096 * MiB, 4, n_written=3) == (1, stores, True, 64)                        # config 2 recorded unfused: 1R + 3W
     assert shape(256 * MiB, 4, n_written=3) == (2, stores, False, 0)
     assert shape(128 * MiB, 4, n_written=3) == (2, stores, False, 0)
     assert shape(127 * MiB, 4, n_written=3) == (2, loads, False, 0)                          # below: the usual policy is ahead
     assert shape(96 * MiB, 6, n_written=3) == (2, loads, False, 0)                           # config 5 as recorded: 3R + 3W
-    assert shape(1024 * MiB, 4, n_written=2) == (2, loads, True, 0)                          # 2R + 2W
-    assert shape(1024 * MiB, 3, n_written=2) == (2, loads, True, 0)                          # 1R + 2W: one more, not two
-    assert shape(1280 * MiB, 5, n_written=2) == (2, loads, True, 0)                          # config 3 joined: 3R + 2W
-    assert shape(1536 * MiB, 6, n_written=5) == (2, stores, True, 0)                         # 1R + 5W
+    assert shape(1024 * MiB, 4, n_written=2) == (1, loads, True, 64)                         # 2R + 2W
+    assert shape(768 * MiB, 4, n_written=2) == (2, loads, True, 0)
+    assert shape(1024 * MiB, 3, n_written=2) == (1, loads, True, 64)                         # 1R + 2W: one more, not two
+    assert shape(1280 * MiB, 5, n_written=2) == (1, loads, True, 64)                         # config 3 joined: 3R + 2W
+    assert shape(1536 * MiB, 6, n_written=5) == (1, stores, True, 64)                        # 1R + 5W
+    assert shape(512 * MiB, 6, n_written=5) == (2, stores, True, 0)
     assert shape(1536 * MiB, 6, n_written=5, revisits=False) == (1, stores, True, 64)
     with pytest.raises(capi.CustosHipError):
         shape(1 * MiB, 2, n_written=3)
