@@ -338,6 +338,9 @@ int32_t custos_hip_preferred_shape(uint64_t footprint_bytes, int32_t n_operands,
                                    int32_t *nontemporal, int32_t *alternate);
 /* The shape of the generated kernel that was launched directly, or planned into a graph by
  * custos_hip_capture_end, last on this device (same three values; all 0 before the first).
+ * `nontemporal` may carry 256 << i on top of the bits of custos_hip_tuning: input i of the launch
+ * keeps temporal loads although bit 0 is set, because the launch before it read that input too
+ * and the memory-side cache is left to it (see custos_hip_preferred_shape_of).
  * No counterpart in the reference, whose launches have one shape. */
 int32_t custos_hip_last_launch_shape(custos_hip_device *dev, int32_t *unroll, int32_t *nontemporal,
                                      int32_t *alternate);
