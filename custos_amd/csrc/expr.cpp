@@ -197,7 +197,7 @@ struct Parser {
 
         if (c == '(') {
             pos++;
-            int lhs;
+            int lhs = -1;
             if (!parse(&lhs, depth + 1)) return false;
             skip_ws();
             if (pos < s.size() && s[pos] == ')') {  // plain parentheses
@@ -214,7 +214,7 @@ struct Parser {
             else if (s[pos] == '*') op = Op::Mul, pos++;
             else if (s[pos] == '/') op = Op::Div, pos++;
             else return fail(CUSTOS_HIP_ERR_EXPR_SYNTAX, "expected a binary operator");
-            int rhs;
+            int rhs = -1;
             if (!parse(&rhs, depth + 1)) return false;
             if (!expect(')')) return false;
             Node n;
@@ -230,7 +230,7 @@ struct Parser {
             while (look < s.size() && s[look] == ' ') look++;
             if (look < s.size() && s[look] == '(') {  // "-(e)": Neg
                 pos = look + 1;
-                int inner;
+                int inner = -1;
                 if (!parse(&inner, depth + 1)) return false;
                 if (!expect(')')) return false;
                 Node n;

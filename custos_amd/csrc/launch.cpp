@@ -155,7 +155,7 @@ int32_t launch_or_record(custos_hip_device* dev, custos_hip_kernel* k, const std
             return CUSTOS_HIP_OK;
         }
     }
-    unsigned long long head, n_vec, count = n;
+    unsigned long long head = 0, n_vec = 0, count = n;
     int32_t rc = plan_launch(dev, k, ops, n, &head, &n_vec);
     if (rc != CUSTOS_HIP_OK) return rc;
     if (dev->capturing) {
