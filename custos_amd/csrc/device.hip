@@ -886,7 +886,7 @@ void OperandSetChecker::reserve(size_t max_sets) {
 }
 
 int32_t OperandSetChecker::check(const uint64_t* operands, int n_ptrs, size_t n_sets, int written, uint64_t bytes, const char** why) {
-    if (slots.size() < 2 * n_sets || bytes == 0 || written < 0 || written >= n_ptrs) {
+    if (slots.size() < 2 || slots.size() < 2 * n_sets || bytes == 0 || written < 0 || written >= n_ptrs) {
         *why = "operand check called outside its limits";
         return CUSTOS_HIP_ERR_INVALID_ARGUMENT;
     }
