@@ -28,6 +28,8 @@ int32_t hip_fail(custos_hip_device* dev, hipError_t e, const char* what) {
 
 const std::string& thread_last_error() { return g_last_error; }
 
+bool g_single_gpu = false;
+
 constexpr size_t kStagedReadMax = 64u << 10;  // reads and writes up to this size go through pinned staging memory
 constexpr size_t kSignalledReadMax = 4u << 10;  // reads up to this size: the copy kernel also writes the wait's completion word
 constexpr size_t kWriteSlots = 16;            // staging slots of short writes (the first slot of the block is the read's)
@@ -454,6 +456,7 @@ int32_t custos_hip_device_create(int32_t idx, custos_hip_device** out) {
     *out = nullptr;
     int count = 0;
     HIP_TRY(nullptr, hipGetDeviceCount(&count));
+    g_single_gpu = count == 1;
     if (idx < 0 || idx >= count)
         return set_error(nullptr, CUSTOS_HIP_ERR_INVALID_DEVICE_INDEX,
                          "device index " + std::to_string(idx) + " out of range: " + std::to_string(count) + " device(s)");
